@@ -1,0 +1,169 @@
+/* plow_moe.h — C-ABI of the gfx950 (MI355X) Mixture-of-Experts expert-FFN operator.
+ *
+ * The library behind this header is a drop-in for plow's MoE op family on one AMD GPU: it takes the
+ * same 64-byte op descriptor plow's interpreters execute, with the same operand slots, tensor
+ * layouts, sentinels and refusal behaviour, and runs it as dedicated HIP kernels on a caller-owned
+ * stream. Nothing here allocates per call, synchronises the host, or reads device routing data on
+ * the host, so a caller may record the calls into a HIP graph.
+ *
+ * Reference interfaces this header replaces (paths relative to the plow tree):
+ *   descriptor + sentinels   runtime/common/dev_isa.h:1586-1613, :1575, :2064
+ *   CPU kernel entry shape   runtime/cpu/dev/cpu_dev.h:172-181   (fn(inst, slice, nblk, tensors, ctx))
+ *   op slot maps             runtime/common/dev_isa.h:363-370, :435-474, :495-508, :565-569,
+ *                            :653-661, :682-709, :1429-1439; runtime/amd/interp.hip:6202-6293,
+ *                            :6384-6399, :6468-6635
+ *   native-segment route     crates/plowrt/src/exec/gpu/moe_lt.rs:24-60, :697-814, :1134-1322
+ *                            (the moe_pf_lt / moe_dec_lt variants), knobs
+ *                            crates/plowrt/src/config.rs:2023-2060
+ *
+ * All entry points return 0 on success or a negative PLOW_MOE_E* code; they never throw or abort.
+ */
+#ifndef PLOW_MOE_H
+#define PLOW_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- descriptor (byte-identical to PlowDevInst, runtime/common/dev_isa.h:1607-1613) ---------- */
+
+typedef union {
+    float    f;
+    uint32_t u;
+} PlowFJ;
+
+typedef struct {
+    uint16_t op;
+    uint16_t blocks; /* workgroups the producer sliced the op across; advisory for this library */
+    PlowFJ   fj[3];
+    uint16_t t[8];   /* handles into the tensor table; PLOW_TENSOR_NONE = absent => NULL */
+    uint32_t i[8];
+} PlowDevInst;
+
+#define PLOW_TENSOR_NONE   0xFFFFu      /* dev_isa.h:2064 */
+#define PLOW_EXPERT_UNUSED 0xFFFFFFFFu  /* dev_isa.h:1575 */
+
+/* Routing table entry (runtime/cpu/dev/golden/gptoss.h:24-28). */
+typedef struct {
+    uint32_t eid;
+    float    gate;
+} PlowMoeRoute;
+
+/* Rows each expert's gathered segment is padded to (runtime/amd/op_moe.h:1921-1923) and the
+ * capacity contract of the gathered arrays (op_moe.h:2252-2255). */
+#define PLOW_MPF_BM 64u
+#define PLOW_MPF_META_INTS(n_exp) (3u * (n_exp) + 1u)
+#define PLOW_MPF_MAX_ROWS(T, k, n_exp) ((T) * (k) + (n_exp) * (PLOW_MPF_BM - 1u))
+#define PLOW_ROUTE_MAX_TOPK 16u         /* golden/moe_route.c:15 */
+#define PLOW_ROUTE_MAX_GROUPS 64u       /* runtime/common/moe_route_key.h:33 */
+
+/* ---- opcodes served (numbers from runtime/common/dev_isa.h) ---------------------------------- */
+enum {
+    PLOW_DOP_GEMM                          = 8,   /* dense bf16 GEMM (shared-expert down)        */
+    PLOW_DOP_GEMM_GLU                      = 20,  /* dense bf16 gate|up + GLU (shared expert)    */
+    PLOW_DOP_QUANT_FP8                     = 32,  /* per-row e4m3 activation quant               */
+    PLOW_DOP_MOE_COMBINE                   = 43,
+    PLOW_DOP_MOE_GROUP_GLU_FP8_BLK         = 48,  /* decode, table-driven, i6 = enc              */
+    PLOW_DOP_MOE_GROUP_DOWN_FP8_BLK        = 49,
+    PLOW_DOP_MOE_ROUTER_TOPK               = 56,
+    PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8      = 65,  /* decode, per-channel fp8, fused gate_up table */
+    PLOW_DOP_MOE_EXPERT_DOWN_GEMMA_FP8     = 66,
+    PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF_W8A8   = 81,  /* grouped, per-channel fp8 x per-row fp8      */
+    PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8  = 82,
+    PLOW_DOP_MOE_ROUTER_TOPK_PF            = 83,
+    PLOW_DOP_MOE_ALIGN_PF                  = 84,
+    PLOW_DOP_MOE_GROUP_GLU_PF              = 85,
+    PLOW_DOP_MOE_GROUP_DOWN_PF             = 86,
+    PLOW_DOP_MOE_COMBINE_PF                = 87,
+    PLOW_DOP_GEMM_F32                      = 180, /* router score: bf16 x bf16 -> f32 logits     */
+    PLOW_DOP_QUANT_FP8_BLOCK128            = 184  /* 1x128 e4m3 activation quant                 */
+};
+
+/* Weight encodings (i3 on ops 85/86, i6 on ops 48/49; dev_isa.h:442-461, :691-702). */
+enum { PLOW_MOE_ENC_BF16 = 0, PLOW_MOE_ENC_FP8BLK = 1, PLOW_MOE_ENC_MXFP4 = 2 };
+
+/* Arms of ops 85/86 (i7; runtime/amd/interp.hip:6500-6604). 0 and 2/3 are the reference's; 8 is
+ * this library's name for "mxfp4 weights, bf16 activations" on gathered rows (the arithmetic of the
+ * reference's decode ops 48/49 at enc 2); the reference's enc-2 default (fp4 on both operands) is
+ * refused with PLOW_MOE_EUNSUPPORTED. */
+enum {
+    PLOW_MOE_ARM_A16       = 0, /* bf16 activations (enc 0 bf16 weights, enc 1 W8A16)             */
+    PLOW_MOE_ARM_W8A8      = 2, /* enc 1: e4m3 activations with 1x128 scales; DOWN writes f32 part */
+    PLOW_MOE_ARM_W8A8_P16  = 3, /* DOWN only: as 2 with a bf16 part                                */
+    PLOW_MOE_ARM_W4A16     = 8
+};
+
+/* GLU activations (i5; runtime/amd/op_moe.h:216-241, golden/golden.h:107-133). */
+enum { PLOW_MOE_ACT_GELU_TANH = 0, PLOW_MOE_ACT_SILU = 1 };
+
+/* Router flags (i3 of ops 56/83; runtime/amd/op_moe.h:453-467). */
+enum {
+    PLOW_ROUTE_SIGMOID   = 1u, /* else softmax */
+    PLOW_ROUTE_NORM_TOPK = 2u,
+    PLOW_ROUTE_BIAS      = 4u, /* t3 is bound */
+    PLOW_ROUTE_F32_LOGIT = 8u
+};
+
+/* ---- error codes -------------------------------------------------------------------------------- */
+enum {
+    PLOW_MOE_OK           = 0,
+    PLOW_MOE_EINVAL       = -22, /* malformed descriptor / operand wiring / geometry                */
+    PLOW_MOE_EUNSUPPORTED = -95, /* opcode, encoding or arm this library refuses                    */
+    PLOW_MOE_EDEVICE      = -5,  /* a HIP call failed; plow_moe_last_error has the text             */
+    PLOW_MOE_ENOMEM       = -12,
+    PLOW_MOE_ROLLBACK     = 1    /* segment entry points only: the knob says "leave it to the
+                                  * interpreter" (config.rs:2023-2060, value 0 or rows < min_rows) */
+};
+
+typedef struct PlowMoeCtx PlowMoeCtx;
+
+/* ABI marker, the analogue of the `plow_moe_lt_abi` word plowrt reads from a loaded object
+ * (crates/plowrt/src/exec/gpu/moe_lt.rs:713-724). */
+uint32_t plow_moe_abi(void);
+
+/* Create / destroy an operator context on HIP device `device`. The context owns a small fixed
+ * workspace (routing scratch, the device copy of descriptors); per-call work allocates nothing.
+ * Replaces the per-engine load step of moe_lt.rs:697-814. */
+int  plow_moe_create(PlowMoeCtx** out, int device);
+void plow_moe_destroy(PlowMoeCtx* ctx);
+
+/* Text of the last failure on this context (valid until the next call on it). */
+const char* plow_moe_last_error(const PlowMoeCtx* ctx);
+
+/* Execute ONE op descriptor asynchronously on `stream` (a hipStream_t; NULL = the null stream).
+ * `tensors` is the handle table: tensors[inst->t[j]] is a device pointer. Replaces the
+ * per-instruction dispatch of runtime/amd/interp.hip:6202-6635 and the CPU twin's
+ * plow_cpu_kernel(op)(inst, slice, nblk, tensors, ctx) (runtime/cpu/dev/cpu_dev.h:172-176); the
+ * (slice, nblk) split is internal here. */
+int plow_moe_exec(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors, void* stream);
+
+/* Execute a run of descriptors in order on `stream`. */
+int plow_moe_exec_many(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst,
+                       void* const* tensors, void* stream);
+
+/* Segment-level entry points: the moe_pf_lt / moe_dec_lt variants. `insts[0..n_inst)` is one MoE
+ * segment as plowrt isolates it: the grouped GLU + DOWN pair (ops 85+86, 81+82 or 48+49), optionally
+ * preceded by its router/align/quant prologue and followed by its combine. The run is validated as
+ * a whole (operand wiring between the ops, geometry, encodings; moe_lt.rs:159-248) and refused with
+ * PLOW_MOE_EINVAL before anything is launched. `rows` is the live token count of this step.
+ * Knob semantics follow PLOW_MOE_PF_LT / PLOW_MOE_DEC_LT: see plow_moe_set_min_rows. */
+int plow_moe_pf(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, void* const* tensors,
+                uint32_t rows, void* stream);
+int plow_moe_dec(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, void* const* tensors,
+                 uint32_t rows, void* stream);
+
+/* variant: 0 = prefill (plow_moe_pf), 1 = decode (plow_moe_dec).
+ * min_rows < 0: unset, every segment is served; 0: the variant is switched off and the entry point
+ * returns PLOW_MOE_ROLLBACK; N > 0: segments with rows < N return PLOW_MOE_ROLLBACK. */
+int plow_moe_set_min_rows(PlowMoeCtx* ctx, int variant, int min_rows);
+
+/* Validate one descriptor against this library's contract without launching (0 = would run). */
+int plow_moe_check(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PLOW_MOE_H */

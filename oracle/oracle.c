@@ -1,0 +1,854 @@
+/* oracle.c — CPU restatement of plow's MoE expert-FFN path, one function per device op.
+ *
+ * TEST INFRASTRUCTURE ONLY. This file is the checker the HIP operator is compared against (and the
+ * "port" CPU baseline a benchmark may time). The shipped library never includes, links or calls it.
+ *
+ * Every op takes the same descriptor and handle table as the operator (include/plow_moe.h) with
+ * HOST pointers in the table, in the reference's worker form fn(inst, slice, nblk, tensors):
+ * slice s of nblk owns a share of the op's outputs, so nblk threads can run one op concurrently.
+ *
+ * What each function follows (paths relative to the plow tree):
+ *   op 180 router score        runtime/cpu/dev/golden/f32_primitives.c:235-252
+ *   op 83/56 router top-k      runtime/cpu/dev/golden/moe_route.c:27-86 (flat arm);
+ *                              group-limited arm runtime/common/moe_route_key.h:61-80 +
+ *                              runtime/amd/op_moe.h:377-420; shared tail slot op_moe.h:2417-2434;
+ *                              logit scale op_moe.h:444-446
+ *   op 84 align                runtime/cpu/dev/golden/moe_route.c:91-127
+ *   op 87/43 combine           runtime/cpu/dev/golden/moe_route.c:130-147; t_row0 / part16
+ *                              runtime/amd/interp.hip:6605-6635
+ *   op 184 1x128 quant         runtime/amd/op_gemm_common.h:2582-2621
+ *   op 32 per-row quant        runtime/cpu/dev/golden/fp8.c:9-30
+ *   op 85/86 enc 0 (bf16)      runtime/cpu/dev/golden/moe_gemma.c:244-302 through the wtab[E][3]
+ *                              table of runtime/amd/op_moe.h:1242-1249
+ *   op 85/86 enc 1 arm 0       runtime/amd/op_moe.h:3299-3310 (per-128-K promotion), :3799-3823,
+ *                              :3906-3927 (epilogues); decode twin op_moe.h:674-702
+ *   op 85/86 enc 1 arm 2/3     runtime/amd/moe_pf_w8a8.h:1-19, :368-379, :401-473
+ *   op 85/86 enc 2 arm 8, and
+ *   op 48/49 (all enc)         runtime/cpu/dev/golden/moe.c:21-174 with runtime/cpu/dev/
+ *                              mxfp4_common.h:30-40 as the row dot; op_moe.h:1234-1399
+ *   op 65/66                   runtime/cpu/dev/golden/fp8.c:33-41, :173-214
+ *   op 81/82                   runtime/amd/op_moe.h:6655-6700 (per-row x per-channel epilogue)
+ *   op 20 / op 8               runtime/cpu/dev/golden/gemm.c:45-96
+ *   GLU activations            runtime/cpu/dev/golden/golden.h:101-133
+ *
+ * Parity pins are listed per function in tests/test_oracle_*.py. Unpinned at bit level (tolerance
+ * level only): the f32 summation order INSIDE one 128-K block of the fp8 x fp8 arms, which the
+ * reference leaves to its MFMA; this file sums a block with eight interleaved f32 partials.
+ */
+#include "oracle.h"
+#include "codec.h"
+
+#include <pthread.h>
+#include <stdlib.h>
+
+#define TEN(in, T, k) ((in)->t[(k)] == PLOW_TENSOR_NONE ? (void*)0 : (T)[(in)->t[(k)]])
+
+static void own_range(uint32_t n, uint32_t slice, uint32_t nblk, uint32_t* lo, uint32_t* hi) {
+    const uint32_t per = (n + nblk - 1u) / nblk;
+    const uint64_t a = (uint64_t)slice * per, b = a + per;
+    *lo = a > n ? n : (uint32_t)a;
+    *hi = b > n ? n : (uint32_t)b;
+}
+
+/* ---- GLU epilogue ------------------------------------------------------------------------------ */
+
+static float act_gelu_tanh(float x) {
+    const float c = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(c));
+}
+static float act_silu(float x) { return x / (1.0f + expf(-x)); }
+/* act 0 gelu_tanh, 1 silu; the pair forms (2 situ, 3 swiglu_oai, 4 clamp) are not on this path and
+ * poison, as a gate-only epilogue does in the reference. */
+static float glu(float g, float u, uint32_t act) {
+    if (act == 1u) return act_silu(g) * u;
+    if (act == 0u) return act_gelu_tanh(g) * u;
+    return NAN;
+}
+
+/* ---- op 180: router score ---------------------------------------------------------------------- */
+
+static void op_gemm_f32(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    float* out = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    const orc_bf16* w = TEN(in, T, 2);
+    const uint32_t M = in->i[0], N = in->i[1], K = in->i[2];
+    uint32_t lo, hi;
+    own_range(N, slice, nblk, &lo, &hi);
+    for (uint32_t m = 0; m < M; m++)
+        for (uint32_t n = lo; n < hi; n++) {
+            float s = 0.0f; /* one accumulator, ascending k; a bf16 product is exact in f32 */
+            for (uint32_t k = 0; k < K; k++) {
+                s += orc_bf2f(x[(size_t)m * K + k]) * orc_bf2f(w[(size_t)n * K + k]);
+            }
+            out[(size_t)m * N + n] = s;
+        }
+}
+
+/* ---- ops 83 / 56: router top-k ----------------------------------------------------------------- */
+
+static int group_active(uint32_t n_exp, uint32_t n_group, uint32_t topk_group) {
+    return n_group > 1u && topk_group > 0u && topk_group < n_group &&
+           n_group <= PLOW_ROUTE_MAX_GROUPS && n_exp % n_group == 0u;
+}
+
+static void route_one(PlowMoeRoute* tab, const void* logit, const float* bias, uint32_t n_exp,
+                      uint32_t k, uint32_t flags, float route_scale, float logit_scale,
+                      uint32_t n_group, uint32_t topk_group, float* score, uint64_t* key) {
+    const int sigmoid = (flags & PLOW_ROUTE_SIGMOID) != 0, norm = (flags & PLOW_ROUTE_NORM_TOPK) != 0;
+    const int f32l = (flags & PLOW_ROUTE_F32_LOGIT) != 0;
+    const float ls = logit_scale != 0.0f ? logit_scale : 1.0f;
+    for (uint32_t j = PLOW_ROUTE_MAX_TOPK; j < k; j++) { tab[j].eid = PLOW_EXPERT_UNUSED; tab[j].gate = 0.0f; }
+    if (k > PLOW_ROUTE_MAX_TOPK) k = PLOW_ROUTE_MAX_TOPK;
+#define LOGIT(e) ((f32l ? ((const float*)logit)[e] : orc_bf2f(((const orc_bf16*)logit)[e])) * ls)
+    if (sigmoid) {
+        for (uint32_t e = 0; e < n_exp; e++) score[e] = 1.0f / (1.0f + expf(-LOGIT(e)));
+    } else {
+        float m = -1e30f, s = 0.0f;
+        for (uint32_t e = 0; e < n_exp; e++) { score[e] = LOGIT(e); if (score[e] > m) m = score[e]; }
+        for (uint32_t e = 0; e < n_exp; e++) { score[e] = expf(score[e] - m); s += score[e]; }
+        for (uint32_t e = 0; e < n_exp; e++) score[e] /= s;
+    }
+#undef LOGIT
+    /* packed selection key: ord(score + bias) above the inverted id, so ties go to the lowest id */
+    for (uint32_t e = 0; e < n_exp; e++)
+        key[e] = ((uint64_t)orc_ord(score[e] + (bias ? bias[e] : 0.0f)) << 20) |
+                 (uint64_t)((n_exp - 1u - e) & 0xFFFFFu);
+    if (group_active(n_exp, n_group, topk_group)) {
+        const uint32_t gsz = n_exp / n_group;
+        uint64_t gk[PLOW_ROUTE_MAX_GROUPS];
+        for (uint32_t g = 0; g < n_group; g++) {
+            float m1 = -3.0e38f, m2 = -3.0e38f; /* top-2 of the group's BIASED scores, index order */
+            for (uint32_t i = 0; i < gsz; i++) {
+                const uint32_t e = g * gsz + i;
+                const float s = score[e] + (bias ? bias[e] : 0.0f);
+                if (s > m1) { m2 = m1; m1 = s; } else if (s > m2) m2 = s;
+            }
+            gk[g] = ((uint64_t)orc_ord(m1 + m2) << 8) | (uint64_t)((n_group - 1u - g) & 0xFFu);
+        }
+        for (uint32_t g = 0; g < n_group; g++) {
+            uint32_t rank = 0;
+            for (uint32_t f = 0; f < n_group; f++) rank += gk[f] > gk[g];
+            if (rank >= topk_group) /* dropped group: its experts keep only their id bits */
+                for (uint32_t i = 0; i < gsz; i++) {
+                    const uint32_t e = g * gsz + i;
+                    key[e] = (uint64_t)((n_exp - 1u - e) & 0xFFFFFu);
+                }
+        }
+    }
+    uint32_t win[PLOW_ROUTE_MAX_TOPK];
+    for (uint32_t j = 0; j < k; j++) win[j] = n_exp - 1u;
+    for (uint32_t e = 0; e < n_exp; e++) {
+        uint32_t rank = 0;
+        for (uint32_t f = 0; f < n_exp; f++) rank += key[f] > key[e];
+        if (rank < k) win[rank] = e;
+    }
+    float gate[PLOW_ROUTE_MAX_TOPK], sum = 0.0f;
+    for (uint32_t j = 0; j < k; j++) { gate[j] = score[win[j]]; sum += gate[j]; }
+    for (uint32_t j = 0; j < k; j++) {
+        if (norm && sum != 0.0f) gate[j] /= sum;
+        gate[j] *= route_scale;
+        tab[j].eid = win[j];
+        tab[j].gate = gate[j];
+    }
+}
+
+/* t0=table t1=logit t3=bias? i1=n_exp i2=k i3=flags i4=T(0=1) i5=shared_tail i6=n_group
+ * i7=topk_group f0=route_scale f1=logit_scale. Token t is owned by slice t % nblk. */
+static void op_router_topk(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    PlowMoeRoute* table = TEN(in, T, 0);
+    const uint8_t* logit = TEN(in, T, 1);
+    const float* bias = TEN(in, T, 3);
+    const uint32_t n_exp = in->i[1], k = in->i[2], flags = in->i[3], nt = in->i[4] ? in->i[4] : 1u;
+    const uint32_t tail = (in->op == PLOW_DOP_MOE_ROUTER_TOPK_PF && in->i[5]) ? 1u : 0u;
+    const size_t esz = (flags & PLOW_ROUTE_F32_LOGIT) ? 4u : 2u;
+    float* score = malloc((size_t)n_exp * 4u);
+    uint64_t* key = malloc((size_t)n_exp * 8u);
+    for (uint32_t tok = slice; tok < nt; tok += nblk) {
+        PlowMoeRoute* row = table + (size_t)tok * (k + tail);
+        route_one(row, logit + (size_t)tok * n_exp * esz, bias, n_exp, k, flags, in->fj[0].f,
+                  in->fj[1].f, in->i[6], in->i[7], score, key);
+        if (tail) { row[k].eid = n_exp; row[k].gate = 1.0f; }
+    }
+    free(score);
+    free(key);
+}
+
+/* ---- op 84: align ------------------------------------------------------------------------------ */
+
+static void op_align(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    if (slice != 0u || nblk == 0u) return;
+    int32_t* meta = TEN(in, T, 0);
+    const PlowMoeRoute* table = TEN(in, T, 1);
+    uint32_t* row_token = TEN(in, T, 2);
+    uint32_t* row_partidx = TEN(in, T, 3);
+    float* row_gate = TEN(in, T, 4);
+    const uint32_t nt = in->i[0], E = in->i[1], k = in->i[2], nslot = nt * k;
+    int32_t *rowoff = meta, *cnt = meta + E, *tilep = meta + 2u * E;
+    for (uint32_t e = 0; e < E; e++) cnt[e] = 0;
+    for (uint32_t s = 0; s < nslot; s++) if (table[s].eid < E) cnt[table[s].eid]++;
+    uint32_t off = 0, tiles = 0;
+    for (uint32_t e = 0; e < E; e++) {
+        const uint32_t t = ((uint32_t)cnt[e] + PLOW_MPF_BM - 1u) / PLOW_MPF_BM;
+        rowoff[e] = (int32_t)off;
+        tilep[e] = (int32_t)tiles;
+        tiles += t;
+        off += t * PLOW_MPF_BM;
+    }
+    tilep[E] = (int32_t)tiles;
+    for (uint32_t r = 0; r < off; r++) {
+        row_token[r] = PLOW_EXPERT_UNUSED;
+        row_partidx[r] = PLOW_EXPERT_UNUSED;
+        row_gate[r] = 0.0f;
+    }
+    uint32_t* cur = calloc(E ? E : 1u, 4u);
+    for (uint32_t s = 0; s < nslot; s++) { /* ascending slot => stable within an expert */
+        const uint32_t e = table[s].eid;
+        if (e >= E) continue;
+        const uint32_t pos = (uint32_t)rowoff[e] + cur[e]++;
+        row_token[pos] = s / k;
+        row_partidx[pos] = s;
+        row_gate[pos] = table[s].gate;
+    }
+    free(cur);
+}
+
+/* ---- ops 87 / 43: combine ---------------------------------------------------------------------- */
+
+static void op_combine(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    const int pf = in->op == PLOW_DOP_MOE_COMBINE_PF;
+    const uint32_t H = in->i[0], k = in->i[1], nt = pf ? (in->i[2] ? in->i[2] : 1u) : 1u;
+    const size_t r0 = pf ? in->i[3] : 0u;
+    const int part16 = pf && in->i[7];
+    orc_bf16* out = (orc_bf16*)TEN(in, T, 0) + r0 * H;
+    const orc_bf16* residual = TEN(in, T, 1);
+    const orc_bf16* shared = TEN(in, T, 2);
+    const uint8_t* part = TEN(in, T, 3);
+    if (residual) residual += r0 * H;
+    if (shared) shared += r0 * H;
+    part += r0 * k * H * (part16 ? 2u : 4u);
+    uint32_t lo, hi;
+    own_range(nt * H, slice, nblk, &lo, &hi);
+    for (uint32_t i = lo; i < hi; i++) {
+        const uint32_t tok = i / H, h = i - tok * H;
+        float acc = residual ? orc_bf2f(residual[i]) : 0.0f;
+        if (shared) acc += orc_bf2f(shared[i]);
+        for (uint32_t j = 0; j < k; j++) {
+            const size_t at = ((size_t)tok * k + j) * H + h;
+            acc += part16 ? orc_bf2f(((const orc_bf16*)part)[at]) : ((const float*)part)[at];
+        }
+        out[i] = orc_f2bf(acc);
+    }
+}
+
+/* ---- ops 184 / 32: activation quant ------------------------------------------------------------ */
+
+/* t0=xq t1=x t2=scale(f32 [K/128][pitch]) i0=M i1=K i2=pitch(0 = M). */
+static void op_quant_block128(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    uint8_t* xq = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    float* scale = TEN(in, T, 2);
+    const uint32_t M = in->i[0], K = in->i[1], pitch = in->i[2] ? in->i[2] : M, G = K / 128u;
+    uint32_t lo, hi;
+    own_range(M, slice, nblk, &lo, &hi);
+    for (uint32_t m = lo; m < hi; m++)
+        for (uint32_t g = 0; g < G; g++) {
+            const orc_bf16* src = x + (size_t)m * K + g * 128u;
+            float amax = 1e-10f; /* the amax is floored, not the scale */
+            for (uint32_t j = 0; j < 128u; j++) amax = fmaxf(amax, fabsf(orc_bf2f(src[j])));
+            const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
+            scale[(size_t)g * pitch + m] = s;
+            for (uint32_t j = 0; j < 128u; j++)
+                xq[(size_t)m * K + g * 128u + j] = orc_f32_to_e4m3(orc_bf2f(src[j]) * inv);
+        }
+}
+
+/* t0=xq t1=x t2=a_scale(f32 [M]) i0=M i1=K (the fused gate/up arm of the reference is not on this
+ * path: t3/t4 bound => poison the scales). */
+static void op_quant_row(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    uint8_t* xq = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    float* scale = TEN(in, T, 2);
+    const uint32_t M = in->i[0], K = in->i[1];
+    uint32_t lo, hi;
+    own_range(M, slice, nblk, &lo, &hi);
+    for (uint32_t m = lo; m < hi; m++) {
+        if (TEN(in, T, 3) || TEN(in, T, 4)) { scale[m] = NAN; continue; }
+        float amax = 0.0f;
+        for (uint32_t k = 0; k < K; k++) amax = fmaxf(amax, fabsf(orc_bf2f(x[(size_t)m * K + k])));
+        scale[m] = fmaxf(amax * (1.0f / 448.0f), 1e-12f);
+        const float inv = 1.0f / scale[m];
+        for (uint32_t k = 0; k < K; k++)
+            xq[(size_t)m * K + k] = orc_f32_to_e4m3(orc_bf2f(x[(size_t)m * K + k]) * inv);
+    }
+}
+
+/* ---- row dots, one per weight encoding --------------------------------------------------------- */
+
+/* Every operand of this path (bf16, e4m3, e2m1) is exact in f32 and so is any product of two of
+ * them, so a fused and an unfused multiply-add give the same bits; the ORDER of the additions is
+ * what each function below fixes. */
+static void decode_bf16_row(float* dst, const orc_bf16* src, uint32_t K) {
+    for (uint32_t k = 0; k < K; k++) dst[k] = orc_bf2f(src[k]);
+}
+static void decode_e4m3_row(float* dst, const uint8_t* src, uint32_t K) {
+    for (uint32_t k = 0; k < K; k++) dst[k] = orc_e4m3_to_f32(src[k]);
+}
+static void decode_mxfp4_row(float* dst, const uint8_t* src, uint32_t K) {
+    for (uint32_t k = 0; k < K; k++) dst[k] = orc_mxfp4_at(src, k);
+}
+
+/* Plain ascending-k sum with one accumulator (golden/moe_gemma.c gm_dot_bf16, golden/fp8.c
+ * dot_a_w8). */
+static float dot_seq(const float* wf, const float* a, uint32_t K) {
+    float acc = 0.0f;
+    for (uint32_t k = 0; k < K; k++) acc += a[k] * wf[k];
+    return acc;
+}
+
+/* Sum of one <=128-long block with eight interleaved f32 partials (the order inside a block is the
+ * reference MFMA's and is not pinned). */
+static float block_dot(const float* w, const float* a, uint32_t n) {
+    float p[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    uint32_t k = 0;
+    for (; k + 8u <= n; k += 8u)
+        for (uint32_t j = 0; j < 8u; j++) p[j] += w[k + j] * a[k + j];
+    for (; k < n; k++) p[k & 7u] += w[k] * a[k];
+    return ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
+}
+
+/* Block-fp8 weights, bf16 activations: per 128-K block, dot then `acc += dot * block_scale`.
+ * srow = this channel's scale row [ceil(K/128)]. */
+static float dot_fp8blk_a16(const float* wf, const float* srow, const float* a, uint32_t K) {
+    float acc = 0.0f;
+    for (uint32_t k0 = 0, kb = 0; k0 < K; k0 += 128u, kb++) {
+        const uint32_t n = K - k0 < 128u ? K - k0 : 128u;
+        acc += block_dot(wf + k0, a + k0, n) * srow[kb];
+    }
+    return acc;
+}
+
+/* Block-fp8 weights, 1x128-scaled e4m3 activations: acc = fmaf(t, as[kb] * ws[kb], acc),
+ * ascending kb. */
+static float dot_fp8blk_a8(const float* wf, const float* srow, const float* a, const float* as,
+                           size_t as_stride, uint32_t K) {
+    float acc = 0.0f;
+    for (uint32_t k0 = 0, kb = 0; k0 < K; k0 += 128u, kb++)
+        acc = fmaf(block_dot(wf + k0, a + k0, 128u), as[(size_t)kb * as_stride] * srow[kb], acc);
+    return acc;
+}
+
+/* mxfp4 weights, bf16 activations (mxfp4_common.h plow_mxfp4_row_dot): sequential f32 per 32-block,
+ * the E8M0 scale multiplied once per block. */
+static float dot_mxfp4(const float* wf, const uint8_t* s, const float* a, uint32_t K) {
+    float acc = 0.0f;
+    for (uint32_t k0 = 0; k0 < K; k0 += 32u) {
+        const uint32_t k1 = k0 + 32u < K ? k0 + 32u : K;
+        float blk = 0.0f;
+        for (uint32_t k = k0; k < k1; k++) blk += wf[k] * a[k];
+        acc += blk * orc_e8m0(s[k0 / 32u]);
+    }
+    return acc;
+}
+
+/* One weight row of an expert matrix under `enc`, decoded to f32 without its scales. */
+typedef struct {
+    const float* sf;   /* enc 1: scale row [ceil(K/128)] */
+    const uint8_t* sb; /* enc 2: E8M0 row [K/32] */
+} RowScale;
+
+static RowScale enc_row(uint32_t enc, const void* W, const void* S, uint32_t n, uint32_t K, float* wf) {
+    RowScale rs = {NULL, NULL};
+    if (enc == PLOW_MOE_ENC_BF16) {
+        decode_bf16_row(wf, (const orc_bf16*)W + (size_t)n * K, K);
+    } else if (enc == PLOW_MOE_ENC_MXFP4) {
+        decode_mxfp4_row(wf, (const uint8_t*)W + (size_t)n * (K / 2u), K);
+        rs.sb = (const uint8_t*)S + (size_t)n * (K / 32u);
+    } else {
+        decode_e4m3_row(wf, (const uint8_t*)W + (size_t)n * K, K);
+        rs.sf = (const float*)S + (size_t)(n >> 7) * ((K + 127u) >> 7);
+    }
+    return rs;
+}
+
+/* bf16-activation dot of a decoded weight row. */
+static float enc_dot(uint32_t enc, const float* wf, RowScale rs, const float* a, uint32_t K) {
+    if (enc == PLOW_MOE_ENC_BF16) return dot_seq(wf, a, K);
+    if (enc == PLOW_MOE_ENC_MXFP4) return dot_mxfp4(wf, rs.sb, a, K);
+    return dot_fp8blk_a16(wf, rs.sf, a, K);
+}
+
+/* ---- ops 85 / 86: grouped experts over aligned rows -------------------------------------------- */
+
+/* Decoded activation rows of one expert's live segment (pad rows flagged dead). */
+typedef struct {
+    float* a;        /* [cap][K] */
+    uint8_t* live;   /* [cap] */
+    uint32_t cap, K;
+    uint32_t expert; /* which expert is cached, ~0 = none */
+} RowCache;
+
+static void cache_init(RowCache* c, uint32_t K) { c->a = NULL; c->live = NULL; c->cap = 0; c->K = K; c->expert = ~0u; }
+static void cache_free(RowCache* c) { free(c->a); free(c->live); }
+static void cache_fit(RowCache* c, uint32_t rows) {
+    if (rows <= c->cap) return;
+    free(c->a); free(c->live);
+    c->cap = rows;
+    c->a = malloc((size_t)rows * c->K * 4u);
+    c->live = malloc(rows);
+}
+
+/* 85: t0=fu_g|fq t1=xn2|xq t2=wtab t3=stab t4=meta t5=row_token t6=xs t7=fs  i0=I i1=H i2=E i3=enc
+ * i4=xs pitch i5=act i7=arm. Work item = (expert, 128-channel group); slices split E*(I/128)
+ * (I rounded up). */
+static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    const uint64_t* wtab = TEN(in, T, 2);
+    const uint64_t* stab = TEN(in, T, 3);
+    const int32_t* meta = TEN(in, T, 4);
+    const uint32_t* row_token = TEN(in, T, 5);
+    const uint32_t I = in->i[0], H = in->i[1], E = in->i[2], enc = in->i[3], act = in->i[5];
+    const uint32_t arm = in->i[7], pitch = in->i[4];
+    const int w8a8 = enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8;
+    const float* xs = TEN(in, T, 6);
+    const uint32_t G = (I + 127u) / 128u, KB = (H + 127u) / 128u;
+    float* wg = malloc((size_t)H * 4u);
+    float* wu = malloc((size_t)H * 4u);
+    float* v = NULL;
+    uint32_t vcap = 0;
+    RowCache rc;
+    cache_init(&rc, H);
+    uint32_t lo, hi;
+    own_range(E * G, slice, nblk, &lo, &hi);
+    for (uint32_t it = lo; it < hi; it++) {
+        const uint32_t e = it / G, g0 = it % G;
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        const void* Wg = (const void*)(uintptr_t)wtab[(size_t)e * 3u + 0u];
+        const void* Wu = (const void*)(uintptr_t)wtab[(size_t)e * 3u + 1u];
+        if (cnt == 0u || !Wg) continue;
+        const void* Sg = stab ? (const void*)(uintptr_t)stab[(size_t)e * 3u + 0u] : NULL;
+        const void* Su = stab ? (const void*)(uintptr_t)stab[(size_t)e * 3u + 1u] : NULL;
+        if (rc.expert != e) {
+            cache_fit(&rc, cnt);
+            for (uint32_t q = 0; q < cnt; q++) {
+                const uint32_t tok = row_token[r0 + q];
+                rc.live[q] = tok != PLOW_EXPERT_UNUSED;
+                if (!rc.live[q]) continue;
+                if (w8a8) decode_e4m3_row(rc.a + (size_t)q * H, (const uint8_t*)TEN(in, T, 1) + (size_t)tok * H, H);
+                else decode_bf16_row(rc.a + (size_t)q * H, (const orc_bf16*)TEN(in, T, 1) + (size_t)tok * H, H);
+            }
+            rc.expert = e;
+        }
+        const uint32_t n0 = g0 * 128u, n1 = n0 + 128u < I ? n0 + 128u : I;
+        if (!w8a8) {
+            orc_bf16* fu = TEN(in, T, 0);
+            for (uint32_t n = n0; n < n1; n++) {
+                const RowScale sg = enc_row(enc, Wg, Sg, n, H, wg);
+                const RowScale su = enc_row(enc, Wu, Su, n, H, wu);
+                for (uint32_t q = 0; q < cnt; q++) {
+                    if (!rc.live[q]) continue;
+                    const float* a = rc.a + (size_t)q * H;
+                    fu[(size_t)(r0 + q) * I + n] =
+                        orc_f2bf(glu(enc_dot(enc, wg, sg, a, H), enc_dot(enc, wu, su, a, H), act));
+                }
+            }
+        } else {
+            /* fp8 x fp8: SwiGLU in f32, then the 1x128 output quant (amax floored at 1e-10) */
+            uint8_t* fq = TEN(in, T, 0);
+            float* fs = TEN(in, T, 7);
+            if (vcap < cnt) { free(v); v = malloc((size_t)cnt * 128u * 4u); vcap = cnt; }
+            for (uint32_t n = n0; n < n1; n++) {
+                decode_e4m3_row(wg, (const uint8_t*)Wg + (size_t)n * H, H);
+                decode_e4m3_row(wu, (const uint8_t*)Wu + (size_t)n * H, H);
+                for (uint32_t q = 0; q < cnt; q++) {
+                    if (!rc.live[q]) continue;
+                    const uint32_t tok = row_token[r0 + q];
+                    const float* a = rc.a + (size_t)q * H;
+                    const float g = dot_fp8blk_a8(wg, (const float*)Sg + (size_t)g0 * KB, a, xs + tok, pitch, H);
+                    const float u = dot_fp8blk_a8(wu, (const float*)Su + (size_t)g0 * KB, a, xs + tok, pitch, H);
+                    v[(size_t)q * 128u + (n - n0)] = glu(g, u, act);
+                }
+            }
+            for (uint32_t q = 0; q < cnt; q++) {
+                if (!rc.live[q]) continue;
+                float amax = 1e-10f;
+                for (uint32_t j = 0; j < n1 - n0; j++) amax = fmaxf(amax, fabsf(v[(size_t)q * 128u + j]));
+                const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
+                fs[(size_t)(r0 + q) * G + g0] = s;
+                for (uint32_t j = 0; j < n1 - n0; j++)
+                    fq[(size_t)(r0 + q) * I + n0 + j] = orc_f32_to_e4m3(v[(size_t)q * 128u + j] * inv);
+            }
+        }
+    }
+    free(wg); free(wu); free(v);
+    cache_free(&rc);
+}
+
+/* 86: t0=part t1=fu_g|fq t2=wtab t3=stab t4=meta t5=fs t6=row_partidx t7=row_gate  i0=H i1=I i2=E
+ * i3=enc i7=arm (2: f32 part, 3: bf16 part; enc 0/1 arm 0 and enc 2 arm 8: f32 part). */
+static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    const uint64_t* wtab = TEN(in, T, 2);
+    const uint64_t* stab = TEN(in, T, 3);
+    const int32_t* meta = TEN(in, T, 4);
+    const uint32_t* row_partidx = TEN(in, T, 6);
+    const float* row_gate = TEN(in, T, 7);
+    const uint32_t H = in->i[0], I = in->i[1], E = in->i[2], enc = in->i[3], arm = in->i[7];
+    const int w8a8 = enc == PLOW_MOE_ENC_FP8BLK &&
+                     (arm == PLOW_MOE_ARM_W8A8 || arm == PLOW_MOE_ARM_W8A8_P16);
+    const int part16 = w8a8 && arm == PLOW_MOE_ARM_W8A8_P16;
+    const float* fs = TEN(in, T, 5);
+    const uint32_t G = (H + 127u) / 128u, KB = (I + 127u) / 128u;
+    float* wd = malloc((size_t)I * 4u);
+    RowCache rc;
+    cache_init(&rc, I);
+    uint32_t lo, hi;
+    own_range(E * G, slice, nblk, &lo, &hi);
+    for (uint32_t it = lo; it < hi; it++) {
+        const uint32_t e = it / G, g0 = it % G;
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        const void* Wd = (const void*)(uintptr_t)wtab[(size_t)e * 3u + 2u];
+        if (cnt == 0u || !Wd) continue;
+        const void* Sd = stab ? (const void*)(uintptr_t)stab[(size_t)e * 3u + 2u] : NULL;
+        if (rc.expert != e) {
+            cache_fit(&rc, cnt);
+            for (uint32_t q = 0; q < cnt; q++) {
+                rc.live[q] = row_partidx[r0 + q] != PLOW_EXPERT_UNUSED;
+                if (!rc.live[q]) continue;
+                if (w8a8) decode_e4m3_row(rc.a + (size_t)q * I, (const uint8_t*)TEN(in, T, 1) + (size_t)(r0 + q) * I, I);
+                else decode_bf16_row(rc.a + (size_t)q * I, (const orc_bf16*)TEN(in, T, 1) + (size_t)(r0 + q) * I, I);
+            }
+            rc.expert = e;
+        }
+        const uint32_t h0 = g0 * 128u, h1 = h0 + 128u < H ? h0 + 128u : H;
+        for (uint32_t h = h0; h < h1; h++) {
+            RowScale rs = {NULL, NULL};
+            if (w8a8) decode_e4m3_row(wd, (const uint8_t*)Wd + (size_t)h * I, I);
+            else rs = enc_row(enc, Wd, Sd, h, I, wd);
+            for (uint32_t q = 0; q < cnt; q++) {
+                if (!rc.live[q]) continue;
+                const uint32_t r = r0 + q, pidx = row_partidx[r];
+                const float* a = rc.a + (size_t)q * I;
+                const float acc = w8a8 ? dot_fp8blk_a8(wd, (const float*)Sd + (size_t)g0 * KB, a,
+                                                       fs + (size_t)r * KB, 1u, I)
+                                       : enc_dot(enc, wd, rs, a, I);
+                const float val = row_gate[r] * acc;
+                if (part16) ((orc_bf16*)TEN(in, T, 0))[(size_t)pidx * H + h] = orc_f2bf(val);
+                else ((float*)TEN(in, T, 0))[(size_t)pidx * H + h] = val;
+            }
+        }
+    }
+    free(wd);
+    cache_free(&rc);
+}
+
+/* ---- ops 48 / 49: table-driven decode experts (slot-major) ------------------------------------- */
+
+/* 48: t0=fu[B*k][I] t1=x t2=table t3=wtab t4=stab  i0=slots i1=I i2=H i3=n_exp i4=slots per x row
+ * (0 = one shared row) i5=act i6=enc. Slot s reads x row s / i4. Sentinel or null base: nothing
+ * written. Slices split slots*I. */
+static void op_dec_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* fu = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    const PlowMoeRoute* tab = TEN(in, T, 2);
+    const uint64_t* wtab = TEN(in, T, 3);
+    const uint64_t* stab = TEN(in, T, 4);
+    const uint32_t nslot = in->i[0], I = in->i[1], H = in->i[2], E = in->i[3], kx = in->i[4];
+    const uint32_t act = in->i[5], enc = in->i[6];
+    float* a = malloc((size_t)H * 4u);
+    float* wg = malloc((size_t)H * 4u);
+    float* wu = malloc((size_t)H * 4u);
+    uint32_t lo, hi, cur = ~0u;
+    own_range(nslot * I, slice, nblk, &lo, &hi);
+    for (uint32_t it = lo; it < hi; it++) {
+        const uint32_t s = it / I, n = it % I, e = tab[s].eid;
+        if (e >= E || !wtab[(size_t)e * 3u]) continue;
+        const void* Wg = (const void*)(uintptr_t)wtab[(size_t)e * 3u + 0u];
+        const void* Wu = (const void*)(uintptr_t)wtab[(size_t)e * 3u + 1u];
+        const void* Sg = stab ? (const void*)(uintptr_t)stab[(size_t)e * 3u + 0u] : NULL;
+        const void* Su = stab ? (const void*)(uintptr_t)stab[(size_t)e * 3u + 1u] : NULL;
+        if (cur != s) { decode_bf16_row(a, x + (size_t)(kx ? s / kx : 0u) * H, H); cur = s; }
+        const RowScale sg = enc_row(enc, Wg, Sg, n, H, wg);
+        const RowScale su = enc_row(enc, Wu, Su, n, H, wu);
+        fu[(size_t)s * I + n] = orc_f2bf(glu(enc_dot(enc, wg, sg, a, H), enc_dot(enc, wu, su, a, H), act));
+    }
+    free(a); free(wg); free(wu);
+}
+
+/* 49: t0=part[B*k][H] t1=fu t2=table t3=wtab t4=stab  i0=slots i1=H i2=I i3=n_exp i6=enc.
+ * part[s] = gate_s * (Wd_e . fu[s]); sentinel or null base writes zeros. */
+static void op_dec_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    float* part = TEN(in, T, 0);
+    const orc_bf16* fu = TEN(in, T, 1);
+    const PlowMoeRoute* tab = TEN(in, T, 2);
+    const uint64_t* wtab = TEN(in, T, 3);
+    const uint64_t* stab = TEN(in, T, 4);
+    const uint32_t nslot = in->i[0], H = in->i[1], I = in->i[2], E = in->i[3], enc = in->i[6];
+    float* a = malloc((size_t)I * 4u);
+    float* wd = malloc((size_t)I * 4u);
+    uint32_t lo, hi, cur = ~0u;
+    own_range(nslot * H, slice, nblk, &lo, &hi);
+    for (uint32_t it = lo; it < hi; it++) {
+        const uint32_t s = it / H, h = it % H, e = tab[s].eid;
+        const void* Wd = e < E ? (const void*)(uintptr_t)wtab[(size_t)e * 3u + 2u] : NULL;
+        if (!Wd) { part[(size_t)s * H + h] = 0.0f; continue; }
+        const void* Sd = stab ? (const void*)(uintptr_t)stab[(size_t)e * 3u + 2u] : NULL;
+        if (cur != s) { decode_bf16_row(a, fu + (size_t)s * I, I); cur = s; }
+        const RowScale rs = enc_row(enc, Wd, Sd, h, I, wd);
+        part[(size_t)s * H + h] = tab[s].gate * enc_dot(enc, wd, rs, a, I);
+    }
+    free(a); free(wd);
+}
+
+/* ---- ops 65 / 66: per-output-channel fp8 decode experts ---------------------------------------- */
+
+/* 65: t0=fu t1=x t2=table t3=ewt[E][2] t4=est[E][2]  i0=k i1=I i2=H i3=E i5=B(0 = 1)
+ * i6 = activation (0 gelu_tanh, the only one the reference has; 1 silu).
+ * ewt[e][0] = fused gate_up rows [2I][H] (gate rows first); est[e][0] = f32 [2I]. */
+static void op_pc_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* fu = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    const PlowMoeRoute* tab = TEN(in, T, 2);
+    const uint64_t* ewt = TEN(in, T, 3);
+    const uint64_t* est = TEN(in, T, 4);
+    const uint32_t k = in->i[0], I = in->i[1], H = in->i[2], E = in->i[3];
+    const uint32_t rows = in->i[5] ? in->i[5] : 1u, act = in->i[6];
+    float* a = malloc((size_t)H * 4u);
+    float* wt = malloc((size_t)H * 4u);
+    uint32_t lo, hi;
+    own_range(rows * k, slice, nblk, &lo, &hi);
+    for (uint32_t s = lo; s < hi; s++) {
+        const uint32_t e = tab[s].eid;
+        if (e >= E || !ewt[2u * e] || !est[2u * e]) continue;
+        const uint8_t* w = (const uint8_t*)(uintptr_t)ewt[2u * e];
+        const float* sc = (const float*)(uintptr_t)est[2u * e];
+        decode_bf16_row(a, x + (size_t)(s / k) * H, H);
+        for (uint32_t n = 0; n < I; n++) {
+            decode_e4m3_row(wt, w + (size_t)n * H, H);
+            const float g = dot_seq(wt, a, H) * sc[n];
+            decode_e4m3_row(wt, w + (size_t)(I + n) * H, H);
+            const float u = dot_seq(wt, a, H) * sc[I + n];
+            fu[(size_t)s * I + n] = orc_f2bf(glu(g, u, act));
+        }
+    }
+    free(a); free(wt);
+}
+
+/* 66: t0=part t1=fu t2=table t3=ewt t4=est  i0=k i1=H i2=I i3=E i5=B. */
+static void op_pc_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    float* part = TEN(in, T, 0);
+    const orc_bf16* fu = TEN(in, T, 1);
+    const PlowMoeRoute* tab = TEN(in, T, 2);
+    const uint64_t* ewt = TEN(in, T, 3);
+    const uint64_t* est = TEN(in, T, 4);
+    const uint32_t k = in->i[0], H = in->i[1], I = in->i[2], E = in->i[3];
+    const uint32_t rows = in->i[5] ? in->i[5] : 1u;
+    float* a = malloc((size_t)I * 4u);
+    float* wt = malloc((size_t)I * 4u);
+    uint32_t lo, hi;
+    own_range(rows * k, slice, nblk, &lo, &hi);
+    for (uint32_t s = lo; s < hi; s++) {
+        const uint32_t e = tab[s].eid;
+        float* pr = part + (size_t)s * H;
+        if (e >= E || !ewt[2u * e + 1u] || !est[2u * e + 1u]) {
+            for (uint32_t h = 0; h < H; h++) pr[h] = 0.0f;
+            continue;
+        }
+        const uint8_t* w = (const uint8_t*)(uintptr_t)ewt[2u * e + 1u];
+        const float* sc = (const float*)(uintptr_t)est[2u * e + 1u];
+        decode_bf16_row(a, fu + (size_t)s * I, I);
+        for (uint32_t h = 0; h < H; h++) {
+            decode_e4m3_row(wt, w + (size_t)h * I, I);
+            pr[h] = tab[s].gate * (dot_seq(wt, a, I) * sc[h]);
+        }
+    }
+    free(a); free(wt);
+}
+
+/* ---- ops 81 / 82: grouped per-channel fp8 x per-row fp8 ---------------------------------------- */
+
+/* 81: t0=fu(bf16 [R][I]) t1=xq8([T][H]) t2=ewt t3=meta t4=row_token t5=ascale(f32 [T]) t6=est
+ *     i0=I i1=H i2=E i5=act. g = (sum_k xq.w) * (ascale[tok] * wsc[n]). */
+static void op_pc_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* fu = TEN(in, T, 0);
+    const uint8_t* xq = TEN(in, T, 1);
+    const uint64_t* ewt = TEN(in, T, 2);
+    const int32_t* meta = TEN(in, T, 3);
+    const uint32_t* row_token = TEN(in, T, 4);
+    const float* ascale = TEN(in, T, 5);
+    const uint64_t* est = TEN(in, T, 6);
+    const uint32_t I = in->i[0], H = in->i[1], E = in->i[2], act = in->i[5];
+    float* a = malloc((size_t)H * 4u);
+    float* wt = malloc((size_t)H * 4u);
+    uint32_t lo, hi;
+    own_range(E, slice, nblk, &lo, &hi);
+    for (uint32_t e = lo; e < hi; e++) {
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        if (cnt == 0u || !ewt[2u * e]) continue;
+        const uint8_t* w = (const uint8_t*)(uintptr_t)ewt[2u * e];
+        const float* sc = (const float*)(uintptr_t)est[2u * e];
+        for (uint32_t r = r0; r < r0 + cnt; r++) {
+            const uint32_t tok = row_token[r];
+            if (tok == PLOW_EXPERT_UNUSED) continue;
+            decode_e4m3_row(a, xq + (size_t)tok * H, H);
+            const float as = ascale[tok];
+            for (uint32_t n = 0; n < I; n++) {
+                decode_e4m3_row(wt, w + (size_t)n * H, H);
+                const float g = dot_seq(wt, a, H) * (as * sc[n]);
+                decode_e4m3_row(wt, w + (size_t)(I + n) * H, H);
+                const float u = dot_seq(wt, a, H) * (as * sc[I + n]);
+                fu[(size_t)r * I + n] = orc_f2bf(glu(g, u, act));
+            }
+        }
+    }
+    free(a); free(wt);
+}
+
+/* 82: t0=part t1=fu8([R][I]) t2=ewt t3=meta t4=row_partidx t5=row_gate t6=est t7=fscale(f32 [R])
+ *     i0=H i1=I i2=E. part = gate * acc * (fscale[r] * wsc[h]). */
+static void op_pc_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    float* part = TEN(in, T, 0);
+    const uint8_t* fu8 = TEN(in, T, 1);
+    const uint64_t* ewt = TEN(in, T, 2);
+    const int32_t* meta = TEN(in, T, 3);
+    const uint32_t* row_partidx = TEN(in, T, 4);
+    const float* row_gate = TEN(in, T, 5);
+    const uint64_t* est = TEN(in, T, 6);
+    const float* fscale = TEN(in, T, 7);
+    const uint32_t H = in->i[0], I = in->i[1], E = in->i[2];
+    float* a = malloc((size_t)I * 4u);
+    float* wt = malloc((size_t)I * 4u);
+    uint32_t lo, hi;
+    own_range(E, slice, nblk, &lo, &hi);
+    for (uint32_t e = lo; e < hi; e++) {
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        if (cnt == 0u || !ewt[2u * e + 1u]) continue;
+        const uint8_t* w = (const uint8_t*)(uintptr_t)ewt[2u * e + 1u];
+        const float* sc = (const float*)(uintptr_t)est[2u * e + 1u];
+        for (uint32_t r = r0; r < r0 + cnt; r++) {
+            const uint32_t pidx = row_partidx[r];
+            if (pidx == PLOW_EXPERT_UNUSED) continue;
+            decode_e4m3_row(a, fu8 + (size_t)r * I, I);
+            for (uint32_t h = 0; h < H; h++) {
+                decode_e4m3_row(wt, w + (size_t)h * I, I);
+                float y = row_gate[r] * dot_seq(wt, a, I);
+                y *= fscale[r] * sc[h];
+                part[(size_t)pidx * H + h] = y;
+            }
+        }
+    }
+    free(a); free(wt);
+}
+
+/* ---- ops 20 / 8: dense bf16 shared expert ------------------------------------------------------ */
+
+static float dot_bf16_seq(const orc_bf16* a, const orc_bf16* b, uint32_t K) {
+    float acc = 0.0f;
+    for (uint32_t k = 0; k < K; k++) acc = fmaf(orc_bf2f(a[k]), orc_bf2f(b[k]), acc);
+    return acc;
+}
+
+/* 20: t0=fu t1=x t2=W_gate t5=W_up  i0=M i1=N i2=K i5=act (biases t6/t7 are not on this path). */
+static void op_gemm_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* C = TEN(in, T, 0);
+    const orc_bf16* A = TEN(in, T, 1);
+    const orc_bf16* Wg = TEN(in, T, 2);
+    const orc_bf16* Wu = TEN(in, T, 5);
+    const uint32_t M = in->i[0], N = in->i[1], K = in->i[2], act = in->i[5];
+    uint32_t lo, hi;
+    own_range(N, slice, nblk, &lo, &hi);
+    for (uint32_t m = 0; m < M; m++)
+        for (uint32_t n = lo; n < hi; n++) {
+            const float g = dot_bf16_seq(A + (size_t)m * K, Wg + (size_t)n * K, K);
+            const float u = dot_bf16_seq(A + (size_t)m * K, Wu + (size_t)n * K, K);
+            C[(size_t)m * N + n] = orc_f2bf(glu(g, u, act));
+        }
+}
+
+/* 8: t0=C t1=A t2=B  i0=M i1=N i2=K i4=a_row0 i5=c_row0. */
+static void op_gemm(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    const uint32_t M = in->i[0], N = in->i[1], K = in->i[2];
+    orc_bf16* C = (orc_bf16*)TEN(in, T, 0) + (size_t)in->i[5] * N;
+    const orc_bf16* A = (const orc_bf16*)TEN(in, T, 1) + (size_t)in->i[4] * K;
+    const orc_bf16* B = TEN(in, T, 2);
+    uint32_t lo, hi;
+    own_range(N, slice, nblk, &lo, &hi);
+    for (uint32_t m = 0; m < M; m++)
+        for (uint32_t n = lo; n < hi; n++)
+            C[(size_t)m * N + n] = orc_f2bf(dot_bf16_seq(A + (size_t)m * K, B + (size_t)n * K, K));
+}
+
+/* ---- dispatch ---------------------------------------------------------------------------------- */
+
+typedef void (*op_fn)(const PlowDevInst*, uint32_t, uint32_t, void* const*);
+
+static op_fn resolve(uint16_t op) {
+    switch (op) {
+    case PLOW_DOP_GEMM_F32: return op_gemm_f32;
+    case PLOW_DOP_MOE_ROUTER_TOPK:
+    case PLOW_DOP_MOE_ROUTER_TOPK_PF: return op_router_topk;
+    case PLOW_DOP_MOE_ALIGN_PF: return op_align;
+    case PLOW_DOP_MOE_COMBINE:
+    case PLOW_DOP_MOE_COMBINE_PF: return op_combine;
+    case PLOW_DOP_QUANT_FP8_BLOCK128: return op_quant_block128;
+    case PLOW_DOP_QUANT_FP8: return op_quant_row;
+    case PLOW_DOP_MOE_GROUP_GLU_PF: return op_group_glu;
+    case PLOW_DOP_MOE_GROUP_DOWN_PF: return op_group_down;
+    case PLOW_DOP_MOE_GROUP_GLU_FP8_BLK: return op_dec_glu;
+    case PLOW_DOP_MOE_GROUP_DOWN_FP8_BLK: return op_dec_down;
+    case PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8: return op_pc_glu;
+    case PLOW_DOP_MOE_EXPERT_DOWN_GEMMA_FP8: return op_pc_down;
+    case PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF_W8A8: return op_pc_group_glu;
+    case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8: return op_pc_group_down;
+    case PLOW_DOP_GEMM_GLU: return op_gemm_glu;
+    case PLOW_DOP_GEMM: return op_gemm;
+    default: return NULL;
+    }
+}
+
+typedef struct {
+    op_fn fn;
+    const PlowDevInst* in;
+    void* const* T;
+    uint32_t slice, nblk;
+} Job;
+
+static void* job_main(void* p) {
+    Job* j = p;
+    j->fn(j->in, j->slice, j->nblk, j->T);
+    return NULL;
+}
+
+int plow_oracle_exec(const PlowDevInst* inst, void* const* tensors, uint32_t nthreads) {
+    op_fn fn = resolve(inst->op);
+    if (!fn) return PLOW_MOE_EUNSUPPORTED;
+    if (nthreads <= 1u) { fn(inst, 0u, 1u, tensors); return 0; }
+    if (nthreads > 256u) nthreads = 256u;
+    pthread_t th[256];
+    Job jobs[256];
+    for (uint32_t s = 0; s < nthreads; s++) {
+        jobs[s] = (Job){fn, inst, tensors, s, nthreads};
+        if (pthread_create(&th[s], NULL, job_main, &jobs[s]) != 0) {
+            for (uint32_t q = 0; q < s; q++) pthread_join(th[q], NULL);
+            return PLOW_MOE_ENOMEM;
+        }
+    }
+    for (uint32_t s = 0; s < nthreads; s++) pthread_join(th[s], NULL);
+    return 0;
+}
+
+int plow_oracle_exec_many(const PlowDevInst* insts, uint32_t n, void* const* tensors, uint32_t nthreads) {
+    for (uint32_t i = 0; i < n; i++) {
+        const int rc = plow_oracle_exec(&insts[i], tensors, nthreads);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+/* ---- codec exports for the tests --------------------------------------------------------------- */
+
+uint16_t plow_oracle_f2bf(float f) { return orc_f2bf(f); }
+float plow_oracle_bf2f(uint16_t h) { return orc_bf2f(h); }
+uint8_t plow_oracle_f32_to_e4m3(float f) { return orc_f32_to_e4m3(f); }
+float plow_oracle_e4m3_to_f32(uint8_t b) { return orc_e4m3_to_f32(b); }
+float plow_oracle_e2m1(uint8_t nib) { return orc_e2m1(nib); }
+float plow_oracle_e8m0(uint8_t s) { return orc_e8m0(s); }
+void plow_oracle_f2bf_n(uint16_t* dst, const float* src, size_t n) { for (size_t i = 0; i < n; i++) dst[i] = orc_f2bf(src[i]); }
+void plow_oracle_e4m3_encode_n(uint8_t* dst, const float* src, size_t n) { for (size_t i = 0; i < n; i++) dst[i] = orc_f32_to_e4m3(src[i]); }

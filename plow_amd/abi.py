@@ -1,0 +1,87 @@
+"""ctypes mirror of include/plow_moe.h: the 64-byte op descriptor, opcodes and enums.
+
+The descriptor is byte-identical to plow's ``PlowDevInst`` (runtime/common/dev_isa.h:1607-1613;
+Rust mirror ``DevInst64`` in crates/packet/src/dev.rs): ``u16 op, u16 blocks, PlowFJ fj[3],
+u16 t[8], u32 i[8]`` with ``t`` at byte 16.
+"""
+import ctypes as C
+
+TENSOR_NONE = 0xFFFF
+EXPERT_UNUSED = 0xFFFFFFFF
+MPF_BM = 64
+ROUTE_MAX_TOPK = 16
+
+# opcodes (runtime/common/dev_isa.h)
+OP_GEMM = 8
+OP_GEMM_GLU = 20
+OP_QUANT_FP8 = 32
+OP_MOE_COMBINE = 43
+OP_MOE_GROUP_GLU_FP8_BLK = 48
+OP_MOE_GROUP_DOWN_FP8_BLK = 49
+OP_MOE_ROUTER_TOPK = 56
+OP_MOE_EXPERT_GLU_GEMMA_FP8 = 65
+OP_MOE_EXPERT_DOWN_GEMMA_FP8 = 66
+OP_MOE_GROUP_GLU_GEMMA_PF_W8A8 = 81
+OP_MOE_GROUP_DOWN_GEMMA_PF_W8A8 = 82
+OP_MOE_ROUTER_TOPK_PF = 83
+OP_MOE_ALIGN_PF = 84
+OP_MOE_GROUP_GLU_PF = 85
+OP_MOE_GROUP_DOWN_PF = 86
+OP_MOE_COMBINE_PF = 87
+OP_GEMM_F32 = 180
+OP_QUANT_FP8_BLOCK128 = 184
+
+ENC_BF16, ENC_FP8BLK, ENC_MXFP4 = 0, 1, 2
+ARM_A16, ARM_W8A8, ARM_W8A8_P16, ARM_W4A16 = 0, 2, 3, 8
+ACT_GELU_TANH, ACT_SILU = 0, 1
+ROUTE_SIGMOID, ROUTE_NORM_TOPK, ROUTE_BIAS, ROUTE_F32_LOGIT = 1, 2, 4, 8
+
+E_OK, E_INVAL, E_UNSUPPORTED, E_DEVICE, E_NOMEM, ROLLBACK = 0, -22, -95, -5, -12, 1
+
+
+class PlowFJ(C.Union):
+    _fields_ = [("f", C.c_float), ("u", C.c_uint32)]
+
+
+class PlowDevInst(C.Structure):
+    _fields_ = [
+        ("op", C.c_uint16),
+        ("blocks", C.c_uint16),
+        ("fj", PlowFJ * 3),
+        ("t", C.c_uint16 * 8),
+        ("i", C.c_uint32 * 8),
+    ]
+
+
+assert C.sizeof(PlowDevInst) == 64 and PlowDevInst.t.offset == 16
+
+
+class PlowMoeRoute(C.Structure):
+    _fields_ = [("eid", C.c_uint32), ("gate", C.c_float)]
+
+
+def max_rows(T, k, n_exp):
+    """Capacity of the gathered arrays (runtime/amd/op_moe.h:2252-2255)."""
+    return T * k + n_exp * (MPF_BM - 1)
+
+
+def inst(op, t=(), i=(), f=(), blocks=1):
+    """Build one descriptor. ``t``: up to 8 handles (None = absent); ``i``: up to 8 ints;
+    ``f``: up to 3 floats placed in fj[n].f."""
+    d = PlowDevInst()
+    d.op, d.blocks = op, blocks
+    for n in range(8):
+        h = t[n] if n < len(t) else None
+        d.t[n] = TENSOR_NONE if h is None else int(h)
+    for n, v in enumerate(i):
+        d.i[n] = int(v) & 0xFFFFFFFF
+    for n, v in enumerate(f):
+        d.fj[n].f = float(v)
+    return d
+
+
+def inst_array(insts):
+    arr = (PlowDevInst * len(insts))()
+    for n, d in enumerate(insts):
+        C.memmove(C.byref(arr, n * 64), C.byref(d), 64)
+    return arr

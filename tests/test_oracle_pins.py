@@ -1,0 +1,467 @@
+"""Pins for the parts of the oracle that plow's CPU kernels cannot replay (tests/test_golden.py
+covers the rest): number formats, group-limited routing, the 1x128 activation quant and the
+block-fp8 arms. Each check is independent of the oracle's own formula: a closed form, a library
+routine (torch float8 / bfloat16 casts, integer matmul), brute force, or an invariant."""
+import numpy as np
+import pytest
+import torch
+
+import cases
+import oracle_lib as ol
+from plow_amd import abi
+
+
+def run(oracle, inst, arrays, nthreads=1):
+    ol.run(oracle.plow_oracle_exec, inst, ol.table_of(arrays), nthreads)
+
+
+# ---- number formats ------------------------------------------------------------------------------
+
+def test_bf16_round_matches_torch(oracle):
+    r = cases.rng_of(1)
+    v = np.concatenate([r.standard_normal(20000).astype(np.float32) * 10.0 ** r.integers(-20, 20, 20000),
+                        # exact ties and their neighbours around every rounding boundary
+                        (np.arange(0x3F800000, 0x3F800000 + 0x40000, 0x4000, dtype=np.uint32) + 0x8000).view(np.float32),
+                        (np.arange(0x3F800000, 0x3F800000 + 0x40000, 0x4000, dtype=np.uint32) + 0x7FFF).view(np.float32),
+                        np.array([0.0, -0.0, np.inf, -np.inf, 3.3895314e38, 1e-40], np.float32)]).astype(np.float32)
+    got = np.zeros(v.size, np.uint16)
+    oracle.plow_oracle_f2bf_n(got.ctypes.data, np.ascontiguousarray(v).ctypes.data, v.size)
+    want = torch.from_numpy(v).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+    assert np.array_equal(ol.f2bf(v), want)
+    nan = oracle.plow_oracle_f2bf(float("nan"))
+    assert (nan & 0x7F80) == 0x7F80 and (nan & 0x7F) != 0
+
+
+def test_e4m3_decode_table_matches_torch(oracle):
+    codes = np.arange(256, dtype=np.uint8)
+    want = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    got = np.array([oracle.plow_oracle_e4m3_to_f32(int(c)) for c in codes], np.float32)
+    fin = np.isfinite(want)
+    assert np.array_equal(got[fin].view(np.uint32), want[fin].view(np.uint32))
+    assert np.isnan(got[0x7F]) and np.isnan(got[0xFF]) and fin.sum() == 254
+    assert got[0x7E] == 448.0 and got[0x01] == 2.0 ** -9 and got[0x08] == 2.0 ** -6
+
+
+def test_e4m3_encode_is_nearest_even_by_brute_force(oracle):
+    codes = np.array([c for c in range(128) if c != 0x7F], np.uint8)
+    grid = np.array([oracle.plow_oracle_e4m3_to_f32(int(c)) for c in codes], np.float64)
+    r = cases.rng_of(2)
+    mids = (grid[:-1] + grid[1:]) / 2
+    v = np.concatenate([r.standard_normal(4000) * 10.0 ** r.integers(-4, 3, 4000), mids,
+                        np.nextafter(mids.astype(np.float32), np.float32(0)),
+                        np.nextafter(mids.astype(np.float32), np.float32(1e9)), grid,
+                        [447.9, 448.0, 463.9, 464.0, 1e9, 1e-12, 0.0]]).astype(np.float32)
+    v = np.concatenate([v, -v])
+    got = np.zeros(v.size, np.uint8)
+    oracle.plow_oracle_e4m3_encode_n(got.ctypes.data, np.ascontiguousarray(v).ctypes.data, v.size)
+    for x, c in zip(v, got):
+        a = abs(float(x))
+        if a >= 448.0:
+            want = 0x7E
+        else:
+            d = np.abs(grid - a)
+            best = np.flatnonzero(d == d.min())
+            want = int(codes[best[0]]) if len(best) == 1 else int(codes[[b for b in best if codes[b] % 2 == 0][0]])
+        assert (c & 0x7F) == want, (x, hex(c), hex(want))
+        assert (c >> 7) == (1 if np.signbit(x) else 0)
+    # the same answers from torch's cast wherever it is defined without saturation
+    inr = np.abs(v) < 448.0
+    tq = torch.from_numpy(v[inr]).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(tq, got[inr])
+    assert oracle.plow_oracle_f32_to_e4m3(float("nan")) & 0x7F == 0x7F
+    assert oracle.plow_oracle_f32_to_e4m3(float("inf")) == 0x7E
+
+
+def test_e2m1_and_e8m0_closed_forms(oracle):
+    mags = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    for n in range(16):
+        v = oracle.plow_oracle_e2m1(n)
+        assert abs(v) == mags[n & 7] and (np.signbit(v) == bool(n & 8))
+    assert oracle.plow_oracle_e8m0(0) == 0.0 and np.isinf(oracle.plow_oracle_e8m0(255))
+    for s in range(1, 255):
+        assert oracle.plow_oracle_e8m0(s) == 2.0 ** (s - 127)
+
+
+# ---- routing: closed forms and invariants --------------------------------------------------------
+
+def route(oracle, logit, bias, E, k, flags, **kw):
+    T = logit.shape[0]
+    tail = kw.get("tail", 0)
+    table = np.zeros(T * (k + tail), dtype=ol.ROUTE_DT)
+    run(oracle, cases.route_inst(E, k, T, flags, bias is not None, **kw), [table, logit, None, bias])
+    return table.reshape(T, k + tail)
+
+
+def test_all_equal_logits_pick_lowest_ids(oracle):
+    lg = np.full((3, 40), 0.25, np.float32)
+    for flags in (8, 8 | 1, 8 | 2):
+        tab = route(oracle, lg, None, 40, 6, flags, route_scale=1.0)
+        assert np.array_equal(tab["eid"], np.tile(np.arange(6, dtype=np.uint32), (3, 1)))
+
+
+def test_softmax_norm_gates_sum_to_scale(oracle):
+    lg = (cases.rng_of(3).standard_normal((50, 128)) * 3).astype(np.float32)
+    tab = route(oracle, lg, None, 128, 8, 8 | 2, route_scale=1.0)
+    assert np.allclose(tab["gate"].sum(1), 1.0, atol=1e-6)
+    tab = route(oracle, lg, None, 128, 8, 8 | 2, route_scale=2.5)
+    assert np.allclose(tab["gate"].sum(1), 2.5, atol=1e-5)
+
+
+def test_flat_selection_is_descending_argsort(oracle):
+    r = cases.rng_of(4)
+    for E, k in ((7, 3), (16, 16), (130, 8)):
+        lg = r.standard_normal((20, E)).astype(np.float32)
+        bias = (r.standard_normal(E) * 0.3).astype(np.float32)
+        tab = route(oracle, lg, bias, E, k, 8 | 1 | 4, route_scale=1.0)
+        score = (1.0 / (1.0 + np.exp(-lg.astype(np.float64)))).astype(np.float32)
+        sel = score + bias
+        for t in range(20):
+            order = sorted(range(E), key=lambda e: (-sel[t, e], e))[:k]
+            assert list(tab["eid"][t]) == order
+            # gates are the UNBIASED scores (to libm rounding), not the selection values
+            assert np.allclose(tab["gate"][t], score[t, order], rtol=1e-6)
+
+
+def test_logit_scale_and_shared_tail(oracle):
+    lg = (cases.rng_of(5).standard_normal((6, 32))).astype(np.float32)
+    a = route(oracle, lg * np.float32(0.5), None, 32, 4, 8 | 1)
+    b = route(oracle, lg, None, 32, 4, 8 | 1, logit_scale=0.5)
+    assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    c = route(oracle, lg * np.float32(0.5), None, 32, 4, 8 | 1, tail=1)
+    assert np.array_equal(c[:, :4].copy().view(np.uint8), a.view(np.uint8))
+    assert np.all(c["eid"][:, 4] == 32) and np.all(c["gate"][:, 4] == 1.0)
+
+
+def noaux_tc(score, bias, k, n_group, topk_group):
+    """Independent restatement of group-limited selection in the DeepSeek-V3 modelling code's terms:
+    mask whole groups, then a plain top-k over what is left."""
+    sel = score + bias
+    E = sel.shape[0]
+    gs = np.sort(sel.reshape(n_group, -1), axis=1)[:, -2:]
+    gscore = (gs[:, 1] + gs[:, 0]).astype(np.float32)      # m1 + m2 in f32
+    keep = sorted(range(n_group), key=lambda g: (-gscore[g], g))[:topk_group]
+    masked = np.full(E, -np.inf)
+    for g in keep:
+        lo = g * (E // n_group)
+        masked[lo:lo + E // n_group] = sel[lo:lo + E // n_group]
+    return sorted(range(E), key=lambda e: (-masked[e], e))[:k], set(keep)
+
+
+@pytest.mark.parametrize("E,k,ng,tg", [(256, 8, 8, 4), (64, 6, 4, 2), (128, 8, 8, 1), (288, 8, 18, 2)])
+def test_group_limited_selection(oracle, E, k, ng, tg):
+    r = cases.rng_of(6)
+    T = 40
+    lg = (r.standard_normal((T, E)) * 1.5).astype(np.float32)
+    bias = (r.standard_normal(E) * 0.1).astype(np.float32)
+    tab = route(oracle, lg, bias, E, k, 8 | 1 | 2 | 4, n_group=ng, topk_group=tg)
+    flat = route(oracle, lg, bias, E, k, 8 | 1 | 2 | 4)
+    # the scores the oracle used are those of the flat arm, which plow's CPU kernel pins bit for bit
+    score = np.zeros((T, E), np.float32)
+    full = route(oracle, lg, None, E, 16, 8 | 1, route_scale=1.0)  # probe: unbiased scores of top 16
+    differs = 0
+    for t in range(T):
+        sc = (1.0 / (1.0 + np.exp(-lg[t].astype(np.float64)))).astype(np.float32)
+        sc[full["eid"][t]] = full["gate"][t]            # exact libm bits where we have them
+        score[t] = sc
+        want, keep = noaux_tc(sc, bias, k, ng, tg)
+        got = list(tab["eid"][t])
+        assert {e // (E // ng) for e in got} <= keep    # every winner lies in a kept group
+        assert got == want
+        differs += got != list(flat["eid"][t])
+    assert differs > 0                                   # the mask really changes the selection
+    for off in ((1, 0), (0, 0), (ng, tg and ng)):        # inactive shapes are the flat arm exactly
+        same = route(oracle, lg, bias, E, k, 8 | 1 | 2 | 4, n_group=off[0], topk_group=off[1])
+        assert np.array_equal(same.view(np.uint8), flat.view(np.uint8))
+
+
+def test_align_structure(oracle):
+    r = cases.rng_of(7)
+    T, E, k = 200, 24, 4
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    for t in range(T):
+        tab["eid"][t * k:(t + 1) * k] = r.choice(E, k, replace=False)
+    tab["eid"][r.choice(T * k, 30, replace=False)] = abi.EXPERT_UNUSED
+    tab["gate"] = r.random(T * k).astype(np.float32)
+    al = cases.align_arrays(tab, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    meta, rt, rp, rg = al[0], al[2], al[3], al[4]
+    rowoff, cnt, tilep = meta[:E], meta[E:2 * E], meta[2 * E:]
+    live = tab["eid"] < E
+    assert cnt.sum() == live.sum()
+    assert np.array_equal(cnt, np.bincount(tab["eid"][live], minlength=E))
+    assert np.array_equal(rowoff, 64 * tilep[:E]) and tilep[E] == ((cnt + 63) // 64).sum()
+    for e in range(E):
+        seg = rp[rowoff[e]:rowoff[e] + cnt[e]]
+        assert np.array_equal(seg, np.flatnonzero(tab["eid"] == e))      # ascending slot order
+        assert np.array_equal(rt[rowoff[e]:rowoff[e] + cnt[e]], seg // k)
+        assert np.array_equal(rg[rowoff[e]:rowoff[e] + cnt[e]], tab["gate"][seg])
+        pad = slice(rowoff[e] + cnt[e], rowoff[e] + 64 * ((cnt[e] + 63) // 64))
+        assert np.all(rt[pad] == abi.EXPERT_UNUSED) and np.all(rp[pad] == abi.EXPERT_UNUSED)
+        assert np.all(rg[pad] == 0.0)
+
+
+# ---- 1x128 activation quant ----------------------------------------------------------------------
+
+def test_quant_block128_closed_form(oracle):
+    r = cases.rng_of(8)
+    M, K, pitch = 5, 384, 9
+    x = cases.randn_bf16(r, (M, K), 2.0)
+    x[2, 128:256] = 0                                   # all-zero group: amax floor 1e-10
+    xq, xs = np.zeros((M, K), np.uint8), np.full((K // 128, pitch), -1.0, np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[M, K, pitch]), [xq, x, xs], 2)
+    xf = ol.bf2f(x).reshape(M, K // 128, 128)
+    amax = np.maximum(np.abs(xf).max(2), np.float32(1e-10))
+    s = (amax * np.float32(1.0 / 448.0)).astype(np.float32)
+    assert np.array_equal(xs[:, :M].T.view(np.uint32), s.view(np.uint32)) and np.all(xs[:, M:] == -1.0)
+    inv = (np.float32(1.0) / s).astype(np.float32)
+    want = torch.from_numpy((xf * inv[:, :, None]).astype(np.float32).clip(-448, 448)).to(
+        torch.float8_e4m3fn).view(torch.uint8).numpy().reshape(M, K)
+    assert np.array_equal(xq, want)
+    # decode(q) * s reproduces x to within half an e4m3 step of the group's amax
+    deq = torch.from_numpy(xq).view(torch.float8_e4m3fn).float().numpy().reshape(M, K // 128, 128) * s[:, :, None]
+    assert np.all(np.abs(deq - xf) <= amax[:, :, None] * (0.0625 / 1.75 + 1e-6))
+
+
+# ---- block-fp8 experts ----------------------------------------------------------------------------
+
+def identity_align(T, E_of_row, E):
+    """Row maps for hand-made segments: token t is routed (k = 1) to expert E_of_row[t]."""
+    tab = np.zeros(T, dtype=ol.ROUTE_DT)
+    tab["eid"], tab["gate"] = E_of_row, 1.0
+    return tab
+
+
+def build_fp8(oracle, r, E, T, H, I, small_int, scales_one):
+    """Tiny block-fp8 layer, k = 1. small_int: payloads are the integers -3..3 (exact in e4m3)."""
+    def payload(shape):
+        if small_int:
+            v = r.integers(-3, 4, size=shape).astype(np.float32)
+            b = np.zeros(v.size, np.uint8)
+            oracle.plow_oracle_e4m3_encode_n(b.ctypes.data, np.ascontiguousarray(v).ctypes.data, v.size)
+            return b.reshape(shape), v
+        b = cases.e4m3_bytes(r, shape)
+        v = torch.from_numpy(b).view(torch.float8_e4m3fn).float().numpy()
+        return b, v
+    W = {n: [payload(s) for _ in range(E)] for n, s in (("g", (I, H)), ("u", (I, H)), ("d", (H, I)))}
+    def grid(N, K):
+        g = np.ones((N // 128, K // 128), np.float32)
+        return g if scales_one else (r.random(g.shape) * 0.02 + 0.001).astype(np.float32)
+    S = {n: [grid(*s) for _ in range(E)] for n, s in (("g", (I, H)), ("u", (I, H)), ("d", (H, I)))}
+    wtab = np.array([[W[n][e][0].ctypes.data for n in "gud"] for e in range(E)], dtype=np.uint64)
+    stab = np.array([[S[n][e].ctypes.data for n in "gud"] for e in range(E)], dtype=np.uint64)
+    return W, S, wtab, stab
+
+
+def dequant(Wv, S):
+    return Wv.astype(np.float64) * np.kron(S.astype(np.float64), np.ones((128, 128)))
+
+
+@pytest.mark.parametrize("arm", [abi.ARM_A16, abi.ARM_W8A8])
+def test_fp8blk_unit_scales_small_integers_is_exact_integer_gemm(oracle, arm):
+    """All scales 1 and integer payloads: every partial sum is an integer below 2^24, so the DOWN
+    arm must equal an integer matmul exactly, whatever the summation order."""
+    r = cases.rng_of(9)
+    E, T, H, I = 3, 7, 256, 128
+    W, S, wtab, stab = build_fp8(oracle, r, E, T, H, I, True, True)
+    eids = r.integers(0, E, T).astype(np.uint32)
+    tab = identity_align(T, eids, E)
+    tab["gate"] = r.integers(1, 4, T).astype(np.float32)
+    al = cases.align_arrays(tab, T, E, 1)
+    run(oracle, cases.align_inst(T, E, 1), al)
+    R = al[2].shape[0]
+    fi = r.integers(-3, 4, size=(R, I)).astype(np.float32)
+    part = np.zeros((T, H), np.float32)
+    if arm == abi.ARM_A16:
+        fu = ol.f2bf(fi)
+        run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, None, 6, 7], i=[H, I, E, 1, 0, 0, 0, 0]),
+            [part, fu, wtab, stab, al[0], None, al[3], al[4]], 2)
+    else:
+        fq = np.zeros(fi.size, np.uint8)
+        oracle.plow_oracle_e4m3_encode_n(fq.ctypes.data, np.ascontiguousarray(fi).ctypes.data, fi.size)
+        fs = np.ones((R, I // 128), np.float32)
+        run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[H, I, E, 1, 0, 0, 0, 2]),
+            [part, fq.reshape(R, I), wtab, stab, al[0], fs, al[3], al[4]], 2)
+    for row in range(int(al[0][-1]) * 64):
+        t = al[3][row]
+        if t == abi.EXPERT_UNUSED:
+            continue
+        e = eids[t]
+        want = tab["gate"][t] * (W["d"][e][1].astype(np.int64) @ fi[row].astype(np.int64))
+        assert np.array_equal(part[t], want.astype(np.float32))
+
+
+def test_fp8blk_one_hot_activation_reads_back_a_dequantized_column(oracle):
+    r = cases.rng_of(10)
+    E, H, I = 2, 256, 128
+    W, S, wtab, stab = build_fp8(oracle, r, E, 4, H, I, False, False)
+    T = 4
+    hot = [3, 130, 200, 255]
+    x = np.zeros((T, H), np.float32)
+    x[np.arange(T), hot] = 1.0
+    eids = np.array([0, 1, 1, 0], np.uint32)
+    tab = identity_align(T, eids, E)
+    al = cases.align_arrays(tab, T, E, 1)
+    run(oracle, cases.align_inst(T, E, 1), al)
+    R = al[2].shape[0]
+    part = np.zeros((T, I), np.float32)
+    # use the GATE matrix as a "down" matrix of shape [I][H] so that the output is its column
+    wt2 = wtab.copy(); st2 = stab.copy()
+    wt2[:, 2], st2[:, 2] = wtab[:, 0], stab[:, 0]
+    xr = np.zeros((R, H), np.uint16)
+    for row in range(int(al[0][-1]) * 64):
+        if al[3][row] != abi.EXPERT_UNUSED:
+            xr[row] = ol.f2bf(x[al[3][row]])
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, None, 6, 7], i=[I, H, E, 1, 0, 0, 0, 0]),
+        [part, xr, wt2, st2, al[0], None, al[3], al[4]])
+    for t in range(T):
+        col = dequant(W["g"][eids[t]][1], S["g"][eids[t]])[:, hot[t]]
+        assert np.array_equal(part[t], col.astype(np.float32))
+
+
+@pytest.mark.parametrize("arm", [abi.ARM_A16, abi.ARM_W8A8])
+def test_fp8blk_layer_against_f64_over_the_same_bytes(oracle, arm):
+    """GLU -> DOWN at a small shape vs an f64 evaluation of the same quantized operands. The W8A8 arm
+    re-derives its own intermediate quantization from the oracle's fq / fs (so that only the GEMM
+    arithmetic is under test here; the quant rule is pinned above)."""
+    r = cases.rng_of(11)
+    E, T, H, I, k = 4, 9, 256, 256, 2
+    W, S, wtab, stab = build_fp8(oracle, r, E, T, H, I, False, False)
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    for t in range(T):
+        tab["eid"][t * k:(t + 1) * k] = r.choice(E, k, replace=False)
+    tab["gate"] = (r.random(T * k) + 0.1).astype(np.float32)
+    al = cases.align_arrays(tab, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    R = al[2].shape[0]
+    x = cases.randn_bf16(r, (T, H), 1.0)
+    part = np.zeros((T * k, H), np.float32)
+    silu = lambda g: g / (1.0 + np.exp(-g))
+    if arm == abi.ARM_A16:
+        fu = np.zeros((R, I), np.uint16)
+        run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5], i=[I, H, E, 1, 0, 1, 0, 0]),
+            [fu, x, wtab, stab, al[0], al[2]], 2)
+        run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, None, 6, 7], i=[H, I, E, 1, 0, 0, 0, 0]),
+            [part, fu, wtab, stab, al[0], None, al[3], al[4]], 2)
+        xa = ol.bf2f(x).astype(np.float64)
+        fa = ol.bf2f(fu).astype(np.float64)
+    else:
+        xq, xs = np.zeros((T, H), np.uint8), np.zeros((H // 128, T), np.float32)
+        run(oracle, abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[T, H, T]), [xq, x, xs])
+        fq, fs = np.zeros((R, I), np.uint8), np.zeros((R, I // 128), np.float32)
+        run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[I, H, E, 1, T, 1, 0, 2]),
+            [fq, xq, wtab, stab, al[0], al[2], xs, fs], 2)
+        run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[H, I, E, 1, 0, 0, 0, 2]),
+            [part, fq, wtab, stab, al[0], fs, al[3], al[4]], 2)
+        xa = torch.from_numpy(xq).view(torch.float8_e4m3fn).double().numpy() * np.repeat(xs.T.astype(np.float64), 128, axis=1)
+        fa = torch.from_numpy(fq).view(torch.float8_e4m3fn).double().numpy() * np.repeat(fs.astype(np.float64), 128, axis=1)
+    for row in range(int(al[0][-1]) * 64):
+        s = al[3][row]
+        if s == abi.EXPERT_UNUSED:
+            continue
+        e, t = tab["eid"][s], s // k
+        g = dequant(W["g"][e][1], S["g"][e]) @ xa[t]
+        u = dequant(W["u"][e][1], S["u"][e]) @ xa[t]
+        v = silu(g) * u
+        # the stored intermediate (bf16, or e4m3 x scale) is the f64 value to format precision
+        tol = 2.0 ** -8 if arm == abi.ARM_A16 else 2.0 ** -4
+        assert np.all(np.abs(fa[row] - v) <= tol * np.abs(v).max() + 1e-6)
+        y = tab["gate"][s] * (dequant(W["d"][e][1], S["d"][e]) @ fa[row])
+        assert np.allclose(part[s], y, rtol=2e-5, atol=2e-5 * np.abs(y).max())
+
+
+def test_fp8blk_constant_block_scale_factors_out(oracle):
+    """A constant scale grid c equals c times the unit-scale result (c a power of two: exactly)."""
+    r = cases.rng_of(12)
+    E, T, H, I = 2, 5, 256, 128
+    W, S, wtab, stab = build_fp8(oracle, r, E, T, H, I, False, True)
+    tab = identity_align(T, r.integers(0, E, T).astype(np.uint32), E)
+    al = cases.align_arrays(tab, T, E, 1)
+    run(oracle, cases.align_inst(T, E, 1), al)
+    R = al[2].shape[0]
+    fu = cases.randn_bf16(r, (R, I), 1.0)
+    outs = []
+    for c in (1.0, 0.25):
+        for e in range(E):
+            S["d"][e][:] = c
+        part = np.zeros((T, H), np.float32)
+        run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, None, 6, 7], i=[H, I, E, 1, 0, 0, 0, 0]),
+            [part, fu, wtab, stab, al[0], None, al[3], al[4]])
+        outs.append(part)
+    assert np.array_equal(outs[1], outs[0] * np.float32(0.25))
+
+
+def test_mxfp4_grouped_arm_equals_decode_arm(oracle):
+    """Ops 85/86 at enc 2 / arm 8 are the arithmetic of the decode ops 48/49 (pinned by plow's flat
+    mxfp4 kernels in tests/test_golden.py) applied to gathered rows: same bits, row for row."""
+    r = cases.rng_of(13)
+    E, T, H, I, k = 5, 6, 128, 64, 2
+    Wg, Wu = [r.integers(0, 256, (I, H // 2), dtype=np.uint8) for _ in range(E)], [r.integers(0, 256, (I, H // 2), dtype=np.uint8) for _ in range(E)]
+    Wd = [r.integers(0, 256, (H, I // 2), dtype=np.uint8) for _ in range(E)]
+    Sg, Su = [r.integers(120, 128, (I, H // 32), dtype=np.uint8) for _ in range(E)], [r.integers(120, 128, (I, H // 32), dtype=np.uint8) for _ in range(E)]
+    Sd = [r.integers(120, 128, (H, I // 32), dtype=np.uint8) for _ in range(E)]
+    wtab = np.array([[Wg[e].ctypes.data, Wu[e].ctypes.data, Wd[e].ctypes.data] for e in range(E)], dtype=np.uint64)
+    stab = np.array([[Sg[e].ctypes.data, Su[e].ctypes.data, Sd[e].ctypes.data] for e in range(E)], dtype=np.uint64)
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    for t in range(T):
+        tab["eid"][t * k:(t + 1) * k] = r.choice(E, k, replace=False)
+    tab["gate"] = r.random(T * k).astype(np.float32)
+    x = cases.randn_bf16(r, (T, H), 1.0)
+    fu_d = np.zeros((T * k, I), np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_FP8_BLK, t=[0, 1, 2, 3, 4], i=[T * k, I, H, E, k, 1, 2]), [fu_d, x, tab, wtab, stab])
+    part_d = np.zeros((T * k, H), np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_FP8_BLK, t=[0, 1, 2, 3, 4], i=[T * k, H, I, E, 0, 0, 2]), [part_d, fu_d, tab, wtab, stab])
+    al = cases.align_arrays(tab, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    R = al[2].shape[0]
+    fu_g = np.zeros((R, I), np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5], i=[I, H, E, 2, 0, 1, 0, 8]), [fu_g, x, wtab, stab, al[0], al[2]], 2)
+    part_g = np.zeros((T * k, H), np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, None, 6, 7], i=[H, I, E, 2, 0, 0, 0, 8]),
+        [part_g, fu_g, wtab, stab, al[0], None, al[3], al[4]], 2)
+    for row in range(int(al[0][-1]) * 64):
+        if al[3][row] != abi.EXPERT_UNUSED:
+            assert np.array_equal(fu_g[row], fu_d[al[3][row]])
+    assert np.array_equal(part_g.view(np.uint32), part_d.view(np.uint32))
+
+
+def test_per_channel_w8a8_against_f64(oracle):
+    """Ops 32 -> 81 -> 32 -> 82 vs f64 over the same quantized bytes (sequential-sum f32 arithmetic,
+    as the reference's own GPU test checks them: runtime/tests/moe_gemma_gfx950_test.c:1140-1200)."""
+    r = cases.rng_of(14)
+    E, T, H, I, k = 3, 8, 128, 64, 2
+    gu8 = [cases.e4m3_bytes(r, (2 * I, H)) for _ in range(E)]
+    d8 = [cases.e4m3_bytes(r, (H, I)) for _ in range(E)]
+    sgu = [(r.random(2 * I) * 0.01 + 1e-3).astype(np.float32) for _ in range(E)]
+    sd = [(r.random(H) * 0.01 + 1e-3).astype(np.float32) for _ in range(E)]
+    ewt = np.array([[a.ctypes.data, b.ctypes.data] for a, b in zip(gu8, d8)], dtype=np.uint64)
+    est = np.array([[a.ctypes.data, b.ctypes.data] for a, b in zip(sgu, sd)], dtype=np.uint64)
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    for t in range(T):
+        tab["eid"][t * k:(t + 1) * k] = r.choice(E, k, replace=False)
+    tab["gate"] = (r.random(T * k) + 0.1).astype(np.float32)
+    al = cases.align_arrays(tab, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    R = al[2].shape[0]
+    x = cases.randn_bf16(r, (T, H), 1.0)
+    xq, asc = np.zeros((T, H), np.uint8), np.zeros(T, np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8, t=[0, 1, 2], i=[T, H]), [xq, x, asc])
+    fu = np.zeros((R, I), np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_GEMMA_PF_W8A8, t=[0, 1, 2, 3, 4, 5, 6], i=[I, H, E, 0, 0, 1]),
+        [fu, xq, ewt, al[0], al[2], asc, est], 2)
+    fu8, fsc = np.zeros((R, I), np.uint8), np.zeros(R, np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8, t=[0, 1, 2], i=[R, I]), [fu8, fu, fsc])
+    part = np.zeros((T * k, H), np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_GEMMA_PF_W8A8, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[H, I, E]),
+        [part, fu8, ewt, al[0], al[3], al[4], est, fsc], 2)
+    dec = lambda b: torch.from_numpy(np.ascontiguousarray(b)).view(torch.float8_e4m3fn).double().numpy()
+    for row in range(int(al[0][-1]) * 64):
+        s = al[3][row]
+        if s == abi.EXPERT_UNUSED:
+            continue
+        e, t = tab["eid"][s], s // k
+        gu = (dec(gu8[e]) @ dec(xq[t])) * asc[t] * sgu[e]
+        v = gu[:I] / (1 + np.exp(-gu[:I])) * gu[I:]
+        assert np.all(np.abs(ol.bf2f(fu[row]) - v) <= 2.0 ** -8 * np.abs(v) + 1e-7)
+        y = tab["gate"][s] * ((dec(d8[e]) @ dec(fu8[row])) * fsc[row] * sd[e])
+        assert np.allclose(part[s], y, rtol=1e-5, atol=1e-6)
