@@ -290,8 +290,10 @@ static void op_quant_row(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
 static void decode_bf16_row(float* dst, const orc_bf16* src, uint32_t K) {
     for (uint32_t k = 0; k < K; k++) dst[k] = orc_bf2f(src[k]);
 }
+static float e4m3_lut[256]; /* orc_e4m3_to_f32 of every code, filled once by plow_oracle_exec */
+static int e4m3_lut_ready;
 static void decode_e4m3_row(float* dst, const uint8_t* src, uint32_t K) {
-    for (uint32_t k = 0; k < K; k++) dst[k] = orc_e4m3_to_f32(src[k]);
+    for (uint32_t k = 0; k < K; k++) dst[k] = e4m3_lut[src[k]];
 }
 static void decode_mxfp4_row(float* dst, const uint8_t* src, uint32_t K) {
     for (uint32_t k = 0; k < K; k++) dst[k] = orc_mxfp4_at(src, k);
@@ -819,6 +821,10 @@ static void* job_main(void* p) {
 int plow_oracle_exec(const PlowDevInst* inst, void* const* tensors, uint32_t nthreads) {
     op_fn fn = resolve(inst->op);
     if (!fn) return PLOW_MOE_EUNSUPPORTED;
+    if (!e4m3_lut_ready) {
+        for (int b = 0; b < 256; b++) e4m3_lut[b] = orc_e4m3_to_f32((uint8_t)b);
+        e4m3_lut_ready = 1;
+    }
     if (nthreads <= 1u) { fn(inst, 0u, 1u, tensors); return 0; }
     if (nthreads > 256u) nthreads = 256u;
     pthread_t th[256];

@@ -1,0 +1,57 @@
+"""Builds the operator library ``plow_amd/libplow_moe_gfx950.so`` from ``plow_amd/csrc`` with hipcc.
+
+gfx950 (MI355X, CDNA4) only. hipcc cross-compiles without a GPU, so this runs anywhere the ROCm
+toolchain is installed. ``python -m plow_amd.build`` rebuilds unconditionally.
+"""
+import concurrent.futures as cf
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "libplow_moe_gfx950.so")
+
+COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-fast-math",
+          # packed-FP32 VALU forms are kept out of every kernel
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# Translation units whose floating-point results must match the CPU reference bit for bit are built
+# without multiply-add contraction.
+SOURCES = {
+    "route.hip": ["-ffp-contract=off"],
+    "quant.hip": ["-ffp-contract=off"],
+    "experts_w8a8.hip": [],
+    "api.hip": [],
+}
+
+
+def _compile(src, extra):
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    cmd = ["hipcc", *COMMON, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "not a recognized feature" not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    return obj, err
+
+
+def build(verbose=True):
+    os.makedirs(OBJ, exist_ok=True)
+    with cf.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
+        results = list(ex.map(lambda kv: _compile(*kv), SOURCES.items()))
+    objs = [o for o, _ in results]
+    for _, err in results:
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

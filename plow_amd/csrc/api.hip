@@ -1,0 +1,283 @@
+/* api.hip — the C-ABI of the operator (include/plow_moe.h): context, descriptor validation and the
+ * op -> kernel dispatch. Host code only; the kernels live in the other translation units.
+ *
+ * The validation mirrors what plow's host does before it launches a native MoE segment: typed refusal
+ * of wrong wiring or geometry before anything is enqueued (crates/plowrt/src/exec/gpu/moe_lt.rs:
+ * 159-248, crates/plowrt/src/exec/amd.rs:3450-3480). */
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "../../include/plow_moe.h"
+#include "kernels.h"
+
+struct PlowMoeCtx {
+    int device;
+    int min_rows[2]; /* [0] prefill, [1] decode; < 0 unset */
+    char err[256];
+};
+
+static int fail(PlowMoeCtx* c, int code, const char* fmt, ...) {
+    if (c) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(c->err, sizeof c->err, fmt, ap);
+        va_end(ap);
+    }
+    return code;
+}
+
+static inline void* ten(const PlowDevInst* in, void* const* T, int k) {
+    return in->t[k] == PLOW_TENSOR_NONE ? nullptr : T[in->t[k]];
+}
+
+extern "C" uint32_t plow_moe_abi(void) { return 1u; }
+
+extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
+    if (!out) return PLOW_MOE_EINVAL;
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) return PLOW_MOE_EDEVICE;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return PLOW_MOE_EDEVICE;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return PLOW_MOE_EUNSUPPORTED; /* CDNA4 only */
+    PlowMoeCtx* c = new (std::nothrow) PlowMoeCtx();
+    if (!c) return PLOW_MOE_ENOMEM;
+    c->device = device;
+    c->min_rows[0] = c->min_rows[1] = -1;
+    c->err[0] = 0;
+    *out = c;
+    return 0;
+}
+
+extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) { delete ctx; }
+
+extern "C" const char* plow_moe_last_error(const PlowMoeCtx* ctx) { return ctx ? ctx->err : "no context"; }
+
+extern "C" int plow_moe_set_min_rows(PlowMoeCtx* ctx, int variant, int min_rows) {
+    if (!ctx || variant < 0 || variant > 1) return PLOW_MOE_EINVAL;
+    ctx->min_rows[variant] = min_rows;
+    return 0;
+}
+
+/* ---- per-op validation + launch --------------------------------------------------------------- */
+
+#define NEED(c, cond, ...) \
+    do { if (!(cond)) return fail(c, PLOW_MOE_EINVAL, __VA_ARGS__); } while (0)
+
+static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStream_t st, bool launch) {
+    const uint32_t* i = in->i;
+    switch (in->op) {
+    case PLOW_DOP_GEMM_F32: {
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2), "op 180: t0 logits, t1 x, t2 W must be bound");
+        NEED(c, i[0] && i[1] && i[2] && i[2] % 8u == 0u, "op 180: M, N, K must be non-zero and K a multiple of 8");
+        if (!launch) return 0;
+        return launch_router_score((float*)ten(in, T, 0), ten(in, T, 1), ten(in, T, 2), i[0], i[1], i[2], st);
+    }
+    case PLOW_DOP_MOE_ROUTER_TOPK:
+    case PLOW_DOP_MOE_ROUTER_TOPK_PF: {
+        const bool pf = in->op == PLOW_DOP_MOE_ROUTER_TOPK_PF;
+        const uint32_t E = i[1], k = i[2], flags = i[3], rows = i[4] ? i[4] : 1u;
+        NEED(c, ten(in, T, 0) && ten(in, T, 1), "router top-k: t0 table and t1 logits must be bound");
+        NEED(c, E >= 1u && E <= 1024u, "router top-k: n_exp %u outside 1..1024", E);
+        NEED(c, k >= 1u, "router top-k: k = 0");
+        /* the bias operand is read by the GPU reference only under flag bit 2 and by the CPU reference
+         * whenever it is bound: a packet where the two disagree is ambiguous and refused */
+        NEED(c, ((flags & PLOW_ROUTE_BIAS) != 0u) == (ten(in, T, 3) != nullptr),
+             "router top-k: bias flag (bit 2) and the t3 binding disagree");
+        if (i[6] > 1u && i[7] > 0u && i[7] < i[6])
+            NEED(c, i[6] <= PLOW_ROUTE_MAX_GROUPS && E % i[6] == 0u && E / i[6] >= 2u &&
+                        (uint64_t)i[7] * (E / i[6]) >= (k < 16u ? k : 16u),
+                 "router top-k: group shape n_group=%u topk_group=%u is not selectable for n_exp=%u k=%u",
+                 i[6], i[7], E, k);
+        if (!launch) return 0;
+        return launch_router_topk(ten(in, T, 0), ten(in, T, 1), (const float*)ten(in, T, 3), E, k, flags,
+                                  rows, pf && i[5] ? 1u : 0u, i[6], i[7], in->fj[0].f, in->fj[1].f, st);
+    }
+    case PLOW_DOP_MOE_ALIGN_PF: {
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4),
+             "op 84: t0 meta, t1 table, t2 row_token, t3 row_partidx, t4 row_gate must be bound");
+        NEED(c, i[1] >= 1u && i[1] <= 1056u && i[2] >= 1u, "op 84: n_exp %u outside 1..1056 or k = 0", i[1]);
+        NEED(c, (uint64_t)i[0] * i[2] < (1ull << 31), "op 84: T * k overflows");
+        if (!launch) return 0;
+        return launch_align((int32_t*)ten(in, T, 0), ten(in, T, 1), (uint32_t*)ten(in, T, 2),
+                            (uint32_t*)ten(in, T, 3), (float*)ten(in, T, 4), i[0], i[1], i[2], st);
+    }
+    case PLOW_DOP_MOE_COMBINE:
+    case PLOW_DOP_MOE_COMBINE_PF: {
+        const bool pf = in->op == PLOW_DOP_MOE_COMBINE_PF;
+        const uint32_t H = i[0], k = i[1], rows = pf ? (i[2] ? i[2] : 1u) : 1u;
+        const size_t r0 = pf ? i[3] : 0u;
+        const uint32_t p16 = pf && i[7] ? 1u : 0u;
+        NEED(c, ten(in, T, 0) && ten(in, T, 3), "combine: t0 out and t3 part must be bound");
+        NEED(c, H && H % 4u == 0u, "combine: H %u must be a non-zero multiple of 4", H);
+        if (!launch) return 0;
+        const char* res = (const char*)ten(in, T, 1);
+        const char* sh = (const char*)ten(in, T, 2);
+        return launch_combine((char*)ten(in, T, 0) + r0 * H * 2u, res ? res + r0 * H * 2u : nullptr,
+                              sh ? sh + r0 * H * 2u : nullptr,
+                              (const char*)ten(in, T, 3) + r0 * k * H * (p16 ? 2u : 4u), H, k, rows, p16, st);
+    }
+    case PLOW_DOP_QUANT_FP8_BLOCK128: {
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2), "op 184: t0 xq, t1 x, t2 scale must be bound");
+        NEED(c, i[0] && i[1] && i[1] % 128u == 0u, "op 184: K %u must be a non-zero multiple of 128", i[1]);
+        NEED(c, i[2] == 0u || i[2] >= i[0], "op 184: scale pitch %u below M %u", i[2], i[0]);
+        if (!launch) return 0;
+        return launch_quant_block128(ten(in, T, 0), ten(in, T, 1), (float*)ten(in, T, 2), i[0], i[1], i[2], st);
+    }
+    case PLOW_DOP_QUANT_FP8: {
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2), "op 32: t0 xq, t1 x, t2 scale must be bound");
+        NEED(c, !ten(in, T, 3) && !ten(in, T, 4), "op 32: the fused gate/up arm (t3/t4) is not on this path");
+        NEED(c, i[0] && i[1] && i[1] % 8u == 0u, "op 32: K %u must be a non-zero multiple of 8", i[1]);
+        if (!launch) return 0;
+        return launch_quant_row(ten(in, T, 0), ten(in, T, 1), (float*)ten(in, T, 2), i[0], i[1], st);
+    }
+    case PLOW_DOP_MOE_GROUP_GLU_PF: {
+        const uint32_t I = i[0], H = i[1], E = i[2], enc = i[3], arm = i[7];
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 4) && ten(in, T, 5),
+             "op 85: t0 fu, t1 x, t2 wtab, t4 meta, t5 row_token must be bound");
+        NEED(c, I && H && E, "op 85: zero geometry");
+        if (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8) {
+            NEED(c, ten(in, T, 3) && ten(in, T, 6) && ten(in, T, 7), "op 85 W8A8: t3 stab, t6 xs, t7 fs must be bound");
+            NEED(c, I % 128u == 0u && H % 128u == 0u, "op 85 W8A8: I %u and H %u must be multiples of 128", I, H);
+            NEED(c, i[4] != 0u, "op 85 W8A8: i4 (row pitch of the activation scales) is zero");
+            NEED(c, i[5] <= 1u, "op 85: activation %u is not served", i[5]);
+            if (!launch) return 0;
+            GroupW8A8 g = {};
+            g.out = ten(in, T, 0); g.out_scale = (float*)ten(in, T, 7);
+            g.a = ten(in, T, 1); g.a_scale = (const float*)ten(in, T, 6);
+            g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 3);
+            g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
+            g.N = I; g.K = H; g.E = E; g.pitch = i[4]; g.act = i[5];
+            return launch_group_glu_w8a8(g, st);
+        }
+        return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85: encoding %u arm %u is not served", enc, arm);
+    }
+    case PLOW_DOP_MOE_GROUP_DOWN_PF: {
+        const uint32_t H = i[0], I = i[1], E = i[2], enc = i[3], arm = i[7];
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 4) && ten(in, T, 6) && ten(in, T, 7),
+             "op 86: t0 part, t1 fu, t2 wtab, t4 meta, t6 row_partidx, t7 row_gate must be bound");
+        NEED(c, I && H && E, "op 86: zero geometry");
+        if (enc == PLOW_MOE_ENC_FP8BLK && (arm == PLOW_MOE_ARM_W8A8 || arm == PLOW_MOE_ARM_W8A8_P16)) {
+            NEED(c, ten(in, T, 3) && ten(in, T, 5), "op 86 W8A8: t3 stab and t5 fs must be bound");
+            NEED(c, I % 128u == 0u && H % 128u == 0u, "op 86 W8A8: I %u and H %u must be multiples of 128", I, H);
+            if (!launch) return 0;
+            GroupW8A8 g = {};
+            g.out = ten(in, T, 0);
+            g.a = ten(in, T, 1); g.a_scale = (const float*)ten(in, T, 5);
+            g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 3);
+            g.meta = (const int32_t*)ten(in, T, 4);
+            g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
+            g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_W8A8_P16;
+            return launch_group_down_w8a8(g, st);
+        }
+        return fail(c, PLOW_MOE_EUNSUPPORTED, "op 86: encoding %u arm %u is not served", enc, arm);
+    }
+    default:
+        return fail(c, PLOW_MOE_EUNSUPPORTED, "opcode %u is not served by this library", (unsigned)in->op);
+    }
+}
+
+static int finish(PlowMoeCtx* c, int rc, const PlowDevInst* in) {
+    if (rc) {
+        if (rc != PLOW_MOE_EINVAL && rc != PLOW_MOE_EUNSUPPORTED) fail(c, rc, "op %u: launcher refused (%d)", (unsigned)in->op, rc);
+        else if (!c->err[0]) fail(c, rc, "op %u: refused (%d)", (unsigned)in->op, rc);
+        return rc;
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(c, PLOW_MOE_EDEVICE, "op %u: %s", (unsigned)in->op, hipGetErrorString(e));
+    return 0;
+}
+
+extern "C" int plow_moe_check(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors) {
+    if (!ctx || !inst || !tensors) return PLOW_MOE_EINVAL;
+    ctx->err[0] = 0;
+    return run_op(ctx, inst, tensors, nullptr, false);
+}
+
+extern "C" int plow_moe_exec(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors, void* stream) {
+    if (!ctx || !inst || !tensors) return PLOW_MOE_EINVAL;
+    ctx->err[0] = 0;
+    return finish(ctx, run_op(ctx, inst, tensors, (hipStream_t)stream, true), inst);
+}
+
+extern "C" int plow_moe_exec_many(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst,
+                                  void* const* tensors, void* stream) {
+    if (!ctx || !insts || !tensors) return PLOW_MOE_EINVAL;
+    ctx->err[0] = 0;
+    for (uint32_t n = 0; n < n_inst; n++) { /* refuse the whole run before launching any of it */
+        const int rc = run_op(ctx, &insts[n], tensors, nullptr, false);
+        if (rc) return rc;
+    }
+    for (uint32_t n = 0; n < n_inst; n++) {
+        const int rc = finish(ctx, run_op(ctx, &insts[n], tensors, (hipStream_t)stream, true), &insts[n]);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+/* ---- segment entry points ---------------------------------------------------------------------- */
+
+static bool is_glu(uint16_t op) {
+    return op == PLOW_DOP_MOE_GROUP_GLU_PF || op == PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF_W8A8 ||
+           op == PLOW_DOP_MOE_GROUP_GLU_FP8_BLK || op == PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8;
+}
+static bool is_down(uint16_t op) {
+    return op == PLOW_DOP_MOE_GROUP_DOWN_PF || op == PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8 ||
+           op == PLOW_DOP_MOE_GROUP_DOWN_FP8_BLK || op == PLOW_DOP_MOE_EXPERT_DOWN_GEMMA_FP8;
+}
+
+/* A segment is a run holding exactly one GLU and one DOWN of the same family, GLU first, whose
+ * intermediate, expert table and geometry agree; everything else in the run must be an op of this
+ * library. */
+static int check_segment(PlowMoeCtx* c, const PlowDevInst* insts, uint32_t n) {
+    int glu = -1, down = -1;
+    for (uint32_t j = 0; j < n; j++) {
+        if (is_glu(insts[j].op)) { NEED(c, glu < 0, "segment: more than one GLU op"); glu = (int)j; }
+        if (is_down(insts[j].op)) { NEED(c, down < 0, "segment: more than one DOWN op"); down = (int)j; }
+    }
+    NEED(c, glu >= 0 && down >= 0 && glu < down, "segment: needs one GLU followed by one DOWN");
+    const PlowDevInst &g = insts[glu], &d = insts[down];
+    NEED(c, d.op == g.op + 1u, "segment: GLU op %u and DOWN op %u are not a pair", (unsigned)g.op, (unsigned)d.op);
+    if (g.op == PLOW_DOP_MOE_GROUP_GLU_PF) {
+        NEED(c, g.i[0] == d.i[1] && g.i[1] == d.i[0] && g.i[2] == d.i[2], "segment: GLU (I,H,E) and DOWN (H,I,E) disagree");
+        NEED(c, g.i[3] == d.i[3], "segment: GLU and DOWN weight encodings differ");
+        NEED(c, g.t[2] == d.t[2] && g.t[3] == d.t[3] && g.t[4] == d.t[4], "segment: wtab / stab / meta handles differ");
+        const bool quantized_mid = g.i[7] == PLOW_MOE_ARM_W8A8;
+        NEED(c, g.t[0] == d.t[1], "segment: DOWN does not read the GLU's output");
+        if (quantized_mid) NEED(c, g.t[7] == d.t[5], "segment: DOWN does not read the GLU's output scales");
+        NEED(c, (g.i[7] == PLOW_MOE_ARM_W8A8) == (d.i[7] == PLOW_MOE_ARM_W8A8 || d.i[7] == PLOW_MOE_ARM_W8A8_P16),
+             "segment: GLU arm %u and DOWN arm %u disagree", g.i[7], d.i[7]);
+    } else if (g.op == PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF_W8A8) {
+        NEED(c, g.i[0] == d.i[1] && g.i[1] == d.i[0] && g.i[2] == d.i[2], "segment: GLU (I,H,E) and DOWN (H,I,E) disagree");
+        NEED(c, g.t[2] == d.t[2] && g.t[3] == d.t[3] && g.t[6] == d.t[6], "segment: ewt / meta / est handles differ");
+    } else {
+        NEED(c, g.i[1] == d.i[2] && g.i[2] == d.i[1] && g.i[3] == d.i[3], "segment: GLU (I,H,E) and DOWN (H,I,E) disagree");
+        NEED(c, g.t[0] == d.t[1] && g.t[2] == d.t[2] && g.t[3] == d.t[3], "segment: fu / table / weight-table handles differ");
+    }
+    return 0;
+}
+
+static int run_segment(PlowMoeCtx* ctx, int variant, const PlowDevInst* insts, uint32_t n_inst,
+                       void* const* tensors, uint32_t rows, void* stream) {
+    if (!ctx || !insts || !tensors || n_inst == 0) return PLOW_MOE_EINVAL;
+    ctx->err[0] = 0;
+    const int mr = ctx->min_rows[variant];
+    if (mr == 0 || (mr > 0 && rows < (uint32_t)mr)) return PLOW_MOE_ROLLBACK;
+    const int rc = check_segment(ctx, insts, n_inst);
+    if (rc) return rc;
+    return plow_moe_exec_many(ctx, insts, n_inst, tensors, stream);
+}
+
+extern "C" int plow_moe_pf(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst,
+                           void* const* tensors, uint32_t rows, void* stream) {
+    return run_segment(ctx, 0, insts, n_inst, tensors, rows, stream);
+}
+
+extern "C" int plow_moe_dec(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst,
+                            void* const* tensors, uint32_t rows, void* stream) {
+    return run_segment(ctx, 1, insts, n_inst, tensors, rows, stream);
+}

@@ -1,0 +1,224 @@
+/* experts_w8a8.hip — grouped expert GEMMs over aligned rows, block-fp8 weights (128x128 f32 scales)
+ * times 1x128-scaled e4m3 activations (ops 85 / 86, arm 2 / 3).
+ *
+ * Arithmetic (plow runtime/amd/moe_pf_w8a8.h:368-379, :401-473): per 128-K block one fp8 x fp8
+ * matrix product t accumulated in f32, promoted with acc = fmaf(t, a_scale[row][kb] * w_scale[nb][kb],
+ * acc) in ascending kb. GLU: SwiGLU in f32, then per (row, 128 columns) amax = max(1e-10, |v|),
+ * fs = amax / 448, fq = e4m3(v * (1 / fs)). DOWN: part[row_partidx[r]] = row_gate[r] * acc.
+ *
+ * WEIGHT-STREAMING KERNEL (few rows per expert; the decode shape). The job is to pull every weight
+ * byte of every hit expert through the chip exactly once at HBM speed; the matrix cores are nearly
+ * idle. One workgroup = (expert, 128 output channels), 8 waves, each wave 16 channels. The weights
+ * are the A operand of v_mfma_f32_16x16x128_f8f6f4 (lane = (channel c, k-chunk q) holds 32 bytes of
+ * one weight row) and go from global memory straight into the operand registers, DEPTH k-steps
+ * ahead of their use; an expert's few activation rows are the B operand (lane = (row c, k-chunk q))
+ * and come through the vector L1, since all 8 waves of the workgroup read the same rows. A lane's
+ * 32 operand bytes are two 16-byte loads; k is permuted inside the 128 block (the same way for both
+ * operands, which leaves the dot product unchanged) so that the four lanes of a row cover 64
+ * contiguous bytes per load: lane q holds bytes [16q, 16q+16) and [64+16q, 64+16q+16).
+ * The accumulator holds D[channel 4q+i][row c], so gate and up of one output element sit in the same
+ * lane and the GLU epilogue needs no exchange; only the per-row amax crosses waves (through LDS).
+ */
+#include "common.h"
+#include "kernels.h"
+
+#define SK_WAVES 8u
+#define SK_THREADS (SK_WAVES * WAVE)
+#define SK_BN 128u /* output channels per workgroup */
+
+template <int N>
+struct Depth { static constexpr int v = N; };
+
+/* Pipeline depth by row tiles: operand registers are 8 (B) per row tile and step. */
+template <int RT> struct DepthOf { static constexpr int v = RT == 1 ? 4 : (RT == 2 ? 3 : 2); };
+
+__device__ __forceinline__ v4i ldg16(const uint8_t* p) { return *(const v4i*)p; }
+
+template <int RT, bool GLU>
+__device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t ct, uint32_t r0,
+                                        uint32_t rb, uint32_t cnt, float* s_red) {
+    constexpr int D = DepthOf<RT>::v;
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6, c = lane & 15u, q = lane >> 4;
+    const uint32_t K = g.K, KB = K / 128u, N = g.N;
+    const uint32_t ch = ct * SK_BN + wv * 16u + c; /* this lane's weight row */
+    const uint8_t* w0 = (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * 3u + (GLU ? 0u : 2u)] + (size_t)ch * K + 16u * q;
+    const uint8_t* w1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * 3u + 1u] + (size_t)ch * K + 16u * q : nullptr;
+    const float* s0 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u + (GLU ? 0u : 2u)] + (size_t)ct * KB;
+    const float* s1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * 3u + 1u] + (size_t)ct * KB : nullptr;
+
+    /* B operand rows of this lane, one per row tile */
+    const uint8_t* ap[RT];
+    const float* asp[RT];
+    uint32_t as_stride;
+    bool valid[RT];
+    uint32_t rowidx[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+        const uint32_t off = rb + (uint32_t)rt * 16u + c;
+        rowidx[rt] = r0 + off;
+        valid[rt] = off < cnt;
+        if (GLU) {
+            const uint32_t tok = valid[rt] ? g.row_token[rowidx[rt]] : PLOW_EXPERT_UNUSED;
+            valid[rt] = tok != PLOW_EXPERT_UNUSED;
+            const uint32_t t = valid[rt] ? tok : 0u;
+            ap[rt] = (const uint8_t*)g.a + (size_t)t * K + 16u * q;
+            asp[rt] = g.a_scale + t;
+        } else {
+            const uint32_t pi = valid[rt] ? g.row_partidx[rowidx[rt]] : PLOW_EXPERT_UNUSED;
+            valid[rt] = pi != PLOW_EXPERT_UNUSED;
+            const uint32_t r = valid[rt] ? rowidx[rt] : r0;
+            ap[rt] = (const uint8_t*)g.a + (size_t)r * K + 16u * q;
+            asp[rt] = g.a_scale + (size_t)r * KB;
+        }
+    }
+    as_stride = GLU ? g.pitch : 1u;
+
+    v4i wa[D][2], wb[D][2], xa[D][RT][2];
+    float xs[D][RT], sa[D], sb[D];
+    auto issue = [&](int d, uint32_t kb) {
+        const uint32_t ko = kb * 128u;
+        wa[d][0] = ldg16(w0 + ko);
+        wa[d][1] = ldg16(w0 + ko + 64u);
+        if (GLU) {
+            wb[d][0] = ldg16(w1 + ko);
+            wb[d][1] = ldg16(w1 + ko + 64u);
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            xa[d][rt][0] = (v4i){0, 0, 0, 0};
+            xa[d][rt][1] = (v4i){0, 0, 0, 0};
+            xs[d][rt] = 0.0f;
+            if (valid[rt]) {
+                xa[d][rt][0] = ldg16(ap[rt] + ko);
+                xa[d][rt][1] = ldg16(ap[rt] + ko + 64u);
+                xs[d][rt] = asp[rt][(size_t)kb * as_stride];
+            }
+        }
+        sa[d] = s0[kb];
+        if (GLU) sb[d] = s1[kb];
+    };
+
+    v4f acc0[RT], acc1[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+        acc0[rt] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+        acc1[rt] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if ((uint32_t)d < KB) issue(d, (uint32_t)d);
+    for (uint32_t kb0 = 0; kb0 < KB; kb0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            const uint32_t kb = kb0 + (uint32_t)d;
+            if (kb < KB) {
+                const v8i A0 = __builtin_shufflevector(wa[d][0], wa[d][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                v8i A1;
+                if (GLU) A1 = __builtin_shufflevector(wb[d][0], wb[d][1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++) {
+                    const v8i B = __builtin_shufflevector(xa[d][rt][0], xa[d][rt][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
+                    const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A0, B, z, 0, 0, 0, 0, 0, 0);
+                    const float sc0 = xs[d][rt] * sa[d];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc0[rt][i] = fmaf(t0[i], sc0, acc0[rt][i]);
+                    if (GLU) {
+                        const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, z, 0, 0, 0, 0, 0, 0);
+                        const float sc1 = xs[d][rt] * sb[d];
+#pragma unroll
+                        for (int i = 0; i < 4; i++) acc1[rt][i] = fmaf(t1[i], sc1, acc1[rt][i]);
+                    }
+                }
+                if (kb + D < KB) issue(d, kb + D);
+            }
+        }
+    }
+
+    /* ---- epilogue: lane holds channels ct*128 + wv*16 + 4q + i (i = 0..3) of row c ---- */
+    const uint32_t col = ct * SK_BN + wv * 16u + 4u * q;
+    if (GLU) {
+        float v[RT][4];
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            float m = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                v[rt][i] = moe_glu(acc0[rt][i], acc1[rt][i], g.act);
+                m = fmaxf(m, fabsf(v[rt][i]));
+            }
+            m = fmaxf(m, __shfl_xor(m, 16, 64));
+            m = fmaxf(m, __shfl_xor(m, 32, 64));
+            if (q == 0) s_red[wv * 64u + (uint32_t)rt * 16u + c] = m;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            float amax = 1e-10f;
+#pragma unroll
+            for (uint32_t w = 0; w < SK_WAVES; w++) amax = fmaxf(amax, s_red[w * 64u + (uint32_t)rt * 16u + c]);
+            const float s = amax * (1.0f / 448.0f);
+            const float inv = 1.0f / s;
+            if (valid[rt]) {
+                const uint32_t pk = cvt4_e4m3(v[rt][0] * inv, v[rt][1] * inv, v[rt][2] * inv, v[rt][3] * inv);
+                *(uint32_t*)((uint8_t*)g.out + (size_t)rowidx[rt] * N + col) = pk;
+                if (wv == 0 && q == 0) g.out_scale[(size_t)rowidx[rt] * (N / 128u) + ct] = s;
+            }
+        }
+        __syncthreads(); /* s_red is reused by the next row block */
+    } else {
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            if (!valid[rt]) continue;
+            const uint32_t pidx = g.row_partidx[rowidx[rt]];
+            const float gate = g.row_gate[rowidx[rt]];
+            const float y0 = gate * acc0[rt][0], y1 = gate * acc0[rt][1], y2 = gate * acc0[rt][2], y3 = gate * acc0[rt][3];
+            if (g.part16) {
+                uint2 o;
+                o.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16);
+                o.y = (uint32_t)f2bf(y2) | ((uint32_t)f2bf(y3) << 16);
+                *(uint2*)((bf16_t*)g.out + (size_t)pidx * N + col) = o;
+            } else {
+                *(float4*)((float*)g.out + (size_t)pidx * N + col) = make_float4(y0, y1, y2, y3);
+            }
+        }
+    }
+}
+
+template <bool GLU>
+__global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
+    __shared__ float s_red[SK_WAVES * 64u];
+    const uint32_t tiles = g.N / SK_BN;
+    const uint32_t e = blockIdx.x / tiles, ct = blockIdx.x % tiles;
+    const uint32_t cnt = (uint32_t)g.meta[g.E + e];
+    if (cnt == 0u) return;
+    if (g.wtab[(size_t)e * 3u + (GLU ? 0u : 2u)] == 0ull) return; /* expert not resident: skipped */
+    const uint32_t r0 = (uint32_t)g.meta[e];
+    for (uint32_t rb = 0; rb < cnt; rb += 64u) {
+        const uint32_t left = cnt - rb;
+        if (left <= 16u) sk_body<1, GLU>(g, e, ct, r0, rb, cnt, s_red);
+        else if (left <= 32u) sk_body<2, GLU>(g, e, ct, r0, rb, cnt, s_red);
+        else sk_body<4, GLU>(g, e, ct, r0, rb, cnt, s_red);
+    }
+}
+
+static int check_w8a8(const GroupW8A8& g) {
+    if (g.N == 0 || g.K == 0 || g.E == 0) return PLOW_MOE_EINVAL;
+    if (g.N % SK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
+    if ((uint64_t)g.E * (g.N / SK_BN) > 0x7FFFFFFFull) return PLOW_MOE_EINVAL;
+    return 0;
+}
+
+int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
+    const int rc = check_w8a8(g);
+    if (rc) return rc;
+    k_group_w8a8_stream<true><<<g.E * (g.N / SK_BN), SK_THREADS, 0, st>>>(g);
+    return 0;
+}
+
+int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
+    const int rc = check_w8a8(g);
+    if (rc) return rc;
+    k_group_w8a8_stream<false><<<g.E * (g.N / SK_BN), SK_THREADS, 0, st>>>(g);
+    return 0;
+}

@@ -1,0 +1,40 @@
+/* kernels.h — host-callable launchers of the device kernels (one per op family). Every launcher is
+ * asynchronous on `st`, allocates nothing and returns 0 or a negative PLOW_MOE_E* code. */
+#ifndef PLOW_MOE_KERNELS_H
+#define PLOW_MOE_KERNELS_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+int launch_router_score(float* out, const void* x, const void* w, uint32_t M, uint32_t N, uint32_t K,
+                        hipStream_t st);
+int launch_router_topk(void* table, const void* logit, const float* bias, uint32_t n_exp, uint32_t k,
+                       uint32_t flags, uint32_t T, uint32_t tail, uint32_t n_group, uint32_t topk_group,
+                       float route_scale, float logit_scale, hipStream_t st);
+int launch_align(int32_t* meta, const void* table, uint32_t* row_token, uint32_t* row_partidx,
+                 float* row_gate, uint32_t T, uint32_t E, uint32_t k, hipStream_t st);
+int launch_combine(void* out, const void* residual, const void* shared, const void* part, uint32_t H,
+                   uint32_t k, uint32_t T, uint32_t part16, hipStream_t st);
+
+int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uint32_t K, uint32_t pitch,
+                          hipStream_t st);
+int launch_quant_row(void* xq, const void* x, float* scale, uint32_t M, uint32_t K, hipStream_t st);
+
+/* Grouped experts over aligned rows, block-fp8 weights x 1x128-scaled e4m3 activations. */
+struct GroupW8A8 {
+    void* out;            /* GLU: fq u8 [R][N]; DOWN: part f32|bf16 [T*k][N] */
+    float* out_scale;     /* GLU: fs f32 [R][N/128] */
+    const void* a;        /* GLU: xq u8 [T][K]; DOWN: fq u8 [R][K] */
+    const float* a_scale; /* GLU: xs f32 [K/128][pitch]; DOWN: fs f32 [R][K/128] */
+    const uint64_t* wtab; /* [E][3] */
+    const uint64_t* stab; /* [E][3] */
+    const int32_t* meta;
+    const uint32_t* row_token;   /* GLU */
+    const uint32_t* row_partidx; /* DOWN */
+    const float* row_gate;       /* DOWN */
+    uint32_t N, K, E, pitch, act, part16, T;
+};
+int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st);
+int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);
+
+#endif

@@ -1,0 +1,502 @@
+/* route.hip — the routing half of the MoE path on gfx950: router score (op 180), router top-k
+ * (ops 83 / 56), align / sort / offset scan (op 84) and combine (ops 87 / 43).
+ *
+ * Everything integer here (selected experts, their order, counts, offsets, the row permutation) is
+ * bit-identical to plow's CPU reference (runtime/cpu/dev/golden/moe_route.c), and so are the f32
+ * logits and gates, because every floating-point step is done in the reference's own order with
+ * correctly rounded IEEE operations and the exponential of pm_expf.h.
+ * This file is compiled with -ffp-contract=off: no multiply-add is fused unless written as fmaf.
+ */
+#include "common.h"
+#include "kernels.h"
+#include "pm_expf.h"
+
+/* ============================ op 180: router score ============================================= */
+/* logit[m][n] = sum_k bf(x[m][k]) * bf(w[n][k]) with ONE f32 accumulator per output walking k in
+ * ascending order (plow runtime/cpu/dev/golden/f32_primitives.c:235-252). The product of two bf16
+ * values is exact in f32, so fmaf(a, b, acc) rounds exactly like the reference's `acc += a * b`.
+ * Threads form a 16 x 16 grid; each owns a TM x TN block of outputs and both operands are staged
+ * through LDS, transposed to [k][row] f32, one KC-wide chunk at a time with the next chunk's global
+ * loads already in flight. */
+template <int TM, int TN, int KC>
+__global__ __launch_bounds__(256) void k_router_score(float* __restrict__ out,
+                                                      const bf16_t* __restrict__ x,
+                                                      const bf16_t* __restrict__ w, uint32_t M,
+                                                      uint32_t N, uint32_t K) {
+    constexpr int BM = 16 * TM, BN = 16 * TN;
+    constexpr int XCH = BM * KC / 8, WCH = BN * KC / 8;         /* 16-byte pieces per chunk */
+    constexpr int XPT = (XCH + 255) / 256, WPT = (WCH + 255) / 256;
+    __shared__ float xs[KC][BM + 1];
+    __shared__ float ws[KC][BN + 1];
+    const uint32_t tid = threadIdx.x, tx = tid & 15u, ty = tid >> 4;
+    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    float acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = 0.0f;
+
+    uint4 xr[XPT], wr[WPT];
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int p = 0; p < XPT; p++) {
+            const uint32_t c = tid + 256u * p, row = c / (KC / 8), kc = c % (KC / 8);
+            const uint32_t k = k0 + kc * 8u;
+            xr[p] = make_uint4(0, 0, 0, 0);
+            if (c < (uint32_t)XCH && m0 + row < M && k < K)
+                xr[p] = *(const uint4*)(x + (size_t)(m0 + row) * K + k);
+        }
+#pragma unroll
+        for (int p = 0; p < WPT; p++) {
+            const uint32_t c = tid + 256u * p, row = c / (KC / 8), kc = c % (KC / 8);
+            const uint32_t k = k0 + kc * 8u;
+            wr[p] = make_uint4(0, 0, 0, 0);
+            if (c < (uint32_t)WCH && n0 + row < N && k < K)
+                wr[p] = *(const uint4*)(w + (size_t)(n0 + row) * K + k);
+        }
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int p = 0; p < XPT; p++) {
+            const uint32_t c = tid + 256u * p, row = c / (KC / 8), kc = c % (KC / 8);
+            if (c < (uint32_t)XCH) {
+                const uint32_t v[4] = {xr[p].x, xr[p].y, xr[p].z, xr[p].w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    xs[kc * 8 + 2 * j][row] = __uint_as_float(v[j] << 16);
+                    xs[kc * 8 + 2 * j + 1][row] = __uint_as_float(v[j] & 0xFFFF0000u);
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < WPT; p++) {
+            const uint32_t c = tid + 256u * p, row = c / (KC / 8), kc = c % (KC / 8);
+            if (c < (uint32_t)WCH) {
+                const uint32_t v[4] = {wr[p].x, wr[p].y, wr[p].z, wr[p].w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    ws[kc * 8 + 2 * j][row] = __uint_as_float(v[j] << 16);
+                    ws[kc * 8 + 2 * j + 1][row] = __uint_as_float(v[j] & 0xFFFF0000u);
+                }
+            }
+        }
+    };
+
+    fetch(0);
+    for (uint32_t k0 = 0; k0 < K; k0 += KC) {
+        __syncthreads(); /* everyone is done reading the previous chunk */
+        commit();
+        __syncthreads();
+        if (k0 + KC < K) fetch(k0 + KC);
+        const uint32_t kn = K - k0 < (uint32_t)KC ? K - k0 : (uint32_t)KC;
+        if (kn == (uint32_t)KC) {
+#pragma unroll 8
+            for (int kk = 0; kk < KC; kk++) {
+                float a[TM], b[TN];
+#pragma unroll
+                for (int i = 0; i < TM; i++) a[i] = xs[kk][ty * TM + i];
+#pragma unroll
+                for (int j = 0; j < TN; j++) b[j] = ws[kk][tx * TN + j];
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+            }
+        } else {
+            for (uint32_t kk = 0; kk < kn; kk++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = fmaf(xs[kk][ty * TM + i], ws[kk][tx * TN + j], acc[i][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const uint32_t m = m0 + ty * TM + i, n = n0 + tx * TN + j;
+            if (m < M && n < N) out[(size_t)m * N + n] = acc[i][j];
+        }
+}
+
+int launch_router_score(float* out, const void* x, const void* w, uint32_t M, uint32_t N, uint32_t K,
+                        hipStream_t st) {
+    if (K % 8u) return PLOW_MOE_EINVAL;
+    if ((uint64_t)M * N >= (1u << 19)) {
+        dim3 g((N + 63) / 64, (M + 63) / 64);
+        k_router_score<4, 4, 32><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+    } else {
+        dim3 g((N + 15) / 16, (M + 15) / 16);
+        k_router_score<1, 1, 128><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+    }
+    return 0;
+}
+
+/* ============================ ops 83 / 56: router top-k ======================================== */
+/* One wave per token. Lane l holds experts l, l + 64, ... in registers; scores and packed 64-bit
+ * selection keys also sit in LDS so that every lane can walk all of them (a same-address LDS read
+ * is a broadcast). Selection is the reference's rank rule: the winner of slot j is the expert with
+ * exactly j keys above it (plow runtime/common/moe_route_key.h). */
+#define RT_MAX_E 1024u
+#define RT_WAVES 4u
+
+struct RouterArgs {
+    PlowMoeRoute* table;
+    const void* logit;
+    const float* bias;
+    uint32_t n_exp, k, flags, T, tail, n_group, topk_group;
+    float route_scale, logit_scale;
+};
+
+template <uint32_t RT_EPL> /* experts per lane: n_exp <= 64 * RT_EPL */
+__global__ __launch_bounds__(RT_WAVES* WAVE) void k_router_topk(RouterArgs a) {
+    __shared__ float s_score[RT_WAVES][64u * RT_EPL];
+    __shared__ unsigned long long s_key[RT_WAVES][64u * RT_EPL];
+    __shared__ uint32_t s_win[RT_WAVES][PLOW_ROUTE_MAX_TOPK];
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
+    const uint32_t tok = blockIdx.x * RT_WAVES + wv;
+    if (tok >= a.T) return; /* whole wave leaves together; no block-level barrier below */
+    float* score = s_score[wv];
+    unsigned long long* key = s_key[wv];
+    uint32_t* win = s_win[wv];
+    const uint32_t E = a.n_exp;
+    const bool sigmoid = a.flags & PLOW_ROUTE_SIGMOID, norm = a.flags & PLOW_ROUTE_NORM_TOPK;
+    const bool f32l = a.flags & PLOW_ROUTE_F32_LOGIT;
+    const float ls = a.logit_scale != 0.0f ? a.logit_scale : 1.0f;
+    uint32_t k = a.k;
+    PlowMoeRoute* row = a.table + (size_t)tok * (a.k + a.tail);
+    for (uint32_t j = PLOW_ROUTE_MAX_TOPK + lane; j < k; j += WAVE) {
+        row[j].eid = PLOW_EXPERT_UNUSED;
+        row[j].gate = 0.0f;
+    }
+    if (k > PLOW_ROUTE_MAX_TOPK) k = PLOW_ROUTE_MAX_TOPK;
+
+    /* --- score transform --- */
+    float sc[RT_EPL];
+    if (sigmoid) {
+#pragma unroll
+        for (uint32_t j = 0; j < RT_EPL; j++) {
+            const uint32_t e = lane + WAVE * j;
+            if (e < E) {
+                const float l = (f32l ? ((const float*)a.logit)[(size_t)tok * E + e]
+                                      : bf2f(((const bf16_t*)a.logit)[(size_t)tok * E + e])) * ls;
+                sc[j] = 1.0f / (1.0f + pm_expf(-l));
+                score[e] = sc[j];
+            }
+        }
+    } else {
+        float m = -1e30f; /* the maximum is the same value in any visiting order */
+#pragma unroll
+        for (uint32_t j = 0; j < RT_EPL; j++) {
+            const uint32_t e = lane + WAVE * j;
+            if (e < E) {
+                sc[j] = (f32l ? ((const float*)a.logit)[(size_t)tok * E + e]
+                              : bf2f(((const bf16_t*)a.logit)[(size_t)tok * E + e])) * ls;
+                if (sc[j] > m) m = sc[j];
+            }
+        }
+        m = wave_max(m);
+#pragma unroll
+        for (uint32_t j = 0; j < RT_EPL; j++) {
+            const uint32_t e = lane + WAVE * j;
+            if (e < E) score[e] = pm_expf(sc[j] - m);
+        }
+        __builtin_amdgcn_wave_barrier();
+        float s = 0.0f; /* the sum IS order dependent: ascending expert id, one accumulator */
+        for (uint32_t e = 0; e < E; e++) s += score[e];
+#pragma unroll
+        for (uint32_t j = 0; j < RT_EPL; j++) {
+            const uint32_t e = lane + WAVE * j;
+            if (e < E) {
+                sc[j] = score[e] / s;
+                score[e] = sc[j];
+            }
+        }
+    }
+
+    /* --- packed keys, group mask --- */
+    unsigned long long ky[RT_EPL];
+    float sel[RT_EPL];
+#pragma unroll
+    for (uint32_t j = 0; j < RT_EPL; j++) {
+        const uint32_t e = lane + WAVE * j;
+        if (e < E) {
+            sel[j] = sc[j] + (a.bias ? a.bias[e] : 0.0f);
+            ky[j] = ((unsigned long long)route_ord(sel[j]) << 20) | (unsigned long long)((E - 1u - e) & 0xFFFFFu);
+        }
+    }
+    const bool grouped = a.n_group > 1u && a.topk_group > 0u && a.topk_group < a.n_group &&
+                         a.n_group <= PLOW_ROUTE_MAX_GROUPS && E % a.n_group == 0u;
+    if (grouped) {
+        /* biased scores to LDS (in the key array's storage), one lane per group scans its group in
+         * index order, groups ranked by (ord(top-2 sum), lowest id) */
+        float* selv = (float*)key;
+#pragma unroll
+        for (uint32_t j = 0; j < RT_EPL; j++) {
+            const uint32_t e = lane + WAVE * j;
+            if (e < E) selv[e] = sel[j];
+        }
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t gsz = E / a.n_group;
+        unsigned long long gk = 0ull;
+        if (lane < a.n_group) {
+            float m1 = -3.0e38f, m2 = -3.0e38f;
+            for (uint32_t i = 0; i < gsz; i++) {
+                const float s = selv[lane * gsz + i];
+                if (s > m1) { m2 = m1; m1 = s; } else if (s > m2) m2 = s;
+            }
+            gk = ((unsigned long long)route_ord(m1 + m2) << 8) | (unsigned long long)((a.n_group - 1u - lane) & 0xFFu);
+        }
+        uint32_t grank = 0;
+        for (uint32_t f = 0; f < a.n_group; f++) {
+            const unsigned long long other = __shfl(gk, (int)f, 64);
+            grank += other > gk;
+        }
+        const unsigned long long keep = __ballot(lane < a.n_group && grank < a.topk_group);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (uint32_t j = 0; j < RT_EPL; j++) {
+            const uint32_t e = lane + WAVE * j;
+            if (e < E && !((keep >> (e / gsz)) & 1ull)) ky[j] = (unsigned long long)((E - 1u - e) & 0xFFFFFu);
+        }
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < RT_EPL; j++) {
+        const uint32_t e = lane + WAVE * j;
+        if (e < E) key[e] = ky[j];
+    }
+    if (lane < k) win[lane] = E - 1u;
+    __builtin_amdgcn_wave_barrier();
+
+    /* --- rank select --- */
+    uint32_t rank[RT_EPL];
+#pragma unroll
+    for (uint32_t j = 0; j < RT_EPL; j++) rank[j] = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < RT_EPL; j++)
+        if (lane + WAVE * j >= E) ky[j] = ~0ull; /* absent experts never count and never win */
+#pragma unroll 4
+    for (uint32_t f = 0; f < E; f++) {
+        const unsigned long long kf = key[f];
+#pragma unroll
+        for (uint32_t j = 0; j < RT_EPL; j++) rank[j] += kf > ky[j];
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < RT_EPL; j++) {
+        const uint32_t e = lane + WAVE * j;
+        if (e < E && rank[j] < k) win[rank[j]] = e;
+    }
+    __builtin_amdgcn_wave_barrier();
+
+    /* --- gates: unbiased scores of the winners, summed in slot order --- */
+    float sum = 0.0f;
+    for (uint32_t j = 0; j < k; j++) sum += score[win[j]];
+    if (lane < k) {
+        float g = score[win[lane]];
+        if (norm && sum != 0.0f) g /= sum;
+        g *= a.route_scale;
+        row[lane].eid = win[lane];
+        row[lane].gate = g;
+    }
+    if (a.tail && lane == 0) {
+        row[a.k].eid = E;
+        row[a.k].gate = 1.0f;
+    }
+}
+
+int launch_router_topk(void* table, const void* logit, const float* bias, uint32_t n_exp, uint32_t k,
+                       uint32_t flags, uint32_t T, uint32_t tail, uint32_t n_group, uint32_t topk_group,
+                       float route_scale, float logit_scale, hipStream_t st) {
+    if (n_exp == 0 || n_exp > RT_MAX_E || k == 0 || T == 0) return PLOW_MOE_EINVAL;
+    RouterArgs a = {(PlowMoeRoute*)table, logit, bias, n_exp, k, flags, T, tail, n_group, topk_group,
+                    route_scale, logit_scale};
+    const dim3 g((T + RT_WAVES - 1) / RT_WAVES), b(RT_WAVES * WAVE);
+    if (n_exp <= 128u) k_router_topk<2><<<g, b, 0, st>>>(a);
+    else if (n_exp <= 256u) k_router_topk<4><<<g, b, 0, st>>>(a);
+    else if (n_exp <= 512u) k_router_topk<8><<<g, b, 0, st>>>(a);
+    else k_router_topk<16><<<g, b, 0, st>>>(a);
+    return 0;
+}
+
+/* ============================ op 84: align ===================================================== */
+/* One workgroup of 16 waves; a counting sort with one chunk per wave, so the scatter needs no
+ * atomics and the result is the reference's order (ascending slot inside each expert,
+ * plow runtime/cpu/dev/golden/moe_route.c:118-125):
+ *   A  wave w histograms its contiguous range of slots into hist[w][*]          (LDS atomics: a
+ *      count does not depend on arrival order)
+ *   B  per expert: exclusive prefix over the 16 waves -> base[w][e]; padded prefix over experts ->
+ *      rowoff / tilep; pad rows marked
+ *   C  wave w walks its range in order, 64 slots a step; lanes with the same expert get consecutive
+ *      positions by lane order (ballot + popcount), and the wave's cursor base[w][e] advances. */
+#define AL_WAVES 16u
+#define AL_MAX_E 1056u
+
+struct AlignArgs {
+    int32_t* meta;
+    const PlowMoeRoute* table;
+    uint32_t* row_token;
+    uint32_t* row_partidx;
+    float* row_gate;
+    uint32_t T, E, k;
+};
+
+__global__ __launch_bounds__(AL_WAVES* WAVE) void k_align(AlignArgs a) {
+    __shared__ uint32_t hist[AL_WAVES][AL_MAX_E];
+    __shared__ uint32_t s_rowoff[AL_MAX_E];
+    __shared__ uint32_t s_cnt[AL_MAX_E];
+    __shared__ uint32_t s_carry;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
+    const uint32_t E = a.E, nslot = a.T * a.k;
+    /* slots per wave, a multiple of 64 so that every step of phase C is a whole wave */
+    const uint32_t per = ((nslot + AL_WAVES * WAVE - 1u) / (AL_WAVES * WAVE)) * WAVE;
+    const uint32_t lo = wv * per, hi = lo + per < nslot ? lo + per : nslot;
+
+    for (uint32_t i = tid; i < AL_WAVES * E; i += AL_WAVES * WAVE) hist[i / E][i % E] = 0u;
+    __syncthreads();
+    for (uint32_t s = lo + lane; s < hi; s += WAVE) {
+        const uint32_t e = a.table[s].eid;
+        if (e < E) atomicAdd(&hist[wv][e], 1u);
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < E; e += AL_WAVES * WAVE) {
+        uint32_t run = 0;
+#pragma unroll
+        for (uint32_t w = 0; w < AL_WAVES; w++) {
+            const uint32_t c = hist[w][e];
+            hist[w][e] = run;
+            run += c;
+        }
+        s_cnt[e] = run;
+    }
+    if (tid == 0) s_carry = 0u;
+    __syncthreads();
+    if (wv == 0) { /* padded exclusive prefix over experts, 64 at a time */
+        for (uint32_t e0 = 0; e0 < E; e0 += WAVE) {
+            const uint32_t e = e0 + lane;
+            const uint32_t c = e < E ? s_cnt[e] : 0u;
+            const uint32_t tiles = (c + PLOW_MPF_BM - 1u) / PLOW_MPF_BM;
+            uint32_t inc = tiles;
+#pragma unroll
+            for (uint32_t o = 1; o < WAVE; o <<= 1) {
+                const uint32_t v = __shfl_up(inc, o, 64);
+                if (lane >= o) inc += v;
+            }
+            const uint32_t carry = s_carry;
+            const uint32_t excl = carry + inc - tiles;
+            if (e < E) {
+                s_rowoff[e] = excl * PLOW_MPF_BM;
+                a.meta[e] = (int32_t)(excl * PLOW_MPF_BM);
+                a.meta[E + e] = (int32_t)c;
+                a.meta[2u * E + e] = (int32_t)excl;
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (lane == WAVE - 1u) s_carry = carry + inc;
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (lane == 0) a.meta[3u * E] = (int32_t)s_carry;
+    }
+    __syncthreads();
+    /* pad rows: [rowoff + cnt, rowoff + 64 * ceil(cnt / 64)) */
+    for (uint32_t i = tid; i < E * PLOW_MPF_BM; i += AL_WAVES * WAVE) {
+        const uint32_t e = i / PLOW_MPF_BM, j = i % PLOW_MPF_BM;
+        const uint32_t c = s_cnt[e], r = s_rowoff[e] + c + j;
+        if (c + j < ((c + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM) {
+            a.row_token[r] = PLOW_EXPERT_UNUSED;
+            a.row_partidx[r] = PLOW_EXPERT_UNUSED;
+            a.row_gate[r] = 0.0f;
+        }
+    }
+    /* stable scatter, each wave on its own range and its own cursors (no block barrier needed) */
+    for (uint32_t s0 = lo; s0 < hi; s0 += WAVE) {
+        const uint32_t s = s0 + lane;
+        const bool in = s < hi;
+        const uint32_t e = in ? a.table[s].eid : PLOW_EXPERT_UNUSED;
+        const float g = in ? a.table[s].gate : 0.0f;
+        const bool live = e < E;
+        unsigned long long todo = __ballot(live);
+        uint32_t pos = 0;
+        while (todo) {
+            const uint32_t leader = (uint32_t)__builtin_ctzll(todo);
+            const uint32_t e0 = (uint32_t)__shfl((int)e, (int)leader, 64);
+            const unsigned long long same = __ballot(live && e == e0);
+            const uint32_t cursor = hist[wv][e0];
+            if (live && e == e0)
+                pos = s_rowoff[e0] + cursor + (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
+            __builtin_amdgcn_wave_barrier();
+            if (lane == leader) hist[wv][e0] = cursor + (uint32_t)__builtin_popcountll(same);
+            __builtin_amdgcn_wave_barrier();
+            todo &= ~same;
+        }
+        if (live) {
+            a.row_token[pos] = s / a.k;
+            a.row_partidx[pos] = s;
+            a.row_gate[pos] = g;
+        }
+    }
+}
+
+int launch_align(int32_t* meta, const void* table, uint32_t* row_token, uint32_t* row_partidx,
+                 float* row_gate, uint32_t T, uint32_t E, uint32_t k, hipStream_t st) {
+    if (E == 0 || E > AL_MAX_E || k == 0) return PLOW_MOE_EINVAL;
+    AlignArgs a = {meta, (const PlowMoeRoute*)table, row_token, row_partidx, row_gate, T, E, k};
+    k_align<<<1, AL_WAVES * WAVE, 0, st>>>(a);
+    return 0;
+}
+
+/* ============================ ops 87 / 43: combine ============================================= */
+/* out[t][h] = bf16(residual? + shared? + sum_{j<k} part[t*k+j][h]), f32, that order
+ * (plow runtime/cpu/dev/golden/moe_route.c:130-147). Four consecutive h per thread. */
+struct CombineArgs {
+    bf16_t* out;
+    const bf16_t* residual;
+    const bf16_t* shared;
+    const void* part;
+    uint32_t H, k, T, part16;
+};
+
+__global__ __launch_bounds__(256) void k_combine(CombineArgs a) {
+    const uint32_t H4 = a.H / 4u;
+    const size_t total = (size_t)a.T * H4;
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < total; i += (size_t)gridDim.x * 256u) {
+        const uint32_t tok = (uint32_t)(i / H4), h = (uint32_t)(i % H4) * 4u;
+        const size_t o = (size_t)tok * a.H + h;
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (a.residual) {
+            const uint2 r = *(const uint2*)(a.residual + o);
+            acc[0] = __uint_as_float(r.x << 16); acc[1] = __uint_as_float(r.x & 0xFFFF0000u);
+            acc[2] = __uint_as_float(r.y << 16); acc[3] = __uint_as_float(r.y & 0xFFFF0000u);
+        }
+        if (a.shared) {
+            const uint2 r = *(const uint2*)(a.shared + o);
+            acc[0] += __uint_as_float(r.x << 16); acc[1] += __uint_as_float(r.x & 0xFFFF0000u);
+            acc[2] += __uint_as_float(r.y << 16); acc[3] += __uint_as_float(r.y & 0xFFFF0000u);
+        }
+        for (uint32_t j = 0; j < a.k; j++) {
+            const size_t p = ((size_t)tok * a.k + j) * a.H + h;
+            if (a.part16) {
+                const uint2 r = *(const uint2*)((const bf16_t*)a.part + p);
+                acc[0] += __uint_as_float(r.x << 16); acc[1] += __uint_as_float(r.x & 0xFFFF0000u);
+                acc[2] += __uint_as_float(r.y << 16); acc[3] += __uint_as_float(r.y & 0xFFFF0000u);
+            } else {
+                const float4 v = *(const float4*)((const float*)a.part + p);
+                acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+            }
+        }
+        uint2 w;
+        w.x = (uint32_t)f2bf(acc[0]) | ((uint32_t)f2bf(acc[1]) << 16);
+        w.y = (uint32_t)f2bf(acc[2]) | ((uint32_t)f2bf(acc[3]) << 16);
+        *(uint2*)(a.out + o) = w;
+    }
+}
+
+int launch_combine(void* out, const void* residual, const void* shared, const void* part, uint32_t H,
+                   uint32_t k, uint32_t T, uint32_t part16, hipStream_t st) {
+    if (H % 4u || T == 0) return PLOW_MOE_EINVAL;
+    CombineArgs a = {(bf16_t*)out, (const bf16_t*)residual, (const bf16_t*)shared, part, H, k, T, part16};
+    const size_t total = (size_t)T * (H / 4u);
+    uint32_t blocks = (uint32_t)((total + 255u) / 256u);
+    if (blocks > 4096u) blocks = 4096u;
+    k_combine<<<blocks, 256, 0, st>>>(a);
+    return 0;
+}

@@ -1,0 +1,199 @@
+"""Routing on the GPU (ops 180, 83, 84, 87, 184, 32) against golden vectors from plow's CPU kernels
+and against the oracle: everything bit-exact."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import cases
+import oracle_lib as ol
+from gpu_harness import dev_table, from_dev, to_dev
+from plow_amd import abi
+
+pytestmark = pytest.mark.gpu
+
+G = np.load(os.path.join(os.path.dirname(__file__), "golden", "plow_cpu_golden.npz"))
+
+
+@pytest.fixture(scope="module")
+def moe():
+    from plow_amd.lib import Moe
+    m = Moe(0)
+    yield m
+    m.close()
+
+
+def gpu_route(moe, logit, bias, E, k, T, flags, **kw):
+    tail = kw.get("tail", 0)
+    table = torch.zeros((T * (k + tail), 2), dtype=torch.int32, device="cuda")
+    arrs = [table, to_dev(logit), None, to_dev(bias)]
+    moe.exec(cases.route_inst(E, k, T, flags, bias is not None, **kw), dev_table(arrs))
+    torch.cuda.synchronize()
+    return from_dev(table, ol.ROUTE_DT)
+
+
+def gpu_align(moe, table, T, E, k):
+    R = abi.max_rows(T, k, E)
+    arrs = [torch.zeros(3 * E + 1, dtype=torch.int32, device="cuda"), to_dev(table),
+            torch.full((R,), 7, dtype=torch.int32, device="cuda"),
+            torch.full((R,), 7, dtype=torch.int32, device="cuda"),
+            torch.full((R,), 7.0, dtype=torch.float32, device="cuda")]
+    moe.exec(cases.align_inst(T, E, k), dev_table(arrs))
+    torch.cuda.synchronize()
+    return (arrs[0].cpu().numpy(), arrs[2].cpu().numpy().view(np.uint32),
+            arrs[3].cpu().numpy().view(np.uint32), arrs[4].cpu().numpy())
+
+
+@pytest.mark.parametrize("case", cases.ROUTE_CASES, ids=[c[0] for c in cases.ROUTE_CASES])
+def test_route_and_align_match_plow_cpu_golden(moe, case):
+    name, E, k, T, flags, ties, wb = case
+    print(f"[case] route {name}", flush=True)
+    logit = G[f"route/{name}/logit"]
+    bias = G[f"route/{name}/bias"] if wb else None
+    if flags & 4 and not wb:
+        flags &= ~4
+    table = gpu_route(moe, logit, bias, E, k, T, flags)
+    assert np.array_equal(table.view(np.uint32).reshape(-1, 2), G[f"route/{name}/table"])
+    meta, rt, rp, rg = gpu_align(moe, table, T, E, k)
+    assert np.array_equal(meta, G[f"route/{name}/meta"])
+    rows = int(meta[3 * E]) * abi.MPF_BM
+    assert np.array_equal(rt[:rows], G[f"route/{name}/row_token"])
+    assert np.array_equal(rp[:rows], G[f"route/{name}/row_partidx"])
+    assert np.array_equal(rg[:rows].view(np.uint32), G[f"route/{name}/row_gate"].view(np.uint32))
+    assert np.all(rt[rows:] == 7)
+
+
+@pytest.mark.parametrize("E,k,T,flags,ng,tg,tail", [
+    (256, 8, 4096, 1 | 2 | 4 | 8, 8, 4, 1),      # DeepSeek-V3 prefill routing
+    (256, 8, 64, 1 | 2 | 4 | 8, 8, 4, 1),
+    (384, 8, 128, 1 | 2 | 4 | 8, 0, 0, 1),       # Kimi-K2
+    (128, 8, 2048, 2 | 8, 0, 0, 0),              # Qwen3, softmax + renorm
+    (64, 6, 16, 8, 0, 0, 0),
+    (1000, 16, 5, 1 | 8, 20, 7, 0),
+    (96, 20, 3, 8, 0, 0, 1),                     # k above 16: sentinel slots
+])
+def test_route_and_align_match_oracle(moe, oracle, E, k, T, flags, ng, tg, tail):
+    print(f"[case] route-oracle E={E} k={k} T={T} flags={flags} groups={ng}/{tg}", flush=True)
+    r = cases.rng_of(E * 7 + T)
+    logit = (r.standard_normal((T, E)) * 1.5).astype(np.float32)
+    if T >= 64:  # engineered near-ties: duplicate a few logits inside rows
+        logit[::3, 5] = logit[::3, 9]
+        logit[::5, E - 1] = logit[::5, 0]
+    bias = (r.standard_normal(E) * 0.05).astype(np.float32) if flags & 4 else None
+    kw = dict(n_group=ng, topk_group=tg, tail=tail, route_scale=2.5)
+    got = gpu_route(moe, logit, bias, E, k, T, flags, **kw)
+    want = np.zeros(T * (k + tail), dtype=ol.ROUTE_DT)
+    ol.run(oracle.plow_oracle_exec, cases.route_inst(E, k, T, flags, bias is not None, **kw),
+           ol.table_of([want, logit, None, bias]), 8)
+    assert np.array_equal(got["eid"], want["eid"])
+    assert np.array_equal(got["gate"].view(np.uint32), want["gate"].view(np.uint32))
+    ka, Ea = k + tail, E + tail
+    dev = gpu_align(moe, got, T, Ea, ka)
+    al = cases.align_arrays(want, T, Ea, ka)
+    ol.run(oracle.plow_oracle_exec, cases.align_inst(T, Ea, ka), ol.table_of(al), 1)
+    rows = int(al[0][3 * Ea]) * abi.MPF_BM
+    assert np.array_equal(dev[0], al[0])
+    assert np.array_equal(dev[1][:rows], al[2][:rows]) and np.array_equal(dev[2][:rows], al[3][:rows])
+    assert np.array_equal(dev[3][:rows].view(np.uint32), al[4][:rows].view(np.uint32))
+
+
+@pytest.mark.parametrize("M,N,K", [(6, 40, 768), (64, 256, 7168), (1, 384, 7168), (700, 1000, 264)])
+def test_router_score_bit_exact(moe, oracle, M, N, K):
+    print(f"[case] score {M}x{N}x{K}", flush=True)
+    if (M, N, K) == (6, 40, 768):
+        x, w, want = G["score/x"], G["score/w"], G["score/out"]
+    else:
+        r = cases.rng_of(M + N)
+        x, w = cases.randn_bf16(r, (M, K), 1.0), cases.randn_bf16(r, (N, K), 0.02)
+        want = np.zeros((M, N), np.float32)
+        ol.run(oracle.plow_oracle_exec, abi.inst(abi.OP_GEMM_F32, t=[0, 1, 2], i=[M, N, K]),
+               ol.table_of([want, x, w]), 8)
+    out = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    moe.exec(abi.inst(abi.OP_GEMM_F32, t=[0, 1, 2], i=[M, N, K]), dev_table([out, to_dev(x), to_dev(w)]))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_combine_bit_exact(moe, oracle):
+    part, res, sh = G["combine/part"], G["combine/res"], G["combine/shared"]
+    T, H = res.shape
+    k = part.shape[0] // T
+    out = torch.zeros((T, H), dtype=torch.int16, device="cuda")
+    moe.exec(abi.inst(abi.OP_MOE_COMBINE_PF, t=[0, 1, 2, 3], i=[H, k, T]),
+             dev_table([out, to_dev(res), to_dev(sh), to_dev(part)]))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), G["combine/out"])
+    out.zero_()
+    moe.exec(abi.inst(abi.OP_MOE_COMBINE_PF, t=[0, None, None, 3], i=[H, k, T]),
+             dev_table([out, None, None, to_dev(part)]))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), G["combine/out_plain"])
+    # a larger ragged case incl. the row-band form (i3 = first row) against the oracle
+    r = cases.rng_of(5)
+    T, H, k = 37, 7168, 9
+    part = r.standard_normal((T * k, H)).astype(np.float32)
+    res = cases.randn_bf16(r, (T, H), 1.0)
+    want = np.zeros((T, H), np.uint16)
+    ol.run(oracle.plow_oracle_exec, abi.inst(abi.OP_MOE_COMBINE_PF, t=[0, 1, None, 3], i=[H, k, T]),
+           ol.table_of([want, res, None, part]), 8)
+    out = torch.zeros((T, H), dtype=torch.int16, device="cuda")
+    tbl = dev_table([out, to_dev(res), None, to_dev(part)])
+    moe.exec(abi.inst(abi.OP_MOE_COMBINE_PF, t=[0, 1, None, 3], i=[H, k, 20, 0]), tbl)
+    moe.exec(abi.inst(abi.OP_MOE_COMBINE_PF, t=[0, 1, None, 3], i=[H, k, 17, 20]), tbl)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want)
+
+
+def test_quant_ops_bit_exact(moe, oracle):
+    r = cases.rng_of(9)
+    # 1x128: random rows, an all-zero group, and rows whose group amax is exactly 448 so that the
+    # scale is 1 and the hardware conversion is exercised on every e4m3 rounding boundary
+    grid = np.array([oracle.plow_oracle_e4m3_to_f32(c) for c in range(127)], np.float32)
+    mids = ((grid[:-1].astype(np.float64) + grid[1:]) / 2).astype(np.float32)
+    vals = np.concatenate([grid, mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(999))])
+    vals = ol.bf2f(ol.f2bf(vals))  # the op's input is bf16
+    M, K = 16, 1024
+    x = ol.bf2f(cases.randn_bf16(r, (M, K), 2.0))
+    x[3, 256:384] = 0
+    both_signs = np.concatenate([vals, -vals])
+    blk = np.resize(both_signs, (8 * 8, 127))    # 64 groups of 127 crafted values + one 448
+    assert blk.size >= both_signs.size
+    for n in range(blk.shape[0]):
+        row, grp = 6 + n // 8, n % 8
+        x[row, grp * 128:grp * 128 + 127] = blk[n]
+        x[row, grp * 128 + 127] = 448.0
+    xb = ol.f2bf(x)
+    want_q, want_s = np.zeros((M, K), np.uint8), np.zeros((K // 128, M + 3), np.float32)
+    inst = abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[M, K, M + 3])
+    ol.run(oracle.plow_oracle_exec, inst, ol.table_of([want_q, xb, want_s]), 4)
+    q = torch.zeros((M, K), dtype=torch.uint8, device="cuda")
+    s = torch.zeros((K // 128, M + 3), dtype=torch.float32, device="cuda")
+    moe.exec(inst, dev_table([q, to_dev(xb), s]))
+    torch.cuda.synchronize()
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    assert np.array_equal(q.cpu().numpy(), want_q)
+    # per-row
+    x2 = G["quant32/x"]
+    M2, K2 = x2.shape
+    q2 = torch.zeros((M2, K2), dtype=torch.uint8, device="cuda")
+    s2 = torch.zeros(M2, dtype=torch.float32, device="cuda")
+    moe.exec(abi.inst(abi.OP_QUANT_FP8, t=[0, 1, 2], i=[M2, K2]), dev_table([q2, to_dev(x2), s2]))
+    torch.cuda.synchronize()
+    assert np.array_equal(q2.cpu().numpy(), G["quant32/xq"])
+    assert np.array_equal(s2.cpu().numpy().view(np.uint32), G["quant32/scale"].view(np.uint32))
+
+
+def test_refusals(moe):
+    """Typed refusal before launch, with a message; nothing is enqueued."""
+    t = dev_table([torch.zeros(8, device="cuda")] * 8)
+    assert moe.check(abi.inst(999, t=[0]), t) == abi.E_UNSUPPORTED
+    assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1, None, 3], i=[0, 64, 4, 1, 2]), t) == abi.E_INVAL
+    assert "bias" in moe.last_error()
+    assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 1, 2, 0, 8, 1]), t) == 0
+    assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 60, 8, 1, 2, 0, 8, 4]), t) == abi.E_INVAL
+    assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 1, 2, 0, 32, 2]), t) == abi.E_INVAL
+    assert moe.check(abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5], i=[256, 256, 4, 2, 0, 1, 0, 0]), t) == abi.E_UNSUPPORTED
+    assert moe.check(abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[4, 100]), t) == abi.E_INVAL
+    with pytest.raises(Exception):
+        moe.exec(abi.inst(abi.OP_MOE_ALIGN_PF, t=[0, 1, 2, 3], i=[4, 8, 2]), t)
