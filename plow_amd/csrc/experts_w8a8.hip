@@ -22,22 +22,21 @@
 #include "common.h"
 #include "kernels.h"
 
+#include <cstdlib>
+
 #define SK_WAVES 8u
 #define SK_THREADS (SK_WAVES * WAVE)
 #define SK_BN 128u /* output channels per workgroup */
+#ifndef SK_DEPTH
+#define SK_DEPTH 3 /* k-steps of weight loads in flight per wave */
+#endif
 
-template <int N>
-struct Depth { static constexpr int v = N; };
-
-/* Pipeline depth by row tiles: operand registers are 8 (B) per row tile and step. */
-template <int RT> struct DepthOf { static constexpr int v = RT == 1 ? 4 : (RT == 2 ? 3 : 2); };
 
 __device__ __forceinline__ v4i ldg16(const uint8_t* p) { return *(const v4i*)p; }
 
-template <int RT, bool GLU>
+template <int RT, bool GLU, int D>
 __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t ct, uint32_t r0,
                                         uint32_t rb, uint32_t cnt, float* s_red) {
-    constexpr int D = DepthOf<RT>::v;
     const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6, c = lane & 15u, q = lane >> 4;
     const uint32_t K = g.K, KB = K / 128u, N = g.N;
     const uint32_t ch = ct * SK_BN + wv * 16u + c; /* this lane's weight row */
@@ -185,21 +184,31 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
     }
 }
 
-template <bool GLU>
+template <bool GLU, int D>
 __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     __shared__ float s_red[SK_WAVES * 64u];
     const uint32_t tiles = g.N / SK_BN;
-    const uint32_t e = blockIdx.x / tiles, ct = blockIdx.x % tiles;
+    /* highest expert id first: a folded shared expert (id E-1, every token routed to it) is the one
+     * segment that needs several passes, so it must start early instead of forming the tail */
+    const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles;
     const uint32_t cnt = (uint32_t)g.meta[g.E + e];
     if (cnt == 0u) return;
     if (g.wtab[(size_t)e * 3u + (GLU ? 0u : 2u)] == 0ull) return; /* expert not resident: skipped */
     const uint32_t r0 = (uint32_t)g.meta[e];
-    for (uint32_t rb = 0; rb < cnt; rb += 64u) {
-        const uint32_t left = cnt - rb;
-        if (left <= 16u) sk_body<1, GLU>(g, e, ct, r0, rb, cnt, s_red);
-        else if (left <= 32u) sk_body<2, GLU>(g, e, ct, r0, rb, cnt, s_red);
-        else sk_body<4, GLU>(g, e, ct, r0, rb, cnt, s_red);
+    /* 16 rows a pass; an expert with more rows streams its weights once per pass (the tiled
+     * kernel, not this one, is the tool for many rows per expert) */
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D>(g, e, ct, r0, rb, cnt, s_red);
+}
+
+/* k-steps of weight loads a wave keeps in flight; PLOW_MOE_SK_DEPTH (2..4) overrides for tuning */
+static int stream_depth() {
+    static int d = 0;
+    if (!d) {
+        const char* e = getenv("PLOW_MOE_SK_DEPTH");
+        d = e ? atoi(e) : SK_DEPTH;
+        if (d < 2 || d > 4) d = SK_DEPTH;
     }
+    return d;
 }
 
 static int check_w8a8(const GroupW8A8& g) {
@@ -212,13 +221,23 @@ static int check_w8a8(const GroupW8A8& g) {
 int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
     const int rc = check_w8a8(g);
     if (rc) return rc;
-    k_group_w8a8_stream<true><<<g.E * (g.N / SK_BN), SK_THREADS, 0, st>>>(g);
+    const dim3 grid(g.E * (g.N / SK_BN));
+    switch (stream_depth()) {
+    case 2: k_group_w8a8_stream<true, 2><<<grid, SK_THREADS, 0, st>>>(g); break;
+    case 4: k_group_w8a8_stream<true, 4><<<grid, SK_THREADS, 0, st>>>(g); break;
+    default: k_group_w8a8_stream<true, 3><<<grid, SK_THREADS, 0, st>>>(g); break;
+    }
     return 0;
 }
 
 int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
     const int rc = check_w8a8(g);
     if (rc) return rc;
-    k_group_w8a8_stream<false><<<g.E * (g.N / SK_BN), SK_THREADS, 0, st>>>(g);
+    const dim3 grid(g.E * (g.N / SK_BN));
+    switch (stream_depth()) {
+    case 2: k_group_w8a8_stream<false, 2><<<grid, SK_THREADS, 0, st>>>(g); break;
+    case 4: k_group_w8a8_stream<false, 4><<<grid, SK_THREADS, 0, st>>>(g); break;
+    default: k_group_w8a8_stream<false, 3><<<grid, SK_THREADS, 0, st>>>(g); break;
+    }
     return 0;
 }
