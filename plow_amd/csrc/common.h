@@ -63,6 +63,13 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-/* Launch parameter blocks are passed by value; every kernel takes exactly one of them. */
+/* Workgroup barrier that orders LDS traffic only. __syncthreads() also drains every outstanding
+ * global load (s_waitcnt vmcnt(0)), which would serialise a kernel that keeps loads in flight across
+ * the barrier; this one leaves them in flight. Use it when the data exchanged lives in LDS. */
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 #endif

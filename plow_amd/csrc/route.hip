@@ -84,9 +84,9 @@ __global__ __launch_bounds__(256) void k_router_score(float* __restrict__ out,
 
     fetch(0);
     for (uint32_t k0 = 0; k0 < K; k0 += KC) {
-        __syncthreads(); /* everyone is done reading the previous chunk */
+        lds_barrier(); /* everyone is done reading the previous chunk */
         commit();
-        __syncthreads();
+        lds_barrier();
         if (k0 + KC < K) fetch(k0 + KC);
         const uint32_t kn = K - k0 < (uint32_t)KC ? K - k0 : (uint32_t)KC;
         if (kn == (uint32_t)KC) {
@@ -120,6 +120,105 @@ __global__ __launch_bounds__(256) void k_router_score(float* __restrict__ out,
         }
 }
 
+/* Small problems (decode). Two things bound this shape: the dependent chain of K multiply-adds per
+ * output, and LDS bandwidth (every multiply-add of every lane reads a fresh operand pair). Both say
+ * "spread thin": one wave per workgroup (so one wave per CU's LDS), an 8 x 8 block of outputs per
+ * wave, one output per lane. Operands sit in LDS as f32 [row][k] (double buffered) and are read four
+ * k at a time; global loads run RSW_PF chunks ahead in a ring of register stages, and the barriers
+ * order LDS only so those loads stay in flight. */
+#define RSW_KC 256
+#define RSW_PF 3
+__global__ __launch_bounds__(64) void k_router_score_wave(float* __restrict__ out,
+                                                          const bf16_t* __restrict__ x,
+                                                          const bf16_t* __restrict__ w, uint32_t M,
+                                                          uint32_t N, uint32_t K) {
+    constexpr int KC = RSW_KC, LD = KC + 4; /* +4 floats: the 8 rows start 4 banks apart */
+    __shared__ __attribute__((aligned(16))) float xs[2][8][LD];
+    __shared__ __attribute__((aligned(16))) float ws[2][8][LD];
+    const uint32_t lane = threadIdx.x, my = lane >> 3, nx = lane & 7u;
+    const uint32_t m0 = blockIdx.y * 8u, n0 = blockIdx.x * 8u;
+    /* staging: a row of a chunk is KC / 8 = 32 16-byte pieces; lane l loads piece l % 32 of rows
+     * l / 32, l / 32 + 2, ... (4 rows of each operand) */
+    const uint32_t pc = lane & 31u, rsel = lane >> 5;
+    uint4 xr[RSW_PF][4], wr[RSW_PF][4];
+    auto fetch = [&](int s, uint32_t k0) {
+        const uint32_t k = k0 + pc * 8u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t r = rsel + 2u * i;
+            xr[s][i] = make_uint4(0, 0, 0, 0);
+            wr[s][i] = make_uint4(0, 0, 0, 0);
+            if (m0 + r < M && k < K) xr[s][i] = *(const uint4*)(x + (size_t)(m0 + r) * K + k);
+            if (n0 + r < N && k < K) wr[s][i] = *(const uint4*)(w + (size_t)(n0 + r) * K + k);
+        }
+    };
+    auto put = [&](float* d, uint4 a) {
+        *(float4*)d = make_float4(__uint_as_float(a.x << 16), __uint_as_float(a.x & 0xFFFF0000u),
+                                  __uint_as_float(a.y << 16), __uint_as_float(a.y & 0xFFFF0000u));
+        *(float4*)(d + 4) = make_float4(__uint_as_float(a.z << 16), __uint_as_float(a.z & 0xFFFF0000u),
+                                        __uint_as_float(a.w << 16), __uint_as_float(a.w & 0xFFFF0000u));
+    };
+    auto commit = [&](int s, uint32_t buf) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t r = rsel + 2u * i;
+            put(&xs[buf][r][pc * 8u], xr[s][i]);
+            put(&ws[buf][r][pc * 8u], wr[s][i]);
+        }
+    };
+    float acc = 0.0f;
+#pragma unroll
+    for (int s = 0; s < RSW_PF; s++) fetch(s, (uint32_t)s * KC);
+    commit(0, 0);
+    lds_barrier();
+    uint32_t buf = 0;
+    for (uint32_t kbase = 0; kbase < K; kbase += RSW_PF * KC) {
+#pragma unroll
+        for (int s = 0; s < RSW_PF; s++) {
+            const uint32_t k0 = kbase + (uint32_t)s * KC;
+            if (k0 < K) {
+                const uint32_t kn = K - k0 < (uint32_t)KC ? K - k0 : (uint32_t)KC;
+                const float* xp = xs[buf][my];
+                const float* wp = ws[buf][nx];
+                uint32_t kk = 0;
+                if (kn == (uint32_t)KC) {
+                    /* full chunk: operand reads run one 16-k group ahead of the multiply-adds */
+                    float4 a[2][4], b[2][4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) { a[0][u] = *(const float4*)(xp + 4 * u); b[0][u] = *(const float4*)(wp + 4 * u); }
+#pragma unroll
+                    for (int gq = 0; gq < KC / 16; gq++) {
+                        const int cur = gq & 1, nxt = cur ^ 1;
+                        if (gq + 1 < KC / 16) {
+#pragma unroll
+                            for (int u = 0; u < 4; u++) {
+                                a[nxt][u] = *(const float4*)(xp + 16 * (gq + 1) + 4 * u);
+                                b[nxt][u] = *(const float4*)(wp + 16 * (gq + 1) + 4 * u);
+                            }
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; u++) {
+                            acc = fmaf(a[cur][u].x, b[cur][u].x, acc);
+                            acc = fmaf(a[cur][u].y, b[cur][u].y, acc);
+                            acc = fmaf(a[cur][u].z, b[cur][u].z, acc);
+                            acc = fmaf(a[cur][u].w, b[cur][u].w, acc);
+                        }
+                    }
+                    kk = KC;
+                }
+                for (; kk < kn; kk++) acc = fmaf(xp[kk], wp[kk], acc);
+                /* publish the next chunk (fetched RSW_PF - 1 chunks ago), refill this stage */
+                if (k0 + KC < K) commit((s + 1) % RSW_PF, buf ^ 1u);
+                fetch(s, k0 + RSW_PF * KC);
+                lds_barrier();
+                buf ^= 1u;
+            }
+        }
+    }
+    const uint32_t m = m0 + my, n = n0 + nx;
+    if (m < M && n < N) out[(size_t)m * N + n] = acc;
+}
+
 int launch_router_score(float* out, const void* x, const void* w, uint32_t M, uint32_t N, uint32_t K,
                         hipStream_t st) {
     if (K % 8u) return PLOW_MOE_EINVAL;
@@ -127,17 +226,18 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
         dim3 g((N + 63) / 64, (M + 63) / 64);
         k_router_score<4, 4, 32><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else {
-        dim3 g((N + 15) / 16, (M + 15) / 16);
-        k_router_score<1, 1, 128><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        dim3 g((N + 7) / 8, (M + 7) / 8);
+        k_router_score_wave<<<g, 64, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     }
     return 0;
 }
 
 /* ============================ ops 83 / 56: router top-k ======================================== */
-/* One wave per token. Lane l holds experts l, l + 64, ... in registers; scores and packed 64-bit
- * selection keys also sit in LDS so that every lane can walk all of them (a same-address LDS read
- * is a broadcast). Selection is the reference's rank rule: the winner of slot j is the expert with
- * exactly j keys above it (plow runtime/common/moe_route_key.h). */
+/* One wave per token; lane l holds experts l, l + 64, ... in registers. Selection is k rounds of a
+ * wave-wide maximum over the packed key (ord(score + bias), lowest id wins ties). Keys are unique,
+ * so round j returns the expert with exactly j keys above it: the reference's rank rule
+ * (plow runtime/common/moe_route_key.h) with the same winners in the same order. A wave-wide max is
+ * four DPP steps inside each row of 16 lanes plus a scalar max over the four rows. */
 #define RT_MAX_E 1024u
 #define RT_WAVES 4u
 
@@ -149,17 +249,25 @@ struct RouterArgs {
     float route_scale, logit_scale;
 };
 
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
+    uint32_t t;
+    t = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, false); v = v > t ? v : t; /* quad_perm 1,0,3,2 */
+    t = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, false); v = v > t ? v : t; /* quad_perm 2,3,0,1 */
+    t = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, false); v = v > t ? v : t; /* row_half_mirror */
+    t = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, false); v = v > t ? v : t; /* row_mirror */
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+
 template <uint32_t RT_EPL> /* experts per lane: n_exp <= 64 * RT_EPL */
 __global__ __launch_bounds__(RT_WAVES* WAVE) void k_router_topk(RouterArgs a) {
     __shared__ float s_score[RT_WAVES][64u * RT_EPL];
-    __shared__ unsigned long long s_key[RT_WAVES][64u * RT_EPL];
-    __shared__ uint32_t s_win[RT_WAVES][PLOW_ROUTE_MAX_TOPK];
     const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
     const uint32_t tok = blockIdx.x * RT_WAVES + wv;
     if (tok >= a.T) return; /* whole wave leaves together; no block-level barrier below */
     float* score = s_score[wv];
-    unsigned long long* key = s_key[wv];
-    uint32_t* win = s_win[wv];
     const uint32_t E = a.n_exp;
     const bool sigmoid = a.flags & PLOW_ROUTE_SIGMOID, norm = a.flags & PLOW_ROUTE_NORM_TOPK;
     const bool f32l = a.flags & PLOW_ROUTE_F32_LOGIT;
@@ -174,28 +282,22 @@ __global__ __launch_bounds__(RT_WAVES* WAVE) void k_router_topk(RouterArgs a) {
 
     /* --- score transform --- */
     float sc[RT_EPL];
+#pragma unroll
+    for (uint32_t j = 0; j < RT_EPL; j++) {
+        const uint32_t e = lane + WAVE * j;
+        sc[j] = 0.0f;
+        if (e < E)
+            sc[j] = (f32l ? ((const float*)a.logit)[(size_t)tok * E + e]
+                          : bf2f(((const bf16_t*)a.logit)[(size_t)tok * E + e])) * ls;
+    }
     if (sigmoid) {
 #pragma unroll
-        for (uint32_t j = 0; j < RT_EPL; j++) {
-            const uint32_t e = lane + WAVE * j;
-            if (e < E) {
-                const float l = (f32l ? ((const float*)a.logit)[(size_t)tok * E + e]
-                                      : bf2f(((const bf16_t*)a.logit)[(size_t)tok * E + e])) * ls;
-                sc[j] = 1.0f / (1.0f + pm_expf(-l));
-                score[e] = sc[j];
-            }
-        }
+        for (uint32_t j = 0; j < RT_EPL; j++) sc[j] = 1.0f / (1.0f + pm_expf(-sc[j]));
     } else {
         float m = -1e30f; /* the maximum is the same value in any visiting order */
 #pragma unroll
-        for (uint32_t j = 0; j < RT_EPL; j++) {
-            const uint32_t e = lane + WAVE * j;
-            if (e < E) {
-                sc[j] = (f32l ? ((const float*)a.logit)[(size_t)tok * E + e]
-                              : bf2f(((const bf16_t*)a.logit)[(size_t)tok * E + e])) * ls;
-                if (sc[j] > m) m = sc[j];
-            }
-        }
+        for (uint32_t j = 0; j < RT_EPL; j++)
+            if (lane + WAVE * j < E && sc[j] > m) m = sc[j];
         m = wave_max(m);
 #pragma unroll
         for (uint32_t j = 0; j < RT_EPL; j++) {
@@ -204,99 +306,109 @@ __global__ __launch_bounds__(RT_WAVES* WAVE) void k_router_topk(RouterArgs a) {
         }
         __builtin_amdgcn_wave_barrier();
         float s = 0.0f; /* the sum IS order dependent: ascending expert id, one accumulator */
+#pragma unroll 8
         for (uint32_t e = 0; e < E; e++) s += score[e];
 #pragma unroll
         for (uint32_t j = 0; j < RT_EPL; j++) {
             const uint32_t e = lane + WAVE * j;
-            if (e < E) {
-                sc[j] = score[e] / s;
-                score[e] = sc[j];
-            }
+            if (e < E) sc[j] = score[e] / s;
         }
+        __builtin_amdgcn_wave_barrier();
     }
 
-    /* --- packed keys, group mask --- */
-    unsigned long long ky[RT_EPL];
+    /* --- selection keys: ord(score + bias); a dropped group's experts fall to ord 0 --- */
+    uint32_t ordv[RT_EPL];
     float sel[RT_EPL];
 #pragma unroll
     for (uint32_t j = 0; j < RT_EPL; j++) {
         const uint32_t e = lane + WAVE * j;
-        if (e < E) {
-            sel[j] = sc[j] + (a.bias ? a.bias[e] : 0.0f);
-            ky[j] = ((unsigned long long)route_ord(sel[j]) << 20) | (unsigned long long)((E - 1u - e) & 0xFFFFFu);
-        }
+        sel[j] = sc[j] + ((a.bias && e < E) ? a.bias[e] : 0.0f);
+        ordv[j] = route_ord(sel[j]);
     }
     const bool grouped = a.n_group > 1u && a.topk_group > 0u && a.topk_group < a.n_group &&
                          a.n_group <= PLOW_ROUTE_MAX_GROUPS && E % a.n_group == 0u;
     if (grouped) {
-        /* biased scores to LDS (in the key array's storage), one lane per group scans its group in
-         * index order, groups ranked by (ord(top-2 sum), lowest id) */
-        float* selv = (float*)key;
+        /* group score = sum of the top-2 biased scores of the group (a multiset, so any visiting
+         * order gives the same pair); groups ranked by (ord(sum), lowest id) */
+        const uint32_t ng = a.n_group, gsz = E / ng;
 #pragma unroll
         for (uint32_t j = 0; j < RT_EPL; j++) {
             const uint32_t e = lane + WAVE * j;
-            if (e < E) selv[e] = sel[j];
+            if (e < E) score[e] = sel[j];
         }
         __builtin_amdgcn_wave_barrier();
-        const uint32_t gsz = E / a.n_group;
-        unsigned long long gk = 0ull;
-        if (lane < a.n_group) {
-            float m1 = -3.0e38f, m2 = -3.0e38f;
-            for (uint32_t i = 0; i < gsz; i++) {
-                const float s = selv[lane * gsz + i];
+        const uint32_t lpg = WAVE / ng; /* lanes per group on the fast path */
+        const bool fast = (ng & (ng - 1u)) == 0u && gsz % lpg == 0u;
+        float m1 = -3.0e38f, m2 = -3.0e38f;
+        uint32_t g_of_lane, leader;
+        if (fast) {
+            g_of_lane = lane / lpg;
+            leader = (lane % lpg) == 0u;
+            for (uint32_t i = lane % lpg; i < gsz; i += lpg) {
+                const float s = score[g_of_lane * gsz + i];
                 if (s > m1) { m2 = m1; m1 = s; } else if (s > m2) m2 = s;
             }
-            gk = ((unsigned long long)route_ord(m1 + m2) << 8) | (unsigned long long)((a.n_group - 1u - lane) & 0xFFu);
+            for (uint32_t o = 1; o < lpg; o <<= 1) {
+                const float b1 = __shfl_xor(m1, (int)o, 64), b2 = __shfl_xor(m2, (int)o, 64);
+                const float hi = fmaxf(m1, b1), lo = fminf(m1, b1);
+                m2 = fmaxf(lo, fmaxf(m2, b2));
+                m1 = hi;
+            }
+        } else {
+            g_of_lane = lane;
+            leader = lane < ng;
+            if (leader)
+                for (uint32_t i = 0; i < gsz; i++) {
+                    const float s = score[lane * gsz + i];
+                    if (s > m1) { m2 = m1; m1 = s; } else if (s > m2) m2 = s;
+                }
         }
+        const uint32_t gord = route_ord(m1 + m2);
+        const uint32_t step = fast ? lpg : 1u;
         uint32_t grank = 0;
-        for (uint32_t f = 0; f < a.n_group; f++) {
-            const unsigned long long other = __shfl(gk, (int)f, 64);
-            grank += other > gk;
+        for (uint32_t f = 0; f < ng; f++) {
+            const uint32_t o = (uint32_t)__shfl((int)gord, (int)(f * step), 64);
+            grank += (o > gord) || (o == gord && f < g_of_lane); /* lower id outranks on a tie */
         }
-        const unsigned long long keep = __ballot(lane < a.n_group && grank < a.topk_group);
+        const unsigned long long keep = __ballot(leader && grank < a.topk_group);
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (uint32_t j = 0; j < RT_EPL; j++) {
             const uint32_t e = lane + WAVE * j;
-            if (e < E && !((keep >> (e / gsz)) & 1ull)) ky[j] = (unsigned long long)((E - 1u - e) & 0xFFFFFu);
+            if (e < E && !((keep >> ((e / gsz) * step)) & 1ull)) ordv[j] = 0u;
         }
     }
-#pragma unroll
-    for (uint32_t j = 0; j < RT_EPL; j++) {
-        const uint32_t e = lane + WAVE * j;
-        if (e < E) key[e] = ky[j];
-    }
-    if (lane < k) win[lane] = E - 1u;
-    __builtin_amdgcn_wave_barrier();
 
-    /* --- rank select --- */
-    uint32_t rank[RT_EPL];
+    /* --- k rounds of wave-wide max; inv = E - e (1..E) so that 0 means "no candidate" --- */
+    uint32_t picked = 0u; /* bit j: this lane's expert j is already a winner */
+    float sum = 0.0f, my_g = 0.0f;
+    uint32_t my_e = E - 1u;
+    for (uint32_t r = 0; r < k; r++) {
+        uint32_t bo = 0u, bi = 0u;
 #pragma unroll
-    for (uint32_t j = 0; j < RT_EPL; j++) rank[j] = 0;
+        for (uint32_t j = 0; j < RT_EPL; j++) {
+            const uint32_t e = lane + WAVE * j, inv = E - e;
+            const bool cand = e < E && !((picked >> j) & 1u);
+            if (cand && (bi == 0u || ordv[j] > bo || (ordv[j] == bo && inv > bi))) { bo = ordv[j]; bi = inv; }
+        }
+        const uint32_t mo = wave_umax(bi ? bo : 0u);
+        const uint32_t mi = wave_umax((bi && bo == mo) ? bi : 0u);
+        const uint32_t ew = mi ? E - mi : E - 1u; /* nothing left: the reference's pre-filled E - 1 */
+        const uint32_t wl = ew & 63u, ws = ew >> 6;
+        float cand_score = sc[0];
 #pragma unroll
-    for (uint32_t j = 0; j < RT_EPL; j++)
-        if (lane + WAVE * j >= E) ky[j] = ~0ull; /* absent experts never count and never win */
-#pragma unroll 4
-    for (uint32_t f = 0; f < E; f++) {
-        const unsigned long long kf = key[f];
-#pragma unroll
-        for (uint32_t j = 0; j < RT_EPL; j++) rank[j] += kf > ky[j];
+        for (uint32_t j = 1; j < RT_EPL; j++)
+            if (ws == j) cand_score = sc[j];
+        const float g = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(cand_score), (int)wl));
+        if (mi && lane == wl) picked |= 1u << ws;
+        sum += g; /* slot order, one accumulator, identical in every lane */
+        if (lane == r) { my_e = ew; my_g = g; }
     }
-#pragma unroll
-    for (uint32_t j = 0; j < RT_EPL; j++) {
-        const uint32_t e = lane + WAVE * j;
-        if (e < E && rank[j] < k) win[rank[j]] = e;
-    }
-    __builtin_amdgcn_wave_barrier();
-
-    /* --- gates: unbiased scores of the winners, summed in slot order --- */
-    float sum = 0.0f;
-    for (uint32_t j = 0; j < k; j++) sum += score[win[j]];
     if (lane < k) {
-        float g = score[win[lane]];
+        float g = my_g;
         if (norm && sum != 0.0f) g /= sum;
         g *= a.route_scale;
-        row[lane].eid = win[lane];
+        row[lane].eid = my_e;
         row[lane].gate = g;
     }
     if (a.tail && lane == 0) {
