@@ -22,6 +22,7 @@ SOURCES = {
     "route.hip": ["-ffp-contract=off"],
     "quant.hip": ["-ffp-contract=off"],
     "experts_w8a8.hip": [],
+    "experts_a16.hip": [],
     "api.hip": [],
 }
 

@@ -14,10 +14,20 @@
 #include "../../include/plow_moe.h"
 #include "kernels.h"
 
+/* Slot-major ops (48 / 49 / 65 / 66) are served by sorting their slots by expert into this
+ * context-owned workspace first, so that every hit expert streams its weights once. */
+#define WS_MAX_E 1056u
+#define WS_MAX_SLOTS (1u << 18)
+#define WS_MAX_ROWS (WS_MAX_SLOTS + WS_MAX_E * (PLOW_MPF_BM - 1u))
+
 struct PlowMoeCtx {
     int device;
     int min_rows[2]; /* [0] prefill, [1] decode; < 0 unset */
     char err[256];
+    int32_t* ws_meta;        /* [3 * WS_MAX_E + 1] */
+    uint32_t* ws_row_token;  /* [WS_MAX_ROWS] */
+    uint32_t* ws_row_partidx;
+    float* ws_row_gate;
 };
 
 static int fail(PlowMoeCtx* c, int code, const char* fmt, ...) {
@@ -35,6 +45,7 @@ static inline void* ten(const PlowDevInst* in, void* const* T, int k) {
 }
 
 extern "C" uint32_t plow_moe_abi(void) { return 1u; }
+extern "C" void plow_moe_destroy(PlowMoeCtx* ctx);
 
 extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
     if (!out) return PLOW_MOE_EINVAL;
@@ -45,15 +56,35 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
     if (hipGetDeviceProperties(&prop, device) != hipSuccess) return PLOW_MOE_EDEVICE;
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return PLOW_MOE_EUNSUPPORTED; /* CDNA4 only */
     PlowMoeCtx* c = new (std::nothrow) PlowMoeCtx();
+    if (c) memset(c, 0, sizeof *c);
     if (!c) return PLOW_MOE_ENOMEM;
     c->device = device;
     c->min_rows[0] = c->min_rows[1] = -1;
     c->err[0] = 0;
+    int prev = 0;
+    hipGetDevice(&prev);
+    hipSetDevice(device);
+    const bool ok = hipMalloc(&c->ws_meta, (3u * WS_MAX_E + 1u) * 4u) == hipSuccess &&
+                    hipMalloc(&c->ws_row_token, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
+                    hipMalloc(&c->ws_row_partidx, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
+                    hipMalloc(&c->ws_row_gate, (size_t)WS_MAX_ROWS * 4u) == hipSuccess;
+    hipSetDevice(prev);
+    if (!ok) {
+        plow_moe_destroy(c);
+        return PLOW_MOE_ENOMEM;
+    }
     *out = c;
     return 0;
 }
 
-extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) { delete ctx; }
+extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) {
+    if (!ctx) return;
+    hipFree(ctx->ws_meta);
+    hipFree(ctx->ws_row_token);
+    hipFree(ctx->ws_row_partidx);
+    hipFree(ctx->ws_row_gate);
+    delete ctx;
+}
 
 extern "C" const char* plow_moe_last_error(const PlowMoeCtx* ctx) { return ctx ? ctx->err : "no context"; }
 
@@ -154,6 +185,23 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.N = I; g.K = H; g.E = E; g.pitch = i[4]; g.act = i[5];
             return launch_group_glu_w8a8(g, st);
         }
+        const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
+                         (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
+                         (enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_W4A16);
+        if (a16) {
+            NEED(c, enc == PLOW_MOE_ENC_BF16 || ten(in, T, 3), "op 85: t3 stab must be bound for encoding %u", enc);
+            NEED(c, I % 128u == 0u && H % 128u == 0u, "op 85: I %u and H %u must be multiples of 128", I, H);
+            NEED(c, i[5] <= 1u, "op 85: activation %u is not served", i[5]);
+            if (!launch) return 0;
+            GroupA16 g = {};
+            g.out = ten(in, T, 0); g.a = ten(in, T, 1);
+            g.wtab = (const uint64_t*)ten(in, T, 2);
+            g.stab = enc == PLOW_MOE_ENC_BF16 ? nullptr : (const uint64_t*)ten(in, T, 3);
+            g.meta = (const int32_t*)ten(in, T, 4); g.a_idx = (const uint32_t*)ten(in, T, 5);
+            g.N = I; g.K = H; g.E = E; g.enc = enc; g.act = i[5];
+            g.wcols = 3; g.wsel0 = 0; g.wsel1 = 1;
+            return launch_group_glu_a16(g, st);
+        }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85: encoding %u arm %u is not served", enc, arm);
     }
     case PLOW_DOP_MOE_GROUP_DOWN_PF: {
@@ -174,7 +222,118 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_W8A8_P16;
             return launch_group_down_w8a8(g, st);
         }
+        const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
+                         (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
+                         (enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_W4A16);
+        if (a16) {
+            NEED(c, enc == PLOW_MOE_ENC_BF16 || ten(in, T, 3), "op 86: t3 stab must be bound for encoding %u", enc);
+            NEED(c, I % 128u == 0u && H % 128u == 0u, "op 86: I %u and H %u must be multiples of 128", I, H);
+            if (!launch) return 0;
+            GroupA16 g = {};
+            g.out = ten(in, T, 0); g.a = ten(in, T, 1);
+            g.wtab = (const uint64_t*)ten(in, T, 2);
+            g.stab = enc == PLOW_MOE_ENC_BF16 ? nullptr : (const uint64_t*)ten(in, T, 3);
+            g.meta = (const int32_t*)ten(in, T, 4);
+            g.o_idx = (const uint32_t*)ten(in, T, 6); g.gate = (const float*)ten(in, T, 7);
+            g.N = H; g.K = I; g.E = E; g.enc = enc;
+            g.wcols = 3; g.wsel0 = 2; g.wsel1 = 2;
+            return launch_group_down_a16(g, st);
+        }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 86: encoding %u arm %u is not served", enc, arm);
+    }
+    case PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF_W8A8: {
+        const uint32_t I = i[0], H = i[1], E = i[2];
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5) && ten(in, T, 6),
+             "op 81: t0 fu, t1 xq8, t2 ewt, t3 meta, t4 row_token, t5 ascale, t6 est must be bound");
+        NEED(c, I && H && E && I % 128u == 0u && H % 128u == 0u, "op 81: I %u and H %u must be non-zero multiples of 128", I, H);
+        NEED(c, i[5] <= 1u, "op 81: activation %u is not served", i[5]);
+        if (!launch) return 0;
+        GroupW8A8 g = {};
+        g.out = ten(in, T, 0); g.a = ten(in, T, 1); g.a_scale = (const float*)ten(in, T, 5);
+        g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 6);
+        g.meta = (const int32_t*)ten(in, T, 3); g.row_token = (const uint32_t*)ten(in, T, 4);
+        g.N = I; g.K = H; g.E = E; g.act = i[5]; g.per_channel = 1;
+        return launch_group_glu_w8a8(g, st);
+    }
+    case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8: {
+        const uint32_t H = i[0], I = i[1], E = i[2];
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5) && ten(in, T, 6) && ten(in, T, 7),
+             "op 82: t0 part, t1 fu8, t2 ewt, t3 meta, t4 row_partidx, t5 row_gate, t6 est, t7 fscale must be bound");
+        NEED(c, I && H && E && I % 128u == 0u && H % 128u == 0u, "op 82: I %u and H %u must be non-zero multiples of 128", I, H);
+        if (!launch) return 0;
+        GroupW8A8 g = {};
+        g.out = ten(in, T, 0); g.a = ten(in, T, 1); g.a_scale = (const float*)ten(in, T, 7);
+        g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 6);
+        g.meta = (const int32_t*)ten(in, T, 3);
+        g.row_partidx = (const uint32_t*)ten(in, T, 4); g.row_gate = (const float*)ten(in, T, 5);
+        g.N = H; g.K = I; g.E = E; g.per_channel = 1;
+        return launch_group_down_w8a8(g, st);
+    }
+    case PLOW_DOP_MOE_GROUP_GLU_FP8_BLK:
+    case PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8:
+    case PLOW_DOP_MOE_GROUP_DOWN_FP8_BLK:
+    case PLOW_DOP_MOE_EXPERT_DOWN_GEMMA_FP8: {
+        /* slot-major decode experts: sort the slots by expert into the context workspace, then run
+         * the grouped kernel with slot-major input / output rows */
+        const bool pc = in->op == PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8 || in->op == PLOW_DOP_MOE_EXPERT_DOWN_GEMMA_FP8;
+        const bool glu = in->op == PLOW_DOP_MOE_GROUP_GLU_FP8_BLK || in->op == PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8;
+        uint32_t nslot, kx, N, K, E, enc, act;
+        if (pc) { /* i0=k i1=N i2=K i3=E i5=B(0 = 1); act: i6 on the GLU (0 gelu_tanh, 1 silu) */
+            nslot = i[0] * (i[5] ? i[5] : 1u); kx = i[0]; N = i[1]; K = i[2]; E = i[3];
+            enc = 3u; act = glu ? i[6] : 0u;
+        } else {  /* i0=slots i1=N i2=K i3=E i4=slots per x row (GLU; 0 = one shared row) i5=act i6=enc */
+            nslot = i[0]; kx = glu ? (i[4] ? i[4] : i[0]) : 1u; N = i[1]; K = i[2]; E = i[3];
+            enc = i[6]; act = glu ? i[5] : 0u;
+        }
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3), "op %u: t0 out, t1 in, t2 table, t3 weight table must be bound", (unsigned)in->op);
+        NEED(c, pc || enc <= 2u, "op %u: encoding %u is not one of bf16 / block-fp8 / mxfp4", (unsigned)in->op, enc);
+        NEED(c, !pc || i[4] == 0u, "op %u: a non-zero slot offset (i4) is not served", (unsigned)in->op);
+        NEED(c, (enc == PLOW_MOE_ENC_BF16 || ten(in, T, 4)), "op %u: scale table t4 must be bound for encoding %u", (unsigned)in->op, enc);
+        NEED(c, nslot && kx && N && K && E && N % 128u == 0u && K % 128u == 0u, "op %u: N %u and K %u must be non-zero multiples of 128", (unsigned)in->op, N, K);
+        NEED(c, E <= WS_MAX_E && nslot <= WS_MAX_SLOTS, "op %u: %u slots / %u experts exceed the context workspace", (unsigned)in->op, nslot, E);
+        NEED(c, act <= 1u, "op %u: activation %u is not served", (unsigned)in->op, act);
+        if (!launch) return 0;
+        /* align with k = slots per input row: row_token = slot / kx, row_partidx = slot */
+        int rc = launch_align(c->ws_meta, ten(in, T, 2), c->ws_row_token, c->ws_row_partidx, c->ws_row_gate,
+                              (nslot + kx - 1u) / kx, E, kx, st);
+        if (rc) return rc;
+        GroupA16 g = {};
+        g.out = ten(in, T, 0); g.a = ten(in, T, 1);
+        g.wtab = (const uint64_t*)ten(in, T, 3);
+        g.stab = enc == PLOW_MOE_ENC_BF16 ? nullptr : (const uint64_t*)ten(in, T, 4);
+        g.meta = c->ws_meta;
+        g.N = N; g.K = K; g.E = E; g.enc = enc; g.act = act;
+        g.wcols = pc ? 2u : 3u;
+        g.o_idx = c->ws_row_partidx;
+        if (glu) {
+            g.a_idx = c->ws_row_token;
+            g.wsel0 = 0; g.wsel1 = pc ? 0u : 1u; g.wrow1 = pc ? N : 0u;
+            return launch_group_glu_a16(g, st);
+        }
+        g.a_idx = c->ws_row_partidx; g.gate = c->ws_row_gate;
+        g.wsel0 = g.wsel1 = pc ? 1u : 2u;
+        rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), g.wtab, g.stab, g.wcols, g.wsel0, nslot, E, N, st);
+        if (rc) return rc;
+        return launch_group_down_a16(g, st);
+    }
+    case PLOW_DOP_GEMM_GLU:
+    case PLOW_DOP_GEMM: {
+        /* dense bf16 shared expert: one "expert" whose rows are the tokens themselves */
+        const bool glu = in->op == PLOW_DOP_GEMM_GLU;
+        const uint32_t M = i[0], N = i[1], K = i[2];
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && (!glu || ten(in, T, 5)), "op %u: output, input and weight tensors must be bound", (unsigned)in->op);
+        NEED(c, !ten(in, T, 6) && !ten(in, T, 7), "op %u: the bias operands are not on this path", (unsigned)in->op);
+        NEED(c, glu || (!ten(in, T, 3) && !ten(in, T, 4)), "op 8: the folded-norm operands are not on this path");
+        NEED(c, M && N && K && N % 128u == 0u && K % 128u == 0u, "op %u: N %u and K %u must be non-zero multiples of 128", (unsigned)in->op, N, K);
+        NEED(c, !glu || i[5] <= 1u, "op 20: activation %u is not served", i[5]);
+        if (!launch) return 0;
+        GroupA16 g = {};
+        g.out = (char*)ten(in, T, 0) + (glu ? 0u : (size_t)i[5] * N * 2u);
+        g.a = (const char*)ten(in, T, 1) + (glu ? 0u : (size_t)i[4] * K * 2u);
+        g.wdirect[0] = ten(in, T, 2); g.wdirect[1] = glu ? ten(in, T, 5) : ten(in, T, 2);
+        g.N = N; g.K = K; g.E = 1; g.enc = 0; g.act = glu ? i[5] : 0u;
+        g.wcols = 1; g.out_bf16 = 1; g.dense_rows = M;
+        return glu ? launch_group_glu_a16(g, st) : launch_group_down_a16(g, st);
     }
     default:
         return fail(c, PLOW_MOE_EUNSUPPORTED, "opcode %u is not served by this library", (unsigned)in->op);

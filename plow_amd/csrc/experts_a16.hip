@@ -1,0 +1,261 @@
+/* experts_a16.hip — grouped expert GEMMs with bf16 activations: bf16 weights (enc 0), block-fp8
+ * weights with 128x128 f32 scales (enc 1, arm 0), mxfp4 weights (enc 2, arm 8) and per-output-channel
+ * fp8 weights (ops 65 / 66). Also serves the dense bf16 shared expert (ops 20 / 8) as a one-expert
+ * group.
+ *
+ * Arithmetic, per weight encoding (the weight is decoded EXACTLY to bf16, the product runs on the bf16
+ * matrix cores with f32 accumulation):
+ *   bf16        acc = sum_k w * x                      plow runtime/cpu/dev/golden/moe_gemma.c:35-39
+ *   block-fp8   per 128-K block t = sum w * x, acc += t * S[n/128][kb]
+ *                                                       plow runtime/amd/op_moe.h:3299-3310, :674-702
+ *   mxfp4       w = e2m1 * 2^(s-127) folded exactly into the bf16 operand (one E8M0 per 32 k)
+ *                                                       plow runtime/cpu/dev/mxfp4_common.h:30-40,
+ *                                                       runtime/amd/op_moe.h:843-964
+ *   fp8 / chan  acc = (sum_k w * x) * sc[n]             plow runtime/cpu/dev/golden/fp8.c:33-41, :173-214
+ * GLU: out = bf16(act(gate) * up); DOWN: out = gate_r * acc as f32 (or bf16 for the dense op 8).
+ *
+ * WEIGHT-STREAMING KERNEL, same shape as the fp8 x fp8 one: workgroup = (expert, 128 output channels),
+ * 8 waves x 16 channels, weights are the A operand of v_mfma_f32_16x16x32_bf16 (lane = (channel c,
+ * k-chunk q)), read from global memory DEPTH 128-k steps ahead and decoded in registers; the
+ * expert's rows are the B operand. A 128-k step is four matrix instructions of 32 k. The k order
+ * inside a step is permuted identically for both operands so that every load is 16 bytes per lane:
+ *   bf16 weights  instruction j of the step uses k = 32 j + 8 q .. + 8
+ *   fp8 weights   the lane's 32 bytes are [16q, 16q+16) and [64+16q, 64+16q+16); instruction j uses
+ *                 its bytes 8 j .. 8 j + 8
+ *   mxfp4         the lane's 16 bytes are one whole MX block, k = 32 q .. 32 q + 32; instruction j
+ *                 uses values 8 j .. 8 j + 8
+ * Rows are addressed through two index arrays so that one kernel serves the gathered (ops 85 / 86)
+ * and the slot-major (ops 48 / 49 / 65 / 66, after an internal sort by expert) layouts:
+ * a_idx[r] = row of `a` feeding aligned row r, o_idx[r] = output row; ~0 marks a pad row.
+ */
+#include "common.h"
+#include "kernels.h"
+
+#define AK_WAVES 8u
+#define AK_THREADS (AK_WAVES * WAVE)
+#define AK_BN 128u
+
+enum { AENC_BF16 = 0, AENC_FP8BLK = 1, AENC_MXFP4 = 2, AENC_FP8PC = 3 };
+
+template <int ENC> struct WStep;                 /* registers one lane loads per stream and 128-k step */
+template <> struct WStep<AENC_BF16> { v4i r[4]; };
+template <> struct WStep<AENC_FP8BLK> { v4i r[2]; };
+template <> struct WStep<AENC_FP8PC> { v4i r[2]; };
+template <> struct WStep<AENC_MXFP4> { v4i r[1]; uint32_t s; };
+
+/* byte offset inside the 128-k step of the activation piece instruction j needs (16 bytes, 8 bf16) */
+template <int ENC>
+__device__ __forceinline__ uint32_t x_off(uint32_t q, int j) {
+    if (ENC == AENC_BF16) return (32u * j + 8u * q) * 2u;
+    if (ENC == AENC_MXFP4) return (32u * q + 8u * j) * 2u;
+    return ((j < 2 ? 16u * q + 8u * j : 64u + 16u * q + 8u * (j - 2))) * 2u;
+}
+
+template <int ENC>
+__device__ __forceinline__ void w_issue(WStep<ENC>& d, const uint8_t* w, const uint8_t* s, uint32_t kb,
+                                        uint32_t q) {
+    if (ENC == AENC_BF16) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) d.r[j] = *(const v4i*)(w + (size_t)kb * 256u + (32u * j + 8u * q) * 2u);
+    } else if (ENC == AENC_MXFP4) {
+        d.r[0] = *(const v4i*)(w + (size_t)kb * 64u + 16u * q);
+        ((WStep<AENC_MXFP4>&)d).s = s[kb * 4u + q];
+    } else {
+        d.r[0] = *(const v4i*)(w + (size_t)kb * 128u + 16u * q);
+        d.r[1] = *(const v4i*)(w + (size_t)kb * 128u + 64u + 16u * q);
+    }
+}
+
+/* 8 bf16 operand values of instruction j from a lane's step registers */
+template <int ENC>
+__device__ __forceinline__ v8bf w_operand(const WStep<ENC>& d, int j) {
+    if (ENC == AENC_BF16) {
+        return __builtin_bit_cast(v8bf, d.r[j]);
+    } else if (ENC == AENC_MXFP4) {
+        const float sc = __uint_as_float(((const WStep<AENC_MXFP4>&)d).s << 23); /* E8M0: 2^(s-127) */
+        const uint32_t wd = (uint32_t)d.r[0][j];                                 /* 8 nibbles, low = even k */
+        const v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 0);
+        const v2bf p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 1);
+        const v2bf p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 2);
+        const v2bf p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 3);
+        return (v8bf){p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+    } else {
+        const uint32_t lo = (uint32_t)d.r[j >> 1][(j & 1) * 2], hi = (uint32_t)d.r[j >> 1][(j & 1) * 2 + 1];
+        const v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+        const v2bf p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+        const v2bf p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+        const v2bf p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+        return (v8bf){p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+    }
+}
+
+template <int ENC> struct DepthA { static constexpr int v = 2; };
+template <> struct DepthA<AENC_MXFP4> { static constexpr int v = 3; };
+
+template <int ENC, bool GLU>
+__device__ __forceinline__ void ak_body(const GroupA16& g, uint32_t e, uint32_t ct, uint32_t r0,
+                                        uint32_t rb, uint32_t cnt) {
+    constexpr int D = DepthA<ENC>::v;
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6, c = lane & 15u, q = lane >> 4;
+    const uint32_t K = g.K, KB = K / 128u, N = g.N;
+    const uint32_t ch = ct * AK_BN + wv * 16u + c; /* this lane's weight row */
+    /* bytes per weight row and per scale row */
+    const size_t wrow = ENC == AENC_BF16 ? (size_t)K * 2u : (ENC == AENC_MXFP4 ? K / 2u : K);
+    const uint64_t* wt = g.wtab ? g.wtab + (size_t)e * g.wcols : nullptr;
+    const uint64_t* stt = g.stab ? g.stab + (size_t)e * g.wcols : nullptr;
+    const uint8_t* wbase0 = wt ? (const uint8_t*)(uintptr_t)wt[g.wsel0] : (const uint8_t*)g.wdirect[0];
+    const uint8_t* wbase1 = wt ? (const uint8_t*)(uintptr_t)wt[g.wsel1] : (const uint8_t*)g.wdirect[1];
+    const uint8_t* w0 = wbase0 + (size_t)(ch + g.wrow0) * wrow;
+    const uint8_t* w1 = GLU ? wbase1 + (size_t)(ch + g.wrow1) * wrow : nullptr;
+    const uint8_t* sb0 = stt ? (const uint8_t*)(uintptr_t)stt[g.wsel0] : nullptr;
+    const uint8_t* sb1 = (GLU && stt) ? (const uint8_t*)(uintptr_t)stt[g.wsel1] : nullptr;
+    const uint8_t *ms0 = nullptr, *ms1 = nullptr; /* mxfp4: this row's E8M0 bytes */
+    const float *bs0 = nullptr, *bs1 = nullptr;   /* block-fp8: this channel block's scale row */
+    if (ENC == AENC_MXFP4) {
+        ms0 = sb0 + (size_t)(ch + g.wrow0) * (K / 32u);
+        if (GLU) ms1 = sb1 + (size_t)(ch + g.wrow1) * (K / 32u);
+    }
+    if (ENC == AENC_FP8BLK) {
+        bs0 = (const float*)sb0 + (size_t)((ct * AK_BN + g.wrow0) / 128u) * KB;
+        if (GLU) bs1 = (const float*)sb1 + (size_t)((ct * AK_BN + g.wrow1) / 128u) * KB;
+    }
+
+    /* the B-operand row of this lane */
+    const uint32_t off = rb + c, r = r0 + off;
+    bool valid = off < cnt;
+    const uint32_t ai = valid ? (g.a_idx ? g.a_idx[r] : r) : PLOW_EXPERT_UNUSED;
+    valid = ai != PLOW_EXPERT_UNUSED;
+    const uint8_t* ap = (const uint8_t*)g.a + (size_t)(valid ? ai : 0u) * K * 2u;
+
+    WStep<ENC> wa[D], wb[D];
+    v4i xa[D][4];
+    float sa[D], sbv[D];
+    auto issue = [&](int d, uint32_t kb) {
+        w_issue<ENC>(wa[d], w0, ms0, kb, q);
+        if (GLU) w_issue<ENC>(wb[d], w1, ms1, kb, q);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            xa[d][j] = (v4i){0, 0, 0, 0};
+            if (valid) xa[d][j] = *(const v4i*)(ap + (size_t)kb * 256u + x_off<ENC>(q, j));
+        }
+        if (ENC == AENC_FP8BLK) {
+            sa[d] = bs0[kb];
+            if (GLU) sbv[d] = bs1[kb];
+        }
+    };
+
+    v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if ((uint32_t)d < KB) issue(d, (uint32_t)d);
+    for (uint32_t kb0 = 0; kb0 < KB; kb0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            const uint32_t kb = kb0 + (uint32_t)d;
+            if (kb < KB) {
+                v4f t0 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc0;
+                v4f t1 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc1;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const v8bf B = __builtin_bit_cast(v8bf, xa[d][j]);
+                    t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(wa[d], j), B, t0, 0, 0, 0);
+                    if (GLU) t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(wb[d], j), B, t1, 0, 0, 0);
+                }
+                if (ENC == AENC_FP8BLK) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        acc0[i] = fmaf(t0[i], sa[d], acc0[i]);
+                        if (GLU) acc1[i] = fmaf(t1[i], sbv[d], acc1[i]);
+                    }
+                } else {
+                    acc0 = t0;
+                    if (GLU) acc1 = t1;
+                }
+                if (kb + D < KB) issue(d, kb + D);
+            }
+        }
+    }
+
+    /* ---- epilogue: lane holds channels ct*128 + wv*16 + 4q + i of row c ---- */
+    if (!valid) return;
+    const uint32_t col = ct * AK_BN + wv * 16u + 4u * q;
+    if (ENC == AENC_FP8PC) {
+        const float* sc0 = (const float*)sb0 + g.wrow0 + col;
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc0[i] *= sc0[i];
+        if (GLU) {
+            const float* sc1 = (const float*)sb1 + g.wrow1 + col;
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc1[i] *= sc1[i];
+        }
+    }
+    const uint32_t oi = g.o_idx ? g.o_idx[r] : r;
+    if (oi == PLOW_EXPERT_UNUSED) return;
+    if (GLU) {
+        uint2 o;
+        o.x = (uint32_t)f2bf(moe_glu(acc0[0], acc1[0], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[1], acc1[1], g.act)) << 16);
+        o.y = (uint32_t)f2bf(moe_glu(acc0[2], acc1[2], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[3], acc1[3], g.act)) << 16);
+        *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
+    } else {
+        const float gate = g.gate ? g.gate[r] : 1.0f;
+        const float y0 = gate * acc0[0], y1 = gate * acc0[1], y2 = gate * acc0[2], y3 = gate * acc0[3];
+        if (g.out_bf16) {
+            uint2 o;
+            o.x = (uint32_t)f2bf(g.gate ? y0 : acc0[0]) | ((uint32_t)f2bf(g.gate ? y1 : acc0[1]) << 16);
+            o.y = (uint32_t)f2bf(g.gate ? y2 : acc0[2]) | ((uint32_t)f2bf(g.gate ? y3 : acc0[3]) << 16);
+            *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
+        } else {
+            *(float4*)((float*)g.out + (size_t)oi * N + col) = make_float4(y0, y1, y2, y3);
+        }
+    }
+}
+
+template <int ENC, bool GLU>
+__global__ __launch_bounds__(AK_THREADS) void k_group_a16_stream(GroupA16 g) {
+    const uint32_t tiles = g.N / AK_BN;
+    const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
+    const uint32_t cnt = g.meta ? (uint32_t)g.meta[g.E + e] : g.dense_rows;
+    if (cnt == 0u) return;
+    if (g.wtab && g.wtab[(size_t)e * g.wcols + g.wsel0] == 0ull) return; /* expert not resident: skipped */
+    if (g.stab && ENC != AENC_BF16 && g.stab[(size_t)e * g.wcols + g.wsel0] == 0ull) return;
+    const uint32_t r0 = g.meta ? (uint32_t)g.meta[e] : 0u;
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) ak_body<ENC, GLU>(g, e, ct, r0, rb, cnt);
+}
+
+template <bool GLU>
+static int launch_a16(const GroupA16& g, hipStream_t st) {
+    if (g.N == 0 || g.K == 0 || g.E == 0 || g.N % AK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
+    if ((uint64_t)g.E * (g.N / AK_BN) > 0x7FFFFFFFull) return PLOW_MOE_EINVAL;
+    const dim3 grid(g.E * (g.N / AK_BN));
+    switch (g.enc) {
+    case AENC_BF16: k_group_a16_stream<AENC_BF16, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
+    case AENC_FP8BLK: k_group_a16_stream<AENC_FP8BLK, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
+    case AENC_MXFP4: k_group_a16_stream<AENC_MXFP4, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
+    case AENC_FP8PC: k_group_a16_stream<AENC_FP8PC, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
+    default: return PLOW_MOE_EUNSUPPORTED;
+    }
+    return 0;
+}
+
+int launch_group_glu_a16(const GroupA16& g, hipStream_t st) { return launch_a16<true>(g, st); }
+int launch_group_down_a16(const GroupA16& g, hipStream_t st) { return launch_a16<false>(g, st); }
+
+/* Slot-major ops: zero part[s][*] of every slot that no expert serves (sentinel id or a null weight
+ * base), which the reference's decode DOWN bodies do (plow runtime/cpu/dev/golden/moe.c:76-80). */
+__global__ __launch_bounds__(256) void k_zero_skipped(float* part, const PlowMoeRoute* table,
+                                                      const uint64_t* wtab, const uint64_t* stab,
+                                                      uint32_t wcols, uint32_t wsel, uint32_t nslot,
+                                                      uint32_t E, uint32_t H) {
+    const uint32_t s = blockIdx.x;
+    if (s >= nslot) return;
+    const uint32_t e = table[s].eid;
+    if (e < E && wtab[(size_t)e * wcols + wsel] != 0ull && (!stab || stab[(size_t)e * wcols + wsel] != 0ull)) return;
+    for (uint32_t h = threadIdx.x; h < H; h += 256u) part[(size_t)s * H + h] = 0.0f;
+}
+
+int launch_zero_skipped(float* part, const void* table, const uint64_t* wtab, const uint64_t* stab,
+                        uint32_t wcols, uint32_t wsel, uint32_t nslot, uint32_t E, uint32_t H, hipStream_t st) {
+    if (nslot == 0) return 0;
+    k_zero_skipped<<<nslot, 256, 0, st>>>(part, (const PlowMoeRoute*)table, wtab, stab, wcols, wsel, nslot, E, H);
+    return 0;
+}

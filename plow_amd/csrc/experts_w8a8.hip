@@ -34,16 +34,20 @@
 
 __device__ __forceinline__ v4i ldg16(const uint8_t* p) { return *(const v4i*)p; }
 
-template <int RT, bool GLU, int D>
+template <int RT, bool GLU, int D, bool PC>
 __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t ct, uint32_t r0,
                                         uint32_t rb, uint32_t cnt, float* s_red) {
     const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6, c = lane & 15u, q = lane >> 4;
     const uint32_t K = g.K, KB = K / 128u, N = g.N;
     const uint32_t ch = ct * SK_BN + wv * 16u + c; /* this lane's weight row */
-    const uint8_t* w0 = (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * 3u + (GLU ? 0u : 2u)] + (size_t)ch * K + 16u * q;
-    const uint8_t* w1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * 3u + 1u] + (size_t)ch * K + 16u * q : nullptr;
-    const float* s0 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u + (GLU ? 0u : 2u)] + (size_t)ct * KB;
-    const float* s1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * 3u + 1u] + (size_t)ct * KB : nullptr;
+    /* block mode: {gate, up, down} tables, scale rows [N/128][KB]; per-channel mode: {gate_up fused,
+     * down} tables (up rows follow the N gate rows), one f32 scale per weight row */
+    const uint32_t wcols = PC ? 2u : 3u, sel0 = PC ? (GLU ? 0u : 1u) : (GLU ? 0u : 2u), sel1 = PC ? 0u : 1u;
+    const uint8_t* w0 = (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * wcols + sel0] + (size_t)ch * K + 16u * q;
+    const uint8_t* w1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * wcols + sel1] +
+                                  (size_t)(ch + (PC ? N : 0u)) * K + 16u * q : nullptr;
+    const float* s0 = (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel0] + (PC ? 0u : (size_t)ct * KB);
+    const float* s1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel1] + (PC ? (size_t)N : (size_t)ct * KB) : nullptr;
 
     /* B operand rows of this lane, one per row tile */
     const uint8_t* ap[RT];
@@ -62,6 +66,12 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             const uint32_t t = valid[rt] ? tok : 0u;
             ap[rt] = (const uint8_t*)g.a + (size_t)t * K + 16u * q;
             asp[rt] = g.a_scale + t;
+        } else if (PC) {
+            const uint32_t pi = valid[rt] ? g.row_partidx[rowidx[rt]] : PLOW_EXPERT_UNUSED;
+            valid[rt] = pi != PLOW_EXPERT_UNUSED;
+            const uint32_t r = valid[rt] ? rowidx[rt] : r0;
+            ap[rt] = (const uint8_t*)g.a + (size_t)r * K + 16u * q;
+            asp[rt] = g.a_scale + r;
         } else {
             const uint32_t pi = valid[rt] ? g.row_partidx[rowidx[rt]] : PLOW_EXPERT_UNUSED;
             valid[rt] = pi != PLOW_EXPERT_UNUSED;
@@ -90,11 +100,13 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             if (valid[rt]) {
                 xa[d][rt][0] = ldg16(ap[rt] + ko);
                 xa[d][rt][1] = ldg16(ap[rt] + ko + 64u);
-                xs[d][rt] = asp[rt][(size_t)kb * as_stride];
+                if (!PC) xs[d][rt] = asp[rt][(size_t)kb * as_stride];
             }
         }
-        sa[d] = s0[kb];
-        if (GLU) sb[d] = s1[kb];
+        if (!PC) {
+            sa[d] = s0[kb];
+            if (GLU) sb[d] = s1[kb];
+        }
     };
 
     v4f acc0[RT], acc1[RT];
@@ -117,16 +129,21 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) {
                     const v8i B = __builtin_shufflevector(xa[d][rt][0], xa[d][rt][1], 0, 1, 2, 3, 4, 5, 6, 7);
-                    const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
-                    const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A0, B, z, 0, 0, 0, 0, 0, 0);
-                    const float sc0 = xs[d][rt] * sa[d];
+                    if (PC) { /* scales are outside the K reduction: accumulate straight through */
+                        acc0[rt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A0, B, acc0[rt], 0, 0, 0, 0, 0, 0);
+                        if (GLU) acc1[rt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, acc1[rt], 0, 0, 0, 0, 0, 0);
+                    } else {
+                        const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
+                        const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A0, B, z, 0, 0, 0, 0, 0, 0);
+                        const float sc0 = xs[d][rt] * sa[d];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) acc0[rt][i] = fmaf(t0[i], sc0, acc0[rt][i]);
-                    if (GLU) {
-                        const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, z, 0, 0, 0, 0, 0, 0);
-                        const float sc1 = xs[d][rt] * sb[d];
+                        for (int i = 0; i < 4; i++) acc0[rt][i] = fmaf(t0[i], sc0, acc0[rt][i]);
+                        if (GLU) {
+                            const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, z, 0, 0, 0, 0, 0, 0);
+                            const float sc1 = xs[d][rt] * sb[d];
 #pragma unroll
-                        for (int i = 0; i < 4; i++) acc1[rt][i] = fmaf(t1[i], sc1, acc1[rt][i]);
+                            for (int i = 0; i < 4; i++) acc1[rt][i] = fmaf(t1[i], sc1, acc1[rt][i]);
+                        }
                     }
                 }
                 if (kb + D < KB) issue(d, kb + D);
@@ -136,6 +153,42 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
 
     /* ---- epilogue: lane holds channels ct*128 + wv*16 + 4q + i (i = 0..3) of row c ---- */
     const uint32_t col = ct * SK_BN + wv * 16u + 4u * q;
+    if (PC) {
+        /* per-channel arm (plow runtime/amd/op_moe.h:6655-6700): g = acc * (as * wsc[n]); GLU stores
+         * bf16(act(g) * u) and zeroes pad rows, DOWN stores gate * acc, then * (as * wsc[h]) */
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            const uint32_t off = rb + (uint32_t)rt * 16u + c;
+            if (GLU) {
+                if (!valid[rt]) {
+                    if (off < ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM)
+                        *(uint2*)((bf16_t*)g.out + (size_t)rowidx[rt] * N + col) = make_uint2(0u, 0u);
+                    continue;
+                }
+                const float as = asp[rt][0];
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    o[i] = moe_glu(acc0[rt][i] * (as * s0[col + i]), acc1[rt][i] * (as * s1[col + i]), g.act);
+                uint2 pk;
+                pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
+                pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
+                *(uint2*)((bf16_t*)g.out + (size_t)rowidx[rt] * N + col) = pk;
+            } else {
+                if (!valid[rt]) continue;
+                const uint32_t pidx = g.row_partidx[rowidx[rt]];
+                const float gate = g.row_gate[rowidx[rt]], as = asp[rt][0];
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    o[i] = gate * acc0[rt][i];
+                    o[i] *= as * s0[col + i];
+                }
+                *(float4*)((float*)g.out + (size_t)pidx * N + col) = make_float4(o[0], o[1], o[2], o[3]);
+            }
+        }
+        return;
+    }
     if (GLU) {
         float v[RT][4];
 #pragma unroll
@@ -184,7 +237,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
     }
 }
 
-template <bool GLU, int D>
+template <bool GLU, int D, bool PC>
 __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     __shared__ float s_red[SK_WAVES * 64u];
     const uint32_t tiles = g.N / SK_BN;
@@ -193,11 +246,21 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles;
     const uint32_t cnt = (uint32_t)g.meta[g.E + e];
     if (cnt == 0u) return;
-    if (g.wtab[(size_t)e * 3u + (GLU ? 0u : 2u)] == 0ull) return; /* expert not resident: skipped */
+    if (g.wtab[(size_t)e * (PC ? 2u : 3u) + (PC ? (GLU ? 0u : 1u) : (GLU ? 0u : 2u))] == 0ull) return; /* not resident */
     const uint32_t r0 = (uint32_t)g.meta[e];
     /* 16 rows a pass; an expert with more rows streams its weights once per pass (the tiled
      * kernel, not this one, is the tool for many rows per expert) */
-    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D>(g, e, ct, r0, rb, cnt, s_red);
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D, PC>(g, e, ct, r0, rb, cnt, s_red);
+    if (PC && GLU) {
+        /* the per-channel GLU zeroes the pad rows of its 64-row tile (the partial 16-row pass above
+         * did its own); the row quantizer that follows reads every aligned row */
+        const uint32_t padded = ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
+        const uint32_t first = ((cnt + 15u) / 16u) * 16u;
+        for (uint32_t i = threadIdx.x; i < (padded - first) * (SK_BN / 4u); i += SK_THREADS) {
+            const uint32_t r = r0 + first + i / (SK_BN / 4u), col = ct * SK_BN + (i % (SK_BN / 4u)) * 4u;
+            *(uint2*)((bf16_t*)g.out + (size_t)r * g.N + col) = make_uint2(0u, 0u);
+        }
+    }
 }
 
 /* k-steps of weight loads a wave keeps in flight; PLOW_MOE_SK_DEPTH (2..4) overrides for tuning */
@@ -222,10 +285,11 @@ int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
     const int rc = check_w8a8(g);
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
+    if (g.per_channel) { k_group_w8a8_stream<true, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
     switch (stream_depth()) {
-    case 2: k_group_w8a8_stream<true, 2><<<grid, SK_THREADS, 0, st>>>(g); break;
-    case 4: k_group_w8a8_stream<true, 4><<<grid, SK_THREADS, 0, st>>>(g); break;
-    default: k_group_w8a8_stream<true, 3><<<grid, SK_THREADS, 0, st>>>(g); break;
+    case 2: k_group_w8a8_stream<true, 2, false><<<grid, SK_THREADS, 0, st>>>(g); break;
+    case 4: k_group_w8a8_stream<true, 4, false><<<grid, SK_THREADS, 0, st>>>(g); break;
+    default: k_group_w8a8_stream<true, 3, false><<<grid, SK_THREADS, 0, st>>>(g); break;
     }
     return 0;
 }
@@ -234,10 +298,11 @@ int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
     const int rc = check_w8a8(g);
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
+    if (g.per_channel) { k_group_w8a8_stream<false, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
     switch (stream_depth()) {
-    case 2: k_group_w8a8_stream<false, 2><<<grid, SK_THREADS, 0, st>>>(g); break;
-    case 4: k_group_w8a8_stream<false, 4><<<grid, SK_THREADS, 0, st>>>(g); break;
-    default: k_group_w8a8_stream<false, 3><<<grid, SK_THREADS, 0, st>>>(g); break;
+    case 2: k_group_w8a8_stream<false, 2, false><<<grid, SK_THREADS, 0, st>>>(g); break;
+    case 4: k_group_w8a8_stream<false, 4, false><<<grid, SK_THREADS, 0, st>>>(g); break;
+    default: k_group_w8a8_stream<false, 3, false><<<grid, SK_THREADS, 0, st>>>(g); break;
     }
     return 0;
 }

@@ -33,8 +33,33 @@ struct GroupW8A8 {
     const uint32_t* row_partidx; /* DOWN */
     const float* row_gate;       /* DOWN */
     uint32_t N, K, E, pitch, act, part16, T;
+    /* per-channel mode (ops 81 / 82): weights through ewt[E][2] = {gate_up fused [2N][K], down [N][K]},
+     * f32 channel scales through est[E][2], one f32 activation scale per row; GLU writes bf16 */
+    uint32_t per_channel;
 };
 int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);
+
+
+/* Grouped experts with bf16 activations (see experts_a16.hip). */
+struct GroupA16 {
+    void* out;              /* GLU: bf16 [rows][N]; DOWN: f32 (or bf16) [rows][N] */
+    const void* a;          /* bf16 [rows][K] */
+    const uint64_t* wtab;   /* [E][wcols] device pointers */
+    const uint64_t* stab;   /* [E][wcols] or NULL (bf16 weights) */
+    const int32_t* meta;    /* rowoff | cnt | tilep, or NULL = one dense expert of dense_rows rows */
+    const uint32_t* a_idx;  /* aligned row -> row of `a` (NULL = identity) */
+    const uint32_t* o_idx;  /* aligned row -> output row (NULL = identity) */
+    const float* gate;      /* DOWN: aligned row -> gate (NULL = 1) */
+    uint32_t N, K, E, enc, act;
+    uint32_t wcols, wsel0, wsel1; /* table width, column of the first / second weight stream */
+    uint32_t wrow0, wrow1;        /* first weight row of each stream inside its tensor (fused gate_up) */
+    uint32_t out_bf16, dense_rows;
+    const void* wdirect[2]; /* used when wtab is NULL: the two weight tensors themselves (dense ops) */
+};
+int launch_group_glu_a16(const GroupA16& g, hipStream_t st);
+int launch_group_down_a16(const GroupA16& g, hipStream_t st);
+int launch_zero_skipped(float* part, const void* table, const uint64_t* wtab, const uint64_t* stab,
+                        uint32_t wcols, uint32_t wsel, uint32_t nslot, uint32_t E, uint32_t H, hipStream_t st);
 
 #endif

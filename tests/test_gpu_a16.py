@@ -1,0 +1,219 @@
+"""bf16-activation expert arms on the GPU against the oracle and the golden vectors of plow's CPU
+kernels: bf16 weights (enc 0), block-fp8 W8A16 (enc 1 arm 0), mxfp4 W4A16 (enc 2 arm 8),
+per-channel fp8 (ops 65 / 66 and the W8A8 pair 81 / 82), the slot-major decode ops 48 / 49 and the
+dense shared expert (ops 20 / 8)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import cases
+import oracle_lib as ol
+from gpu_harness import (assert_output_close, assert_routing_equal, both, dev_table, from_dev, to_dev)
+from plow_amd import abi, layer
+
+pytestmark = pytest.mark.gpu
+
+G = np.load(os.path.join(os.path.dirname(__file__), "golden", "plow_cpu_golden.npz"))
+
+
+@pytest.fixture(scope="module")
+def moe():
+    from plow_amd.lib import Moe
+    m = Moe(0)
+    yield m
+    m.close()
+
+
+def close(a, b, what, max_frac=2e-2, mean_rel=5e-3):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    assert np.all(np.isfinite(a)), what
+    err = np.abs(a - b)
+    mx = err.max() / max(np.abs(b).max(), 1e-30)
+    mr = err.mean() / max(np.abs(b).mean(), 1e-30)
+    print(f"[parity] {what}: max_abs/max|ref| = {mx:.3e}, mean rel = {mr:.3e}", flush=True)
+    assert mx <= max_frac and mr <= mean_rel, (what, mx, mr)
+
+
+def check_chain(plan, dev, host):
+    rows = assert_routing_equal(plan, dev, host)
+    assert np.array_equal(dev.np("logit").view(np.uint32), host.np("logit").view(np.uint32))
+    if "fu" in dev.t:
+        spec_rows = plan.specs["fu"].shape[0]
+        if spec_rows == plan.cfg.R_max:   # gathered layout: compare live rows only
+            live = host.np("row_partidx")[:rows] != abi.EXPERT_UNUSED
+            close(ol.bf2f(dev.np("fu")[:rows][live]), ol.bf2f(host.np("fu")[:rows][live]), "fu")
+        else:
+            close(ol.bf2f(dev.np("fu")), ol.bf2f(host.np("fu")), "fu")
+    close(dev.np("part"), host.np("part"), "part")
+    return assert_output_close(dev.np("out"), host.np("out"))
+
+
+MINI = dict(H=512, E=16, I=256, k=4)
+
+
+@pytest.mark.parametrize("T", [1, 5, 40])
+def test_bf16_layer_with_dense_shared_experts(moe, oracle, T):
+    cfg = layer.MoeConfig("bf16-mini", T=T, scoring="softmax", norm_topk=False, enc="bf16", arm="a16",
+                          n_shared=2, shared_mode="dense", **MINI)
+    plan, dev, host = both(moe, oracle, cfg, seed=T)
+    check_chain(plan, dev, host)
+    close(ol.bf2f(dev.np("shared")), ol.bf2f(host.np("shared")), "shared")
+
+
+@pytest.mark.parametrize("T", [3, 33])
+def test_block_fp8_w8a16_layer(moe, oracle, T):
+    cfg = layer.MoeConfig("w8a16-mini", T=T, scoring="sigmoid", norm_topk=True, bias=True, n_group=4,
+                          topk_group=2, route_scale=2.5, enc="fp8blk", arm="a16", n_shared=1,
+                          shared_mode="fold", residual=True, **MINI)
+    check_chain(*both(moe, oracle, cfg, seed=T))
+
+
+@pytest.mark.parametrize("T", [1, 16, 70])
+def test_mxfp4_w4a16_layer(moe, oracle, T):
+    cfg = layer.MoeConfig("mxfp4-mini", T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          route_scale=2.827, enc="mxfp4", arm="a16", n_shared=1, shared_mode="fold", **MINI)
+    check_chain(*both(moe, oracle, cfg, seed=T))
+
+
+@pytest.mark.parametrize("arm", ["a16", "w8a8"])
+@pytest.mark.parametrize("T", [2, 50])
+def test_per_channel_fp8_layer(moe, oracle, T, arm):
+    cfg = layer.MoeConfig("fp8pc-mini", T=T, scoring="softmax", norm_topk=True, enc="fp8pc", arm=arm, **MINI)
+    plan, dev, host = both(moe, oracle, cfg, seed=T)
+    if arm == "w8a8":
+        assert np.array_equal(dev.np("xq"), host.np("xq"))
+        assert np.array_equal(dev.np("ascale").view(np.uint32), host.np("ascale").view(np.uint32))
+    check_chain(plan, dev, host)
+
+
+def test_mxfp4_decode_ops_match_plow_cpu_golden(moe):
+    """Ops 48 / 49 at enc 2 against vectors written by plow's flat mxfp4 kernels (ops 150 / 151),
+    including a sentinel slot (GLU writes nothing, DOWN writes zeros)."""
+    Wgu, Sgu, Wd, Sd = (to_dev(G[f"mxdec/{n}"]) for n in ("Wgu", "Sgu", "Wd", "Sd"))
+    x, tab = to_dev(G["mxdec/x"]), to_dev(G["mxdec/table"].view(np.int32))
+    E, I2, K2 = G["mxdec/Wgu"].shape
+    I, K, B, k = I2 // 2, K2 * 2, G["mxdec/x"].shape[0], 2
+    es = Wgu.element_size()
+    wtab = torch.tensor([[Wgu[e].data_ptr(), Wgu[e].data_ptr() + I * (K // 2), Wd[e].data_ptr()] for e in range(E)],
+                        dtype=torch.int64).cuda()
+    stab = torch.tensor([[Sgu[e].data_ptr(), Sgu[e].data_ptr() + I * (K // 32), Sd[e].data_ptr()] for e in range(E)],
+                        dtype=torch.int64).cuda()
+    # geometry of the fixture is below the kernels' 128-multiples: expect a typed refusal, not a launch
+    fu = torch.full((B * k, I), 0x1234, dtype=torch.int16, device="cuda")
+    inst = abi.inst(abi.OP_MOE_GROUP_GLU_FP8_BLK, t=[0, 1, 2, 3, 4], i=[B * k, I, K, E, k, 1, 2])
+    assert moe.check(inst, dev_table([fu, x, tab, wtab, stab])) == abi.E_INVAL
+
+
+def run_decode_pair(moe, oracle, enc, seed, nslot_rows=(3, 2), pc=False):
+    """Slot-major decode ops on random data incl. a sentinel slot and a non-resident expert."""
+    r = cases.rng_of(seed)
+    B, k = nslot_rows
+    E, H, I = 6, 256, 128
+    def weights(N, K):
+        if enc == abi.ENC_BF16:
+            return cases.randn_bf16(r, (N, K), 0.05), None
+        if enc == abi.ENC_MXFP4:
+            return (r.integers(0, 256, (N, K // 2), dtype=np.uint8), r.integers(120, 128, (N, K // 32), dtype=np.uint8))
+        if pc:
+            return cases.e4m3_bytes(r, (N, K)), (r.random(N) * 0.01 + 1e-3).astype(np.float32)
+        return cases.e4m3_bytes(r, (N, K)), (r.random(((N + 127) // 128, K // 128)) * 0.02 + 1e-3).astype(np.float32)
+    mats = []
+    for _ in range(E):
+        if pc:
+            mats.append([weights(2 * I, H), weights(H, I)])
+        else:
+            mats.append([weights(I, H), weights(I, H), weights(H, I)])
+    x = cases.randn_bf16(r, (B, H), 1.0)
+    tab = np.zeros(B * k, dtype=ol.ROUTE_DT)
+    tab["eid"] = r.integers(0, E, B * k)
+    tab["eid"][1] = abi.EXPERT_UNUSED
+    tab["eid"][2] = 4                       # expert 4 is not resident
+    tab["gate"] = (r.random(B * k) + 0.1).astype(np.float32)
+    ncol = 2 if pc else 3
+    def tables(get_ptr):
+        wt = np.zeros((E, ncol), np.uint64)
+        st = np.zeros((E, ncol), np.uint64)
+        for e in range(E):
+            for j in range(ncol):
+                wt[e, j] = get_ptr(mats[e][j][0])
+                st[e, j] = 0 if mats[e][j][1] is None else get_ptr(mats[e][j][1])
+        wt[4] = 0
+        return wt, st
+    if pc:
+        glu = abi.inst(abi.OP_MOE_EXPERT_GLU_GEMMA_FP8, t=[0, 1, 2, 3, 4], i=[k, I, H, E, 0, B, 1])
+        down = abi.inst(abi.OP_MOE_EXPERT_DOWN_GEMMA_FP8, t=[0, 1, 2, 3, 4], i=[k, H, I, E, 0, B])
+    else:
+        st_h = 4 if enc != abi.ENC_BF16 else None
+        glu = abi.inst(abi.OP_MOE_GROUP_GLU_FP8_BLK, t=[0, 1, 2, 3, st_h], i=[B * k, I, H, E, k, 1, enc])
+        down = abi.inst(abi.OP_MOE_GROUP_DOWN_FP8_BLK, t=[0, 1, 2, 3, st_h], i=[B * k, H, I, E, 0, 0, enc])
+    # oracle
+    wt, st = tables(lambda a: a.ctypes.data)
+    fu_h = np.full((B * k, I), 0x1234, np.uint16)
+    part_h = np.full((B * k, H), 9.0, np.float32)
+    ol.run(oracle.plow_oracle_exec, glu, ol.table_of([fu_h, x, tab, wt, st]), 2)
+    ol.run(oracle.plow_oracle_exec, down, ol.table_of([part_h, fu_h, tab, wt, st]), 2)
+    # device
+    keep = []
+    def dptr(a):
+        t = to_dev(a)
+        keep.append(t)
+        return t.data_ptr()
+    wtd, std = tables(dptr)
+    fu_d = torch.full((B * k, I), 0x1234, dtype=torch.int16, device="cuda")
+    part_d = torch.full((B * k, H), 9.0, dtype=torch.float32, device="cuda")
+    tbl = [None, to_dev(x), to_dev(tab), to_dev(wtd), to_dev(std)]
+    print(f"[case] decode pair enc={enc} pc={pc}", flush=True)
+    moe.exec(glu, dev_table([fu_d] + tbl[1:]))
+    # DOWN reads the oracle's fu so that only the DOWN arithmetic is compared
+    moe.exec(down, dev_table([part_d, to_dev(fu_h)] + tbl[2:]))
+    torch.cuda.synchronize()
+    fu_g = fu_d.cpu().numpy().view(np.uint16)
+    served = np.array([e < E and e != 4 for e in tab["eid"]])
+    assert np.all(fu_g[~served] == 0x1234)                   # skipped slots: GLU writes nothing
+    close(ol.bf2f(fu_g[served]), ol.bf2f(fu_h[served]), "fu")
+    part_g = part_d.cpu().numpy()
+    assert np.all(part_g[~served] == 0.0)                    # skipped slots: DOWN writes zeros
+    close(part_g, part_h, "part", mean_rel=1e-4, max_frac=1e-4)
+
+
+@pytest.mark.parametrize("enc", [abi.ENC_BF16, abi.ENC_FP8BLK, abi.ENC_MXFP4])
+def test_slot_major_decode_ops(moe, oracle, enc):
+    run_decode_pair(moe, oracle, enc, seed=20 + enc)
+    run_decode_pair(moe, oracle, enc, seed=30 + enc, nslot_rows=(1, 8))
+
+
+def test_per_channel_decode_ops(moe, oracle):
+    run_decode_pair(moe, oracle, abi.ENC_FP8BLK, seed=41, pc=True)
+
+
+def test_dense_ops_match_plow_cpu_golden_shape_rules(moe):
+    """The dense fixture (N 48) is below the kernels' 128-multiple rule: typed refusal."""
+    x, wg = to_dev(G["dense/x"]), to_dev(G["dense/wg"])
+    M, K = G["dense/x"].shape
+    N = G["dense/wg"].shape[0]
+    fu = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+    inst = abi.inst(abi.OP_GEMM_GLU, t=[0, 1, 2, None, None, 5], i=[M, N, K, 0, 0, 1])
+    assert moe.check(inst, dev_table([fu, x, wg, None, None, wg])) == abi.E_INVAL
+
+
+def test_dense_ops_against_oracle(moe, oracle):
+    r = cases.rng_of(50)
+    M, N, K = 37, 256, 384
+    x = cases.randn_bf16(r, (M + 2, K), 1.0)
+    wg, wu, wd = cases.randn_bf16(r, (N, K), 0.05), cases.randn_bf16(r, (N, K), 0.05), cases.randn_bf16(r, (K, N), 0.05)
+    glu = abi.inst(abi.OP_GEMM_GLU, t=[0, 1, 2, None, None, 5], i=[M + 2, N, K, 0, 0, 1])
+    gemm = abi.inst(abi.OP_GEMM, t=[0, 1, 2], i=[M, K, N, 0, 2, 1])   # a_row0 = 2, c_row0 = 1
+    fu_h, y_h = np.zeros((M + 2, N), np.uint16), np.zeros((M + 1, K), np.uint16)
+    ol.run(oracle.plow_oracle_exec, glu, ol.table_of([fu_h, x, wg, None, None, wu]), 4)
+    ol.run(oracle.plow_oracle_exec, gemm, ol.table_of([y_h, fu_h, wd]), 4)
+    fu_d = torch.zeros((M + 2, N), dtype=torch.int16, device="cuda")
+    y_d = torch.zeros((M + 1, K), dtype=torch.int16, device="cuda")
+    moe.exec(glu, dev_table([fu_d, to_dev(x), to_dev(wg), None, None, to_dev(wu)]))
+    moe.exec(gemm, dev_table([y_d, to_dev(fu_h), to_dev(wd)]))
+    torch.cuda.synchronize()
+    close(ol.bf2f(fu_d.cpu().numpy().view(np.uint16)), ol.bf2f(fu_h), "dense fu")
+    yg = y_d.cpu().numpy().view(np.uint16)
+    assert np.all(yg[0] == 0)
+    close(ol.bf2f(yg[1:]), ol.bf2f(y_h[1:]), "dense y")
