@@ -110,7 +110,11 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{cfg.name}: H={cfg.H} E={cfg.E}+{cfg.n_shared} I={cfg.I} top{cfg.k} "
                                f"T={cfg.T} enc={cfg.enc} arm={cfg.arm} groups={cfg.n_group}/{cfg.topk_group}",
-                   "tokens": T, "experts_hit": hit, "rows": int(cnt.sum())},
+                   "tokens": T, "experts_hit": hit, "rows": int(cnt.sum()),
+                   "rows_per_expert": {"min": int(cnt[:cfg.E].min()), "median": float(np.median(cnt[:cfg.E])),
+                                       "max": int(cnt[:cfg.E].max()), "mean": float(cnt[:cfg.E].mean()),
+                                       "below_64": int((cnt[:cfg.E] < 64).sum()),
+                                       "pad_frac": round(float(((cnt + 63) // 64 * 64).sum() / max(1, cnt.sum()) - 1.0), 4)}},
         "tokens_per_s": round(T / (ms * 1e-3), 1),
         "layer": {"algorithmic_bytes": int(layer_bytes), "hbm_frac": round(layer_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                   "flops": flops, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / FP8_PEAK_TFLOPS, 4)},

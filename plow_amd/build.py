@@ -23,6 +23,7 @@ SOURCES = {
     "quant.hip": ["-ffp-contract=off"],
     "experts_w8a8.hip": [],
     "experts_a16.hip": [],
+    "experts_w8a8_tiled.hip": [],
     "api.hip": [],
 }
 

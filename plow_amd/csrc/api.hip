@@ -8,6 +8,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -24,6 +25,12 @@ struct PlowMoeCtx {
     int device;
     int min_rows[2]; /* [0] prefill, [1] decode; < 0 unset */
     char err[256];
+    /* which form of the block-fp8 x fp8 kernels serves ops 85 / 86: 0 weight-streaming (few rows per
+     * expert), 1 tiled (many). Decided at the GLU from its row pitch (op 86 carries no row count and
+     * follows the GLU before it on this context); the segment entry points set it from their variant;
+     * PLOW_MOE_W8A8_KERNEL=stream|tiled forces it. */
+    int tiled;
+    int forced; /* -1 none, 0 stream, 1 tiled (segment entry point or environment) */
     int32_t* ws_meta;        /* [3 * WS_MAX_E + 1] */
     uint32_t* ws_row_token;  /* [WS_MAX_ROWS] */
     uint32_t* ws_row_partidx;
@@ -61,6 +68,11 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
     c->device = device;
     c->min_rows[0] = c->min_rows[1] = -1;
     c->err[0] = 0;
+    c->forced = -1;
+    if (const char* k = getenv("PLOW_MOE_W8A8_KERNEL")) {
+        if (!strcmp(k, "stream")) c->forced = 0;
+        if (!strcmp(k, "tiled")) c->forced = 1;
+    }
     int prev = 0;
     hipGetDevice(&prev);
     hipSetDevice(device);
@@ -183,7 +195,9 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 3);
             g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.pitch = i[4]; g.act = i[5];
-            return launch_group_glu_w8a8(g, st);
+            /* many rows per expert (row pitch >= 2 rows per expert per routed slot): tiled form */
+            c->tiled = c->forced >= 0 ? c->forced : (i[4] >= 2u * E ? 1 : 0);
+            return c->tiled ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
                          (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
@@ -220,7 +234,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4);
             g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_W8A8_P16;
-            return launch_group_down_w8a8(g, st);
+            const int tiled = c->forced >= 0 ? c->forced : c->tiled;
+            return tiled ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
                          (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
@@ -426,9 +441,13 @@ static int run_segment(PlowMoeCtx* ctx, int variant, const PlowDevInst* insts, u
     ctx->err[0] = 0;
     const int mr = ctx->min_rows[variant];
     if (mr == 0 || (mr > 0 && rows < (uint32_t)mr)) return PLOW_MOE_ROLLBACK;
-    const int rc = check_segment(ctx, insts, n_inst);
+    int rc = check_segment(ctx, insts, n_inst);
     if (rc) return rc;
-    return plow_moe_exec_many(ctx, insts, n_inst, tensors, stream);
+    const int saved = ctx->forced;
+    if (saved < 0) ctx->forced = variant == 0 ? 1 : 0; /* prefill: tiled form, decode: streaming form */
+    rc = plow_moe_exec_many(ctx, insts, n_inst, tensors, stream);
+    ctx->forced = saved;
+    return rc;
 }
 
 extern "C" int plow_moe_pf(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst,

@@ -64,3 +64,46 @@ def test_dsv3_decode_b64_full_shape(moe, oracle):
     check_layer(plan, dev, host)
     cnt = host.np("meta")[cfg.E_all:2 * cfg.E_all]
     print(f"[c2] experts hit {int((cnt[:cfg.E] > 0).sum())} / {cfg.E}, max rows {int(cnt[:cfg.E].max())}", flush=True)
+
+
+@pytest.mark.parametrize("T,E,k", [(300, 4, 2), (700, 8, 4), (1030, 3, 1)])
+def test_tiled_kernel_many_rows_per_expert(moe, oracle, T, E, k):
+    """Row counts of 60..1030 per expert run the tiled (prefill) form: partial, full and multiple
+    256-row tiles; routing bit-exact, output within tolerance."""
+    cfg = layer.MoeConfig("tiled", H=384, E=E, I=256, k=k, T=T, scoring="softmax", norm_topk=True,
+                          enc="fp8blk", arm="w8a8", n_shared=1, shared_mode="fold", residual=True)
+    plan, dev, host = both(moe, oracle, cfg, seed=T)
+    check_layer(plan, dev, host)
+
+
+def test_segment_entry_points(moe, oracle):
+    """plow_moe_pf / plow_moe_dec: same results as op-by-op execution, the min-rows knob, and typed
+    refusal of a mis-wired segment."""
+    from gpu_harness import run_device, run_oracle
+    from plow_amd import synth
+    cfg = layer.MoeConfig("seg", H=256, E=8, I=128, k=2, T=40, scoring="sigmoid", norm_topk=True,
+                          enc="fp8blk", arm="w8a8", n_shared=1, shared_mode="fold")
+    plan = layer.plan_layer(cfg)
+    dev = synth.bind(plan, "cuda", seed=5)
+    host = synth.to_host(dev)
+    run_oracle(oracle, plan, host)
+    for entry in (moe.pf, moe.dec):
+        for name in ("fq", "part", "out"):
+            dev.t[name].zero_()
+        assert entry(plan.insts, dev.table(), cfg.T) == 0
+        torch.cuda.synchronize()
+        assert_routing_equal(plan, dev, host)
+        assert_output_close(dev.np("out"), host.np("out"))
+    moe.set_min_rows(1, 64)                      # decode variant: segments below 64 rows roll back
+    assert moe.dec(plan.insts, dev.table(), cfg.T) == abi.ROLLBACK
+    assert moe.dec(plan.insts, dev.table(), 64) == 0
+    moe.set_min_rows(0, 0)                       # prefill variant switched off
+    assert moe.pf(plan.insts, dev.table(), cfg.T) == abi.ROLLBACK
+    moe.set_min_rows(0, -1)
+    moe.set_min_rows(1, -1)
+    torch.cuda.synchronize()
+    bad = [abi.PlowDevInst.from_buffer_copy(d) for d in plan.insts]
+    bad[plan.index("down")].i[1] = cfg.I * 2     # DOWN's K no longer equals the GLU's N
+    with pytest.raises(Exception) as ei:
+        moe.pf(bad, dev.table(), cfg.T)
+    assert "disagree" in str(ei.value)
