@@ -20,6 +20,10 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0          # MI355X datasheet
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled
+# by what the same counter reads for a 1 GiB copy): profiles/c2_decode_b64_pmc_fetch_write.txt.
+# Keyed by (config, tokens, kernel); anything not measured reports null.
+MEASURED_TRAFFIC = {("c2", 64, "glu"): 6532905574, ("c2", 64, "down"): 3258872013}
 FP8_PEAK_TFLOPS = 5000.0       # dense fp8 MFMA
 
 
@@ -43,6 +47,9 @@ def main():
     ap.add_argument("--config", default="c2")
     ap.add_argument("--tokens", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib", action="store_true",
+                    help="also run a plain 1 GiB device copy three times (a kernel of known traffic, "
+                         "for scaling hardware counters read under rocprofv3 --pmc)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU (all experts of a layer resident, no collectives); "
@@ -89,6 +96,14 @@ def main():
             per_op[name].append(evs[n].elapsed_time(evs[n + 1]) * 1e3)
     op_us = {n: statistics.mean(v) for n, v in per_op.items()}
 
+    if a.calib:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     meta = dev.np("meta")
     cnt = meta[cfg.E_all:2 * cfg.E_all]
     hit = int((cnt > 0).sum())                       # experts whose weights must stream (incl. shared)
@@ -120,7 +135,8 @@ def main():
                   "flops": flops, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / FP8_PEAK_TFLOPS, 4)},
         "op_us": {n: round(v, 2) for n, v in op_us.items()},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((cfg.name, T, dom)),
                      "bytes_per_launch": int(dom_bytes), "us_per_launch": round(op_us[dom], 2)},
     }
 
