@@ -20,6 +20,7 @@
 #define WS_MAX_E 1056u
 #define WS_MAX_SLOTS (1u << 18)
 #define WS_MAX_ROWS (WS_MAX_SLOTS + WS_MAX_E * (PLOW_MPF_BM - 1u))
+#define WS_MAX_CHUNKS (WS_MAX_SLOTS / 1024u)
 
 struct PlowMoeCtx {
     int device;
@@ -35,6 +36,7 @@ struct PlowMoeCtx {
     uint32_t* ws_row_token;  /* [WS_MAX_ROWS] */
     uint32_t* ws_row_partidx;
     float* ws_row_gate;
+    uint32_t* ws_chunk_hist; /* [WS_MAX_CHUNKS][n_exp] scratch of the multi-workgroup align */
 };
 
 static int fail(PlowMoeCtx* c, int code, const char* fmt, ...) {
@@ -79,7 +81,8 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
     const bool ok = hipMalloc(&c->ws_meta, (3u * WS_MAX_E + 1u) * 4u) == hipSuccess &&
                     hipMalloc(&c->ws_row_token, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
                     hipMalloc(&c->ws_row_partidx, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
-                    hipMalloc(&c->ws_row_gate, (size_t)WS_MAX_ROWS * 4u) == hipSuccess;
+                    hipMalloc(&c->ws_row_gate, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
+                    hipMalloc(&c->ws_chunk_hist, (size_t)WS_MAX_CHUNKS * WS_MAX_E * 4u) == hipSuccess;
     hipSetDevice(prev);
     if (!ok) {
         plow_moe_destroy(c);
@@ -95,6 +98,7 @@ extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) {
     hipFree(ctx->ws_row_token);
     hipFree(ctx->ws_row_partidx);
     hipFree(ctx->ws_row_gate);
+    hipFree(ctx->ws_chunk_hist);
     delete ctx;
 }
 
@@ -147,7 +151,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, (uint64_t)i[0] * i[2] < (1ull << 31), "op 84: T * k overflows");
         if (!launch) return 0;
         return launch_align((int32_t*)ten(in, T, 0), ten(in, T, 1), (uint32_t*)ten(in, T, 2),
-                            (uint32_t*)ten(in, T, 3), (float*)ten(in, T, 4), i[0], i[1], i[2], st);
+                            (uint32_t*)ten(in, T, 3), (float*)ten(in, T, 4), i[0], i[1], i[2],
+                            c->ws_chunk_hist, WS_MAX_CHUNKS, st);
     }
     case PLOW_DOP_MOE_COMBINE:
     case PLOW_DOP_MOE_COMBINE_PF: {
@@ -310,7 +315,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         if (!launch) return 0;
         /* align with k = slots per input row: row_token = slot / kx, row_partidx = slot */
         int rc = launch_align(c->ws_meta, ten(in, T, 2), c->ws_row_token, c->ws_row_partidx, c->ws_row_gate,
-                              (nslot + kx - 1u) / kx, E, kx, st);
+                              (nslot + kx - 1u) / kx, E, kx, c->ws_chunk_hist, WS_MAX_CHUNKS, st);
         if (rc) return rc;
         GroupA16 g = {};
         g.out = ten(in, T, 0); g.a = ten(in, T, 1);

@@ -33,20 +33,33 @@
 
 
 __device__ __forceinline__ v4i ldg16(const uint8_t* p) { return *(const v4i*)p; }
+/* weight bytes are read exactly once per launch: stream them past the caches */
+__device__ __forceinline__ v4i ldg16_stream(const uint8_t* p) {
+#ifdef SK_NT_WEIGHTS
+    return __builtin_nontemporal_load((const v4i*)p);
+#else
+    return *(const v4i*)p;
+#endif
+}
 
-template <int RT, bool GLU, int D, bool PC>
+/* WIDE (DOWN, block mode only): a wave owns 32 channels as two 16-channel streams, a workgroup 256
+ * channels; the short K loop of the down projection then amortises its prologue over twice the bytes. */
+template <int RT, bool GLU, int D, bool PC, bool WIDE>
 __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t ct, uint32_t r0,
                                         uint32_t rb, uint32_t cnt, float* s_red) {
     const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6, c = lane & 15u, q = lane >> 4;
     const uint32_t K = g.K, KB = K / 128u, N = g.N;
-    const uint32_t ch = ct * SK_BN + wv * 16u + c; /* this lane's weight row */
+    constexpr bool TWO = GLU || WIDE; /* two weight streams per wave */
+    const uint32_t ch = WIDE ? ct * 256u + wv * 32u + c : ct * SK_BN + wv * 16u + c; /* this lane's weight row */
     /* block mode: {gate, up, down} tables, scale rows [N/128][KB]; per-channel mode: {gate_up fused,
      * down} tables (up rows follow the N gate rows), one f32 scale per weight row */
     const uint32_t wcols = PC ? 2u : 3u, sel0 = PC ? (GLU ? 0u : 1u) : (GLU ? 0u : 2u), sel1 = PC ? 0u : 1u;
     const uint8_t* w0 = (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * wcols + sel0] + (size_t)ch * K + 16u * q;
     const uint8_t* w1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * wcols + sel1] +
-                                  (size_t)(ch + (PC ? N : 0u)) * K + 16u * q : nullptr;
-    const float* s0 = (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel0] + (PC ? 0u : (size_t)ct * KB);
+                                  (size_t)(ch + (PC ? N : 0u)) * K + 16u * q
+                            : (WIDE ? w0 + (size_t)16u * K : nullptr);
+    const float* s0 = (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel0] +
+                      (PC ? 0u : (WIDE ? (size_t)(ct * 2u + (wv >> 2)) * KB : (size_t)ct * KB));
     const float* s1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel1] + (PC ? (size_t)N : (size_t)ct * KB) : nullptr;
 
     /* B operand rows of this lane, one per row tile */
@@ -86,11 +99,11 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
     float xs[D][RT], sa[D], sb[D];
     auto issue = [&](int d, uint32_t kb) {
         const uint32_t ko = kb * 128u;
-        wa[d][0] = ldg16(w0 + ko);
-        wa[d][1] = ldg16(w0 + ko + 64u);
-        if (GLU) {
-            wb[d][0] = ldg16(w1 + ko);
-            wb[d][1] = ldg16(w1 + ko + 64u);
+        wa[d][0] = ldg16_stream(w0 + ko);
+        wa[d][1] = ldg16_stream(w0 + ko + 64u);
+        if (TWO) {
+            wb[d][0] = ldg16_stream(w1 + ko);
+            wb[d][1] = ldg16_stream(w1 + ko + 64u);
         }
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
@@ -125,7 +138,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             if (kb < KB) {
                 const v8i A0 = __builtin_shufflevector(wa[d][0], wa[d][1], 0, 1, 2, 3, 4, 5, 6, 7);
                 v8i A1;
-                if (GLU) A1 = __builtin_shufflevector(wb[d][0], wb[d][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                if (TWO) A1 = __builtin_shufflevector(wb[d][0], wb[d][1], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) {
                     const v8i B = __builtin_shufflevector(xa[d][rt][0], xa[d][rt][1], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -138,9 +151,9 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
                         const float sc0 = xs[d][rt] * sa[d];
 #pragma unroll
                         for (int i = 0; i < 4; i++) acc0[rt][i] = fmaf(t0[i], sc0, acc0[rt][i]);
-                        if (GLU) {
+                        if (TWO) {
                             const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, z, 0, 0, 0, 0, 0, 0);
-                            const float sc1 = xs[d][rt] * sb[d];
+                            const float sc1 = xs[d][rt] * (WIDE ? sa[d] : sb[d]);
 #pragma unroll
                             for (int i = 0; i < 4; i++) acc1[rt][i] = fmaf(t1[i], sc1, acc1[rt][i]);
                         }
@@ -152,7 +165,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
     }
 
     /* ---- epilogue: lane holds channels ct*128 + wv*16 + 4q + i (i = 0..3) of row c ---- */
-    const uint32_t col = ct * SK_BN + wv * 16u + 4u * q;
+    const uint32_t col = WIDE ? ct * 256u + wv * 32u + 4u * q : ct * SK_BN + wv * 16u + 4u * q;
     if (PC) {
         /* per-channel arm (plow runtime/amd/op_moe.h:6655-6700): g = acc * (as * wsc[n]); GLU stores
          * bf16(act(g) * u) and zeroes pad rows, DOWN stores gate * acc, then * (as * wsc[h]) */
@@ -233,14 +246,25 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             } else {
                 *(float4*)((float*)g.out + (size_t)pidx * N + col) = make_float4(y0, y1, y2, y3);
             }
+            if (WIDE) { /* the second 16-channel stream */
+                const float z0 = gate * acc1[rt][0], z1 = gate * acc1[rt][1], z2 = gate * acc1[rt][2], z3 = gate * acc1[rt][3];
+                if (g.part16) {
+                    uint2 o;
+                    o.x = (uint32_t)f2bf(z0) | ((uint32_t)f2bf(z1) << 16);
+                    o.y = (uint32_t)f2bf(z2) | ((uint32_t)f2bf(z3) << 16);
+                    *(uint2*)((bf16_t*)g.out + (size_t)pidx * N + col + 16u) = o;
+                } else {
+                    *(float4*)((float*)g.out + (size_t)pidx * N + col + 16u) = make_float4(z0, z1, z2, z3);
+                }
+            }
         }
     }
 }
 
-template <bool GLU, int D, bool PC>
+template <bool GLU, int D, bool PC, bool WIDE = false>
 __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     __shared__ float s_red[SK_WAVES * 64u];
-    const uint32_t tiles = g.N / SK_BN;
+    const uint32_t tiles = g.N / (WIDE ? 256u : SK_BN);
     /* highest expert id first: a folded shared expert (id E-1, every token routed to it) is the one
      * segment that needs several passes, so it must start early instead of forming the tail */
     const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles;
@@ -250,7 +274,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     const uint32_t r0 = (uint32_t)g.meta[e];
     /* 16 rows a pass; an expert with more rows streams its weights once per pass (the tiled
      * kernel, not this one, is the tool for many rows per expert) */
-    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D, PC>(g, e, ct, r0, rb, cnt, s_red);
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D, PC, WIDE>(g, e, ct, r0, rb, cnt, s_red);
     if (PC && GLU) {
         /* the per-channel GLU zeroes the pad rows of its 64-row tile (the partial 16-row pass above
          * did its own); the row quantizer that follows reads every aligned row */
@@ -299,6 +323,15 @@ int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<false, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
+    if (g.N % 256u == 0u && !getenv("PLOW_MOE_SK_NARROW")) {
+        const dim3 wgrid(g.E * (g.N / 256u));
+        switch (stream_depth()) {
+        case 2: k_group_w8a8_stream<false, 2, false, true><<<wgrid, SK_THREADS, 0, st>>>(g); break;
+        case 4: k_group_w8a8_stream<false, 4, false, true><<<wgrid, SK_THREADS, 0, st>>>(g); break;
+        default: k_group_w8a8_stream<false, 3, false, true><<<wgrid, SK_THREADS, 0, st>>>(g); break;
+        }
+        return 0;
+    }
     switch (stream_depth()) {
     case 2: k_group_w8a8_stream<false, 2, false><<<grid, SK_THREADS, 0, st>>>(g); break;
     case 4: k_group_w8a8_stream<false, 4, false><<<grid, SK_THREADS, 0, st>>>(g); break;

@@ -11,8 +11,10 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
 int launch_router_topk(void* table, const void* logit, const float* bias, uint32_t n_exp, uint32_t k,
                        uint32_t flags, uint32_t T, uint32_t tail, uint32_t n_group, uint32_t topk_group,
                        float route_scale, float logit_scale, hipStream_t st);
+/* chunk_hist: u32 [chunk_cap][E] scratch for the multi-workgroup form (NULL = single workgroup) */
 int launch_align(int32_t* meta, const void* table, uint32_t* row_token, uint32_t* row_partidx,
-                 float* row_gate, uint32_t T, uint32_t E, uint32_t k, hipStream_t st);
+                 float* row_gate, uint32_t T, uint32_t E, uint32_t k, uint32_t* chunk_hist,
+                 uint32_t chunk_cap, hipStream_t st);
 int launch_combine(void* out, const void* residual, const void* shared, const void* part, uint32_t H,
                    uint32_t k, uint32_t T, uint32_t part16, hipStream_t st);
 

@@ -14,108 +14,80 @@
 /* ============================ op 180: router score ============================================= */
 /* logit[m][n] = sum_k bf(x[m][k]) * bf(w[n][k]) with ONE f32 accumulator per output walking k in
  * ascending order (plow runtime/cpu/dev/golden/f32_primitives.c:235-252). The product of two bf16
- * values is exact in f32, so fmaf(a, b, acc) rounds exactly like the reference's `acc += a * b`.
- * Threads form a 16 x 16 grid; each owns a TM x TN block of outputs and both operands are staged
- * through LDS, transposed to [k][row] f32, one KC-wide chunk at a time with the next chunk's global
- * loads already in flight. */
-template <int TM, int TN, int KC>
-__global__ __launch_bounds__(256) void k_router_score(float* __restrict__ out,
-                                                      const bf16_t* __restrict__ x,
-                                                      const bf16_t* __restrict__ w, uint32_t M,
-                                                      uint32_t N, uint32_t K) {
-    constexpr int BM = 16 * TM, BN = 16 * TN;
-    constexpr int XCH = BM * KC / 8, WCH = BN * KC / 8;         /* 16-byte pieces per chunk */
-    constexpr int XPT = (XCH + 255) / 256, WPT = (WCH + 255) / 256;
-    __shared__ float xs[KC][BM + 1];
-    __shared__ float ws[KC][BN + 1];
+ * values is exact in f32, so fmaf(a, b, acc) rounds exactly like the reference's `acc += a * b`. */
+/* Large problems (prefill): 64 x 64 outputs per workgroup, 4 x 4 per thread (16 independent chains
+ * per lane keep the FMA pipe full), operands double buffered in LDS as f32 [k][row] and read as
+ * float4, one LDS-only barrier per 32-k chunk, the next chunk's global loads already in flight. */
+#define RST_KC 32
+#define RST_LD 68 /* floats per LDS row: 64 + 4 keeps float4 reads aligned */
+__global__ __launch_bounds__(256) void k_router_score_tile(float* __restrict__ out,
+                                                           const bf16_t* __restrict__ x,
+                                                           const bf16_t* __restrict__ w, uint32_t M,
+                                                           uint32_t N, uint32_t K) {
+    __shared__ __attribute__((aligned(16))) float xs[2][RST_KC][RST_LD];
+    __shared__ __attribute__((aligned(16))) float ws[2][RST_KC][RST_LD];
     const uint32_t tid = threadIdx.x, tx = tid & 15u, ty = tid >> 4;
-    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    float acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = 0.0f;
-
-    uint4 xr[XPT], wr[WPT];
+    const uint32_t m0 = blockIdx.y * 64u, n0 = blockIdx.x * 64u;
+    /* staging: 64 rows x 32 k bf16 = 256 16-byte pieces per operand, one per thread */
+    const uint32_t srow = tid >> 2, skc = tid & 3u;
+    uint4 xr, wr;
     auto fetch = [&](uint32_t k0) {
+        const uint32_t k = k0 + skc * 8u;
+        xr = make_uint4(0, 0, 0, 0);
+        wr = make_uint4(0, 0, 0, 0);
+        if (m0 + srow < M && k < K) xr = *(const uint4*)(x + (size_t)(m0 + srow) * K + k);
+        if (n0 + srow < N && k < K) wr = *(const uint4*)(w + (size_t)(n0 + srow) * K + k);
+    };
+    auto commit = [&](uint32_t buf) {
+        const uint32_t a[4] = {xr.x, xr.y, xr.z, xr.w}, b[4] = {wr.x, wr.y, wr.z, wr.w};
 #pragma unroll
-        for (int p = 0; p < XPT; p++) {
-            const uint32_t c = tid + 256u * p, row = c / (KC / 8), kc = c % (KC / 8);
-            const uint32_t k = k0 + kc * 8u;
-            xr[p] = make_uint4(0, 0, 0, 0);
-            if (c < (uint32_t)XCH && m0 + row < M && k < K)
-                xr[p] = *(const uint4*)(x + (size_t)(m0 + row) * K + k);
-        }
-#pragma unroll
-        for (int p = 0; p < WPT; p++) {
-            const uint32_t c = tid + 256u * p, row = c / (KC / 8), kc = c % (KC / 8);
-            const uint32_t k = k0 + kc * 8u;
-            wr[p] = make_uint4(0, 0, 0, 0);
-            if (c < (uint32_t)WCH && n0 + row < N && k < K)
-                wr[p] = *(const uint4*)(w + (size_t)(n0 + row) * K + k);
+        for (int j = 0; j < 4; j++) {
+            xs[buf][skc * 8 + 2 * j][srow] = __uint_as_float(a[j] << 16);
+            xs[buf][skc * 8 + 2 * j + 1][srow] = __uint_as_float(a[j] & 0xFFFF0000u);
+            ws[buf][skc * 8 + 2 * j][srow] = __uint_as_float(b[j] << 16);
+            ws[buf][skc * 8 + 2 * j + 1][srow] = __uint_as_float(b[j] & 0xFFFF0000u);
         }
     };
-    auto commit = [&]() {
+    float acc[4][4];
 #pragma unroll
-        for (int p = 0; p < XPT; p++) {
-            const uint32_t c = tid + 256u * p, row = c / (KC / 8), kc = c % (KC / 8);
-            if (c < (uint32_t)XCH) {
-                const uint32_t v[4] = {xr[p].x, xr[p].y, xr[p].z, xr[p].w};
+    for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    xs[kc * 8 + 2 * j][row] = __uint_as_float(v[j] << 16);
-                    xs[kc * 8 + 2 * j + 1][row] = __uint_as_float(v[j] & 0xFFFF0000u);
-                }
-            }
-        }
-#pragma unroll
-        for (int p = 0; p < WPT; p++) {
-            const uint32_t c = tid + 256u * p, row = c / (KC / 8), kc = c % (KC / 8);
-            if (c < (uint32_t)WCH) {
-                const uint32_t v[4] = {wr[p].x, wr[p].y, wr[p].z, wr[p].w};
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    ws[kc * 8 + 2 * j][row] = __uint_as_float(v[j] << 16);
-                    ws[kc * 8 + 2 * j + 1][row] = __uint_as_float(v[j] & 0xFFFF0000u);
-                }
-            }
-        }
-    };
-
+        for (int j = 0; j < 4; j++) acc[i][j] = 0.0f;
     fetch(0);
-    for (uint32_t k0 = 0; k0 < K; k0 += KC) {
-        lds_barrier(); /* everyone is done reading the previous chunk */
-        commit();
-        lds_barrier();
-        if (k0 + KC < K) fetch(k0 + KC);
-        const uint32_t kn = K - k0 < (uint32_t)KC ? K - k0 : (uint32_t)KC;
-        if (kn == (uint32_t)KC) {
-#pragma unroll 8
-            for (int kk = 0; kk < KC; kk++) {
-                float a[TM], b[TN];
+    commit(0);
+    lds_barrier();
+    uint32_t buf = 0;
+    for (uint32_t k0 = 0; k0 < K; k0 += RST_KC, buf ^= 1u) {
+        const bool more = k0 + RST_KC < K;
+        if (more) fetch(k0 + RST_KC);
+        const uint32_t kn = K - k0 < (uint32_t)RST_KC ? K - k0 : (uint32_t)RST_KC;
+        if (kn == (uint32_t)RST_KC) {
 #pragma unroll
-                for (int i = 0; i < TM; i++) a[i] = xs[kk][ty * TM + i];
+            for (int kk = 0; kk < RST_KC; kk++) {
+                const float4 a = *(const float4*)&xs[buf][kk][ty * 4u];
+                const float4 b = *(const float4*)&ws[buf][kk][tx * 4u];
+                const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
 #pragma unroll
-                for (int j = 0; j < TN; j++) b[j] = ws[kk][tx * TN + j];
+                for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+                    for (int j = 0; j < 4; j++) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
             }
         } else {
             for (uint32_t kk = 0; kk < kn; kk++)
 #pragma unroll
-                for (int i = 0; i < TM; i++)
+                for (int i = 0; i < 4; i++)
 #pragma unroll
-                    for (int j = 0; j < TN; j++)
-                        acc[i][j] = fmaf(xs[kk][ty * TM + i], ws[kk][tx * TN + j], acc[i][j]);
+                    for (int j = 0; j < 4; j++)
+                        acc[i][j] = fmaf(xs[buf][kk][ty * 4u + i], ws[buf][kk][tx * 4u + j], acc[i][j]);
         }
+        if (more) commit(buf ^ 1u);
+        lds_barrier();
     }
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const uint32_t m = m0 + ty * TM + i, n = n0 + tx * TN + j;
+        for (int j = 0; j < 4; j++) {
+            const uint32_t m = m0 + ty * 4u + i, n = n0 + tx * 4u + j;
             if (m < M && n < N) out[(size_t)m * N + n] = acc[i][j];
         }
 }
@@ -224,7 +196,7 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
     if (K % 8u) return PLOW_MOE_EINVAL;
     if ((uint64_t)M * N >= (1u << 19)) {
         dim3 g((N + 63) / 64, (M + 63) / 64);
-        k_router_score<4, 4, 32><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        k_router_score_tile<<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else {
         dim3 g((N + 7) / 8, (M + 7) / 8);
         k_router_score_wave<<<g, 64, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
@@ -548,11 +520,137 @@ __global__ __launch_bounds__(AL_WAVES* WAVE) void k_align(AlignArgs a) {
     }
 }
 
+/* Many slots (prefill): the same counting sort spread over the chip in three launches.
+ *   hist     one workgroup per chunk of 1024 slots: per-expert counts of the chunk -> chunk_hist
+ *   scan     one workgroup: per expert, exclusive prefix over the chunks (in place); counts, padded
+ *            offsets and tile prefix -> meta; pad rows marked
+ *   scatter  one workgroup per chunk: the single-workgroup algorithm above on the chunk's 16 waves,
+ *            starting from rowoff[e] + chunk prefix
+ * chunk_hist is u32 [chunks][E] in the context workspace. */
+#define AL_CHUNK (AL_WAVES * WAVE)
+
+__global__ __launch_bounds__(AL_CHUNK) void k_align_hist(const PlowMoeRoute* __restrict__ table,
+                                                         uint32_t* __restrict__ chunk_hist,
+                                                         uint32_t nslot, uint32_t E) {
+    __shared__ uint32_t h[AL_MAX_E];
+    const uint32_t tid = threadIdx.x, s = blockIdx.x * AL_CHUNK + tid;
+    for (uint32_t e = tid; e < E; e += AL_CHUNK) h[e] = 0u;
+    __syncthreads();
+    if (s < nslot) {
+        const uint32_t e = table[s].eid;
+        if (e < E) atomicAdd(&h[e], 1u);
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < E; e += AL_CHUNK) chunk_hist[(size_t)blockIdx.x * E + e] = h[e];
+}
+
+__global__ __launch_bounds__(AL_CHUNK) void k_align_scan(AlignArgs a, uint32_t* __restrict__ chunk_hist,
+                                                         uint32_t nchunk) {
+    __shared__ uint32_t s_rowoff[AL_MAX_E];
+    __shared__ uint32_t s_cnt[AL_MAX_E];
+    __shared__ uint32_t s_carry;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6, E = a.E;
+    for (uint32_t e = tid; e < E; e += AL_CHUNK) {
+        uint32_t run = 0;
+        for (uint32_t c = 0; c < nchunk; c++) {
+            const uint32_t v = chunk_hist[(size_t)c * E + e];
+            chunk_hist[(size_t)c * E + e] = run;
+            run += v;
+        }
+        s_cnt[e] = run;
+    }
+    if (tid == 0) s_carry = 0u;
+    __syncthreads();
+    if (wv == 0) {
+        for (uint32_t e0 = 0; e0 < E; e0 += WAVE) {
+            const uint32_t e = e0 + lane;
+            const uint32_t c = e < E ? s_cnt[e] : 0u;
+            const uint32_t tiles = (c + PLOW_MPF_BM - 1u) / PLOW_MPF_BM;
+            uint32_t inc = tiles;
+#pragma unroll
+            for (uint32_t o = 1; o < WAVE; o <<= 1) {
+                const uint32_t v = __shfl_up(inc, o, 64);
+                if (lane >= o) inc += v;
+            }
+            const uint32_t carry = s_carry;
+            const uint32_t excl = carry + inc - tiles;
+            if (e < E) {
+                s_rowoff[e] = excl * PLOW_MPF_BM;
+                a.meta[e] = (int32_t)(excl * PLOW_MPF_BM);
+                a.meta[E + e] = (int32_t)c;
+                a.meta[2u * E + e] = (int32_t)excl;
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (lane == WAVE - 1u) s_carry = carry + inc;
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (lane == 0) a.meta[3u * E] = (int32_t)s_carry;
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < E * PLOW_MPF_BM; i += AL_CHUNK) {
+        const uint32_t e = i / PLOW_MPF_BM, j = i % PLOW_MPF_BM;
+        const uint32_t c = s_cnt[e], r = s_rowoff[e] + c + j;
+        if (c + j < ((c + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM) {
+            a.row_token[r] = PLOW_EXPERT_UNUSED;
+            a.row_partidx[r] = PLOW_EXPERT_UNUSED;
+            a.row_gate[r] = 0.0f;
+        }
+    }
+}
+
+__global__ __launch_bounds__(AL_CHUNK) void k_align_scatter(AlignArgs a, const uint32_t* __restrict__ chunk_hist) {
+    __shared__ uint32_t hist[AL_WAVES][AL_MAX_E];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
+    const uint32_t E = a.E, nslot = a.T * a.k;
+    const uint32_t s = blockIdx.x * AL_CHUNK + tid;
+    for (uint32_t i = tid; i < AL_WAVES * E; i += AL_CHUNK) hist[i / E][i % E] = 0u;
+    __syncthreads();
+    const bool in = s < nslot;
+    const uint32_t e = in ? a.table[s].eid : PLOW_EXPERT_UNUSED;
+    const float g = in ? a.table[s].gate : 0.0f;
+    const bool live = e < E;
+    if (live) atomicAdd(&hist[wv][e], 1u);
+    __syncthreads();
+    /* exclusive prefix over the waves, started at this chunk's global position in the expert */
+    for (uint32_t x = tid; x < E; x += AL_CHUNK) {
+        uint32_t run = (uint32_t)a.meta[x] + chunk_hist[(size_t)blockIdx.x * E + x];
+#pragma unroll
+        for (uint32_t w = 0; w < AL_WAVES; w++) {
+            const uint32_t c = hist[w][x];
+            hist[w][x] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    unsigned long long todo = __ballot(live);
+    uint32_t pos = 0;
+    while (todo) {
+        const uint32_t leader = (uint32_t)__builtin_ctzll(todo);
+        const uint32_t e0 = (uint32_t)__shfl((int)e, (int)leader, 64);
+        const unsigned long long same = __ballot(live && e == e0);
+        if (live && e == e0) pos = hist[wv][e0] + (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
+        todo &= ~same;
+    }
+    if (live) {
+        a.row_token[pos] = s / a.k;
+        a.row_partidx[pos] = s;
+        a.row_gate[pos] = g;
+    }
+}
+
 int launch_align(int32_t* meta, const void* table, uint32_t* row_token, uint32_t* row_partidx,
-                 float* row_gate, uint32_t T, uint32_t E, uint32_t k, hipStream_t st) {
+                 float* row_gate, uint32_t T, uint32_t E, uint32_t k, uint32_t* chunk_hist,
+                 uint32_t chunk_cap, hipStream_t st) {
     if (E == 0 || E > AL_MAX_E || k == 0) return PLOW_MOE_EINVAL;
     AlignArgs a = {meta, (const PlowMoeRoute*)table, row_token, row_partidx, row_gate, T, E, k};
-    k_align<<<1, AL_WAVES * WAVE, 0, st>>>(a);
+    const uint32_t nslot = T * k, nchunk = (nslot + AL_CHUNK - 1u) / AL_CHUNK;
+    if (nslot <= 4u * AL_CHUNK || !chunk_hist || nchunk > chunk_cap) {
+        k_align<<<1, AL_WAVES * WAVE, 0, st>>>(a);
+        return 0;
+    }
+    k_align_hist<<<nchunk, AL_CHUNK, 0, st>>>((const PlowMoeRoute*)table, chunk_hist, nslot, E);
+    k_align_scan<<<1, AL_CHUNK, 0, st>>>(a, chunk_hist, nchunk);
+    k_align_scatter<<<nchunk, AL_CHUNK, 0, st>>>(a, chunk_hist);
     return 0;
 }
 
