@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libplow_moe_gfx950.so")
 
-COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-fast-math",
+COMMON = ["--offload-arch=gfx950", "-O3", *os.environ.get("PLOW_MOE_EXTRA_FLAGS", "").split(), "-std=c++17", "-fPIC", "-fno-fast-math",
           # packed-FP32 VALU forms are kept out of every kernel
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # Translation units whose floating-point results must match the CPU reference bit for bit are built

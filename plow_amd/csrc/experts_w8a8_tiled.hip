@@ -20,10 +20,8 @@
  * scale, so they contribute nothing and are never stored.
  * Per 128-k block: t = two chained matrix instructions (k 0..63, 64..127), then
  * acc = fmaf(t, a_scale[row][kb] * w_scale[nb][kb], acc).
- * Tiles are enumerated (expert, 128-row tile, channel tile) with the channel tile fastest and walked
- * by persistent workgroups (one per CU): the tiles that share an expert's weight rows are a
- * multiple of 8 workgroups apart, which the hardware dispatch order places on the same XCD, and run
- * at the same time, so the second reader hits in that XCD's L2. */
+ * Tiles are walked by persistent workgroups (one per CU) in an order that puts the tiles sharing
+ * activation rows and weight rows on one XCD at the same time (see the tile loop). */
 #include "common.h"
 #include "kernels.h"
 
@@ -76,6 +74,12 @@ __device__ __forceinline__ void lds_operand(uint32_t base, uint32_t row, uint32_
 /* wait until at most n of this wave's loads are outstanding, then the workgroup barrier */
 #define STAGE_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(n) : "memory")
 
+#ifdef T2_PROF
+__device__ unsigned long long t2_prof[2][256][8];
+#define PROF_STAMP(v) const unsigned long long v = __builtin_readcyclecounter()
+#else
+#define PROF_STAMP(v)
+#endif
 template <bool GLU>
 __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
@@ -106,12 +110,25 @@ __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             __syncthreads();
         }
     }
+#ifdef T2_PROF
+    unsigned long long pf_setup = 0, pf_ramp = 0, pf_loop = 0, pf_epi = 0, pf_tiles = 0;
+    const unsigned long long pf_begin = __builtin_readcyclecounter();
+#endif
     const uint32_t total = L.prefix[g.E - 1u] * NT;
     const uint32_t K = g.K, KB = K / 128u;
     const uint32_t wr = wv & 1u, wc = wv >> 1, l32 = lane & 31u, lh = lane >> 5;
 
-    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
-        const uint32_t nt = tile % NT, mt_global = tile / NT;
+    /* Workgroup w runs on XCD w % 8 (round-robin dispatch), and each XCD has its own L2. The logical
+     * index below makes the 32 workgroups of one XCD take 32 consecutive tiles of every sweep, and the
+     * tile order inside an expert is (16-channel-tile chunk, row tile, channel tile in the chunk): those
+     * 32 tiles are then two row tiles x 16 channel tiles of one expert, which read the same activation
+     * rows and the same weight rows at about the same time and meet in that L2. */
+    const uint32_t G = gridDim.x;
+    const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const uint32_t FC = NT / 16u, RC = NT % 16u;
+    for (uint32_t tile = wg; tile < total; tile += G) {
+        PROF_STAMP(ts0);
+        const uint32_t mt_global = tile / NT;
         uint32_t lo = 0, hi = g.E - 1u; /* first expert whose inclusive prefix exceeds mt_global */
         while (lo < hi) {
             const uint32_t mid = (lo + hi) >> 1;
@@ -120,7 +137,18 @@ __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
         /* the same value in every lane; made explicit so that everything indexed by the expert (pointer
          * tables, block scales) is read with scalar loads and never waits on the vector-load counter */
         const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)lo);
-        const uint32_t mt = (uint32_t)__builtin_amdgcn_readfirstlane((int)(mt_global - (e ? L.prefix[e - 1u] : 0u)));
+        const uint32_t pbase = e ? L.prefix[e - 1u] : 0u, Me = L.prefix[e] - pbase;
+        const uint32_t idx = tile - pbase * NT;
+        uint32_t mt_v, nt_v;
+        if (idx < FC * Me * 16u) {
+            const uint32_t chunk = idx / (Me * 16u), rem = idx % (Me * 16u);
+            mt_v = rem / 16u, nt_v = chunk * 16u + rem % 16u;
+        } else {
+            const uint32_t rem = idx - FC * Me * 16u;
+            mt_v = rem / RC, nt_v = FC * 16u + rem % RC;
+        }
+        const uint32_t mt = (uint32_t)__builtin_amdgcn_readfirstlane((int)mt_v);
+        const uint32_t nt = (uint32_t)__builtin_amdgcn_readfirstlane((int)nt_v);
         const uint32_t cnt = (uint32_t)g.meta[g.E + e], r0 = (uint32_t)g.meta[e] + mt * T2_BM;
         const uint32_t rows = cnt - mt * T2_BM < T2_BM ? cnt - mt * T2_BM : T2_BM; /* live rows here */
         const uint64_t wp0 = g.wtab[(size_t)e * 3u + (GLU ? 0u : 2u)];
@@ -171,6 +199,9 @@ __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
         }
         auto issue = [&](uint32_t kb) {
             const uint32_t st = kb % T2_STAGES;
+#ifdef T2_NOSTREAM
+            kb &= 1u;
+#endif
             __builtin_amdgcn_global_load_lds((const void*)(ssrc + (size_t)kb * sstep),
                                              (lds_void*)&L.as[st][(wv & 1u) * 64u], 4, 0, 0);
 #pragma unroll
@@ -213,11 +244,18 @@ __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
         if (KB > 1u) issue(1);
         const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]), s_base = lds_off(&L.as[0][0]);
         const uint32_t c_base = lds_off(&L.wsc[0][0]);
+        PROF_STAMP(ts1);
+#ifdef T2_PROF
+        unsigned long long ts2 = 0;
+#endif
         for (uint32_t kb = 0; kb < KB; kb++) {
             const uint32_t st = kb % T2_STAGES;
             /* this wave's loads of stage kb have landed once at most the next stage's are outstanding;
              * after the barrier stage kb is complete and the buffer of stage kb-1 is free */
             if (kb + 1u < KB) STAGE_BARRIER(NLOAD); else STAGE_BARRIER(0);
+#ifdef T2_PROF
+            if (kb == 0) ts2 = __builtin_readcyclecounter();
+#endif
             if (kb + 2u < KB) issue(kb + 2u);
             if (wave_live) {
                 float ws0 = ds_read4(c_base + kb * 4u);
@@ -267,6 +305,7 @@ __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             }
         }
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); /* ring drained */
+        PROF_STAMP(ts3);
 
         /* ---- epilogue. Lane: row = wr*64 + rt*32 + l32; channels wc*32 + 8*(i/4) + 4*lh + (i%4) ---- */
         if (GLU) {
@@ -320,8 +359,26 @@ __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             }
         }
         lds_barrier(); /* every wave is done with the ring and with L.red before the next tile refills them */
+#ifdef T2_PROF
+        {
+            const unsigned long long ts4 = __builtin_readcyclecounter();
+            pf_setup += ts1 - ts0, pf_ramp += ts2 - ts1, pf_loop += ts3 - ts2, pf_epi += ts4 - ts3, pf_tiles++;
+        }
+#endif
     }
+#ifdef T2_PROF
+    if (tid == 0 && blockIdx.x < 256u) {
+        unsigned long long* o = t2_prof[GLU][blockIdx.x];
+        o[0] = pf_setup, o[1] = pf_ramp, o[2] = pf_loop, o[3] = pf_epi, o[4] = pf_tiles;
+        o[5] = __builtin_readcyclecounter() - pf_begin;
+    }
+#endif
 }
+#ifdef T2_PROF
+extern "C" int plow_moe_debug_prof(unsigned long long* out) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(t2_prof), sizeof(t2_prof));
+}
+#endif
 
 /* Persistent launch: one workgroup per CU; the tile count is computed on the device from meta. */
 template <bool GLU>

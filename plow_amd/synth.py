@@ -133,7 +133,7 @@ def skewed_bias(E: int, hot: float, device, seed: int) -> torch.Tensor:
     """Router bias ~N(0, 0.01) with expert 0 raised so that it draws about ``hot`` x the mean load."""
     b = torch.randn(E, generator=_gen(device, seed), device=device) * 0.01
     if hot > 1.0:
-        b[0] += 0.02 * hot
+        b[0] += 0.0175 * hot
     return b
 
 
