@@ -1,128 +1,139 @@
 /* experts_w8a8_tiled.hip — the many-rows-per-expert (prefill) form of the block-fp8 x fp8 grouped
  * GEMMs (ops 85 / 86, arm 2 / 3). Same arithmetic as experts_w8a8.hip; different data flow.
  *
- * With hundreds of rows per expert the weights must be reused across rows from on-chip memory, so
- * this is a tiled GEMM: workgroup tile = 128 aligned rows x 128 output channels (GLU: 128 gate + 128
- * up weight rows), 8 waves as 2 (rows) x 4 (channels), each wave 64 rows x 32 channels on
- * v_mfma_f32_32x32x64_f8f6f4 with the weights as the A operand and the rows as the B operand, so
- * that a lane's accumulators belong to ONE row (token): its 1x128 activation scale is one value per
- * lane, and the GLU epilogue's per-row amax is an in-lane reduction plus one shuffle and one LDS hop.
+ * Workgroup tile = 128 aligned rows x 256 weight rows (GLU: 128 gate + 128 up rows of one
+ * 128-channel block; DOWN: 256 output channels), K walked in 128-k blocks through a ring of three
+ * LDS stages. The twelve waves are specialised:
  *
- * The layer is bound by the weight stream, so the loop is built to keep global loads in flight at
- * all times: both operands go global -> LDS directly (global_load_lds_dwordx4, no staging
- * registers) into a ring of three 128-k stages; while stage s is multiplied, stages s+1 and s+2 are
- * in flight. Each wave waits for its own loads of a stage with s_waitcnt vmcnt(n), then an LDS-only
- * barrier publishes the stage. A direct load writes the 64 lanes' 16-byte pieces to consecutive LDS
- * addresses, so rows sit unpadded (128 B) and bank conflicts are avoided by swizzling on the GLOBAL
- * side: LDS piece p of row r holds global piece p ^ ((r >> 1) & 7); the operand reads of 16
- * consecutive rows then cover all 64 banks.
- * Rows of the tile beyond the expert's live rows read some valid row and carry a zero activation
- * scale, so they contribute nothing and are never stored.
- * Per 128-k block: t = two chained matrix instructions (k 0..63, 64..127), then
- * acc = fmaf(t, a_scale[row][kb] * w_scale[nb][kb], acc).
+ *   waves 8..11, loaders   issue every global load of the tile, all of them direct global -> LDS
+ *                          (global_load_lds_dwordx4), with 8 consecutive lanes on one 128-byte line,
+ *                          the only lane -> address shape the vector memory pipeline takes at full
+ *                          rate (a "lane = matrix row" load runs at a quarter of it). A loader that
+ *                          finds the load queue full stalls only itself.
+ *   waves 0..7, consumers  two per SIMD; read operands from LDS and multiply. Consumer c owns 32 of
+ *                          the 256 weight rows (two 16-row groups; GLU: gate and up of channels
+ *                          16c..16c+15) and all 128 token rows, on
+ *                          v_mfma_f32_16x16x128_f8f6f4 with weights as the A operand and token rows
+ *                          as the B operand: a lane's accumulators belong to ONE token row (lane & 15
+ *                          of each 16-row group) and four consecutive channels, so the 1x128
+ *                          activation scale is one value per lane and row group, and gate / up of a
+ *                          channel sit in the same lane and register index.
+ *
+ * Per 128-k block: a loader waits for its own loads of the block (s_waitcnt vmcnt(n)), then all
+ * waves meet at one barrier; after it the consumers multiply the block while the loaders refill the
+ * stage the consumers have just left, two blocks ahead. Per 16-row group a consumer issues two
+ * matrix instructions (one per weight group) and acc = fmaf(t, a_scale[row][kb] * w_scale, acc); the
+ * next group's B operand is read from LDS meanwhile.
+ *
+ * A direct load writes the 64 lanes' 16-byte pieces to consecutive LDS addresses, so rows sit
+ * unpadded (128 B); bank conflicts are avoided by swizzling on the GLOBAL side: LDS piece p of row r
+ * holds global piece p ^ ((r >> 1) & 7), and the operand reads of 16 consecutive rows then cover all
+ * 64 banks. Rows of the tile beyond the expert's live rows read the tile's first row and carry a
+ * zero activation scale; 16-row groups with no live row are skipped by the consumers.
  * Tiles are walked by persistent workgroups (one per CU) in an order that puts the tiles sharing
- * activation rows and weight rows on one XCD at the same time (see the tile loop). */
+ * token rows and weight rows on one XCD at the same time (see the tile loop). */
 #include "common.h"
 #include "kernels.h"
 
-#define T2_BM 128u
-#define T2_BN 128u
-#define T2_THREADS 512u
-#define T2_STAGES 3u
+#define T5_BM 128u
+#define T5_THREADS 768u /* 8 consumer waves + 4 loader waves */
+#define T5_STAGES 3u
+#define T5_NLOAD 13 /* direct loads per loader and block: 1 scale, 4 token-row, 8 weight-row */
 
-struct T2Lds {
-    uint8_t a[T2_STAGES][T2_BM * 128u]; /* activations, swizzled */
-    uint8_t w[T2_STAGES][256u * 128u];  /* weights, swizzled (GLU: rows 0..127 gate, 128..255 up) */
-    float as[T2_STAGES][T2_BM];         /* activation scales of the stage's 128-k block */
-    float wsc[2][128];                  /* this tile's weight block scales, all of K (gate|down, up) */
-    float red[4][T2_BM];                /* GLU: per-row amax of each 32-channel wave column */
-    uint32_t scan[T2_THREADS];
+struct T5Lds {
+    uint8_t a[T5_STAGES][T5_BM * 128u]; /* token rows of a 128-k block, swizzled */
+    uint8_t w[T5_STAGES][256u * 128u];  /* weight rows, swizzled; row = 32 * consumer + 16 * group + r */
+    float as[T5_STAGES][T5_BM];         /* activation scales of the block */
+    float wsc[2][128];                  /* this tile's weight block scales, all of K */
+    float red[8][T5_BM];                /* GLU: per-row amax of each consumer's 16 channels */
     uint32_t prefix[1056];
 };
 
 typedef __attribute__((address_space(3))) void lds_void;
 
-/* vmcnt(n) with lgkmcnt / expcnt left open (gfx9 encoding: vmcnt = [3:0] | [15:14]) */
-#define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
-
-/* The stage buffers are written by direct global -> LDS loads that the compiler would otherwise
- * fence conservatively (a full s_waitcnt vmcnt(0) before every LDS read and barrier, which would
- * serialise the ring). So the ring is read with explicit ds_read instructions and synchronised with
- * explicit waits: the code below, not the compiler, decides which loads must have landed. */
+/* The ring is written by direct global -> LDS loads that the compiler would otherwise fence
+ * conservatively (a full s_waitcnt vmcnt(0) before every LDS read and barrier). So the ring is read
+ * with explicit ds_read instructions and synchronised with explicit waits. */
 __device__ __forceinline__ uint32_t lds_off(const void* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }
+template <uint32_t OFF>
 __device__ __forceinline__ v4i ds_read16(uint32_t addr) {
     v4i r;
-    asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
     return r;
 }
+template <uint32_t OFF>
 __device__ __forceinline__ float ds_read4(uint32_t addr) {
     float r;
-    asm volatile("ds_read_b32 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
     return r;
 }
-/* logical 16-byte pieces j, j + 1 of `row` (j even); piece p lives at p ^ ((row >> 1) & 7) */
-__device__ __forceinline__ void lds_operand(uint32_t base, uint32_t row, uint32_t j, v4i& lo, v4i& hi) {
-    const uint32_t sw = (row >> 1) & 7u;
-    lo = ds_read16(base + row * 128u + ((j ^ sw) << 4));
-    hi = ds_read16(base + row * 128u + (((j + 1u) ^ sw) << 4));
-}
-/* all ds_reads issued so far have returned; the operands are tied so nothing is hoisted above */
-#define LDS_WAIT4(a, b, c, d) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d))
-#define LDS_WAIT2F(a, b) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b))
+/* all ds_reads issued so far have returned; the operands are tied so no use is hoisted above */
+#define LDS_WAIT2(a, b) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b))
+#define LDS_WAIT_F(a) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a))
+#define LDS_WAIT_ALL() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
+#define WG_BARRIER() asm volatile("s_barrier" ::: "memory")
 /* wait until at most n of this wave's loads are outstanding, then the workgroup barrier */
 #define STAGE_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(n) : "memory")
 
-#ifdef T2_PROF
-__device__ unsigned long long t2_prof[2][256][8];
+#ifdef T5_PROF
+__device__ unsigned long long t5_prof[2][256][8];
 #define PROF_STAMP(v) const unsigned long long v = __builtin_readcyclecounter()
 #else
 #define PROF_STAMP(v)
 #endif
+
 template <bool GLU>
-__global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
+__global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    T2Lds& L = *(T2Lds*)lds_raw;
+    T5Lds& L = *(T5Lds*)lds_raw;
+    constexpr uint32_t BN = GLU ? 128u : 256u; /* output channels per tile */
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t NT = g.N / T2_BN;
-    constexpr uint32_t WG_PER_WAVE = GLU ? 4u : 2u; /* 8-row weight groups each wave loads per stage */
-    constexpr uint32_t NLOAD = 3u + WG_PER_WAVE;    /* direct loads per wave and stage: 2 row groups of
-                                                     * activations, the weight groups, 64 scales */
+    const bool loader = wv >= 8u;
+    const uint32_t cw = loader ? wv - 8u : wv; /* loader index 0..3, or consumer index 0..7 */
+    const uint32_t NT = (g.N + BN - 1u) / BN;
+    const uint32_t r16 = lane & 15u, q = lane >> 4;
 
-    /* ---- tile directory: inclusive prefix of ceil(cnt / 128) over experts, in LDS ---- */
+    /* ---- tile directory: inclusive prefix of ceil(cnt / 128) over experts, in LDS (the scan
+     *      scratch borrows the ring, which is idle here) ---- */
     {
+        uint32_t* scan = (uint32_t*)&L.a[0][0];
         uint32_t carry = 0;
-        for (uint32_t e0 = 0; e0 < g.E; e0 += T2_THREADS) {
+        for (uint32_t e0 = 0; e0 < g.E; e0 += T5_THREADS) {
             const uint32_t e = e0 + tid;
-            const uint32_t t = e < g.E ? ((uint32_t)g.meta[g.E + e] + T2_BM - 1u) / T2_BM : 0u;
-            L.scan[tid] = t;
+            const uint32_t t = e < g.E ? ((uint32_t)g.meta[g.E + e] + T5_BM - 1u) / T5_BM : 0u;
+            scan[tid] = t;
             __syncthreads();
-            for (uint32_t o = 1; o < T2_THREADS; o <<= 1) {
-                const uint32_t v = tid >= o ? L.scan[tid - o] : 0u;
+            for (uint32_t o = 1; o < T5_THREADS; o <<= 1) {
+                const uint32_t v = tid >= o ? scan[tid - o] : 0u;
                 __syncthreads();
-                L.scan[tid] += v;
+                scan[tid] += v;
                 __syncthreads();
             }
-            if (e < g.E) L.prefix[e] = carry + L.scan[tid];
-            carry += L.scan[T2_THREADS - 1u];
+            if (e < g.E) L.prefix[e] = carry + scan[tid];
+            carry += scan[T5_THREADS - 1u];
             __syncthreads();
         }
     }
-#ifdef T2_PROF
+#ifdef T5_PROF
     unsigned long long pf_setup = 0, pf_ramp = 0, pf_loop = 0, pf_epi = 0, pf_tiles = 0;
     const unsigned long long pf_begin = __builtin_readcyclecounter();
 #endif
     const uint32_t total = L.prefix[g.E - 1u] * NT;
     const uint32_t K = g.K, KB = K / 128u;
-    const uint32_t wr = wv & 1u, wc = wv >> 1, l32 = lane & 31u, lh = lane >> 5;
+    const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]);
+    const uint32_t s_base = lds_off(&L.as[0][0]), c_base = lds_off(&L.wsc[0][0]);
+    /* consumer: this lane's operand pieces 2q, 2q + 1 of row (16 * group + r16) */
+    const uint32_t sw = (r16 >> 1) & 7u;
+    const uint32_t op_lo = r16 * 128u + (((2u * q) ^ sw) << 4), op_hi = r16 * 128u + (((2u * q + 1u) ^ sw) << 4);
 
     /* Workgroup w runs on XCD w % 8 (round-robin dispatch), and each XCD has its own L2. The logical
      * index below makes the 32 workgroups of one XCD take 32 consecutive tiles of every sweep, and the
-     * tile order inside an expert is (16-channel-tile chunk, row tile, channel tile in the chunk): those
-     * 32 tiles are then two row tiles x 16 channel tiles of one expert, which read the same activation
-     * rows and the same weight rows at about the same time and meet in that L2. */
+     * tile order inside an expert is (16-channel-tile chunk, row tile, channel tile in the chunk), so
+     * that those tiles read the same token rows and the same weight rows at about the same time and
+     * meet in that L2. */
     const uint32_t G = gridDim.x;
     const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
     const uint32_t FC = NT / 16u, RC = NT % 16u;
@@ -134,8 +145,8 @@ __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             const uint32_t mid = (lo + hi) >> 1;
             if (L.prefix[mid] > mt_global) hi = mid; else lo = mid + 1u;
         }
-        /* the same value in every lane; made explicit so that everything indexed by the expert (pointer
-         * tables, block scales) is read with scalar loads and never waits on the vector-load counter */
+        /* the same value in every lane; made explicit so that everything indexed by the expert is
+         * read with scalar loads */
         const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)lo);
         const uint32_t pbase = e ? L.prefix[e - 1u] : 0u, Me = L.prefix[e] - pbase;
         const uint32_t idx = tile - pbase * NT;
@@ -149,247 +160,270 @@ __global__ __launch_bounds__(T2_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
         }
         const uint32_t mt = (uint32_t)__builtin_amdgcn_readfirstlane((int)mt_v);
         const uint32_t nt = (uint32_t)__builtin_amdgcn_readfirstlane((int)nt_v);
-        const uint32_t cnt = (uint32_t)g.meta[g.E + e], r0 = (uint32_t)g.meta[e] + mt * T2_BM;
-        const uint32_t rows = cnt - mt * T2_BM < T2_BM ? cnt - mt * T2_BM : T2_BM; /* live rows here */
+        const uint32_t cnt = (uint32_t)g.meta[g.E + e], r0 = (uint32_t)g.meta[e] + mt * T5_BM;
+        const uint32_t rows = cnt - mt * T5_BM < T5_BM ? cnt - mt * T5_BM : T5_BM; /* live rows here */
+        const uint32_t ngrp = (rows + 15u) / 16u;                                   /* live 16-row groups */
         const uint64_t wp0 = g.wtab[(size_t)e * 3u + (GLU ? 0u : 2u)];
-        if (wp0 == 0ull) continue; /* expert not resident */
-        const uint8_t* W0 = (const uint8_t*)(uintptr_t)wp0;
-        const uint8_t* W1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * 3u + 1u] : nullptr;
-        const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u + (GLU ? 0u : 2u)] + (size_t)nt * KB;
-        const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * 3u + 1u] + (size_t)nt * KB : nullptr;
+        if (wp0 == 0ull) continue; /* expert not resident (the same decision in every wave) */
+        const uint32_t nblk = g.N / 128u;
 
-        /* ---- loader: a direct load covers 8 rows x 128 B; lane -> (row l>>3, LDS piece l&7) ---- */
-        const uint8_t* asrc[2];
-        const uint8_t* wsrc[WG_PER_WAVE];
-#pragma unroll
-        for (uint32_t i = 0; i < 2u; i++) { /* activation rows 16*wv + 8*i + (lane >> 3) */
-            const uint32_t row = 16u * wv + 8u * i + (lane >> 3), p = lane & 7u;
-            uint32_t src; /* a pad row reads the tile's first row; its scale is zero */
-            if (GLU) {
-                const uint32_t tok = row < rows ? g.row_token[r0 + row] : PLOW_EXPERT_UNUSED;
-                src = tok != PLOW_EXPERT_UNUSED ? tok : g.row_token[r0];
-            } else {
-                src = r0 + (row < rows ? row : 0u);
-            }
-            asrc[i] = (const uint8_t*)g.a + (size_t)src * K + ((p ^ ((row >> 1) & 7u)) << 4);
-        }
-#pragma unroll
-        for (uint32_t i = 0; i < WG_PER_WAVE; i++) { /* weight rows 8*(WG_PER_WAVE*wv + i) + (lane >> 3) */
-            const uint32_t row = 8u * (WG_PER_WAVE * wv + i) + (lane >> 3), p = lane & 7u;
-            const uint8_t* base = (GLU && row >= 128u) ? W1 : W0;
-            wsrc[i] = base + (size_t)(nt * T2_BN + (row & 127u)) * K + ((p ^ ((row >> 1) & 7u)) << 4);
-        }
-        /* activation scale of row (wv & 1) * 64 + lane (every wave pair loads the same 64 values);
-         * a pad row reads tilep[0], which is always 0 */
-        const float* ssrc;
-        uint32_t sstep;
+        /* weight block scales of the tile: GLU gate | up of channel block nt; DOWN blocks 2nt, 2nt + 1 */
         {
-            const uint32_t row = (wv & 1u) * 64u + lane;
-            bool ok = row < rows;
-            if (GLU) {
-                const uint32_t tok = ok ? g.row_token[r0 + row] : PLOW_EXPERT_UNUSED;
-                ok = tok != PLOW_EXPERT_UNUSED;
-                ssrc = ok ? g.a_scale + tok : (const float*)(g.meta + 2u * g.E);
-                sstep = ok ? g.pitch : 0u;
-            } else {
-                ok = ok && g.row_partidx[r0 + row] != PLOW_EXPERT_UNUSED;
-                ssrc = ok ? g.a_scale + (size_t)(r0 + row) * KB : (const float*)(g.meta + 2u * g.E);
-                sstep = ok ? 1u : 0u;
+            const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u + (GLU ? 0u : 2u)];
+            const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * 3u + 1u] : S0;
+            const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
+            for (uint32_t i = tid; i < KB; i += T5_THREADS) {
+                L.wsc[0][i] = S0[(size_t)nb0 * KB + i];
+                L.wsc[1][i] = S1[(size_t)nb1 * KB + i];
             }
         }
-        auto issue = [&](uint32_t kb) {
-            const uint32_t st = kb % T2_STAGES;
-#ifdef T2_NOSTREAM
-            kb &= 1u;
-#endif
-            __builtin_amdgcn_global_load_lds((const void*)(ssrc + (size_t)kb * sstep),
-                                             (lds_void*)&L.as[st][(wv & 1u) * 64u], 4, 0, 0);
-#pragma unroll
-            for (uint32_t i = 0; i < 2u; i++)
-                __builtin_amdgcn_global_load_lds((const void*)(asrc[i] + (size_t)kb * 128u),
-                                                 (lds_void*)&L.a[st][(16u * wv + 8u * i) * 128u], 16, 0, 0);
-#pragma unroll
-            for (uint32_t i = 0; i < WG_PER_WAVE; i++)
-                __builtin_amdgcn_global_load_lds((const void*)(wsrc[i] + (size_t)kb * 128u),
-                                                 (lds_void*)&L.w[st][8u * (WG_PER_WAVE * wv + i) * 128u], 16, 0, 0);
-        };
 
-        /* ---- this lane's two B-operand rows ---- */
-        bool rvalid[2];
+        if (loader) {
+            /* ================= loader ================= */
+            /* a direct load covers 8 rows x 128 B: lane -> (row l >> 3, LDS piece l & 7) */
+            const uint32_t lr = lane >> 3, p = lane & 7u;
+            /* per-lane 32-bit byte offsets from uniform bases: the loads take (scalar base + k offset,
+             * vector offset) and the loader keeps 12 offsets instead of 12 pointers */
+            const uint8_t* const A0 = (const uint8_t*)g.a;
+            const uint8_t* const W0 = (const uint8_t*)(uintptr_t)wp0;
+            const uint8_t* const W1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * 3u + 1u] : W0;
+            uint32_t aoff[4]; /* token rows 32 * cw + 8 * i + lr */
 #pragma unroll
-        for (int rt = 0; rt < 2; rt++) {
-            const uint32_t row = wr * 64u + (uint32_t)rt * 32u + l32;
-            rvalid[rt] = row < rows;
-            if (GLU) rvalid[rt] = rvalid[rt] && g.row_token[r0 + row] != PLOW_EXPERT_UNUSED;
-            else rvalid[rt] = rvalid[rt] && g.row_partidx[r0 + row] != PLOW_EXPERT_UNUSED;
-        }
-        const bool wave_live = wr * 64u < rows; /* a wave whose rows are all pad does no matrix work */
-
-        v16f acc[2][GLU ? 2 : 1];
+            for (uint32_t i = 0; i < 4u; i++) {
+                const uint32_t row = 32u * cw + 8u * i + lr;
+                uint32_t src; /* a pad row reads the tile's first row; its scale is zero */
+                if (GLU) {
+                    const uint32_t tok = row < rows ? g.row_token[r0 + row] : PLOW_EXPERT_UNUSED;
+                    src = tok != PLOW_EXPERT_UNUSED ? tok : g.row_token[r0];
+                } else {
+                    src = r0 + (row < rows ? row : 0u);
+                }
+                aoff[i] = src * K + ((p ^ ((row >> 1) & 7u)) << 4);
+            }
+            /* LDS weight rows R = 64 * cw + 8 * i + lr: consumer R / 32, group (R / 16) & 1 = (i >> 1) & 1 */
+            uint32_t woff[8];
 #pragma unroll
-        for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-            for (int gu = 0; gu < (GLU ? 2 : 1); gu++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) acc[rt][gu][i] = 0.0f;
-
-        /* the tile's weight block scales go to LDS once, so that the loop below has no ordinary
-         * vector load whose wait would also wait for the ring */
-        for (uint32_t i = tid; i < KB; i += T2_THREADS) {
-            L.wsc[0][i] = S0[i];
-            if (GLU) L.wsc[1][i] = S1[i];
-        }
-        __syncthreads();
-        issue(0);
-        if (KB > 1u) issue(1);
-        const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]), s_base = lds_off(&L.as[0][0]);
-        const uint32_t c_base = lds_off(&L.wsc[0][0]);
-        PROF_STAMP(ts1);
-#ifdef T2_PROF
-        unsigned long long ts2 = 0;
-#endif
-        for (uint32_t kb = 0; kb < KB; kb++) {
-            const uint32_t st = kb % T2_STAGES;
-            /* this wave's loads of stage kb have landed once at most the next stage's are outstanding;
-             * after the barrier stage kb is complete and the buffer of stage kb-1 is free */
-            if (kb + 1u < KB) STAGE_BARRIER(NLOAD); else STAGE_BARRIER(0);
-#ifdef T2_PROF
-            if (kb == 0) ts2 = __builtin_readcyclecounter();
-#endif
-            if (kb + 2u < KB) issue(kb + 2u);
-            if (wave_live) {
-                float ws0 = ds_read4(c_base + kb * 4u);
-                float ws1 = ds_read4(c_base + ((GLU ? 128u : 0u) + kb) * 4u);
-                const uint32_t ab = a_base + st * (T2_BM * 128u), wb = w_base + st * (256u * 128u);
-                v4i bl[2][2], bh[2][2];
-#pragma unroll
-                for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-                    for (int kk = 0; kk < 2; kk++)
-                        lds_operand(ab, wr * 64u + (uint32_t)rt * 32u + l32, 4u * kk + 2u * lh, bl[rt][kk], bh[rt][kk]);
-                float asv0 = ds_read4(s_base + (st * T2_BM + wr * 64u + l32) * 4u);
-                float asv1 = ds_read4(s_base + (st * T2_BM + wr * 64u + 32u + l32) * 4u);
-                LDS_WAIT4(bl[0][0], bh[0][0], bl[0][1], bh[0][1]);
-                LDS_WAIT4(bl[1][0], bh[1][0], bl[1][1], bh[1][1]);
-                LDS_WAIT2F(asv0, asv1);
-                LDS_WAIT2F(ws0, ws1);
-                const float asv[2] = {asv0, asv1};
-                v8i bf[2][2];
-#pragma unroll
-                for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-                    for (int kk = 0; kk < 2; kk++)
-                        bf[rt][kk] = __builtin_shufflevector(bl[rt][kk], bh[rt][kk], 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-                for (int gu = 0; gu < (GLU ? 2 : 1); gu++) {
-                    const uint32_t wrow = (uint32_t)gu * 128u + wc * 32u + l32;
-                    v4i a0l, a0h, a1l, a1h;
-                    lds_operand(wb, wrow, 2u * lh, a0l, a0h);
-                    lds_operand(wb, wrow, 4u + 2u * lh, a1l, a1h);
-                    LDS_WAIT4(a0l, a0h, a1l, a1h);
-                    const v8i af0 = __builtin_shufflevector(a0l, a0h, 0, 1, 2, 3, 4, 5, 6, 7);
-                    const v8i af1 = __builtin_shufflevector(a1l, a1h, 0, 1, 2, 3, 4, 5, 6, 7);
-                    const float wsc = gu ? ws1 : ws0;
-#pragma unroll
-                    for (int rt = 0; rt < 2; rt++) {
-                        v16f t;
-#pragma unroll
-                        for (int i = 0; i < 16; i++) t[i] = 0.0f;
-                        t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af0, bf[rt][0], t, 0, 0, 0, 0, 0, 0);
-                        t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af1, bf[rt][1], t, 0, 0, 0, 0, 0, 0);
-                        const float sc = asv[rt] * wsc;
-#pragma unroll
-                        for (int i = 0; i < 16; i++) acc[rt][gu][i] = fmaf(t[i], sc, acc[rt][gu][i]);
-                    }
+            for (uint32_t i = 0; i < 8u; i++) {
+                const uint32_t R = 64u * cw + 8u * i + lr;
+                uint32_t ch;
+                if (GLU) {
+                    ch = nt * 128u + 16u * (R >> 5) + (R & 15u);
+                } else {
+                    ch = nt * 256u + R;
+                    if (ch >= g.N) ch = 0; /* past the last channel: any valid row, never stored */
+                }
+                woff[i] = ch * K + ((p ^ ((R >> 1) & 7u)) << 4);
+            }
+            /* activation scale of row (cw & 1) * 64 + lane (loaders 0, 2 and 1, 3 load the same 64
+             * values); a pad row reads tilep[0], which is always 0 */
+            const float* ssrc;
+            uint32_t sstep;
+            {
+                const uint32_t row = (cw & 1u) * 64u + lane;
+                bool ok = row < rows;
+                if (GLU) {
+                    const uint32_t tok = ok ? g.row_token[r0 + row] : PLOW_EXPERT_UNUSED;
+                    ok = tok != PLOW_EXPERT_UNUSED;
+                    ssrc = ok ? g.a_scale + tok : (const float*)(g.meta + 2u * g.E);
+                    sstep = ok ? g.pitch : 0u;
+                } else {
+                    ok = ok && g.row_partidx[r0 + row] != PLOW_EXPERT_UNUSED;
+                    ssrc = ok ? g.a_scale + (size_t)(r0 + row) * KB : (const float*)(g.meta + 2u * g.E);
+                    sstep = ok ? 1u : 0u;
                 }
             }
-        }
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); /* ring drained */
-        PROF_STAMP(ts3);
-
-        /* ---- epilogue. Lane: row = wr*64 + rt*32 + l32; channels wc*32 + 8*(i/4) + 4*lh + (i%4) ---- */
-        if (GLU) {
-            float v[2][16];
+            auto issue = [&](uint32_t kb) {
+                const uint32_t st = kb % T5_STAGES;
+#ifdef T5_NOSTREAM
+                kb &= 1u;
+#endif
+                __builtin_amdgcn_global_load_lds((const void*)(ssrc + (size_t)kb * sstep),
+                                                 (lds_void*)&L.as[st][(cw & 1u) * 64u], 4, 0, 0);
+                const uint8_t* const ak = A0 + (size_t)kb * 128u;
+                const uint8_t* const wk0 = W0 + (size_t)kb * 128u;
+                const uint8_t* const wk1 = W1 + (size_t)kb * 128u;
 #pragma unroll
-            for (int rt = 0; rt < 2; rt++) {
-                float m = 0.0f;
+                for (uint32_t i = 0; i < 4u; i++)
+                    __builtin_amdgcn_global_load_lds((const void*)(ak + aoff[i]),
+                                                     (lds_void*)&L.a[st][(32u * cw + 8u * i) * 128u], 16, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    v[rt][i] = moe_glu(acc[rt][0][i], acc[rt][GLU ? 1 : 0][i], g.act);
-                    m = fmaxf(m, fabsf(v[rt][i]));
-                }
-                m = fmaxf(m, __shfl_xor(m, 32, 64));
-                if (lh == 0) L.red[wc][wr * 64u + (uint32_t)rt * 32u + l32] = m;
+                for (uint32_t i = 0; i < 8u; i++)
+                    __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + woff[i]),
+                                                     (lds_void*)&L.w[st][(64u * cw + 8u * i) * 128u], 16, 0, 0);
+            };
+            __syncthreads(); /* tile start: L.wsc written, every wave done with the previous tile */
+            issue(0);
+            if (KB > 1u) issue(1);
+            for (uint32_t kb = 0; kb < KB; kb++) {
+                /* loads return in order: block kb has landed once at most block kb + 1's are outstanding.
+                 * After the barrier the consumers are done with block kb - 1, whose stage is refilled. */
+                if (kb + 1u < KB) STAGE_BARRIER(T5_NLOAD); else STAGE_BARRIER(0);
+                if (kb + 2u < KB) issue(kb + 2u);
             }
-            lds_barrier();
-#pragma unroll
-            for (int rt = 0; rt < 2; rt++) {
-                const uint32_t row = wr * 64u + (uint32_t)rt * 32u + l32;
-                if (!rvalid[rt]) continue;
-                const float amax = fmaxf(fmaxf(1e-10f, L.red[0][row]), fmaxf(fmaxf(L.red[1][row], L.red[2][row]), L.red[3][row]));
-                const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
-                uint8_t* orow = (uint8_t*)g.out + (size_t)(r0 + row) * g.N + nt * T2_BN + wc * 32u + 4u * lh;
-#pragma unroll
-                for (int i4 = 0; i4 < 4; i4++)
-                    *(uint32_t*)(orow + i4 * 8) = cvt4_e4m3(v[rt][4 * i4] * inv, v[rt][4 * i4 + 1] * inv,
-                                                            v[rt][4 * i4 + 2] * inv, v[rt][4 * i4 + 3] * inv);
-                if (wc == 0 && lh == 0) g.out_scale[(size_t)(r0 + row) * NT + nt] = s;
-            }
+            WG_BARRIER(); /* end of the k loop: GLU amax exchange; L.wsc may be rewritten after it */
         } else {
+            /* ================= consumer ================= */
+            const uint32_t ch0 = GLU ? nt * 128u + 16u * cw : nt * 256u + 32u * cw; /* first channel */
+            const bool wave_on = ch0 < g.N; /* DOWN: N may end mid-tile (N is a multiple of 128) */
+            const uint32_t ngrp_w = wave_on ? ngrp : 0u;
+            bool rvalid[8];
 #pragma unroll
-            for (int rt = 0; rt < 2; rt++) {
-                const uint32_t row = wr * 64u + (uint32_t)rt * 32u + l32;
-                if (!rvalid[rt]) continue;
-                const uint32_t pidx = g.row_partidx[r0 + row];
-                const float gate = g.row_gate[r0 + row];
-                const size_t ocol = (size_t)pidx * g.N + nt * T2_BN + wc * 32u + 4u * lh;
+            for (int rg = 0; rg < 8; rg++) {
+                const uint32_t row = 16u * (uint32_t)rg + r16;
+                rvalid[rg] = row < rows;
+                if (rvalid[rg]) rvalid[rg] = (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) != PLOW_EXPERT_UNUSED;
+            }
+            v4f acc[8][2];
 #pragma unroll
-                for (int i4 = 0; i4 < 4; i4++) {
-                    const float y0 = gate * acc[rt][0][4 * i4], y1 = gate * acc[rt][0][4 * i4 + 1];
-                    const float y2 = gate * acc[rt][0][4 * i4 + 2], y3 = gate * acc[rt][0][4 * i4 + 3];
-                    if (g.part16) {
-                        uint2 o;
-                        o.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16);
-                        o.y = (uint32_t)f2bf(y2) | ((uint32_t)f2bf(y3) << 16);
-                        *(uint2*)((bf16_t*)g.out + ocol + i4 * 8) = o;
-                    } else {
-                        *(float4*)((float*)g.out + ocol + i4 * 8) = make_float4(y0, y1, y2, y3);
+            for (int rg = 0; rg < 8; rg++)
+#pragma unroll
+                for (int t = 0; t < 2; t++) acc[rg][t] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+            __syncthreads(); /* tile start (pairs with the loaders') */
+            PROF_STAMP(ts1);
+#ifdef T5_PROF
+            unsigned long long ts2 = 0;
+#endif
+            for (uint32_t kb = 0; kb < KB; kb++) {
+                WG_BARRIER(); /* block kb is in LDS */
+#ifdef T5_PROF
+                if (kb == 0) ts2 = __builtin_readcyclecounter();
+#endif
+                const uint32_t st = kb % T5_STAGES;
+                const uint32_t ab = a_base + st * (T5_BM * 128u), wb = w_base + st * (256u * 128u) + cw * (32u * 128u);
+                const uint32_t blo = ab + op_lo, bhi = ab + op_hi;
+                const uint32_t alo = wb + op_lo, ahi = wb + op_hi;
+                const uint32_t sl = s_base + st * (T5_BM * 4u) + r16 * 4u;
+                const uint32_t cl = c_base + kb * 4u;
+                if (ngrp_w == 0u) continue;
+                float ws0 = ds_read4<0>(cl);
+                float ws1 = ds_read4<512>(cl);
+                v4i al[2], ah[2];
+                al[0] = ds_read16<0>(alo), ah[0] = ds_read16<0>(ahi);
+                al[1] = ds_read16<2048>(alo), ah[1] = ds_read16<2048>(ahi);
+                v4i bl[2], bh[2];
+                float as_[2];
+                bl[0] = ds_read16<0>(blo), bh[0] = ds_read16<0>(bhi);
+                as_[0] = ds_read4<0>(sl);
+                LDS_WAIT2(ws0, ws1);
+                LDS_WAIT2(al[0], ah[0]);
+                LDS_WAIT2(al[1], ah[1]);
+                if (!GLU) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);
+                v8i aop[2];
+#pragma unroll
+                for (int t = 0; t < 2; t++) aop[t] = __builtin_shufflevector(al[t], ah[t], 0, 1, 2, 3, 4, 5, 6, 7);
+#define T5_GROUP(RG)                                                                                         \
+    if ((RG) < ngrp_w) {                                                                                     \
+        LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                               \
+        LDS_WAIT_F(as_[(RG) & 1]);                                                                           \
+        if ((RG) + 1 < 8 && (RG) + 1 < ngrp_w) {                                                             \
+            bl[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(blo);                                   \
+            bh[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(bhi);                                   \
+            as_[((RG) + 1) & 1] = ds_read4<(((RG) + 1) & 7) * 64u>(sl);                                      \
+        }                                                                                                    \
+        const v8i b = __builtin_shufflevector(bl[(RG) & 1], bh[(RG) & 1], 0, 1, 2, 3, 4, 5, 6, 7);           \
+        const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};                                                              \
+        const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, z, 0, 0, 0, 0, 0, 0);     \
+        const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, z, 0, 0, 0, 0, 0, 0);     \
+        const float sc0 = as_[(RG) & 1] * ws0, sc1 = as_[(RG) & 1] * ws1;                                    \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                      \
+            acc[RG][0][i] = fmaf(t0[i], sc0, acc[RG][0][i]);                                                 \
+            acc[RG][1][i] = fmaf(t1[i], sc1, acc[RG][1][i]);                                                 \
+        }                                                                                                    \
+    }
+                T5_GROUP(0) T5_GROUP(1) T5_GROUP(2) T5_GROUP(3) T5_GROUP(4) T5_GROUP(5) T5_GROUP(6) T5_GROUP(7)
+#undef T5_GROUP
+                LDS_WAIT_ALL(); /* nothing of this block is still being read when the next barrier is passed */
+            }
+            PROF_STAMP(ts3);
+
+            /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
+             *      group 0 and up in group 1; DOWN channel = ch0 + 16 * t + 4q + i ---- */
+            if (GLU) {
+                float v[8][4];
+#pragma unroll
+                for (int rg = 0; rg < 8; rg++) {
+                    float m = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        v[rg][i] = moe_glu(acc[rg][0][i], acc[rg][1][i], g.act);
+                        m = fmaxf(m, fabsf(v[rg][i]));
+                    }
+                    m = fmaxf(m, __shfl_xor(m, 16, 64));
+                    m = fmaxf(m, __shfl_xor(m, 32, 64));
+                    if (q == 0) L.red[cw][16u * (uint32_t)rg + r16] = m;
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+                for (int rg = 0; rg < 8; rg++) {
+                    const uint32_t row = 16u * (uint32_t)rg + r16;
+                    if (!rvalid[rg]) continue;
+                    float amax = 1e-10f;
+#pragma unroll
+                    for (int x = 0; x < 8; x++) amax = fmaxf(amax, L.red[x][row]);
+                    const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
+                    uint8_t* orow = (uint8_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
+                    *(uint32_t*)orow = cvt4_e4m3(v[rg][0] * inv, v[rg][1] * inv, v[rg][2] * inv, v[rg][3] * inv);
+                    if (cw == 0 && q == 0) g.out_scale[(size_t)(r0 + row) * NT + nt] = s;
+                }
+            } else {
+                WG_BARRIER(); /* end of the k loop (pairs with the loaders') */
+            }
+            if (!GLU && wave_on) {
+#pragma unroll
+                for (int rg = 0; rg < 8; rg++) {
+                    const uint32_t row = 16u * (uint32_t)rg + r16;
+                    if (!rvalid[rg]) continue;
+                    const uint32_t pidx = g.row_partidx[r0 + row];
+                    const float gate = g.row_gate[r0 + row];
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const size_t ocol = (size_t)pidx * g.N + ch0 + 16u * (uint32_t)t + 4u * q;
+                        const float y0 = gate * acc[rg][t][0], y1 = gate * acc[rg][t][1];
+                        const float y2 = gate * acc[rg][t][2], y3 = gate * acc[rg][t][3];
+                        if (g.part16) {
+                            uint2 o;
+                            o.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16);
+                            o.y = (uint32_t)f2bf(y2) | ((uint32_t)f2bf(y3) << 16);
+                            *(uint2*)((bf16_t*)g.out + ocol) = o;
+                        } else {
+                            *(float4*)((float*)g.out + ocol) = make_float4(y0, y1, y2, y3);
+                        }
                     }
                 }
             }
-        }
-        lds_barrier(); /* every wave is done with the ring and with L.red before the next tile refills them */
-#ifdef T2_PROF
-        {
-            const unsigned long long ts4 = __builtin_readcyclecounter();
-            pf_setup += ts1 - ts0, pf_ramp += ts2 - ts1, pf_loop += ts3 - ts2, pf_epi += ts4 - ts3, pf_tiles++;
-        }
+#ifdef T5_PROF
+            {
+                const unsigned long long ts4 = __builtin_readcyclecounter();
+                pf_setup += ts1 - ts0, pf_ramp += ts2 - ts1, pf_loop += ts3 - ts2, pf_epi += ts4 - ts3, pf_tiles++;
+            }
 #endif
+        }
     }
-#ifdef T2_PROF
+#ifdef T5_PROF
     if (tid == 0 && blockIdx.x < 256u) {
-        unsigned long long* o = t2_prof[GLU][blockIdx.x];
+        unsigned long long* o = t5_prof[GLU][blockIdx.x];
         o[0] = pf_setup, o[1] = pf_ramp, o[2] = pf_loop, o[3] = pf_epi, o[4] = pf_tiles;
         o[5] = __builtin_readcyclecounter() - pf_begin;
     }
 #endif
 }
-#ifdef T2_PROF
+#ifdef T5_PROF
 extern "C" int plow_moe_debug_prof(unsigned long long* out) {
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(t2_prof), sizeof(t2_prof));
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(t5_prof), sizeof(t5_prof));
 }
 #endif
 
 /* Persistent launch: one workgroup per CU; the tile count is computed on the device from meta. */
 template <bool GLU>
 static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
-    if (g.N == 0 || g.K == 0 || g.E == 0 || g.E > 1056u || g.N % T2_BN || g.K % 128u) return PLOW_MOE_EINVAL;
+    if (g.N == 0 || g.K == 0 || g.E == 0 || g.E > 1056u || g.N % 128u || g.K % 128u) return PLOW_MOE_EINVAL;
     if (g.K > 128u * 128u) return PLOW_MOE_EINVAL; /* the tile keeps K / 128 block scales in LDS */
     static bool attr_set[2] = {false, false};
     static int n_cu = 0;
     if (!attr_set[GLU]) {
         if (hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)sizeof(T2Lds)) != hipSuccess)
+                                (int)sizeof(T5Lds)) != hipSuccess)
             return PLOW_MOE_EDEVICE;
         attr_set[GLU] = true;
     }
@@ -399,7 +433,7 @@ static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return PLOW_MOE_EDEVICE;
         n_cu = prop.multiProcessorCount;
     }
-    k_group_w8a8_tiled<GLU><<<(uint32_t)n_cu, T2_THREADS, sizeof(T2Lds), st>>>(g);
+    k_group_w8a8_tiled<GLU><<<(uint32_t)n_cu, T5_THREADS, sizeof(T5Lds), st>>>(g);
     return 0;
 }
 
