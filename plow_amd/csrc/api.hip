@@ -202,6 +202,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.N = I; g.K = H; g.E = E; g.pitch = i[4]; g.act = i[5];
             /* many rows per expert (row pitch >= 2 rows per expert per routed slot): tiled form */
             c->tiled = c->forced >= 0 ? c->forced : (i[4] >= 2u * E ? 1 : 0);
+            if (H < 256u || I < 256u) c->tiled = 0; /* the tiled form needs two 128-k blocks in both GEMMs */
             return c->tiled ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||

@@ -44,7 +44,7 @@ struct T5Lds {
     uint8_t a[T5_STAGES][T5_BM * 128u]; /* token rows of a 128-k block, swizzled */
     uint8_t w[T5_STAGES][256u * 128u];  /* weight rows, swizzled; row = 32 * consumer + 16 * group + r */
     float as[T5_STAGES][T5_BM];         /* activation scales of the block */
-    float wsc[2][128];                  /* this tile's weight block scales, all of K */
+    float wsc[2][2][128];               /* [tile parity][gate|down, up] weight block scales, all of K */
     float red[8][T5_BM];                /* GLU: per-row amax of each consumer's 16 channels */
     uint32_t prefix[1056];
 };
@@ -75,7 +75,7 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
 #define LDS_WAIT_ALL() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
 #define WG_BARRIER() asm volatile("s_barrier" ::: "memory")
 /* wait until at most n of this wave's loads are outstanding, then the workgroup barrier */
-#define STAGE_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(n) : "memory")
+#define LOADER_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory")
 
 #ifdef T5_PROF
 __device__ unsigned long long t5_prof[2][256][8];
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
     const uint32_t total = L.prefix[g.E - 1u] * NT;
     const uint32_t K = g.K, KB = K / 128u;
     const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]);
-    const uint32_t s_base = lds_off(&L.as[0][0]), c_base = lds_off(&L.wsc[0][0]);
+    const uint32_t s_base = lds_off(&L.as[0][0]), c_base = lds_off(&L.wsc[0][0][0]);
     /* consumer: this lane's operand pieces 2q, 2q + 1 of row (16 * group + r16) */
     const uint32_t sw = (r16 >> 1) & 7u;
     const uint32_t op_lo = r16 * 128u + (((2u * q) ^ sw) << 4), op_hi = r16 * 128u + (((2u * q + 1u) ^ sw) << 4);
@@ -137,18 +137,23 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
     const uint32_t G = gridDim.x;
     const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
     const uint32_t FC = NT / 16u, RC = NT % 16u;
-    for (uint32_t tile = wg; tile < total; tile += G) {
-        PROF_STAMP(ts0);
+    const uint32_t nblk = g.N / 128u;
+    struct Tile {
+        uint32_t e, nt, r0, rows;
+        uint64_t wp0;
+    };
+    /* every value is the same in all lanes (made explicit with readfirstlane so that what is indexed
+     * by them is read with scalar loads) */
+    auto locate = [&](uint32_t tile) -> Tile {
         const uint32_t mt_global = tile / NT;
         uint32_t lo = 0, hi = g.E - 1u; /* first expert whose inclusive prefix exceeds mt_global */
         while (lo < hi) {
             const uint32_t mid = (lo + hi) >> 1;
             if (L.prefix[mid] > mt_global) hi = mid; else lo = mid + 1u;
         }
-        /* the same value in every lane; made explicit so that everything indexed by the expert is
-         * read with scalar loads */
-        const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)lo);
-        const uint32_t pbase = e ? L.prefix[e - 1u] : 0u, Me = L.prefix[e] - pbase;
+        Tile t;
+        t.e = (uint32_t)__builtin_amdgcn_readfirstlane((int)lo);
+        const uint32_t pbase = t.e ? L.prefix[t.e - 1u] : 0u, Me = L.prefix[t.e] - pbase;
         const uint32_t idx = tile - pbase * NT;
         uint32_t mt_v, nt_v;
         if (idx < FC * Me * 16u) {
@@ -159,51 +164,77 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             mt_v = rem / RC, nt_v = FC * 16u + rem % RC;
         }
         const uint32_t mt = (uint32_t)__builtin_amdgcn_readfirstlane((int)mt_v);
-        const uint32_t nt = (uint32_t)__builtin_amdgcn_readfirstlane((int)nt_v);
-        const uint32_t cnt = (uint32_t)g.meta[g.E + e], r0 = (uint32_t)g.meta[e] + mt * T5_BM;
-        const uint32_t rows = cnt - mt * T5_BM < T5_BM ? cnt - mt * T5_BM : T5_BM; /* live rows here */
-        const uint32_t ngrp = (rows + 15u) / 16u;                                   /* live 16-row groups */
-        const uint64_t wp0 = g.wtab[(size_t)e * 3u + (GLU ? 0u : 2u)];
-        if (wp0 == 0ull) continue; /* expert not resident (the same decision in every wave) */
-        const uint32_t nblk = g.N / 128u;
-
-        /* weight block scales of the tile: GLU gate | up of channel block nt; DOWN blocks 2nt, 2nt + 1 */
-        {
-            const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u + (GLU ? 0u : 2u)];
-            const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * 3u + 1u] : S0;
-            const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
-            for (uint32_t i = tid; i < KB; i += T5_THREADS) {
-                L.wsc[0][i] = S0[(size_t)nb0 * KB + i];
-                L.wsc[1][i] = S1[(size_t)nb1 * KB + i];
-            }
+        t.nt = (uint32_t)__builtin_amdgcn_readfirstlane((int)nt_v);
+        const uint32_t cnt = (uint32_t)g.meta[g.E + t.e];
+        t.r0 = (uint32_t)g.meta[t.e] + mt * T5_BM;
+        t.rows = cnt - mt * T5_BM < T5_BM ? cnt - mt * T5_BM : T5_BM; /* live rows of the tile */
+        t.wp0 = g.wtab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
+        return t;
+    };
+    /* this workgroup's next tile at or after `from` whose expert is resident (`total` if none); loaders
+     * and consumers walk the same sequence */
+    auto next_tile = [&](uint32_t from, Tile& t) -> uint32_t {
+        for (uint32_t tile = from; tile < total; tile += G) {
+            t = locate(tile);
+            if (t.wp0 != 0ull) return tile;
         }
+        return total;
+    };
 
-        if (loader) {
-            /* ================= loader ================= */
-            /* a direct load covers 8 rows x 128 B: lane -> (row l >> 3, LDS piece l & 7) */
-            const uint32_t lr = lane >> 3, p = lane & 7u;
+    /* Barrier protocol, identical in both roles: per tile, one barrier per 128-k block ("block kb of
+     * this tile is in LDS; everyone is done with the block before it") and one after the last block
+     * (GLU amax exchange). Ring slots and the L.wsc half alternate over a count that runs across
+     * tiles, so the loaders work ahead into the next tile while the consumers finish this one. */
+    if (loader) {
+        /* ================= loaders ================= */
+        /* a direct load covers 8 rows x 128 B: lane -> (row l >> 3, LDS piece l & 7) */
+        const uint32_t lr = lane >> 3, p = lane & 7u;
+        struct Src {
             /* per-lane 32-bit byte offsets from uniform bases: the loads take (scalar base + k offset,
-             * vector offset) and the loader keeps 12 offsets instead of 12 pointers */
-            const uint8_t* const A0 = (const uint8_t*)g.a;
-            const uint8_t* const W0 = (const uint8_t*)(uintptr_t)wp0;
-            const uint8_t* const W1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * 3u + 1u] : W0;
-            uint32_t aoff[4]; /* token rows 32 * cw + 8 * i + lr */
+             * vector offset) */
+            uint32_t aoff[4], woff[8], sstep;
+            const float* ssrc;
+            const uint8_t *W0, *W1;
+        };
+        const uint8_t* const A0 = (const uint8_t*)g.a;
+        /* Set-up of a tile's sources in two halves, so that its loads (row -> token, scales) are in
+         * flight while the loader keeps feeding the tile before: fetch() only issues loads, finish()
+         * uses them a few blocks later. Rows below the live count always hold a token. */
+        struct Pre {
+            uint32_t tok[4], stok;
+            float w0, w1;
+        };
+        auto fetch = [&](const Tile& t, Pre& P) {
+            const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
+#pragma unroll
+            for (uint32_t i = 0; i < 4u; i++) { /* token rows 32 * cw + 8 * i + lr; a pad row reads the first row */
+                const uint32_t row = 32u * cw + 8u * i + lr;
+                P.tok[i] = GLU ? g.row_token[r0 + (row < rows ? row : 0u)] : r0 + (row < rows ? row : 0u);
+            }
+            {
+                const uint32_t row = (cw & 1u) * 64u + lane; /* the row whose activation scale this lane loads */
+                P.stok = row < rows ? (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
+            }
+            /* weight block scales of the tile: GLU gate | up of channel block nt; DOWN blocks 2nt, 2nt + 1 */
+            const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
+            const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : S0;
+            const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
+            const uint32_t i = tid - 8u * 64u; /* 0..255 over the four loaders; KB <= 128 */
+            P.w0 = i < KB ? S0[(size_t)nb0 * KB + i] : 0.0f;
+            P.w1 = i < KB ? S1[(size_t)nb1 * KB + i] : 0.0f;
+        };
+        auto finish = [&](const Tile& t, const Pre& P, uint32_t par, Src& S) {
+            const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
+            S.W0 = (const uint8_t*)(uintptr_t)t.wp0;
+            S.W1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)t.e * 3u + 1u] : S.W0;
 #pragma unroll
             for (uint32_t i = 0; i < 4u; i++) {
                 const uint32_t row = 32u * cw + 8u * i + lr;
-                uint32_t src; /* a pad row reads the tile's first row; its scale is zero */
-                if (GLU) {
-                    const uint32_t tok = row < rows ? g.row_token[r0 + row] : PLOW_EXPERT_UNUSED;
-                    src = tok != PLOW_EXPERT_UNUSED ? tok : g.row_token[r0];
-                } else {
-                    src = r0 + (row < rows ? row : 0u);
-                }
-                aoff[i] = src * K + ((p ^ ((row >> 1) & 7u)) << 4);
+                const uint32_t src = GLU ? (P.tok[i] < g.pitch ? P.tok[i] : 0u) : P.tok[i];
+                S.aoff[i] = src * K + ((p ^ ((row >> 1) & 7u)) << 4);
             }
-            /* LDS weight rows R = 64 * cw + 8 * i + lr: consumer R / 32, group (R / 16) & 1 = (i >> 1) & 1 */
-            uint32_t woff[8];
 #pragma unroll
-            for (uint32_t i = 0; i < 8u; i++) {
+            for (uint32_t i = 0; i < 8u; i++) { /* LDS weight rows R = 64 * cw + 8 * i + lr: consumer R / 32, group (R / 16) & 1 */
                 const uint32_t R = 64u * cw + 8u * i + lr;
                 uint32_t ch;
                 if (GLU) {
@@ -212,74 +243,92 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                     ch = nt * 256u + R;
                     if (ch >= g.N) ch = 0; /* past the last channel: any valid row, never stored */
                 }
-                woff[i] = ch * K + ((p ^ ((R >> 1) & 7u)) << 4);
+                S.woff[i] = ch * K + ((p ^ ((R >> 1) & 7u)) << 4);
             }
             /* activation scale of row (cw & 1) * 64 + lane (loaders 0, 2 and 1, 3 load the same 64
              * values); a pad row reads tilep[0], which is always 0 */
-            const float* ssrc;
-            uint32_t sstep;
             {
                 const uint32_t row = (cw & 1u) * 64u + lane;
-                bool ok = row < rows;
+                const bool ok = P.stok != PLOW_EXPERT_UNUSED && (!GLU || P.stok < g.pitch);
                 if (GLU) {
-                    const uint32_t tok = ok ? g.row_token[r0 + row] : PLOW_EXPERT_UNUSED;
-                    ok = tok != PLOW_EXPERT_UNUSED;
-                    ssrc = ok ? g.a_scale + tok : (const float*)(g.meta + 2u * g.E);
-                    sstep = ok ? g.pitch : 0u;
+                    S.ssrc = ok ? g.a_scale + P.stok : (const float*)(g.meta + 2u * g.E);
+                    S.sstep = ok ? g.pitch : 0u;
                 } else {
-                    ok = ok && g.row_partidx[r0 + row] != PLOW_EXPERT_UNUSED;
-                    ssrc = ok ? g.a_scale + (size_t)(r0 + row) * KB : (const float*)(g.meta + 2u * g.E);
-                    sstep = ok ? 1u : 0u;
+                    S.ssrc = ok ? g.a_scale + (size_t)(r0 + row) * KB : (const float*)(g.meta + 2u * g.E);
+                    S.sstep = ok ? 1u : 0u;
                 }
             }
-            auto issue = [&](uint32_t kb) {
-                const uint32_t st = kb % T5_STAGES;
-#ifdef T5_NOSTREAM
-                kb &= 1u;
-#endif
-                __builtin_amdgcn_global_load_lds((const void*)(ssrc + (size_t)kb * sstep),
-                                                 (lds_void*)&L.as[st][(cw & 1u) * 64u], 4, 0, 0);
-                const uint8_t* const ak = A0 + (size_t)kb * 128u;
-                const uint8_t* const wk0 = W0 + (size_t)kb * 128u;
-                const uint8_t* const wk1 = W1 + (size_t)kb * 128u;
-#pragma unroll
-                for (uint32_t i = 0; i < 4u; i++)
-                    __builtin_amdgcn_global_load_lds((const void*)(ak + aoff[i]),
-                                                     (lds_void*)&L.a[st][(32u * cw + 8u * i) * 128u], 16, 0, 0);
-#pragma unroll
-                for (uint32_t i = 0; i < 8u; i++)
-                    __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + woff[i]),
-                                                     (lds_void*)&L.w[st][(64u * cw + 8u * i) * 128u], 16, 0, 0);
-            };
-            __syncthreads(); /* tile start: L.wsc written, every wave done with the previous tile */
-            issue(0);
-            if (KB > 1u) issue(1);
-            for (uint32_t kb = 0; kb < KB; kb++) {
-                /* loads return in order: block kb has landed once at most block kb + 1's are outstanding.
-                 * After the barrier the consumers are done with block kb - 1, whose stage is refilled. */
-                if (kb + 1u < KB) STAGE_BARRIER(T5_NLOAD); else STAGE_BARRIER(0);
-                if (kb + 2u < KB) issue(kb + 2u);
+            const uint32_t i = tid - 8u * 64u;
+            if (i < KB) {
+                L.wsc[par][0][i] = P.w0;
+                L.wsc[par][1][i] = P.w1;
             }
-            WG_BARRIER(); /* end of the k loop: GLU amax exchange; L.wsc may be rewritten after it */
-        } else {
-            /* ================= consumer ================= */
+        };
+        auto issue = [&](const Src& S, uint32_t kb, uint32_t st) {
+#ifdef T5_NOSTREAM
+            kb &= 1u;
+#endif
+            __builtin_amdgcn_global_load_lds((const void*)(S.ssrc + (size_t)kb * S.sstep),
+                                             (lds_void*)&L.as[st][(cw & 1u) * 64u], 4, 0, 0);
+            const uint8_t* const ak = A0 + (size_t)kb * 128u;
+            const uint8_t* const wk0 = S.W0 + (size_t)kb * 128u;
+            const uint8_t* const wk1 = S.W1 + (size_t)kb * 128u;
+#pragma unroll
+            for (uint32_t i = 0; i < 4u; i++)
+                __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[i]),
+                                                 (lds_void*)&L.a[st][(32u * cw + 8u * i) * 128u], 16, 0, 0);
+#pragma unroll
+            for (uint32_t i = 0; i < 8u; i++)
+                __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + S.woff[i]),
+                                                 (lds_void*)&L.w[st][(64u * cw + 8u * i) * 128u], 16, 0, 0);
+        };
+        Tile tcur, tnxt;
+        Src cur, nxt;
+        Pre pre;
+        uint32_t tile = next_tile(wg, tcur), par = 0, slot = 0; /* slot of the current tile's block 0 */
+        if (tile < total) {
+            fetch(tcur, pre);
+            finish(tcur, pre, 0u, cur);
+            issue(cur, 0u, 0u);
+            issue(cur, 1u, 1u);
+        }
+        const uint32_t kb_finish = KB >= 3u ? KB - 3u : 0u; /* the next tile's sources are needed from block KB - 2 on */
+        while (tile < total) {
+            const uint32_t ntile = next_tile(tile + G, tnxt);
+            const bool more = ntile < total;
+            uint32_t st = slot; /* slot of block kb */
+            for (uint32_t kb = 0; kb < KB; kb++) {
+                /* loads return in order: block kb has landed once at most the next block's loads (of this
+                 * tile or the next) are outstanding. After the barrier the consumers are done with the
+                 * block before kb, whose slot takes the block two ahead. */
+                if (kb + 1u < KB || more) LOADER_BARRIER(T5_NLOAD); else LOADER_BARRIER(0);
+                const uint32_t st2 = st >= 1u ? st - 1u : 2u; /* (st + 2) % 3 */
+                if (kb + 2u < KB) issue(cur, kb + 2u, st2);
+                else if (more) issue(nxt, kb + 2u - KB, st2);
+                st = st == 2u ? 0u : st + 1u;
+                if (more && kb == 0u) fetch(tnxt, pre);
+                if (more && kb == kb_finish) finish(tnxt, pre, par ^ 1u, nxt);
+            }
+            WG_BARRIER(); /* after the last block (the consumers' amax exchange) */
+            slot = st;
+            cur = nxt, tcur = tnxt, tile = ntile, par ^= 1u;
+        }
+    } else {
+        /* ================= consumers ================= */
+        Tile t;
+        uint32_t par = 0, st = 0;
+        for (uint32_t tile = next_tile(wg, t); tile < total; tile = next_tile(tile + G, t), par ^= 1u) {
+            PROF_STAMP(ts0);
+            const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
+            const uint32_t ngrp = (rows + 15u) / 16u; /* live 16-row groups */
             const uint32_t ch0 = GLU ? nt * 128u + 16u * cw : nt * 256u + 32u * cw; /* first channel */
             const bool wave_on = ch0 < g.N; /* DOWN: N may end mid-tile (N is a multiple of 128) */
             const uint32_t ngrp_w = wave_on ? ngrp : 0u;
-            bool rvalid[8];
-#pragma unroll
-            for (int rg = 0; rg < 8; rg++) {
-                const uint32_t row = 16u * (uint32_t)rg + r16;
-                rvalid[rg] = row < rows;
-                if (rvalid[rg]) rvalid[rg] = (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) != PLOW_EXPERT_UNUSED;
-            }
             v4f acc[8][2];
 #pragma unroll
             for (int rg = 0; rg < 8; rg++)
 #pragma unroll
-                for (int t = 0; t < 2; t++) acc[rg][t] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-
-            __syncthreads(); /* tile start (pairs with the loaders') */
+                for (int x = 0; x < 2; x++) acc[rg][x] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             PROF_STAMP(ts1);
 #ifdef T5_PROF
             unsigned long long ts2 = 0;
@@ -289,12 +338,12 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 #ifdef T5_PROF
                 if (kb == 0) ts2 = __builtin_readcyclecounter();
 #endif
-                const uint32_t st = kb % T5_STAGES;
                 const uint32_t ab = a_base + st * (T5_BM * 128u), wb = w_base + st * (256u * 128u) + cw * (32u * 128u);
                 const uint32_t blo = ab + op_lo, bhi = ab + op_hi;
                 const uint32_t alo = wb + op_lo, ahi = wb + op_hi;
                 const uint32_t sl = s_base + st * (T5_BM * 4u) + r16 * 4u;
-                const uint32_t cl = c_base + kb * 4u;
+                const uint32_t cl = c_base + par * 1024u + kb * 4u;
+                st = st == 2u ? 0u : st + 1u;
                 if (ngrp_w == 0u) continue;
                 float ws0 = ds_read4<0>(cl);
                 float ws1 = ds_read4<512>(cl);
@@ -311,7 +360,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                 if (!GLU) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);
                 v8i aop[2];
 #pragma unroll
-                for (int t = 0; t < 2; t++) aop[t] = __builtin_shufflevector(al[t], ah[t], 0, 1, 2, 3, 4, 5, 6, 7);
+                for (int x = 0; x < 2; x++) aop[x] = __builtin_shufflevector(al[x], ah[x], 0, 1, 2, 3, 4, 5, 6, 7);
 #define T5_GROUP(RG)                                                                                         \
     if ((RG) < ngrp_w) {                                                                                     \
         LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                               \
@@ -338,7 +387,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             PROF_STAMP(ts3);
 
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
-             *      group 0 and up in group 1; DOWN channel = ch0 + 16 * t + 4q + i ---- */
+             *      group 0 and up in group 1; DOWN channel = ch0 + 16 * x + 4q + i ---- */
             if (GLU) {
                 float v[8][4];
 #pragma unroll
@@ -351,13 +400,15 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                     }
                     m = fmaxf(m, __shfl_xor(m, 16, 64));
                     m = fmaxf(m, __shfl_xor(m, 32, 64));
+                    /* L.red of the tile before has been read by everyone: its readers have passed this
+                     * tile's block barriers since */
                     if (q == 0) L.red[cw][16u * (uint32_t)rg + r16] = m;
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
                 for (int rg = 0; rg < 8; rg++) {
                     const uint32_t row = 16u * (uint32_t)rg + r16;
-                    if (!rvalid[rg]) continue;
+                    if (row >= rows || g.row_token[r0 + row] == PLOW_EXPERT_UNUSED) continue;
                     float amax = 1e-10f;
 #pragma unroll
                     for (int x = 0; x < 8; x++) amax = fmaxf(amax, L.red[x][row]);
@@ -367,27 +418,28 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                     if (cw == 0 && q == 0) g.out_scale[(size_t)(r0 + row) * NT + nt] = s;
                 }
             } else {
-                WG_BARRIER(); /* end of the k loop (pairs with the loaders') */
-            }
-            if (!GLU && wave_on) {
+                WG_BARRIER(); /* after the last block (pairs with the loaders') */
+                if (wave_on) {
 #pragma unroll
-                for (int rg = 0; rg < 8; rg++) {
-                    const uint32_t row = 16u * (uint32_t)rg + r16;
-                    if (!rvalid[rg]) continue;
-                    const uint32_t pidx = g.row_partidx[r0 + row];
-                    const float gate = g.row_gate[r0 + row];
+                    for (int rg = 0; rg < 8; rg++) {
+                        const uint32_t row = 16u * (uint32_t)rg + r16;
+                        if (row >= rows) continue;
+                        const uint32_t pidx = g.row_partidx[r0 + row];
+                        if (pidx == PLOW_EXPERT_UNUSED) continue;
+                        const float gate = g.row_gate[r0 + row];
 #pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        const size_t ocol = (size_t)pidx * g.N + ch0 + 16u * (uint32_t)t + 4u * q;
-                        const float y0 = gate * acc[rg][t][0], y1 = gate * acc[rg][t][1];
-                        const float y2 = gate * acc[rg][t][2], y3 = gate * acc[rg][t][3];
-                        if (g.part16) {
-                            uint2 o;
-                            o.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16);
-                            o.y = (uint32_t)f2bf(y2) | ((uint32_t)f2bf(y3) << 16);
-                            *(uint2*)((bf16_t*)g.out + ocol) = o;
-                        } else {
-                            *(float4*)((float*)g.out + ocol) = make_float4(y0, y1, y2, y3);
+                        for (int x = 0; x < 2; x++) {
+                            const size_t ocol = (size_t)pidx * g.N + ch0 + 16u * (uint32_t)x + 4u * q;
+                            const float y0 = gate * acc[rg][x][0], y1 = gate * acc[rg][x][1];
+                            const float y2 = gate * acc[rg][x][2], y3 = gate * acc[rg][x][3];
+                            if (g.part16) {
+                                uint2 o;
+                                o.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16);
+                                o.y = (uint32_t)f2bf(y2) | ((uint32_t)f2bf(y3) << 16);
+                                *(uint2*)((bf16_t*)g.out + ocol) = o;
+                            } else {
+                                *(float4*)((float*)g.out + ocol) = make_float4(y0, y1, y2, y3);
+                            }
                         }
                     }
                 }
@@ -418,7 +470,8 @@ extern "C" int plow_moe_debug_prof(unsigned long long* out) {
 template <bool GLU>
 static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
     if (g.N == 0 || g.K == 0 || g.E == 0 || g.E > 1056u || g.N % 128u || g.K % 128u) return PLOW_MOE_EINVAL;
-    if (g.K > 128u * 128u) return PLOW_MOE_EINVAL; /* the tile keeps K / 128 block scales in LDS */
+    /* the tile keeps K / 128 block scales in LDS; the load ring runs two blocks ahead */
+    if (g.K > 128u * 128u || g.K < 256u) return PLOW_MOE_EINVAL;
     static bool attr_set[2] = {false, false};
     static int n_cu = 0;
     if (!attr_set[GLU]) {
