@@ -240,7 +240,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4);
             g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_W8A8_P16;
-            const int tiled = c->forced >= 0 ? c->forced : c->tiled;
+            const int tiled = (c->forced >= 0 ? c->forced : c->tiled) && g.K >= 256u && g.N >= 256u;
             return tiled ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||

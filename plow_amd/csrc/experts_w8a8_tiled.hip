@@ -292,10 +292,16 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             issue(cur, 0u, 0u);
             issue(cur, 1u, 1u);
         }
-        const uint32_t kb_finish = KB >= 3u ? KB - 3u : 0u; /* the next tile's sources are needed from block KB - 2 on */
+        /* the next tile's sources are needed when block KB - 2 of this tile has been passed: they are
+         * fetched during block 0 and finished during block KB - 3 (before the loop if K has two blocks) */
+        const bool early = KB < 3u;
         while (tile < total) {
             const uint32_t ntile = next_tile(tile + G, tnxt);
             const bool more = ntile < total;
+            if (more && early) {
+                fetch(tnxt, pre);
+                finish(tnxt, pre, par ^ 1u, nxt);
+            }
             uint32_t st = slot; /* slot of block kb */
             for (uint32_t kb = 0; kb < KB; kb++) {
                 /* loads return in order: block kb has landed once at most the next block's loads (of this
@@ -306,8 +312,8 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                 if (kb + 2u < KB) issue(cur, kb + 2u, st2);
                 else if (more) issue(nxt, kb + 2u - KB, st2);
                 st = st == 2u ? 0u : st + 1u;
-                if (more && kb == 0u) fetch(tnxt, pre);
-                if (more && kb == kb_finish) finish(tnxt, pre, par ^ 1u, nxt);
+                if (more && !early && kb == 0u) fetch(tnxt, pre);
+                if (more && !early && kb == KB - 3u) finish(tnxt, pre, par ^ 1u, nxt);
             }
             WG_BARRIER(); /* after the last block (the consumers' amax exchange) */
             slot = st;
