@@ -47,6 +47,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c2")
     ap.add_argument("--tokens", type=int, default=0)
+    ap.add_argument("--arm", default="", help="override the configuration's arm (a16 | w8a8)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib", action="store_true",
                     help="also run a plain 1 GiB device copy three times (a kernel of known traffic, "
@@ -64,9 +65,16 @@ def main():
 
     torch.cuda.set_device(0)
     cfg = layer.config(a.config, a.tokens or None)
+    if a.config == "c5":
+        # Zipf(1.2)-like expert popularity through a selection bias; the prefill pair (ops 81 / 82)
+        # from 128 tokens on, the decode ops (65 / 66 semantics, bf16 activations) below
+        cfg.bias = True
+        cfg.arm = "w8a8" if cfg.T >= 128 else "a16"
+    if a.arm:
+        cfg.arm = a.arm
     plan = layer.plan_layer(cfg)
     hot = 3.0 if a.config == "c3" else 0.0
-    dev = synth.bind(plan, "cuda", seed=0, hot_expert=hot)
+    dev = synth.bind(plan, "cuda", seed=0, hot_expert=hot, zipf=1.2 if a.config == "c5" else 0.0)
     moe = Moe(0)
     stream = torch.cuda.current_stream().cuda_stream
     insts = abi.inst_array(plan.insts)

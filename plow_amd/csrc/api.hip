@@ -31,6 +31,9 @@ struct PlowMoeCtx {
      * follows the GLU before it on this context); the segment entry points set it from their variant;
      * PLOW_MOE_W8A8_KERNEL=stream|tiled forces it. */
     int tiled;
+    /* slots per expert of the last align (op 84) on this context: ops 81 / 82 carry no row count and
+     * pick their kernel form from it (0 = unknown: streaming form) */
+    uint32_t rows_hint;
     int forced; /* -1 none, 0 stream, 1 tiled (segment entry point or environment) */
     int32_t* ws_meta;        /* [3 * WS_MAX_E + 1] */
     uint32_t* ws_row_token;  /* [WS_MAX_ROWS] */
@@ -150,6 +153,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, i[1] >= 1u && i[1] <= 1056u && i[2] >= 1u, "op 84: n_exp %u outside 1..1056 or k = 0", i[1]);
         NEED(c, (uint64_t)i[0] * i[2] < (1ull << 31), "op 84: T * k overflows");
         if (!launch) return 0;
+        c->rows_hint = (uint32_t)(((uint64_t)i[0] * i[2]) / i[1]);
         return launch_align((int32_t*)ten(in, T, 0), ten(in, T, 1), (uint32_t*)ten(in, T, 2),
                             (uint32_t*)ten(in, T, 3), (float*)ten(in, T, 4), i[0], i[1], i[2],
                             c->ws_chunk_hist, WS_MAX_CHUNKS, st);
@@ -274,7 +278,9 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 6);
         g.meta = (const int32_t*)ten(in, T, 3); g.row_token = (const uint32_t*)ten(in, T, 4);
         g.N = I; g.K = H; g.E = E; g.act = i[5]; g.per_channel = 1;
-        return launch_group_glu_w8a8(g, st);
+        /* many rows per expert (16 or more on average): tiled form, as for the block-fp8 pair */
+        c->tiled = (c->forced >= 0 ? c->forced : (c->rows_hint >= 16u ? 1 : 0)) && H >= 256u && I >= 256u;
+        return c->tiled ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
     }
     case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8: {
         const uint32_t H = i[0], I = i[1], E = i[2];
@@ -288,7 +294,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 3);
         g.row_partidx = (const uint32_t*)ten(in, T, 4); g.row_gate = (const float*)ten(in, T, 5);
         g.N = H; g.K = I; g.E = E; g.per_channel = 1;
-        return launch_group_down_w8a8(g, st);
+        const int tiled = (c->forced >= 0 ? c->forced : c->tiled) && g.K >= 256u && g.N >= 256u;
+        return tiled ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_FP8_BLK:
     case PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8:

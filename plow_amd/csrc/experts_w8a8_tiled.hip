@@ -84,7 +84,7 @@ __device__ unsigned long long t5_prof[2][256][8];
 #define PROF_STAMP(v)
 #endif
 
-template <bool GLU>
+template <bool GLU, bool PC>
 __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     T5Lds& L = *(T5Lds*)lds_raw;
@@ -168,7 +168,8 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
         const uint32_t cnt = (uint32_t)g.meta[g.E + t.e];
         t.r0 = (uint32_t)g.meta[t.e] + mt * T5_BM;
         t.rows = cnt - mt * T5_BM < T5_BM ? cnt - mt * T5_BM : T5_BM; /* live rows of the tile */
-        t.wp0 = g.wtab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
+        /* block mode: {gate, up, down} tables; per-channel mode: {gate_up fused [2N][K], down} */
+        t.wp0 = PC ? g.wtab[(size_t)t.e * 2u + (GLU ? 0u : 1u)] : g.wtab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
         return t;
     };
     /* this workgroup's next tile at or after `from` whose expert is resident (`total` if none); loaders
@@ -213,24 +214,30 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             }
             {
                 const uint32_t row = (cw & 1u) * 64u + lane; /* the row whose activation scale this lane loads */
-                P.stok = row < rows ? (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
+                /* per-channel mode has one activation scale per row, applied in the epilogue: its ring slot
+                 * carries zeros */
+                P.stok = (!PC && row < rows) ? (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
             }
             /* weight block scales of the tile: GLU gate | up of channel block nt; DOWN blocks 2nt, 2nt + 1 */
-            const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
-            const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : S0;
-            const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
-            const uint32_t i = tid - 8u * 64u; /* 0..255 over the four loaders; KB <= 128 */
-            P.w0 = i < KB ? S0[(size_t)nb0 * KB + i] : 0.0f;
-            P.w1 = i < KB ? S1[(size_t)nb1 * KB + i] : 0.0f;
+            P.w0 = P.w1 = 0.0f;
+            if (!PC) {
+                const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
+                const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : S0;
+                const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
+                const uint32_t i = tid - 8u * 64u; /* 0..255 over the four loaders; KB <= 128 */
+                P.w0 = i < KB ? S0[(size_t)nb0 * KB + i] : 0.0f;
+                P.w1 = i < KB ? S1[(size_t)nb1 * KB + i] : 0.0f;
+            }
         };
         auto finish = [&](const Tile& t, const Pre& P, uint32_t par, Src& S) {
             const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
             S.W0 = (const uint8_t*)(uintptr_t)t.wp0;
-            S.W1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)t.e * 3u + 1u] : S.W0;
+            S.W1 = !GLU ? S.W0 : PC ? S.W0 + (size_t)g.N * K /* up rows follow the N gate rows */
+                               : (const uint8_t*)(uintptr_t)g.wtab[(size_t)t.e * 3u + 1u];
 #pragma unroll
             for (uint32_t i = 0; i < 4u; i++) {
                 const uint32_t row = 32u * cw + 8u * i + lr;
-                const uint32_t src = GLU ? (P.tok[i] < g.pitch ? P.tok[i] : 0u) : P.tok[i];
+                const uint32_t src = (GLU && P.tok[i] == PLOW_EXPERT_UNUSED) ? 0u : P.tok[i];
                 S.aoff[i] = src * K + ((p ^ ((row >> 1) & 7u)) << 4);
             }
 #pragma unroll
@@ -249,7 +256,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
              * values); a pad row reads tilep[0], which is always 0 */
             {
                 const uint32_t row = (cw & 1u) * 64u + lane;
-                const bool ok = P.stok != PLOW_EXPERT_UNUSED && (!GLU || P.stok < g.pitch);
+                const bool ok = P.stok != PLOW_EXPERT_UNUSED;
                 if (GLU) {
                     S.ssrc = ok ? g.a_scale + P.stok : (const float*)(g.meta + 2u * g.E);
                     S.sstep = ok ? g.pitch : 0u;
@@ -351,39 +358,50 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                 const uint32_t cl = c_base + par * 1024u + kb * 4u;
                 st = st == 2u ? 0u : st + 1u;
                 if (ngrp_w == 0u) continue;
-                float ws0 = ds_read4<0>(cl);
-                float ws1 = ds_read4<512>(cl);
+                float ws0 = 0.0f, ws1 = 0.0f;
+                if (!PC) {
+                    ws0 = ds_read4<0>(cl);
+                    ws1 = ds_read4<512>(cl);
+                }
                 v4i al[2], ah[2];
                 al[0] = ds_read16<0>(alo), ah[0] = ds_read16<0>(ahi);
                 al[1] = ds_read16<2048>(alo), ah[1] = ds_read16<2048>(ahi);
                 v4i bl[2], bh[2];
                 float as_[2];
                 bl[0] = ds_read16<0>(blo), bh[0] = ds_read16<0>(bhi);
-                as_[0] = ds_read4<0>(sl);
-                LDS_WAIT2(ws0, ws1);
+                as_[0] = as_[1] = 0.0f;
+                if (!PC) as_[0] = ds_read4<0>(sl);
+                if (!PC) LDS_WAIT2(ws0, ws1);
                 LDS_WAIT2(al[0], ah[0]);
                 LDS_WAIT2(al[1], ah[1]);
-                if (!GLU) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);
+                if (!GLU && !PC) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);
                 v8i aop[2];
 #pragma unroll
                 for (int x = 0; x < 2; x++) aop[x] = __builtin_shufflevector(al[x], ah[x], 0, 1, 2, 3, 4, 5, 6, 7);
+/* per-channel mode: the scales are outside the K reduction, so the matrix unit accumulates straight
+ * through; block mode: one scaled add per 128-k block */
 #define T5_GROUP(RG)                                                                                         \
     if ((RG) < ngrp_w) {                                                                                     \
         LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                               \
-        LDS_WAIT_F(as_[(RG) & 1]);                                                                           \
+        if (!PC) LDS_WAIT_F(as_[(RG) & 1]);                                                                  \
         if ((RG) + 1 < 8 && (RG) + 1 < ngrp_w) {                                                             \
             bl[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(blo);                                   \
             bh[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(bhi);                                   \
-            as_[((RG) + 1) & 1] = ds_read4<(((RG) + 1) & 7) * 64u>(sl);                                      \
+            if (!PC) as_[((RG) + 1) & 1] = ds_read4<(((RG) + 1) & 7) * 64u>(sl);                             \
         }                                                                                                    \
         const v8i b = __builtin_shufflevector(bl[(RG) & 1], bh[(RG) & 1], 0, 1, 2, 3, 4, 5, 6, 7);           \
-        const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};                                                              \
-        const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, z, 0, 0, 0, 0, 0, 0);     \
-        const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, z, 0, 0, 0, 0, 0, 0);     \
-        const float sc0 = as_[(RG) & 1] * ws0, sc1 = as_[(RG) & 1] * ws1;                                    \
-        _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                      \
-            acc[RG][0][i] = fmaf(t0[i], sc0, acc[RG][0][i]);                                                 \
-            acc[RG][1][i] = fmaf(t1[i], sc1, acc[RG][1][i]);                                                 \
+        if (PC) {                                                                                            \
+            acc[RG][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, acc[RG][0], 0, 0, 0, 0, 0, 0); \
+            acc[RG][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, acc[RG][1], 0, 0, 0, 0, 0, 0); \
+        } else {                                                                                             \
+            const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};                                                          \
+            const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, z, 0, 0, 0, 0, 0, 0); \
+            const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, z, 0, 0, 0, 0, 0, 0); \
+            const float sc0 = as_[(RG) & 1] * ws0, sc1 = as_[(RG) & 1] * ws1;                                \
+            _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                  \
+                acc[RG][0][i] = fmaf(t0[i], sc0, acc[RG][0][i]);                                             \
+                acc[RG][1][i] = fmaf(t1[i], sc1, acc[RG][1][i]);                                             \
+            }                                                                                                \
         }                                                                                                    \
     }
                 T5_GROUP(0) T5_GROUP(1) T5_GROUP(2) T5_GROUP(3) T5_GROUP(4) T5_GROUP(5) T5_GROUP(6) T5_GROUP(7)
@@ -394,7 +412,59 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
              *      group 0 and up in group 1; DOWN channel = ch0 + 16 * x + 4q + i ---- */
-            if (GLU) {
+            if (PC) {
+                /* per-channel arm (plow runtime/amd/op_moe.h:6655-6700): g = acc * (as * wsc[n]); GLU stores
+                 * bf16(act(g) * u) and zeroes the expert's pad rows, DOWN stores gate * acc, then
+                 * * (as * wsc[h]) */
+                WG_BARRIER(); /* after the last block (pairs with the loaders') */
+                const float* es = (const float*)(uintptr_t)g.stab[(size_t)t.e * 2u + (GLU ? 0u : 1u)];
+                const uint32_t cnt_e = (uint32_t)g.meta[g.E + t.e], erow0 = r0 - (uint32_t)g.meta[t.e];
+                const uint32_t padded = ((cnt_e + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
+                if (wave_on) {
+#pragma unroll
+                    for (int rg = 0; rg < 8; rg++) {
+                        const uint32_t row = 16u * (uint32_t)rg + r16;
+                        if (row >= rows) {
+                            if (GLU && erow0 + row < padded)
+                                *(uint2*)((bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q) = make_uint2(0u, 0u);
+                            continue;
+                        }
+                        if (GLU) {
+                            const uint32_t tok = g.row_token[r0 + row];
+                            bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
+                            if (tok == PLOW_EXPERT_UNUSED) {
+                                *(uint2*)orow = make_uint2(0u, 0u);
+                                continue;
+                            }
+                            const float as = g.a_scale[tok];
+                            float o[4];
+#pragma unroll
+                            for (int i = 0; i < 4; i++)
+                                o[i] = moe_glu(acc[rg][0][i] * (as * es[ch0 + 4u * q + i]),
+                                               acc[rg][1][i] * (as * es[g.N + ch0 + 4u * q + i]), g.act);
+                            uint2 pk;
+                            pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
+                            pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
+                            *(uint2*)orow = pk;
+                        } else {
+                            const uint32_t pidx = g.row_partidx[r0 + row];
+                            if (pidx == PLOW_EXPERT_UNUSED) continue;
+                            const float gate = g.row_gate[r0 + row], as = g.a_scale[r0 + row];
+#pragma unroll
+                            for (int x = 0; x < 2; x++) {
+                                const uint32_t col = ch0 + 16u * (uint32_t)x + 4u * q;
+                                float o[4];
+#pragma unroll
+                                for (int i = 0; i < 4; i++) {
+                                    o[i] = gate * acc[rg][x][i];
+                                    o[i] *= as * es[col + i];
+                                }
+                                *(float4*)((float*)g.out + (size_t)pidx * g.N + col) = make_float4(o[0], o[1], o[2], o[3]);
+                            }
+                        }
+                    }
+                }
+            } else if (GLU) {
                 float v[8][4];
 #pragma unroll
                 for (int rg = 0; rg < 8; rg++) {
@@ -473,18 +543,15 @@ extern "C" int plow_moe_debug_prof(unsigned long long* out) {
 #endif
 
 /* Persistent launch: one workgroup per CU; the tile count is computed on the device from meta. */
-template <bool GLU>
-static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
-    if (g.N == 0 || g.K == 0 || g.E == 0 || g.E > 1056u || g.N % 128u || g.K % 128u) return PLOW_MOE_EINVAL;
-    /* the tile keeps K / 128 block scales in LDS; the load ring runs two blocks ahead */
-    if (g.K > 128u * 128u || g.K < 256u) return PLOW_MOE_EINVAL;
-    static bool attr_set[2] = {false, false};
+template <bool GLU, bool PC>
+static int launch_tiled_t(const GroupW8A8& g, hipStream_t st) {
+    static bool attr_set = false;
     static int n_cu = 0;
-    if (!attr_set[GLU]) {
-        if (hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU, PC>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)sizeof(T5Lds)) != hipSuccess)
             return PLOW_MOE_EDEVICE;
-        attr_set[GLU] = true;
+        attr_set = true;
     }
     if (!n_cu) {
         int dev = 0;
@@ -492,8 +559,17 @@ static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return PLOW_MOE_EDEVICE;
         n_cu = prop.multiProcessorCount;
     }
-    k_group_w8a8_tiled<GLU><<<(uint32_t)n_cu, T5_THREADS, sizeof(T5Lds), st>>>(g);
+    k_group_w8a8_tiled<GLU, PC><<<(uint32_t)n_cu, T5_THREADS, sizeof(T5Lds), st>>>(g);
     return 0;
+}
+
+/* Persistent launch: one workgroup per CU; the tile count is computed on the device from meta. */
+template <bool GLU>
+static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
+    if (g.N == 0 || g.K == 0 || g.E == 0 || g.E > 1056u || g.N % 128u || g.K % 128u) return PLOW_MOE_EINVAL;
+    /* the tile keeps K / 128 block scales in LDS; the load ring runs two blocks ahead */
+    if (g.K > 128u * 128u || g.K < 256u) return PLOW_MOE_EINVAL;
+    return g.per_channel ? launch_tiled_t<GLU, true>(g, st) : launch_tiled_t<GLU, false>(g, st);
 }
 
 int launch_group_glu_w8a8_tiled(const GroupW8A8& g, hipStream_t st) { return launch_tiled<true>(g, st); }

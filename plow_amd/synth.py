@@ -137,8 +137,17 @@ def skewed_bias(E: int, hot: float, device, seed: int) -> torch.Tensor:
     return b
 
 
+def zipf_bias(E: int, s: float, device, seed: int, alpha: float = 0.01) -> torch.Tensor:
+    """Selection bias alpha * ln(rank ** -s) over a seeded permutation of the experts: expert
+    popularity falls off Zipf-like with exponent ``s`` while gates stay the unbiased scores."""
+    perm = torch.randperm(E, generator=_gen("cpu", seed)).to(device)
+    rank = torch.empty(E, device=device)
+    rank[perm] = torch.arange(1, E + 1, device=device, dtype=torch.float32)
+    return (-s * alpha) * torch.log(rank)
+
+
 def bind(plan: LayerPlan, device, seed: int = 0, x_std: float = 1.0, w_std: float = 0.02,
-         hot_expert: float = 0.0, experts_alias: int = 0) -> Bound:
+         hot_expert: float = 0.0, experts_alias: int = 0, zipf: float = 0.0) -> Bound:
     """Allocate and fill every tensor of ``plan`` on ``device``.
 
     ``experts_alias`` > 0 generates only that many distinct expert weight sets and lets the pointer
@@ -153,7 +162,8 @@ def bind(plan: LayerPlan, device, seed: int = 0, x_std: float = 1.0, w_std: floa
     b.t["x"] = randn_bf16((cfg.T, cfg.H), x_std, dev, seed * 1000 + 1)
     b.t["Wr"] = randn_bf16((cfg.E, cfg.H), w_std, dev, seed * 1000 + 2)
     if cfg.bias:
-        b.t["bias"] = (skewed_bias(cfg.E, hot_expert, dev, seed * 1000 + 3) if hot_expert
+        b.t["bias"] = (zipf_bias(cfg.E, zipf, dev, seed * 1000 + 3) if zipf
+                       else skewed_bias(cfg.E, hot_expert, dev, seed * 1000 + 3) if hot_expert
                        else torch.randn(cfg.E, generator=_gen(dev, seed * 1000 + 3), device=dev) * 0.01)
     if cfg.residual:
         b.t["residual"] = randn_bf16((cfg.T, cfg.H), x_std, dev, seed * 1000 + 4)

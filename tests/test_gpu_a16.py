@@ -88,6 +88,17 @@ def test_per_channel_fp8_layer(moe, oracle, T, arm):
     check_chain(plan, dev, host)
 
 
+@pytest.mark.parametrize("T,E,k", [(300, 4, 2), (1030, 3, 1), (640, 8, 4)])
+def test_per_channel_w8a8_tiled_many_rows(moe, oracle, T, E, k):
+    """Ops 81 / 82 with 60..1030 rows per expert run the tiled (prefill) form: partial, full and
+    multiple 128-row tiles, two and three 128-k blocks."""
+    cfg = layer.MoeConfig("fp8pc-tiled", H=384, E=E, I=256, k=k, T=T, scoring="softmax", norm_topk=True,
+                          enc="fp8pc", arm="w8a8")
+    plan, dev, host = both(moe, oracle, cfg, seed=T)
+    assert np.array_equal(dev.np("xq"), host.np("xq"))
+    check_chain(plan, dev, host)
+
+
 def test_mxfp4_decode_ops_match_plow_cpu_golden(moe):
     """Ops 48 / 49 at enc 2 against vectors written by plow's flat mxfp4 kernels (ops 150 / 151),
     including a sentinel slot (GLU writes nothing, DOWN writes zeros)."""
