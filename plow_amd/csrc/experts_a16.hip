@@ -41,7 +41,7 @@ template <int ENC> struct WStep;                 /* registers one lane loads per
 template <> struct WStep<AENC_BF16> { v4i r[4]; };
 template <> struct WStep<AENC_FP8BLK> { v4i r[2]; };
 template <> struct WStep<AENC_FP8PC> { v4i r[2]; };
-template <> struct WStep<AENC_MXFP4> { v4i r[1]; uint32_t s; };
+template <> struct WStep<AENC_MXFP4> { v4i r[1]; };
 
 /* byte offset inside the 128-k step of the activation piece instruction j needs (16 bytes, 8 bf16) */
 template <int ENC>
@@ -59,7 +59,6 @@ __device__ __forceinline__ void w_issue(WStep<ENC>& d, const uint8_t* w, const u
         for (int j = 0; j < 4; j++) d.r[j] = *(const v4i*)(w + (size_t)kb * 256u + (32u * j + 8u * q) * 2u);
     } else if (ENC == AENC_MXFP4) {
         d.r[0] = *(const v4i*)(w + (size_t)kb * 64u + 16u * q);
-        ((WStep<AENC_MXFP4>&)d).s = s[kb * 4u + q];
     } else {
         d.r[0] = *(const v4i*)(w + (size_t)kb * 128u + 16u * q);
         d.r[1] = *(const v4i*)(w + (size_t)kb * 128u + 64u + 16u * q);
@@ -68,11 +67,11 @@ __device__ __forceinline__ void w_issue(WStep<ENC>& d, const uint8_t* w, const u
 
 /* 8 bf16 operand values of instruction j from a lane's step registers */
 template <int ENC>
-__device__ __forceinline__ v8bf w_operand(const WStep<ENC>& d, int j) {
+__device__ __forceinline__ v8bf w_operand(const WStep<ENC>& d, int j, uint32_t e8m0 = 0) {
     if (ENC == AENC_BF16) {
         return __builtin_bit_cast(v8bf, d.r[j]);
     } else if (ENC == AENC_MXFP4) {
-        const float sc = __uint_as_float(((const WStep<AENC_MXFP4>&)d).s << 23); /* E8M0: 2^(s-127) */
+        const float sc = __uint_as_float(e8m0 << 23); /* E8M0: 2^(s-127) */
         const uint32_t wd = (uint32_t)d.r[0][j];                                 /* 8 nibbles, low = even k */
         const v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 0);
         const v2bf p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 1);
@@ -90,7 +89,7 @@ __device__ __forceinline__ v8bf w_operand(const WStep<ENC>& d, int j) {
 }
 
 template <int ENC> struct DepthA { static constexpr int v = 2; };
-template <> struct DepthA<AENC_MXFP4> { static constexpr int v = 3; };
+template <> struct DepthA<AENC_MXFP4> { static constexpr int v = 4; }; /* = the scale group below */
 
 template <int ENC, bool GLU>
 __device__ __forceinline__ void ak_body(const GroupA16& g, uint32_t e, uint32_t ct, uint32_t r0,
@@ -128,38 +127,68 @@ __device__ __forceinline__ void ak_body(const GroupA16& g, uint32_t e, uint32_t 
     const uint8_t* ap = (const uint8_t*)g.a + (size_t)(valid ? ai : 0u) * K * 2u;
 
     WStep<ENC> wa[D], wb[D];
-    v4i xa[D][4];
+    constexpr int DX = 2; /* the rows come from L1 / L2: two steps ahead is enough, and it halves their registers */
+    v4i xa[DX][4];
     float sa[D], sbv[D];
+    /* mxfp4: the E8M0 bytes of a row are read 16 at a time (four 128-k steps x four k-chunks), one load
+     * per stream and four steps instead of one byte load per step: a load instruction costs the memory
+     * pipeline the same whatever its width. Step d of a group uses byte 4 d + q. */
+    v4i sg0[2] = {}, sg1[2] = {};
+    auto issue_scales = [&](int slot, uint32_t kb) { /* kb a multiple of 4; the row's tail reads what exists */
+        if (ENC != AENC_MXFP4) return;
+        const uint32_t nb = K / 32u; /* bytes per scale row */
+        if (kb * 4u + 16u <= nb) {
+            sg0[slot] = *(const v4i*)(ms0 + kb * 4u);
+            if (GLU) sg1[slot] = *(const v4i*)(ms1 + kb * 4u);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                sg0[slot][i] = kb * 4u + 4u * i < nb ? *(const int*)(ms0 + kb * 4u + 4u * i) : 0;
+                if (GLU) sg1[slot][i] = kb * 4u + 4u * i < nb ? *(const int*)(ms1 + kb * 4u + 4u * i) : 0;
+            }
+        }
+    };
     auto issue = [&](int d, uint32_t kb) {
         w_issue<ENC>(wa[d], w0, ms0, kb, q);
         if (GLU) w_issue<ENC>(wb[d], w1, ms1, kb, q);
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            xa[d][j] = (v4i){0, 0, 0, 0};
-            if (valid) xa[d][j] = *(const v4i*)(ap + (size_t)kb * 256u + x_off<ENC>(q, j));
-        }
         if (ENC == AENC_FP8BLK) {
             sa[d] = bs0[kb];
             if (GLU) sbv[d] = bs1[kb];
         }
     };
 
+    auto issue_x = [&](int dx, uint32_t kb) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            xa[dx][j] = (v4i){0, 0, 0, 0};
+            if (valid) xa[dx][j] = *(const v4i*)(ap + (size_t)kb * 256u + x_off<ENC>(q, j));
+        }
+    };
+
     v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+    issue_scales(0, 0u);
 #pragma unroll
     for (int d = 0; d < D; d++)
         if ((uint32_t)d < KB) issue(d, (uint32_t)d);
+#pragma unroll
+    for (int d = 0; d < DX; d++)
+        if ((uint32_t)d < KB) issue_x(d, (uint32_t)d);
+    static_assert(D % DX == 0, "the row ring must divide the weight ring");
     for (uint32_t kb0 = 0; kb0 < KB; kb0 += D) {
+        if (ENC == AENC_MXFP4 && kb0 + D < KB) issue_scales(1, kb0 + D); /* the next group's scales */
 #pragma unroll
         for (int d = 0; d < D; d++) {
             const uint32_t kb = kb0 + (uint32_t)d;
             if (kb < KB) {
+                const uint32_t e0 = ENC == AENC_MXFP4 ? ((uint32_t)sg0[0][d] >> (8u * q)) & 0xFFu : 0u;
+                const uint32_t e1 = (ENC == AENC_MXFP4 && GLU) ? ((uint32_t)sg1[0][d] >> (8u * q)) & 0xFFu : 0u;
                 v4f t0 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc0;
                 v4f t1 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc1;
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const v8bf B = __builtin_bit_cast(v8bf, xa[d][j]);
-                    t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(wa[d], j), B, t0, 0, 0, 0);
-                    if (GLU) t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(wb[d], j), B, t1, 0, 0, 0);
+                    const v8bf B = __builtin_bit_cast(v8bf, xa[d % DX][j]);
+                    t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(wa[d], j, e0), B, t0, 0, 0, 0);
+                    if (GLU) t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(wb[d], j, e1), B, t1, 0, 0, 0);
                 }
                 if (ENC == AENC_FP8BLK) {
 #pragma unroll
@@ -172,8 +201,10 @@ __device__ __forceinline__ void ak_body(const GroupA16& g, uint32_t e, uint32_t 
                     if (GLU) acc1 = t1;
                 }
                 if (kb + D < KB) issue(d, kb + D);
+                if (kb + DX < KB) issue_x(d % DX, kb + DX);
             }
         }
+        if (ENC == AENC_MXFP4) sg0[0] = sg0[1], sg1[0] = sg1[1];
     }
 
     /* ---- epilogue: lane holds channels ct*128 + wv*16 + 4q + i of row c ---- */
@@ -211,7 +242,7 @@ __device__ __forceinline__ void ak_body(const GroupA16& g, uint32_t e, uint32_t 
 }
 
 template <int ENC, bool GLU>
-__global__ __launch_bounds__(AK_THREADS) void k_group_a16_stream(GroupA16 g) {
+__global__ __launch_bounds__(AK_THREADS, GLU ? 2 : 4) void k_group_a16_stream(GroupA16 g) {
     const uint32_t tiles = g.N / AK_BN;
     const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
     const uint32_t cnt = g.meta ? (uint32_t)g.meta[g.E + e] : g.dense_rows;
