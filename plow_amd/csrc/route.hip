@@ -100,92 +100,103 @@ __global__ __launch_bounds__(256) void k_router_score_tile(float* __restrict__ o
  * order LDS only so those loads stay in flight. */
 #define RSW_KC 256
 #define RSW_PF 3
-__global__ __launch_bounds__(64) void k_router_score_wave(float* __restrict__ out,
-                                                          const bf16_t* __restrict__ x,
-                                                          const bf16_t* __restrict__ w, uint32_t M,
-                                                          uint32_t N, uint32_t K) {
+/* Two waves per workgroup: wave 1 stages (global loads RSW_PF chunks ahead, bf16 -> f32, LDS writes),
+ * wave 0 only reads operands from LDS and runs the chain of multiply-adds, which is the critical
+ * path (K dependent operations per output). One LDS-scoped barrier per chunk hands a buffer over:
+ * after barrier i chunk i is in buffer i % 2, and the stager fills the other buffer with chunk i + 1
+ * while chunk i is being consumed. */
+__global__ __launch_bounds__(128) void k_router_score_wave(float* __restrict__ out,
+                                                           const bf16_t* __restrict__ x,
+                                                           const bf16_t* __restrict__ w, uint32_t M,
+                                                           uint32_t N, uint32_t K) {
     constexpr int KC = RSW_KC, LD = KC + 4; /* +4 floats: the 8 rows start 4 banks apart */
     __shared__ __attribute__((aligned(16))) float xs[2][8][LD];
     __shared__ __attribute__((aligned(16))) float ws[2][8][LD];
-    const uint32_t lane = threadIdx.x, my = lane >> 3, nx = lane & 7u;
+    const uint32_t lane = threadIdx.x & 63u;
+    const bool stager = threadIdx.x >= 64u;
     const uint32_t m0 = blockIdx.y * 8u, n0 = blockIdx.x * 8u;
-    /* staging: a row of a chunk is KC / 8 = 32 16-byte pieces; lane l loads piece l % 32 of rows
-     * l / 32, l / 32 + 2, ... (4 rows of each operand) */
-    const uint32_t pc = lane & 31u, rsel = lane >> 5;
-    uint4 xr[RSW_PF][4], wr[RSW_PF][4];
-    auto fetch = [&](int s, uint32_t k0) {
-        const uint32_t k = k0 + pc * 8u;
+    const uint32_t NC = (K + KC - 1u) / KC;
+    if (stager) {
+        /* a row of a chunk is KC / 8 = 32 16-byte pieces; lane l loads piece l % 32 of rows
+         * l / 32, l / 32 + 2, ... (4 rows of each operand) */
+        const uint32_t pc = lane & 31u, rsel = lane >> 5;
+        uint4 xr[RSW_PF][4], wr[RSW_PF][4];
+        auto fetch = [&](int s, uint32_t k0) {
+            const uint32_t k = k0 + pc * 8u;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t r = rsel + 2u * i;
-            xr[s][i] = make_uint4(0, 0, 0, 0);
-            wr[s][i] = make_uint4(0, 0, 0, 0);
-            if (m0 + r < M && k < K) xr[s][i] = *(const uint4*)(x + (size_t)(m0 + r) * K + k);
-            if (n0 + r < N && k < K) wr[s][i] = *(const uint4*)(w + (size_t)(n0 + r) * K + k);
-        }
-    };
-    auto put = [&](float* d, uint4 a) {
-        *(float4*)d = make_float4(__uint_as_float(a.x << 16), __uint_as_float(a.x & 0xFFFF0000u),
-                                  __uint_as_float(a.y << 16), __uint_as_float(a.y & 0xFFFF0000u));
-        *(float4*)(d + 4) = make_float4(__uint_as_float(a.z << 16), __uint_as_float(a.z & 0xFFFF0000u),
-                                        __uint_as_float(a.w << 16), __uint_as_float(a.w & 0xFFFF0000u));
-    };
-    auto commit = [&](int s, uint32_t buf) {
+            for (int i = 0; i < 4; i++) {
+                const uint32_t r = rsel + 2u * i;
+                xr[s][i] = make_uint4(0, 0, 0, 0);
+                wr[s][i] = make_uint4(0, 0, 0, 0);
+                if (m0 + r < M && k < K) xr[s][i] = *(const uint4*)(x + (size_t)(m0 + r) * K + k);
+                if (n0 + r < N && k < K) wr[s][i] = *(const uint4*)(w + (size_t)(n0 + r) * K + k);
+            }
+        };
+        auto put = [&](float* d, uint4 a) {
+            *(float4*)d = make_float4(__uint_as_float(a.x << 16), __uint_as_float(a.x & 0xFFFF0000u),
+                                      __uint_as_float(a.y << 16), __uint_as_float(a.y & 0xFFFF0000u));
+            *(float4*)(d + 4) = make_float4(__uint_as_float(a.z << 16), __uint_as_float(a.z & 0xFFFF0000u),
+                                            __uint_as_float(a.w << 16), __uint_as_float(a.w & 0xFFFF0000u));
+        };
+        auto commit = [&](int s, uint32_t buf) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t r = rsel + 2u * i;
-            put(&xs[buf][r][pc * 8u], xr[s][i]);
-            put(&ws[buf][r][pc * 8u], wr[s][i]);
-        }
-    };
-    float acc = 0.0f;
+            for (int i = 0; i < 4; i++) {
+                const uint32_t r = rsel + 2u * i;
+                put(&xs[buf][r][pc * 8u], xr[s][i]);
+                put(&ws[buf][r][pc * 8u], wr[s][i]);
+            }
+        };
 #pragma unroll
-    for (int s = 0; s < RSW_PF; s++) fetch(s, (uint32_t)s * KC);
-    commit(0, 0);
-    lds_barrier();
-    uint32_t buf = 0;
-    for (uint32_t kbase = 0; kbase < K; kbase += RSW_PF * KC) {
+        for (int s = 0; s < RSW_PF; s++) fetch(s, (uint32_t)s * KC);
+        commit(0, 0);
+        for (uint32_t c0 = 0; c0 < NC; c0 += RSW_PF) {
 #pragma unroll
-        for (int s = 0; s < RSW_PF; s++) {
-            const uint32_t k0 = kbase + (uint32_t)s * KC;
-            if (k0 < K) {
-                const uint32_t kn = K - k0 < (uint32_t)KC ? K - k0 : (uint32_t)KC;
-                const float* xp = xs[buf][my];
-                const float* wp = ws[buf][nx];
-                uint32_t kk = 0;
-                if (kn == (uint32_t)KC) {
-                    /* full chunk: operand reads run one 16-k group ahead of the multiply-adds */
-                    float4 a[2][4], b[2][4];
-#pragma unroll
-                    for (int u = 0; u < 4; u++) { a[0][u] = *(const float4*)(xp + 4 * u); b[0][u] = *(const float4*)(wp + 4 * u); }
-#pragma unroll
-                    for (int gq = 0; gq < KC / 16; gq++) {
-                        const int cur = gq & 1, nxt = cur ^ 1;
-                        if (gq + 1 < KC / 16) {
-#pragma unroll
-                            for (int u = 0; u < 4; u++) {
-                                a[nxt][u] = *(const float4*)(xp + 16 * (gq + 1) + 4 * u);
-                                b[nxt][u] = *(const float4*)(wp + 16 * (gq + 1) + 4 * u);
-                            }
-                        }
-#pragma unroll
-                        for (int u = 0; u < 4; u++) {
-                            acc = fmaf(a[cur][u].x, b[cur][u].x, acc);
-                            acc = fmaf(a[cur][u].y, b[cur][u].y, acc);
-                            acc = fmaf(a[cur][u].z, b[cur][u].z, acc);
-                            acc = fmaf(a[cur][u].w, b[cur][u].w, acc);
-                        }
-                    }
-                    kk = KC;
+            for (int s = 0; s < RSW_PF; s++) {
+                const uint32_t c = c0 + (uint32_t)s;
+                if (c < NC) {
+                    lds_barrier(); /* chunk c is published; the consumer is done with chunk c - 1 */
+                    fetch(s, (c + RSW_PF) * KC); /* register stage s held chunk c, already in LDS */
+                    if (c + 1u < NC) commit((s + 1) % RSW_PF, (c + 1u) & 1u);
                 }
-                for (; kk < kn; kk++) acc = fmaf(xp[kk], wp[kk], acc);
-                /* publish the next chunk (fetched RSW_PF - 1 chunks ago), refill this stage */
-                if (k0 + KC < K) commit((s + 1) % RSW_PF, buf ^ 1u);
-                fetch(s, k0 + RSW_PF * KC);
-                lds_barrier();
-                buf ^= 1u;
             }
         }
+        return;
+    }
+    const uint32_t my = lane >> 3, nx = lane & 7u;
+    float acc = 0.0f;
+    for (uint32_t c = 0; c < NC; c++) {
+        lds_barrier(); /* chunk c is in buffer c & 1 */
+        const uint32_t k0 = c * KC, buf = c & 1u;
+        const uint32_t kn = K - k0 < (uint32_t)KC ? K - k0 : (uint32_t)KC;
+        const float* xp = xs[buf][my];
+        const float* wp = ws[buf][nx];
+        uint32_t kk = 0;
+        if (kn == (uint32_t)KC) {
+            /* full chunk: operand reads run one 16-k group ahead of the multiply-adds */
+            float4 a[2][4], b[2][4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) { a[0][u] = *(const float4*)(xp + 4 * u); b[0][u] = *(const float4*)(wp + 4 * u); }
+#pragma unroll
+            for (int gq = 0; gq < KC / 16; gq++) {
+                const int cur = gq & 1, nxt = cur ^ 1;
+                if (gq + 1 < KC / 16) {
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        a[nxt][u] = *(const float4*)(xp + 16 * (gq + 1) + 4 * u);
+                        b[nxt][u] = *(const float4*)(wp + 16 * (gq + 1) + 4 * u);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    acc = fmaf(a[cur][u].x, b[cur][u].x, acc);
+                    acc = fmaf(a[cur][u].y, b[cur][u].y, acc);
+                    acc = fmaf(a[cur][u].z, b[cur][u].z, acc);
+                    acc = fmaf(a[cur][u].w, b[cur][u].w, acc);
+                }
+            }
+            kk = KC;
+        }
+        for (; kk < kn; kk++) acc = fmaf(xp[kk], wp[kk], acc);
     }
     const uint32_t m = m0 + my, n = n0 + nx;
     if (m < M && n < N) out[(size_t)m * N + n] = acc;
@@ -199,7 +210,7 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
         k_router_score_tile<<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else {
         dim3 g((N + 7) / 8, (M + 7) / 8);
-        k_router_score_wave<<<g, 64, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        k_router_score_wave<<<g, 128, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     }
     return 0;
 }
