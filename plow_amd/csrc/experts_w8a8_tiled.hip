@@ -69,6 +69,29 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
     asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
     return r;
 }
+/* The B operand (and scale) of a row group, requested only when `live` (wave-uniform): the reads
+ * execute with EXEC = 0 otherwise, which skips them in hardware. For the compiler the statement is
+ * unconditional, so a register written by these asynchronous reads never passes a control-flow merge
+ * on its way to its wait (a copy placed at a merge would run before the data has arrived). EXEC is
+ * all ones wherever this is used. */
+template <uint32_t OFF, uint32_t SOFF, bool WITH_SCALE>
+__device__ __forceinline__ void ds_read_group(uint32_t live, uint32_t alo, uint32_t ahi, uint32_t asc, v4i& lo,
+                                              v4i& hi, float& sc) {
+    if (WITH_SCALE)
+        asm volatile("s_cmp_lg_u32 %6, 0\n\ts_cselect_b64 exec, -1, 0\n\t"
+                     "ds_read_b128 %0, %3 offset:%7\n\tds_read_b128 %1, %4 offset:%7\n\tds_read_b32 %2, %5 offset:%8\n\t"
+                     "s_mov_b64 exec, -1"
+                     : "=v"(lo), "=v"(hi), "=v"(sc)
+                     : "v"(alo), "v"(ahi), "v"(asc), "s"(live), "n"(OFF), "n"(SOFF)
+                     : "memory", "scc");
+    else
+        asm volatile("s_cmp_lg_u32 %4, 0\n\ts_cselect_b64 exec, -1, 0\n\t"
+                     "ds_read_b128 %0, %2 offset:%5\n\tds_read_b128 %1, %3 offset:%5\n\t"
+                     "s_mov_b64 exec, -1"
+                     : "=v"(lo), "=v"(hi)
+                     : "v"(alo), "v"(ahi), "s"(live), "n"(OFF)
+                     : "memory", "scc");
+}
 /* all ds_reads issued so far have returned; the operands are tied so no use is hoisted above */
 #define LDS_WAIT2(a, b) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b))
 #define LDS_WAIT_F(a) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a))
@@ -379,16 +402,15 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 #pragma unroll
                 for (int x = 0; x < 2; x++) aop[x] = __builtin_shufflevector(al[x], ah[x], 0, 1, 2, 3, 4, 5, 6, 7);
 /* per-channel mode: the scales are outside the K reduction, so the matrix unit accumulates straight
- * through; block mode: one scaled add per 128-k block */
+ * through; block mode: one scaled add per 128-k block. The read of group RG + 1 is in flight while
+ * group RG multiplies. */
 #define T5_GROUP(RG)                                                                                         \
+    LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                                   \
+    if (!PC) LDS_WAIT_F(as_[(RG) & 1]);                                                                      \
+    if ((RG) + 1 < 8)                                                                                        \
+        ds_read_group<(((RG) + 1) & 7) * 2048u, (((RG) + 1) & 7) * 64u, !PC>(                                \
+            (uint32_t)__builtin_amdgcn_readfirstlane((RG) + 1u < ngrp_w ? 1 : 0), blo, bhi, sl, bl[((RG) + 1) & 1], bh[((RG) + 1) & 1], as_[((RG) + 1) & 1]); \
     if ((RG) < ngrp_w) {                                                                                     \
-        LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                               \
-        if (!PC) LDS_WAIT_F(as_[(RG) & 1]);                                                                  \
-        if ((RG) + 1 < 8 && (RG) + 1 < ngrp_w) {                                                             \
-            bl[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(blo);                                   \
-            bh[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(bhi);                                   \
-            if (!PC) as_[((RG) + 1) & 1] = ds_read4<(((RG) + 1) & 7) * 64u>(sl);                             \
-        }                                                                                                    \
         const v8i b = __builtin_shufflevector(bl[(RG) & 1], bh[(RG) & 1], 0, 1, 2, 3, 4, 5, 6, 7);           \
         if (PC) {                                                                                            \
             acc[RG][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, acc[RG][0], 0, 0, 0, 0, 0, 0); \
