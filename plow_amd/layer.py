@@ -37,6 +37,7 @@ class MoeConfig:
     shared_mode: Optional[str] = None  # "fold" (slot {E, 1.0}) | "dense" (ops 20 + 8) | None
     act: int = abi.ACT_SILU
     residual: bool = False
+    part_bf16: bool = False         # block-fp8 W8A8 only: bf16 partials (arm 3) instead of f32
 
     @property
     def tail(self) -> int:
@@ -132,7 +133,8 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
     row_token = p._t("row_token", "u32", (R,), "scratch")
     row_partidx = p._t("row_partidx", "u32", (R,), "scratch")
     row_gate = p._t("row_gate", "f32", (R,), "scratch")
-    part = p._t("part", "f32", (T * ka, H), "scratch")
+    p16 = cfg.part_bf16 and cfg.enc == "fp8blk" and cfg.arm == "w8a8"
+    part = p._t("part", "bf16" if p16 else "f32", (T * ka, H), "scratch")
     out = p._t("out", "bf16", (T, H), "out")
     residual = p._t("residual", "bf16", (T, H), "in") if cfg.residual else None
 
@@ -183,7 +185,7 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
                                     i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8]))
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
                                      t=[part, fq, wtab, stab, meta, fs, row_partidx, row_gate],
-                                     i=[H, I, Ea, enc, 0, 0, 0, abi.ARM_W8A8]))
+                                     i=[H, I, Ea, enc, 0, 0, 0, abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8]))
         else:
             arm = abi.ARM_W4A16 if enc == abi.ENC_MXFP4 else abi.ARM_A16
             fu = p._t("fu", "bf16", (R, I), "scratch")
@@ -205,5 +207,6 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
         p._emit("shared_glu", abi.inst(abi.OP_GEMM_GLU, t=[sfu, x, wsg, None, None, wsu],
                                        i=[T, Is, H, 0, 0, cfg.act]))
         p._emit("shared_down", abi.inst(abi.OP_GEMM, t=[shared, sfu, wsd], i=[T, H, Is]))
-    p._emit("combine", abi.inst(abi.OP_MOE_COMBINE_PF, t=[out, residual, shared, part], i=[H, ka, T]))
+    p._emit("combine", abi.inst(abi.OP_MOE_COMBINE_PF, t=[out, residual, shared, part],
+                                i=[H, ka, T, 0, 0, 0, 0, 1 if p16 else 0]))
     return p

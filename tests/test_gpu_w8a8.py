@@ -76,6 +76,39 @@ def test_tiled_kernel_many_rows_per_expert(moe, oracle, T, E, k):
     check_layer(plan, dev, host)
 
 
+@pytest.mark.parametrize("T", [40, 700])
+def test_bf16_partials(moe, oracle, T):
+    """Arm 3: the down op writes bf16 partials and the combine reads them (streaming and tiled form)."""
+    cfg = layer.MoeConfig("p16", H=384, E=8, I=256, k=4, T=T, scoring="sigmoid", norm_topk=True,
+                          enc="fp8blk", arm="w8a8", n_shared=1, shared_mode="fold", residual=True, part_bf16=True)
+    plan, dev, host = both(moe, oracle, cfg, seed=T)
+    assert_routing_equal(plan, dev, host)
+    assert_output_close(dev.np("part").reshape(-1), host.np("part").reshape(-1), "part (bf16)")
+    assert_output_close(dev.np("out"), host.np("out"))
+
+
+def test_tiled_skips_non_resident_expert(moe, oracle):
+    """A null weight-table row (expert not resident on this rank): the grouped ops leave its rows alone."""
+    from gpu_harness import run_device, run_oracle
+    from plow_amd import synth
+    cfg = layer.MoeConfig("tiled-null", H=384, E=4, I=256, k=2, T=300, scoring="softmax", norm_topk=True,
+                          enc="fp8blk", arm="w8a8", n_shared=1, shared_mode="fold")
+    plan = layer.plan_layer(cfg)
+    dev = synth.bind(plan, "cuda", seed=11)
+    dev.t["wtab"][1].zero_()                       # expert 1 is elsewhere
+    dev.t["part"].fill_(0.25)                      # untouched rows must keep this
+    dev.t["fq"].fill_(7)
+    host = synth.to_host(dev)
+    host.t["wtab"][1].zero_()                      # (the host table holds host pointers of its own)
+    run_device(moe, plan, dev)
+    run_oracle(oracle, plan, host)
+    assert_routing_equal(plan, dev, host)
+    pd, ph = dev.np("part"), host.np("part")
+    untouched = (ph == 0.25).all(axis=1)
+    assert untouched.any() and np.array_equal(pd[untouched], ph[untouched])
+    assert_output_close(dev.np("out"), host.np("out"))
+
+
 def test_segment_entry_points(moe, oracle):
     """plow_moe_pf / plow_moe_dec: same results as op-by-op execution, the min-rows knob, and typed
     refusal of a mis-wired segment."""
