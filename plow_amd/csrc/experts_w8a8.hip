@@ -23,6 +23,7 @@
 #include "kernels.h"
 
 #include <cstdlib>
+#include <cstring>
 
 #define SK_WAVES 8u
 #define SK_THREADS (SK_WAVES * WAVE)
@@ -287,6 +288,170 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     }
 }
 
+
+/* ---------------------------------------------------------------------------------------------------
+ * GLU, block mode, second form: every load goes global -> LDS directly (global_load_lds_dwordx4) with
+ * 8 consecutive lanes on one 128-byte line, into a ring that is PRIVATE to the wave, and the operands
+ * are read back from LDS in the matrix layout. The "lane = weight row" loads of the first form cost
+ * the vector memory pipeline four times as much per instruction, which shows at the gate|up shape
+ * (two matrices, rows 7 KB apart). No workgroup barrier in the K loop: a wave waits for its own loads
+ * (s_waitcnt vmcnt) and nobody else's. Pad rows read the pass's first row and carry a zero scale.
+ * LDS pieces are swizzled on the global side: piece p of row r holds global piece p ^ ((r >> 1) & 7). */
+#define SD_STAGES 3
+#define SD_NLOAD 7 /* per wave and 128-k block: 1 scale, 2 activation-row, 4 weight-row direct loads */
+struct SdSlot {
+    uint8_t w[32u * 128u]; /* rows 0..15 gate, 16..31 up of this wave's 16 channels */
+    uint8_t x[16u * 128u]; /* the pass's 16 activation rows */
+    float xs[64];          /* their scales (lanes 16..63 write copies) */
+};
+struct SdLds {
+    SdSlot ring[SK_WAVES][SD_STAGES];
+    float red[SK_WAVES * 16u];
+    float wsc[2][128]; /* the tile's weight block scales (gate, up), all of K: K <= 16384 */
+};
+typedef __attribute__((address_space(3))) void sd_lds_void;
+__device__ __forceinline__ uint32_t sd_lds_off(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+template <uint32_t OFF>
+__device__ __forceinline__ v4i sd_read16(uint32_t addr) {
+    v4i r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+    return r;
+}
+__device__ __forceinline__ float sd_read4(uint32_t addr) {
+    float r;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+    return r;
+}
+#define SD_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
+
+__global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t sd_raw[];
+    SdLds& L = *(SdLds*)sd_raw;
+    const uint32_t tiles = g.N / SK_BN;
+    const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
+    const uint32_t cnt = (uint32_t)g.meta[g.E + e];
+    if (cnt == 0u) return;
+    const uint64_t wp0 = g.wtab[(size_t)e * 3u], wp1 = g.wtab[(size_t)e * 3u + 1u];
+    if (wp0 == 0ull) return; /* not resident */
+    const uint32_t r0 = (uint32_t)g.meta[e];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, 32-byte chunk q */
+    const uint32_t lr = lane >> 3, p = lane & 7u; /* load layout: row lr of a group of 8, piece p */
+    const uint32_t K = g.K, KB = K / 128u, N = g.N;
+    const uint32_t chw = ct * SK_BN + wv * 16u;   /* this wave's first channel */
+    const float* s0 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u] + (size_t)ct * KB;
+    const float* s1 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u + 1u] + (size_t)ct * KB;
+
+    /* weight rows: load j covers LDS rows 8j .. 8j + 7 (j < 2 gate, else up) */
+    const uint8_t* wsrc[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4u; j++) {
+        const uint32_t R = 8u * j + lr;
+        const uint8_t* base = (const uint8_t*)(uintptr_t)(j < 2u ? wp0 : wp1);
+        wsrc[j] = base + (size_t)(chw + (R & 15u)) * K + ((p ^ ((R >> 1) & 7u)) << 4);
+    }
+    /* the weight block scales go to LDS once: an ordinary load inside the K loop would make the
+     * compiler wait for every outstanding load of the ring */
+    for (uint32_t i = threadIdx.x; i < KB; i += SK_THREADS) {
+        L.wsc[0][i] = s0[i];
+        L.wsc[1][i] = s1[i];
+    }
+    __syncthreads();
+    const uint32_t wsc_base = sd_lds_off(&L.wsc[0][0]);
+    SdSlot* const ring = L.ring[wv];
+    const uint32_t swz = (c >> 1) & 7u;
+    const uint32_t o_lo = c * 128u + (((2u * q) ^ swz) << 4), o_hi = c * 128u + (((2u * q + 1u) ^ swz) << 4);
+
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) {
+        /* activation rows of the pass: load i covers rows 8i .. 8i + 7 */
+        const uint32_t tok0 = g.row_token[r0 + rb];
+        const uint8_t* xsrc[2];
+#pragma unroll
+        for (uint32_t i = 0; i < 2u; i++) {
+            const uint32_t row = 8u * i + lr, off = rb + row;
+            uint32_t tok = off < cnt ? g.row_token[r0 + off] : PLOW_EXPERT_UNUSED;
+            if (tok == PLOW_EXPERT_UNUSED) tok = tok0;
+            xsrc[i] = (const uint8_t*)g.a + (size_t)tok * K + ((p ^ ((row >> 1) & 7u)) << 4);
+        }
+        const float* ssrc;
+        uint32_t sstep;
+        {
+            const uint32_t off = rb + c;
+            const uint32_t tok = off < cnt ? g.row_token[r0 + off] : PLOW_EXPERT_UNUSED;
+            const bool ok = tok != PLOW_EXPERT_UNUSED;
+            ssrc = ok ? g.a_scale + tok : (const float*)(g.meta + 2u * g.E); /* tilep[0] = 0 */
+            sstep = ok ? g.pitch : 0u;
+        }
+        const bool valid = rb + c < cnt && g.row_token[r0 + rb + c] != PLOW_EXPERT_UNUSED;
+        auto issue = [&](uint32_t kb) {
+            SdSlot* s = ring + kb % SD_STAGES;
+            __builtin_amdgcn_global_load_lds((const void*)(ssrc + (size_t)kb * sstep), (sd_lds_void*)&s->xs[0], 4, 0, 0);
+#pragma unroll
+            for (uint32_t i = 0; i < 2u; i++)
+                __builtin_amdgcn_global_load_lds((const void*)(xsrc[i] + (size_t)kb * 128u),
+                                                 (sd_lds_void*)&s->x[8u * i * 128u], 16, 0, 0);
+#pragma unroll
+            for (uint32_t j = 0; j < 4u; j++)
+                __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)kb * 128u),
+                                                 (sd_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
+        };
+        v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* the row maps above are loaded; the count starts at zero */
+        issue(0);
+        if (KB > 1u) issue(1);
+        for (uint32_t kb = 0; kb < KB; kb++) {
+            /* loads return in order: block kb has landed once at most block kb + 1's are outstanding */
+            if (kb + 1u < KB) SD_WAIT_VM(SD_NLOAD); else SD_WAIT_VM(0);
+            const uint32_t base = sd_lds_off(ring + kb % SD_STAGES);
+            v4i a0l = sd_read16<0>(base + o_lo), a0h = sd_read16<0>(base + o_hi);
+            v4i a1l = sd_read16<2048>(base + o_lo), a1h = sd_read16<2048>(base + o_hi);
+            v4i bl = sd_read16<4096>(base + o_lo), bh = sd_read16<4096>(base + o_hi);
+            float xs = sd_read4(base + 6144u + c * 4u);
+            float sa = sd_read4(wsc_base + kb * 4u), sb = sd_read4(wsc_base + 512u + kb * 4u);
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0l), "+v"(a0h), "+v"(a1l), "+v"(a1h));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(bl), "+v"(bh), "+v"(xs), "+v"(sa), "+v"(sb));
+            /* block kb - 1's slot is free (its reads were waited for one iteration ago): refill it */
+            if (kb + 2u < KB) issue(kb + 2u);
+            const v8i A0 = __builtin_shufflevector(a0l, a0h, 0, 1, 2, 3, 4, 5, 6, 7);
+            const v8i A1 = __builtin_shufflevector(a1l, a1h, 0, 1, 2, 3, 4, 5, 6, 7);
+            const v8i B = __builtin_shufflevector(bl, bh, 0, 1, 2, 3, 4, 5, 6, 7);
+            const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
+            const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A0, B, z, 0, 0, 0, 0, 0, 0);
+            const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, z, 0, 0, 0, 0, 0, 0);
+            const float sc0 = xs * sa, sc1 = xs * sb;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                acc0[i] = fmaf(t0[i], sc0, acc0[i]);
+                acc1[i] = fmaf(t1[i], sc1, acc1[i]);
+            }
+        }
+        /* ---- epilogue: lane holds channels chw + 4q + i (i = 0..3) of row rb + c ---- */
+        float v[4], m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[i] = moe_glu(acc0[i], acc1[i], g.act);
+            m = fmaxf(m, fabsf(v[i]));
+        }
+        m = fmaxf(m, __shfl_xor(m, 16, 64));
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        if (q == 0) L.red[wv * 16u + c] = m;
+        __syncthreads();
+        float amax = 1e-10f;
+#pragma unroll
+        for (uint32_t w = 0; w < SK_WAVES; w++) amax = fmaxf(amax, L.red[w * 16u + c]);
+        const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
+        if (valid) {
+            const uint32_t row = r0 + rb + c, col = chw + 4u * q;
+            *(uint32_t*)((uint8_t*)g.out + (size_t)row * N + col) = cvt4_e4m3(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+            if (wv == 0 && q == 0) g.out_scale[(size_t)row * (N / 128u) + ct] = s;
+        }
+        __syncthreads(); /* L.red is reused by the next pass */
+    }
+}
+
 /* k-steps of weight loads a wave keeps in flight; PLOW_MOE_SK_DEPTH (2..4) overrides for tuning */
 static int stream_depth() {
     static int d = 0;
@@ -296,6 +461,16 @@ static int stream_depth() {
         if (d < 2 || d > 4) d = SK_DEPTH;
     }
     return d;
+}
+
+/* PLOW_MOE_SK_GLU=regs selects the first form of the block-mode GLU (weights straight into registers) */
+static bool glu_dma_form() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = getenv("PLOW_MOE_SK_GLU");
+        v = (e && !strcmp(e, "regs")) ? 0 : 1;
+    }
+    return v == 1;
 }
 
 static int check_w8a8(const GroupW8A8& g) {
@@ -310,6 +485,17 @@ int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<true, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
+    if (glu_dma_form()) {
+        static bool attr_set = false;
+        if (!attr_set) {
+            if (hipFuncSetAttribute((const void*)k_group_glu_w8a8_dma, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)sizeof(SdLds)) != hipSuccess)
+                return PLOW_MOE_EDEVICE;
+            attr_set = true;
+        }
+        k_group_glu_w8a8_dma<<<grid, SK_THREADS, sizeof(SdLds), st>>>(g);
+        return 0;
+    }
     switch (stream_depth()) {
     case 2: k_group_w8a8_stream<true, 2, false><<<grid, SK_THREADS, 0, st>>>(g); break;
     case 4: k_group_w8a8_stream<true, 4, false><<<grid, SK_THREADS, 0, st>>>(g); break;
