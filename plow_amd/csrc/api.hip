@@ -79,14 +79,14 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
         if (!strcmp(k, "tiled")) c->forced = 1;
     }
     int prev = 0;
-    hipGetDevice(&prev);
-    hipSetDevice(device);
+    (void)hipGetDevice(&prev);
+    (void)hipSetDevice(device);
     const bool ok = hipMalloc(&c->ws_meta, (3u * WS_MAX_E + 1u) * 4u) == hipSuccess &&
                     hipMalloc(&c->ws_row_token, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
                     hipMalloc(&c->ws_row_partidx, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
                     hipMalloc(&c->ws_row_gate, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
                     hipMalloc(&c->ws_chunk_hist, (size_t)WS_MAX_CHUNKS * WS_MAX_E * 4u) == hipSuccess;
-    hipSetDevice(prev);
+    (void)hipSetDevice(prev);
     if (!ok) {
         plow_moe_destroy(c);
         return PLOW_MOE_ENOMEM;
@@ -97,11 +97,11 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
 
 extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) {
     if (!ctx) return;
-    hipFree(ctx->ws_meta);
-    hipFree(ctx->ws_row_token);
-    hipFree(ctx->ws_row_partidx);
-    hipFree(ctx->ws_row_gate);
-    hipFree(ctx->ws_chunk_hist);
+    (void)hipFree(ctx->ws_meta);
+    (void)hipFree(ctx->ws_row_token);
+    (void)hipFree(ctx->ws_row_partidx);
+    (void)hipFree(ctx->ws_row_gate);
+    (void)hipFree(ctx->ws_chunk_hist);
     delete ctx;
 }
 

@@ -297,7 +297,9 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
  * (two matrices, rows 7 KB apart). No workgroup barrier in the K loop: a wave waits for its own loads
  * (s_waitcnt vmcnt) and nobody else's. Pad rows read the pass's first row and carry a zero scale.
  * LDS pieces are swizzled on the global side: piece p of row r holds global piece p ^ ((r >> 1) & 7). */
+#ifndef SD_STAGES
 #define SD_STAGES 3
+#endif
 #define SD_NLOAD 7 /* per wave and 128-k block: 1 scale, 2 activation-row, 4 weight-row direct loads */
 struct SdSlot {
     uint8_t w[32u * 128u]; /* rows 0..15 gate, 16..31 up of this wave's 16 channels */
