@@ -23,8 +23,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X datasheet
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled
 # by what the same counter reads for a 1 GiB copy): profiles/c2_decode_b64_pmc_fetch_write.txt.
 # Keyed by (config, tokens, kernel); anything not measured reports null.
-MEASURED_TRAFFIC = {("c2", 64, "glu"): 6532970260, ("c2", 64, "down"): 3263894003,
-                    ("c3", 4096, "glu"): 12212020838, ("c3", 4096, "down"): 6973987635}
+MEASURED_TRAFFIC = {("c2", 64, "glu"): 6511993344, ("c2", 64, "down"): 3263917773,
+                    ("c3", 4096, "glu"): 12239974707, ("c3", 4096, "down"): 6986212864}
 FP8_PEAK_TFLOPS = 5000.0       # dense fp8 MFMA
 
 
