@@ -64,7 +64,9 @@ typedef struct {
 enum {
     PLOW_DOP_GEMM                          = 8,   /* dense bf16 GEMM (shared-expert down)        */
     PLOW_DOP_GEMM_GLU                      = 20,  /* dense bf16 gate|up + GLU (shared expert)    */
-    PLOW_DOP_QUANT_FP8                     = 32,  /* per-row e4m3 activation quant               */
+    PLOW_DOP_QUANT_FP8                     = 32,  /* per-row e4m3 activation quant; any K; with
+                                                   * t3 gate / t4 up bound the row is produced
+                                                   * first, x = bf16(act_i2(gate) * up)          */
     PLOW_DOP_MOE_COMBINE                   = 43,
     PLOW_DOP_MOE_GROUP_GLU_FP8_BLK         = 48,  /* decode, table-driven, i6 = enc              */
     PLOW_DOP_MOE_GROUP_DOWN_FP8_BLK        = 49,

@@ -262,23 +262,28 @@ static void op_quant_block128(const PlowDevInst* in, uint32_t slice, uint32_t nb
         }
 }
 
-/* t0=xq t1=x t2=a_scale(f32 [M]) i0=M i1=K (the fused gate/up arm of the reference is not on this
- * path: t3/t4 bound => poison the scales). */
+/* t0=xq t1=x t2=a_scale(f32 [M]) i0=M i1=K; with t3=gate t4=up bound the row is first produced,
+ * x = bf16(act(gate) * up) with act = i2 (0 gelu_tanh, 1 silu, else poison), stored, then quantized
+ * (plow runtime/cpu/dev/golden/fp8.c:9-30). */
 static void op_quant_row(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
     uint8_t* xq = TEN(in, T, 0);
-    const orc_bf16* x = TEN(in, T, 1);
+    orc_bf16* x = TEN(in, T, 1);
     float* scale = TEN(in, T, 2);
+    const orc_bf16* gate = TEN(in, T, 3);
+    const orc_bf16* up = TEN(in, T, 4);
     const uint32_t M = in->i[0], K = in->i[1];
     uint32_t lo, hi;
     own_range(M, slice, nblk, &lo, &hi);
     for (uint32_t m = lo; m < hi; m++) {
-        if (TEN(in, T, 3) || TEN(in, T, 4)) { scale[m] = NAN; continue; }
+        orc_bf16* xr = x + (size_t)m * K;
         float amax = 0.0f;
-        for (uint32_t k = 0; k < K; k++) amax = fmaxf(amax, fabsf(orc_bf2f(x[(size_t)m * K + k])));
+        for (uint32_t k = 0; k < K; k++) {
+            if (gate) xr[k] = orc_f2bf(glu(orc_bf2f(gate[(size_t)m * K + k]), orc_bf2f(up[(size_t)m * K + k]), in->i[2]));
+            amax = fmaxf(amax, fabsf(orc_bf2f(xr[k])));
+        }
         scale[m] = fmaxf(amax * (1.0f / 448.0f), 1e-12f);
         const float inv = 1.0f / scale[m];
-        for (uint32_t k = 0; k < K; k++)
-            xq[(size_t)m * K + k] = orc_f32_to_e4m3(orc_bf2f(x[(size_t)m * K + k]) * inv);
+        for (uint32_t k = 0; k < K; k++) xq[(size_t)m * K + k] = orc_f32_to_e4m3(orc_bf2f(xr[k]) * inv);
     }
 }
 

@@ -182,10 +182,11 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
     }
     case PLOW_DOP_QUANT_FP8: {
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2), "op 32: t0 xq, t1 x, t2 scale must be bound");
-        NEED(c, !ten(in, T, 3) && !ten(in, T, 4), "op 32: the fused gate/up arm (t3/t4) is not on this path");
-        NEED(c, i[0] && i[1] && i[1] % 8u == 0u, "op 32: K %u must be a non-zero multiple of 8", i[1]);
+        NEED(c, !ten(in, T, 3) == !ten(in, T, 4), "op 32: gate (t3) and up (t4) must be bound together");
+        NEED(c, i[0] && i[1], "op 32: M %u and K %u must be non-zero", i[0], i[1]);
         if (!launch) return 0;
-        return launch_quant_row(ten(in, T, 0), ten(in, T, 1), (float*)ten(in, T, 2), i[0], i[1], st);
+        return launch_quant_row(ten(in, T, 0), ten(in, T, 1), (float*)ten(in, T, 2), ten(in, T, 3), ten(in, T, 4),
+                                i[2], i[0], i[1], st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_PF: {
         const uint32_t I = i[0], H = i[1], E = i[2], enc = i[3], arm = i[7];

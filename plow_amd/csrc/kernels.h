@@ -20,7 +20,8 @@ int launch_combine(void* out, const void* residual, const void* shared, const vo
 
 int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uint32_t K, uint32_t pitch,
                           hipStream_t st);
-int launch_quant_row(void* xq, const void* x, float* scale, uint32_t M, uint32_t K, hipStream_t st);
+int launch_quant_row(void* xq, void* x, float* scale, const void* gate, const void* up, uint32_t act,
+                     uint32_t M, uint32_t K, hipStream_t st);
 
 /* Grouped experts over aligned rows, block-fp8 weights x 1x128-scaled e4m3 activations. */
 struct GroupW8A8 {

@@ -3,6 +3,7 @@
  * the reference (plow runtime/amd/op_gemm_common.h:2582-2621, runtime/cpu/dev/golden/fp8.c:9-30). */
 #include "common.h"
 #include "kernels.h"
+#include "pm_expf.h"
 
 /* 16 lanes per (row, 128-group), 8 bf16 each. scale[g][row] with row pitch `pitch`. */
 __global__ __launch_bounds__(256) void k_quant_block128(uint8_t* __restrict__ xq,
@@ -47,19 +48,75 @@ int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uin
     return 0;
 }
 
-/* One workgroup per row: amax over K, scale = max(amax / 448, 1e-12), q = e4m3(x * (1 / scale)). */
-__global__ __launch_bounds__(256) void k_quant_row(uint8_t* __restrict__ xq, const bf16_t* __restrict__ x,
-                                                   float* __restrict__ scale, uint32_t K) {
+/* e4m3 byte of plow's plow_f32_to_e4m3 (runtime/cpu/dev/fp8_common.h:16-33) for EVERY product
+ * prod = x * inv: NaN keeps its sign (0x7f / 0xff), anything at or above 448 in magnitude saturates to
+ * the signed 0x7e; in range the hardware conversion rounds as the reference does. A NaN that the
+ * multiply itself made (an infinite x times the zero reciprocal of an infinite scale) is the negative
+ * default NaN on the reference's x86 host and the positive one here: it takes the reference's byte. */
+__device__ __forceinline__ uint32_t e4m3_any(float prod, float x) {
+    if (prod != prod && x == x) return 0xFFu;
+    const uint32_t u = __float_as_uint(prod), sign = (u >> 24) & 0x80u, mag = u & 0x7FFFFFFFu;
+    if (mag > 0x7F800000u) return sign | 0x7Fu;
+    if (mag >= 0x43E00000u) return sign | 0x7Eu;
+    return cvt2_e4m3(prod, 0.0f) & 0xFFu;
+}
+__device__ __forceinline__ bool e4m3_in_range(float v) { return (__float_as_uint(v) & 0x7FFFFFFFu) < 0x43E00000u; }
+
+/* activation of the gate alone (plow runtime/cpu/dev/golden/golden.h:103-115): 0 gelu_tanh, 1 silu with
+ * the bit-reproducible exponential, anything else poisons */
+__device__ __forceinline__ float act_gate_only(float g, uint32_t act) {
+    if (act == PLOW_MOE_ACT_SILU) return g / (1.0f + pm_expf(-g));
+    if (act == PLOW_MOE_ACT_GELU_TANH) {
+        const float c = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+        return 0.5f * g * (1.0f + tanhf(c));
+    }
+    return __builtin_nanf("");
+}
+
+/* One workgroup per row (plow runtime/cpu/dev/golden/fp8.c:9-30). With gate / up bound the row is first
+ * produced: x = bf16(act(gate) * up), stored, then quantized. amax over K skips NaN (fmaxf) and takes
+ * infinities; scale = max(amax / 448, 1e-12), q = e4m3(x * (1 / scale)). VEC: K is a multiple of 8 and
+ * every row is 16-byte aligned; otherwise elements are visited one at a time. Each thread quantizes
+ * exactly the elements it produced, so no fence is needed between the two passes. */
+template <bool VEC>
+__global__ __launch_bounds__(256) void k_quant_row(uint8_t* __restrict__ xq, bf16_t* __restrict__ x,
+                                                   float* __restrict__ scale, const bf16_t* __restrict__ gate,
+                                                   const bf16_t* __restrict__ up, uint32_t act, uint32_t K) {
     __shared__ float red[4];
     const uint32_t row = blockIdx.x, tid = threadIdx.x;
-    const bf16_t* xr = x + (size_t)row * K;
+    bf16_t* xr = x + (size_t)row * K;
     float amax = 0.0f;
-    for (uint32_t k = tid * 8u; k < K; k += 2048u) {
-        const uint4 raw = *(const uint4*)(xr + k);
-        const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+    if (VEC) {
+        for (uint32_t k = tid * 8u; k < K; k += 2048u) {
+            uint4 raw;
+            if (gate) {
+                const uint4 g4 = *(const uint4*)(gate + (size_t)row * K + k);
+                const uint4 u4 = *(const uint4*)(up + (size_t)row * K + k);
+                const uint32_t gv[4] = {g4.x, g4.y, g4.z, g4.w}, uv[4] = {u4.x, u4.y, u4.z, u4.w};
+                uint32_t o[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-            amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(v[j] << 16)), fabsf(__uint_as_float(v[j] & 0xFFFF0000u))));
+                for (int j = 0; j < 4; j++) {
+                    const float lo = act_gate_only(__uint_as_float(gv[j] << 16), act) * __uint_as_float(uv[j] << 16);
+                    const float hi = act_gate_only(__uint_as_float(gv[j] & 0xFFFF0000u), act) *
+                                     __uint_as_float(uv[j] & 0xFFFF0000u);
+                    o[j] = (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+                }
+                raw = make_uint4(o[0], o[1], o[2], o[3]);
+                *(uint4*)(xr + k) = raw;
+            } else {
+                raw = *(const uint4*)(xr + k);
+            }
+            const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(v[j] << 16)), fabsf(__uint_as_float(v[j] & 0xFFFF0000u))));
+        }
+    } else {
+        for (uint32_t k = tid; k < K; k += 256u) {
+            if (gate)
+                xr[k] = f2bf(act_gate_only(bf2f(gate[(size_t)row * K + k]), act) * bf2f(up[(size_t)row * K + k]));
+            amax = fmaxf(amax, fabsf(bf2f(xr[k])));
+        }
     }
     amax = wave_max(amax);
     if ((tid & 63u) == 0) red[tid >> 6] = amax;
@@ -68,24 +125,48 @@ __global__ __launch_bounds__(256) void k_quant_row(uint8_t* __restrict__ xq, con
     const float s = fmaxf(amax * (1.0f / 448.0f), 1e-12f);
     const float inv = 1.0f / s;
     if (tid == 0) scale[row] = s;
-    for (uint32_t k = tid * 8u; k < K; k += 2048u) {
-        const uint4 raw = *(const uint4*)(xr + k);
-        const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
-        float f[8];
+    if (VEC) {
+        for (uint32_t k = tid * 8u; k < K; k += 2048u) {
+            const uint4 raw = *(const uint4*)(xr + k);
+            const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+            float xf[8], f[8];
+            bool plain = true;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            f[2 * j] = __uint_as_float(v[j] << 16);
-            f[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+            for (int j = 0; j < 4; j++) {
+                xf[2 * j] = __uint_as_float(v[j] << 16);
+                xf[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                f[j] = xf[j] * inv;
+                plain = plain && e4m3_in_range(f[j]);
+            }
+            uint2 q;
+            if (plain) {
+                q.x = cvt4_e4m3(f[0], f[1], f[2], f[3]);
+                q.y = cvt4_e4m3(f[4], f[5], f[6], f[7]);
+            } else { /* NaN or infinities among the eight: every byte by the total rule */
+                q.x = q.y = 0u;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    q.x |= e4m3_any(f[j], xf[j]) << (8 * j);
+                    q.y |= e4m3_any(f[4 + j], xf[4 + j]) << (8 * j);
+                }
+            }
+            *(uint2*)(xq + (size_t)row * K + k) = q;
         }
-        uint2 q;
-        q.x = cvt4_e4m3(f[0] * inv, f[1] * inv, f[2] * inv, f[3] * inv);
-        q.y = cvt4_e4m3(f[4] * inv, f[5] * inv, f[6] * inv, f[7] * inv);
-        *(uint2*)(xq + (size_t)row * K + k) = q;
+    } else {
+        for (uint32_t k = tid; k < K; k += 256u) xq[(size_t)row * K + k] = (uint8_t)e4m3_any(bf2f(xr[k]) * inv, bf2f(xr[k]));
     }
 }
 
-int launch_quant_row(void* xq, const void* x, float* scale, uint32_t M, uint32_t K, hipStream_t st) {
-    if (K % 8u || M == 0) return PLOW_MOE_EINVAL;
-    k_quant_row<<<M, 256, 0, st>>>((uint8_t*)xq, (const bf16_t*)x, scale, K);
+int launch_quant_row(void* xq, void* x, float* scale, const void* gate, const void* up, uint32_t act,
+                     uint32_t M, uint32_t K, hipStream_t st) {
+    if (K == 0 || M == 0 || (gate == nullptr) != (up == nullptr)) return PLOW_MOE_EINVAL;
+    const uintptr_t al = (uintptr_t)x | (uintptr_t)gate | (uintptr_t)up;
+    if (K % 8u == 0u && al % 16u == 0u && (uintptr_t)xq % 8u == 0u)
+        k_quant_row<true><<<M, 256, 0, st>>>((uint8_t*)xq, (bf16_t*)x, scale, (const bf16_t*)gate, (const bf16_t*)up, act, K);
+    else
+        k_quant_row<false><<<M, 256, 0, st>>>((uint8_t*)xq, (bf16_t*)x, scale, (const bf16_t*)gate, (const bf16_t*)up, act, K);
     return 0;
 }

@@ -145,6 +145,33 @@ def main():
     run(abi.inst(8, t=[0, 1, 2], i=[M, K, N]), [y, fu, wd], nblk=2)
     out.update({"dense/x": x, "dense/wg": wg, "dense/wu": wu, "dense/wd": wd, "dense/fu": fu, "dense/y": y})
 
+    # --- op 32 edges (drawn last so that the vectors above keep their values): widths that are not a
+    # multiple of the vector width, rows with NaN / infinities, and the fused gate/up arm ----------
+    for K in (1, 15, 17, 257):
+        M = 3
+        x = cases.randn_bf16(r, (M, K), 2.0)
+        x[1] = 0x8000 * (np.arange(K) & 1)      # signed zeros only: the 1e-12 scale floor
+        x[2, 0] = ol.f2bf(np.float32(448.0))
+        xq, sc = np.zeros((M, K), np.uint8), np.zeros(M, np.float32)
+        run(abi.inst(32, t=[0, 1, 2], i=[M, K]), [xq, x.copy(), sc], nblk=2)
+        out.update({f"quant32w/{K}/x": x, f"quant32w/{K}/xq": xq, f"quant32w/{K}/scale": sc})
+    M, K = 4, 40
+    x = cases.randn_bf16(r, (M, K), 2.0)
+    x[0, 3], x[0, 17] = 0x7FC0, 0xFFC1          # NaN of either sign among finite values
+    x[1, 5] = 0x7F80                            # +inf
+    x[2, 8], x[2, 9], x[2, 30] = 0xFF80, 0x7FC0, 0x7F80
+    xq, sc = np.zeros((M, K), np.uint8), np.zeros(M, np.float32)
+    run(abi.inst(32, t=[0, 1, 2], i=[M, K]), [xq, x.copy(), sc])
+    out.update({"quant32n/x": x, "quant32n/xq": xq, "quant32n/scale": sc})
+    for act in (0, 1):
+        for K in (17, 1024):
+            M = 5
+            gate, up = cases.randn_bf16(r, (M, K), 3.0), cases.randn_bf16(r, (M, K), 1.5)
+            x, xq, sc = np.zeros((M, K), np.uint16), np.zeros((M, K), np.uint8), np.zeros(M, np.float32)
+            run(abi.inst(32, t=[0, 1, 2, 3, 4], i=[M, K, act]), [xq, x, sc, gate, up], nblk=2)
+            out.update({f"quant32f/{act}/{K}/gate": gate, f"quant32f/{act}/{K}/up": up, f"quant32f/{act}/{K}/x": x,
+                        f"quant32f/{act}/{K}/xq": xq, f"quant32f/{act}/{K}/scale": sc})
+
     path = os.path.join(HERE, "plow_cpu_golden.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

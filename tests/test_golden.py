@@ -139,6 +139,31 @@ def test_per_row_quant(oracle):
     assert np.array_equal(sc.view(np.uint32), G["quant32/scale"].view(np.uint32))
 
 
+@pytest.mark.parametrize("key", ["quant32w/1", "quant32w/15", "quant32w/17", "quant32w/257", "quant32n"])
+def test_per_row_quant_edges(oracle, key):
+    """Widths off the vector width, signed-zero rows, and rows with NaN / infinities."""
+    x = G[key + "/x"].copy()
+    M, K = x.shape
+    xq, sc = np.zeros((M, K), np.uint8), np.zeros(M, np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8, t=[0, 1, 2], i=[M, K]), [xq, x, sc], 3)
+    assert np.array_equal(xq, G[key + "/xq"])
+    assert np.array_equal(sc.view(np.uint32), G[key + "/scale"].view(np.uint32))
+
+
+@pytest.mark.parametrize("act", [0, 1])
+@pytest.mark.parametrize("K", [17, 1024])
+def test_per_row_quant_fused_gate_up(oracle, act, K):
+    """Reference op 32 with gate / up bound: x = bf16(act(gate) * up) is produced, then quantized."""
+    key = f"quant32f/{act}/{K}"
+    gate, up = G[key + "/gate"], G[key + "/up"]
+    M = gate.shape[0]
+    x, xq, sc = np.zeros((M, K), np.uint16), np.zeros((M, K), np.uint8), np.zeros(M, np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8, t=[0, 1, 2, 3, 4], i=[M, K, act]), [xq, x, sc, gate, up], 2)
+    assert np.array_equal(x, G[key + "/x"])
+    assert np.array_equal(xq, G[key + "/xq"])
+    assert np.array_equal(sc.view(np.uint32), G[key + "/scale"].view(np.uint32))
+
+
 def test_dense_shared_expert(oracle):
     x, wg, wu, wd = G["dense/x"], G["dense/wg"], G["dense/wu"], G["dense/wd"]
     M, K = x.shape
