@@ -46,6 +46,8 @@ struct T5Lds {
     float as[T5_STAGES][T5_BM];         /* activation scales of the block */
     float wsc[2][2][128];               /* [tile parity][gate|down, up] weight block scales, all of K */
     float red[8][T5_BM];                /* GLU: per-row amax of each consumer's 16 channels */
+    uint32_t epi_idx[2][T5_BM];         /* [tile parity] GLU: row_token, DOWN: row_partidx of the tile's rows */
+    float epi_gate[2][T5_BM];           /* [tile parity] DOWN: row_gate */
     uint32_t prefix[1056];
 };
 
@@ -225,8 +227,8 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
          * flight while the loader keeps feeding the tile before: fetch() only issues loads, finish()
          * uses them a few blocks later. Rows below the live count always hold a token. */
         struct Pre {
-            uint32_t tok[4], stok;
-            float w0, w1;
+            uint32_t tok[4], stok, eidx;
+            float w0, w1, egate;
         };
         auto fetch = [&](const Tile& t, Pre& P) {
             const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
@@ -239,7 +241,9 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                 const uint32_t row = (cw & 1u) * 64u + lane; /* the row whose activation scale this lane loads */
                 /* per-channel mode has one activation scale per row, applied in the epilogue: its ring slot
                  * carries zeros */
-                P.stok = (!PC && row < rows) ? (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
+                P.eidx = row < rows ? (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
+                P.stok = PC ? PLOW_EXPERT_UNUSED : P.eidx;
+                P.egate = (!GLU && row < rows) ? g.row_gate[r0 + row] : 0.0f;
             }
             /* weight block scales of the tile: GLU gate | up of channel block nt; DOWN blocks 2nt, 2nt + 1 */
             P.w0 = P.w1 = 0.0f;
@@ -293,6 +297,12 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                 L.wsc[par][0][i] = P.w0;
                 L.wsc[par][1][i] = P.w1;
             }
+            /* what the consumers' epilogue needs per row, so that it does not start with a round trip to
+             * memory: loaders 0 and 1 hold rows 0..63 and 64..127 */
+            if (cw < 2u) {
+                L.epi_idx[par][cw * 64u + lane] = P.eidx;
+                if (!GLU) L.epi_gate[par][cw * 64u + lane] = P.egate;
+            }
         };
         auto issue = [&](const Src& S, uint32_t kb, uint32_t st) {
 #ifdef T5_NOSTREAM
@@ -323,15 +333,13 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             issue(cur, 1u, 1u);
         }
         /* the next tile's sources are needed when block KB - 2 of this tile has been passed: they are
-         * fetched during block 0 and finished during block KB - 3 (before the loop if K has two blocks) */
+         * fetched during block 0 and finished during block KB - 3 (fetched before the loop and finished
+         * right after the first barrier if K has two blocks) */
         const bool early = KB < 3u;
         while (tile < total) {
             const uint32_t ntile = next_tile(tile + G, tnxt);
             const bool more = ntile < total;
-            if (more && early) {
-                fetch(tnxt, pre);
-                finish(tnxt, pre, par ^ 1u, nxt);
-            }
+            if (more && early) fetch(tnxt, pre);
             uint32_t st = slot; /* slot of block kb */
             for (uint32_t kb = 0; kb < KB; kb++) {
                 /* loads return in order: block kb has landed once at most the next block's loads (of this
@@ -339,6 +347,9 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                  * block before kb, whose slot takes the block two ahead. */
                 if (kb + 1u < KB || more) LOADER_BARRIER(T5_NLOAD); else LOADER_BARRIER(0);
                 const uint32_t st2 = st >= 1u ? st - 1u : 2u; /* (st + 2) % 3 */
+                /* not before this barrier: until it, the consumers may still be in the epilogue of the tile
+                 * before, reading the L.epi_* half that finish() overwrites */
+                if (more && early && kb == 0u) finish(tnxt, pre, par ^ 1u, nxt);
                 if (kb + 2u < KB) issue(cur, kb + 2u, st2);
                 else if (more) issue(nxt, kb + 2u - KB, st2);
                 st = st == 2u ? 0u : st + 1u;
@@ -452,7 +463,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                             continue;
                         }
                         if (GLU) {
-                            const uint32_t tok = g.row_token[r0 + row];
+                            const uint32_t tok = L.epi_idx[par][row];
                             bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
                             if (tok == PLOW_EXPERT_UNUSED) {
                                 *(uint2*)orow = make_uint2(0u, 0u);
@@ -469,9 +480,9 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                             pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
                             *(uint2*)orow = pk;
                         } else {
-                            const uint32_t pidx = g.row_partidx[r0 + row];
+                            const uint32_t pidx = L.epi_idx[par][row];
                             if (pidx == PLOW_EXPERT_UNUSED) continue;
-                            const float gate = g.row_gate[r0 + row], as = g.a_scale[r0 + row];
+                            const float gate = L.epi_gate[par][row], as = g.a_scale[r0 + row];
 #pragma unroll
                             for (int x = 0; x < 2; x++) {
                                 const uint32_t col = ch0 + 16u * (uint32_t)x + 4u * q;
@@ -506,7 +517,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 #pragma unroll
                 for (int rg = 0; rg < 8; rg++) {
                     const uint32_t row = 16u * (uint32_t)rg + r16;
-                    if (row >= rows || g.row_token[r0 + row] == PLOW_EXPERT_UNUSED) continue;
+                    if (row >= rows || L.epi_idx[par][row] == PLOW_EXPERT_UNUSED) continue;
                     float amax = 1e-10f;
 #pragma unroll
                     for (int x = 0; x < 8; x++) amax = fmaxf(amax, L.red[x][row]);
@@ -522,9 +533,9 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                     for (int rg = 0; rg < 8; rg++) {
                         const uint32_t row = 16u * (uint32_t)rg + r16;
                         if (row >= rows) continue;
-                        const uint32_t pidx = g.row_partidx[r0 + row];
+                        const uint32_t pidx = L.epi_idx[par][row];
                         if (pidx == PLOW_EXPERT_UNUSED) continue;
-                        const float gate = g.row_gate[r0 + row];
+                        const float gate = L.epi_gate[par][row];
 #pragma unroll
                         for (int x = 0; x < 2; x++) {
                             const size_t ocol = (size_t)pidx * g.N + ch0 + 16u * (uint32_t)x + 4u * q;
