@@ -109,6 +109,115 @@ __device__ unsigned long long t5_prof[2][256][8];
 #define PROF_STAMP(v)
 #endif
 
+/* ---- one 128-k block of a consumer wave (names are those of the kernel body) -------------------- */
+#define T5_BLOCK_HEAD()                                                                                      \
+    const uint32_t ab = a_base + st * (T5_BM * 128u), wb = w_base + st * (256u * 128u) + cw * (32u * 128u);  \
+    const uint32_t blo = ab + op_lo, bhi = ab + op_hi;                                                       \
+    const uint32_t alo = wb + op_lo, ahi = wb + op_hi;                                                       \
+    const uint32_t sl = s_base + st * (T5_BM * 4u) + r16 * 4u;                                               \
+    const uint32_t cl = c_base + par * 1024u + kb * 4u;                                                      \
+    st = st == 2u ? 0u : st + 1u;
+#define T5_BLOCK_OPERANDS()                                                                                  \
+    float ws0 = 0.0f, ws1 = 0.0f;                                                                            \
+    if (!PC) {                                                                                               \
+        ws0 = ds_read4<0>(cl);                                                                               \
+        ws1 = ds_read4<512>(cl);                                                                             \
+    }                                                                                                        \
+    v4i al[2], ah[2];                                                                                        \
+    al[0] = ds_read16<0>(alo), ah[0] = ds_read16<0>(ahi);                                                    \
+    al[1] = ds_read16<2048>(alo), ah[1] = ds_read16<2048>(ahi);                                              \
+    v4i bl[2], bh[2];                                                                                        \
+    float as_[2];                                                                                            \
+    bl[0] = ds_read16<0>(blo), bh[0] = ds_read16<0>(bhi);                                                    \
+    as_[0] = as_[1] = 0.0f;                                                                                  \
+    if (!PC) as_[0] = ds_read4<0>(sl);                                                                       \
+    if (!PC) LDS_WAIT2(ws0, ws1);                                                                            \
+    LDS_WAIT2(al[0], ah[0]);                                                                                 \
+    LDS_WAIT2(al[1], ah[1]);                                                                                 \
+    if (!GLU && !PC) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);                                                    \
+    v8i aop[2];                                                                                              \
+    _Pragma("unroll") for (int x = 0; x < 2; x++) aop[x] = __builtin_shufflevector(al[x], ah[x], 0, 1, 2, 3, 4, 5, 6, 7);
+
+/* Tiles with dead row groups. Per-channel mode: the scales are outside the K reduction, so the matrix
+ * unit accumulates straight through; block mode: one scaled add per 128-k block. The read of group
+ * RG + 1 is in flight while group RG multiplies. */
+#define T5_GROUP_PARTIAL(RG)                                                                                 \
+    LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                                   \
+    if (!PC) LDS_WAIT_F(as_[(RG) & 1]);                                                                      \
+    if ((RG) + 1 < 8)                                                                                        \
+        ds_read_group<(((RG) + 1) & 7) * 2048u, (((RG) + 1) & 7) * 64u, !PC>(                                \
+            (uint32_t)__builtin_amdgcn_readfirstlane((RG) + 1u < ngrp_w ? 1 : 0), blo, bhi, sl, bl[((RG) + 1) & 1], bh[((RG) + 1) & 1], as_[((RG) + 1) & 1]); \
+    if ((RG) < ngrp_w) {                                                                                     \
+        const v8i b = __builtin_shufflevector(bl[(RG) & 1], bh[(RG) & 1], 0, 1, 2, 3, 4, 5, 6, 7);           \
+        if (PC) {                                                                                            \
+            acc[RG][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, acc[RG][0], 0, 0, 0, 0, 0, 0); \
+            acc[RG][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, acc[RG][1], 0, 0, 0, 0, 0, 0); \
+        } else {                                                                                             \
+            const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};                                                          \
+            const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, z, 0, 0, 0, 0, 0, 0); \
+            const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, z, 0, 0, 0, 0, 0, 0); \
+            const float sc0 = as_[(RG) & 1] * ws0, sc1 = as_[(RG) & 1] * ws1;                                \
+            _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                  \
+                acc[RG][0][i] = fmaf(t0[i], sc0, acc[RG][0][i]);                                             \
+                acc[RG][1][i] = fmaf(t1[i], sc1, acc[RG][1][i]);                                             \
+            }                                                                                                \
+        }                                                                                                    \
+    }
+#define T5_BLOCK_PARTIAL()                                                                                   \
+    T5_BLOCK_HEAD()                                                                                          \
+    if (ngrp_w == 0u) continue;                                                                              \
+    T5_BLOCK_OPERANDS()                                                                                      \
+    T5_GROUP_PARTIAL(0) T5_GROUP_PARTIAL(1) T5_GROUP_PARTIAL(2) T5_GROUP_PARTIAL(3)                          \
+    T5_GROUP_PARTIAL(4) T5_GROUP_PARTIAL(5) T5_GROUP_PARTIAL(6) T5_GROUP_PARTIAL(7)
+
+/* Tiles with all eight row groups live: no condition anywhere, so no value is ever copied between
+ * registers; in block mode the scaled adds of group RG follow the matrix instructions of group RG + 1,
+ * never wait for a result and overlap with the matrix unit. */
+#define T5_SCALE_FULL(RG)                                                                                    \
+    if (!PC) {                                                                                               \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                      \
+            acc[RG][0][i] = fmaf(t[(RG) & 1][0][i], sc[(RG) & 1][0], acc[RG][0][i]);                         \
+            acc[RG][1][i] = fmaf(t[(RG) & 1][1][i], sc[(RG) & 1][1], acc[RG][1][i]);                         \
+        }                                                                                                    \
+    }
+#define T5_GROUP_FULL(RG)                                                                                    \
+    LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                                   \
+    if (!PC) {                                                                                               \
+        LDS_WAIT_F(as_[(RG) & 1]);                                                                           \
+        sc[(RG) & 1][0] = as_[(RG) & 1] * ws0;                                                               \
+        sc[(RG) & 1][1] = as_[(RG) & 1] * ws1;                                                               \
+    }                                                                                                        \
+    if ((RG) + 1 < 8) {                                                                                      \
+        bl[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(blo);                                       \
+        bh[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(bhi);                                       \
+        if (!PC) as_[((RG) + 1) & 1] = ds_read4<(((RG) + 1) & 7) * 64u>(sl);                                 \
+    }                                                                                                        \
+    {                                                                                                        \
+        const v8i b = __builtin_shufflevector(bl[(RG) & 1], bh[(RG) & 1], 0, 1, 2, 3, 4, 5, 6, 7);           \
+        if (PC) {                                                                                            \
+            acc[RG][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, acc[RG][0], 0, 0, 0, 0, 0, 0); \
+            acc[RG][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, acc[RG][1], 0, 0, 0, 0, 0, 0); \
+        } else {                                                                                             \
+            const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};                                                          \
+            t[(RG) & 1][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, z, 0, 0, 0, 0, 0, 0); \
+            t[(RG) & 1][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, z, 0, 0, 0, 0, 0, 0); \
+        }                                                                                                    \
+    }
+#define T5_BLOCK_FULL()                                                                                      \
+    T5_BLOCK_HEAD()                                                                                          \
+    T5_BLOCK_OPERANDS()                                                                                      \
+    v4f t[2][2];                                                                                             \
+    float sc[2][2];                                                                                          \
+    T5_GROUP_FULL(0)                                                                                         \
+    T5_GROUP_FULL(1) T5_SCALE_FULL(0)                                                                        \
+    T5_GROUP_FULL(2) T5_SCALE_FULL(1)                                                                        \
+    T5_GROUP_FULL(3) T5_SCALE_FULL(2)                                                                        \
+    T5_GROUP_FULL(4) T5_SCALE_FULL(3)                                                                        \
+    T5_GROUP_FULL(5) T5_SCALE_FULL(4)                                                                        \
+    T5_GROUP_FULL(6) T5_SCALE_FULL(5)                                                                        \
+    T5_GROUP_FULL(7) T5_SCALE_FULL(6)                                                                        \
+    T5_SCALE_FULL(7)
+
 template <bool GLU, bool PC>
 __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
@@ -380,66 +489,27 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 #ifdef T5_PROF
             unsigned long long ts2 = 0;
 #endif
-            for (uint32_t kb = 0; kb < KB; kb++) {
-                WG_BARRIER(); /* block kb is in LDS */
+            /* Two forms of the block loop: tiles whose eight row groups are all live (the common case) run
+             * code without a condition in it, which lets the scaled adds of a group be issued after the
+             * matrix instructions of the next group; the other tiles skip their dead groups. */
+            if (ngrp_w == 8u) {
+                for (uint32_t kb = 0; kb < KB; kb++) {
+                    WG_BARRIER(); /* block kb is in LDS */
 #ifdef T5_PROF
-                if (kb == 0) ts2 = __builtin_readcyclecounter();
+                    if (kb == 0) ts2 = __builtin_readcyclecounter();
 #endif
-                const uint32_t ab = a_base + st * (T5_BM * 128u), wb = w_base + st * (256u * 128u) + cw * (32u * 128u);
-                const uint32_t blo = ab + op_lo, bhi = ab + op_hi;
-                const uint32_t alo = wb + op_lo, ahi = wb + op_hi;
-                const uint32_t sl = s_base + st * (T5_BM * 4u) + r16 * 4u;
-                const uint32_t cl = c_base + par * 1024u + kb * 4u;
-                st = st == 2u ? 0u : st + 1u;
-                if (ngrp_w == 0u) continue;
-                float ws0 = 0.0f, ws1 = 0.0f;
-                if (!PC) {
-                    ws0 = ds_read4<0>(cl);
-                    ws1 = ds_read4<512>(cl);
+                    T5_BLOCK_FULL()
+                    LDS_WAIT_ALL(); /* nothing of this block is still being read when the next barrier is passed */
                 }
-                v4i al[2], ah[2];
-                al[0] = ds_read16<0>(alo), ah[0] = ds_read16<0>(ahi);
-                al[1] = ds_read16<2048>(alo), ah[1] = ds_read16<2048>(ahi);
-                v4i bl[2], bh[2];
-                float as_[2];
-                bl[0] = ds_read16<0>(blo), bh[0] = ds_read16<0>(bhi);
-                as_[0] = as_[1] = 0.0f;
-                if (!PC) as_[0] = ds_read4<0>(sl);
-                if (!PC) LDS_WAIT2(ws0, ws1);
-                LDS_WAIT2(al[0], ah[0]);
-                LDS_WAIT2(al[1], ah[1]);
-                if (!GLU && !PC) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);
-                v8i aop[2];
-#pragma unroll
-                for (int x = 0; x < 2; x++) aop[x] = __builtin_shufflevector(al[x], ah[x], 0, 1, 2, 3, 4, 5, 6, 7);
-/* per-channel mode: the scales are outside the K reduction, so the matrix unit accumulates straight
- * through; block mode: one scaled add per 128-k block. The read of group RG + 1 is in flight while
- * group RG multiplies. */
-#define T5_GROUP(RG)                                                                                         \
-    LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                                   \
-    if (!PC) LDS_WAIT_F(as_[(RG) & 1]);                                                                      \
-    if ((RG) + 1 < 8)                                                                                        \
-        ds_read_group<(((RG) + 1) & 7) * 2048u, (((RG) + 1) & 7) * 64u, !PC>(                                \
-            (uint32_t)__builtin_amdgcn_readfirstlane((RG) + 1u < ngrp_w ? 1 : 0), blo, bhi, sl, bl[((RG) + 1) & 1], bh[((RG) + 1) & 1], as_[((RG) + 1) & 1]); \
-    if ((RG) < ngrp_w) {                                                                                     \
-        const v8i b = __builtin_shufflevector(bl[(RG) & 1], bh[(RG) & 1], 0, 1, 2, 3, 4, 5, 6, 7);           \
-        if (PC) {                                                                                            \
-            acc[RG][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, acc[RG][0], 0, 0, 0, 0, 0, 0); \
-            acc[RG][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, acc[RG][1], 0, 0, 0, 0, 0, 0); \
-        } else {                                                                                             \
-            const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};                                                          \
-            const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, z, 0, 0, 0, 0, 0, 0); \
-            const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, z, 0, 0, 0, 0, 0, 0); \
-            const float sc0 = as_[(RG) & 1] * ws0, sc1 = as_[(RG) & 1] * ws1;                                \
-            _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                  \
-                acc[RG][0][i] = fmaf(t0[i], sc0, acc[RG][0][i]);                                             \
-                acc[RG][1][i] = fmaf(t1[i], sc1, acc[RG][1][i]);                                             \
-            }                                                                                                \
-        }                                                                                                    \
-    }
-                T5_GROUP(0) T5_GROUP(1) T5_GROUP(2) T5_GROUP(3) T5_GROUP(4) T5_GROUP(5) T5_GROUP(6) T5_GROUP(7)
-#undef T5_GROUP
-                LDS_WAIT_ALL(); /* nothing of this block is still being read when the next barrier is passed */
+            } else {
+                for (uint32_t kb = 0; kb < KB; kb++) {
+                    WG_BARRIER(); /* block kb is in LDS */
+#ifdef T5_PROF
+                    if (kb == 0) ts2 = __builtin_readcyclecounter();
+#endif
+                    T5_BLOCK_PARTIAL()
+                    LDS_WAIT_ALL();
+                }
             }
             PROF_STAMP(ts3);
 
