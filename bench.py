@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X datasheet
 # by what the same counter reads for a 1 GiB copy): profiles/c2_decode_b64_pmc_fetch_write.txt.
 # Keyed by (config, tokens, kernel); anything not measured reports null.
 MEASURED_TRAFFIC = {("c2", 64, "glu"): 6511993344, ("c2", 64, "down"): 3263917773,
-                    ("c3", 4096, "glu"): 12239974707, ("c3", 4096, "down"): 6986212864}
+                    ("c3", 4096, "glu"): 11578979226, ("c3", 4096, "down"): 6576948429}
 FP8_PEAK_TFLOPS = 5000.0       # dense fp8 MFMA
 
 
