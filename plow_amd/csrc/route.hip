@@ -15,42 +15,52 @@
 /* logit[m][n] = sum_k bf(x[m][k]) * bf(w[n][k]) with ONE f32 accumulator per output walking k in
  * ascending order (plow runtime/cpu/dev/golden/f32_primitives.c:235-252). The product of two bf16
  * values is exact in f32, so fmaf(a, b, acc) rounds exactly like the reference's `acc += a * b`. */
-/* Large problems (prefill): 64 x 64 outputs per workgroup, 4 x 4 per thread (16 independent chains
- * per lane keep the FMA pipe full), operands double buffered in LDS as f32 [k][row] and read as
- * float4, one LDS-only barrier per 32-k chunk, the next chunk's global loads already in flight. */
+/* Large problems (prefill): (16 * TM) x 64 outputs per workgroup, TM x 4 per thread (independent chains
+ * per lane keep the FMA pipe full), operands double buffered in LDS as f32 [k][row] and read as float4
+ * (float2 for TM = 2), one LDS-only barrier per 32-k chunk, the next chunk's global loads already in
+ * flight.
+ * TM = 4 moves the fewest LDS bytes per multiply-add. Per chunk its four waves still pull 256 KB through
+ * the LDS while each SIMD issues 512 multiply-adds, about the same number of cycles, and a lone wave per
+ * SIMD overlaps the two poorly (measured: it issues 53 % of the cycles). With fewer than two such
+ * workgroups per CU, TM = 2 gives every SIMD a second wave to run in the gaps, which more than pays for
+ * its extra LDS reads. */
 #define RST_KC 32
-#define RST_LD 68 /* floats per LDS row: 64 + 4 keeps float4 reads aligned */
+#define RST_LD 68 /* floats per LDS row of 64: + 4 keeps float4 reads aligned */
+template <int TM>
 __global__ __launch_bounds__(256) void k_router_score_tile(float* __restrict__ out,
                                                            const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ w, uint32_t M,
                                                            uint32_t N, uint32_t K) {
-    __shared__ __attribute__((aligned(16))) float xs[2][RST_KC][RST_LD];
+    constexpr uint32_t BM = 16u * TM;
+    __shared__ __attribute__((aligned(16))) float xs[2][RST_KC][BM + 4];
     __shared__ __attribute__((aligned(16))) float ws[2][RST_KC][RST_LD];
     const uint32_t tid = threadIdx.x, tx = tid & 15u, ty = tid >> 4;
-    const uint32_t m0 = blockIdx.y * 64u, n0 = blockIdx.x * 64u;
-    /* staging: 64 rows x 32 k bf16 = 256 16-byte pieces per operand, one per thread */
+    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * 64u;
+    /* staging: rows x 32 k bf16 in 16-byte pieces, one per thread (the x tile has 4 * BM of them) */
     const uint32_t srow = tid >> 2, skc = tid & 3u;
     uint4 xr, wr;
     auto fetch = [&](uint32_t k0) {
         const uint32_t k = k0 + skc * 8u;
         xr = make_uint4(0, 0, 0, 0);
         wr = make_uint4(0, 0, 0, 0);
-        if (m0 + srow < M && k < K) xr = *(const uint4*)(x + (size_t)(m0 + srow) * K + k);
+        if (srow < BM && m0 + srow < M && k < K) xr = *(const uint4*)(x + (size_t)(m0 + srow) * K + k);
         if (n0 + srow < N && k < K) wr = *(const uint4*)(w + (size_t)(n0 + srow) * K + k);
     };
     auto commit = [&](uint32_t buf) {
         const uint32_t a[4] = {xr.x, xr.y, xr.z, xr.w}, b[4] = {wr.x, wr.y, wr.z, wr.w};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            xs[buf][skc * 8 + 2 * j][srow] = __uint_as_float(a[j] << 16);
-            xs[buf][skc * 8 + 2 * j + 1][srow] = __uint_as_float(a[j] & 0xFFFF0000u);
+            if (srow < BM) {
+                xs[buf][skc * 8 + 2 * j][srow] = __uint_as_float(a[j] << 16);
+                xs[buf][skc * 8 + 2 * j + 1][srow] = __uint_as_float(a[j] & 0xFFFF0000u);
+            }
             ws[buf][skc * 8 + 2 * j][srow] = __uint_as_float(b[j] << 16);
             ws[buf][skc * 8 + 2 * j + 1][srow] = __uint_as_float(b[j] & 0xFFFF0000u);
         }
     };
-    float acc[4][4];
+    float acc[TM][4];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = 0.0f;
     fetch(0);
@@ -64,30 +74,37 @@ __global__ __launch_bounds__(256) void k_router_score_tile(float* __restrict__ o
         if (kn == (uint32_t)RST_KC) {
 #pragma unroll
             for (int kk = 0; kk < RST_KC; kk++) {
-                const float4 a = *(const float4*)&xs[buf][kk][ty * 4u];
+                float av[TM];
+                if (TM == 4) {
+                    const float4 a = *(const float4*)&xs[buf][kk][ty * 4u];
+                    av[0] = a.x, av[1] = a.y, av[TM - 2] = a.z, av[TM - 1] = a.w;
+                } else {
+                    const float2 a = *(const float2*)&xs[buf][kk][ty * 2u];
+                    av[0] = a.x, av[1] = a.y;
+                }
                 const float4 b = *(const float4*)&ws[buf][kk][tx * 4u];
-                const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+                const float bv[4] = {b.x, b.y, b.z, b.w};
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < TM; i++)
 #pragma unroll
                     for (int j = 0; j < 4; j++) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
             }
         } else {
             for (uint32_t kk = 0; kk < kn; kk++)
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < TM; i++)
 #pragma unroll
                     for (int j = 0; j < 4; j++)
-                        acc[i][j] = fmaf(xs[buf][kk][ty * 4u + i], ws[buf][kk][tx * 4u + j], acc[i][j]);
+                        acc[i][j] = fmaf(xs[buf][kk][ty * TM + i], ws[buf][kk][tx * 4u + j], acc[i][j]);
         }
         if (more) commit(buf ^ 1u);
         lds_barrier();
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint32_t m = m0 + ty * 4u + i, n = n0 + tx * 4u + j;
+            const uint32_t m = m0 + ty * TM + i, n = n0 + tx * 4u + j;
             if (m < M && n < N) out[(size_t)m * N + n] = acc[i][j];
         }
 }
@@ -206,8 +223,13 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
                         hipStream_t st) {
     if (K % 8u) return PLOW_MOE_EINVAL;
     if ((uint64_t)M * N >= (1u << 19)) {
-        dim3 g((N + 63) / 64, (M + 63) / 64);
-        k_router_score_tile<<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        if ((uint64_t)((N + 63) / 64) * ((M + 63) / 64) < 512u) { /* fewer than two 64-row workgroups per CU */
+            dim3 g((N + 63) / 64, (M + 31) / 32);
+            k_router_score_tile<2><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        } else {
+            dim3 g((N + 63) / 64, (M + 63) / 64);
+            k_router_score_tile<4><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        }
     } else {
         dim3 g((N + 7) / 8, (M + 7) / 8);
         k_router_score_wave<<<g, 128, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
