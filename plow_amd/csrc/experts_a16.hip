@@ -30,6 +30,7 @@
  */
 #include "common.h"
 #include "kernels.h"
+#include <string.h>
 
 #define AK_WAVES 8u
 #define AK_THREADS (AK_WAVES * WAVE)
@@ -253,6 +254,201 @@ __global__ __launch_bounds__(AK_THREADS, GLU ? 2 : 4) void k_group_a16_stream(Gr
     for (uint32_t rb = 0; rb < cnt; rb += 16u) ak_body<ENC, GLU>(g, e, ct, r0, rb, cnt);
 }
 
+/* ---- mxfp4 weights, second form: every load goes global -> LDS in the coalesced shape ---------------
+ * The kernel above reads its operands the way the matrix instruction wants them (lane = row), which the
+ * vector memory pipeline serves at a quarter of its rate: 16 rows, so 16 cache lines, per load
+ * instruction. With half a byte per weight that instruction rate, not memory, bounds it. Here a step is
+ * 256 k, i.e. one whole 128-byte line per weight row, and
+ *   weights   per wave and stream 16 rows x 128 B = two direct loads (8 consecutive lanes per line) into a
+ *             wave-private ring; E8M0 bytes (8 per row and step) one 4-byte direct load per stream;
+ *   rows      the 16 activation rows of the pass are the same for all eight waves: 16 x 512 B per step in
+ *             a ring shared by the workgroup, wave w loading rows 2w and 2w + 1 (32 lanes per row);
+ *   sync      rings of three steps, loads two steps ahead; per step each wave waits for its own loads
+ *             (s_waitcnt vmcnt) and all meet at one barrier, after which the step before is free;
+ *   swizzle   direct loads write LDS contiguously, so bank conflicts are avoided on the global side:
+ *             LDS piece p of weight row r holds global piece p ^ ((r >> 1) & 7); piece p of activation
+ *             row r holds global piece (p & 16) | ((p ^ r) & 15).
+ * Same arithmetic and the same order of additions as the first form. K must be a multiple of 256. */
+#define MX_STAGES 3u
+struct MxWSlot {
+    uint8_t w[2][16u * 128u]; /* [stream][row][128 B] */
+    uint8_t sc[2][256];       /* [stream][row][8 B]; lanes 32..63 write copies behind */
+};
+struct MxLds {
+    uint8_t x[MX_STAGES][16u * 512u];
+    MxWSlot ring[AK_WAVES][MX_STAGES];
+};
+typedef __attribute__((address_space(3))) void mx_lds_void;
+__device__ __forceinline__ uint32_t mx_lds_off(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+__device__ __forceinline__ v4i mx_read16(uint32_t addr) {
+    v4i r;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+    return r;
+}
+__device__ __forceinline__ uint2 mx_read8(uint32_t addr) {
+    uint2 r;
+    asm volatile("ds_read_b64 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+    return r;
+}
+
+template <bool GLU>
+__global__ __launch_bounds__(AK_THREADS) void k_group_mx_dma(GroupA16 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t mx_raw[];
+    MxLds& L = *(MxLds*)mx_raw;
+    constexpr int NL = GLU ? 7 : 4; /* direct loads per wave and step: weights 2 per stream, scales 1 per stream, rows 1 */
+    const uint32_t tiles = g.N / AK_BN;
+    const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
+    const uint32_t cnt = (uint32_t)g.meta[g.E + e];
+    if (cnt == 0u) return;
+    const uint64_t* wt = g.wtab + (size_t)e * g.wcols;
+    const uint64_t* stt = g.stab + (size_t)e * g.wcols;
+    if (wt[g.wsel0] == 0ull || stt[g.wsel0] == 0ull) return; /* expert not resident: skipped */
+    const uint32_t r0 = (uint32_t)g.meta[e];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, MX block q of a 128-k half */
+    const uint32_t K = g.K, KS = K / 256u, N = g.N;
+    const uint32_t chw = ct * AK_BN + wv * 16u;   /* this wave's first channel */
+
+    /* weight loads: load j covers rows 8j .. 8j + 7 of a stream (lane = row lr of the group, piece p) */
+    const uint32_t lr = lane >> 3, p = lane & 7u;
+    const uint8_t* wsrc[2][2];
+    const uint8_t* ssrc[2];
+#pragma unroll
+    for (int sidx = 0; sidx < (GLU ? 2 : 1); sidx++) {
+        const uint8_t* wbase = (const uint8_t*)(uintptr_t)wt[sidx ? g.wsel1 : g.wsel0];
+        const uint8_t* sbase = (const uint8_t*)(uintptr_t)stt[sidx ? g.wsel1 : g.wsel0];
+        const uint32_t row0 = chw + (sidx ? g.wrow1 : g.wrow0);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; j++) {
+            const uint32_t R = 8u * j + lr;
+            wsrc[sidx][j] = wbase + (size_t)(row0 + R) * (K / 2u) + ((p ^ ((R >> 1) & 7u)) << 4);
+        }
+        /* scales: lane -> (row (lane & 31) >> 1, dword lane & 1) of the step's 8 bytes per row */
+        ssrc[sidx] = sbase + (size_t)(row0 + ((lane & 31u) >> 1)) * (K / 32u) + (lane & 1u) * 4u;
+    }
+    const uint32_t swz = (c >> 1) & 7u;
+    const uint32_t x_base = mx_lds_off(&L.x[0][0]);
+    const uint32_t w_base = mx_lds_off(&L.ring[wv][0]);
+
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) {
+        /* this wave's share of the pass's rows: rows 2 wv and 2 wv + 1, 32 lanes each; a pad row reads the
+         * pass's first row and is never stored */
+        const uint32_t xrow = 2u * wv + (lane >> 5), pc = lane & 31u;
+        const uint8_t* xsrc;
+        {
+            const uint32_t first = g.a_idx ? g.a_idx[r0 + rb] : r0 + rb;
+            const uint32_t off = rb + xrow;
+            uint32_t ai = off < cnt ? (g.a_idx ? g.a_idx[r0 + off] : r0 + off) : PLOW_EXPERT_UNUSED;
+            if (ai == PLOW_EXPERT_UNUSED) ai = first == PLOW_EXPERT_UNUSED ? 0u : first;
+            xsrc = (const uint8_t*)g.a + (size_t)ai * K * 2u + (((pc & 16u) | ((pc ^ xrow) & 15u)) << 4);
+        }
+        /* the B-operand row of this lane */
+        const uint32_t off = rb + c, r = r0 + off;
+        bool valid = off < cnt;
+        const uint32_t ai_c = valid ? (g.a_idx ? g.a_idx[r] : r) : PLOW_EXPERT_UNUSED;
+        valid = ai_c != PLOW_EXPERT_UNUSED;
+
+        auto issue = [&](uint32_t S) {
+            const uint32_t st = S % MX_STAGES;
+            MxWSlot* slot = &L.ring[wv][st];
+#pragma unroll
+            for (int sidx = 0; sidx < (GLU ? 2 : 1); sidx++) {
+#pragma unroll
+                for (uint32_t j = 0; j < 2u; j++)
+                    __builtin_amdgcn_global_load_lds((const void*)(wsrc[sidx][j] + (size_t)S * 128u),
+                                                     (mx_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)S * 8u),
+                                                 (mx_lds_void*)&slot->sc[sidx][0], 4, 0, 0);
+            }
+            __builtin_amdgcn_global_load_lds((const void*)(xsrc + (size_t)S * 512u),
+                                             (mx_lds_void*)&L.x[st][2u * wv * 512u], 16, 0, 0);
+        };
+        v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
+        /* the row maps above are loaded (the count of outstanding loads starts at zero), and every wave
+         * has left the pass before (its ring slots are free) */
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        issue(0);
+        if (KS > 1u) issue(1);
+        for (uint32_t S = 0; S < KS; S++) {
+            /* loads return in order: step S has landed once at most step S + 1's are outstanding; after the
+             * barrier every wave's share of the rows is there and nobody reads step S - 1 any more */
+            if (S + 1u < KS) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NL) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if (S + 2u < KS) issue(S + 2u);
+            const uint32_t st = S % MX_STAGES;
+            const uint32_t wb = w_base + st * (uint32_t)sizeof(MxWSlot), xb = x_base + st * (16u * 512u) + c * 512u;
+            uint2 e0 = mx_read8(wb + 4096u + c * 8u), e1 = e0;
+            if (GLU) e1 = mx_read8(wb + 4096u + 256u + c * 8u);
+            v4i wa[2], wbv[2], xa[2][4];
+#pragma unroll
+            for (uint32_t u = 0; u < 2u; u++) {
+                const uint32_t wo = c * 128u + (((4u * u + q) ^ swz) << 4);
+                wa[u] = mx_read16(wb + wo);
+                wbv[u] = wa[u];
+                if (GLU) wbv[u] = mx_read16(wb + 2048u + wo);
+#pragma unroll
+                for (uint32_t j = 0; j < 4u; j++) {
+                    const uint32_t P = 16u * u + 4u * q + j;
+                    xa[u][j] = mx_read16(xb + (((P & 16u) | ((P ^ c) & 15u)) << 4));
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e0), "+v"(e1), "+v"(wa[0]), "+v"(wa[1]), "+v"(wbv[0]), "+v"(wbv[1]));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0][0]), "+v"(xa[0][1]), "+v"(xa[0][2]), "+v"(xa[0][3]));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[1][0]), "+v"(xa[1][1]), "+v"(xa[1][2]), "+v"(xa[1][3]));
+#pragma unroll
+            for (uint32_t u = 0; u < 2u; u++) {
+                const uint32_t s0 = ((u ? e0.y : e0.x) >> (8u * q)) & 0xFFu, s1 = ((u ? e1.y : e1.x) >> (8u * q)) & 0xFFu;
+                WStep<AENC_MXFP4> da, db;
+                da.r[0] = wa[u];
+                db.r[0] = wbv[u];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const v8bf B = __builtin_bit_cast(v8bf, xa[u][j]);
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(da, j, s0), B, acc0, 0, 0, 0);
+                    if (GLU) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(db, j, s1), B, acc1, 0, 0, 0);
+                }
+            }
+        }
+        /* ---- epilogue: lane holds channels chw + 4q + i of row rb + c ---- */
+        if (valid) {
+            const uint32_t col = chw + 4u * q;
+            const uint32_t oi = g.o_idx ? g.o_idx[r] : r;
+            if (oi != PLOW_EXPERT_UNUSED) {
+                if (GLU) {
+                    uint2 o;
+                    o.x = (uint32_t)f2bf(moe_glu(acc0[0], acc1[0], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[1], acc1[1], g.act)) << 16);
+                    o.y = (uint32_t)f2bf(moe_glu(acc0[2], acc1[2], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[3], acc1[3], g.act)) << 16);
+                    *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
+                } else {
+                    const float gate = g.gate ? g.gate[r] : 1.0f;
+                    const float y0 = gate * acc0[0], y1 = gate * acc0[1], y2 = gate * acc0[2], y3 = gate * acc0[3];
+                    if (g.out_bf16) {
+                        uint2 o;
+                        o.x = (uint32_t)f2bf(g.gate ? y0 : acc0[0]) | ((uint32_t)f2bf(g.gate ? y1 : acc0[1]) << 16);
+                        o.y = (uint32_t)f2bf(g.gate ? y2 : acc0[2]) | ((uint32_t)f2bf(g.gate ? y3 : acc0[3]) << 16);
+                        *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
+                    } else {
+                        *(float4*)((float*)g.out + (size_t)oi * N + col) = make_float4(y0, y1, y2, y3);
+                    }
+                }
+            }
+        }
+    }
+}
+
+/* PLOW_MOE_MX_KERNEL=regs selects the first form for mxfp4 weights */
+static bool mx_dma_form() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = getenv("PLOW_MOE_MX_KERNEL");
+        v = (e && !strcmp(e, "regs")) ? 0 : 1;
+    }
+    return v == 1;
+}
+
 template <bool GLU>
 static int launch_a16(const GroupA16& g, hipStream_t st) {
     if (g.N == 0 || g.K == 0 || g.E == 0 || g.N % AK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
@@ -261,7 +457,20 @@ static int launch_a16(const GroupA16& g, hipStream_t st) {
     switch (g.enc) {
     case AENC_BF16: k_group_a16_stream<AENC_BF16, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
     case AENC_FP8BLK: k_group_a16_stream<AENC_FP8BLK, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
-    case AENC_MXFP4: k_group_a16_stream<AENC_MXFP4, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
+    case AENC_MXFP4:
+        if (g.K % 256u == 0u && g.meta && g.wtab && g.stab && mx_dma_form()) {
+            static bool attr_set = false;
+            if (!attr_set) {
+                if (hipFuncSetAttribute((const void*)k_group_mx_dma<GLU>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)sizeof(MxLds)) != hipSuccess)
+                    return PLOW_MOE_EDEVICE;
+                attr_set = true;
+            }
+            k_group_mx_dma<GLU><<<grid, AK_THREADS, sizeof(MxLds), st>>>(g);
+        } else {
+            k_group_a16_stream<AENC_MXFP4, GLU><<<grid, AK_THREADS, 0, st>>>(g);
+        }
+        break;
     case AENC_FP8PC: k_group_a16_stream<AENC_FP8PC, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
     default: return PLOW_MOE_EUNSUPPORTED;
     }
