@@ -254,96 +254,133 @@ __global__ __launch_bounds__(AK_THREADS, GLU ? 2 : 4) void k_group_a16_stream(Gr
     for (uint32_t rb = 0; rb < cnt; rb += 16u) ak_body<ENC, GLU>(g, e, ct, r0, rb, cnt);
 }
 
-/* ---- mxfp4 weights, second form: every load goes global -> LDS in the coalesced shape ---------------
+/* ---- second form: every load goes global -> LDS in the coalesced shape -------------------------------
  * The kernel above reads its operands the way the matrix instruction wants them (lane = row), which the
- * vector memory pipeline serves at a quarter of its rate: 16 rows, so 16 cache lines, per load
- * instruction. With half a byte per weight that instruction rate, not memory, bounds it. Here a step is
- * 256 k, i.e. one whole 128-byte line per weight row, and
+ * vector memory pipeline serves at a quarter of its rate: 16 rows, so 16 or more cache lines, per load
+ * instruction. That instruction rate, not memory, bounds it. Here a step is one whole 128-byte line per
+ * weight row (256 k of mxfp4, 128 k of fp8, 64 k of bf16), and
  *   weights   per wave and stream 16 rows x 128 B = two direct loads (8 consecutive lanes per line) into a
- *             wave-private ring; E8M0 bytes (8 per row and step) one 4-byte direct load per stream;
- *   rows      the 16 activation rows of the pass are the same for all eight waves: 16 x 512 B per step in
- *             a ring shared by the workgroup, wave w loading rows 2w and 2w + 1 (32 lanes per row);
+ *             wave-private ring; mxfp4: the step's E8M0 bytes (8 per row) by one 4-byte direct load per
+ *             stream; block-fp8: the tile's block scales sit in LDS for all of K;
+ *   rows      the 16 activation rows of the pass are the same for all eight waves: 16 rows x 2 bytes per k
+ *             of the step, in a ring shared by the workgroup and loaded 1 KB per wave (the first 8, 4 or 2
+ *             waves);
  *   sync      rings of three steps, loads two steps ahead; per step each wave waits for its own loads
  *             (s_waitcnt vmcnt) and all meet at one barrier, after which the step before is free;
  *   swizzle   direct loads write LDS contiguously, so bank conflicts are avoided on the global side:
- *             LDS piece p of weight row r holds global piece p ^ ((r >> 1) & 7); piece p of activation
- *             row r holds global piece (p & 16) | ((p ^ r) & 15).
- * Same arithmetic and the same order of additions as the first form. K must be a multiple of 256. */
-#define MX_STAGES 3u
-struct MxWSlot {
+ *             LDS piece p of weight row r holds global piece p ^ ((r >> 1) & 7), and likewise for
+ *             activation rows of 128 B; piece p of a longer activation row r holds global piece
+ *             (p & ~15) | ((p ^ r) & 15).
+ * Same arithmetic and the same order of additions as the first form. */
+#define DM_STAGES 3u
+template <int ENC> struct DmGeom;
+template <> struct DmGeom<AENC_MXFP4> { static constexpr uint32_t KSTEP = 256u; };
+template <> struct DmGeom<AENC_FP8PC> { static constexpr uint32_t KSTEP = 128u; };
+template <> struct DmGeom<AENC_FP8BLK> { static constexpr uint32_t KSTEP = 128u; };
+template <> struct DmGeom<AENC_BF16> { static constexpr uint32_t KSTEP = 64u; };
+struct DmWSlot {
     uint8_t w[2][16u * 128u]; /* [stream][row][128 B] */
-    uint8_t sc[2][256];       /* [stream][row][8 B]; lanes 32..63 write copies behind */
+    uint8_t sc[2][256];       /* mxfp4: [stream][row][8 B]; lanes 32..63 write copies behind */
 };
-struct MxLds {
-    uint8_t x[MX_STAGES][16u * 512u];
-    MxWSlot ring[AK_WAVES][MX_STAGES];
+template <int ENC>
+struct DmLds {
+    uint8_t x[DM_STAGES][16u * DmGeom<ENC>::KSTEP * 2u];
+    DmWSlot ring[AK_WAVES][DM_STAGES];
+    float bsc[2][128]; /* block-fp8: the tile's weight block scales, all of K (K <= 16384) */
 };
-typedef __attribute__((address_space(3))) void mx_lds_void;
-__device__ __forceinline__ uint32_t mx_lds_off(const void* p) {
+typedef __attribute__((address_space(3))) void dm_lds_void;
+__device__ __forceinline__ uint32_t dm_lds_off(const void* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }
-__device__ __forceinline__ v4i mx_read16(uint32_t addr) {
+__device__ __forceinline__ v4i dm_read16(uint32_t addr) {
     v4i r;
     asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr) : "memory");
     return r;
 }
-__device__ __forceinline__ uint2 mx_read8(uint32_t addr) {
+__device__ __forceinline__ uint2 dm_read8(uint32_t addr) {
     uint2 r;
     asm volatile("ds_read_b64 %0, %1" : "=v"(r) : "v"(addr) : "memory");
     return r;
 }
+__device__ __forceinline__ float dm_read4(uint32_t addr) {
+    float r;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+    return r;
+}
+/* wait until at most n of this wave's loads are outstanding (and its LDS reads are done), then the
+ * workgroup barrier */
+#define DM_WAIT_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory")
 
-template <bool GLU>
-__global__ __launch_bounds__(AK_THREADS) void k_group_mx_dma(GroupA16 g) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t mx_raw[];
-    MxLds& L = *(MxLds*)mx_raw;
-    constexpr int NL = GLU ? 7 : 4; /* direct loads per wave and step: weights 2 per stream, scales 1 per stream, rows 1 */
+template <int ENC, bool GLU>
+__global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
+    DmLds<ENC>& L = *(DmLds<ENC>*)dm_raw;
+    constexpr uint32_t KSTEP = DmGeom<ENC>::KSTEP, XROW = KSTEP * 2u; /* activation bytes per row and step */
+    constexpr uint32_t NP = XROW / 16u;                              /* 16-byte pieces per activation row */
+    constexpr uint32_t XL = 16u * XROW / 1024u;                      /* waves that load activation rows */
+    constexpr uint32_t XRPL = 64u / NP;                              /* rows per activation load */
+    constexpr int NS = GLU ? 2 : 1;
+    /* direct loads per wave and step: weights 2 per stream, mxfp4 scales 1 per stream, rows 1 (first XL waves) */
+    constexpr int NLW = NS * (ENC == AENC_MXFP4 ? 3 : 2);
     const uint32_t tiles = g.N / AK_BN;
     const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
-    const uint32_t cnt = (uint32_t)g.meta[g.E + e];
+    const uint32_t cnt = g.meta ? (uint32_t)g.meta[g.E + e] : g.dense_rows;
     if (cnt == 0u) return;
-    const uint64_t* wt = g.wtab + (size_t)e * g.wcols;
-    const uint64_t* stt = g.stab + (size_t)e * g.wcols;
-    if (wt[g.wsel0] == 0ull || stt[g.wsel0] == 0ull) return; /* expert not resident: skipped */
-    const uint32_t r0 = (uint32_t)g.meta[e];
+    const uint64_t* wt = g.wtab ? g.wtab + (size_t)e * g.wcols : nullptr;
+    const uint64_t* stt = g.stab ? g.stab + (size_t)e * g.wcols : nullptr;
+    if (wt && wt[g.wsel0] == 0ull) return; /* expert not resident: skipped */
+    if (stt && ENC != AENC_BF16 && stt[g.wsel0] == 0ull) return;
+    const uint32_t r0 = g.meta ? (uint32_t)g.meta[e] : 0u;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, MX block q of a 128-k half */
-    const uint32_t K = g.K, KS = K / 256u, N = g.N;
+    const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, k-chunk q */
+    const uint32_t K = g.K, KS = K / KSTEP, N = g.N;
     const uint32_t chw = ct * AK_BN + wv * 16u;   /* this wave's first channel */
+    const uint32_t wrow = ENC == AENC_BF16 ? K * 2u : (ENC == AENC_MXFP4 ? K / 2u : K); /* bytes per weight row */
 
     /* weight loads: load j covers rows 8j .. 8j + 7 of a stream (lane = row lr of the group, piece p) */
     const uint32_t lr = lane >> 3, p = lane & 7u;
     const uint8_t* wsrc[2][2];
-    const uint8_t* ssrc[2];
+    const uint8_t* ssrc[2] = {nullptr, nullptr};
+    const float* pcs[2] = {nullptr, nullptr}; /* per-channel fp8: this lane's four output scales per stream */
 #pragma unroll
-    for (int sidx = 0; sidx < (GLU ? 2 : 1); sidx++) {
-        const uint8_t* wbase = (const uint8_t*)(uintptr_t)wt[sidx ? g.wsel1 : g.wsel0];
-        const uint8_t* sbase = (const uint8_t*)(uintptr_t)stt[sidx ? g.wsel1 : g.wsel0];
-        const uint32_t row0 = chw + (sidx ? g.wrow1 : g.wrow0);
+    for (int sidx = 0; sidx < NS; sidx++) {
+        const uint32_t sel = sidx ? g.wsel1 : g.wsel0;
+        const uint8_t* wbase = wt ? (const uint8_t*)(uintptr_t)wt[sel] : (const uint8_t*)g.wdirect[sidx];
+        const uint8_t* sbase = stt ? (const uint8_t*)(uintptr_t)stt[sel] : nullptr;
+        const uint32_t wr0 = sidx ? g.wrow1 : g.wrow0, row0 = chw + wr0;
 #pragma unroll
         for (uint32_t j = 0; j < 2u; j++) {
             const uint32_t R = 8u * j + lr;
-            wsrc[sidx][j] = wbase + (size_t)(row0 + R) * (K / 2u) + ((p ^ ((R >> 1) & 7u)) << 4);
+            wsrc[sidx][j] = wbase + (size_t)(row0 + R) * wrow + ((p ^ ((R >> 1) & 7u)) << 4);
         }
-        /* scales: lane -> (row (lane & 31) >> 1, dword lane & 1) of the step's 8 bytes per row */
-        ssrc[sidx] = sbase + (size_t)(row0 + ((lane & 31u) >> 1)) * (K / 32u) + (lane & 1u) * 4u;
+        /* mxfp4 scales: lane -> (row (lane & 31) >> 1, dword lane & 1) of the step's 8 bytes per row */
+        if (ENC == AENC_MXFP4) ssrc[sidx] = sbase + (size_t)(row0 + ((lane & 31u) >> 1)) * (K / 32u) + (lane & 1u) * 4u;
+        if (ENC == AENC_FP8PC) pcs[sidx] = (const float*)sbase + wr0 + chw + 4u * q;
+        if (ENC == AENC_FP8BLK) { /* the channel block's scale row goes to LDS once */
+            const float* bs = (const float*)sbase + (size_t)((ct * AK_BN + wr0) / 128u) * (K / 128u);
+            for (uint32_t i = threadIdx.x; i < K / 128u; i += AK_THREADS) L.bsc[sidx][i] = bs[i];
+        }
     }
     const uint32_t swz = (c >> 1) & 7u;
-    const uint32_t x_base = mx_lds_off(&L.x[0][0]);
-    const uint32_t w_base = mx_lds_off(&L.ring[wv][0]);
+    const uint32_t x_base = dm_lds_off(&L.x[0][0]);
+    const uint32_t w_base = dm_lds_off(&L.ring[wv][0]);
+    const uint32_t b_base = dm_lds_off(&L.bsc[0][0]);
+    /* LDS position of logical piece P of activation row c */
+    auto xpos = [&](uint32_t P) -> uint32_t { return NP >= 16u ? ((P & ~15u) | ((P ^ c) & 15u)) : (P ^ swz); };
 
     for (uint32_t rb = 0; rb < cnt; rb += 16u) {
-        /* this wave's share of the pass's rows: rows 2 wv and 2 wv + 1, 32 lanes each; a pad row reads the
-         * pass's first row and is never stored */
-        const uint32_t xrow = 2u * wv + (lane >> 5), pc = lane & 31u;
-        const uint8_t* xsrc;
-        {
+        /* this wave's share of the pass's rows (waves 0 .. XL - 1): XRPL rows, NP lanes each; a pad row
+         * reads the pass's first row and is never stored */
+        const uint32_t xrow = XRPL * wv + lane / NP, pc = lane % NP;
+        const uint8_t* xsrc = nullptr;
+        if (wv < XL) {
             const uint32_t first = g.a_idx ? g.a_idx[r0 + rb] : r0 + rb;
             const uint32_t off = rb + xrow;
             uint32_t ai = off < cnt ? (g.a_idx ? g.a_idx[r0 + off] : r0 + off) : PLOW_EXPERT_UNUSED;
             if (ai == PLOW_EXPERT_UNUSED) ai = first == PLOW_EXPERT_UNUSED ? 0u : first;
-            xsrc = (const uint8_t*)g.a + (size_t)ai * K * 2u + (((pc & 16u) | ((pc ^ xrow) & 15u)) << 4);
+            const uint32_t gp = NP >= 16u ? ((pc & ~15u) | ((pc ^ xrow) & 15u)) : (pc ^ ((xrow >> 1) & 7u));
+            xsrc = (const uint8_t*)g.a + (size_t)ai * K * 2u + (gp << 4);
         }
         /* the B-operand row of this lane */
         const uint32_t off = rb + c, r = r0 + off;
@@ -352,69 +389,136 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_mx_dma(GroupA16 g) {
         valid = ai_c != PLOW_EXPERT_UNUSED;
 
         auto issue = [&](uint32_t S) {
-            const uint32_t st = S % MX_STAGES;
-            MxWSlot* slot = &L.ring[wv][st];
+            const uint32_t st = S % DM_STAGES;
+            DmWSlot* slot = &L.ring[wv][st];
 #pragma unroll
-            for (int sidx = 0; sidx < (GLU ? 2 : 1); sidx++) {
+            for (int sidx = 0; sidx < NS; sidx++) {
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; j++)
                     __builtin_amdgcn_global_load_lds((const void*)(wsrc[sidx][j] + (size_t)S * 128u),
-                                                     (mx_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)S * 8u),
-                                                 (mx_lds_void*)&slot->sc[sidx][0], 4, 0, 0);
+                                                     (dm_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, 0);
+                if (ENC == AENC_MXFP4)
+                    __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)S * 8u),
+                                                     (dm_lds_void*)&slot->sc[sidx][0], 4, 0, 0);
             }
-            __builtin_amdgcn_global_load_lds((const void*)(xsrc + (size_t)S * 512u),
-                                             (mx_lds_void*)&L.x[st][2u * wv * 512u], 16, 0, 0);
+            if (wv < XL)
+                __builtin_amdgcn_global_load_lds((const void*)(xsrc + (size_t)S * XROW),
+                                                 (dm_lds_void*)&L.x[st][XRPL * wv * XROW], 16, 0, 0);
         };
         v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
         /* the row maps above are loaded (the count of outstanding loads starts at zero), and every wave
-         * has left the pass before (its ring slots are free) */
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+         * has left the pass before (its ring slots are free; the block scales are written) */
+        DM_WAIT_BARRIER(0);
         issue(0);
         if (KS > 1u) issue(1);
         for (uint32_t S = 0; S < KS; S++) {
             /* loads return in order: step S has landed once at most step S + 1's are outstanding; after the
              * barrier every wave's share of the rows is there and nobody reads step S - 1 any more */
-            if (S + 1u < KS) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NL) : "memory");
-            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if (S + 1u >= KS) DM_WAIT_BARRIER(0);
+            else if (wv < XL) DM_WAIT_BARRIER(NLW + 1);
+            else DM_WAIT_BARRIER(NLW);
             if (S + 2u < KS) issue(S + 2u);
-            const uint32_t st = S % MX_STAGES;
-            const uint32_t wb = w_base + st * (uint32_t)sizeof(MxWSlot), xb = x_base + st * (16u * 512u) + c * 512u;
-            uint2 e0 = mx_read8(wb + 4096u + c * 8u), e1 = e0;
-            if (GLU) e1 = mx_read8(wb + 4096u + 256u + c * 8u);
-            v4i wa[2], wbv[2], xa[2][4];
+            const uint32_t st = S % DM_STAGES;
+            const uint32_t wb = w_base + st * (uint32_t)sizeof(DmWSlot), xb = x_base + st * (16u * XROW) + c * XROW;
+            if (ENC == AENC_MXFP4) {
+                uint2 e0 = dm_read8(wb + 4096u + c * 8u), e1 = e0;
+                if (GLU) e1 = dm_read8(wb + 4096u + 256u + c * 8u);
+                v4i wa[2], wbv[2], xa[2][4];
 #pragma unroll
-            for (uint32_t u = 0; u < 2u; u++) {
-                const uint32_t wo = c * 128u + (((4u * u + q) ^ swz) << 4);
-                wa[u] = mx_read16(wb + wo);
-                wbv[u] = wa[u];
-                if (GLU) wbv[u] = mx_read16(wb + 2048u + wo);
+                for (uint32_t u = 0; u < 2u; u++) {
+                    const uint32_t wo = c * 128u + (((4u * u + q) ^ swz) << 4);
+                    wa[u] = dm_read16(wb + wo);
+                    wbv[u] = wa[u];
+                    if (GLU) wbv[u] = dm_read16(wb + 2048u + wo);
 #pragma unroll
-                for (uint32_t j = 0; j < 4u; j++) {
-                    const uint32_t P = 16u * u + 4u * q + j;
-                    xa[u][j] = mx_read16(xb + (((P & 16u) | ((P ^ c) & 15u)) << 4));
+                    for (uint32_t j = 0; j < 4u; j++) xa[u][j] = dm_read16(xb + (xpos(16u * u + 4u * q + j) << 4));
                 }
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e0), "+v"(e1), "+v"(wa[0]), "+v"(wa[1]), "+v"(wbv[0]), "+v"(wbv[1]));
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0][0]), "+v"(xa[0][1]), "+v"(xa[0][2]), "+v"(xa[0][3]));
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[1][0]), "+v"(xa[1][1]), "+v"(xa[1][2]), "+v"(xa[1][3]));
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e0), "+v"(e1), "+v"(wa[0]), "+v"(wa[1]), "+v"(wbv[0]), "+v"(wbv[1]));
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0][0]), "+v"(xa[0][1]), "+v"(xa[0][2]), "+v"(xa[0][3]));
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[1][0]), "+v"(xa[1][1]), "+v"(xa[1][2]), "+v"(xa[1][3]));
 #pragma unroll
-            for (uint32_t u = 0; u < 2u; u++) {
-                const uint32_t s0 = ((u ? e0.y : e0.x) >> (8u * q)) & 0xFFu, s1 = ((u ? e1.y : e1.x) >> (8u * q)) & 0xFFu;
-                WStep<AENC_MXFP4> da, db;
-                da.r[0] = wa[u];
-                db.r[0] = wbv[u];
+                for (uint32_t u = 0; u < 2u; u++) {
+                    const uint32_t s0 = ((u ? e0.y : e0.x) >> (8u * q)) & 0xFFu, s1 = ((u ? e1.y : e1.x) >> (8u * q)) & 0xFFu;
+                    WStep<AENC_MXFP4> da, db;
+                    da.r[0] = wa[u];
+                    db.r[0] = wbv[u];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const v8bf B = __builtin_bit_cast(v8bf, xa[u][j]);
+                        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(da, j, s0), B, acc0, 0, 0, 0);
+                        if (GLU) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(db, j, s1), B, acc1, 0, 0, 0);
+                    }
+                }
+            } else if (ENC == AENC_BF16) {
+                /* 64 k: instruction j uses k = 32 j + 8 q .. + 8 of both operands */
+                v4i wa[2], wbv[2], xa[2];
+#pragma unroll
+                for (uint32_t j = 0; j < 2u; j++) {
+                    const uint32_t wo = c * 128u + (((4u * j + q) ^ swz) << 4);
+                    wa[j] = dm_read16(wb + wo);
+                    wbv[j] = wa[j];
+                    if (GLU) wbv[j] = dm_read16(wb + 2048u + wo);
+                    xa[j] = dm_read16(xb + (xpos(4u * j + q) << 4));
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wa[0]), "+v"(wa[1]), "+v"(wbv[0]), "+v"(wbv[1]), "+v"(xa[0]), "+v"(xa[1]));
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const v8bf B = __builtin_bit_cast(v8bf, xa[j]);
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wa[j]), B, acc0, 0, 0, 0);
+                    if (GLU) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wbv[j]), B, acc1, 0, 0, 0);
+                }
+            } else {
+                /* fp8, 128 k: the lane's weight bytes are [16q, 16q + 16) and [64 + 16q, 64 + 16q + 16);
+                 * instruction j uses bytes 8 (j & 1) .. + 8 of half j >> 1 */
+                WStep<ENC> da, db;
+                v4i xa[4];
+                float sa = 1.0f, sb = 1.0f;
+#pragma unroll
+                for (uint32_t h = 0; h < 2u; h++) {
+                    const uint32_t wo = c * 128u + (((4u * h + q) ^ swz) << 4);
+                    da.r[h] = dm_read16(wb + wo);
+                    db.r[h] = da.r[h];
+                    if (GLU) db.r[h] = dm_read16(wb + 2048u + wo);
+                }
+#pragma unroll
+                for (uint32_t j = 0; j < 4u; j++) xa[j] = dm_read16(xb + (xpos(8u * (j >> 1) + 2u * q + (j & 1u)) << 4));
+                if (ENC == AENC_FP8BLK) {
+                    sa = dm_read4(b_base + S * 4u);
+                    sb = sa;
+                    if (GLU) sb = dm_read4(b_base + 512u + S * 4u);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(da.r[0]), "+v"(da.r[1]), "+v"(db.r[0]), "+v"(db.r[1]), "+v"(sa), "+v"(sb));
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0]), "+v"(xa[1]), "+v"(xa[2]), "+v"(xa[3]));
+                v4f t0 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc0;
+                v4f t1 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc1;
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const v8bf B = __builtin_bit_cast(v8bf, xa[u][j]);
-                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(da, j, s0), B, acc0, 0, 0, 0);
-                    if (GLU) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(db, j, s1), B, acc1, 0, 0, 0);
+                    const v8bf B = __builtin_bit_cast(v8bf, xa[j]);
+                    t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(da, j), B, t0, 0, 0, 0);
+                    if (GLU) t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(db, j), B, t1, 0, 0, 0);
+                }
+                if (ENC == AENC_FP8BLK) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        acc0[i] = fmaf(t0[i], sa, acc0[i]);
+                        if (GLU) acc1[i] = fmaf(t1[i], sb, acc1[i]);
+                    }
+                } else {
+                    acc0 = t0;
+                    if (GLU) acc1 = t1;
                 }
             }
         }
         /* ---- epilogue: lane holds channels chw + 4q + i of row rb + c ---- */
         if (valid) {
             const uint32_t col = chw + 4u * q;
+            if (ENC == AENC_FP8PC) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    acc0[i] *= pcs[0][i];
+                    if (GLU) acc1[i] *= pcs[1][i];
+                }
+            }
             const uint32_t oi = g.o_idx ? g.o_idx[r] : r;
             if (oi != PLOW_EXPERT_UNUSED) {
                 if (GLU) {
@@ -439,14 +543,27 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_mx_dma(GroupA16 g) {
     }
 }
 
-/* PLOW_MOE_MX_KERNEL=regs selects the first form for mxfp4 weights */
-static bool mx_dma_form() {
+/* PLOW_MOE_A16_KERNEL=regs selects the first form */
+static bool a16_dma_form() {
     static int v = -1;
     if (v < 0) {
-        const char* e = getenv("PLOW_MOE_MX_KERNEL");
+        const char* e = getenv("PLOW_MOE_A16_KERNEL");
         v = (e && !strcmp(e, "regs")) ? 0 : 1;
     }
     return v == 1;
+}
+
+template <int ENC, bool GLU>
+static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)k_group_a16_dma<ENC, GLU>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)sizeof(DmLds<ENC>)) != hipSuccess)
+            return PLOW_MOE_EDEVICE;
+        attr_set = true;
+    }
+    k_group_a16_dma<ENC, GLU><<<grid, AK_THREADS, sizeof(DmLds<ENC>), st>>>(g);
+    return 0;
 }
 
 template <bool GLU>
@@ -454,24 +571,27 @@ static int launch_a16(const GroupA16& g, hipStream_t st) {
     if (g.N == 0 || g.K == 0 || g.E == 0 || g.N % AK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
     if ((uint64_t)g.E * (g.N / AK_BN) > 0x7FFFFFFFull) return PLOW_MOE_EINVAL;
     const dim3 grid(g.E * (g.N / AK_BN));
+    /* second form: needs whole steps of K (one 128-byte line per weight row) and the block scales of a
+     * tile to fit its LDS table */
+    const bool dma = a16_dma_form() && g.K <= 16384u &&
+                     g.K % (g.enc == AENC_MXFP4 ? 256u : 128u) == 0u && (g.enc == AENC_BF16 || g.stab);
     switch (g.enc) {
-    case AENC_BF16: k_group_a16_stream<AENC_BF16, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
-    case AENC_FP8BLK: k_group_a16_stream<AENC_FP8BLK, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
-    case AENC_MXFP4:
-        if (g.K % 256u == 0u && g.meta && g.wtab && g.stab && mx_dma_form()) {
-            static bool attr_set = false;
-            if (!attr_set) {
-                if (hipFuncSetAttribute((const void*)k_group_mx_dma<GLU>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        (int)sizeof(MxLds)) != hipSuccess)
-                    return PLOW_MOE_EDEVICE;
-                attr_set = true;
-            }
-            k_group_mx_dma<GLU><<<grid, AK_THREADS, sizeof(MxLds), st>>>(g);
-        } else {
-            k_group_a16_stream<AENC_MXFP4, GLU><<<grid, AK_THREADS, 0, st>>>(g);
-        }
+    case AENC_BF16:
+        if (dma) return launch_a16_dma<AENC_BF16, GLU>(g, grid, st);
+        k_group_a16_stream<AENC_BF16, GLU><<<grid, AK_THREADS, 0, st>>>(g);
         break;
-    case AENC_FP8PC: k_group_a16_stream<AENC_FP8PC, GLU><<<grid, AK_THREADS, 0, st>>>(g); break;
+    case AENC_FP8BLK:
+        if (dma) return launch_a16_dma<AENC_FP8BLK, GLU>(g, grid, st);
+        k_group_a16_stream<AENC_FP8BLK, GLU><<<grid, AK_THREADS, 0, st>>>(g);
+        break;
+    case AENC_MXFP4:
+        if (dma) return launch_a16_dma<AENC_MXFP4, GLU>(g, grid, st);
+        k_group_a16_stream<AENC_MXFP4, GLU><<<grid, AK_THREADS, 0, st>>>(g);
+        break;
+    case AENC_FP8PC:
+        if (dma) return launch_a16_dma<AENC_FP8PC, GLU>(g, grid, st);
+        k_group_a16_stream<AENC_FP8PC, GLU><<<grid, AK_THREADS, 0, st>>>(g);
+        break;
     default: return PLOW_MOE_EUNSUPPORTED;
     }
     return 0;
