@@ -286,7 +286,7 @@ template <int ENC>
 struct DmLds {
     uint8_t x[DM_STAGES][16u * DmGeom<ENC>::KSTEP * 2u];
     DmWSlot ring[AK_WAVES][DM_STAGES];
-    float bsc[2][128]; /* block-fp8: the tile's weight block scales, all of K (K <= 16384) */
+    float bsc[4][2][128]; /* block-fp8: the weight block scales of the workgroup's tiles, all of K (K <= 16384) */
 };
 typedef __attribute__((address_space(3))) void dm_lds_void;
 __device__ __forceinline__ uint32_t dm_lds_off(const void* p) {
@@ -323,7 +323,17 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     /* direct loads per wave and step: weights 2 per stream, mxfp4 scales 1 per stream, rows 1 (first XL waves) */
     constexpr int NLW = NS * (ENC == AENC_MXFP4 ? 3 : 2);
     const uint32_t tiles = g.N / AK_BN;
-    const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
+    /* With plenty of tiles to go round and a short K loop, a workgroup takes TPW consecutive channel tiles
+     * of its expert and keeps the load rings running across them, which hides the ramp of the loop. meta[3E], the
+     * number of 64-row tiles, is at least the number of experts with rows. The grid has one workgroup per
+     * tile; the first E * tiles / TPW of them do the work (consecutive indices, so that they spread over
+     * all XCDs) and the rest leave at once. */
+    const uint32_t busy = (g.meta ? (uint32_t)g.meta[3u * g.E] : 1u) * tiles;
+    const bool short_k = g.K / DmGeom<ENC>::KSTEP <= 16u; /* a long K loop amortises its ramp by itself */
+    const uint32_t TPW = !short_k ? 1u : (busy >= 4096u && tiles % 4u == 0u) ? 4u : ((busy >= 2048u && tiles % 2u == 0u) ? 2u : 1u);
+    const uint32_t wpe = tiles / TPW; /* workgroups per expert */
+    if (blockIdx.x >= g.E * wpe) return;
+    const uint32_t e = g.E - 1u - blockIdx.x / wpe, ct = (blockIdx.x % wpe) * TPW; /* heavy (folded shared) expert first */
     const uint32_t cnt = g.meta ? (uint32_t)g.meta[g.E + e] : g.dense_rows;
     if (cnt == 0u) return;
     const uint64_t* wt = g.wtab ? g.wtab + (size_t)e * g.wcols : nullptr;
@@ -334,7 +344,7 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, k-chunk q */
-    const uint32_t K = g.K, KS = K / KSTEP, N = g.N;
+    const uint32_t K = g.K, KS = K / KSTEP, N = g.N, GS = TPW * KS; /* steps of a pass over all its tiles */
     const uint32_t chw = ct * AK_BN + wv * 16u;   /* this wave's first channel */
     const uint32_t wrow = ENC == AENC_BF16 ? K * 2u : (ENC == AENC_MXFP4 ? K / 2u : K); /* bytes per weight row */
 
@@ -357,15 +367,17 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
         /* mxfp4 scales: lane -> (row (lane & 31) >> 1, dword lane & 1) of the step's 8 bytes per row */
         if (ENC == AENC_MXFP4) ssrc[sidx] = sbase + (size_t)(row0 + ((lane & 31u) >> 1)) * (K / 32u) + (lane & 1u) * 4u;
         if (ENC == AENC_FP8PC) pcs[sidx] = (const float*)sbase + wr0 + chw + 4u * q;
-        if (ENC == AENC_FP8BLK) { /* the channel block's scale row goes to LDS once */
-            const float* bs = (const float*)sbase + (size_t)((ct * AK_BN + wr0) / 128u) * (K / 128u);
-            for (uint32_t i = threadIdx.x; i < K / 128u; i += AK_THREADS) L.bsc[sidx][i] = bs[i];
+        if (ENC == AENC_FP8BLK) { /* the channel blocks' scale rows go to LDS once */
+            for (uint32_t t = 0; t < TPW; t++) {
+                const float* bs = (const float*)sbase + (size_t)(((ct + t) * AK_BN + wr0) / 128u) * (K / 128u);
+                for (uint32_t i = threadIdx.x; i < K / 128u; i += AK_THREADS) L.bsc[t][sidx][i] = bs[i];
+            }
         }
     }
     const uint32_t swz = (c >> 1) & 7u;
     const uint32_t x_base = dm_lds_off(&L.x[0][0]);
     const uint32_t w_base = dm_lds_off(&L.ring[wv][0]);
-    const uint32_t b_base = dm_lds_off(&L.bsc[0][0]);
+    const uint32_t b_base = dm_lds_off(&L.bsc[0][0][0]);
     /* LDS position of logical piece P of activation row c */
     auto xpos = [&](uint32_t P) -> uint32_t { return NP >= 16u ? ((P & ~15u) | ((P ^ c) & 15u)) : (P ^ swz); };
 
@@ -387,38 +399,65 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
         bool valid = off < cnt;
         const uint32_t ai_c = valid ? (g.a_idx ? g.a_idx[r] : r) : PLOW_EXPERT_UNUSED;
         valid = ai_c != PLOW_EXPERT_UNUSED;
+        /* what the epilogues need from memory is read here, before the rings start: an ordinary load
+         * inside the stream would make the compiler wait for every outstanding direct load */
+        const uint32_t oi = valid ? (g.o_idx ? g.o_idx[r] : r) : PLOW_EXPERT_UNUSED;
+        const float gate = (!GLU && valid && g.gate) ? g.gate[r] : 1.0f;
+        float4 pc0[4], pc1[4];
+        if (ENC == AENC_FP8PC) {
+#pragma unroll
+            for (uint32_t t = 0; t < 4u; t++) {
+                pc0[t] = pc1[t] = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+                if (t < TPW) {
+                    pc0[t] = *(const float4*)(pcs[0] + t * AK_BN);
+                    if (GLU) pc1[t] = *(const float4*)(pcs[1] + t * AK_BN);
+                }
+            }
+        }
 
-        auto issue = [&](uint32_t S) {
-            const uint32_t st = S % DM_STAGES;
-            DmWSlot* slot = &L.ring[wv][st];
+        /* a use the compiler cannot move: its own wait for these loads lands here and not behind the
+         * first direct loads */
+        asm volatile("" ::"v"(oi), "v"(gate));
+        if (ENC == AENC_FP8PC) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) asm volatile("" ::"v"(pc0[t].x), "v"(pc0[t].w), "v"(pc1[t].x), "v"(pc1[t].w));
+        }
+
+        /* the load cursor walks (tile, step) in order; ring slots follow the running step count */
+        uint32_t ld_t = 0, ld_S = 0, ld_st = 0;
+        auto issue = [&]() {
+            DmWSlot* slot = &L.ring[wv][ld_st];
+            const size_t wofs = (size_t)ld_t * AK_BN * wrow + (size_t)ld_S * 128u;
 #pragma unroll
             for (int sidx = 0; sidx < NS; sidx++) {
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; j++)
-                    __builtin_amdgcn_global_load_lds((const void*)(wsrc[sidx][j] + (size_t)S * 128u),
+                    __builtin_amdgcn_global_load_lds((const void*)(wsrc[sidx][j] + wofs),
                                                      (dm_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, 0);
                 if (ENC == AENC_MXFP4)
-                    __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)S * 8u),
+                    __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)ld_t * AK_BN * (K / 32u) + (size_t)ld_S * 8u),
                                                      (dm_lds_void*)&slot->sc[sidx][0], 4, 0, 0);
             }
             if (wv < XL)
-                __builtin_amdgcn_global_load_lds((const void*)(xsrc + (size_t)S * XROW),
-                                                 (dm_lds_void*)&L.x[st][XRPL * wv * XROW], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((const void*)(xsrc + (size_t)ld_S * XROW),
+                                                 (dm_lds_void*)&L.x[ld_st][XRPL * wv * XROW], 16, 0, 0);
+            ld_st = ld_st + 1u == DM_STAGES ? 0u : ld_st + 1u;
+            if (++ld_S == KS) ld_S = 0u, ld_t++;
         };
         v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
         /* the row maps above are loaded (the count of outstanding loads starts at zero), and every wave
          * has left the pass before (its ring slots are free; the block scales are written) */
         DM_WAIT_BARRIER(0);
-        issue(0);
-        if (KS > 1u) issue(1);
-        for (uint32_t S = 0; S < KS; S++) {
-            /* loads return in order: step S has landed once at most step S + 1's are outstanding; after the
-             * barrier every wave's share of the rows is there and nobody reads step S - 1 any more */
-            if (S + 1u >= KS) DM_WAIT_BARRIER(0);
+        issue();
+        if (GS > 1u) issue();
+        uint32_t st = 0;
+        for (uint32_t G = 0, t = 0, S = 0; G < GS; G++) {
+            /* loads return in order: step G has landed once at most step G + 1's are outstanding; after the
+             * barrier every wave's share of the rows is there and nobody reads step G - 1 any more */
+            if (G + 1u >= GS) DM_WAIT_BARRIER(0);
             else if (wv < XL) DM_WAIT_BARRIER(NLW + 1);
             else DM_WAIT_BARRIER(NLW);
-            if (S + 2u < KS) issue(S + 2u);
-            const uint32_t st = S % DM_STAGES;
+            if (G + 2u < GS) issue();
             const uint32_t wb = w_base + st * (uint32_t)sizeof(DmWSlot), xb = x_base + st * (16u * XROW) + c * XROW;
             if (ENC == AENC_MXFP4) {
                 uint2 e0 = dm_read8(wb + 4096u + c * 8u), e1 = e0;
@@ -483,9 +522,9 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
 #pragma unroll
                 for (uint32_t j = 0; j < 4u; j++) xa[j] = dm_read16(xb + (xpos(8u * (j >> 1) + 2u * q + (j & 1u)) << 4));
                 if (ENC == AENC_FP8BLK) {
-                    sa = dm_read4(b_base + S * 4u);
+                    sa = dm_read4(b_base + t * 1024u + S * 4u);
                     sb = sa;
-                    if (GLU) sb = dm_read4(b_base + 512u + S * 4u);
+                    if (GLU) sb = dm_read4(b_base + t * 1024u + 512u + S * 4u);
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(da.r[0]), "+v"(da.r[1]), "+v"(db.r[0]), "+v"(db.r[1]), "+v"(sa), "+v"(sb));
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0]), "+v"(xa[1]), "+v"(xa[2]), "+v"(xa[3]));
@@ -508,18 +547,21 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
                     if (GLU) acc1 = t1;
                 }
             }
-        }
-        /* ---- epilogue: lane holds channels chw + 4q + i of row rb + c ---- */
-        if (valid) {
-            const uint32_t col = chw + 4u * q;
+            st = st + 1u == DM_STAGES ? 0u : st + 1u;
+            if (++S < KS) continue;
+            /* ---- a tile is done: lane holds channels chw + 128 t + 4q + i of row rb + c ---- */
+            const uint32_t tdone = t;
+            S = 0u, t++;
+            if (!valid) continue;
+            const uint32_t col = chw + tdone * AK_BN + 4u * q;
             if (ENC == AENC_FP8PC) {
+                float4 s0 = pc0[0], s1 = pc1[0];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    acc0[i] *= pcs[0][i];
-                    if (GLU) acc1[i] *= pcs[1][i];
-                }
+                for (uint32_t t2 = 1; t2 < 4u; t2++)
+                    if (tdone == t2) s0 = pc0[t2], s1 = pc1[t2];
+                acc0[0] *= s0.x, acc0[1] *= s0.y, acc0[2] *= s0.z, acc0[3] *= s0.w;
+                if (GLU) acc1[0] *= s1.x, acc1[1] *= s1.y, acc1[2] *= s1.z, acc1[3] *= s1.w;
             }
-            const uint32_t oi = g.o_idx ? g.o_idx[r] : r;
             if (oi != PLOW_EXPERT_UNUSED) {
                 if (GLU) {
                     uint2 o;
@@ -527,7 +569,6 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
                     o.y = (uint32_t)f2bf(moe_glu(acc0[2], acc1[2], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[3], acc1[3], g.act)) << 16);
                     *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
                 } else {
-                    const float gate = g.gate ? g.gate[r] : 1.0f;
                     const float y0 = gate * acc0[0], y1 = gate * acc0[1], y2 = gate * acc0[2], y3 = gate * acc0[3];
                     if (g.out_bf16) {
                         uint2 o;
@@ -539,6 +580,8 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
                     }
                 }
             }
+            acc0 = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+            acc1 = acc0;
         }
     }
 }
