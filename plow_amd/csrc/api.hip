@@ -34,6 +34,7 @@ struct PlowMoeCtx {
     /* slots per expert of the last align (op 84) on this context: ops 81 / 82 carry no row count and
      * pick their kernel form from it (0 = unknown: streaming form) */
     uint32_t rows_hint;
+    uint32_t slots_hint; /* T * k of the last align (op 84) on this context, 0 = unknown */
     int forced; /* -1 none, 0 stream, 1 tiled (segment entry point or environment) */
     int32_t* ws_meta;        /* [3 * WS_MAX_E + 1] */
     uint32_t* ws_row_token;  /* [WS_MAX_ROWS] */
@@ -154,6 +155,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, (uint64_t)i[0] * i[2] < (1ull << 31), "op 84: T * k overflows");
         if (!launch) return 0;
         c->rows_hint = (uint32_t)(((uint64_t)i[0] * i[2]) / i[1]);
+        c->slots_hint = i[0] * i[2];
         return launch_align((int32_t*)ten(in, T, 0), ten(in, T, 1), (uint32_t*)ten(in, T, 2),
                             (uint32_t*)ten(in, T, 3), (float*)ten(in, T, 4), i[0], i[1], i[2],
                             c->ws_chunk_hist, WS_MAX_CHUNKS, st);
@@ -225,6 +227,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4); g.a_idx = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.enc = enc; g.act = i[5];
             g.wcols = 3; g.wsel0 = 0; g.wsel1 = 1;
+            g.slots_hint = c->slots_hint;
             return launch_group_glu_a16(g, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85: encoding %u arm %u is not served", enc, arm);
@@ -263,6 +266,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.o_idx = (const uint32_t*)ten(in, T, 6); g.gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.enc = enc;
             g.wcols = 3; g.wsel0 = 2; g.wsel1 = 2;
+            g.slots_hint = c->slots_hint;
             return launch_group_down_a16(g, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 86: encoding %u arm %u is not served", enc, arm);
@@ -333,6 +337,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = c->ws_meta;
         g.N = N; g.K = K; g.E = E; g.enc = enc; g.act = act;
         g.wcols = pc ? 2u : 3u;
+        g.slots_hint = nslot;
         g.o_idx = c->ws_row_partidx;
         if (glu) {
             g.a_idx = c->ws_row_token;

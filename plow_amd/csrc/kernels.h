@@ -61,6 +61,7 @@ struct GroupA16 {
     uint32_t wcols, wsel0, wsel1; /* table width, column of the first / second weight stream */
     uint32_t wrow0, wrow1;        /* first weight row of each stream inside its tensor (fused gate_up) */
     uint32_t out_bf16, dense_rows;
+    uint32_t slots_hint; /* routed slots of the batch when the host knows them (0 = unknown): picks the kernel form */
     const void* wdirect[2]; /* used when wtab is NULL: the two weight tensors themselves (dense ops) */
 };
 int launch_group_glu_a16(const GroupA16& g, hipStream_t st);
