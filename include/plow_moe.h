@@ -80,6 +80,10 @@ enum {
     PLOW_DOP_MOE_GROUP_GLU_PF              = 85,
     PLOW_DOP_MOE_GROUP_DOWN_PF             = 86,
     PLOW_DOP_MOE_COMBINE_PF                = 87,
+    PLOW_DOP_MOE_GLU_MX                    = 150, /* decode, flat mxfp4 tensors [E][2I][K/2]     */
+    PLOW_DOP_MOE_DOWN_MX                   = 151,
+    PLOW_DOP_MOE_GLU_MX_PF                 = 152, /* the same on gathered rows (after 83 / 84)   */
+    PLOW_DOP_MOE_DOWN_MX_PF                = 153,
     PLOW_DOP_GEMM_F32                      = 180, /* router score: bf16 x bf16 -> f32 logits     */
     PLOW_DOP_QUANT_FP8_BLOCK128            = 184  /* 1x128 e4m3 activation quant                 */
 };

@@ -782,6 +782,137 @@ static void op_gemm(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* 
             C[(size_t)m * N + n] = orc_f2bf(dot_bf16_seq(A + (size_t)m * K, B + (size_t)n * K, K));
 }
 
+/* ---- ops 150 - 153: flat mxfp4 experts (plow runtime/cpu/dev/golden/moe.c) ------------------------
+ * Expert e of a [E][N][K/2] fp4 tensor starts at W + e*N*(K/2), its E8M0 bytes at S + e*N*(K/32), its
+ * bf16 bias at b + e*N. Gate / up rows of output n: layout 0 interleaved (2n, 2n + 1), layout 1 blocked
+ * (n, I + n) (moe.c:12-16). The bias is added in f32 before the activation (GLU) and before the gate
+ * multiply (DOWN). Activations 0 / 1 as everywhere on this path; the pair forms 2 / 3 poison. */
+static float mx_flat_dot(const uint8_t* We, const uint8_t* Se, uint32_t row, const float* a, uint32_t K, float* wf) {
+    decode_mxfp4_row(wf, We + (size_t)row * (K / 2u), K);
+    return dot_mxfp4(wf, Se + (size_t)row * (K / 32u), a, K);
+}
+
+/* 150: t0=fu[B*k][I] t1=x[B][K] t2=table t3=W_gu t4=S_gu t5=bias? i0=k i1=I i2=K i3=n_exp i4=layout
+ * i5=act i6=n_batch (0 = 1). Sentinel slot: nothing written (moe.c:21-60). */
+static void op_glu_mx(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* fu = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    const PlowMoeRoute* tab = TEN(in, T, 2);
+    const uint8_t* W = TEN(in, T, 3);
+    const uint8_t* S = TEN(in, T, 4);
+    const orc_bf16* bias = TEN(in, T, 5);
+    const uint32_t k = in->i[0], I = in->i[1], K = in->i[2], E = in->i[3], layout = in->i[4], act = in->i[5];
+    const uint32_t B = in->i[6] ? in->i[6] : 1u;
+    float* a = malloc((size_t)K * 4u);
+    float* wf = malloc((size_t)K * 4u);
+    uint32_t lo, hi, cur = ~0u;
+    own_range(B * k * I, slice, nblk, &lo, &hi);
+    for (uint32_t it = lo; it < hi; it++) {
+        const uint32_t s = it / I, n = it % I, e = tab[s].eid;
+        if (e >= E) continue;
+        if (cur != s) { decode_bf16_row(a, x + (size_t)(s / k) * K, K); cur = s; }
+        const uint8_t* We = W + (size_t)e * 2u * I * (K / 2u);
+        const uint8_t* Se = S + (size_t)e * 2u * I * (K / 32u);
+        const uint32_t rg = layout ? n : 2u * n, ru = layout ? I + n : 2u * n + 1u;
+        float g = mx_flat_dot(We, Se, rg, a, K, wf), u = mx_flat_dot(We, Se, ru, a, K, wf);
+        if (bias) { g += orc_bf2f(bias[(size_t)e * 2u * I + rg]); u += orc_bf2f(bias[(size_t)e * 2u * I + ru]); }
+        fu[(size_t)s * I + n] = orc_f2bf(glu(g, u, act));
+    }
+    free(a); free(wf);
+}
+
+/* 151: t0=part[B*k][H] t1=fu t2=table t3=W_d t4=S_d t5=bias? i0=k i1=H i2=I i3=n_exp i6=n_batch.
+ * part[s][h] = gate_s * (W_e[h] . fu[s] + b_e[h]); sentinel slot: zeros (moe.c:65-92). */
+static void op_down_mx(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    float* part = TEN(in, T, 0);
+    const orc_bf16* fu = TEN(in, T, 1);
+    const PlowMoeRoute* tab = TEN(in, T, 2);
+    const uint8_t* W = TEN(in, T, 3);
+    const uint8_t* S = TEN(in, T, 4);
+    const orc_bf16* bias = TEN(in, T, 5);
+    const uint32_t k = in->i[0], H = in->i[1], I = in->i[2], E = in->i[3], B = in->i[6] ? in->i[6] : 1u;
+    float* a = malloc((size_t)I * 4u);
+    float* wf = malloc((size_t)I * 4u);
+    uint32_t lo, hi, cur = ~0u;
+    own_range(B * k * H, slice, nblk, &lo, &hi);
+    for (uint32_t it = lo; it < hi; it++) {
+        const uint32_t s = it / H, h = it % H, e = tab[s].eid;
+        if (e >= E) { part[(size_t)s * H + h] = 0.0f; continue; }
+        if (cur != s) { decode_bf16_row(a, fu + (size_t)s * I, I); cur = s; }
+        float acc = mx_flat_dot(W + (size_t)e * H * (I / 2u), S + (size_t)e * H * (I / 32u), h, a, I, wf);
+        if (bias) acc += orc_bf2f(bias[(size_t)e * H + h]);
+        part[(size_t)s * H + h] = tab[s].gate * acc;
+    }
+    free(a); free(wf);
+}
+
+/* 152: t0=fu_g[rows][I] t1=xn2[T][K] t2=W_gu t3=S_gu t4=meta t5=row_token t6=bias? i0=I i1=K i2=n_exp
+ * i3=layout i5=act. Pad rows (token UNUSED) are skipped (moe.c:98-135). */
+static void op_glu_mx_pf(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* fu = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    const uint8_t* W = TEN(in, T, 2);
+    const uint8_t* S = TEN(in, T, 3);
+    const int32_t* meta = TEN(in, T, 4);
+    const uint32_t* row_token = TEN(in, T, 5);
+    const orc_bf16* bias = TEN(in, T, 6);
+    const uint32_t I = in->i[0], K = in->i[1], E = in->i[2], layout = in->i[3], act = in->i[5];
+    float* a = malloc((size_t)K * 4u);
+    float* wf = malloc((size_t)K * 4u);
+    uint32_t lo, hi;
+    own_range(E, slice, nblk, &lo, &hi);
+    for (uint32_t e = lo; e < hi; e++) {
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        const uint8_t* We = W + (size_t)e * 2u * I * (K / 2u);
+        const uint8_t* Se = S + (size_t)e * 2u * I * (K / 32u);
+        for (uint32_t r = r0; r < r0 + cnt; r++) {
+            const uint32_t tok = row_token[r];
+            if (tok == PLOW_EXPERT_UNUSED) continue;
+            decode_bf16_row(a, x + (size_t)tok * K, K);
+            for (uint32_t n = 0; n < I; n++) {
+                const uint32_t rg = layout ? n : 2u * n, ru = layout ? I + n : 2u * n + 1u;
+                float g = mx_flat_dot(We, Se, rg, a, K, wf), u = mx_flat_dot(We, Se, ru, a, K, wf);
+                if (bias) { g += orc_bf2f(bias[(size_t)e * 2u * I + rg]); u += orc_bf2f(bias[(size_t)e * 2u * I + ru]); }
+                fu[(size_t)r * I + n] = orc_f2bf(glu(g, u, act));
+            }
+        }
+    }
+    free(a); free(wf);
+}
+
+/* 153: t0=part[T*k][H] t1=fu_g t2=W_d t3=S_d t4=meta t5=bias? t6=row_partidx t7=row_gate i0=H i1=I
+ * i2=n_exp. part[row_partidx[r]][h] = row_gate[r] * (W_e[h] . fu_g[r] + b_e[h]); pad rows dropped
+ * (moe.c:140-174). */
+static void op_down_mx_pf(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    float* part = TEN(in, T, 0);
+    const orc_bf16* fu = TEN(in, T, 1);
+    const uint8_t* W = TEN(in, T, 2);
+    const uint8_t* S = TEN(in, T, 3);
+    const int32_t* meta = TEN(in, T, 4);
+    const orc_bf16* bias = TEN(in, T, 5);
+    const uint32_t* row_partidx = TEN(in, T, 6);
+    const float* row_gate = TEN(in, T, 7);
+    const uint32_t H = in->i[0], I = in->i[1], E = in->i[2];
+    float* a = malloc((size_t)I * 4u);
+    float* wf = malloc((size_t)I * 4u);
+    uint32_t lo, hi;
+    own_range(E, slice, nblk, &lo, &hi);
+    for (uint32_t e = lo; e < hi; e++) {
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        for (uint32_t r = r0; r < r0 + cnt; r++) {
+            const uint32_t pidx = row_partidx[r];
+            if (pidx == PLOW_EXPERT_UNUSED) continue;
+            decode_bf16_row(a, fu + (size_t)r * I, I);
+            for (uint32_t h = 0; h < H; h++) {
+                float acc = mx_flat_dot(W + (size_t)e * H * (I / 2u), S + (size_t)e * H * (I / 32u), h, a, I, wf);
+                if (bias) acc += orc_bf2f(bias[(size_t)e * H + h]);
+                part[(size_t)pidx * H + h] = row_gate[r] * acc;
+            }
+        }
+    }
+    free(a); free(wf);
+}
+
 /* ---- dispatch ---------------------------------------------------------------------------------- */
 
 typedef void (*op_fn)(const PlowDevInst*, uint32_t, uint32_t, void* const*);
@@ -806,6 +937,10 @@ static op_fn resolve(uint16_t op) {
     case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8: return op_pc_group_down;
     case PLOW_DOP_GEMM_GLU: return op_gemm_glu;
     case PLOW_DOP_GEMM: return op_gemm;
+    case PLOW_DOP_MOE_GLU_MX: return op_glu_mx;
+    case PLOW_DOP_MOE_DOWN_MX: return op_down_mx;
+    case PLOW_DOP_MOE_GLU_MX_PF: return op_glu_mx_pf;
+    case PLOW_DOP_MOE_DOWN_MX_PF: return op_down_mx_pf;
     default: return NULL;
     }
 }

@@ -28,6 +28,10 @@ OP_MOE_ALIGN_PF = 84
 OP_MOE_GROUP_GLU_PF = 85
 OP_MOE_GROUP_DOWN_PF = 86
 OP_MOE_COMBINE_PF = 87
+OP_MOE_GLU_MX = 150
+OP_MOE_DOWN_MX = 151
+OP_MOE_GLU_MX_PF = 152
+OP_MOE_DOWN_MX_PF = 153
 OP_GEMM_F32 = 180
 OP_QUANT_FP8_BLOCK128 = 184
 

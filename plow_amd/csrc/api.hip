@@ -41,6 +41,7 @@ struct PlowMoeCtx {
     uint32_t* ws_row_partidx;
     float* ws_row_gate;
     uint32_t* ws_chunk_hist; /* [WS_MAX_CHUNKS][n_exp] scratch of the multi-workgroup align */
+    uint64_t* ws_ftab;       /* [2][WS_MAX_E][3] pointer tables built for the flat-tensor ops (150 - 153) */
 };
 
 static int fail(PlowMoeCtx* c, int code, const char* fmt, ...) {
@@ -86,7 +87,8 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
                     hipMalloc(&c->ws_row_token, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
                     hipMalloc(&c->ws_row_partidx, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
                     hipMalloc(&c->ws_row_gate, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
-                    hipMalloc(&c->ws_chunk_hist, (size_t)WS_MAX_CHUNKS * WS_MAX_E * 4u) == hipSuccess;
+                    hipMalloc(&c->ws_chunk_hist, (size_t)WS_MAX_CHUNKS * WS_MAX_E * 4u) == hipSuccess &&
+                    hipMalloc(&c->ws_ftab, (size_t)2u * WS_MAX_E * 3u * 8u) == hipSuccess;
     (void)hipSetDevice(prev);
     if (!ok) {
         plow_moe_destroy(c);
@@ -103,6 +105,7 @@ extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) {
     (void)hipFree(ctx->ws_row_partidx);
     (void)hipFree(ctx->ws_row_gate);
     (void)hipFree(ctx->ws_chunk_hist);
+    (void)hipFree(ctx->ws_ftab);
     delete ctx;
 }
 
@@ -347,6 +350,61 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.a_idx = c->ws_row_partidx; g.gate = c->ws_row_gate;
         g.wsel0 = g.wsel1 = pc ? 1u : 2u;
         rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), g.wtab, g.stab, g.wcols, g.wsel0, nslot, E, N, st);
+        if (rc) return rc;
+        return launch_group_down_a16(g, st);
+    }
+    case PLOW_DOP_MOE_GLU_MX:
+    case PLOW_DOP_MOE_DOWN_MX:
+    case PLOW_DOP_MOE_GLU_MX_PF:
+    case PLOW_DOP_MOE_DOWN_MX_PF: {
+        /* flat mxfp4 tensors (plow runtime/common/dev_isa.h:1285-1335): expert e of [E][rows][K/2] starts
+         * at W + e*rows*(K/2), its E8M0 bytes at S + e*rows*(K/32), its bias at b + e*rows. The per-expert
+         * pointer tables the kernels read are built in the context workspace by a small launch. */
+        const bool glu = in->op == PLOW_DOP_MOE_GLU_MX || in->op == PLOW_DOP_MOE_GLU_MX_PF;
+        const bool pf = in->op == PLOW_DOP_MOE_GLU_MX_PF || in->op == PLOW_DOP_MOE_DOWN_MX_PF;
+        /* decode: t0 out t1 in t2 table t3 W t4 S t5 bias? i0=k i1=N i2=K i3=E i4=layout i5=act i6=B(0 = 1)
+         * prefill GLU:  t0 fu_g t1 xn2 t2 W t3 S t4 meta t5 row_token t6 bias?  i0=I i1=K i2=E i3=layout i5=act
+         * prefill DOWN: t0 part t1 fu_g t2 W t3 S t4 meta t5 bias? t6 row_partidx t7 row_gate  i0=H i1=I i2=E */
+        const uint32_t N = pf ? i[0] : i[1], K = pf ? i[1] : i[2], E = pf ? i[2] : i[3];
+        const uint32_t layout = glu ? (pf ? i[3] : i[4]) : 1u, act = glu ? i[5] : 0u;
+        const uint32_t kx = pf ? 0u : i[0], nslot = pf ? 0u : i[0] * (i[6] ? i[6] : 1u);
+        void* W = ten(in, T, pf ? 2 : 3);
+        void* S = ten(in, T, pf ? 3 : 4);
+        void* bias = ten(in, T, pf ? (glu ? 6 : 5) : 5);
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && W && S, "op %u: output, input, weight and scale tensors must be bound", (unsigned)in->op);
+        NEED(c, pf ? ten(in, T, 4) != nullptr : ten(in, T, 2) != nullptr, "op %u: %s must be bound", (unsigned)in->op, pf ? "t4 meta" : "t2 table");
+        NEED(c, !pf || (glu ? ten(in, T, 5) != nullptr : (ten(in, T, 6) && ten(in, T, 7))), "op %u: the row maps must be bound", (unsigned)in->op);
+        NEED(c, N && K && E && N % 128u == 0u && K % 128u == 0u, "op %u: N %u and K %u must be non-zero multiples of 128", (unsigned)in->op, N, K);
+        NEED(c, E <= WS_MAX_E && nslot <= WS_MAX_SLOTS && (pf || nslot), "op %u: %u slots / %u experts exceed the context workspace", (unsigned)in->op, nslot, E);
+        NEED(c, layout <= 1u, "op %u: layout %u is neither interleaved (0) nor blocked (1)", (unsigned)in->op, layout);
+        if (act > 1u) return fail(c, PLOW_MOE_EUNSUPPORTED, "op %u: activation %u (a pair form) is not served", (unsigned)in->op, act);
+        if (!launch) return 0;
+        const uint32_t rows = glu ? 2u * N : N; /* weight rows per expert */
+        uint64_t* wtab = c->ws_ftab;
+        uint64_t* stab = c->ws_ftab + (size_t)WS_MAX_E * 3u;
+        int rc = launch_flat_tables(wtab, stab, W, S, E, (size_t)rows * (K / 2u), (size_t)rows * (K / 32u), st);
+        if (rc) return rc;
+        GroupA16 g = {};
+        g.out = ten(in, T, 0); g.a = ten(in, T, 1);
+        g.wtab = wtab; g.stab = stab; g.wcols = 3; g.wsel0 = g.wsel1 = 0;
+        g.N = N; g.K = K; g.E = E; g.enc = PLOW_MOE_ENC_MXFP4; g.act = act;
+        g.bias = bias; g.bias_rows = rows;
+        if (glu) { g.wmul = layout ? 1u : 2u; g.wrow0 = 0; g.wrow1 = layout ? N : 1u; }
+        if (pf) {
+            g.meta = (const int32_t*)ten(in, T, 4);
+            g.slots_hint = c->slots_hint;
+            if (glu) { g.a_idx = (const uint32_t*)ten(in, T, 5); return launch_group_glu_a16(g, st); }
+            g.o_idx = (const uint32_t*)ten(in, T, 6); g.gate = (const float*)ten(in, T, 7);
+            return launch_group_down_a16(g, st);
+        }
+        /* slot-major: sort the slots by expert into the context workspace (row_token = slot / k) */
+        rc = launch_align(c->ws_meta, ten(in, T, 2), c->ws_row_token, c->ws_row_partidx, c->ws_row_gate,
+                          nslot / kx, E, kx, c->ws_chunk_hist, WS_MAX_CHUNKS, st);
+        if (rc) return rc;
+        g.meta = c->ws_meta; g.slots_hint = nslot; g.o_idx = c->ws_row_partidx;
+        if (glu) { g.a_idx = c->ws_row_token; return launch_group_glu_a16(g, st); }
+        g.a_idx = c->ws_row_partidx; g.gate = c->ws_row_gate;
+        rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), wtab, stab, 3u, 0u, nslot, E, N, st);
         if (rc) return rc;
         return launch_group_down_a16(g, st);
     }

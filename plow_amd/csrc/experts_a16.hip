@@ -105,15 +105,17 @@ __device__ __forceinline__ void ak_body(const GroupA16& g, uint32_t e, uint32_t 
     const uint64_t* stt = g.stab ? g.stab + (size_t)e * g.wcols : nullptr;
     const uint8_t* wbase0 = wt ? (const uint8_t*)(uintptr_t)wt[g.wsel0] : (const uint8_t*)g.wdirect[0];
     const uint8_t* wbase1 = wt ? (const uint8_t*)(uintptr_t)wt[g.wsel1] : (const uint8_t*)g.wdirect[1];
-    const uint8_t* w0 = wbase0 + (size_t)(ch + g.wrow0) * wrow;
-    const uint8_t* w1 = GLU ? wbase1 + (size_t)(ch + g.wrow1) * wrow : nullptr;
+    const uint32_t wmul = g.wmul ? g.wmul : 1u;
+    const uint32_t wr0 = ch * wmul + g.wrow0, wr1 = ch * wmul + g.wrow1; /* this lane's weight rows */
+    const uint8_t* w0 = wbase0 + (size_t)wr0 * wrow;
+    const uint8_t* w1 = GLU ? wbase1 + (size_t)wr1 * wrow : nullptr;
     const uint8_t* sb0 = stt ? (const uint8_t*)(uintptr_t)stt[g.wsel0] : nullptr;
     const uint8_t* sb1 = (GLU && stt) ? (const uint8_t*)(uintptr_t)stt[g.wsel1] : nullptr;
     const uint8_t *ms0 = nullptr, *ms1 = nullptr; /* mxfp4: this row's E8M0 bytes */
     const float *bs0 = nullptr, *bs1 = nullptr;   /* block-fp8: this channel block's scale row */
     if (ENC == AENC_MXFP4) {
-        ms0 = sb0 + (size_t)(ch + g.wrow0) * (K / 32u);
-        if (GLU) ms1 = sb1 + (size_t)(ch + g.wrow1) * (K / 32u);
+        ms0 = sb0 + (size_t)wr0 * (K / 32u);
+        if (GLU) ms1 = sb1 + (size_t)wr1 * (K / 32u);
     }
     if (ENC == AENC_FP8BLK) {
         bs0 = (const float*)sb0 + (size_t)((ct * AK_BN + g.wrow0) / 128u) * KB;
@@ -211,6 +213,14 @@ __device__ __forceinline__ void ak_body(const GroupA16& g, uint32_t e, uint32_t 
     /* ---- epilogue: lane holds channels ct*128 + wv*16 + 4q + i of row c ---- */
     if (!valid) return;
     const uint32_t col = ct * AK_BN + wv * 16u + 4u * q;
+    if (g.bias) { /* flat-tensor ops: per-expert bias rows laid out like the weight rows */
+        const bf16_t* be = (const bf16_t*)g.bias + (size_t)e * g.bias_rows;
+#pragma unroll
+        for (uint32_t i = 0; i < 4u; i++) {
+            acc0[i] += bf2f(be[(col + i) * wmul + g.wrow0]);
+            if (GLU) acc1[i] += bf2f(be[(col + i) * wmul + g.wrow1]);
+        }
+    }
     if (ENC == AENC_FP8PC) {
         const float* sc0 = (const float*)sb0 + g.wrow0 + col;
 #pragma unroll
@@ -347,6 +357,7 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     const uint32_t K = g.K, KS = K / KSTEP, N = g.N, GS = TPW * KS; /* steps of a pass over all its tiles */
     const uint32_t chw = ct * AK_BN + wv * 16u;   /* this wave's first channel */
     const uint32_t wrow = ENC == AENC_BF16 ? K * 2u : (ENC == AENC_MXFP4 ? K / 2u : K); /* bytes per weight row */
+    const uint32_t wmul = g.wmul ? g.wmul : 1u;
 
     /* weight loads: load j covers rows 8j .. 8j + 7 of a stream (lane = row lr of the group, piece p) */
     const uint32_t lr = lane >> 3, p = lane & 7u;
@@ -358,14 +369,15 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
         const uint32_t sel = sidx ? g.wsel1 : g.wsel0;
         const uint8_t* wbase = wt ? (const uint8_t*)(uintptr_t)wt[sel] : (const uint8_t*)g.wdirect[sidx];
         const uint8_t* sbase = stt ? (const uint8_t*)(uintptr_t)stt[sel] : nullptr;
-        const uint32_t wr0 = sidx ? g.wrow1 : g.wrow0, row0 = chw + wr0;
+        const uint32_t wr0 = sidx ? g.wrow1 : g.wrow0;
 #pragma unroll
         for (uint32_t j = 0; j < 2u; j++) {
             const uint32_t R = 8u * j + lr;
-            wsrc[sidx][j] = wbase + (size_t)(row0 + R) * wrow + ((p ^ ((R >> 1) & 7u)) << 4);
+            wsrc[sidx][j] = wbase + (size_t)((chw + R) * wmul + wr0) * wrow + ((p ^ ((R >> 1) & 7u)) << 4);
         }
         /* mxfp4 scales: lane -> (row (lane & 31) >> 1, dword lane & 1) of the step's 8 bytes per row */
-        if (ENC == AENC_MXFP4) ssrc[sidx] = sbase + (size_t)(row0 + ((lane & 31u) >> 1)) * (K / 32u) + (lane & 1u) * 4u;
+        if (ENC == AENC_MXFP4)
+            ssrc[sidx] = sbase + (size_t)((chw + ((lane & 31u) >> 1)) * wmul + wr0) * (K / 32u) + (lane & 1u) * 4u;
         if (ENC == AENC_FP8PC) pcs[sidx] = (const float*)sbase + wr0 + chw + 4u * q;
         if (ENC == AENC_FP8BLK) { /* the channel blocks' scale rows go to LDS once */
             for (uint32_t t = 0; t < TPW; t++) {
@@ -427,7 +439,7 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
         uint32_t ld_t = 0, ld_S = 0, ld_st = 0;
         auto issue = [&]() {
             DmWSlot* slot = &L.ring[wv][ld_st];
-            const size_t wofs = (size_t)ld_t * AK_BN * wrow + (size_t)ld_S * 128u;
+            const size_t wofs = (size_t)ld_t * AK_BN * wmul * wrow + (size_t)ld_S * 128u;
 #pragma unroll
             for (int sidx = 0; sidx < NS; sidx++) {
 #pragma unroll
@@ -435,7 +447,7 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
                     __builtin_amdgcn_global_load_lds((const void*)(wsrc[sidx][j] + wofs),
                                                      (dm_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, 0);
                 if (ENC == AENC_MXFP4)
-                    __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)ld_t * AK_BN * (K / 32u) + (size_t)ld_S * 8u),
+                    __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)ld_t * AK_BN * wmul * (K / 32u) + (size_t)ld_S * 8u),
                                                      (dm_lds_void*)&slot->sc[sidx][0], 4, 0, 0);
             }
             if (wv < XL)
@@ -616,7 +628,7 @@ static int launch_a16(const GroupA16& g, hipStream_t st) {
     const dim3 grid(g.E * (g.N / AK_BN));
     /* second form: needs whole steps of K (one 128-byte line per weight row) and the block scales of a
      * tile to fit its LDS table */
-    bool dma = a16_dma_form() && g.K <= 16384u &&
+    bool dma = a16_dma_form() && !g.bias && g.K <= 16384u &&
                g.K % (g.enc == AENC_MXFP4 ? 256u : 128u) == 0u && (g.enc == AENC_BF16 || g.stab);
     if (dma && g.slots_hint) {
         /* The second form fills a CU with one workgroup. With a short K loop and between one and three
@@ -658,6 +670,24 @@ static int launch_a16(const GroupA16& g, hipStream_t st) {
 
 int launch_group_glu_a16(const GroupA16& g, hipStream_t st) { return launch_a16<true>(g, st); }
 int launch_group_down_a16(const GroupA16& g, hipStream_t st) { return launch_a16<false>(g, st); }
+
+__global__ void k_flat_tables(uint64_t* wtab, uint64_t* stab, uint64_t W, uint64_t S, uint32_t E, uint64_t w_stride,
+                              uint64_t s_stride) {
+    const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= E) return;
+    for (int j = 0; j < 3; j++) {
+        wtab[(size_t)e * 3u + j] = W + e * w_stride;
+        stab[(size_t)e * 3u + j] = S + e * s_stride;
+    }
+}
+
+int launch_flat_tables(uint64_t* wtab, uint64_t* stab, const void* W, const void* S, uint32_t E, size_t w_stride,
+                       size_t s_stride, hipStream_t st) {
+    if (E == 0) return PLOW_MOE_EINVAL;
+    k_flat_tables<<<(E + 255u) / 256u, 256, 0, st>>>(wtab, stab, (uint64_t)(uintptr_t)W, (uint64_t)(uintptr_t)S, E,
+                                                     (uint64_t)w_stride, (uint64_t)s_stride);
+    return 0;
+}
 
 /* Slot-major ops: zero part[s][*] of every slot that no expert serves (sentinel id or a null weight
  * base), which the reference's decode DOWN bodies do (plow runtime/cpu/dev/golden/moe.c:76-80). */

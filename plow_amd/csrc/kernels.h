@@ -62,10 +62,20 @@ struct GroupA16 {
     uint32_t wrow0, wrow1;        /* first weight row of each stream inside its tensor (fused gate_up) */
     uint32_t out_bf16, dense_rows;
     uint32_t slots_hint; /* routed slots of the batch when the host knows them (0 = unknown): picks the kernel form */
+    /* weight row of output channel n in stream s: n * wmul + wrow_s (wmul 0 reads as 1). Blocked gate | up
+     * rows: wmul 1, wrow1 = N; interleaved (2n, 2n + 1): wmul 2, wrow1 = 1 */
+    uint32_t wmul;
+    /* per-expert bf16 bias rows laid out like the weight rows ([E][bias_rows]), added in f32 before the
+     * activation (GLU) or before the gate multiply (DOWN); NULL = none */
+    const void* bias;
+    uint32_t bias_rows;
     const void* wdirect[2]; /* used when wtab is NULL: the two weight tensors themselves (dense ops) */
 };
 int launch_group_glu_a16(const GroupA16& g, hipStream_t st);
 int launch_group_down_a16(const GroupA16& g, hipStream_t st);
+/* wtab / stab rows {p, p, p} for the experts of one flat tensor: p = W + e * w_stride, S + e * s_stride */
+int launch_flat_tables(uint64_t* wtab, uint64_t* stab, const void* W, const void* S, uint32_t E, size_t w_stride,
+                       size_t s_stride, hipStream_t st);
 int launch_zero_skipped(float* part, const void* table, const uint64_t* wtab, const uint64_t* stab,
                         uint32_t wcols, uint32_t wsel, uint32_t nslot, uint32_t E, uint32_t H, hipStream_t st);
 

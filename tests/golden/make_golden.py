@@ -4,7 +4,7 @@ mounted plow tree into oracle/_ref/libplow_ref.so (scalar golden tier).
 Run where the plow tree is mounted:   make -C oracle ref && python tests/golden/make_golden.py
 The fixtures hold inputs and expected outputs only; tests/test_golden.py replays them through the
 in-repo oracle on any machine. Reference op numbers used: 83/84/87 routing, 180 router score,
-75/76 bf16 grouped experts, 150/151 flat mxfp4 decode experts, 65/66 per-channel fp8 decode
+75/76 bf16 grouped experts, 150-153 flat mxfp4 experts, 65/66 per-channel fp8 decode
 experts, 32 per-row activation quant, 20/8 dense GLU / GEMM.
 """
 import os
@@ -171,6 +171,29 @@ def main():
             run(abi.inst(32, t=[0, 1, 2, 3, 4], i=[M, K, act]), [xq, x, sc, gate, up], nblk=2)
             out.update({f"quant32f/{act}/{K}/gate": gate, f"quant32f/{act}/{K}/up": up, f"quant32f/{act}/{K}/x": x,
                         f"quant32f/{act}/{K}/xq": xq, f"quant32f/{act}/{K}/scale": sc})
+
+    # --- flat mxfp4 ops again (drawn last): interleaved layout with per-expert biases (150 / 151), and
+    # the gathered-row twins 152 / 153 after 84, on the mxdec weights above ----------------------------
+    Wgu, Sgu, Wd, Sd = out["mxdec/Wgu"], out["mxdec/Sgu"], out["mxdec/Wd"], out["mxdec/Sd"]
+    E, I, K = Wgu.shape[0], Wgu.shape[1] // 2, Wgu.shape[2] * 2
+    k, B = 2, 3
+    x = out["mxdec/x"]
+    tab = np.zeros(B * k, dtype=ol.ROUTE_DT)
+    tab["eid"], tab["gate"] = out["mxdec/table"][:, 0], out["mxdec/table"][:, 1].view(np.float32)
+    bgu, bd = cases.randn_bf16(r, (E, 2 * I), 0.5), cases.randn_bf16(r, (E, K), 0.5)
+    fu = np.zeros((B * k, I), np.uint16)
+    run(abi.inst(150, t=[0, 1, 2, 3, 4, 5], i=[k, I, K, E, 0, 0, B]), [fu, x, tab, Wgu, Sgu, bgu], nblk=2)
+    part = np.full((B * k, K), 9.0, np.float32)
+    run(abi.inst(151, t=[0, 1, 2, 3, 4, 5], i=[k, K, I, E, 0, 0, B]), [part, fu, tab, Wd, Sd, bd], nblk=2)
+    out.update({"mxflat/bias_gu": bgu, "mxflat/bias_d": bd, "mxflat/fu_l0_bias_gelu": fu, "mxflat/part_bias": part})
+    al = cases.align_arrays(tab, B, E, k)
+    run(cases.align_inst(B, E, k), al)
+    rows = int(al[0][3 * E]) * abi.MPF_BM
+    fug = np.zeros((rows, I), np.uint16)
+    run(abi.inst(152, t=[0, 1, 2, 3, 4, 5], i=[I, K, E, 1, 0, 1]), [fug, x, Wgu, Sgu, al[0], al[2]], nblk=3)
+    partg = np.full((B * k, K), 9.0, np.float32)
+    run(abi.inst(153, t=[0, 1, 2, 3, 4, None, 6, 7], i=[K, I, E]), [partg, fug, Wd, Sd, al[0], None, al[3], al[4]], nblk=3)
+    out.update({"mxflat/pf_fu": fug, "mxflat/pf_part": partg})
 
     path = os.path.join(HERE, "plow_cpu_golden.npz")
     np.savez_compressed(path, **out)

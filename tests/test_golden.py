@@ -111,6 +111,37 @@ def test_mxfp4_decode_experts(oracle):
     assert np.array_equal(part.view(np.uint32), G["mxdec/part"].view(np.uint32))
 
 
+def test_flat_mxfp4_ops(oracle):
+    """Reference ops 150 - 153 under their own numbers: blocked and interleaved gate / up rows, per-expert
+    biases, and the gathered-row twins after op 84."""
+    Wgu, Sgu = np.ascontiguousarray(G["mxdec/Wgu"]), np.ascontiguousarray(G["mxdec/Sgu"])
+    Wd, Sd = np.ascontiguousarray(G["mxdec/Wd"]), np.ascontiguousarray(G["mxdec/Sd"])
+    x, tab = G["mxdec/x"], as_route(G["mxdec/table"])
+    E, I2, K2 = Wgu.shape
+    I, K, B, k = I2 // 2, K2 * 2, x.shape[0], 2
+    fu = np.zeros((B * k, I), np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[k, I, K, E, 1, 1, B]), [fu, x, tab, Wgu, Sgu], 2)
+    assert np.array_equal(fu, G["mxdec/fu"])
+    part = np.full((B * k, K), 9.0, np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_DOWN_MX, t=[0, 1, 2, 3, 4], i=[k, K, I, E, 0, 0, B]), [part, fu, tab, Wd, Sd], 2)
+    assert np.array_equal(part.view(np.uint32), G["mxdec/part"].view(np.uint32))
+    bgu, bd = G["mxflat/bias_gu"], G["mxflat/bias_d"]
+    run(oracle, abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4, 5], i=[k, I, K, E, 0, 0, B]), [fu, x, tab, Wgu, Sgu, bgu], 3)
+    assert np.array_equal(fu, G["mxflat/fu_l0_bias_gelu"])
+    part[:] = 9.0
+    run(oracle, abi.inst(abi.OP_MOE_DOWN_MX, t=[0, 1, 2, 3, 4, 5], i=[k, K, I, E, 0, 0, B]), [part, fu, tab, Wd, Sd, bd], 3)
+    assert np.array_equal(part.view(np.uint32), G["mxflat/part_bias"].view(np.uint32))
+    al = cases.align_arrays(tab, B, E, k)
+    run(oracle, cases.align_inst(B, E, k), al, 1)
+    fug = np.zeros_like(G["mxflat/pf_fu"])
+    run(oracle, abi.inst(abi.OP_MOE_GLU_MX_PF, t=[0, 1, 2, 3, 4, 5], i=[I, K, E, 1, 0, 1]), [fug, x, Wgu, Sgu, al[0], al[2]], 3)
+    assert np.array_equal(fug, G["mxflat/pf_fu"])
+    partg = np.full((B * k, K), 9.0, np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_DOWN_MX_PF, t=[0, 1, 2, 3, 4, None, 6, 7], i=[K, I, E]),
+        [partg, fug, Wd, Sd, al[0], None, al[3], al[4]], 3)
+    assert np.array_equal(partg.view(np.uint32), G["mxflat/pf_part"].view(np.uint32))
+
+
 def test_per_channel_fp8_decode_experts(oracle):
     gu8, d8 = np.ascontiguousarray(G["pcdec/gu8"]), np.ascontiguousarray(G["pcdec/d8"])
     sgu, sd = np.ascontiguousarray(G["pcdec/sgu"]), np.ascontiguousarray(G["pcdec/sd"])

@@ -228,3 +228,76 @@ def test_dense_ops_against_oracle(moe, oracle):
     yg = y_d.cpu().numpy().view(np.uint16)
     assert np.all(yg[0] == 0)
     close(ol.bf2f(yg[1:]), ol.bf2f(y_h[1:]), "dense y")
+
+
+@pytest.mark.parametrize("layout,with_bias,act", [(1, False, 1), (0, True, 0), (0, False, 1), (1, True, 1)])
+def test_flat_mxfp4_ops(moe, oracle, layout, with_bias, act):
+    """Reference ops 150 - 153 (flat [E][rows][K/2] tensors, blocked or interleaved gate / up rows, optional
+    per-expert bias): slot-major decode incl. a sentinel slot, then the gathered-row twins after op 84."""
+    print(f"[case] flat mxfp4 layout={layout} bias={with_bias} act={act}", flush=True)
+    r = cases.rng_of(70 + 2 * layout + int(with_bias))
+    E, I, K, k, B = 5, 128, 512, 2, 9
+    Wgu = r.integers(0, 256, (E, 2 * I, K // 2), dtype=np.uint8)
+    Sgu = r.integers(120, 128, (E, 2 * I, K // 32), dtype=np.uint8)
+    Wd = r.integers(0, 256, (E, K, I // 2), dtype=np.uint8)
+    Sd = r.integers(120, 128, (E, K, I // 32), dtype=np.uint8)
+    bgu = cases.randn_bf16(r, (E, 2 * I), 2.0) if with_bias else None
+    bd = cases.randn_bf16(r, (E, K), 2.0) if with_bias else None
+    x = cases.randn_bf16(r, (B, K), 1.0)
+    tab = np.zeros(B * k, dtype=ol.ROUTE_DT)
+    tab["eid"] = r.integers(0, E, B * k)
+    tab["eid"][3] = abi.EXPERT_UNUSED
+    tab["gate"] = (r.random(B * k) + 0.1).astype(np.float32)
+    tb = 5 if with_bias else None
+    glu = abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4, tb], i=[k, I, K, E, layout, act, B])
+    down = abi.inst(abi.OP_MOE_DOWN_MX, t=[0, 1, 2, 3, 4, tb], i=[k, K, I, E, 0, 0, B])
+    fu_h = np.full((B * k, I), 0x1234, np.uint16)
+    part_h = np.full((B * k, K), 9.0, np.float32)
+    ol.run(oracle.plow_oracle_exec, glu, ol.table_of([fu_h, x, tab, Wgu, Sgu, bgu]), 4)
+    ol.run(oracle.plow_oracle_exec, down, ol.table_of([part_h, fu_h, tab, Wd, Sd, bd]), 4)
+    d = {n: to_dev(a) for n, a in dict(x=x, tab=tab, Wgu=Wgu, Sgu=Sgu, Wd=Wd, Sd=Sd, bgu=bgu, bd=bd, fu_h=fu_h).items()}
+    fu_d = torch.full((B * k, I), 0x1234, dtype=torch.int16, device="cuda")
+    part_d = torch.full((B * k, K), 9.0, dtype=torch.float32, device="cuda")
+    moe.exec(glu, dev_table([fu_d, d["x"], d["tab"], d["Wgu"], d["Sgu"], d["bgu"]]))
+    moe.exec(down, dev_table([part_d, d["fu_h"], d["tab"], d["Wd"], d["Sd"], d["bd"]]))
+    torch.cuda.synchronize()
+    fu_g = fu_d.cpu().numpy().view(np.uint16)
+    served = tab["eid"] < E
+    assert np.all(fu_g[~served] == 0x1234)
+    close(ol.bf2f(fu_g[served]), ol.bf2f(fu_h[served]), "fu")
+    part_g = part_d.cpu().numpy()
+    assert np.all(part_g[~served] == 0.0)
+    close(part_g, part_h, "part", mean_rel=1e-4, max_frac=1e-4)
+    # gathered rows: 84, then 152 / 153 on the same table
+    al = cases.align_arrays(tab, B, E, k)
+    ol.run(oracle.plow_oracle_exec, cases.align_inst(B, E, k), ol.table_of(al), 1)
+    rows = len(al[2])
+    glu_pf = abi.inst(abi.OP_MOE_GLU_MX_PF, t=[0, 1, 2, 3, 4, 5, 6 if with_bias else None], i=[I, K, E, layout, 0, act])
+    down_pf = abi.inst(abi.OP_MOE_DOWN_MX_PF, t=[0, 1, 2, 3, 4, 5 if with_bias else None, 6, 7], i=[K, I, E])
+    fug_h = np.full((rows, I), 0x1234, np.uint16)
+    partg_h = np.full((B * k, K), 9.0, np.float32)
+    ol.run(oracle.plow_oracle_exec, glu_pf, ol.table_of([fug_h, x, Wgu, Sgu, al[0], al[2], bgu]), 4)
+    ol.run(oracle.plow_oracle_exec, down_pf, ol.table_of([partg_h, fug_h, Wd, Sd, al[0], bd, al[3], al[4]]), 4)
+    meta_d, rt_d, rp_d, rg_d, fug_hd = to_dev(al[0]), to_dev(al[2]), to_dev(al[3]), to_dev(al[4]), to_dev(fug_h)
+    fug_d = torch.full((rows, I), 0x1234, dtype=torch.int16, device="cuda")
+    partg_d = torch.full((B * k, K), 9.0, dtype=torch.float32, device="cuda")
+    moe.exec(glu_pf, dev_table([fug_d, d["x"], d["Wgu"], d["Sgu"], meta_d, rt_d, d["bgu"]]))
+    moe.exec(down_pf, dev_table([partg_d, fug_hd, d["Wd"], d["Sd"], meta_d, d["bd"], rp_d, rg_d]))
+    torch.cuda.synchronize()
+    live = al[2] != abi.EXPERT_UNUSED
+    fug_g = fug_d.cpu().numpy().view(np.uint16)
+    assert np.all(fug_g[~live] == 0x1234)                    # pad rows: nothing written
+    close(ol.bf2f(fug_g[live]), ol.bf2f(fug_h[live]), "fu_g")
+    partg_g = partg_d.cpu().numpy()
+    assert np.all(partg_g[~served] == 9.0)                   # no row maps to a sentinel slot: untouched
+    close(partg_g[served], partg_h[served], "part_g", mean_rel=1e-4, max_frac=1e-4)
+
+
+def test_flat_mxfp4_refusals(moe):
+    t = dev_table([torch.zeros(8, device="cuda")] * 8)
+    ok = abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 1, 1, 3])
+    assert moe.check(ok, t) == 0
+    assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 1, 3, 3]), t) == abi.E_UNSUPPORTED
+    assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 2, 1, 3]), t) == abi.E_INVAL
+    assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 64, 256, 4, 1, 1, 3]), t) == abi.E_INVAL
+    assert moe.check(abi.inst(abi.OP_MOE_DOWN_MX_PF, t=[0, 1, 2, 3, 4], i=[256, 128, 4]), t) == abi.E_INVAL
