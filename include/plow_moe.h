@@ -73,6 +73,8 @@ enum {
     PLOW_DOP_MOE_ROUTER_TOPK               = 56,
     PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8      = 65,  /* decode, per-channel fp8, fused gate_up table */
     PLOW_DOP_MOE_EXPERT_DOWN_GEMMA_FP8     = 66,
+    PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF        = 75,  /* grouped, bf16, fused table ewt[E][2]        */
+    PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF       = 76,
     PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF_W8A8   = 81,  /* grouped, per-channel fp8 x per-row fp8      */
     PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8  = 82,
     PLOW_DOP_MOE_ROUTER_TOPK_PF            = 83,

@@ -782,6 +782,69 @@ static void op_gemm(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* 
             C[(size_t)m * N + n] = orc_f2bf(dot_bf16_seq(A + (size_t)m * K, B + (size_t)n * K, K));
 }
 
+/* ---- ops 75 / 76: bf16 grouped experts over the fused table ewt[E][2] = {gate_up [2I][H], down [H][I]}
+ * (plow runtime/cpu/dev/golden/moe_gemma.c:244-302). 75: t0=fu_g t1=xn2 t2=ewt t3=meta t4=row_token
+ * i0=I i1=H i2=n_exp i5=act; 76: t0=part t1=fu_g t2=ewt t3=meta t4=row_partidx t5=row_gate i0=H i1=I
+ * i2=n_exp. Pad rows are skipped; a null table entry skips the expert. f32 accumulation in k order. */
+static void op_group_glu_gemma(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* fu = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    const uint64_t* ewt = TEN(in, T, 2);
+    const int32_t* meta = TEN(in, T, 3);
+    const uint32_t* row_token = TEN(in, T, 4);
+    const uint32_t I = in->i[0], H = in->i[1], E = in->i[2], act = in->i[5];
+    float* a = malloc((size_t)H * 4u);
+    float* wg = malloc((size_t)H * 4u);
+    float* wu = malloc((size_t)H * 4u);
+    uint32_t lo, hi;
+    own_range(E, slice, nblk, &lo, &hi);
+    for (uint32_t e = lo; e < hi; e++) {
+        const orc_bf16* W = (const orc_bf16*)(uintptr_t)ewt[(size_t)e * 2u];
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        if (!W) continue;
+        for (uint32_t n = 0; n < I; n++) {
+            decode_bf16_row(wg, W + (size_t)n * H, H);
+            decode_bf16_row(wu, W + (size_t)(I + n) * H, H);
+            for (uint32_t r = r0; r < r0 + cnt; r++) {
+                const uint32_t tok = row_token[r];
+                if (tok == PLOW_EXPERT_UNUSED) continue;
+                decode_bf16_row(a, x + (size_t)tok * H, H);
+                fu[(size_t)r * I + n] = orc_f2bf(glu(dot_seq(wg, a, H), dot_seq(wu, a, H), act));
+            }
+        }
+    }
+    free(a); free(wg); free(wu);
+}
+
+static void op_group_down_gemma(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    float* part = TEN(in, T, 0);
+    const orc_bf16* fu = TEN(in, T, 1);
+    const uint64_t* ewt = TEN(in, T, 2);
+    const int32_t* meta = TEN(in, T, 3);
+    const uint32_t* row_partidx = TEN(in, T, 4);
+    const float* row_gate = TEN(in, T, 5);
+    const uint32_t H = in->i[0], I = in->i[1], E = in->i[2];
+    float* a = malloc((size_t)I * 4u);
+    float* wd = malloc((size_t)I * 4u);
+    uint32_t lo, hi;
+    own_range(E, slice, nblk, &lo, &hi);
+    for (uint32_t e = lo; e < hi; e++) {
+        const orc_bf16* W = (const orc_bf16*)(uintptr_t)ewt[(size_t)e * 2u + 1u];
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        if (!W) continue;
+        for (uint32_t h = 0; h < H; h++) {
+            decode_bf16_row(wd, W + (size_t)h * I, I);
+            for (uint32_t r = r0; r < r0 + cnt; r++) {
+                const uint32_t pidx = row_partidx[r];
+                if (pidx == PLOW_EXPERT_UNUSED) continue;
+                decode_bf16_row(a, fu + (size_t)r * I, I);
+                part[(size_t)pidx * H + h] = row_gate[r] * dot_seq(wd, a, I);
+            }
+        }
+    }
+    free(a); free(wd);
+}
+
 /* ---- ops 150 - 153: flat mxfp4 experts (plow runtime/cpu/dev/golden/moe.c) ------------------------
  * Expert e of a [E][N][K/2] fp4 tensor starts at W + e*N*(K/2), its E8M0 bytes at S + e*N*(K/32), its
  * bf16 bias at b + e*N. Gate / up rows of output n: layout 0 interleaved (2n, 2n + 1), layout 1 blocked
@@ -937,6 +1000,8 @@ static op_fn resolve(uint16_t op) {
     case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8: return op_pc_group_down;
     case PLOW_DOP_GEMM_GLU: return op_gemm_glu;
     case PLOW_DOP_GEMM: return op_gemm;
+    case PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF: return op_group_glu_gemma;
+    case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF: return op_group_down_gemma;
     case PLOW_DOP_MOE_GLU_MX: return op_glu_mx;
     case PLOW_DOP_MOE_DOWN_MX: return op_down_mx;
     case PLOW_DOP_MOE_GLU_MX_PF: return op_glu_mx_pf;

@@ -21,6 +21,8 @@ OP_MOE_GROUP_DOWN_FP8_BLK = 49
 OP_MOE_ROUTER_TOPK = 56
 OP_MOE_EXPERT_GLU_GEMMA_FP8 = 65
 OP_MOE_EXPERT_DOWN_GEMMA_FP8 = 66
+OP_MOE_GROUP_GLU_GEMMA_PF = 75
+OP_MOE_GROUP_DOWN_GEMMA_PF = 76
 OP_MOE_GROUP_GLU_GEMMA_PF_W8A8 = 81
 OP_MOE_GROUP_DOWN_GEMMA_PF_W8A8 = 82
 OP_MOE_ROUTER_TOPK_PF = 83

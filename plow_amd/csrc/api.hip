@@ -353,6 +353,33 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         if (rc) return rc;
         return launch_group_down_a16(g, st);
     }
+    case PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF:
+    case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF: {
+        /* bf16 grouped experts over the fused table ewt[E][2] = {gate_up [2I][H], down [H][I]}
+         * (plow runtime/common/dev_isa.h:616-628): 75 t0=fu_g t1=xn2 t2=ewt t3=meta t4=row_token i0=I i1=H
+         * i2=E i5=act; 76 t0=part t1=fu_g t2=ewt t3=meta t4=row_partidx t5=row_gate i0=H i1=I i2=E */
+        const bool glu = in->op == PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF;
+        const uint32_t N = i[0], K = i[1], E = i[2];
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && (glu || ten(in, T, 5)),
+             "op %u: output, input, ewt, meta and the row maps must be bound", (unsigned)in->op);
+        NEED(c, N && K && E && N % 128u == 0u && K % 128u == 0u, "op %u: N %u and K %u must be non-zero multiples of 128", (unsigned)in->op, N, K);
+        NEED(c, !glu || i[5] <= 1u, "op 75: activation %u is not served", i[5]);
+        if (!launch) return 0;
+        GroupA16 g = {};
+        g.out = ten(in, T, 0); g.a = ten(in, T, 1);
+        g.wtab = (const uint64_t*)ten(in, T, 2); g.wcols = 2;
+        g.meta = (const int32_t*)ten(in, T, 3);
+        g.N = N; g.K = K; g.E = E; g.enc = PLOW_MOE_ENC_BF16; g.act = glu ? i[5] : 0u;
+        g.slots_hint = c->slots_hint;
+        if (glu) {
+            g.a_idx = (const uint32_t*)ten(in, T, 4);
+            g.wsel0 = g.wsel1 = 0; g.wrow1 = N;
+            return launch_group_glu_a16(g, st);
+        }
+        g.o_idx = (const uint32_t*)ten(in, T, 4); g.gate = (const float*)ten(in, T, 5);
+        g.wsel0 = g.wsel1 = 1;
+        return launch_group_down_a16(g, st);
+    }
     case PLOW_DOP_MOE_GLU_MX:
     case PLOW_DOP_MOE_DOWN_MX:
     case PLOW_DOP_MOE_GLU_MX_PF:

@@ -90,6 +90,26 @@ def test_bf16_grouped_experts(oracle, act):
     assert np.array_equal(part.view(np.uint32), G[f"bf16grp/part_act{act}"].view(np.uint32))
 
 
+@pytest.mark.parametrize("act", [0, 1])
+def test_bf16_grouped_experts_fused_table(oracle, act):
+    """Reference ops 75 / 76 under their own numbers, over the fused table ewt[E][2]."""
+    logit, x = G["bf16grp/logit"], G["bf16grp/x"]
+    gu, dn = np.ascontiguousarray(G["bf16grp/gate_up"]), np.ascontiguousarray(G["bf16grp/down"])
+    E, I2, H = gu.shape
+    I, T, k = I2 // 2, x.shape[0], 2
+    table = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    run(oracle, cases.route_inst(E, k, T, 8, False, route_scale=1.0), [table, logit, None, None])
+    al = cases.align_arrays(table, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    ewt = np.array([[gu[e].ctypes.data, dn[e].ctypes.data] for e in range(E)], dtype=np.uint64)
+    fu = np.zeros((al[2].shape[0], I), np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_GEMMA_PF, t=[0, 1, 2, 3, 4], i=[I, H, E, 0, 0, act]), [fu, x, ewt, al[0], al[2]], 3)
+    assert np.array_equal(fu, G[f"bf16grp/fu_act{act}"])
+    part = np.zeros((T * k, H), np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_GEMMA_PF, t=[0, 1, 2, 3, 4, 5], i=[H, I, E]), [part, fu, ewt, al[0], al[3], al[4]], 3)
+    assert np.array_equal(part.view(np.uint32), G[f"bf16grp/part_act{act}"].view(np.uint32))
+
+
 def test_mxfp4_decode_experts(oracle):
     """Reference flat ops 150/151 == ops 48/49 at enc 2 over per-expert pointers into the flat tensor."""
     Wgu, Sgu = np.ascontiguousarray(G["mxdec/Wgu"]), np.ascontiguousarray(G["mxdec/Sgu"])

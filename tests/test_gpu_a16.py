@@ -301,3 +301,47 @@ def test_flat_mxfp4_refusals(moe):
     assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 2, 1, 3]), t) == abi.E_INVAL
     assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 64, 256, 4, 1, 1, 3]), t) == abi.E_INVAL
     assert moe.check(abi.inst(abi.OP_MOE_DOWN_MX_PF, t=[0, 1, 2, 3, 4], i=[256, 128, 4]), t) == abi.E_INVAL
+
+
+@pytest.mark.parametrize("act", [0, 1])
+def test_bf16_grouped_fused_table_ops(moe, oracle, act):
+    """Reference ops 75 / 76 (bf16, fused table ewt[E][2]) on gathered rows with a non-resident expert and
+    an expert of more than 16 rows."""
+    print(f"[case] ops 75/76 act={act}", flush=True)
+    r = cases.rng_of(90 + act)
+    E, I, H, k, T = 5, 256, 384, 2, 40
+    gu = [cases.randn_bf16(r, (2 * I, H), 0.05) for _ in range(E)]
+    dn = [cases.randn_bf16(r, (H, I), 0.05) for _ in range(E)]
+    x = cases.randn_bf16(r, (T, H), 1.0)
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    tab["eid"] = np.where(r.random(T * k) < 0.5, 1, r.integers(0, E, T * k))     # expert 1 gets many rows
+    tab["eid"][5] = abi.EXPERT_UNUSED
+    tab["gate"] = (r.random(T * k) + 0.1).astype(np.float32)
+    al = cases.align_arrays(tab, T, E, k)
+    ol.run(oracle.plow_oracle_exec, cases.align_inst(T, E, k), ol.table_of(al), 1)
+    rows = len(al[2])
+    ewt_h = np.array([[g.ctypes.data, d.ctypes.data] for g, d in zip(gu, dn)], dtype=np.uint64)
+    ewt_h[3] = 0
+    glu = abi.inst(abi.OP_MOE_GROUP_GLU_GEMMA_PF, t=[0, 1, 2, 3, 4], i=[I, H, E, 0, 0, act])
+    down = abi.inst(abi.OP_MOE_GROUP_DOWN_GEMMA_PF, t=[0, 1, 2, 3, 4, 5], i=[H, I, E])
+    fu_h = np.full((rows, I), 0x1234, np.uint16)
+    part_h = np.full((T * k, H), 9.0, np.float32)
+    ol.run(oracle.plow_oracle_exec, glu, ol.table_of([fu_h, x, ewt_h, al[0], al[2]]), 4)
+    ol.run(oracle.plow_oracle_exec, down, ol.table_of([part_h, fu_h, ewt_h, al[0], al[3], al[4]]), 4)
+    gd, dd = [to_dev(a) for a in gu], [to_dev(a) for a in dn]
+    ewt_d = np.array([[a.data_ptr(), b.data_ptr()] for a, b in zip(gd, dd)], dtype=np.uint64)
+    ewt_d[3] = 0
+    xd, ewtd, metad, rtd, rpd, rgd, fuhd = (to_dev(a) for a in (x, ewt_d, al[0], al[2], al[3], al[4], fu_h))
+    fu_d = torch.full((rows, I), 0x1234, dtype=torch.int16, device="cuda")
+    part_d = torch.full((T * k, H), 9.0, dtype=torch.float32, device="cuda")
+    moe.exec(glu, dev_table([fu_d, xd, ewtd, metad, rtd]))
+    moe.exec(down, dev_table([part_d, fuhd, ewtd, metad, rpd, rgd]))
+    torch.cuda.synchronize()
+    written = fu_h != 0x1234
+    fu_g = fu_d.cpu().numpy().view(np.uint16)
+    assert np.array_equal(fu_g != 0x1234, written)            # pad rows and expert 3: nothing written
+    close(ol.bf2f(fu_g[written]), ol.bf2f(fu_h[written]), "fu")
+    part_g = part_d.cpu().numpy()
+    touched = part_h != 9.0
+    assert np.array_equal(part_g != 9.0, touched)
+    close(part_g[touched], part_h[touched], "part", mean_rel=1e-4, max_frac=1e-4)
