@@ -35,6 +35,19 @@
 #include "common.h"
 #include "kernels.h"
 
+/* SiLU(g) * u for the tile epilogue, where 128 x 128 of them per tile run on the waves that should be
+ * multiplying: hardware exp2 and reciprocal (about 1 ulp each) instead of the library's expf and an
+ * IEEE division, a third of the instructions. The result is rounded to fp8 (block mode) or bf16
+ * (per-channel mode) right after, far above this error. Limits agree with g / (1 + expf(-g)):
+ * g -> -inf gives -0, +inf gives +inf, NaN stays NaN. */
+__device__ __forceinline__ float t5_glu(float gt, float up, uint32_t act) {
+    if (act == PLOW_MOE_ACT_SILU) {
+        const float e = __builtin_amdgcn_exp2f(gt * -1.4426950408889634f);
+        return (gt * __builtin_amdgcn_rcpf(1.0f + e)) * up;
+    }
+    return moe_glu(gt, up, act);
+}
+
 #define T5_BM 128u
 #define T5_THREADS 768u /* 8 consumer waves + 4 loader waves */
 #define T5_STAGES 3u
@@ -543,7 +556,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                             float o[4];
 #pragma unroll
                             for (int i = 0; i < 4; i++)
-                                o[i] = moe_glu(acc[rg][0][i] * (as * es[ch0 + 4u * q + i]),
+                                o[i] = t5_glu(acc[rg][0][i] * (as * es[ch0 + 4u * q + i]),
                                                acc[rg][1][i] * (as * es[g.N + ch0 + 4u * q + i]), g.act);
                             uint2 pk;
                             pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
@@ -574,7 +587,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                     float m = 0.0f;
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        v[rg][i] = moe_glu(acc[rg][0][i], acc[rg][1][i], g.act);
+                        v[rg][i] = t5_glu(acc[rg][0][i], acc[rg][1][i], g.act);
                         m = fmaxf(m, fabsf(v[rg][i]));
                     }
                     m = fmaxf(m, __shfl_xor(m, 16, 64));
