@@ -48,6 +48,7 @@ def main():
     ap.add_argument("--config", default="c2")
     ap.add_argument("--tokens", type=int, default=0)
     ap.add_argument("--arm", default="", help="override the configuration's arm (a16 | w8a8)")
+    ap.add_argument("--zipf", type=float, default=-1.0, help="override the expert popularity exponent")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib", action="store_true",
                     help="also run a plain 1 GiB device copy three times (a kernel of known traffic, "
@@ -74,7 +75,9 @@ def main():
         cfg.arm = a.arm
     plan = layer.plan_layer(cfg)
     hot = 3.0 if a.config == "c3" else 0.0
-    dev = synth.bind(plan, "cuda", seed=0, hot_expert=hot, zipf=1.2 if a.config == "c5" else 0.0)
+    # c6: popularity falling off like rank^-0.5, as in plow's bench of this shape
+    zipf = a.zipf if a.zipf >= 0.0 else {"c5": 1.2, "c6": 0.5}.get(a.config, 0.0)
+    dev = synth.bind(plan, "cuda", seed=0, hot_expert=hot, zipf=zipf)
     moe = Moe(0)
     stream = torch.cuda.current_stream().cuda_stream
     insts = abi.inst_array(plan.insts)

@@ -611,7 +611,41 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                 }
             } else {
                 WG_BARRIER(); /* after the last block (pairs with the loaders') */
-                if (wave_on) {
+                if (wave_on && !g.part16) {
+                    /* f32 partials: a row's 32 channels of this wave are one 128-byte line. Each 16-row
+                     * group goes through LDS once so that it leaves as two stores of 8 whole lines (8
+                     * consecutive lanes per line) instead of two stores that touch 16 half lines each.
+                     * The staging area is this wave's own weight slice of the ring stage it has just left:
+                     * nobody else reads it, and the loaders refill it only after the next barrier. */
+                    const uint32_t stl = st >= 1u ? st - 1u : 2u;
+                    const uint32_t stg = w_base + stl * (256u * 128u) + cw * (32u * 128u);
+                    const uint32_t wsw = r16 & 7u;
+                    const uint32_t wr0 = stg + r16 * 128u + ((q ^ wsw) << 4), wr1 = stg + r16 * 128u + (((4u + q) ^ wsw) << 4);
+                    const uint32_t lrow = lane >> 3, lp = lane & 7u; /* store layout: row lrow (+ 8), piece lp */
+                    const uint32_t rd = stg + lrow * 128u + ((lp ^ (lrow & 7u)) << 4);
+#pragma unroll
+                    for (int rg = 0; rg < 8; rg++) {
+                        if (16u * (uint32_t)rg >= rows) break; /* uniform */
+                        const uint32_t row = 16u * (uint32_t)rg + r16;
+                        const float gate = L.epi_gate[par][row]; /* 0 for pad rows */
+                        const v4f y0 = acc[rg][0] * gate, y1 = acc[rg][1] * gate;
+                        const uint32_t rowa = 16u * (uint32_t)rg + lrow, rowb = rowa + 8u;
+                        const uint32_t pa = L.epi_idx[par][rowa], pb = L.epi_idx[par][rowb];
+                        v4f oa, ob;
+                        asm volatile("ds_write_b128 %2, %4 offset:%6\n\tds_write_b128 %3, %5 offset:%6\n\t"
+                                     "ds_read_b128 %0, %7 offset:%6\n\tds_read_b128 %1, %7 offset:%8\n\t"
+                                     "s_waitcnt lgkmcnt(0)"
+                                     : "=&v"(oa), "=&v"(ob)
+                                     : "v"(wr0), "v"(wr1), "v"(y0), "v"(y1), "n"((rg & 1) * 2048), "v"(rd),
+                                       "n"((rg & 1) * 2048 + 1024)
+                                     : "memory");
+                        float* const ocol = (float*)g.out + ch0 + 4u * lp;
+                        if (rowa < rows && pa != PLOW_EXPERT_UNUSED)
+                            *(float4*)(ocol + (size_t)pa * g.N) = make_float4(oa[0], oa[1], oa[2], oa[3]);
+                        if (rowb < rows && pb != PLOW_EXPERT_UNUSED)
+                            *(float4*)(ocol + (size_t)pb * g.N) = make_float4(ob[0], ob[1], ob[2], ob[3]);
+                    }
+                } else if (wave_on) {
 #pragma unroll
                     for (int rg = 0; rg < 8; rg++) {
                         const uint32_t row = 16u * (uint32_t)rg + r16;

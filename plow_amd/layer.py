@@ -87,6 +87,10 @@ def config(name: str, T: Optional[int] = None) -> MoeConfig:
     if name == "c5":   # Qwen3-MoE-shaped per-channel fp8, no shared expert
         return MoeConfig("c5", H=4096, E=128, I=1536, k=8, T=T or 64, scoring="softmax",
                          norm_topk=True, enc="fp8pc", arm="a16")
+    if name == "c6":   # GLM-5.3-Flash-shaped block-fp8, one rank's slice of TP8 (the shape of plow's
+        # own gfx950 prefill bench, runtime/bench/amd/moe_fp8_pf_bench.hip:1-7)
+        return MoeConfig("c6", H=4096, E=288, I=256, k=8, T=T or 8192, scoring="sigmoid",
+                         norm_topk=True, bias=True, enc="fp8blk", arm="w8a8")
     raise KeyError(name)
 
 
