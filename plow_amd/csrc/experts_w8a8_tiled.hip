@@ -528,6 +528,32 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
              *      group 0 and up in group 1; DOWN channel = ch0 + 16 * x + 4q + i ---- */
+            /* DOWN, f32 partials: a row's 32 channels of this wave are one 128-byte line. A 16-row group
+             * goes through LDS once so that it leaves as two stores of 8 whole lines (8 consecutive lanes
+             * per line) instead of two stores that touch 16 half lines each. The staging area is this
+             * wave's own weight slice of the ring stage it has just left: nobody else reads it, and the
+             * loaders refill it only after the next barrier. Every lane of the wave must call this. */
+            const uint32_t stg = w_base + (st >= 1u ? st - 1u : 2u) * (256u * 128u) + cw * (32u * 128u);
+            auto down_store_f32 = [&](int rg, v4f y0, v4f y1) {
+                const uint32_t buf = stg + (uint32_t)(rg & 1) * 2048u, wsw = r16 & 7u;
+                const uint32_t wr0 = buf + r16 * 128u + ((q ^ wsw) << 4), wr1 = buf + r16 * 128u + (((4u + q) ^ wsw) << 4);
+                const uint32_t lrow = lane >> 3, lp = lane & 7u; /* store layout: row lrow (+ 8), piece lp */
+                const uint32_t rd = buf + lrow * 128u + ((lp ^ (lrow & 7u)) << 4);
+                const uint32_t rowa = 16u * (uint32_t)rg + lrow, rowb = rowa + 8u;
+                const uint32_t pa = L.epi_idx[par][rowa], pb = L.epi_idx[par][rowb];
+                v4f oa, ob;
+                asm volatile("ds_write_b128 %2, %4\n\tds_write_b128 %3, %5\n\t"
+                             "ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:1024\n\t"
+                             "s_waitcnt lgkmcnt(0)"
+                             : "=&v"(oa), "=&v"(ob)
+                             : "v"(wr0), "v"(wr1), "v"(y0), "v"(y1), "v"(rd)
+                             : "memory");
+                float* const ocol = (float*)g.out + ch0 + 4u * lp;
+                if (rowa < rows && pa != PLOW_EXPERT_UNUSED)
+                    *(float4*)(ocol + (size_t)pa * g.N) = make_float4(oa[0], oa[1], oa[2], oa[3]);
+                if (rowb < rows && pb != PLOW_EXPERT_UNUSED)
+                    *(float4*)(ocol + (size_t)pb * g.N) = make_float4(ob[0], ob[1], ob[2], ob[3]);
+            };
             if (PC) {
                 /* per-channel arm (plow runtime/amd/op_moe.h:6655-6700): g = acc * (as * wsc[n]); GLU stores
                  * bf16(act(g) * u) and zeroes the expert's pad rows, DOWN stores gate * acc, then
@@ -536,7 +562,26 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                 const float* es = (const float*)(uintptr_t)g.stab[(size_t)t.e * 2u + (GLU ? 0u : 1u)];
                 const uint32_t cnt_e = (uint32_t)g.meta[g.E + t.e], erow0 = r0 - (uint32_t)g.meta[t.e];
                 const uint32_t padded = ((cnt_e + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
-                if (wave_on) {
+                if (wave_on && !GLU) {
+#pragma unroll
+                    for (int rg = 0; rg < 8; rg++) {
+                        if (16u * (uint32_t)rg >= rows) break; /* uniform */
+                        const uint32_t row = 16u * (uint32_t)rg + r16;
+                        const float gate = L.epi_gate[par][row]; /* 0 for pad rows */
+                        const float as = row < rows ? g.a_scale[r0 + row] : 0.0f;
+                        v4f y[2];
+#pragma unroll
+                        for (int x = 0; x < 2; x++) {
+                            const uint32_t col = ch0 + 16u * (uint32_t)x + 4u * q;
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                y[x][i] = gate * acc[rg][x][i];
+                                y[x][i] *= as * es[col + i];
+                            }
+                        }
+                        down_store_f32(rg, y[0], y[1]);
+                    }
+                } else if (wave_on) {
 #pragma unroll
                     for (int rg = 0; rg < 8; rg++) {
                         const uint32_t row = 16u * (uint32_t)rg + r16;
@@ -562,21 +607,6 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                             pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
                             pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
                             *(uint2*)orow = pk;
-                        } else {
-                            const uint32_t pidx = L.epi_idx[par][row];
-                            if (pidx == PLOW_EXPERT_UNUSED) continue;
-                            const float gate = L.epi_gate[par][row], as = g.a_scale[r0 + row];
-#pragma unroll
-                            for (int x = 0; x < 2; x++) {
-                                const uint32_t col = ch0 + 16u * (uint32_t)x + 4u * q;
-                                float o[4];
-#pragma unroll
-                                for (int i = 0; i < 4; i++) {
-                                    o[i] = gate * acc[rg][x][i];
-                                    o[i] *= as * es[col + i];
-                                }
-                                *(float4*)((float*)g.out + (size_t)pidx * g.N + col) = make_float4(o[0], o[1], o[2], o[3]);
-                            }
                         }
                     }
                 }
@@ -612,38 +642,11 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
             } else {
                 WG_BARRIER(); /* after the last block (pairs with the loaders') */
                 if (wave_on && !g.part16) {
-                    /* f32 partials: a row's 32 channels of this wave are one 128-byte line. Each 16-row
-                     * group goes through LDS once so that it leaves as two stores of 8 whole lines (8
-                     * consecutive lanes per line) instead of two stores that touch 16 half lines each.
-                     * The staging area is this wave's own weight slice of the ring stage it has just left:
-                     * nobody else reads it, and the loaders refill it only after the next barrier. */
-                    const uint32_t stl = st >= 1u ? st - 1u : 2u;
-                    const uint32_t stg = w_base + stl * (256u * 128u) + cw * (32u * 128u);
-                    const uint32_t wsw = r16 & 7u;
-                    const uint32_t wr0 = stg + r16 * 128u + ((q ^ wsw) << 4), wr1 = stg + r16 * 128u + (((4u + q) ^ wsw) << 4);
-                    const uint32_t lrow = lane >> 3, lp = lane & 7u; /* store layout: row lrow (+ 8), piece lp */
-                    const uint32_t rd = stg + lrow * 128u + ((lp ^ (lrow & 7u)) << 4);
 #pragma unroll
                     for (int rg = 0; rg < 8; rg++) {
                         if (16u * (uint32_t)rg >= rows) break; /* uniform */
-                        const uint32_t row = 16u * (uint32_t)rg + r16;
-                        const float gate = L.epi_gate[par][row]; /* 0 for pad rows */
-                        const v4f y0 = acc[rg][0] * gate, y1 = acc[rg][1] * gate;
-                        const uint32_t rowa = 16u * (uint32_t)rg + lrow, rowb = rowa + 8u;
-                        const uint32_t pa = L.epi_idx[par][rowa], pb = L.epi_idx[par][rowb];
-                        v4f oa, ob;
-                        asm volatile("ds_write_b128 %2, %4 offset:%6\n\tds_write_b128 %3, %5 offset:%6\n\t"
-                                     "ds_read_b128 %0, %7 offset:%6\n\tds_read_b128 %1, %7 offset:%8\n\t"
-                                     "s_waitcnt lgkmcnt(0)"
-                                     : "=&v"(oa), "=&v"(ob)
-                                     : "v"(wr0), "v"(wr1), "v"(y0), "v"(y1), "n"((rg & 1) * 2048), "v"(rd),
-                                       "n"((rg & 1) * 2048 + 1024)
-                                     : "memory");
-                        float* const ocol = (float*)g.out + ch0 + 4u * lp;
-                        if (rowa < rows && pa != PLOW_EXPERT_UNUSED)
-                            *(float4*)(ocol + (size_t)pa * g.N) = make_float4(oa[0], oa[1], oa[2], oa[3]);
-                        if (rowb < rows && pb != PLOW_EXPERT_UNUSED)
-                            *(float4*)(ocol + (size_t)pb * g.N) = make_float4(ob[0], ob[1], ob[2], ob[3]);
+                        const float gate = L.epi_gate[par][16u * (uint32_t)rg + r16]; /* 0 for pad rows */
+                        down_store_f32(rg, acc[rg][0] * gate, acc[rg][1] * gate);
                     }
                 } else if (wave_on) {
 #pragma unroll
