@@ -7,6 +7,8 @@
  * correctly rounded IEEE operations and the exponential of pm_expf.h.
  * This file is compiled with -ffp-contract=off: no multiply-add is fused unless written as fmaf.
  */
+#include <stdlib.h>
+#include <string.h>
 #include "common.h"
 #include "kernels.h"
 #include "pm_expf.h"
@@ -107,6 +109,154 @@ __global__ __launch_bounds__(256) void k_router_score_tile(float* __restrict__ o
             const uint32_t m = m0 + ty * TM + i, n = n0 + tx * 4u + j;
             if (m < M && n < N) out[(size_t)m * N + n] = acc[i][j];
         }
+}
+
+/* Large problems with K a multiple of 64: the same sums on the matrix unit. v_mfma_f32_32x32x2_f32
+ * adds a[i][k] * b[k][j], then a[i][k + 1] * b[k + 1][j], to its f32 accumulator, each step rounded
+ * to nearest even and denormals kept (measured against the fmaf chain, bit for bit, normal and
+ * denormal ranges), so a chain of K / 2 of them IS the reference's sum in the reference's order, at
+ * twice the rate of the vector unit and without an operand broadcast through LDS.
+ * One wave per workgroup computes 32 tokens x 32 experts. Operand rows (bf16, 64 k = one 128-byte line
+ * per row and chunk) come in by direct global -> LDS loads in the coalesced shape into a wave-private
+ * ring of three chunks, two chunks ahead; no barrier anywhere. A lane reads 16 bytes (8 k) of its
+ * token row and of its expert row per piece; lanes 0..31 feed the even k of a pair to the instruction
+ * and lanes 32..63 the odd k (one byte permute each widens bf16 to f32). The next piece's LDS reads
+ * are issued before the four matrix instructions of this piece and waited for after them. LDS piece p
+ * of row r holds global piece p ^ ((r >> 1) & 7): 16 consecutive rows of a piece cover all 64 banks. */
+#define RSM_STAGES 3
+struct RsmStage {
+    uint8_t x[32u * 128u];
+    uint8_t w[32u * 128u];
+};
+typedef __attribute__((address_space(3))) void rsm_lds_void;
+__global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ out, const bf16_t* __restrict__ x,
+                                                           const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
+                                                           uint32_t K) {
+    /* four independent waves per workgroup (a 2 x 2 block of tiles): 96 KB of LDS makes it one workgroup
+     * per CU, which puts exactly one wave on every SIMD */
+    extern __shared__ __attribute__((aligned(16))) uint8_t rsm_raw[];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    RsmStage* const ring = (RsmStage*)rsm_raw + wv * RSM_STAGES;
+    /* Workgroup b runs on XCD b % 8 and each XCD has its own L2: the logical index gives one XCD
+     * consecutive workgroups, which share their token rows (the expert-tile index runs fastest) */
+    const uint32_t G = gridDim.x, gx = (N + 63u) / 64u;
+    const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const uint32_t m0 = ((wg / gx) * 2u + (wv >> 1)) * 32u, n0 = ((wg % gx) * 2u + (wv & 1u)) * 32u;
+    if (m0 >= M || n0 >= N) return; /* whole wave; there is no barrier below */
+    const uint32_t NC = K / 64u;
+    /* load j covers rows 8j .. 8j + 7: lane -> (row lane >> 3, LDS piece lane & 7); rows past the end
+     * of the matrix read its last row and are never stored */
+    const uint32_t lr = lane >> 3, lp = lane & 7u;
+    const uint8_t *xsrc[4], *wsrc[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4u; j++) {
+        const uint32_t row = 8u * j + lr;
+        const uint32_t mr = m0 + row < M ? m0 + row : M - 1u, nr = n0 + row < N ? n0 + row : N - 1u;
+        xsrc[j] = (const uint8_t*)(x + (size_t)mr * K) + ((lp ^ ((row >> 1) & 7u)) << 4);
+        wsrc[j] = (const uint8_t*)(w + (size_t)nr * K) + ((lp ^ ((row >> 1) & 7u)) << 4);
+    }
+    auto issue = [&](uint32_t c) {
+        RsmStage* s = &ring[c % RSM_STAGES];
+#pragma unroll
+        for (uint32_t j = 0; j < 4u; j++)
+            __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
+#pragma unroll
+        for (uint32_t j = 0; j < 4u; j++)
+            __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
+    };
+    /* operand reads: row lane & 31 of the token rows (A) and of the expert rows (B) */
+    const uint32_t orow = lane & 31u, osw = (orow >> 1) & 7u;
+    const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)&ring[0];
+    const uint32_t obase = ring0 + orow * 128u;
+    const uint32_t sel = lane < 32u ? 0x01000c0cu : 0x03020c0cu; /* low / high bf16 of a dword -> f32 bits */
+    v16f acc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+    /* Per piece: issue the next piece's LDS reads, run this piece's four matrix instructions, wait for
+     * the reads, widen them into the other half of the operand registers. An instruction's operands
+     * are never overwritten while it may still be reading them (the vector unit would wait for it), and
+     * the widening runs under the last matrix instruction of the piece. */
+    v4i xa, wb;
+    float af[2][4], bf[2][4];
+    auto read_piece = [&](uint32_t stage, uint32_t pc) {
+        const uint32_t addr = obase + stage * (uint32_t)sizeof(RsmStage) + ((pc ^ osw) << 4);
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:4096" : "=v"(xa), "=v"(wb) : "v"(addr) : "memory");
+    };
+    auto widen = [&](uint32_t h, int d0, int d1) {
+        if (d0 == 0) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa), "+v"(wb));
+#pragma unroll
+        for (int d = d0; d < d1; d++) {
+            af[h][d] = __uint_as_float(__builtin_amdgcn_perm((uint32_t)xa[d], (uint32_t)xa[d], sel));
+            bf[h][d] = __uint_as_float(__builtin_amdgcn_perm((uint32_t)wb[d], (uint32_t)wb[d], sel));
+        }
+    };
+    issue(0u);
+    if (NC > 1u) issue(1u);
+    if (NC > 2u) issue(2u);
+    if (NC > 2u) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if (NC > 1u) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    read_piece(0u, 0u);
+    widen(0u, 0, 4);
+    uint32_t st = 0;
+#define RSM_MFMA(d) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][d], bf[cur][d], acc, 0, 0, 0)
+#define RSM_FENCE() __builtin_amdgcn_sched_barrier(0)
+    for (uint32_t c = 0; c < NC; c++) {
+        const uint32_t stn = st == RSM_STAGES - 1u ? 0u : st + 1u;
+#pragma unroll
+        for (uint32_t pc = 0; pc < 8u; pc++) {
+            const uint32_t cur = pc & 1u, nxt = cur ^ 1u;
+            /* everything that is not a matrix instruction is issued behind one, so that the matrix unit
+             * is busy while the wave issues it */
+            RSM_FENCE();
+            RSM_MFMA(0);
+            RSM_FENCE();
+            if (pc == 7u) {
+                /* every piece of chunk c has been read: chunk c + 1 must have landed before its first
+                 * piece is read, and chunk c's stage takes chunk c + 3 */
+                if (c + 2u < NC) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                read_piece(stn, 0u); /* past the last chunk: stale bytes, never used */
+            } else {
+                read_piece(st, pc + 1u);
+            }
+            RSM_FENCE();
+            RSM_MFMA(1);
+            RSM_FENCE();
+            if (pc == 7u && c + 3u < NC) {
+                RsmStage* s = &ring[(c + 3u) % RSM_STAGES];
+#pragma unroll
+                for (uint32_t j = 0; j < 4u; j++)
+                    __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)(c + 3u) * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
+            }
+            RSM_FENCE();
+            RSM_MFMA(2);
+            RSM_FENCE();
+            if (pc == 7u && c + 3u < NC) {
+                RsmStage* s = &ring[(c + 3u) % RSM_STAGES];
+#pragma unroll
+                for (uint32_t j = 0; j < 4u; j++)
+                    __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)(c + 3u) * 128u), (rsm_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
+            }
+            RSM_FENCE();
+            widen(nxt, 0, 2);
+            RSM_FENCE();
+            RSM_MFMA(3);
+            RSM_FENCE();
+            widen(nxt, 2, 4);
+        }
+        st = stn;
+    }
+#undef RSM_MFMA
+#undef RSM_FENCE
+    /* acc[r] = out[m0 + 8 * (r / 4) + 4 * (lane / 32) + r % 4][n0 + lane % 32] */
+    const uint32_t n = n0 + (lane & 31u);
+#pragma unroll
+    for (uint32_t r = 0; r < 16u; r++) {
+        const uint32_t m = m0 + 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
+        if (m < M && n < N) out[(size_t)m * N + n] = acc[r];
+    }
 }
 
 /* Small problems (decode). Two things bound this shape: the dependent chain of K multiply-adds per
@@ -219,10 +369,30 @@ __global__ __launch_bounds__(128) void k_router_score_wave(float* __restrict__ o
     if (m < M && n < N) out[(size_t)m * N + n] = acc;
 }
 
+/* PLOW_MOE_SCORE_KERNEL=valu keeps the prefill score on the vector unit (for comparison) */
+static bool score_mfma_form() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = getenv("PLOW_MOE_SCORE_KERNEL");
+        v = !(e && !strcmp(e, "valu"));
+    }
+    return v != 0;
+}
+
 int launch_router_score(float* out, const void* x, const void* w, uint32_t M, uint32_t N, uint32_t K,
                         hipStream_t st) {
     if (K % 8u) return PLOW_MOE_EINVAL;
-    if ((uint64_t)M * N >= (1u << 19)) {
+    if ((uint64_t)M * N >= (1u << 18) && K % 64u == 0u && score_mfma_form()) {
+        static bool attr_set = false;
+        const uint32_t lds = 4u * RSM_STAGES * (uint32_t)sizeof(RsmStage);
+        if (!attr_set) {
+            if (hipFuncSetAttribute((const void*)k_router_score_mfma, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+                return PLOW_MOE_EDEVICE;
+            attr_set = true;
+        }
+        const uint32_t g = ((N + 63) / 64) * ((M + 63) / 64);
+        k_router_score_mfma<<<g, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+    } else if ((uint64_t)M * N >= (1u << 19)) {
         if ((uint64_t)((N + 63) / 64) * ((M + 63) / 64) < 512u) { /* fewer than two 64-row workgroups per CU */
             dim3 g((N + 63) / 64, (M + 31) / 32);
             k_router_score_tile<2><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
