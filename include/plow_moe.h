@@ -105,7 +105,13 @@ enum {
 };
 
 /* GLU activations (i5; runtime/amd/op_moe.h:216-241, golden/golden.h:107-133). */
-enum { PLOW_MOE_ACT_GELU_TANH = 0, PLOW_MOE_ACT_SILU = 1 };
+enum {
+    PLOW_MOE_ACT_GELU_TANH = 0,
+    PLOW_MOE_ACT_SILU = 1,
+    PLOW_MOE_ACT_SITU = 2,         /* pair form, fj[0] = beta, fj[1] = linear beta */
+    PLOW_MOE_ACT_SWIGLU_OAI = 3,   /* pair form, fj[0] = alpha, fj[1] = limit (> 0) */
+    PLOW_MOE_ACT_SWIGLU_CLAMP = 4  /* pair form, fj[1] = limit */
+};
 
 /* Router flags (i3 of ops 56/83; runtime/amd/op_moe.h:453-467). */
 enum {

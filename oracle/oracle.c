@@ -57,12 +57,30 @@ static float act_gelu_tanh(float x) {
     return 0.5f * x * (1.0f + tanhf(c));
 }
 static float act_silu(float x) { return x / (1.0f + expf(-x)); }
-/* act 0 gelu_tanh, 1 silu; the pair forms (2 situ, 3 swiglu_oai, 4 clamp) are not on this path and
- * poison, as a gate-only epilogue does in the reference. */
+/* act 0 gelu_tanh, 1 silu; gate-only epilogues poison on the pair forms, as the reference's do
+ * (plow runtime/cpu/dev/golden/golden.h:110-115). */
 static float glu(float g, float u, uint32_t act) {
     if (act == 1u) return act_silu(g) * u;
     if (act == 0u) return act_gelu_tanh(g) * u;
     return NAN;
+}
+/* Every epilogue that takes the activation's immediates f0 / f1 (plow runtime/cpu/dev/golden/
+ * golden.h:116-133): 2 situ (beta, linear beta), 3 swiglu_oai (alpha, limit; limit <= 0 poisons);
+ * 4 the clamped SwiGLU of plow's AMD path only (runtime/amd/op_moe.h:236-239, limit in f1). */
+static float act_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+static float glu_pair(float g, float u, uint32_t act, float f0, float f1) {
+    if (act == 2u) return (f0 * tanhf(g / f0) * act_sigmoid(g)) * (f1 > 0.0f ? f1 * tanhf(u / f1) : u);
+    if (act == 3u) {
+        if (!(f1 > 0.0f)) return NAN;
+        g = g < f1 ? g : f1;
+        u = u < -f1 ? -f1 : (u > f1 ? f1 : u);
+        return g * act_sigmoid(f0 * g) * (u + 1.0f);
+    }
+    if (act == 4u) {
+        const float gc = fminf(g, f1);
+        return (gc / (1.0f + expf(-gc))) * fminf(fmaxf(u, -f1), f1);
+    }
+    return glu(g, u, act);
 }
 
 /* ---- op 180: router score ---------------------------------------------------------------------- */
@@ -454,7 +472,7 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
                     if (!rc.live[q]) continue;
                     const float* a = rc.a + (size_t)q * H;
                     fu[(size_t)(r0 + q) * I + n] =
-                        orc_f2bf(glu(enc_dot(enc, wg, sg, a, H), enc_dot(enc, wu, su, a, H), act));
+                        orc_f2bf(glu_pair(enc_dot(enc, wg, sg, a, H), enc_dot(enc, wu, su, a, H), act, in->fj[0].f, in->fj[1].f));
                 }
             }
         } else {
@@ -471,7 +489,7 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
                     const float* a = rc.a + (size_t)q * H;
                     const float g = dot_fp8blk_a8(wg, (const float*)Sg + (size_t)g0 * KB, a, xs + tok, pitch, H);
                     const float u = dot_fp8blk_a8(wu, (const float*)Su + (size_t)g0 * KB, a, xs + tok, pitch, H);
-                    v[(size_t)q * 128u + (n - n0)] = glu(g, u, act);
+                    v[(size_t)q * 128u + (n - n0)] = glu_pair(g, u, act, in->fj[0].f, in->fj[1].f);
                 }
             }
             for (uint32_t q = 0; q < cnt; q++) {
@@ -849,7 +867,8 @@ static void op_group_down_gemma(const PlowDevInst* in, uint32_t slice, uint32_t 
  * Expert e of a [E][N][K/2] fp4 tensor starts at W + e*N*(K/2), its E8M0 bytes at S + e*N*(K/32), its
  * bf16 bias at b + e*N. Gate / up rows of output n: layout 0 interleaved (2n, 2n + 1), layout 1 blocked
  * (n, I + n) (moe.c:12-16). The bias is added in f32 before the activation (GLU) and before the gate
- * multiply (DOWN). Activations 0 / 1 as everywhere on this path; the pair forms 2 / 3 poison. */
+ * multiply (DOWN). The GLU takes the pair-form activations with fj[0] / fj[1] as their immediates
+ * (moe.c:32, 50). */
 static float mx_flat_dot(const uint8_t* We, const uint8_t* Se, uint32_t row, const float* a, uint32_t K, float* wf) {
     decode_mxfp4_row(wf, We + (size_t)row * (K / 2u), K);
     return dot_mxfp4(wf, Se + (size_t)row * (K / 32u), a, K);
@@ -879,7 +898,7 @@ static void op_glu_mx(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void
         const uint32_t rg = layout ? n : 2u * n, ru = layout ? I + n : 2u * n + 1u;
         float g = mx_flat_dot(We, Se, rg, a, K, wf), u = mx_flat_dot(We, Se, ru, a, K, wf);
         if (bias) { g += orc_bf2f(bias[(size_t)e * 2u * I + rg]); u += orc_bf2f(bias[(size_t)e * 2u * I + ru]); }
-        fu[(size_t)s * I + n] = orc_f2bf(glu(g, u, act));
+        fu[(size_t)s * I + n] = orc_f2bf(glu_pair(g, u, act, in->fj[0].f, in->fj[1].f));
     }
     free(a); free(wf);
 }
@@ -936,7 +955,7 @@ static void op_glu_mx_pf(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
                 const uint32_t rg = layout ? n : 2u * n, ru = layout ? I + n : 2u * n + 1u;
                 float g = mx_flat_dot(We, Se, rg, a, K, wf), u = mx_flat_dot(We, Se, ru, a, K, wf);
                 if (bias) { g += orc_bf2f(bias[(size_t)e * 2u * I + rg]); u += orc_bf2f(bias[(size_t)e * 2u * I + ru]); }
-                fu[(size_t)r * I + n] = orc_f2bf(glu(g, u, act));
+                fu[(size_t)r * I + n] = orc_f2bf(glu_pair(g, u, act, in->fj[0].f, in->fj[1].f));
             }
         }
     }
@@ -1023,13 +1042,22 @@ static void* job_main(void* p) {
     return NULL;
 }
 
-int plow_oracle_exec(const PlowDevInst* inst, void* const* tensors, uint32_t nthreads) {
-    op_fn fn = resolve(inst->op);
-    if (!fn) return PLOW_MOE_EUNSUPPORTED;
-    if (!e4m3_lut_ready) {
-        for (int b = 0; b < 256; b++) e4m3_lut[b] = orc_e4m3_to_f32((uint8_t)b);
-        e4m3_lut_ready = 1;
-    }
+/* plow's CPU workers run with flush-to-zero and denormals-are-zero set (MXCSR bits 15 and 6, plow
+ * runtime/cpu/dev/isa_detect.c:158-164): f32 results and operands below 2^-126 read as zero. The
+ * restatement runs the same way (threads inherit the mode) and puts the caller's mode back. */
+#if defined(__x86_64__)
+static unsigned fp_mode_enter(void) {
+    const unsigned old = __builtin_ia32_stmxcsr();
+    __builtin_ia32_ldmxcsr(old | 0x8040u);
+    return old;
+}
+static void fp_mode_leave(unsigned old) { __builtin_ia32_ldmxcsr((__builtin_ia32_stmxcsr() & ~0x8040u) | (old & 0x8040u)); }
+#else
+static unsigned fp_mode_enter(void) { return 0; }
+static void fp_mode_leave(unsigned old) { (void)old; }
+#endif
+
+static int exec_one(op_fn fn, const PlowDevInst* inst, void* const* tensors, uint32_t nthreads) {
     if (nthreads <= 1u) { fn(inst, 0u, 1u, tensors); return 0; }
     if (nthreads > 256u) nthreads = 256u;
     pthread_t th[256];
@@ -1043,6 +1071,19 @@ int plow_oracle_exec(const PlowDevInst* inst, void* const* tensors, uint32_t nth
     }
     for (uint32_t s = 0; s < nthreads; s++) pthread_join(th[s], NULL);
     return 0;
+}
+
+int plow_oracle_exec(const PlowDevInst* inst, void* const* tensors, uint32_t nthreads) {
+    op_fn fn = resolve(inst->op);
+    if (!fn) return PLOW_MOE_EUNSUPPORTED;
+    if (!e4m3_lut_ready) {
+        for (int b = 0; b < 256; b++) e4m3_lut[b] = orc_e4m3_to_f32((uint8_t)b);
+        e4m3_lut_ready = 1;
+    }
+    const unsigned mode = fp_mode_enter();
+    const int rc = exec_one(fn, inst, tensors, nthreads);
+    fp_mode_leave(mode);
+    return rc;
 }
 
 int plow_oracle_exec_many(const PlowDevInst* insts, uint32_t n, void* const* tensors, uint32_t nthreads) {

@@ -202,7 +202,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             NEED(c, ten(in, T, 3) && ten(in, T, 6) && ten(in, T, 7), "op 85 W8A8: t3 stab, t6 xs, t7 fs must be bound");
             NEED(c, I % 128u == 0u && H % 128u == 0u, "op 85 W8A8: I %u and H %u must be multiples of 128", I, H);
             NEED(c, i[4] != 0u, "op 85 W8A8: i4 (row pitch of the activation scales) is zero");
-            NEED(c, i[5] <= 1u, "op 85: activation %u is not served", i[5]);
+            NEED(c, i[5] <= 2u || i[5] == PLOW_MOE_ACT_SWIGLU_CLAMP, "op 85: activation %u is not served", i[5]);
             if (!launch) return 0;
             GroupW8A8 g = {};
             g.out = ten(in, T, 0); g.out_scale = (float*)ten(in, T, 7);
@@ -210,6 +210,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 3);
             g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.pitch = i[4]; g.act = i[5];
+            g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
             /* many rows per expert (row pitch >= 2 rows per expert per routed slot): tiled form */
             c->tiled = c->forced >= 0 ? c->forced : (i[4] >= 2u * E ? 1 : 0);
             if (H < 256u || I < 256u) c->tiled = 0; /* the tiled form needs two 128-k blocks in both GEMMs */
@@ -221,7 +222,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         if (a16) {
             NEED(c, enc == PLOW_MOE_ENC_BF16 || ten(in, T, 3), "op 85: t3 stab must be bound for encoding %u", enc);
             NEED(c, I % 128u == 0u && H % 128u == 0u, "op 85: I %u and H %u must be multiples of 128", I, H);
-            NEED(c, i[5] <= 1u, "op 85: activation %u is not served", i[5]);
+            NEED(c, i[5] <= 2u || i[5] == PLOW_MOE_ACT_SWIGLU_CLAMP, "op 85: activation %u is not served", i[5]);
             if (!launch) return 0;
             GroupA16 g = {};
             g.out = ten(in, T, 0); g.a = ten(in, T, 1);
@@ -229,6 +230,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.stab = enc == PLOW_MOE_ENC_BF16 ? nullptr : (const uint64_t*)ten(in, T, 3);
             g.meta = (const int32_t*)ten(in, T, 4); g.a_idx = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.enc = enc; g.act = i[5];
+            g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
             g.wcols = 3; g.wsel0 = 0; g.wsel1 = 1;
             g.slots_hint = c->slots_hint;
             return launch_group_glu_a16(g, st);
@@ -404,7 +406,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, N && K && E && N % 128u == 0u && K % 128u == 0u, "op %u: N %u and K %u must be non-zero multiples of 128", (unsigned)in->op, N, K);
         NEED(c, E <= WS_MAX_E && nslot <= WS_MAX_SLOTS && (pf || nslot), "op %u: %u slots / %u experts exceed the context workspace", (unsigned)in->op, nslot, E);
         NEED(c, layout <= 1u, "op %u: layout %u is neither interleaved (0) nor blocked (1)", (unsigned)in->op, layout);
-        if (act > 1u) return fail(c, PLOW_MOE_EUNSUPPORTED, "op %u: activation %u (a pair form) is not served", (unsigned)in->op, act);
+        if (act > PLOW_MOE_ACT_SWIGLU_OAI) return fail(c, PLOW_MOE_EUNSUPPORTED, "op %u: activation %u is not served", (unsigned)in->op, act);
         if (!launch) return 0;
         const uint32_t rows = glu ? 2u * N : N; /* weight rows per expert */
         uint64_t* wtab = c->ws_ftab;
@@ -415,6 +417,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.out = ten(in, T, 0); g.a = ten(in, T, 1);
         g.wtab = wtab; g.stab = stab; g.wcols = 3; g.wsel0 = g.wsel1 = 0;
         g.N = N; g.K = K; g.E = E; g.enc = PLOW_MOE_ENC_MXFP4; g.act = act;
+        g.f0 = in->fj[0].f; g.f1 = in->fj[1].f; /* the activation's immediates (act 2: betas, act 3: alpha, limit) */
         g.bias = bias; g.bias_rows = rows;
         if (glu) { g.wmul = layout ? 1u : 2u; g.wrow0 = 0; g.wrow1 = layout ? N : 1u; }
         if (pf) {

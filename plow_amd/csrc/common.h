@@ -46,13 +46,32 @@ __device__ __forceinline__ uint32_t cvt4_e4m3(float a, float b, float c, float d
     return (uint32_t)v;
 }
 
-/* GLU epilogue (plow runtime/amd/op_moe.h:216-241): act 1 silu, act 0 gelu_tanh, with the C library
- * exponential (not the fast intrinsic), as the reference insists. Other activations poison. */
-__device__ __forceinline__ float moe_glu(float g, float u, uint32_t act) {
+/* GLU epilogue as a pair A(gate) * B(up) (plow runtime/amd/op_moe.h:216-241, runtime/cpu/dev/golden/
+ * golden.h:110-133), with the C library's exponential and tanh (not the fast intrinsics), as the
+ * reference insists. f0 / f1 are the activation's immediates (the descriptor's fj[0], fj[1]):
+ *   0 gelu_tanh(g) * u                 1 silu(g) * u
+ *   2 situ: f0 * tanh(g / f0) * sigmoid(g)  *  (f1 > 0 ? f1 * tanh(u / f1) : u)
+ *   3 swiglu_oai (alpha f0, limit f1 > 0, else poison): g' = min(g, f1), u' = clamp(u, +-f1):
+ *     g' * sigmoid(f0 * g') * (u' + 1)
+ *   4 clamped SwiGLU (limit f1): silu(min(g, f1)) * clamp(u, +-f1)
+ * Anything else poisons. */
+__device__ __forceinline__ float moe_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float moe_glu(float g, float u, uint32_t act, float f0, float f1) {
     if (act == PLOW_MOE_ACT_SILU) return (g / (1.0f + expf(-g))) * u;
     if (act == PLOW_MOE_ACT_GELU_TANH) {
         const float c = 0.7978845608028654f * (g + 0.044715f * g * g * g);
         return (0.5f * g * (1.0f + tanhf(c))) * u;
+    }
+    if (act == PLOW_MOE_ACT_SITU) return (f0 * tanhf(g / f0) * moe_sigmoid(g)) * (f1 > 0.0f ? f1 * tanhf(u / f1) : u);
+    if (act == PLOW_MOE_ACT_SWIGLU_OAI) {
+        if (!(f1 > 0.0f)) return __builtin_nanf("");
+        g = g < f1 ? g : f1;
+        u = u < -f1 ? -f1 : (u > f1 ? f1 : u);
+        return g * moe_sigmoid(f0 * g) * (u + 1.0f);
+    }
+    if (act == PLOW_MOE_ACT_SWIGLU_CLAMP) {
+        const float gc = fminf(g, f1);
+        return (gc / (1.0f + expf(-gc))) * fminf(fmaxf(u, -f1), f1);
     }
     return __builtin_nanf("");
 }

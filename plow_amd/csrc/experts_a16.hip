@@ -235,8 +235,8 @@ __device__ __forceinline__ void ak_body(const GroupA16& g, uint32_t e, uint32_t 
     if (oi == PLOW_EXPERT_UNUSED) return;
     if (GLU) {
         uint2 o;
-        o.x = (uint32_t)f2bf(moe_glu(acc0[0], acc1[0], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[1], acc1[1], g.act)) << 16);
-        o.y = (uint32_t)f2bf(moe_glu(acc0[2], acc1[2], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[3], acc1[3], g.act)) << 16);
+        o.x = (uint32_t)f2bf(moe_glu(acc0[0], acc1[0], g.act, g.f0, g.f1)) | ((uint32_t)f2bf(moe_glu(acc0[1], acc1[1], g.act, g.f0, g.f1)) << 16);
+        o.y = (uint32_t)f2bf(moe_glu(acc0[2], acc1[2], g.act, g.f0, g.f1)) | ((uint32_t)f2bf(moe_glu(acc0[3], acc1[3], g.act, g.f0, g.f1)) << 16);
         *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
     } else {
         const float gate = g.gate ? g.gate[r] : 1.0f;
@@ -577,8 +577,8 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
             if (oi != PLOW_EXPERT_UNUSED) {
                 if (GLU) {
                     uint2 o;
-                    o.x = (uint32_t)f2bf(moe_glu(acc0[0], acc1[0], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[1], acc1[1], g.act)) << 16);
-                    o.y = (uint32_t)f2bf(moe_glu(acc0[2], acc1[2], g.act)) | ((uint32_t)f2bf(moe_glu(acc0[3], acc1[3], g.act)) << 16);
+                    o.x = (uint32_t)f2bf(moe_glu(acc0[0], acc1[0], g.act, g.f0, g.f1)) | ((uint32_t)f2bf(moe_glu(acc0[1], acc1[1], g.act, g.f0, g.f1)) << 16);
+                    o.y = (uint32_t)f2bf(moe_glu(acc0[2], acc1[2], g.act, g.f0, g.f1)) | ((uint32_t)f2bf(moe_glu(acc0[3], acc1[3], g.act, g.f0, g.f1)) << 16);
                     *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
                 } else {
                     const float y0 = gate * acc0[0], y1 = gate * acc0[1], y2 = gate * acc0[2], y3 = gate * acc0[3];

@@ -183,7 +183,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
                 float o[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    o[i] = moe_glu(acc0[rt][i] * (as * s0[col + i]), acc1[rt][i] * (as * s1[col + i]), g.act);
+                    o[i] = moe_glu(acc0[rt][i] * (as * s0[col + i]), acc1[rt][i] * (as * s1[col + i]), g.act, g.f0, g.f1);
                 uint2 pk;
                 pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
                 pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
@@ -210,7 +210,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             float m = 0.0f;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                v[rt][i] = moe_glu(acc0[rt][i], acc1[rt][i], g.act);
+                v[rt][i] = moe_glu(acc0[rt][i], acc1[rt][i], g.act, g.f0, g.f1);
                 m = fmaxf(m, fabsf(v[rt][i]));
             }
             m = fmaxf(m, __shfl_xor(m, 16, 64));
@@ -434,7 +434,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
         float v[4], m = 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            v[i] = moe_glu(acc0[i], acc1[i], g.act);
+            v[i] = moe_glu(acc0[i], acc1[i], g.act, g.f0, g.f1);
             m = fmaxf(m, fabsf(v[i]));
         }
         m = fmaxf(m, __shfl_xor(m, 16, 64));

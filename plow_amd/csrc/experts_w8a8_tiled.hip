@@ -40,12 +40,12 @@
  * IEEE division, a third of the instructions. The result is rounded to fp8 (block mode) or bf16
  * (per-channel mode) right after, far above this error. Limits agree with g / (1 + expf(-g)):
  * g -> -inf gives -0, +inf gives +inf, NaN stays NaN. */
-__device__ __forceinline__ float t5_glu(float gt, float up, uint32_t act) {
+__device__ __forceinline__ float t5_glu(float gt, float up, uint32_t act, float f0, float f1) {
     if (act == PLOW_MOE_ACT_SILU) {
         const float e = __builtin_amdgcn_exp2f(gt * -1.4426950408889634f);
         return (gt * __builtin_amdgcn_rcpf(1.0f + e)) * up;
     }
-    return moe_glu(gt, up, act);
+    return moe_glu(gt, up, act, f0, f1);
 }
 
 #define T5_BM 128u
@@ -602,7 +602,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 #pragma unroll
                             for (int i = 0; i < 4; i++)
                                 o[i] = t5_glu(acc[rg][0][i] * (as * es[ch0 + 4u * q + i]),
-                                               acc[rg][1][i] * (as * es[g.N + ch0 + 4u * q + i]), g.act);
+                                               acc[rg][1][i] * (as * es[g.N + ch0 + 4u * q + i]), g.act, g.f0, g.f1);
                             uint2 pk;
                             pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
                             pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
@@ -617,7 +617,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                     float m = 0.0f;
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        v[rg][i] = t5_glu(acc[rg][0][i], acc[rg][1][i], g.act);
+                        v[rg][i] = t5_glu(acc[rg][0][i], acc[rg][1][i], g.act, g.f0, g.f1);
                         m = fmaxf(m, fabsf(v[rg][i]));
                     }
                     m = fmaxf(m, __shfl_xor(m, 16, 64));

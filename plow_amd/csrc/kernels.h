@@ -36,6 +36,7 @@ struct GroupW8A8 {
     const uint32_t* row_partidx; /* DOWN */
     const float* row_gate;       /* DOWN */
     uint32_t N, K, E, pitch, act, part16, T;
+    float f0, f1; /* the activation's immediates */
     /* per-channel mode (ops 81 / 82): weights through ewt[E][2] = {gate_up fused [2N][K], down [N][K]},
      * f32 channel scales through est[E][2], one f32 activation scale per row; GLU writes bf16 */
     uint32_t per_channel;
@@ -58,6 +59,7 @@ struct GroupA16 {
     const uint32_t* o_idx;  /* aligned row -> output row (NULL = identity) */
     const float* gate;      /* DOWN: aligned row -> gate (NULL = 1) */
     uint32_t N, K, E, enc, act;
+    float f0, f1; /* the activation's immediates */
     uint32_t wcols, wsel0, wsel1; /* table width, column of the first / second weight stream */
     uint32_t wrow0, wrow1;        /* first weight row of each stream inside its tensor (fused gate_up) */
     uint32_t out_bf16, dense_rows;

@@ -36,6 +36,7 @@ class MoeConfig:
     n_shared: int = 0
     shared_mode: Optional[str] = None  # "fold" (slot {E, 1.0}) | "dense" (ops 20 + 8) | None
     act: int = abi.ACT_SILU
+    act_f: Tuple[float, float] = (0.0, 0.0)  # the activation's immediates (fj[0], fj[1]) for the pair forms 2 / 3 / 4
     residual: bool = False
     part_bf16: bool = False         # block-fp8 W8A8 only: bf16 partials (arm 3) instead of f32
 
@@ -186,7 +187,7 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
             p._emit("quant_x", abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[xq, x, xs], i=[T, H, T]))
             p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
                                     t=[fq, xq, wtab, stab, meta, row_token, xs, fs],
-                                    i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8]))
+                                    i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8], f=cfg.act_f))
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
                                      t=[part, fq, wtab, stab, meta, fs, row_partidx, row_gate],
                                      i=[H, I, Ea, enc, 0, 0, 0, abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8]))
@@ -195,7 +196,7 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
             fu = p._t("fu", "bf16", (R, I), "scratch")
             p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
                                     t=[fu, x, wtab, stab, meta, row_token],
-                                    i=[I, H, Ea, enc, 0, cfg.act, 0, arm]))
+                                    i=[I, H, Ea, enc, 0, cfg.act, 0, arm], f=cfg.act_f))
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
                                      t=[part, fu, wtab, stab, meta, None, row_partidx, row_gate],
                                      i=[H, I, Ea, enc, 0, 0, 0, arm]))

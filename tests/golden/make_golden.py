@@ -195,6 +195,16 @@ def main():
     run(abi.inst(153, t=[0, 1, 2, 3, 4, None, 6, 7], i=[K, I, E]), [partg, fug, Wd, Sd, al[0], None, al[3], al[4]], nblk=3)
     out.update({"mxflat/pf_fu": fug, "mxflat/pf_part": partg})
 
+    # --- pair-form activations on the flat mxfp4 GLU ops (drawn after everything above): 2 situ
+    # (beta, linear beta) and 3 swiglu_oai (alpha, limit) with biases, decode (150) and gathered rows (152)
+    for act, f in ((2, (2.0, 1.5)), (3, (1.702, 7.0)), (2, (3.0, 0.0))):
+        fu = np.zeros((B * k, I), np.uint16)
+        run(abi.inst(150, t=[0, 1, 2, 3, 4, 5], i=[k, I, K, E, 1, act, B], f=f), [fu, x, tab, Wgu, Sgu, bgu], nblk=2)
+        out[f"mxflat/fu_act{act}_{f[0]}_{f[1]}"] = fu
+    fug = np.zeros((rows, I), np.uint16)
+    run(abi.inst(152, t=[0, 1, 2, 3, 4, 5, 6], i=[I, K, E, 0, 0, 3], f=(1.702, 7.0)), [fug, x, Wgu, Sgu, al[0], al[2], bgu], nblk=3)
+    out["mxflat/pf_fu_act3"] = fug
+
     path = os.path.join(HERE, "plow_cpu_golden.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

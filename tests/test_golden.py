@@ -162,6 +162,39 @@ def test_flat_mxfp4_ops(oracle):
     assert np.array_equal(partg.view(np.uint32), G["mxflat/pf_part"].view(np.uint32))
 
 
+def test_flat_mxfp4_pair_activations(oracle):
+    """Activations that transform the up branch too (2 situ, 3 swiglu_oai) with their immediates in
+    fj[0] / fj[1], against plow's CPU kernels on ops 150 and 152; a clamp activation (4, plow's AMD path
+    only) against the silu path it reduces to."""
+    Wgu, Sgu = np.ascontiguousarray(G["mxdec/Wgu"]), np.ascontiguousarray(G["mxdec/Sgu"])
+    x, tab, bgu = G["mxdec/x"], as_route(G["mxdec/table"]), G["mxflat/bias_gu"]
+    E, I2, K2 = Wgu.shape
+    I, K, B, k = I2 // 2, K2 * 2, x.shape[0], 2
+    for act, f in ((2, (2.0, 1.5)), (3, (1.702, 7.0)), (2, (3.0, 0.0))):
+        fu = np.zeros((B * k, I), np.uint16)
+        run(oracle, abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4, 5], i=[k, I, K, E, 1, act, B], f=f),
+            [fu, x, tab, Wgu, Sgu, bgu], 2)
+        assert np.array_equal(fu, G[f"mxflat/fu_act{act}_{f[0]}_{f[1]}"]), (act, f)
+    al = cases.align_arrays(tab, B, E, k)
+    run(oracle, cases.align_inst(B, E, k), al, 1)
+    fug = np.zeros_like(G["mxflat/pf_fu_act3"])
+    run(oracle, abi.inst(abi.OP_MOE_GLU_MX_PF, t=[0, 1, 2, 3, 4, 5, 6], i=[I, K, E, 0, 0, 3], f=(1.702, 7.0)),
+        [fug, x, Wgu, Sgu, al[0], al[2], bgu], 3)
+    assert np.array_equal(fug, G["mxflat/pf_fu_act3"])
+    # swiglu_oai with a limit <= 0 poisons
+    fu = np.zeros((B * k, I), np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4, 5], i=[k, I, K, E, 1, 3, B], f=(1.702, 0.0)),
+        [fu, x, tab, Wgu, Sgu, bgu], 2)
+    live = as_route(G["mxdec/table"])["eid"] < E
+    assert np.all((fu[live] & 0x7FFF) > 0x7F80)
+    # the clamp activation with a limit beyond every value is silu(g) * u
+    fa, fb = np.zeros((B * k, I), np.uint16), np.zeros((B * k, I), np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4, 5], i=[k, I, K, E, 1, 4, B], f=(0.0, 1e30)),
+        [fa, x, tab, Wgu, Sgu, bgu], 2)
+    run(oracle, abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4, 5], i=[k, I, K, E, 1, 1, B]), [fb, x, tab, Wgu, Sgu, bgu], 2)
+    assert np.array_equal(fa, fb)
+
+
 def test_per_channel_fp8_decode_experts(oracle):
     gu8, d8 = np.ascontiguousarray(G["pcdec/gu8"]), np.ascontiguousarray(G["pcdec/d8"])
     sgu, sd = np.ascontiguousarray(G["pcdec/sgu"]), np.ascontiguousarray(G["pcdec/sd"])

@@ -77,6 +77,16 @@ def test_mxfp4_w4a16_layer(moe, oracle, T):
     check_chain(*both(moe, oracle, cfg, seed=T))
 
 
+@pytest.mark.parametrize("enc,act,f", [("mxfp4", 2, (2.0, 1.5)), ("fp8blk", 4, (0.0, 0.75)), ("bf16", 4, (0.0, 0.5))])
+def test_pair_form_activations_bf16_arm(moe, oracle, enc, act, f):
+    """Op 85 with bf16 activations under the activations that transform the up branch too (2 situ,
+    4 clamped SwiGLU with a limit small enough to clamp)."""
+    print(f"[case] a16 enc={enc} act={act} f={f}", flush=True)
+    cfg = layer.MoeConfig("a16-act", T=20, scoring="sigmoid", norm_topk=True, bias=True, enc=enc, arm="a16",
+                          n_shared=1, shared_mode="fold", act=act, act_f=f, **MINI)
+    check_chain(*both(moe, oracle, cfg, seed=7 + act))
+
+
 @pytest.mark.parametrize("arm", ["a16", "w8a8"])
 @pytest.mark.parametrize("T", [2, 50])
 def test_per_channel_fp8_layer(moe, oracle, T, arm):
@@ -230,8 +240,10 @@ def test_dense_ops_against_oracle(moe, oracle):
     close(ol.bf2f(yg[1:]), ol.bf2f(y_h[1:]), "dense y")
 
 
-@pytest.mark.parametrize("layout,with_bias,act", [(1, False, 1), (0, True, 0), (0, False, 1), (1, True, 1)])
-def test_flat_mxfp4_ops(moe, oracle, layout, with_bias, act):
+# the last three: activations that transform the up branch too (2 situ, 3 swiglu_oai), immediates in fj[0..1]
+@pytest.mark.parametrize("layout,with_bias,act,fimm", [(1, False, 1, ()), (0, True, 0, ()), (0, False, 1, ()), (1, True, 1, ()),
+                                                        (0, True, 3, (1.702, 7.0)), (1, True, 2, (2.0, 1.5)), (1, False, 2, (3.0, 0.0))])
+def test_flat_mxfp4_ops(moe, oracle, layout, with_bias, act, fimm):
     """Reference ops 150 - 153 (flat [E][rows][K/2] tensors, blocked or interleaved gate / up rows, optional
     per-expert bias): slot-major decode incl. a sentinel slot, then the gathered-row twins after op 84."""
     print(f"[case] flat mxfp4 layout={layout} bias={with_bias} act={act}", flush=True)
@@ -249,7 +261,7 @@ def test_flat_mxfp4_ops(moe, oracle, layout, with_bias, act):
     tab["eid"][3] = abi.EXPERT_UNUSED
     tab["gate"] = (r.random(B * k) + 0.1).astype(np.float32)
     tb = 5 if with_bias else None
-    glu = abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4, tb], i=[k, I, K, E, layout, act, B])
+    glu = abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4, tb], i=[k, I, K, E, layout, act, B], f=fimm)
     down = abi.inst(abi.OP_MOE_DOWN_MX, t=[0, 1, 2, 3, 4, tb], i=[k, K, I, E, 0, 0, B])
     fu_h = np.full((B * k, I), 0x1234, np.uint16)
     part_h = np.full((B * k, K), 9.0, np.float32)
@@ -272,7 +284,7 @@ def test_flat_mxfp4_ops(moe, oracle, layout, with_bias, act):
     al = cases.align_arrays(tab, B, E, k)
     ol.run(oracle.plow_oracle_exec, cases.align_inst(B, E, k), ol.table_of(al), 1)
     rows = len(al[2])
-    glu_pf = abi.inst(abi.OP_MOE_GLU_MX_PF, t=[0, 1, 2, 3, 4, 5, 6 if with_bias else None], i=[I, K, E, layout, 0, act])
+    glu_pf = abi.inst(abi.OP_MOE_GLU_MX_PF, t=[0, 1, 2, 3, 4, 5, 6 if with_bias else None], i=[I, K, E, layout, 0, act], f=fimm)
     down_pf = abi.inst(abi.OP_MOE_DOWN_MX_PF, t=[0, 1, 2, 3, 4, 5 if with_bias else None, 6, 7], i=[K, I, E])
     fug_h = np.full((rows, I), 0x1234, np.uint16)
     partg_h = np.full((B * k, K), 9.0, np.float32)
@@ -297,7 +309,9 @@ def test_flat_mxfp4_refusals(moe):
     t = dev_table([torch.zeros(8, device="cuda")] * 8)
     ok = abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 1, 1, 3])
     assert moe.check(ok, t) == 0
-    assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 1, 3, 3]), t) == abi.E_UNSUPPORTED
+    assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 1, 3, 3], f=(1.702, 7.0)), t) == 0
+    assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 1, 4, 3]), t) == abi.E_UNSUPPORTED
+    assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 1, 5, 3]), t) == abi.E_UNSUPPORTED
     assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 128, 256, 4, 2, 1, 3]), t) == abi.E_INVAL
     assert moe.check(abi.inst(abi.OP_MOE_GLU_MX, t=[0, 1, 2, 3, 4], i=[2, 64, 256, 4, 1, 1, 3]), t) == abi.E_INVAL
     assert moe.check(abi.inst(abi.OP_MOE_DOWN_MX_PF, t=[0, 1, 2, 3, 4], i=[256, 128, 4]), t) == abi.E_INVAL

@@ -49,6 +49,16 @@ def test_small_dsv3_like_layer(moe, oracle, T):
     check_layer(*both(moe, oracle, cfg, seed=T))
 
 
+@pytest.mark.parametrize("T,act,f", [(24, 2, (2.0, 1.5)), (24, 4, (0.0, 0.75)), (600, 2, (3.0, 0.0)), (600, 4, (0.0, 0.75))])
+def test_pair_form_activations(moe, oracle, T, act, f):
+    """Activations that transform the up branch too on op 85's block-fp8 W8A8 arm: 2 situ (beta, linear
+    beta) and 4 clamped SwiGLU (limit in fj[1], small enough here to clamp), streaming and tiled forms."""
+    print(f"[case] w8a8 act={act} f={f} T={T}", flush=True)
+    cfg = layer.MoeConfig("mini-act", H=512, E=8, I=256, k=2, T=T, scoring="sigmoid", norm_topk=True,
+                          bias=True, enc="fp8blk", arm="w8a8", n_shared=1, shared_mode="fold", act=act, act_f=f)
+    check_layer(*both(moe, oracle, cfg, seed=T + act))
+
+
 def test_rows_per_expert_beyond_one_tile(moe, oracle):
     """Few experts, many tokens: segments of 17..300 rows walk every row-tile arm of the kernel."""
     cfg = layer.MoeConfig("dense-ish", H=256, E=4, I=128, k=2, T=300, scoring="softmax",
