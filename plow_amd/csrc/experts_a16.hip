@@ -288,14 +288,21 @@ template <> struct DmGeom<AENC_MXFP4> { static constexpr uint32_t KSTEP = 256u; 
 template <> struct DmGeom<AENC_FP8PC> { static constexpr uint32_t KSTEP = 128u; };
 template <> struct DmGeom<AENC_FP8BLK> { static constexpr uint32_t KSTEP = 128u; };
 template <> struct DmGeom<AENC_BF16> { static constexpr uint32_t KSTEP = 64u; };
-struct DmWSlot {
+template <bool MX> struct DmWSlot;
+template <> struct DmWSlot<true> {
     uint8_t w[2][16u * 128u]; /* [stream][row][128 B] */
     uint8_t sc[2][256];       /* mxfp4: [stream][row][8 B]; lanes 32..63 write copies behind */
 };
-template <int ENC>
+template <> struct DmWSlot<false> {
+    uint8_t w[2][16u * 128u];
+};
+/* RG = 16-row groups of activation rows per pass over the weights (1 for decode; 4 when experts have
+ * many rows: the weights are then streamed a quarter as often and every weight operand read from LDS
+ * feeds four matrix instructions) */
+template <int ENC, int RG>
 struct DmLds {
-    uint8_t x[DM_STAGES][16u * DmGeom<ENC>::KSTEP * 2u];
-    DmWSlot ring[AK_WAVES][DM_STAGES];
+    uint8_t x[DM_STAGES][RG * 16u * DmGeom<ENC>::KSTEP * 2u];
+    DmWSlot<ENC == AENC_MXFP4> ring[AK_WAVES][DM_STAGES];
     float bsc[4][2][128]; /* block-fp8: the weight block scales of the workgroup's tiles, all of K (K <= 16384) */
 };
 typedef __attribute__((address_space(3))) void dm_lds_void;
@@ -321,16 +328,19 @@ __device__ __forceinline__ float dm_read4(uint32_t addr) {
  * workgroup barrier */
 #define DM_WAIT_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory")
 
-template <int ENC, bool GLU>
+template <int ENC, bool GLU, int RG>
 __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
-    DmLds<ENC>& L = *(DmLds<ENC>*)dm_raw;
+    DmLds<ENC, RG>& L = *(DmLds<ENC, RG>*)dm_raw;
+    typedef DmWSlot<ENC == AENC_MXFP4> Slot;
     constexpr uint32_t KSTEP = DmGeom<ENC>::KSTEP, XROW = KSTEP * 2u; /* activation bytes per row and step */
     constexpr uint32_t NP = XROW / 16u;                              /* 16-byte pieces per activation row */
-    constexpr uint32_t XL = 16u * XROW / 1024u;                      /* waves that load activation rows */
+    constexpr uint32_t XL = RG * 16u * XROW / 1024u;                 /* 1 KB activation loads per step */
     constexpr uint32_t XRPL = 64u / NP;                              /* rows per activation load */
+    constexpr uint32_t NXI = (XL + AK_WAVES - 1u) / AK_WAVES;        /* activation loads per wave and step (wave w: w, w + 8, ..) */
+    static_assert(XL < AK_WAVES || XL % AK_WAVES == 0u, "activation loads must split evenly over the waves");
     constexpr int NS = GLU ? 2 : 1;
-    /* direct loads per wave and step: weights 2 per stream, mxfp4 scales 1 per stream, rows 1 (first XL waves) */
+    /* direct loads per wave and step: weights 2 per stream, mxfp4 scales 1 per stream, rows NXI (waves below XL) */
     constexpr int NLW = NS * (ENC == AENC_MXFP4 ? 3 : 2);
     const uint32_t tiles = g.N / AK_BN;
     /* With plenty of tiles to go round and a short K loop, a workgroup takes TPW consecutive channel tiles
@@ -393,28 +403,41 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     /* LDS position of logical piece P of activation row c */
     auto xpos = [&](uint32_t P) -> uint32_t { return NP >= 16u ? ((P & ~15u) | ((P ^ c) & 15u)) : (P ^ swz); };
 
-    for (uint32_t rb = 0; rb < cnt; rb += 16u) {
-        /* this wave's share of the pass's rows (waves 0 .. XL - 1): XRPL rows, NP lanes each; a pad row
-         * reads the pass's first row and is never stored */
-        const uint32_t xrow = XRPL * wv + lane / NP, pc = lane % NP;
-        const uint8_t* xsrc = nullptr;
-        if (wv < XL) {
+    for (uint32_t rb = 0; rb < cnt; rb += 16u * RG) {
+        /* this wave's share of the pass's rows: load i covers rows XRPL * (wv + 8 i) .., NP lanes each; a pad
+         * row reads the pass's first row and is never stored */
+        const uint32_t pc = lane % NP;
+        const uint8_t* xsrc[NXI];
+        {
             const uint32_t first = g.a_idx ? g.a_idx[r0 + rb] : r0 + rb;
-            const uint32_t off = rb + xrow;
-            uint32_t ai = off < cnt ? (g.a_idx ? g.a_idx[r0 + off] : r0 + off) : PLOW_EXPERT_UNUSED;
-            if (ai == PLOW_EXPERT_UNUSED) ai = first == PLOW_EXPERT_UNUSED ? 0u : first;
-            const uint32_t gp = NP >= 16u ? ((pc & ~15u) | ((pc ^ xrow) & 15u)) : (pc ^ ((xrow >> 1) & 7u));
-            xsrc = (const uint8_t*)g.a + (size_t)ai * K * 2u + (gp << 4);
+#pragma unroll
+            for (uint32_t i = 0; i < NXI; i++) {
+                const uint32_t xrow = XRPL * (wv + AK_WAVES * i) + lane / NP;
+                xsrc[i] = nullptr;
+                if (wv + AK_WAVES * i < XL) {
+                    const uint32_t off = rb + xrow;
+                    uint32_t ai = off < cnt ? (g.a_idx ? g.a_idx[r0 + off] : r0 + off) : PLOW_EXPERT_UNUSED;
+                    if (ai == PLOW_EXPERT_UNUSED) ai = first == PLOW_EXPERT_UNUSED ? 0u : first;
+                    const uint32_t gp = NP >= 16u ? ((pc & ~15u) | ((pc ^ xrow) & 15u)) : (pc ^ ((xrow >> 1) & 7u));
+                    xsrc[i] = (const uint8_t*)g.a + (size_t)ai * K * 2u + (gp << 4);
+                }
+            }
         }
-        /* the B-operand row of this lane */
-        const uint32_t off = rb + c, r = r0 + off;
-        bool valid = off < cnt;
-        const uint32_t ai_c = valid ? (g.a_idx ? g.a_idx[r] : r) : PLOW_EXPERT_UNUSED;
-        valid = ai_c != PLOW_EXPERT_UNUSED;
-        /* what the epilogues need from memory is read here, before the rings start: an ordinary load
-         * inside the stream would make the compiler wait for every outstanding direct load */
-        const uint32_t oi = valid ? (g.o_idx ? g.o_idx[r] : r) : PLOW_EXPERT_UNUSED;
-        const float gate = (!GLU && valid && g.gate) ? g.gate[r] : 1.0f;
+        /* the B-operand rows of this lane: row c of each 16-row group */
+        bool valid[RG];
+        uint32_t oi[RG];
+        float gate[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const uint32_t off = rb + 16u * (uint32_t)rg + c, r = r0 + off;
+            valid[rg] = off < cnt;
+            const uint32_t ai_c = valid[rg] ? (g.a_idx ? g.a_idx[r] : r) : PLOW_EXPERT_UNUSED;
+            valid[rg] = ai_c != PLOW_EXPERT_UNUSED;
+            /* what the epilogues need from memory is read here, before the rings start: an ordinary load
+             * inside the stream would make the compiler wait for every outstanding direct load */
+            oi[rg] = valid[rg] ? (g.o_idx ? g.o_idx[r] : r) : PLOW_EXPERT_UNUSED;
+            gate[rg] = (!GLU && valid[rg] && g.gate) ? g.gate[r] : 1.0f;
+        }
         float4 pc0[4], pc1[4];
         if (ENC == AENC_FP8PC) {
 #pragma unroll
@@ -429,7 +452,8 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
 
         /* a use the compiler cannot move: its own wait for these loads lands here and not behind the
          * first direct loads */
-        asm volatile("" ::"v"(oi), "v"(gate));
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) asm volatile("" ::"v"(oi[rg]), "v"(gate[rg]));
         if (ENC == AENC_FP8PC) {
 #pragma unroll
             for (int t = 0; t < 4; t++) asm volatile("" ::"v"(pc0[t].x), "v"(pc0[t].w), "v"(pc1[t].x), "v"(pc1[t].w));
@@ -438,7 +462,7 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
         /* the load cursor walks (tile, step) in order; ring slots follow the running step count */
         uint32_t ld_t = 0, ld_S = 0, ld_st = 0;
         auto issue = [&]() {
-            DmWSlot* slot = &L.ring[wv][ld_st];
+            Slot* slot = &L.ring[wv][ld_st];
             const size_t wofs = (size_t)ld_t * AK_BN * wmul * wrow + (size_t)ld_S * 128u;
 #pragma unroll
             for (int sidx = 0; sidx < NS; sidx++) {
@@ -446,17 +470,21 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
                 for (uint32_t j = 0; j < 2u; j++)
                     __builtin_amdgcn_global_load_lds((const void*)(wsrc[sidx][j] + wofs),
                                                      (dm_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, 0);
-                if (ENC == AENC_MXFP4)
+                if constexpr (ENC == AENC_MXFP4)
                     __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)ld_t * AK_BN * wmul * (K / 32u) + (size_t)ld_S * 8u),
                                                      (dm_lds_void*)&slot->sc[sidx][0], 4, 0, 0);
             }
-            if (wv < XL)
-                __builtin_amdgcn_global_load_lds((const void*)(xsrc + (size_t)ld_S * XROW),
-                                                 (dm_lds_void*)&L.x[ld_st][XRPL * wv * XROW], 16, 0, 0);
+#pragma unroll
+            for (uint32_t i = 0; i < NXI; i++)
+                if (wv + AK_WAVES * i < XL)
+                    __builtin_amdgcn_global_load_lds((const void*)(xsrc[i] + (size_t)ld_S * XROW),
+                                                     (dm_lds_void*)&L.x[ld_st][XRPL * (wv + AK_WAVES * i) * XROW], 16, 0, 0);
             ld_st = ld_st + 1u == DM_STAGES ? 0u : ld_st + 1u;
             if (++ld_S == KS) ld_S = 0u, ld_t++;
         };
-        v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
+        v4f acc0[RG], acc1[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) acc0[rg] = acc1[rg] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
         /* the row maps above are loaded (the count of outstanding loads starts at zero), and every wave
          * has left the pass before (its ring slots are free; the block scales are written) */
         DM_WAIT_BARRIER(0);
@@ -467,62 +495,81 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
             /* loads return in order: step G has landed once at most step G + 1's are outstanding; after the
              * barrier every wave's share of the rows is there and nobody reads step G - 1 any more */
             if (G + 1u >= GS) DM_WAIT_BARRIER(0);
-            else if (wv < XL) DM_WAIT_BARRIER(NLW + 1);
+            else if (XL >= AK_WAVES || wv < XL) DM_WAIT_BARRIER(NLW + (int)NXI);
             else DM_WAIT_BARRIER(NLW);
             if (G + 2u < GS) issue();
-            const uint32_t wb = w_base + st * (uint32_t)sizeof(DmWSlot), xb = x_base + st * (16u * XROW) + c * XROW;
-            if (ENC == AENC_MXFP4) {
+            const uint32_t wb = w_base + st * (uint32_t)sizeof(Slot), xb0 = x_base + st * (RG * 16u * XROW) + c * XROW;
+            /* the weight operands of the step are read once and multiply every row group of the pass */
+            if constexpr (ENC == AENC_MXFP4) {
                 uint2 e0 = dm_read8(wb + 4096u + c * 8u), e1 = e0;
                 if (GLU) e1 = dm_read8(wb + 4096u + 256u + c * 8u);
-                v4i wa[2], wbv[2], xa[2][4];
+                v4i wa[2], wbv[2];
 #pragma unroll
                 for (uint32_t u = 0; u < 2u; u++) {
                     const uint32_t wo = c * 128u + (((4u * u + q) ^ swz) << 4);
                     wa[u] = dm_read16(wb + wo);
                     wbv[u] = wa[u];
                     if (GLU) wbv[u] = dm_read16(wb + 2048u + wo);
-#pragma unroll
-                    for (uint32_t j = 0; j < 4u; j++) xa[u][j] = dm_read16(xb + (xpos(16u * u + 4u * q + j) << 4));
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e0), "+v"(e1), "+v"(wa[0]), "+v"(wa[1]), "+v"(wbv[0]), "+v"(wbv[1]));
-                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0][0]), "+v"(xa[0][1]), "+v"(xa[0][2]), "+v"(xa[0][3]));
-                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[1][0]), "+v"(xa[1][1]), "+v"(xa[1][2]), "+v"(xa[1][3]));
 #pragma unroll
-                for (uint32_t u = 0; u < 2u; u++) {
-                    const uint32_t s0 = ((u ? e0.y : e0.x) >> (8u * q)) & 0xFFu, s1 = ((u ? e1.y : e1.x) >> (8u * q)) & 0xFFu;
-                    WStep<AENC_MXFP4> da, db;
-                    da.r[0] = wa[u];
-                    db.r[0] = wbv[u];
+                for (int rg = 0; rg < RG; rg++) {
+                    const uint32_t xb = xb0 + (uint32_t)rg * (16u * XROW);
+                    v4i xa[2][4];
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const v8bf B = __builtin_bit_cast(v8bf, xa[u][j]);
-                        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(da, j, s0), B, acc0, 0, 0, 0);
-                        if (GLU) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(db, j, s1), B, acc1, 0, 0, 0);
+                    for (uint32_t u = 0; u < 2u; u++)
+#pragma unroll
+                        for (uint32_t j = 0; j < 4u; j++) xa[u][j] = dm_read16(xb + (xpos(16u * u + 4u * q + j) << 4));
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0][0]), "+v"(xa[0][1]), "+v"(xa[0][2]), "+v"(xa[0][3]));
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[1][0]), "+v"(xa[1][1]), "+v"(xa[1][2]), "+v"(xa[1][3]));
+#pragma unroll
+                    for (uint32_t u = 0; u < 2u; u++) {
+                        const uint32_t s0 = ((u ? e0.y : e0.x) >> (8u * q)) & 0xFFu, s1 = ((u ? e1.y : e1.x) >> (8u * q)) & 0xFFu;
+                        WStep<AENC_MXFP4> da, db;
+                        da.r[0] = wa[u];
+                        db.r[0] = wbv[u];
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const v8bf B = __builtin_bit_cast(v8bf, xa[u][j]);
+                            acc0[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(da, j, s0), B, acc0[rg], 0, 0, 0);
+                            if (GLU) acc1[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(db, j, s1), B, acc1[rg], 0, 0, 0);
+                        }
                     }
                 }
-            } else if (ENC == AENC_BF16) {
+            } else if constexpr (ENC == AENC_BF16) {
                 /* 64 k: instruction j uses k = 32 j + 8 q .. + 8 of both operands */
-                v4i wa[2], wbv[2], xa[2];
+                v4i wa[2], wbv[2];
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; j++) {
                     const uint32_t wo = c * 128u + (((4u * j + q) ^ swz) << 4);
                     wa[j] = dm_read16(wb + wo);
                     wbv[j] = wa[j];
                     if (GLU) wbv[j] = dm_read16(wb + 2048u + wo);
-                    xa[j] = dm_read16(xb + (xpos(4u * j + q) << 4));
                 }
-                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wa[0]), "+v"(wa[1]), "+v"(wbv[0]), "+v"(wbv[1]), "+v"(xa[0]), "+v"(xa[1]));
+                v4i xr[2][2];
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const v8bf B = __builtin_bit_cast(v8bf, xa[j]);
-                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wa[j]), B, acc0, 0, 0, 0);
-                    if (GLU) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wbv[j]), B, acc1, 0, 0, 0);
+                for (uint32_t j = 0; j < 2u; j++) xr[0][j] = dm_read16(xb0 + (xpos(4u * j + q) << 4));
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wa[0]), "+v"(wa[1]), "+v"(wbv[0]), "+v"(wbv[1]));
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) {
+                    v4i* const xa = xr[rg & 1];
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0]), "+v"(xa[1]));
+                    if (rg + 1 < RG) {
+                        const uint32_t xb = xb0 + (uint32_t)(rg + 1) * (16u * XROW);
+#pragma unroll
+                        for (uint32_t j = 0; j < 2u; j++) xr[(rg + 1) & 1][j] = dm_read16(xb + (xpos(4u * j + q) << 4));
+                    }
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const v8bf B = __builtin_bit_cast(v8bf, xa[j]);
+                        acc0[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wa[j]), B, acc0[rg], 0, 0, 0);
+                        if (GLU) acc1[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wbv[j]), B, acc1[rg], 0, 0, 0);
+                    }
                 }
             } else {
                 /* fp8, 128 k: the lane's weight bytes are [16q, 16q + 16) and [64 + 16q, 64 + 16q + 16);
                  * instruction j uses bytes 8 (j & 1) .. + 8 of half j >> 1 */
                 WStep<ENC> da, db;
-                v4i xa[4];
                 float sa = 1.0f, sb = 1.0f;
 #pragma unroll
                 for (uint32_t h = 0; h < 2u; h++) {
@@ -531,32 +578,43 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
                     db.r[h] = da.r[h];
                     if (GLU) db.r[h] = dm_read16(wb + 2048u + wo);
                 }
-#pragma unroll
-                for (uint32_t j = 0; j < 4u; j++) xa[j] = dm_read16(xb + (xpos(8u * (j >> 1) + 2u * q + (j & 1u)) << 4));
                 if (ENC == AENC_FP8BLK) {
                     sa = dm_read4(b_base + t * 1024u + S * 4u);
                     sb = sa;
                     if (GLU) sb = dm_read4(b_base + t * 1024u + 512u + S * 4u);
                 }
+                /* the rows of group rg + 1 are read from LDS while group rg multiplies */
+                v4i xr[2][4];
+#pragma unroll
+                for (uint32_t j = 0; j < 4u; j++) xr[0][j] = dm_read16(xb0 + (xpos(8u * (j >> 1) + 2u * q + (j & 1u)) << 4));
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(da.r[0]), "+v"(da.r[1]), "+v"(db.r[0]), "+v"(db.r[1]), "+v"(sa), "+v"(sb));
-                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0]), "+v"(xa[1]), "+v"(xa[2]), "+v"(xa[3]));
-                v4f t0 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc0;
-                v4f t1 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc1;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v8bf B = __builtin_bit_cast(v8bf, xa[j]);
-                    t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(da, j), B, t0, 0, 0, 0);
-                    if (GLU) t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(db, j), B, t1, 0, 0, 0);
-                }
-                if (ENC == AENC_FP8BLK) {
+                for (int rg = 0; rg < RG; rg++) {
+                    v4i* const xa = xr[rg & 1];
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0]), "+v"(xa[1]), "+v"(xa[2]), "+v"(xa[3]));
+                    if (rg + 1 < RG) {
+                        const uint32_t xb = xb0 + (uint32_t)(rg + 1) * (16u * XROW);
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        acc0[i] = fmaf(t0[i], sa, acc0[i]);
-                        if (GLU) acc1[i] = fmaf(t1[i], sb, acc1[i]);
+                        for (uint32_t j = 0; j < 4u; j++) xr[(rg + 1) & 1][j] = dm_read16(xb + (xpos(8u * (j >> 1) + 2u * q + (j & 1u)) << 4));
                     }
-                } else {
-                    acc0 = t0;
-                    if (GLU) acc1 = t1;
+                    v4f t0 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc0[rg];
+                    v4f t1 = ENC == AENC_FP8BLK ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : acc1[rg];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const v8bf B = __builtin_bit_cast(v8bf, xa[j]);
+                        t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(da, j), B, t0, 0, 0, 0);
+                        if (GLU) t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(db, j), B, t1, 0, 0, 0);
+                    }
+                    if (ENC == AENC_FP8BLK) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            acc0[rg][i] = fmaf(t0[i], sa, acc0[rg][i]);
+                            if (GLU) acc1[rg][i] = fmaf(t1[i], sb, acc1[rg][i]);
+                        }
+                    } else {
+                        acc0[rg] = t0;
+                        if (GLU) acc1[rg] = t1;
+                    }
                 }
             }
             st = st + 1u == DM_STAGES ? 0u : st + 1u;
@@ -564,36 +622,40 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
             /* ---- a tile is done: lane holds channels chw + 128 t + 4q + i of row rb + c ---- */
             const uint32_t tdone = t;
             S = 0u, t++;
-            if (!valid) continue;
             const uint32_t col = chw + tdone * AK_BN + 4u * q;
+            float4 s0 = pc0[0], s1 = pc1[0];
             if (ENC == AENC_FP8PC) {
-                float4 s0 = pc0[0], s1 = pc1[0];
 #pragma unroll
                 for (uint32_t t2 = 1; t2 < 4u; t2++)
                     if (tdone == t2) s0 = pc0[t2], s1 = pc1[t2];
-                acc0[0] *= s0.x, acc0[1] *= s0.y, acc0[2] *= s0.z, acc0[3] *= s0.w;
-                if (GLU) acc1[0] *= s1.x, acc1[1] *= s1.y, acc1[2] *= s1.z, acc1[3] *= s1.w;
             }
-            if (oi != PLOW_EXPERT_UNUSED) {
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                v4f a0 = acc0[rg], a1 = acc1[rg];
+                acc0[rg] = acc1[rg] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+                if (!valid[rg] || oi[rg] == PLOW_EXPERT_UNUSED) continue;
+                if (ENC == AENC_FP8PC) {
+                    a0[0] *= s0.x, a0[1] *= s0.y, a0[2] *= s0.z, a0[3] *= s0.w;
+                    if (GLU) a1[0] *= s1.x, a1[1] *= s1.y, a1[2] *= s1.z, a1[3] *= s1.w;
+                }
                 if (GLU) {
                     uint2 o;
-                    o.x = (uint32_t)f2bf(moe_glu(acc0[0], acc1[0], g.act, g.f0, g.f1)) | ((uint32_t)f2bf(moe_glu(acc0[1], acc1[1], g.act, g.f0, g.f1)) << 16);
-                    o.y = (uint32_t)f2bf(moe_glu(acc0[2], acc1[2], g.act, g.f0, g.f1)) | ((uint32_t)f2bf(moe_glu(acc0[3], acc1[3], g.act, g.f0, g.f1)) << 16);
-                    *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
+                    o.x = (uint32_t)f2bf(moe_glu(a0[0], a1[0], g.act, g.f0, g.f1)) | ((uint32_t)f2bf(moe_glu(a0[1], a1[1], g.act, g.f0, g.f1)) << 16);
+                    o.y = (uint32_t)f2bf(moe_glu(a0[2], a1[2], g.act, g.f0, g.f1)) | ((uint32_t)f2bf(moe_glu(a0[3], a1[3], g.act, g.f0, g.f1)) << 16);
+                    *(uint2*)((bf16_t*)g.out + (size_t)oi[rg] * N + col) = o;
                 } else {
-                    const float y0 = gate * acc0[0], y1 = gate * acc0[1], y2 = gate * acc0[2], y3 = gate * acc0[3];
+                    const float gt = gate[rg];
+                    const float y0 = gt * a0[0], y1 = gt * a0[1], y2 = gt * a0[2], y3 = gt * a0[3];
                     if (g.out_bf16) {
                         uint2 o;
-                        o.x = (uint32_t)f2bf(g.gate ? y0 : acc0[0]) | ((uint32_t)f2bf(g.gate ? y1 : acc0[1]) << 16);
-                        o.y = (uint32_t)f2bf(g.gate ? y2 : acc0[2]) | ((uint32_t)f2bf(g.gate ? y3 : acc0[3]) << 16);
-                        *(uint2*)((bf16_t*)g.out + (size_t)oi * N + col) = o;
+                        o.x = (uint32_t)f2bf(g.gate ? y0 : a0[0]) | ((uint32_t)f2bf(g.gate ? y1 : a0[1]) << 16);
+                        o.y = (uint32_t)f2bf(g.gate ? y2 : a0[2]) | ((uint32_t)f2bf(g.gate ? y3 : a0[3]) << 16);
+                        *(uint2*)((bf16_t*)g.out + (size_t)oi[rg] * N + col) = o;
                     } else {
-                        *(float4*)((float*)g.out + (size_t)oi * N + col) = make_float4(y0, y1, y2, y3);
+                        *(float4*)((float*)g.out + (size_t)oi[rg] * N + col) = make_float4(y0, y1, y2, y3);
                     }
                 }
             }
-            acc0 = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
-            acc1 = acc0;
         }
     }
 }
@@ -608,17 +670,25 @@ static bool a16_dma_form() {
     return v == 1;
 }
 
-template <int ENC, bool GLU>
-static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
+template <int ENC, bool GLU, int RG>
+static int launch_a16_dma_rg(const GroupA16& g, dim3 grid, hipStream_t st) {
     static bool attr_set = false;
+    static_assert(sizeof(DmLds<ENC, RG>) <= 160u * 1024u, "the rings must fit the CU's LDS");
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)k_group_a16_dma<ENC, GLU>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)sizeof(DmLds<ENC>)) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)k_group_a16_dma<ENC, GLU, RG>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)sizeof(DmLds<ENC, RG>)) != hipSuccess)
             return PLOW_MOE_EDEVICE;
         attr_set = true;
     }
-    k_group_a16_dma<ENC, GLU><<<grid, AK_THREADS, sizeof(DmLds<ENC>), st>>>(g);
+    k_group_a16_dma<ENC, GLU, RG><<<grid, AK_THREADS, sizeof(DmLds<ENC, RG>), st>>>(g);
     return 0;
+}
+/* Experts with many rows (two dozen or more on average, from the slot count the host knows) take four
+ * 16-row groups per pass over their weights; mxfp4 keeps one (its rings leave no room for 64 rows). */
+template <int ENC, bool GLU>
+static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
+    if (ENC != AENC_MXFP4 && g.slots_hint >= 24u * g.E) return launch_a16_dma_rg<ENC, GLU, ENC == AENC_MXFP4 ? 1 : 4>(g, grid, st);
+    return launch_a16_dma_rg<ENC, GLU, 1>(g, grid, st);
 }
 
 template <bool GLU>

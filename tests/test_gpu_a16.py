@@ -98,6 +98,17 @@ def test_per_channel_fp8_layer(moe, oracle, T, arm):
     check_chain(plan, dev, host)
 
 
+@pytest.mark.parametrize("enc,arm,T,E,k", [("bf16", "a16", 300, 4, 2), ("fp8blk", "a16", 1030, 3, 1), ("fp8blk", "a16", 333, 8, 4),
+                                           ("fp8pc", "a16", 300, 4, 2), ("mxfp4", "a16", 300, 4, 2)])
+def test_bf16_activation_arms_many_rows(moe, oracle, enc, arm, T, E, k):
+    """Experts with 40..1030 rows on the bf16-activation arms: passes of four 16-row groups over the
+    weights (one for mxfp4), ragged last passes, pad rows, a folded shared expert of T rows."""
+    print(f"[case] a16 many rows enc={enc} T={T} E={E} k={k}", flush=True)
+    shared = dict(n_shared=1, shared_mode="fold") if enc != "fp8pc" else {}
+    cfg = layer.MoeConfig("a16-rows", H=384, E=E, I=256, k=k, T=T, scoring="softmax", norm_topk=True, enc=enc, arm=arm, **shared)
+    check_chain(*both(moe, oracle, cfg, seed=T))
+
+
 @pytest.mark.parametrize("T,E,k", [(300, 4, 2), (1030, 3, 1), (640, 8, 4)])
 def test_per_channel_w8a8_tiled_many_rows(moe, oracle, T, E, k):
     """Ops 81 / 82 with 60..1030 rows per expert run the tiled (prefill) form: partial, full and
