@@ -296,9 +296,9 @@ template <> struct DmWSlot<true> {
 template <> struct DmWSlot<false> {
     uint8_t w[2][16u * 128u];
 };
-/* RG = 16-row groups of activation rows per pass over the weights (1 for decode; 4 when experts have
- * many rows: the weights are then streamed a quarter as often and every weight operand read from LDS
- * feeds four matrix instructions) */
+/* RG = 16-row groups of activation rows per pass over the weights (1 for decode; 4, mxfp4 2, when
+ * experts have many rows: the weights are then streamed a quarter as often and every weight operand
+ * read from LDS feeds four matrix instructions) */
 template <int ENC, int RG>
 struct DmLds {
     uint8_t x[DM_STAGES][RG * 16u * DmGeom<ENC>::KSTEP * 2u];
@@ -684,10 +684,11 @@ static int launch_a16_dma_rg(const GroupA16& g, dim3 grid, hipStream_t st) {
     return 0;
 }
 /* Experts with many rows (two dozen or more on average, from the slot count the host knows) take four
- * 16-row groups per pass over their weights; mxfp4 keeps one (its rings leave no room for 64 rows). */
+ * 16-row groups per pass over their weights; mxfp4 two (its rings then fill the CU's LDS exactly). */
 template <int ENC, bool GLU>
 static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
-    if (ENC != AENC_MXFP4 && g.slots_hint >= 24u * g.E) return launch_a16_dma_rg<ENC, GLU, ENC == AENC_MXFP4 ? 1 : 4>(g, grid, st);
+    const bool many = g.meta ? g.slots_hint >= 24u * g.E : g.dense_rows >= 24u; /* a dense op is one expert of dense_rows rows */
+    if (many) return launch_a16_dma_rg<ENC, GLU, ENC == AENC_MXFP4 ? 2 : 4>(g, grid, st);
     return launch_a16_dma_rg<ENC, GLU, 1>(g, grid, st);
 }
 

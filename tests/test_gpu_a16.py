@@ -102,7 +102,7 @@ def test_per_channel_fp8_layer(moe, oracle, T, arm):
                                            ("fp8pc", "a16", 300, 4, 2), ("mxfp4", "a16", 300, 4, 2)])
 def test_bf16_activation_arms_many_rows(moe, oracle, enc, arm, T, E, k):
     """Experts with 40..1030 rows on the bf16-activation arms: passes of four 16-row groups over the
-    weights (one for mxfp4), ragged last passes, pad rows, a folded shared expert of T rows."""
+    weights (two for mxfp4), ragged last passes, pad rows, a folded shared expert of T rows."""
     print(f"[case] a16 many rows enc={enc} T={T} E={E} k={k}", flush=True)
     shared = dict(n_shared=1, shared_mode="fold") if enc != "fp8pc" else {}
     cfg = layer.MoeConfig("a16-rows", H=384, E=E, I=256, k=k, T=T, scoring="softmax", norm_topk=True, enc=enc, arm=arm, **shared)
