@@ -868,32 +868,53 @@ struct CombineArgs {
     uint32_t H, k, T, part16;
 };
 
+/* KT > 0: the slot count is known at compile time, so all of a token's partial rows are requested
+ * before the first is added (same order of additions); KT = 0: any k, one load at a time. */
+template <uint32_t KT>
 __global__ __launch_bounds__(256) void k_combine(CombineArgs a) {
     const uint32_t H4 = a.H / 4u;
     const size_t total = (size_t)a.T * H4;
+    const uint32_t k = KT ? KT : a.k;
     for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < total; i += (size_t)gridDim.x * 256u) {
         const uint32_t tok = (uint32_t)(i / H4), h = (uint32_t)(i % H4) * 4u;
         const size_t o = (size_t)tok * a.H + h;
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (a.residual) {
-            const uint2 r = *(const uint2*)(a.residual + o);
-            acc[0] = __uint_as_float(r.x << 16); acc[1] = __uint_as_float(r.x & 0xFFFF0000u);
-            acc[2] = __uint_as_float(r.y << 16); acc[3] = __uint_as_float(r.y & 0xFFFF0000u);
-        }
-        if (a.shared) {
-            const uint2 r = *(const uint2*)(a.shared + o);
-            acc[0] += __uint_as_float(r.x << 16); acc[1] += __uint_as_float(r.x & 0xFFFF0000u);
-            acc[2] += __uint_as_float(r.y << 16); acc[3] += __uint_as_float(r.y & 0xFFFF0000u);
-        }
-        for (uint32_t j = 0; j < a.k; j++) {
-            const size_t p = ((size_t)tok * a.k + j) * a.H + h;
-            if (a.part16) {
-                const uint2 r = *(const uint2*)((const bf16_t*)a.part + p);
-                acc[0] += __uint_as_float(r.x << 16); acc[1] += __uint_as_float(r.x & 0xFFFF0000u);
-                acc[2] += __uint_as_float(r.y << 16); acc[3] += __uint_as_float(r.y & 0xFFFF0000u);
-            } else {
-                const float4 v = *(const float4*)((const float*)a.part + p);
-                acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+        uint2 rr = make_uint2(0u, 0u), rs = make_uint2(0u, 0u);
+        if (a.residual) rr = *(const uint2*)(a.residual + o);
+        if (a.shared) rs = *(const uint2*)(a.shared + o);
+        if (KT && !a.part16) {
+            float4 v[KT ? KT : 1u];
+#pragma unroll
+            for (uint32_t j = 0; j < KT; j++) v[j] = *(const float4*)((const float*)a.part + ((size_t)tok * KT + j) * a.H + h);
+            if (a.residual) {
+                acc[0] = __uint_as_float(rr.x << 16); acc[1] = __uint_as_float(rr.x & 0xFFFF0000u);
+                acc[2] = __uint_as_float(rr.y << 16); acc[3] = __uint_as_float(rr.y & 0xFFFF0000u);
+            }
+            if (a.shared) {
+                acc[0] += __uint_as_float(rs.x << 16); acc[1] += __uint_as_float(rs.x & 0xFFFF0000u);
+                acc[2] += __uint_as_float(rs.y << 16); acc[3] += __uint_as_float(rs.y & 0xFFFF0000u);
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < KT; j++) { acc[0] += v[j].x; acc[1] += v[j].y; acc[2] += v[j].z; acc[3] += v[j].w; }
+        } else {
+            if (a.residual) {
+                acc[0] = __uint_as_float(rr.x << 16); acc[1] = __uint_as_float(rr.x & 0xFFFF0000u);
+                acc[2] = __uint_as_float(rr.y << 16); acc[3] = __uint_as_float(rr.y & 0xFFFF0000u);
+            }
+            if (a.shared) {
+                acc[0] += __uint_as_float(rs.x << 16); acc[1] += __uint_as_float(rs.x & 0xFFFF0000u);
+                acc[2] += __uint_as_float(rs.y << 16); acc[3] += __uint_as_float(rs.y & 0xFFFF0000u);
+            }
+            for (uint32_t j = 0; j < k; j++) {
+                const size_t p = ((size_t)tok * k + j) * a.H + h;
+                if (a.part16) {
+                    const uint2 r = *(const uint2*)((const bf16_t*)a.part + p);
+                    acc[0] += __uint_as_float(r.x << 16); acc[1] += __uint_as_float(r.x & 0xFFFF0000u);
+                    acc[2] += __uint_as_float(r.y << 16); acc[3] += __uint_as_float(r.y & 0xFFFF0000u);
+                } else {
+                    const float4 v = *(const float4*)((const float*)a.part + p);
+                    acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+                }
             }
         }
         uint2 w;
@@ -910,6 +931,12 @@ int launch_combine(void* out, const void* residual, const void* shared, const vo
     const size_t total = (size_t)T * (H / 4u);
     uint32_t blocks = (uint32_t)((total + 255u) / 256u);
     if (blocks > 4096u) blocks = 4096u;
-    k_combine<<<blocks, 256, 0, st>>>(a);
+    switch (part16 ? 0u : k) {
+    case 4: k_combine<4><<<blocks, 256, 0, st>>>(a); break;
+    case 6: k_combine<6><<<blocks, 256, 0, st>>>(a); break;
+    case 8: k_combine<8><<<blocks, 256, 0, st>>>(a); break;
+    case 9: k_combine<9><<<blocks, 256, 0, st>>>(a); break;
+    default: k_combine<0><<<blocks, 256, 0, st>>>(a); break;
+    }
     return 0;
 }
