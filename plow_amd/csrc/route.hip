@@ -259,6 +259,151 @@ __global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ o
     }
 }
 
+/* The same on v_mfma_f32_16x16x4_f32 (four k per instruction, a quarter of the chain latency per k of
+ * the 32x32x2 form, also bit-identical to the sequential sum): a wave computes 16 tokens x 32 experts as
+ * two independent chains that share the token operand. Half the outputs per operand byte, but twice as
+ * many, shorter-lived waves: this is the form for problems too small to fill the chip with 32 x 32
+ * tiles, where the chain latency is the time (from 2^17 outputs; below that the vector-unit form, whose
+ * chain is shorter still, wins). Lane = (row lane & 15, k lane >> 4): a lane reads the two
+ * dwords of its row's 16-byte piece that hold k = 4 h + (lane >> 4), h = 0, 1, with one ds_read2_b32. */
+#define RS16_NB 2
+struct Rs16Stage {
+    uint8_t x[16u * 128u];
+    uint8_t w[RS16_NB * 16u * 128u];
+};
+__global__ __launch_bounds__(256) void k_router_score_mfma16(float* __restrict__ out, const bf16_t* __restrict__ x,
+                                                             const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
+                                                             uint32_t K) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t rs16_raw[];
+    constexpr int NB = RS16_NB, NLD = 2 + 2 * NB; /* direct loads per chunk */
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    Rs16Stage* const ring = (Rs16Stage*)rs16_raw + wv * RSM_STAGES;
+    const uint32_t G = gridDim.x, tn_count = (N + 16u * NB - 1u) / (16u * NB), tm_count = (M + 15u) / 16u;
+    const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const uint32_t wid = wg * 4u + wv;
+    if (wid >= tn_count * tm_count) return; /* whole wave; there is no barrier below */
+    const uint32_t m0 = (wid / tn_count) * 16u, n0 = (wid % tn_count) * (16u * NB);
+    const uint32_t NC = K / 64u;
+    const uint32_t lr = lane >> 3, lp = lane & 7u;
+    const uint8_t *xsrc[2], *wsrc[2 * NB];
+#pragma unroll
+    for (uint32_t j = 0; j < 2u * NB; j++) {
+        const uint32_t row = 8u * j + lr, sw = ((row & 15u) >> 1) & 7u;
+        const uint32_t nr = n0 + row < N ? n0 + row : N - 1u;
+        wsrc[j] = (const uint8_t*)(w + (size_t)nr * K) + ((lp ^ sw) << 4);
+        if (j < 2u) {
+            const uint32_t mr = m0 + row < M ? m0 + row : M - 1u;
+            xsrc[j] = (const uint8_t*)(x + (size_t)mr * K) + ((lp ^ sw) << 4);
+        }
+    }
+    auto issue = [&](uint32_t c) {
+        Rs16Stage* s = &ring[c % RSM_STAGES];
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; j++)
+            __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u * NB; j++)
+            __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
+    };
+    const uint32_t orow = lane & 15u, ks = lane >> 4, osw = (orow >> 1) & 7u;
+    const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)&ring[0];
+    const uint32_t obase = ring0 + orow * 128u + (ks >> 1) * 4u;
+    const uint32_t sel = (ks & 1u) ? 0x03020c0cu : 0x01000c0cu;
+    v4f acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; b++) acc[b] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    /* Software pipeline over the 8-k pieces: while piece p multiplies, the reads of piece p + 1 (issued
+     * during piece p - 1) are waited for and widened into the other half of the operand registers, and
+     * the reads of piece p + 2 are issued. Everything but matrix instructions is issued behind one. */
+    uint2 xa[2], wb[2][NB];
+    float af[2][2], bf[2][NB][2];
+    auto read_piece = [&](uint32_t stage, uint32_t pc, uint32_t buf) {
+        const uint32_t addr = obase + stage * (uint32_t)sizeof(Rs16Stage) + ((pc ^ osw) << 4);
+        asm volatile("ds_read2_b32 %0, %1 offset1:2" : "=v"(xa[buf]) : "v"(addr) : "memory");
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+            asm volatile("ds_read2_b32 %0, %1 offset1:2" : "=v"(wb[buf][b]) : "v"(addr + 2048u + (uint32_t)b * 2048u) : "memory");
+    };
+    auto wait_reads = [&](uint32_t buf) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[buf]), "+v"(wb[buf][0]), "+v"(wb[buf][NB - 1])); };
+    auto widen_x = [&](uint32_t buf) {
+        af[buf][0] = __uint_as_float(__builtin_amdgcn_perm(xa[buf].x, xa[buf].x, sel));
+        af[buf][1] = __uint_as_float(__builtin_amdgcn_perm(xa[buf].y, xa[buf].y, sel));
+    };
+    auto widen_w = [&](uint32_t buf, int b) {
+        bf[buf][b][0] = __uint_as_float(__builtin_amdgcn_perm(wb[buf][b].x, wb[buf][b].x, sel));
+        bf[buf][b][1] = __uint_as_float(__builtin_amdgcn_perm(wb[buf][b].y, wb[buf][b].y, sel));
+    };
+    issue(0u);
+    if (NC > 1u) issue(1u);
+    if (NC > 2u) issue(2u);
+    if (NC > 2u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
+    else if (NC > 1u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    read_piece(0u, 0u, 0u);
+    wait_reads(0u);
+    widen_x(0u);
+#pragma unroll
+    for (int b = 0; b < NB; b++) widen_w(0u, b);
+    read_piece(0u, 1u, 1u);
+    wait_reads(1u); /* nothing is in flight across the loop's back edge */
+    uint32_t st = 0;
+#define RS16_FENCE() __builtin_amdgcn_sched_barrier(0)
+    for (uint32_t c = 0; c < NC; c++) {
+        const uint32_t stn = st == RSM_STAGES - 1u ? 0u : st + 1u;
+#pragma unroll
+        for (uint32_t pc = 0; pc < 8u; pc++) {
+            const uint32_t cur = pc & 1u, nxt = cur ^ 1u;
+            /* four matrix instructions per piece; the other work is spread over the gaps between them */
+            RS16_FENCE();
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][0], bf[cur][0][0], acc[0], 0, 0, 0);
+            RS16_FENCE();
+            wait_reads(nxt); /* piece p + 1, requested a piece ago */
+            /* piece p + 2 into the raw registers piece p came from (widened a piece ago) */
+            if (pc == 6u) {
+                /* every piece of chunk c has been read (piece 7 was waited for above): chunk c + 1 must have
+                 * landed before its first piece is read, and chunk c's stage takes chunk c + 3 */
+                if (c + 2u < NC) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                read_piece(stn, 0u, cur); /* past the last chunk: stale bytes, never used */
+            } else if (pc == 7u) {
+                read_piece(stn, 1u, cur);
+            } else {
+                read_piece(st, pc + 2u, cur);
+            }
+            RS16_FENCE();
+#pragma unroll
+            for (int b = 1; b < NB; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][0], bf[cur][b][0], acc[b], 0, 0, 0);
+            RS16_FENCE();
+            widen_x(nxt);
+            widen_w(nxt, 0);
+            RS16_FENCE();
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][1], bf[cur][0][1], acc[0], 0, 0, 0);
+            RS16_FENCE();
+#pragma unroll
+            for (int b = 1; b < NB; b++) widen_w(nxt, b);
+            RS16_FENCE();
+#pragma unroll
+            for (int b = 1; b < NB; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][1], bf[cur][b][1], acc[b], 0, 0, 0);
+            RS16_FENCE();
+            if (pc == 6u && c + 3u < NC) issue(c + 3u);
+            if (pc == 7u) wait_reads(cur); /* nothing in flight across the back edge */
+        }
+        st = stn;
+    }
+#undef RS16_FENCE
+    /* acc[b][r] = out[m0 + 4 * (lane / 16) + r][n0 + 16 b + lane % 16] */
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+        const uint32_t n = n0 + 16u * (uint32_t)b + (lane & 15u);
+#pragma unroll
+        for (uint32_t r = 0; r < 4u; r++) {
+            const uint32_t m = m0 + 4u * (lane >> 4) + r;
+            if (m < M && n < N) out[(size_t)m * N + n] = acc[b][r];
+        }
+    }
+}
+
 /* Small problems (decode). Two things bound this shape: the dependent chain of K multiply-adds per
  * output, and LDS bandwidth (every multiply-add of every lane reads a fresh operand pair). Both say
  * "spread thin": one wave per workgroup (so one wave per CU's LDS), an 8 x 8 block of outputs per
@@ -379,10 +524,39 @@ static bool score_mfma_form() {
     return v != 0;
 }
 
+/* PLOW_MOE_SCORE_MFMA32_FROM = number of outputs from which the 32 x 32 tiles are forced (0 / unset: the
+ * rule in launch_router_score decides) */
+static uint64_t score_mfma32_from() {
+    static uint64_t v = ~0ull;
+    if (v == ~0ull) {
+        const char* e = getenv("PLOW_MOE_SCORE_MFMA32_FROM");
+        v = e ? strtoull(e, nullptr, 10) : 0ull;
+    }
+    return v;
+}
+
 int launch_router_score(float* out, const void* x, const void* w, uint32_t M, uint32_t N, uint32_t K,
                         hipStream_t st) {
     if (K % 8u) return PLOW_MOE_EINVAL;
-    if ((uint64_t)M * N >= (1u << 18) && K % 64u == 0u && score_mfma_form()) {
+    /* 32 x 32 tiles (fewer operand bytes per output) when they fill the SIMDs evenly: a whole number of
+     * tiles per SIMD, or at least four; otherwise, from 2^17 outputs, the 16 x 32 tiles */
+    const uint64_t t32 = (uint64_t)((N + 31) / 32) * ((M + 31) / 32);
+    const uint64_t n_simd = 1024; /* 256 CUs x 4 */
+    const uint64_t outputs = (uint64_t)M * N, force32 = score_mfma32_from();
+    const bool mfma_ok = K % 64u == 0u && score_mfma_form();
+    const bool use32 = mfma_ok && outputs >= (1u << 18) && (force32 ? outputs >= force32 : (t32 % n_simd == 0u || t32 >= 4u * n_simd));
+    const bool use16 = mfma_ok && !use32 && outputs >= (1u << 17);
+    if (use16) {
+        static bool attr_set = false;
+        const uint32_t lds = 4u * RSM_STAGES * (uint32_t)sizeof(Rs16Stage);
+        if (!attr_set) {
+            if (hipFuncSetAttribute((const void*)k_router_score_mfma16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+                return PLOW_MOE_EDEVICE;
+            attr_set = true;
+        }
+        const uint32_t waves = ((N + 16u * RS16_NB - 1u) / (16u * RS16_NB)) * ((M + 15u) / 16u);
+        k_router_score_mfma16<<<(waves + 3u) / 4u, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+    } else if (use32) {
         static bool attr_set = false;
         const uint32_t lds = 4u * RSM_STAGES * (uint32_t)sizeof(RsmStage);
         if (!attr_set) {

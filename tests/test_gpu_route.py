@@ -98,9 +98,12 @@ def test_route_and_align_match_oracle(moe, oracle, E, k, T, flags, ng, tg, tail)
     assert np.array_equal(dev[3][:rows].view(np.uint32), al[4][:rows].view(np.uint32))
 
 
-# the last four take the matrix-unit form (M * N >= 2^18, K a multiple of 64) with 4, 2, 1 and 16 chunks
+# K a multiple of 64 and 2^17 outputs or more: the matrix-unit forms. 16 x 32 tiles with 4, 2, 1, 16 and 3
+# chunks (the fifth is ragged in both directions); the last two fill the SIMDs evenly with 32 x 32 tiles and
+# take that form (2 and 3 chunks)
 @pytest.mark.parametrize("M,N,K", [(6, 40, 768), (64, 256, 7168), (1, 384, 7168), (700, 1000, 264),
-                                   (700, 1000, 256), (520, 520, 128), (1030, 300, 64), (1500, 288, 1024)])
+                                   (700, 1000, 256), (520, 520, 128), (1030, 300, 64), (1500, 288, 1024),
+                                   (413, 331, 192), (1024, 1024, 128), (2048, 512, 192)])
 def test_router_score_bit_exact(moe, oracle, M, N, K):
     print(f"[case] score {M}x{N}x{K}", flush=True)
     if (M, N, K) == (6, 40, 768):
