@@ -151,3 +151,42 @@ def test_per_row_quant_refusals_and_poison(moe):
     q, s, xo = gpu_quant_row(moe, np.zeros_like(x), x, x, act=2)
     assert np.all((xo & 0x7F80) == 0x7F80) and np.all((xo & 0x7F) != 0)
     assert np.all((q & 0x7F) == 0x7F)
+
+
+@pytest.mark.parametrize("arm,enc,T", [("w8a8", "fp8blk", 24), ("a16", "mxfp4", 5), ("w8a8", "fp8blk", 600)])
+def test_layer_chain_replays_from_a_hip_graph(moe, arm, enc, T):
+    """The op chain of a layer allocates nothing and clears nothing through the runtime, so a caller may
+    capture it: captured once, replayed four times with new activations and other work in between, every
+    replay must equal the eager result bit for bit."""
+    from plow_amd import layer, synth
+    print(f"[case] graph replay arm={arm} enc={enc} T={T}", flush=True)
+    cfg = layer.MoeConfig("graph", H=512, E=16, I=256, k=4, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          enc=enc, arm=arm, n_shared=1, shared_mode="fold")
+    plan = layer.plan_layer(cfg)
+    dev = synth.bind(plan, "cuda", seed=11)
+    insts, table = abi.inst_array(plan.insts), dev.table()
+    moe.exec_many(insts, table, torch.cuda.current_stream().cuda_stream)   # first calls set kernel attributes
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        moe.exec_many(insts, table, side.cuda_stream)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    xs = [synth.randn_bf16((cfg.T, cfg.H), 1.0, dev.device, 500 + n) for n in range(4)]
+    for n, x in enumerate(xs):
+        dev.t["x"].copy_(x)
+        dev.t["out"].zero_()
+        moe.exec_many(insts, table, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        want_out, want_table = dev.t["out"].clone(), dev.t["table"].clone()
+        dev.t["out"].zero_()
+        dev.t["table"].zero_()
+        scratch = torch.randn(1 << 16, device="cuda").sum()       # unrelated eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dev.t["table"], want_table), f"replay {n}: routing differs"
+        assert torch.equal(dev.t["out"], want_out), f"replay {n}: output differs"
+        assert bool(torch.isfinite(scratch))
