@@ -350,7 +350,9 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
      * all XCDs) and the rest leave at once. */
     const uint32_t busy = (g.meta ? (uint32_t)g.meta[3u * g.E] : 1u) * tiles;
     const bool short_k = g.K / DmGeom<ENC>::KSTEP <= 16u; /* a long K loop amortises its ramp by itself */
-    const uint32_t TPW = !short_k ? 1u : (busy >= 4096u && tiles % 4u == 0u) ? 4u : ((busy >= 2048u && tiles % 2u == 0u) ? 2u : 1u);
+    const uint32_t TPW = !short_k ? 1u
+                         : (ENC == AENC_MXFP4 && busy >= 8192u && tiles % 8u == 0u) ? 8u /* no per-tile tables to hold */
+                         : (busy >= 4096u && tiles % 4u == 0u) ? 4u : ((busy >= 2048u && tiles % 2u == 0u) ? 2u : 1u);
     const uint32_t wpe = tiles / TPW; /* workgroups per expert */
     if (blockIdx.x >= g.E * wpe) return;
     const uint32_t e = g.E - 1u - blockIdx.x / wpe, ct = (blockIdx.x % wpe) * TPW; /* heavy (folded shared) expert first */
