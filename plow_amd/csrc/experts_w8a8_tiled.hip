@@ -32,6 +32,8 @@
  * zero activation scale; 16-row groups with no live row are skipped by the consumers.
  * Tiles are walked by persistent workgroups (one per CU) in an order that puts the tiles sharing
  * token rows and weight rows on one XCD at the same time (see the tile loop). */
+#include <stdlib.h>
+#include <string.h>
 #include "common.h"
 #include "kernels.h"
 
@@ -49,7 +51,6 @@ __device__ __forceinline__ float t5_glu(float gt, float up, uint32_t act, float 
 }
 
 #define T5_BM 128u
-#define T5_THREADS 768u /* 8 consumer waves + 4 loader waves */
 #define T5_STAGES 3u
 #define T5_NLOAD 13 /* direct loads per loader and block: 1 scale, 4 token-row, 8 weight-row */
 
@@ -128,8 +129,8 @@ __device__ unsigned long long t5_prof[2][256][8];
     const uint32_t blo = ab + op_lo, bhi = ab + op_hi;                                                       \
     const uint32_t alo = wb + op_lo, ahi = wb + op_hi;                                                       \
     const uint32_t sl = s_base + st * (T5_BM * 4u) + r16 * 4u;                                               \
-    const uint32_t cl = c_base + par * 1024u + kb * 4u;                                                      \
-    st = st == 2u ? 0u : st + 1u;
+    const uint32_t cl = c_base + par * 1024u + kb * 4u;
+#define T5_ADVANCE() st = st == 2u ? 0u : st + 1u
 #define T5_BLOCK_OPERANDS()                                                                                  \
     float ws0 = 0.0f, ws1 = 0.0f;                                                                            \
     if (!PC) {                                                                                               \
@@ -178,10 +179,11 @@ __device__ unsigned long long t5_prof[2][256][8];
     }
 #define T5_BLOCK_PARTIAL()                                                                                   \
     T5_BLOCK_HEAD()                                                                                          \
-    if (ngrp_w == 0u) continue;                                                                              \
-    T5_BLOCK_OPERANDS()                                                                                      \
-    T5_GROUP_PARTIAL(0) T5_GROUP_PARTIAL(1) T5_GROUP_PARTIAL(2) T5_GROUP_PARTIAL(3)                          \
-    T5_GROUP_PARTIAL(4) T5_GROUP_PARTIAL(5) T5_GROUP_PARTIAL(6) T5_GROUP_PARTIAL(7)
+    if (ngrp_w != 0u) {                                                                                      \
+        T5_BLOCK_OPERANDS()                                                                                  \
+        T5_GROUP_PARTIAL(0) T5_GROUP_PARTIAL(1) T5_GROUP_PARTIAL(2) T5_GROUP_PARTIAL(3)                      \
+        T5_GROUP_PARTIAL(4) T5_GROUP_PARTIAL(5) T5_GROUP_PARTIAL(6) T5_GROUP_PARTIAL(7)                      \
+    }
 
 /* Tiles with all eight row groups live: no condition anywhere, so no value is ever copied between
  * registers; in block mode the scaled adds of group RG follow the matrix instructions of group RG + 1,
@@ -231,15 +233,19 @@ __device__ unsigned long long t5_prof[2][256][8];
     T5_GROUP_FULL(7) T5_SCALE_FULL(6)                                                                        \
     T5_SCALE_FULL(7)
 
-template <bool GLU, bool PC>
-__global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+/* NCW = consumer waves: 8 (768 threads, the library's own launch) or 4 (512 threads: a wave then runs
+ * two of the eight consumers' shares one after the other in every block, for callers whose launch shape
+ * is fixed at 512 threads). The body takes its LDS as a pointer so that it can also sit in a kernel
+ * with static LDS. */
+template <bool GLU, bool PC, uint32_t NCW>
+__device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     T5Lds& L = *(T5Lds*)lds_raw;
     constexpr uint32_t BN = GLU ? 128u : 256u; /* output channels per tile */
+    constexpr uint32_t NTHR = (NCW + 4u) * 64u, SUBS = 8u / NCW;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const bool loader = wv >= 8u;
-    const uint32_t cw = loader ? wv - 8u : wv; /* loader index 0..3, or consumer index 0..7 */
+    const bool loader = wv >= NCW;
+    const uint32_t cw = loader ? wv - NCW : wv; /* loader index 0..3, or consumer wave index */
     const uint32_t NT = (g.N + BN - 1u) / BN;
     const uint32_t r16 = lane & 15u, q = lane >> 4;
 
@@ -248,19 +254,19 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
     {
         uint32_t* scan = (uint32_t*)&L.a[0][0];
         uint32_t carry = 0;
-        for (uint32_t e0 = 0; e0 < g.E; e0 += T5_THREADS) {
+        for (uint32_t e0 = 0; e0 < g.E; e0 += NTHR) {
             const uint32_t e = e0 + tid;
             const uint32_t t = e < g.E ? ((uint32_t)g.meta[g.E + e] + T5_BM - 1u) / T5_BM : 0u;
             scan[tid] = t;
             __syncthreads();
-            for (uint32_t o = 1; o < T5_THREADS; o <<= 1) {
+            for (uint32_t o = 1; o < NTHR; o <<= 1) {
                 const uint32_t v = tid >= o ? scan[tid - o] : 0u;
                 __syncthreads();
                 scan[tid] += v;
                 __syncthreads();
             }
             if (e < g.E) L.prefix[e] = carry + scan[tid];
-            carry += scan[T5_THREADS - 1u];
+            carry += scan[NTHR - 1u];
             __syncthreads();
         }
     }
@@ -373,7 +379,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                 const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
                 const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : S0;
                 const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
-                const uint32_t i = tid - 8u * 64u; /* 0..255 over the four loaders; KB <= 128 */
+                const uint32_t i = tid - NCW * 64u; /* 0..255 over the four loaders; KB <= 128 */
                 P.w0 = i < KB ? S0[(size_t)nb0 * KB + i] : 0.0f;
                 P.w1 = i < KB ? S1[(size_t)nb1 * KB + i] : 0.0f;
             }
@@ -414,7 +420,7 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
                     S.sstep = ok ? 1u : 0u;
                 }
             }
-            const uint32_t i = tid - 8u * 64u;
+            const uint32_t i = tid - NCW * 64u;
             if (i < KB) {
                 L.wsc[par][0][i] = P.w0;
                 L.wsc[par][1][i] = P.w1;
@@ -484,20 +490,25 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
         }
     } else {
         /* ================= consumers ================= */
+        /* Consumer wave w runs the shares of the logical consumers SUBS * w .. SUBS * w + SUBS - 1 (one
+         * with eight consumer waves, two with four): `cw` below is the logical consumer. */
         Tile t;
         uint32_t par = 0, st = 0;
+        const uint32_t cw0 = SUBS * cw;
         for (uint32_t tile = next_tile(wg, t); tile < total; tile = next_tile(tile + G, t), par ^= 1u) {
             PROF_STAMP(ts0);
             const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
             const uint32_t ngrp = (rows + 15u) / 16u; /* live 16-row groups */
-            const uint32_t ch0 = GLU ? nt * 128u + 16u * cw : nt * 256u + 32u * cw; /* first channel */
-            const bool wave_on = ch0 < g.N; /* DOWN: N may end mid-tile (N is a multiple of 128) */
+            /* DOWN: N may end mid-tile (N is a multiple of 128, so a wave's consumers are in or out together) */
+            const bool wave_on = (GLU ? nt * 128u + 16u * cw0 : nt * 256u + 32u * cw0) < g.N;
             const uint32_t ngrp_w = wave_on ? ngrp : 0u;
-            v4f acc[8][2];
+            v4f accs[SUBS][8][2];
 #pragma unroll
-            for (int rg = 0; rg < 8; rg++)
+            for (uint32_t sub = 0; sub < SUBS; sub++)
 #pragma unroll
-                for (int x = 0; x < 2; x++) acc[rg][x] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+                for (int rg = 0; rg < 8; rg++)
+#pragma unroll
+                    for (int x = 0; x < 2; x++) accs[sub][rg][x] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             PROF_STAMP(ts1);
 #ifdef T5_PROF
             unsigned long long ts2 = 0;
@@ -511,7 +522,13 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 #ifdef T5_PROF
                     if (kb == 0) ts2 = __builtin_readcyclecounter();
 #endif
-                    T5_BLOCK_FULL()
+#pragma unroll
+                    for (uint32_t sub = 0; sub < SUBS; sub++) {
+                        const uint32_t cw = cw0 + sub;
+                        v4f(&acc)[8][2] = accs[sub];
+                        T5_BLOCK_FULL()
+                    }
+                    T5_ADVANCE();
                     LDS_WAIT_ALL(); /* nothing of this block is still being read when the next barrier is passed */
                 }
             } else {
@@ -520,7 +537,13 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 #ifdef T5_PROF
                     if (kb == 0) ts2 = __builtin_readcyclecounter();
 #endif
-                    T5_BLOCK_PARTIAL()
+#pragma unroll
+                    for (uint32_t sub = 0; sub < SUBS; sub++) {
+                        const uint32_t cw = cw0 + sub;
+                        v4f(&acc)[8][2] = accs[sub];
+                        T5_BLOCK_PARTIAL()
+                    }
+                    T5_ADVANCE();
                     LDS_WAIT_ALL();
                 }
             }
@@ -528,146 +551,155 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
 
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
              *      group 0 and up in group 1; DOWN channel = ch0 + 16 * x + 4q + i ---- */
-            /* DOWN, f32 partials: a row's 32 channels of this wave are one 128-byte line. A 16-row group
-             * goes through LDS once so that it leaves as two stores of 8 whole lines (8 consecutive lanes
-             * per line) instead of two stores that touch 16 half lines each. The staging area is this
-             * wave's own weight slice of the ring stage it has just left: nobody else reads it, and the
-             * loaders refill it only after the next barrier. Every lane of the wave must call this. */
-            const uint32_t stg = w_base + (st >= 1u ? st - 1u : 2u) * (256u * 128u) + cw * (32u * 128u);
-            auto down_store_f32 = [&](int rg, v4f y0, v4f y1) {
-                const uint32_t buf = stg + (uint32_t)(rg & 1) * 2048u, wsw = r16 & 7u;
-                const uint32_t wr0 = buf + r16 * 128u + ((q ^ wsw) << 4), wr1 = buf + r16 * 128u + (((4u + q) ^ wsw) << 4);
-                const uint32_t lrow = lane >> 3, lp = lane & 7u; /* store layout: row lrow (+ 8), piece lp */
-                const uint32_t rd = buf + lrow * 128u + ((lp ^ (lrow & 7u)) << 4);
-                const uint32_t rowa = 16u * (uint32_t)rg + lrow, rowb = rowa + 8u;
-                const uint32_t pa = L.epi_idx[par][rowa], pb = L.epi_idx[par][rowb];
-                v4f oa, ob;
-                asm volatile("ds_write_b128 %2, %4\n\tds_write_b128 %3, %5\n\t"
-                             "ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:1024\n\t"
-                             "s_waitcnt lgkmcnt(0)"
-                             : "=&v"(oa), "=&v"(ob)
-                             : "v"(wr0), "v"(wr1), "v"(y0), "v"(y1), "v"(rd)
-                             : "memory");
-                float* const ocol = (float*)g.out + ch0 + 4u * lp;
-                if (rowa < rows && pa != PLOW_EXPERT_UNUSED)
-                    *(float4*)(ocol + (size_t)pa * g.N) = make_float4(oa[0], oa[1], oa[2], oa[3]);
-                if (rowb < rows && pb != PLOW_EXPERT_UNUSED)
-                    *(float4*)(ocol + (size_t)pb * g.N) = make_float4(ob[0], ob[1], ob[2], ob[3]);
-            };
-            if (PC) {
-                /* per-channel arm (plow runtime/amd/op_moe.h:6655-6700): g = acc * (as * wsc[n]); GLU stores
-                 * bf16(act(g) * u) and zeroes the expert's pad rows, DOWN stores gate * acc, then
-                 * * (as * wsc[h]) */
-                WG_BARRIER(); /* after the last block (pairs with the loaders') */
-                const float* es = (const float*)(uintptr_t)g.stab[(size_t)t.e * 2u + (GLU ? 0u : 1u)];
-                const uint32_t cnt_e = (uint32_t)g.meta[g.E + t.e], erow0 = r0 - (uint32_t)g.meta[t.e];
-                const uint32_t padded = ((cnt_e + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
-                if (wave_on && !GLU) {
+            const uint32_t stl = st >= 1u ? st - 1u : 2u; /* the ring stage the tile has just left */
+            if (!PC && GLU) {
+                float v[SUBS][8][4];
+#pragma unroll
+                for (uint32_t sub = 0; sub < SUBS; sub++) {
+                    const uint32_t cw = cw0 + sub;
+                    v4f(&acc)[8][2] = accs[sub];
 #pragma unroll
                     for (int rg = 0; rg < 8; rg++) {
-                        if (16u * (uint32_t)rg >= rows) break; /* uniform */
-                        const uint32_t row = 16u * (uint32_t)rg + r16;
-                        const float gate = L.epi_gate[par][row]; /* 0 for pad rows */
-                        const float as = row < rows ? g.a_scale[r0 + row] : 0.0f;
-                        v4f y[2];
+                        float m = 0.0f;
 #pragma unroll
-                        for (int x = 0; x < 2; x++) {
-                            const uint32_t col = ch0 + 16u * (uint32_t)x + 4u * q;
-#pragma unroll
-                            for (int i = 0; i < 4; i++) {
-                                y[x][i] = gate * acc[rg][x][i];
-                                y[x][i] *= as * es[col + i];
-                            }
+                        for (int i = 0; i < 4; i++) {
+                            v[sub][rg][i] = t5_glu(acc[rg][0][i], acc[rg][1][i], g.act, g.f0, g.f1);
+                            m = fmaxf(m, fabsf(v[sub][rg][i]));
                         }
-                        down_store_f32(rg, y[0], y[1]);
+                        m = fmaxf(m, __shfl_xor(m, 16, 64));
+                        m = fmaxf(m, __shfl_xor(m, 32, 64));
+                        /* L.red of the tile before has been read by everyone: its readers have passed this
+                         * tile's block barriers since */
+                        if (q == 0) L.red[cw][16u * (uint32_t)rg + r16] = m;
                     }
-                } else if (wave_on) {
-#pragma unroll
-                    for (int rg = 0; rg < 8; rg++) {
-                        const uint32_t row = 16u * (uint32_t)rg + r16;
-                        if (row >= rows) {
-                            if (GLU && erow0 + row < padded)
-                                *(uint2*)((bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q) = make_uint2(0u, 0u);
-                            continue;
-                        }
-                        if (GLU) {
-                            const uint32_t tok = L.epi_idx[par][row];
-                            bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
-                            if (tok == PLOW_EXPERT_UNUSED) {
-                                *(uint2*)orow = make_uint2(0u, 0u);
-                                continue;
-                            }
-                            const float as = g.a_scale[tok];
-                            float o[4];
-#pragma unroll
-                            for (int i = 0; i < 4; i++)
-                                o[i] = t5_glu(acc[rg][0][i] * (as * es[ch0 + 4u * q + i]),
-                                               acc[rg][1][i] * (as * es[g.N + ch0 + 4u * q + i]), g.act, g.f0, g.f1);
-                            uint2 pk;
-                            pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
-                            pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
-                            *(uint2*)orow = pk;
-                        }
-                    }
-                }
-            } else if (GLU) {
-                float v[8][4];
-#pragma unroll
-                for (int rg = 0; rg < 8; rg++) {
-                    float m = 0.0f;
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        v[rg][i] = t5_glu(acc[rg][0][i], acc[rg][1][i], g.act, g.f0, g.f1);
-                        m = fmaxf(m, fabsf(v[rg][i]));
-                    }
-                    m = fmaxf(m, __shfl_xor(m, 16, 64));
-                    m = fmaxf(m, __shfl_xor(m, 32, 64));
-                    /* L.red of the tile before has been read by everyone: its readers have passed this
-                     * tile's block barriers since */
-                    if (q == 0) L.red[cw][16u * (uint32_t)rg + r16] = m;
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-                for (int rg = 0; rg < 8; rg++) {
-                    const uint32_t row = 16u * (uint32_t)rg + r16;
-                    if (row >= rows || L.epi_idx[par][row] == PLOW_EXPERT_UNUSED) continue;
-                    float amax = 1e-10f;
-#pragma unroll
-                    for (int x = 0; x < 8; x++) amax = fmaxf(amax, L.red[x][row]);
-                    const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
-                    uint8_t* orow = (uint8_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
-                    *(uint32_t*)orow = cvt4_e4m3(v[rg][0] * inv, v[rg][1] * inv, v[rg][2] * inv, v[rg][3] * inv);
-                    if (cw == 0 && q == 0) g.out_scale[(size_t)(r0 + row) * NT + nt] = s;
-                }
-            } else {
-                WG_BARRIER(); /* after the last block (pairs with the loaders') */
-                if (wave_on && !g.part16) {
-#pragma unroll
-                    for (int rg = 0; rg < 8; rg++) {
-                        if (16u * (uint32_t)rg >= rows) break; /* uniform */
-                        const float gate = L.epi_gate[par][16u * (uint32_t)rg + r16]; /* 0 for pad rows */
-                        down_store_f32(rg, acc[rg][0] * gate, acc[rg][1] * gate);
-                    }
-                } else if (wave_on) {
+                for (uint32_t sub = 0; sub < SUBS; sub++) {
+                    const uint32_t cw = cw0 + sub, ch0 = nt * 128u + 16u * cw;
 #pragma unroll
                     for (int rg = 0; rg < 8; rg++) {
                         const uint32_t row = 16u * (uint32_t)rg + r16;
-                        if (row >= rows) continue;
-                        const uint32_t pidx = L.epi_idx[par][row];
-                        if (pidx == PLOW_EXPERT_UNUSED) continue;
-                        const float gate = L.epi_gate[par][row];
+                        if (row >= rows || L.epi_idx[par][row] == PLOW_EXPERT_UNUSED) continue;
+                        float amax = 1e-10f;
 #pragma unroll
-                        for (int x = 0; x < 2; x++) {
-                            const size_t ocol = (size_t)pidx * g.N + ch0 + 16u * (uint32_t)x + 4u * q;
-                            const float y0 = gate * acc[rg][x][0], y1 = gate * acc[rg][x][1];
-                            const float y2 = gate * acc[rg][x][2], y3 = gate * acc[rg][x][3];
-                            if (g.part16) {
+                        for (int x = 0; x < 8; x++) amax = fmaxf(amax, L.red[x][row]);
+                        const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
+                        uint8_t* orow = (uint8_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
+                        *(uint32_t*)orow = cvt4_e4m3(v[sub][rg][0] * inv, v[sub][rg][1] * inv, v[sub][rg][2] * inv, v[sub][rg][3] * inv);
+                        if (cw == 0 && q == 0) g.out_scale[(size_t)(r0 + row) * NT + nt] = s;
+                    }
+                }
+            } else {
+                WG_BARRIER(); /* after the last block (pairs with the loaders') */
+#pragma unroll
+                for (uint32_t sub = 0; sub < SUBS; sub++) {
+                    const uint32_t cw = cw0 + sub;
+                    const uint32_t ch0 = GLU ? nt * 128u + 16u * cw : nt * 256u + 32u * cw; /* first channel */
+                    v4f(&acc)[8][2] = accs[sub];
+                    /* DOWN, f32 partials: a row's 32 channels of this consumer are one 128-byte line. A 16-row
+                     * group goes through LDS once so that it leaves as two stores of 8 whole lines (8 consecutive
+                     * lanes per line) instead of two stores that touch 16 half lines each. The staging area is
+                     * the consumer's own weight slice of the ring stage it has just left: nobody else reads it,
+                     * and the loaders refill it only after the next barrier. Every lane of the wave must call
+                     * this. */
+                    const uint32_t stg = w_base + stl * (256u * 128u) + cw * (32u * 128u);
+                    auto down_store_f32 = [&](int rg, v4f y0, v4f y1) {
+                        const uint32_t buf = stg + (uint32_t)(rg & 1) * 2048u, wsw = r16 & 7u;
+                        const uint32_t wr0 = buf + r16 * 128u + ((q ^ wsw) << 4), wr1 = buf + r16 * 128u + (((4u + q) ^ wsw) << 4);
+                        const uint32_t lrow = lane >> 3, lp = lane & 7u; /* store layout: row lrow (+ 8), piece lp */
+                        const uint32_t rd = buf + lrow * 128u + ((lp ^ (lrow & 7u)) << 4);
+                        const uint32_t rowa = 16u * (uint32_t)rg + lrow, rowb = rowa + 8u;
+                        const uint32_t pa = L.epi_idx[par][rowa], pb = L.epi_idx[par][rowb];
+                        v4f oa, ob;
+                        asm volatile("ds_write_b128 %2, %4\n\tds_write_b128 %3, %5\n\t"
+                                     "ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:1024\n\t"
+                                     "s_waitcnt lgkmcnt(0)"
+                                     : "=&v"(oa), "=&v"(ob)
+                                     : "v"(wr0), "v"(wr1), "v"(y0), "v"(y1), "v"(rd)
+                                     : "memory");
+                        float* const ocol = (float*)g.out + ch0 + 4u * lp;
+                        if (rowa < rows && pa != PLOW_EXPERT_UNUSED)
+                            *(float4*)(ocol + (size_t)pa * g.N) = make_float4(oa[0], oa[1], oa[2], oa[3]);
+                        if (rowb < rows && pb != PLOW_EXPERT_UNUSED)
+                            *(float4*)(ocol + (size_t)pb * g.N) = make_float4(ob[0], ob[1], ob[2], ob[3]);
+                    };
+                    if (PC) {
+                        /* per-channel arm (plow runtime/amd/op_moe.h:6655-6700): g = acc * (as * wsc[n]); GLU
+                         * stores bf16(act(g) * u) and zeroes the expert's pad rows, DOWN stores gate * acc, then
+                         * * (as * wsc[h]) */
+                        const float* es = (const float*)(uintptr_t)g.stab[(size_t)t.e * 2u + (GLU ? 0u : 1u)];
+                        const uint32_t cnt_e = (uint32_t)g.meta[g.E + t.e], erow0 = r0 - (uint32_t)g.meta[t.e];
+                        const uint32_t padded = ((cnt_e + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
+                        if (wave_on && !GLU) {
+#pragma unroll
+                            for (int rg = 0; rg < 8; rg++) {
+                                if (16u * (uint32_t)rg >= rows) break; /* uniform */
+                                const uint32_t row = 16u * (uint32_t)rg + r16;
+                                const float gate = L.epi_gate[par][row]; /* 0 for pad rows */
+                                const float as = row < rows ? g.a_scale[r0 + row] : 0.0f;
+                                v4f y[2];
+#pragma unroll
+                                for (int x = 0; x < 2; x++) {
+                                    const uint32_t col = ch0 + 16u * (uint32_t)x + 4u * q;
+#pragma unroll
+                                    for (int i = 0; i < 4; i++) {
+                                        y[x][i] = gate * acc[rg][x][i];
+                                        y[x][i] *= as * es[col + i];
+                                    }
+                                }
+                                down_store_f32(rg, y[0], y[1]);
+                            }
+                        } else if (wave_on) {
+#pragma unroll
+                            for (int rg = 0; rg < 8; rg++) {
+                                const uint32_t row = 16u * (uint32_t)rg + r16;
+                                bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
+                                if (row >= rows) {
+                                    if (erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u);
+                                    continue;
+                                }
+                                const uint32_t tok = L.epi_idx[par][row];
+                                if (tok == PLOW_EXPERT_UNUSED) {
+                                    *(uint2*)orow = make_uint2(0u, 0u);
+                                    continue;
+                                }
+                                const float as = g.a_scale[tok];
+                                float o[4];
+#pragma unroll
+                                for (int i = 0; i < 4; i++)
+                                    o[i] = t5_glu(acc[rg][0][i] * (as * es[ch0 + 4u * q + i]),
+                                                   acc[rg][1][i] * (as * es[g.N + ch0 + 4u * q + i]), g.act, g.f0, g.f1);
+                                uint2 pk;
+                                pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
+                                pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
+                                *(uint2*)orow = pk;
+                            }
+                        }
+                    } else if (wave_on && !g.part16) {
+#pragma unroll
+                        for (int rg = 0; rg < 8; rg++) {
+                            if (16u * (uint32_t)rg >= rows) break; /* uniform */
+                            const float gate = L.epi_gate[par][16u * (uint32_t)rg + r16]; /* 0 for pad rows */
+                            down_store_f32(rg, acc[rg][0] * gate, acc[rg][1] * gate);
+                        }
+                    } else if (wave_on) {
+#pragma unroll
+                        for (int rg = 0; rg < 8; rg++) {
+                            const uint32_t row = 16u * (uint32_t)rg + r16;
+                            if (row >= rows) continue;
+                            const uint32_t pidx = L.epi_idx[par][row];
+                            if (pidx == PLOW_EXPERT_UNUSED) continue;
+                            const float gate = L.epi_gate[par][row];
+#pragma unroll
+                            for (int x = 0; x < 2; x++) {
+                                const size_t ocol = (size_t)pidx * g.N + ch0 + 16u * (uint32_t)x + 4u * q;
+                                const float y0 = gate * acc[rg][x][0], y1 = gate * acc[rg][x][1];
+                                const float y2 = gate * acc[rg][x][2], y3 = gate * acc[rg][x][3];
                                 uint2 o;
                                 o.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16);
                                 o.y = (uint32_t)f2bf(y2) | ((uint32_t)f2bf(y3) << 16);
                                 *(uint2*)((bf16_t*)g.out + ocol) = o;
-                            } else {
-                                *(float4*)((float*)g.out + ocol) = make_float4(y0, y1, y2, y3);
                             }
                         }
                     }
@@ -689,19 +721,35 @@ __global__ __launch_bounds__(T5_THREADS) void k_group_w8a8_tiled(GroupW8A8 g) {
     }
 #endif
 }
+template <bool GLU, bool PC, uint32_t NCW>
+__global__ __launch_bounds__((NCW + 4u) * 64u) void k_group_w8a8_tiled(GroupW8A8 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    t5_body<GLU, PC, NCW>(g, lds_raw);
+}
+
 #ifdef T5_PROF
 extern "C" int plow_moe_debug_prof(unsigned long long* out) {
     return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(t5_prof), sizeof(t5_prof));
 }
 #endif
 
+/* PLOW_MOE_W8A8_TILE_WAVES=4 runs the 512-thread form (four consumer waves) instead of the 768-thread one */
+static bool tiled_four_consumers() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = getenv("PLOW_MOE_W8A8_TILE_WAVES");
+        v = (e && !strcmp(e, "4")) ? 1 : 0;
+    }
+    return v == 1;
+}
+
 /* Persistent launch: one workgroup per CU; the tile count is computed on the device from meta. */
-template <bool GLU, bool PC>
+template <bool GLU, bool PC, uint32_t NCW>
 static int launch_tiled_t(const GroupW8A8& g, hipStream_t st) {
     static bool attr_set = false;
     static int n_cu = 0;
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU, PC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        if (hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU, PC, NCW>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)sizeof(T5Lds)) != hipSuccess)
             return PLOW_MOE_EDEVICE;
         attr_set = true;
@@ -712,7 +760,7 @@ static int launch_tiled_t(const GroupW8A8& g, hipStream_t st) {
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return PLOW_MOE_EDEVICE;
         n_cu = prop.multiProcessorCount;
     }
-    k_group_w8a8_tiled<GLU, PC><<<(uint32_t)n_cu, T5_THREADS, sizeof(T5Lds), st>>>(g);
+    k_group_w8a8_tiled<GLU, PC, NCW><<<(uint32_t)n_cu, (NCW + 4u) * 64u, sizeof(T5Lds), st>>>(g);
     return 0;
 }
 
@@ -722,7 +770,8 @@ static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
     if (g.N == 0 || g.K == 0 || g.E == 0 || g.E > 1056u || g.N % 128u || g.K % 128u) return PLOW_MOE_EINVAL;
     /* the tile keeps K / 128 block scales in LDS; the load ring runs two blocks ahead */
     if (g.K > 128u * 128u || g.K < 256u) return PLOW_MOE_EINVAL;
-    return g.per_channel ? launch_tiled_t<GLU, true>(g, st) : launch_tiled_t<GLU, false>(g, st);
+    if (tiled_four_consumers()) return g.per_channel ? launch_tiled_t<GLU, true, 4u>(g, st) : launch_tiled_t<GLU, false, 4u>(g, st);
+    return g.per_channel ? launch_tiled_t<GLU, true, 8u>(g, st) : launch_tiled_t<GLU, false, 8u>(g, st);
 }
 
 int launch_group_glu_w8a8_tiled(const GroupW8A8& g, hipStream_t st) { return launch_tiled<true>(g, st); }
