@@ -12,6 +12,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libplow_moe_gfx950.so")
+# the device code object plowrt loads by this name (plow crates/plowrt/src/exec/amd.rs:11718-11760)
+ELF = os.path.join(HERE, "moe_fp8_pf_gfx950.elf")
 
 COMMON = ["--offload-arch=gfx950", "-O3", *os.environ.get("PLOW_MOE_EXTRA_FLAGS", "").split(), "-std=c++17", "-fPIC", "-fno-fast-math",
           # packed-FP32 VALU forms are kept out of every kernel
@@ -38,10 +40,27 @@ def _compile(src, extra):
     return obj, err
 
 
+def _code_object():
+    """One raw (unbundled) gfx950 ELF with plow's kernel names, built the way plow builds its own
+    (hipcc -O3, device only; plow runtime/cmake/hipcc_hsaco.sh)."""
+    cmd = ["hipcc", *[f for f in COMMON if f != "-fPIC"], "--cuda-device-only", "--no-gpu-bundle-output",
+           "-o", ELF, os.path.join(CSRC, "plowrt_obj.hip")]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "not a recognized feature" not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on plowrt_obj.hip:\n{err}")
+    return ELF, err
+
+
 def build(verbose=True):
     os.makedirs(OBJ, exist_ok=True)
-    with cf.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
+    with cf.ThreadPoolExecutor(max_workers=min(8, len(SOURCES) + 1)) as ex:
+        elf = ex.submit(_code_object)
         results = list(ex.map(lambda kv: _compile(*kv), SOURCES.items()))
+        results.append(elf.result())
+    results, (_, elf_err) = results[:-1], results[-1]
+    if verbose and elf_err.strip():
+        print(elf_err, file=sys.stderr)
     objs = [o for o, _ in results]
     for _, err in results:
         if verbose and err.strip():
@@ -52,6 +71,7 @@ def build(verbose=True):
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
         print("built", LIB)
+        print("built", ELF)
     return LIB
 
 

@@ -328,9 +328,10 @@ __device__ __forceinline__ float dm_read4(uint32_t addr) {
  * workgroup barrier */
 #define DM_WAIT_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory")
 
+/* The body works on workgroup index `bid` of a logical grid of E * N / 128 and takes its LDS as a pointer,
+ * so that a kernel with a fixed launch shape (any 1-D grid, static LDS) can walk that grid itself. */
 template <int ENC, bool GLU, int RG>
-__global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
+__device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw, uint32_t bid) {
     DmLds<ENC, RG>& L = *(DmLds<ENC, RG>*)dm_raw;
     typedef DmWSlot<ENC == AENC_MXFP4> Slot;
     constexpr uint32_t KSTEP = DmGeom<ENC>::KSTEP, XROW = KSTEP * 2u; /* activation bytes per row and step */
@@ -354,8 +355,8 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
                          : (ENC == AENC_MXFP4 && busy >= 8192u && tiles % 8u == 0u) ? 8u /* no per-tile tables to hold */
                          : (busy >= 4096u && tiles % 4u == 0u) ? 4u : ((busy >= 2048u && tiles % 2u == 0u) ? 2u : 1u);
     const uint32_t wpe = tiles / TPW; /* workgroups per expert */
-    if (blockIdx.x >= g.E * wpe) return;
-    const uint32_t e = g.E - 1u - blockIdx.x / wpe, ct = (blockIdx.x % wpe) * TPW; /* heavy (folded shared) expert first */
+    if (bid >= g.E * wpe) return;
+    const uint32_t e = g.E - 1u - bid / wpe, ct = (bid % wpe) * TPW; /* heavy (folded shared) expert first */
     const uint32_t cnt = g.meta ? (uint32_t)g.meta[g.E + e] : g.dense_rows;
     if (cnt == 0u) return;
     const uint64_t* wt = g.wtab ? g.wtab + (size_t)e * g.wcols : nullptr;
@@ -660,6 +661,12 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
             }
         }
     }
+}
+
+template <int ENC, bool GLU, int RG>
+__global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
+    a16_dma_body<ENC, GLU, RG>(g, dm_raw, blockIdx.x);
 }
 
 /* PLOW_MOE_A16_KERNEL=regs selects the first form */

@@ -676,6 +676,26 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                                 *(uint2*)orow = pk;
                             }
                         }
+                    } else if (wave_on && g.acc_topk) {
+                        /* fused combine: add into the bf16 output row of the slot's token */
+                        typedef short bf16x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+                        for (int rg = 0; rg < 8; rg++) {
+                            const uint32_t row = 16u * (uint32_t)rg + r16;
+                            if (row >= rows) continue;
+                            const uint32_t pidx = L.epi_idx[par][row];
+                            if (pidx == PLOW_EXPERT_UNUSED) continue;
+                            const float gate = L.epi_gate[par][row];
+                            bf16_t* orow = (bf16_t*)g.out + (size_t)(pidx / g.acc_topk) * g.N + ch0 + 4u * q;
+#pragma unroll
+                            for (int x = 0; x < 2; x++)
+#pragma unroll
+                                for (int h = 0; h < 2; h++) {
+                                    const uint32_t pk = (uint32_t)f2bf(gate * acc[rg][x][2 * h]) | ((uint32_t)f2bf(gate * acc[rg][x][2 * h + 1]) << 16);
+                                    __builtin_amdgcn_global_atomic_fadd_v2bf16((bf16x2_t*)(orow + 16u * (uint32_t)x + 2u * (uint32_t)h),
+                                                                               __builtin_bit_cast(bf16x2_t, pk));
+                                }
+                        }
                     } else if (wave_on && !g.part16) {
 #pragma unroll
                         for (int rg = 0; rg < 8; rg++) {

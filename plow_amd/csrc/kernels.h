@@ -40,6 +40,10 @@ struct GroupW8A8 {
     /* per-channel mode (ops 81 / 82): weights through ewt[E][2] = {gate_up fused [2N][K], down [N][K]},
      * f32 channel scales through est[E][2], one f32 activation scale per row; GLU writes bf16 */
     uint32_t per_channel;
+    /* DOWN, block mode: when non-zero, `out` is the bf16 [T][N] layer output and every live row adds
+     * gate * acc into row (row_partidx / acc_topk) with packed bf16 atomics (order-dependent rounding;
+     * plow's fused-combine variant, runtime/amd/moe_fp8_pf.hip:1219-1230) */
+    uint32_t acc_topk;
 };
 int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);

@@ -1,0 +1,151 @@
+"""The device code object for an unmodified plowrt (plow_amd/moe_fp8_pf_gfx950.elf): its ELF carries the
+kernel symbols, the ABI marker and a launch shape plowrt can use (CPU test); launched the way plowrt
+launches it (any 1-D grid, 512 threads, no dynamic LDS, one by-value argument block) it matches the
+oracle (GPU tests)."""
+import ctypes as C
+import os
+import struct
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ELF = os.path.join(ROOT, "plow_amd", "moe_fp8_pf_gfx950.elf")
+KERNELS = ["plow_moe_fp8_glu_pf_gfx950", "plow_moe_fp8_down_pf_gfx950", "plow_moe_w8a8_glu_pf_gfx950",
+           "plow_moe_w8a8_down_pf_gfx950", "plow_moe_w8a8_down_acc_pf_gfx950"]   # amd.rs:11720-11740
+
+
+def elf_symbols(path):
+    """Names in .symtab / .dynsym of a 64-bit little-endian ELF."""
+    b = open(path, "rb").read()
+    assert b[:4] == b"\x7fELF" and b[4] == 2 and b[5] == 1, "not a raw 64-bit ELF (plowrt loads unbundled objects)"
+    shoff, = struct.unpack_from("<Q", b, 0x28)
+    shentsize, shnum = struct.unpack_from("<HH", b, 0x3A)
+    secs = [struct.unpack_from("<IIQQQQIIQQ", b, shoff + i * shentsize) for i in range(shnum)]
+    names = set()
+    for (_, typ, _, _, off, size, link, _, _, entsize) in secs:
+        if typ not in (2, 11):          # SHT_SYMTAB, SHT_DYNSYM
+            continue
+        stroff = secs[link][4]
+        for k in range(size // entsize):
+            st_name, = struct.unpack_from("<I", b, off + k * entsize)
+            end = b.index(b"\0", stroff + st_name)
+            names.add(b[stroff + st_name:end].decode())
+    return names, b
+
+
+def test_code_object_symbols_and_launch_shape():
+    if not os.path.exists(ELF):
+        pytest.fail(f"{ELF} is not built; run `python -m plow_amd.build`")
+    names, blob = elf_symbols(ELF)
+    assert "plow_moe_fp8_pf_abi_2" in names          # the marker plowrt insists on (amd.rs:11750-11753)
+    for k in KERNELS:
+        assert k in names and k + ".kd" in names, k  # entry point and kernel descriptor
+    # every kernel declares 512 threads and static LDS within the CU's 160 KB (metadata note, msgpack text keys)
+    assert blob.count(b".max_flat_workgroup_size") >= len(KERNELS)
+    import re
+    import subprocess
+    readelf = "/opt/rocm/llvm/bin/llvm-readelf"
+    if os.path.exists(readelf):
+        notes = subprocess.run([readelf, "--notes", ELF], capture_output=True, text=True).stdout
+        for k in KERNELS:
+            m = re.search(r"\.group_segment_fixed_size: (\d+)\n(?:.*\n)*?\s*\.max_flat_workgroup_size: (\d+)\n\s*\.name:\s+" + k + r"\n", notes)
+            assert m, k
+            assert int(m.group(1)) <= 160 * 1024 and int(m.group(2)) == 512, (k, m.groups())
+
+
+# ---- GPU: launch it the way plowrt does --------------------------------------------------------------
+
+class GluArgs(C.Structure):       # plow crates/plowrt/src/exec/amd.rs:1784-1807, 96 bytes
+    _fields_ = [(n, C.c_uint64) for n in ("out", "x", "weight_table", "scale_table", "meta", "row_token", "x_scale", "out_scale")] + \
+               [("inter", C.c_uint32), ("hidden", C.c_uint32), ("experts", C.c_uint32), ("act", C.c_uint32),
+                ("beta", C.c_float), ("linear_beta", C.c_float), ("x_pitch", C.c_uint32), ("reserved", C.c_uint32)]
+
+
+class DownArgs(C.Structure):      # amd.rs:1809-1828, 80 bytes
+    _fields_ = [(n, C.c_uint64) for n in ("part", "fu", "weight_table", "scale_table", "meta", "row_partidx", "row_gate", "fu_scale")] + \
+               [("hidden", C.c_uint32), ("inter", C.c_uint32), ("experts", C.c_uint32), ("reserved", C.c_uint32)]
+
+
+assert C.sizeof(GluArgs) == 96 and C.sizeof(DownArgs) == 80
+
+
+class Module:
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.mod = C.c_void_p()
+        assert self.hip.hipModuleLoad(C.byref(self.mod), ELF.encode()) == 0
+        dptr, size = C.c_void_p(), C.c_size_t()
+        assert self.hip.hipModuleGetGlobal(C.byref(dptr), C.byref(size), self.mod, b"plow_moe_fp8_pf_abi_2") == 0
+        assert size.value == 4
+        self.marker = dptr.value
+
+    def launch(self, name, args, grid):
+        f = C.c_void_p()
+        assert self.hip.hipModuleGetFunction(C.byref(f), self.mod, name.encode()) == 0, name
+        size = C.c_size_t(C.sizeof(args))
+        extra = (C.c_void_p * 5)(1, C.cast(C.byref(args), C.c_void_p), 2, C.cast(C.byref(size), C.c_void_p), 3)
+        rc = self.hip.hipModuleLaunchKernel(f, grid, 1, 1, 512, 1, 1, 0, None, None, extra)
+        assert rc == 0, (name, rc)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("arm,T,grid", [("w8a8", 300, 37), ("w8a8", 24, 256), ("a16", 300, 37), ("a16", 24, 5)])
+def test_code_object_launched_like_plowrt(oracle, arm, T, grid):
+    import torch
+    from gpu_harness import assert_output_close, assert_routing_equal, run_oracle
+    from plow_amd import abi, layer, synth
+    from plow_amd.lib import Moe
+    print(f"[case] plowrt object arm={arm} T={T} grid={grid}", flush=True)
+    cfg = layer.MoeConfig("obj", H=512, E=8, I=256, k=2, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          enc="fp8blk", arm=arm, n_shared=1, shared_mode="fold")
+    plan = layer.plan_layer(cfg)
+    dev = synth.bind(plan, "cuda", seed=T)
+    host = synth.to_host(dev)
+    run_oracle(oracle, plan, host)
+    moe, m = Moe(0), Module()
+    marker = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert m.hip.hipMemcpy(C.c_void_p(marker.data_ptr()), C.c_void_p(m.marker), 4, 3) == 0   # device to device
+    assert int(marker.item()) == 1
+    table = dev.table()
+    glu, down = plan.insts[plan.index("glu")], plan.insts[plan.index("down")]
+    # everything before the GLU through the library, the two expert ops through the object, combine through the library
+    pre = [d for n, d in zip(plan.names, plan.insts) if n not in ("glu", "down", "combine")]
+    moe.exec_many(pre, table)
+    torch.cuda.synchronize()
+    p = lambda name: dev.t[name].data_ptr() if name in dev.t else 0
+    Ea = cfg.E_all
+    if arm == "w8a8":
+        ga = GluArgs(p("fq"), p("xq"), p("wtab"), p("stab"), p("meta"), p("row_token"), p("xs"), p("fs"),
+                     cfg.I, cfg.H, Ea, cfg.act, 0.0, 0.0, glu.i[4], 0)
+        da = DownArgs(p("part"), p("fq"), p("wtab"), p("stab"), p("meta"), p("row_partidx"), p("row_gate"), p("fs"),
+                      cfg.H, cfg.I, Ea, 0)
+        m.launch("plow_moe_w8a8_glu_pf_gfx950", ga, grid)
+        m.launch("plow_moe_w8a8_down_pf_gfx950", da, grid)
+    else:
+        ga = GluArgs(p("fu"), p("x"), p("wtab"), p("stab"), p("meta"), p("row_token"), 0, 0,
+                     cfg.I, cfg.H, Ea, cfg.act, 0.0, 0.0, 0, 0)
+        da = DownArgs(p("part"), p("fu"), p("wtab"), p("stab"), p("meta"), p("row_partidx"), p("row_gate"), 0,
+                      cfg.H, cfg.I, Ea, 0)
+        m.launch("plow_moe_fp8_glu_pf_gfx950", ga, grid)
+        m.launch("plow_moe_fp8_down_pf_gfx950", da, grid)
+    torch.cuda.synchronize()
+    moe.exec_many([plan.insts[plan.index("combine")]], table)
+    torch.cuda.synchronize()
+    assert_routing_equal(plan, dev, host)
+    pd, ph = dev.np("part"), host.np("part")
+    assert np.all(np.isfinite(pd))
+    assert np.abs(pd - ph).max() / np.abs(ph).max() < 2e-2
+    assert_output_close(dev.np("out"), host.np("out"))
+    if arm == "w8a8":
+        # the fused-combine DOWN adds gate * acc into a bf16 [T][H] output seeded with zeros: the same
+        # sums as combine, rounded to bf16 after every addition in an order that depends on timing
+        acc = torch.zeros((cfg.T, cfg.H), dtype=torch.bfloat16, device="cuda")
+        da.part, da.reserved = acc.data_ptr(), cfg.k_all
+        m.launch("plow_moe_w8a8_down_acc_pf_gfx950", da, grid)
+        torch.cuda.synchronize()
+        got, want = acc.float().cpu().numpy(), host.np("out").astype(np.uint32)
+        want = (want << 16).view(np.float32)
+        assert np.abs(got - want).max() <= 3e-2 * np.abs(want).max()
+        assert np.abs(got - want).mean() <= 1e-2 * np.abs(want).mean()
+    moe.close()
