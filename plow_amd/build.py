@@ -14,6 +14,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libplow_moe_gfx950.so")
 # the device code object plowrt loads by this name (plow crates/plowrt/src/exec/amd.rs:11718-11760)
 ELF = os.path.join(HERE, "moe_fp8_pf_gfx950.elf")
+ELF_COMBINE = os.path.join(HERE, "moe_combine_gfx950.elf")   # amd.rs:11666-11716
 
 COMMON = ["--offload-arch=gfx950", "-O3", *os.environ.get("PLOW_MOE_EXTRA_FLAGS", "").split(), "-std=c++17", "-fPIC", "-fno-fast-math",
           # packed-FP32 VALU forms are kept out of every kernel
@@ -40,27 +41,28 @@ def _compile(src, extra):
     return obj, err
 
 
-def _code_object():
+def _code_object(src="plowrt_obj.hip", out=None, extra=()):
     """One raw (unbundled) gfx950 ELF with plow's kernel names, built the way plow builds its own
     (hipcc -O3, device only; plow runtime/cmake/hipcc_hsaco.sh)."""
-    cmd = ["hipcc", *[f for f in COMMON if f != "-fPIC"], "--cuda-device-only", "--no-gpu-bundle-output",
-           "-o", ELF, os.path.join(CSRC, "plowrt_obj.hip")]
+    out = out or ELF
+    cmd = ["hipcc", *[f for f in COMMON if f != "-fPIC"], *extra, "--cuda-device-only", "--no-gpu-bundle-output",
+           "-o", out, os.path.join(CSRC, src)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "not a recognized feature" not in l)
     if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed on plowrt_obj.hip:\n{err}")
-    return ELF, err
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    return out, err
 
 
 def build(verbose=True):
     os.makedirs(OBJ, exist_ok=True)
-    with cf.ThreadPoolExecutor(max_workers=min(8, len(SOURCES) + 1)) as ex:
-        elf = ex.submit(_code_object)
+    with cf.ThreadPoolExecutor(max_workers=8) as ex:
+        elfs = [ex.submit(_code_object), ex.submit(_code_object, "plowrt_combine_obj.hip", ELF_COMBINE, ("-ffp-contract=off",))]
         results = list(ex.map(lambda kv: _compile(*kv), SOURCES.items()))
-        results.append(elf.result())
-    results, (_, elf_err) = results[:-1], results[-1]
-    if verbose and elf_err.strip():
-        print(elf_err, file=sys.stderr)
+        for f in elfs:
+            _, elf_err = f.result()
+            if verbose and elf_err.strip():
+                print(elf_err, file=sys.stderr)
     objs = [o for o, _ in results]
     for _, err in results:
         if verbose and err.strip():
@@ -72,6 +74,7 @@ def build(verbose=True):
     if verbose:
         print("built", LIB)
         print("built", ELF)
+        print("built", ELF_COMBINE)
     return LIB
 
 

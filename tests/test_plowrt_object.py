@@ -1,7 +1,7 @@
-"""The device code object for an unmodified plowrt (plow_amd/moe_fp8_pf_gfx950.elf): its ELF carries the
-kernel symbols, the ABI marker and a launch shape plowrt can use (CPU test); launched the way plowrt
-launches it (any 1-D grid, 512 threads, no dynamic LDS, one by-value argument block) it matches the
-oracle (GPU tests)."""
+"""The device code objects for an unmodified plowrt (plow_amd/moe_fp8_pf_gfx950.elf, the expert GEMMs;
+plow_amd/moe_combine_gfx950.elf, the combine): each ELF carries the kernel symbols, the ABI markers and a
+launch shape plowrt can use (CPU tests); launched the way plowrt launches them (1-D grid, 512 / 256
+threads, no dynamic LDS, one by-value argument block) they match the oracle (GPU tests)."""
 import ctypes as C
 import os
 import struct
@@ -11,6 +11,11 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ELF = os.path.join(ROOT, "plow_amd", "moe_fp8_pf_gfx950.elf")
+ELF_COMBINE = os.path.join(ROOT, "plow_amd", "moe_combine_gfx950.elf")
+COMBINE_KERNEL = "plow_moe_combine_fixed_order_gfx950"                           # amd.rs:11668
+COMBINE_MARKERS = ["plow_moe_combine_fixed_order_abi_1", "plow_moe_combine_fixed_order_slots16_1",
+                   "plow_moe_combine_materialized_f32_1", "plow_moe_combine_wave64_1",
+                   "plow_moe_combine_no_spill_1"]                                  # amd.rs:11669-11675
 KERNELS = ["plow_moe_fp8_glu_pf_gfx950", "plow_moe_fp8_down_pf_gfx950", "plow_moe_w8a8_glu_pf_gfx950",
            "plow_moe_w8a8_down_pf_gfx950", "plow_moe_w8a8_down_acc_pf_gfx950"]   # amd.rs:11720-11740
 
@@ -54,6 +59,32 @@ def test_code_object_symbols_and_launch_shape():
             assert int(m.group(1)) <= 160 * 1024 and int(m.group(2)) == 512, (k, m.groups())
 
 
+def test_combine_object_symbols_and_launch_shape():
+    """plowrt takes the combine object only with its kernel, five markers, a 48-byte argument block (or
+    48 + 256 bytes of hidden arguments), no LDS, no private memory and room for 256 threads
+    (plow crates/plowrt/src/exec/amd.rs:11666-11716)."""
+    if not os.path.exists(ELF_COMBINE):
+        pytest.fail(f"{ELF_COMBINE} is not built; run `python -m plow_amd.build`")
+    names, _ = elf_symbols(ELF_COMBINE)
+    assert COMBINE_KERNEL in names and COMBINE_KERNEL + ".kd" in names
+    for mk in COMBINE_MARKERS:
+        assert mk in names, mk
+    import re
+    import subprocess
+    readelf = "/opt/rocm/llvm/bin/llvm-readelf"
+    if os.path.exists(readelf):
+        notes = subprocess.run([readelf, "--notes", ELF_COMBINE], capture_output=True, text=True).stdout
+        kernels = re.findall(r"\.name:\s+(\S+)\n", notes)
+        assert [k for k in kernels if k.startswith("plow_") or k.startswith("_Z")] == [COMBINE_KERNEL]
+        field = lambda f: int(re.search(r"\." + f + r":\s+(\d+)", notes).group(1))
+        assert field("group_segment_fixed_size") == 0
+        assert field("private_segment_fixed_size") == 0
+        assert field("kernarg_segment_size") in (48, 48 + 256)
+        assert field("max_flat_workgroup_size") >= 256
+        assert field("wavefront_size") == 64
+        assert field("sgpr_spill_count") == 0 and field("vgpr_spill_count") == 0
+
+
 # ---- GPU: launch it the way plowrt does --------------------------------------------------------------
 
 class GluArgs(C.Structure):       # plow crates/plowrt/src/exec/amd.rs:1784-1807, 96 bytes
@@ -67,25 +98,31 @@ class DownArgs(C.Structure):      # amd.rs:1809-1828, 80 bytes
                [("hidden", C.c_uint32), ("inter", C.c_uint32), ("experts", C.c_uint32), ("reserved", C.c_uint32)]
 
 
-assert C.sizeof(GluArgs) == 96 and C.sizeof(DownArgs) == 80
+class CombineArgs(C.Structure):   # amd.rs:1768-1782, 48 bytes
+    _fields_ = [(n, C.c_uint64) for n in ("out", "residual", "shared", "part")] + \
+               [(n, C.c_uint32) for n in ("hidden", "topk", "tokens", "reserved")]
+
+
+assert C.sizeof(GluArgs) == 96 and C.sizeof(DownArgs) == 80 and C.sizeof(CombineArgs) == 48
 
 
 class Module:
-    def __init__(self):
+    def __init__(self, elf=ELF, markers=("plow_moe_fp8_pf_abi_2",)):
         self.hip = C.CDLL("libamdhip64.so")
         self.mod = C.c_void_p()
-        assert self.hip.hipModuleLoad(C.byref(self.mod), ELF.encode()) == 0
-        dptr, size = C.c_void_p(), C.c_size_t()
-        assert self.hip.hipModuleGetGlobal(C.byref(dptr), C.byref(size), self.mod, b"plow_moe_fp8_pf_abi_2") == 0
-        assert size.value == 4
-        self.marker = dptr.value
+        assert self.hip.hipModuleLoad(C.byref(self.mod), elf.encode()) == 0
+        for mk in markers:
+            dptr, size = C.c_void_p(), C.c_size_t()
+            assert self.hip.hipModuleGetGlobal(C.byref(dptr), C.byref(size), self.mod, mk.encode()) == 0, mk
+            assert size.value == 4
+            self.marker = dptr.value
 
-    def launch(self, name, args, grid):
+    def launch(self, name, args, grid, threads=512):
         f = C.c_void_p()
         assert self.hip.hipModuleGetFunction(C.byref(f), self.mod, name.encode()) == 0, name
         size = C.c_size_t(C.sizeof(args))
         extra = (C.c_void_p * 5)(1, C.cast(C.byref(args), C.c_void_p), 2, C.cast(C.byref(size), C.c_void_p), 3)
-        rc = self.hip.hipModuleLaunchKernel(f, grid, 1, 1, 512, 1, 1, 0, None, None, extra)
+        rc = self.hip.hipModuleLaunchKernel(f, grid, 1, 1, threads, 1, 1, 0, None, None, extra)
         assert rc == 0, (name, rc)
 
 
@@ -148,4 +185,47 @@ def test_code_object_launched_like_plowrt(oracle, arm, T, grid):
         want = (want << 16).view(np.float32)
         assert np.abs(got - want).max() <= 3e-2 * np.abs(want).max()
         assert np.abs(got - want).mean() <= 1e-2 * np.abs(want).mean()
+    moe.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,H,k,res,shr", [(1, 512, 16, True, True), (37, 1024, 8, True, False), (700, 512, 9, False, True),
+                                           (1500, 2048, 16, True, True), (64, 520, 3, False, False)])
+def test_combine_object_launched_like_plowrt(T, H, k, res, shr):
+    """min(tokens, 512) workgroups of 256 threads (amd.rs:4018-4036): bit-exact with the library's op 87 and
+    with the f32 sum in slot order on top of residual + shared, rounded to bf16 once
+    (plow runtime/cpu/dev/golden/moe_route.c:130-147)."""
+    import torch
+    print(f"[case] plowrt combine object T={T} H={H} k={k} residual={res} shared={shr}", flush=True)
+    g = torch.Generator(device="cpu").manual_seed(T * 131 + k)
+    part = torch.randn((T * k, H), generator=g, dtype=torch.float32)
+    residual = torch.randn((T, H), generator=g, dtype=torch.float32).bfloat16()
+    shared = torch.randn((T, H), generator=g, dtype=torch.float32).bfloat16()
+    want = torch.zeros((T, H), dtype=torch.float32)
+    if res:
+        want = want + residual.float()
+    if shr:
+        want = want + shared.float()
+    p3 = part.view(T, k, H)
+    for j in range(k):
+        want = want + p3[:, j, :]
+    want = want.bfloat16()
+    d_part, d_res, d_shr = part.cuda(), residual.cuda(), shared.cuda()
+    out = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device="cuda")
+    m = Module(ELF_COMBINE, COMBINE_MARKERS)
+    a = CombineArgs(out.data_ptr(), d_res.data_ptr() if res else 0, d_shr.data_ptr() if shr else 0,
+                    d_part.data_ptr(), H, k, T, 0)
+    m.launch(COMBINE_KERNEL, a, min(T, 512), threads=256)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().view(torch.int16), want.view(torch.int16))
+    # and the library's own op 87 on the same buffers
+    from plow_amd import abi
+    from plow_amd.lib import Moe
+    moe = Moe(0)
+    out2 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device="cuda")
+    d = abi.inst(87, t=[0, 1 if res else None, 2 if shr else None, 3], i=[H, k, T])
+    table = (C.c_void_p * 4)(out2.data_ptr(), d_res.data_ptr(), d_shr.data_ptr(), d_part.data_ptr())
+    moe.exec_many([d], table)
+    torch.cuda.synchronize()
+    assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
     moe.close()
