@@ -101,6 +101,9 @@ enum {
     PLOW_MOE_ARM_A16       = 0, /* bf16 activations (enc 0 bf16 weights, enc 1 W8A16)             */
     PLOW_MOE_ARM_W8A8      = 2, /* enc 1: e4m3 activations with 1x128 scales; DOWN writes f32 part */
     PLOW_MOE_ARM_W8A8_P16  = 3, /* DOWN only: as 2 with a bf16 part                                */
+    PLOW_MOE_ARM_W8A8_XQ   = 6, /* GLU only, enc 1: t1 holds the bf16 rows, quantized 1x128 where they
+                                   are loaded; equals op 184 + arm 2 bit for bit, writes arm 2's fq / fs
+                                   (runtime/amd/moe_pf_w8a8.h:118-121); t6 and i4 unused              */
     PLOW_MOE_ARM_W4A16     = 8
 };
 

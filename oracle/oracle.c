@@ -432,9 +432,14 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
     const uint32_t* row_token = TEN(in, T, 5);
     const uint32_t I = in->i[0], H = in->i[1], E = in->i[2], enc = in->i[3], act = in->i[5];
     const uint32_t arm = in->i[7], pitch = in->i[4];
-    const int w8a8 = enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8;
+    /* arm 6: t1 holds the bf16 rows; each 1x128 group is quantized with op 184's arithmetic and the
+     * rest is arm 2 (plow runtime/amd/moe_pf_w8a8.h:118-121, :255-283) */
+    const int xq_inline = enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ;
+    const int w8a8 = (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8) || xq_inline;
     const float* xs = TEN(in, T, 6);
     const uint32_t G = (I + 127u) / 128u, KB = (H + 127u) / 128u;
+    float* rowxs = NULL; /* arm 6: [cached row][KB] scales of the rows quantized here */
+    uint32_t rowxs_cap = 0;
     float* wg = malloc((size_t)H * 4u);
     float* wu = malloc((size_t)H * 4u);
     float* v = NULL;
@@ -453,11 +458,23 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
         const void* Su = stab ? (const void*)(uintptr_t)stab[(size_t)e * 3u + 1u] : NULL;
         if (rc.expert != e) {
             cache_fit(&rc, cnt);
+            if (xq_inline && rowxs_cap < cnt) { free(rowxs); rowxs = malloc((size_t)cnt * KB * 4u); rowxs_cap = cnt; }
             for (uint32_t q = 0; q < cnt; q++) {
                 const uint32_t tok = row_token[r0 + q];
                 rc.live[q] = tok != PLOW_EXPERT_UNUSED;
                 if (!rc.live[q]) continue;
-                if (w8a8) decode_e4m3_row(rc.a + (size_t)q * H, (const uint8_t*)TEN(in, T, 1) + (size_t)tok * H, H);
+                if (xq_inline) {
+                    const orc_bf16* src = (const orc_bf16*)TEN(in, T, 1) + (size_t)tok * H;
+                    for (uint32_t kb = 0; kb < KB; kb++) {
+                        float amax = 1e-10f; /* the amax is floored, not the scale */
+                        for (uint32_t j = 0; j < 128u; j++) amax = fmaxf(amax, fabsf(orc_bf2f(src[kb * 128u + j])));
+                        const float sc = amax * (1.0f / 448.0f), inv = 1.0f / sc;
+                        rowxs[(size_t)q * KB + kb] = sc;
+                        for (uint32_t j = 0; j < 128u; j++)
+                            rc.a[(size_t)q * H + kb * 128u + j] =
+                                e4m3_lut[orc_f32_to_e4m3(orc_bf2f(src[kb * 128u + j]) * inv)];
+                    }
+                } else if (w8a8) decode_e4m3_row(rc.a + (size_t)q * H, (const uint8_t*)TEN(in, T, 1) + (size_t)tok * H, H);
                 else decode_bf16_row(rc.a + (size_t)q * H, (const orc_bf16*)TEN(in, T, 1) + (size_t)tok * H, H);
             }
             rc.expert = e;
@@ -487,8 +504,10 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
                     if (!rc.live[q]) continue;
                     const uint32_t tok = row_token[r0 + q];
                     const float* a = rc.a + (size_t)q * H;
-                    const float g = dot_fp8blk_a8(wg, (const float*)Sg + (size_t)g0 * KB, a, xs + tok, pitch, H);
-                    const float u = dot_fp8blk_a8(wu, (const float*)Su + (size_t)g0 * KB, a, xs + tok, pitch, H);
+                    const float* as = xq_inline ? rowxs + (size_t)q * KB : xs + tok;
+                    const uint32_t as_step = xq_inline ? 1u : pitch;
+                    const float g = dot_fp8blk_a8(wg, (const float*)Sg + (size_t)g0 * KB, a, as, as_step, H);
+                    const float u = dot_fp8blk_a8(wu, (const float*)Su + (size_t)g0 * KB, a, as, as_step, H);
                     v[(size_t)q * 128u + (n - n0)] = glu_pair(g, u, act, in->fj[0].f, in->fj[1].f);
                 }
             }
@@ -503,7 +522,7 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
             }
         }
     }
-    free(wg); free(wu); free(v);
+    free(wg); free(wu); free(v); free(rowxs);
     cache_free(&rc);
 }
 

@@ -38,7 +38,7 @@ OP_GEMM_F32 = 180
 OP_QUANT_FP8_BLOCK128 = 184
 
 ENC_BF16, ENC_FP8BLK, ENC_MXFP4 = 0, 1, 2
-ARM_A16, ARM_W8A8, ARM_W8A8_P16, ARM_W4A16 = 0, 2, 3, 8
+ARM_A16, ARM_W8A8, ARM_W8A8_P16, ARM_W8A8_XQ, ARM_W4A16 = 0, 2, 3, 6, 8
 ACT_GELU_TANH, ACT_SILU = 0, 1
 ROUTE_SIGMOID, ROUTE_NORM_TOPK, ROUTE_BIAS, ROUTE_F32_LOGIT = 1, 2, 4, 8
 

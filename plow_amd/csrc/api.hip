@@ -216,6 +216,20 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             if (H < 256u || I < 256u) c->tiled = 0; /* the tiled form needs two 128-k blocks in both GEMMs */
             return c->tiled ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
         }
+        if (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ) {
+            NEED(c, ten(in, T, 3) && ten(in, T, 7), "op 85 W8A8 (bf16 rows): t3 stab, t7 fs must be bound");
+            NEED(c, I % 128u == 0u && H % 128u == 0u, "op 85 W8A8: I %u and H %u must be multiples of 128", I, H);
+            NEED(c, i[5] <= 2u || i[5] == PLOW_MOE_ACT_SWIGLU_CLAMP, "op 85: activation %u is not served", i[5]);
+            if (!launch) return 0;
+            GroupW8A8 g = {};
+            g.out = ten(in, T, 0); g.out_scale = (float*)ten(in, T, 7);
+            g.a = ten(in, T, 1); g.a_bf16 = 1;
+            g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 3);
+            g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
+            g.N = I; g.K = H; g.E = E; g.act = i[5];
+            g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
+            return launch_group_glu_w8a8(g, st); /* the streaming form serves this arm at every row count */
+        }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
                          (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
                          (enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_W4A16);

@@ -44,24 +44,30 @@ __device__ __forceinline__ v4i ldg16_stream(const uint8_t* p) {
 }
 
 /* WIDE (DOWN, block mode only): a wave owns 32 channels as two 16-channel streams, a workgroup 256
- * channels; the short K loop of the down projection then amortises its prologue over twice the bytes. */
-template <int RT, bool GLU, int D, bool PC, bool WIDE>
+ * channels; the short K loop of the down projection then amortises its prologue over twice the bytes.
+ * NW: waves in the workgroup. The work item is always that of eight waves (128 channels, 256 WIDE);
+ * with NW = 4 a wave runs the shares of logical waves wv and wv + 4 one after the other and keeps the
+ * first share's GLU values until the amax over all 128 channels is known.
+ * AQ (GLU, block mode): g.a holds the bf16 rows themselves and every 1x128 group is quantized where it
+ * is loaded: amax floored at 1e-10, scale amax / 448, e4m3 of x * (1 / scale), the arithmetic of the
+ * separate quantizer op, so the result equals quantizer + plain GLU bit for bit
+ * (plow runtime/amd/moe_pf_w8a8.h:118-121, :255-283). */
+template <int RT, bool GLU, int D, bool PC, bool WIDE, uint32_t NW = SK_WAVES, bool AQ = false>
 __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t ct, uint32_t r0,
                                         uint32_t rb, uint32_t cnt, float* s_red) {
+    static_assert(NW == 8u || NW == 4u, "eight waves, or four running two shares each");
+    static_assert(!AQ || (GLU && !PC), "in-place activation quantization is a block-mode GLU form");
+    constexpr uint32_t SUBS = SK_WAVES / NW;
     const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6, c = lane & 15u, q = lane >> 4;
     const uint32_t K = g.K, KB = K / 128u, N = g.N;
     constexpr bool TWO = GLU || WIDE; /* two weight streams per wave */
-    const uint32_t ch = WIDE ? ct * 256u + wv * 32u + c : ct * SK_BN + wv * 16u + c; /* this lane's weight row */
     /* block mode: {gate, up, down} tables, scale rows [N/128][KB]; per-channel mode: {gate_up fused,
      * down} tables (up rows follow the N gate rows), one f32 scale per weight row */
     const uint32_t wcols = PC ? 2u : 3u, sel0 = PC ? (GLU ? 0u : 1u) : (GLU ? 0u : 2u), sel1 = PC ? 0u : 1u;
-    const uint8_t* w0 = (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * wcols + sel0] + (size_t)ch * K + 16u * q;
-    const uint8_t* w1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * wcols + sel1] +
-                                  (size_t)(ch + (PC ? N : 0u)) * K + 16u * q
-                            : (WIDE ? w0 + (size_t)16u * K : nullptr);
-    const float* s0 = (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel0] +
-                      (PC ? 0u : (WIDE ? (size_t)(ct * 2u + (wv >> 2)) * KB : (size_t)ct * KB));
-    const float* s1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel1] + (PC ? (size_t)N : (size_t)ct * KB) : nullptr;
+    const uint8_t* const wbase0 = (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * wcols + sel0];
+    const uint8_t* const wbase1 = GLU ? (const uint8_t*)(uintptr_t)g.wtab[(size_t)e * wcols + sel1] : nullptr;
+    const float* const sbase0 = (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel0];
+    const float* const sbase1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)e * wcols + sel1] : nullptr;
 
     /* B operand rows of this lane, one per row tile */
     const uint8_t* ap[RT];
@@ -78,8 +84,8 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             const uint32_t tok = valid[rt] ? g.row_token[rowidx[rt]] : PLOW_EXPERT_UNUSED;
             valid[rt] = tok != PLOW_EXPERT_UNUSED;
             const uint32_t t = valid[rt] ? tok : 0u;
-            ap[rt] = (const uint8_t*)g.a + (size_t)t * K + 16u * q;
-            asp[rt] = g.a_scale + t;
+            ap[rt] = (const uint8_t*)g.a + ((size_t)t * K + 16u * q) * (AQ ? 2u : 1u);
+            asp[rt] = AQ ? nullptr : g.a_scale + t;
         } else if (PC) {
             const uint32_t pi = valid[rt] ? g.row_partidx[rowidx[rt]] : PLOW_EXPERT_UNUSED;
             valid[rt] = pi != PLOW_EXPERT_UNUSED;
@@ -96,7 +102,18 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
     }
     as_stride = GLU ? g.pitch : 1u;
 
-    v4i wa[D][2], wb[D][2], xa[D][RT][2];
+    float vkeep[SUBS][RT][4]; /* block-mode GLU: a share's values until the group's amax is known */
+#pragma unroll
+    for (uint32_t sub = 0; sub < SUBS; sub++) {
+    const uint32_t lw = wv + NW * sub; /* the logical wave (of eight) whose share this is */
+    const uint32_t ch = WIDE ? ct * 256u + lw * 32u + c : ct * SK_BN + lw * 16u + c; /* this lane's weight row */
+    const uint8_t* w0 = wbase0 + (size_t)ch * K + 16u * q;
+    const uint8_t* w1 = GLU ? wbase1 + (size_t)(ch + (PC ? N : 0u)) * K + 16u * q
+                            : (WIDE ? w0 + (size_t)16u * K : nullptr);
+    const float* s0 = sbase0 + (PC ? 0u : (WIDE ? (size_t)(ct * 2u + (lw >> 2)) * KB : (size_t)ct * KB));
+    const float* s1 = GLU ? sbase1 + (PC ? (size_t)N : (size_t)ct * KB) : nullptr;
+
+    v4i wa[D][2], wb[D][2], xa[D][RT][AQ ? 4 : 2];
     float xs[D][RT], sa[D], sb[D];
     auto issue = [&](int d, uint32_t kb) {
         const uint32_t ko = kb * 128u;
@@ -108,13 +125,20 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
         }
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
-            xa[d][rt][0] = (v4i){0, 0, 0, 0};
-            xa[d][rt][1] = (v4i){0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < (AQ ? 4 : 2); j++) xa[d][rt][j] = (v4i){0, 0, 0, 0};
             xs[d][rt] = 0.0f;
             if (valid[rt]) {
-                xa[d][rt][0] = ldg16(ap[rt] + ko);
-                xa[d][rt][1] = ldg16(ap[rt] + ko + 64u);
-                if (!PC) xs[d][rt] = asp[rt][(size_t)kb * as_stride];
+                if (AQ) { /* bf16 elements ko + 16q .. + 15 and ko + 64 + 16q .. + 15 */
+                    xa[d][rt][0] = ldg16(ap[rt] + 2u * ko);
+                    xa[d][rt][1] = ldg16(ap[rt] + 2u * ko + 16u);
+                    xa[d][rt][2] = ldg16(ap[rt] + 2u * ko + 128u);
+                    xa[d][rt][3] = ldg16(ap[rt] + 2u * ko + 144u);
+                } else {
+                    xa[d][rt][0] = ldg16(ap[rt] + ko);
+                    xa[d][rt][1] = ldg16(ap[rt] + ko + 64u);
+                    if (!PC) xs[d][rt] = asp[rt][(size_t)kb * as_stride];
+                }
             }
         }
         if (!PC) {
@@ -142,19 +166,45 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
                 if (TWO) A1 = __builtin_shufflevector(wb[d][0], wb[d][1], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) {
-                    const v8i B = __builtin_shufflevector(xa[d][rt][0], xa[d][rt][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    v8i B;
+                    float xsc;
+                    if (AQ) {
+                        /* the lane's 32 bf16 of the row's 128-group; the group's other lanes are q ^ 1, 2, 3 */
+                        float f[32];
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                const uint32_t w = (uint32_t)xa[d][rt][j][i];
+                                f[8 * j + 2 * i] = __uint_as_float(w << 16);
+                                f[8 * j + 2 * i + 1] = __uint_as_float(w & 0xFFFF0000u);
+                            }
+                        float amax = 1e-10f; /* the amax is floored, not the scale */
+#pragma unroll
+                        for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(f[i]));
+                        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+                        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                        xsc = amax * (1.0f / 448.0f);
+                        const float inv = 1.0f / xsc;
+#pragma unroll
+                        for (int i = 0; i < 8; i++)
+                            B[i] = (int)cvt4_e4m3(f[4 * i] * inv, f[4 * i + 1] * inv, f[4 * i + 2] * inv, f[4 * i + 3] * inv);
+                    } else {
+                        B = __builtin_shufflevector(xa[d][rt][0], xa[d][rt][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                        xsc = xs[d][rt];
+                    }
                     if (PC) { /* scales are outside the K reduction: accumulate straight through */
                         acc0[rt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A0, B, acc0[rt], 0, 0, 0, 0, 0, 0);
                         if (GLU) acc1[rt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, acc1[rt], 0, 0, 0, 0, 0, 0);
                     } else {
                         const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
                         const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A0, B, z, 0, 0, 0, 0, 0, 0);
-                        const float sc0 = xs[d][rt] * sa[d];
+                        const float sc0 = xsc * sa[d];
 #pragma unroll
                         for (int i = 0; i < 4; i++) acc0[rt][i] = fmaf(t0[i], sc0, acc0[rt][i]);
                         if (TWO) {
                             const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, z, 0, 0, 0, 0, 0, 0);
-                            const float sc1 = xs[d][rt] * (WIDE ? sa[d] : sb[d]);
+                            const float sc1 = xsc * (WIDE ? sa[d] : sb[d]);
 #pragma unroll
                             for (int i = 0; i < 4; i++) acc1[rt][i] = fmaf(t1[i], sc1, acc1[rt][i]);
                         }
@@ -165,8 +215,8 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
         }
     }
 
-    /* ---- epilogue: lane holds channels ct*128 + wv*16 + 4q + i (i = 0..3) of row c ---- */
-    const uint32_t col = WIDE ? ct * 256u + wv * 32u + 4u * q : ct * SK_BN + wv * 16u + 4u * q;
+    /* ---- epilogue: lane holds channels ct*128 + lw*16 + 4q + i (i = 0..3) of row c ---- */
+    const uint32_t col = WIDE ? ct * 256u + lw * 32u + 4u * q : ct * SK_BN + lw * 16u + 4u * q;
     if (PC) {
         /* per-channel arm (plow runtime/amd/op_moe.h:6655-6700): g = acc * (as * wsc[n]); GLU stores
          * bf16(act(g) * u) and zeroes pad rows, DOWN stores gate * acc, then * (as * wsc[h]) */
@@ -201,37 +251,19 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
                 *(float4*)((float*)g.out + (size_t)pidx * N + col) = make_float4(o[0], o[1], o[2], o[3]);
             }
         }
-        return;
-    }
-    if (GLU) {
-        float v[RT][4];
+    } else if (GLU) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
             float m = 0.0f;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                v[rt][i] = moe_glu(acc0[rt][i], acc1[rt][i], g.act, g.f0, g.f1);
-                m = fmaxf(m, fabsf(v[rt][i]));
+                vkeep[sub][rt][i] = moe_glu(acc0[rt][i], acc1[rt][i], g.act, g.f0, g.f1);
+                m = fmaxf(m, fabsf(vkeep[sub][rt][i]));
             }
             m = fmaxf(m, __shfl_xor(m, 16, 64));
             m = fmaxf(m, __shfl_xor(m, 32, 64));
-            if (q == 0) s_red[wv * 64u + (uint32_t)rt * 16u + c] = m;
+            if (q == 0) s_red[lw * 64u + (uint32_t)rt * 16u + c] = m;
         }
-        __syncthreads();
-#pragma unroll
-        for (int rt = 0; rt < RT; rt++) {
-            float amax = 1e-10f;
-#pragma unroll
-            for (uint32_t w = 0; w < SK_WAVES; w++) amax = fmaxf(amax, s_red[w * 64u + (uint32_t)rt * 16u + c]);
-            const float s = amax * (1.0f / 448.0f);
-            const float inv = 1.0f / s;
-            if (valid[rt]) {
-                const uint32_t pk = cvt4_e4m3(v[rt][0] * inv, v[rt][1] * inv, v[rt][2] * inv, v[rt][3] * inv);
-                *(uint32_t*)((uint8_t*)g.out + (size_t)rowidx[rt] * N + col) = pk;
-                if (wv == 0 && q == 0) g.out_scale[(size_t)rowidx[rt] * (N / 128u) + ct] = s;
-            }
-        }
-        __syncthreads(); /* s_red is reused by the next row block */
     } else {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
@@ -260,9 +292,32 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             }
         }
     }
+    } /* sub */
+
+    if (GLU && !PC) {
+        __syncthreads();
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            float amax = 1e-10f;
+#pragma unroll
+            for (uint32_t w = 0; w < SK_WAVES; w++) amax = fmaxf(amax, s_red[w * 64u + (uint32_t)rt * 16u + c]);
+            const float s = amax * (1.0f / 448.0f);
+            const float inv = 1.0f / s;
+            if (valid[rt]) {
+#pragma unroll
+                for (uint32_t sub = 0; sub < SUBS; sub++) {
+                    const uint32_t col = ct * SK_BN + (wv + NW * sub) * 16u + 4u * q;
+                    const float* v = vkeep[sub][rt];
+                    *(uint32_t*)((uint8_t*)g.out + (size_t)rowidx[rt] * N + col) = cvt4_e4m3(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+                }
+                if (wv == 0 && q == 0) g.out_scale[(size_t)rowidx[rt] * (N / 128u) + ct] = s;
+            }
+        }
+        __syncthreads(); /* s_red is reused by the next row block */
+    }
 }
 
-template <bool GLU, int D, bool PC, bool WIDE = false>
+template <bool GLU, int D, bool PC, bool WIDE = false, bool AQ = false>
 __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     __shared__ float s_red[SK_WAVES * 64u];
     const uint32_t tiles = g.N / (WIDE ? 256u : SK_BN);
@@ -275,7 +330,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     const uint32_t r0 = (uint32_t)g.meta[e];
     /* 16 rows a pass; an expert with more rows streams its weights once per pass (the tiled
      * kernel, not this one, is the tool for many rows per expert) */
-    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D, PC, WIDE>(g, e, ct, r0, rb, cnt, s_red);
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D, PC, WIDE, SK_WAVES, AQ>(g, e, ct, r0, rb, cnt, s_red);
     if (PC && GLU) {
         /* the per-channel GLU zeroes the pad rows of its 64-row tile (the partial 16-row pass above
          * did its own); the row quantizer that follows reads every aligned row */
@@ -487,6 +542,10 @@ int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<true, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
+    if (g.a_bf16) { /* bf16 rows, quantized where they are loaded */
+        k_group_w8a8_stream<true, 3, false, false, true><<<grid, SK_THREADS, 0, st>>>(g);
+        return 0;
+    }
     if (glu_dma_form()) {
         static bool attr_set = false;
         if (!attr_set) {

@@ -44,6 +44,9 @@ struct GroupW8A8 {
      * gate * acc into row (row_partidx / acc_topk) with packed bf16 atomics (order-dependent rounding;
      * plow's fused-combine variant, runtime/amd/moe_fp8_pf.hip:1219-1230) */
     uint32_t acc_topk;
+    /* GLU, block mode: when non-zero, `a` holds the bf16 rows [T][K] themselves and the kernel quantizes
+     * every 1x128 group as it loads it (a_scale and pitch unused; plow's arm i7 = 6) */
+    uint32_t a_bf16;
 };
 int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);

@@ -32,7 +32,8 @@ class MoeConfig:
     topk_group: int = 1
     route_scale: float = 1.0
     enc: str = "fp8blk"             # "bf16" | "fp8blk" | "mxfp4" | "fp8pc" (per-channel)
-    arm: str = "w8a8"               # "a16" (bf16 activations) | "w8a8"
+    arm: str = "w8a8"               # "a16" (bf16 activations) | "w8a8" | "w8a8q" (block-fp8 only: the GLU
+                                    # quantizes the bf16 rows itself, plow's arm 6; no quantizer op)
     n_shared: int = 0
     shared_mode: Optional[str] = None  # "fold" (slot {E, 1.0}) | "dense" (ops 20 + 8) | None
     act: int = abi.ACT_SILU
@@ -138,7 +139,7 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
     row_token = p._t("row_token", "u32", (R,), "scratch")
     row_partidx = p._t("row_partidx", "u32", (R,), "scratch")
     row_gate = p._t("row_gate", "f32", (R,), "scratch")
-    p16 = cfg.part_bf16 and cfg.enc == "fp8blk" and cfg.arm == "w8a8"
+    p16 = cfg.part_bf16 and cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q")
     part = p._t("part", "bf16" if p16 else "f32", (T * ka, H), "scratch")
     out = p._t("out", "bf16", (T, H), "out")
     residual = p._t("residual", "bf16", (T, H), "in") if cfg.residual else None
@@ -179,15 +180,20 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
         enc = {"bf16": abi.ENC_BF16, "fp8blk": abi.ENC_FP8BLK, "mxfp4": abi.ENC_MXFP4}[cfg.enc]
         wtab = p._t("wtab", "u64", (Ea, 3), "table")
         stab = p._t("stab", "u64", (Ea, 3), "table") if enc != abi.ENC_BF16 else None
-        if enc == abi.ENC_FP8BLK and cfg.arm == "w8a8":
-            xq = p._t("xq", "u8", (T, H), "scratch")
-            xs = p._t("xs", "f32", (H // 128, T), "scratch")
+        if enc == abi.ENC_FP8BLK and cfg.arm in ("w8a8", "w8a8q"):
             fq = p._t("fq", "u8", (R, I), "scratch")
             fs = p._t("fs", "f32", (R, I // 128), "scratch")
-            p._emit("quant_x", abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[xq, x, xs], i=[T, H, T]))
-            p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
-                                    t=[fq, xq, wtab, stab, meta, row_token, xs, fs],
-                                    i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8], f=cfg.act_f))
+            if cfg.arm == "w8a8q":
+                p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
+                                        t=[fq, x, wtab, stab, meta, row_token, None, fs],
+                                        i=[I, H, Ea, enc, 0, cfg.act, 0, abi.ARM_W8A8_XQ], f=cfg.act_f))
+            else:
+                xq = p._t("xq", "u8", (T, H), "scratch")
+                xs = p._t("xs", "f32", (H // 128, T), "scratch")
+                p._emit("quant_x", abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[xq, x, xs], i=[T, H, T]))
+                p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
+                                        t=[fq, xq, wtab, stab, meta, row_token, xs, fs],
+                                        i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8], f=cfg.act_f))
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
                                      t=[part, fq, wtab, stab, meta, fs, row_partidx, row_gate],
                                      i=[H, I, Ea, enc, 0, 0, 0, abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8]))

@@ -23,8 +23,9 @@ def check_layer(plan, dev, host):
     cfg = plan.cfg
     rows = assert_routing_equal(plan, dev, host)
     assert np.array_equal(dev.np("logit").view(np.uint32), host.np("logit").view(np.uint32))
-    assert np.array_equal(dev.np("xq"), host.np("xq"))
-    assert np.array_equal(dev.np("xs").view(np.uint32), host.np("xs").view(np.uint32))
+    if "xq" in dev.t:
+        assert np.array_equal(dev.np("xq"), host.np("xq"))
+        assert np.array_equal(dev.np("xs").view(np.uint32), host.np("xs").view(np.uint32))
     # intermediate: dequantized fq * fs of live rows agrees to fp8 precision
     live = host.np("row_partidx")[:rows] != abi.EXPERT_UNUSED
     fqd, fqh = dev.np("fq")[:rows][live], host.np("fq")[:rows][live]
@@ -47,6 +48,20 @@ def test_small_dsv3_like_layer(moe, oracle, T):
                           bias=True, n_group=4, topk_group=2, route_scale=2.5, enc="fp8blk",
                           arm="w8a8", n_shared=1, shared_mode="fold")
     check_layer(*both(moe, oracle, cfg, seed=T))
+
+
+@pytest.mark.parametrize("T", [1, 19, 100, 333])
+def test_glu_quantizes_bf16_rows_itself(moe, oracle, T):
+    """Op 85 arm 6: bf16 rows in, quantized 1x128 where the kernel loads them, no quantizer op and no
+    xq / xs tensors (plow runtime/amd/moe_pf_w8a8.h:118-121). The fq bytes and fs scales must also be the
+    very ones the quantizer + arm 2 chain of the same library produces on the same inputs when that chain
+    runs the same streaming kernel (few rows per expert)."""
+    print(f"[case] w8a8 arm 6 T={T}", flush=True)
+    kw = dict(H=512, E=32, I=256, k=4, T=T, scoring="sigmoid", norm_topk=True, bias=True, n_group=4,
+              topk_group=2, route_scale=2.5, enc="fp8blk", n_shared=1, shared_mode="fold")
+    plan, dev, host = both(moe, oracle, layer.MoeConfig("mini-xq", arm="w8a8q", **kw), seed=T)
+    assert "xq" not in dev.t and "quant_x" not in plan.names
+    check_layer(plan, dev, host)
 
 
 @pytest.mark.parametrize("T,act,f", [(24, 2, (2.0, 1.5)), (24, 4, (0.0, 0.75)), (600, 2, (3.0, 0.0)), (600, 4, (0.0, 0.75))])

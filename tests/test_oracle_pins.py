@@ -370,6 +370,34 @@ def test_fp8blk_layer_against_f64_over_the_same_bytes(oracle, arm):
         assert np.allclose(part[s], y, rtol=2e-5, atol=2e-5 * np.abs(y).max())
 
 
+def test_fp8blk_inline_quant_arm_equals_quantizer_plus_plain_arm(oracle):
+    """Op 85 arm 6 takes the bf16 rows and quantizes each 1x128 group itself: by definition the quantizer
+    op followed by arm 2, bit for bit (plow runtime/amd/moe_pf_w8a8.h:118-121)."""
+    r = cases.rng_of(23)
+    E, T, H, I, k = 5, 21, 384, 256, 2
+    W, S, wtab, stab = build_fp8(oracle, r, E, T, H, I, False, False)
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    for t in range(T):
+        tab["eid"][t * k:(t + 1) * k] = r.choice(E, k, replace=False)
+    tab["gate"] = (r.random(T * k) + 0.1).astype(np.float32)
+    al = cases.align_arrays(tab, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    R = al[2].shape[0]
+    x = cases.randn_bf16(r, (T, H), 1.0)
+    x[3, 128:256] = 0                     # an all-zero group: the floored amax
+    xq, xs = np.zeros((T, H), np.uint8), np.zeros((H // 128, T), np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[T, H, T]), [xq, x, xs])
+    fq2, fs2 = np.full((R, I), 0x55, np.uint8), np.full((R, I // 128), 7.0, np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[I, H, E, 1, T, 1, 0, abi.ARM_W8A8]),
+        [fq2, xq, wtab, stab, al[0], al[2], xs, fs2], 2)
+    fq6, fs6 = np.full((R, I), 0x55, np.uint8), np.full((R, I // 128), 7.0, np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5, None, 7], i=[I, H, E, 1, 0, 1, 0, abi.ARM_W8A8_XQ]),
+        [fq6, x, wtab, stab, al[0], al[2], None, fs6], 3)
+    assert np.array_equal(fq6, fq2)
+    assert np.array_equal(fs6.view(np.uint32), fs2.view(np.uint32))
+    assert (fq6 != 0x55).any()
+
+
 def test_fp8blk_constant_block_scale_factors_out(oracle):
     """A constant scale grid c equals c times the unit-scale result (c a power of two: exactly)."""
     r = cases.rng_of(12)
