@@ -15,6 +15,7 @@ LIB = os.path.join(HERE, "libplow_moe_gfx950.so")
 # the device code object plowrt loads by this name (plow crates/plowrt/src/exec/amd.rs:11718-11760)
 ELF = os.path.join(HERE, "moe_fp8_pf_gfx950.elf")
 ELF_COMBINE = os.path.join(HERE, "moe_combine_gfx950.elf")   # amd.rs:11666-11716
+ELF_DEC = os.path.join(HERE, "moe_w8a8_dec_gfx950.elf")      # amd.rs:10799-10852
 
 COMMON = ["--offload-arch=gfx950", "-O3", *os.environ.get("PLOW_MOE_EXTRA_FLAGS", "").split(), "-std=c++17", "-fPIC", "-fno-fast-math",
           # packed-FP32 VALU forms are kept out of every kernel
@@ -57,7 +58,8 @@ def _code_object(src="plowrt_obj.hip", out=None, extra=()):
 def build(verbose=True):
     os.makedirs(OBJ, exist_ok=True)
     with cf.ThreadPoolExecutor(max_workers=8) as ex:
-        elfs = [ex.submit(_code_object), ex.submit(_code_object, "plowrt_combine_obj.hip", ELF_COMBINE, ("-ffp-contract=off",))]
+        elfs = [ex.submit(_code_object), ex.submit(_code_object, "plowrt_combine_obj.hip", ELF_COMBINE, ("-ffp-contract=off",)),
+                ex.submit(_code_object, "plowrt_dec_obj.hip", ELF_DEC)]
         results = list(ex.map(lambda kv: _compile(*kv), SOURCES.items()))
         for f in elfs:
             _, elf_err = f.result()
@@ -75,6 +77,7 @@ def build(verbose=True):
         print("built", LIB)
         print("built", ELF)
         print("built", ELF_COMBINE)
+        print("built", ELF_DEC)
     return LIB
 
 

@@ -228,7 +228,10 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.act = i[5];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
-            return launch_group_glu_w8a8(g, st); /* the streaming form serves this arm at every row count */
+            /* the streaming form serves this arm at every row count; the DOWN that follows reads plain
+             * fq / fs rows and takes the tiled form when the last align saw 16 or more rows per expert */
+            c->tiled = (c->forced >= 0 ? c->forced : (c->rows_hint >= 16u ? 1 : 0)) && H >= 256u && I >= 256u;
+            return launch_group_glu_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
                          (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||

@@ -16,6 +16,9 @@ COMBINE_KERNEL = "plow_moe_combine_fixed_order_gfx950"                          
 COMBINE_MARKERS = ["plow_moe_combine_fixed_order_abi_1", "plow_moe_combine_fixed_order_slots16_1",
                    "plow_moe_combine_materialized_f32_1", "plow_moe_combine_wave64_1",
                    "plow_moe_combine_no_spill_1"]                                  # amd.rs:11669-11675
+ELF_DEC = os.path.join(ROOT, "plow_amd", "moe_w8a8_dec_gfx950.elf")
+DEC_MARKER = "plow_moe_w8a8_dec_abi_1"                                            # amd.rs:10810
+DEC_KERNELS = {"plow_moe_w8a8_dec_glu": 96, "plow_moe_w8a8_dec_down": 80, "plow_moe_w8a8_dec_pair": 192}  # amd.rs:10827-10840
 KERNELS = ["plow_moe_fp8_glu_pf_gfx950", "plow_moe_fp8_down_pf_gfx950", "plow_moe_w8a8_glu_pf_gfx950",
            "plow_moe_w8a8_down_pf_gfx950", "plow_moe_w8a8_down_acc_pf_gfx950"]   # amd.rs:11720-11740
 
@@ -85,6 +88,38 @@ def test_combine_object_symbols_and_launch_shape():
         assert field("sgpr_spill_count") == 0 and field("vgpr_spill_count") == 0
 
 
+def test_decode_object_symbols_and_launch_shape():
+    """plowrt takes the decode object only with its marker, three kernels whose argument segments are 96,
+    80 and 192 bytes (or those + 256 bytes of hidden arguments) and no private memory; it launches 256
+    threads with no dynamic LDS (plow crates/plowrt/src/exec/amd.rs:10799-10852, :17748-17790)."""
+    if not os.path.exists(ELF_DEC):
+        pytest.fail(f"{ELF_DEC} is not built; run `python -m plow_amd.build`")
+    names, _ = elf_symbols(ELF_DEC)
+    assert DEC_MARKER in names
+    for k in DEC_KERNELS:
+        assert k in names and k + ".kd" in names, k
+    import re
+    import subprocess
+    readelf = "/opt/rocm/llvm/bin/llvm-readelf"
+    if os.path.exists(readelf):
+        notes = subprocess.run([readelf, "--notes", ELF_DEC], capture_output=True, text=True).stdout
+        blocks = re.split(r"\n\s+- \.agpr_count:", notes)
+        seen = 0
+        for blk in blocks:
+            m = re.search(r"\.name:\s+(plow_moe_w8a8_dec_\w+)\n", blk)
+            if not m:
+                continue
+            seen += 1
+            field = lambda f: int(re.search(r"\." + f + r":\s+(\d+)", blk).group(1))
+            want = DEC_KERNELS[m.group(1)]
+            assert field("kernarg_segment_size") in (want, want + 256), (m.group(1), field("kernarg_segment_size"))
+            assert field("private_segment_fixed_size") == 0
+            assert field("sgpr_spill_count") == 0 and field("vgpr_spill_count") == 0
+            assert field("max_flat_workgroup_size") >= 256
+            assert field("group_segment_fixed_size") <= 64 * 1024
+        assert seen == 3
+
+
 # ---- GPU: launch it the way plowrt does --------------------------------------------------------------
 
 class GluArgs(C.Structure):       # plow crates/plowrt/src/exec/amd.rs:1784-1807, 96 bytes
@@ -103,7 +138,12 @@ class CombineArgs(C.Structure):   # amd.rs:1768-1782, 48 bytes
                [(n, C.c_uint32) for n in ("hidden", "topk", "tokens", "reserved")]
 
 
+class DecPairArgs(C.Structure):   # amd.rs:3420-3430, 192 bytes
+    _fields_ = [("glu", GluArgs), ("down", DownArgs), ("ctr", C.c_uint64), ("grid_glu", C.c_uint32), ("reserved", C.c_uint32)]
+
+
 assert C.sizeof(GluArgs) == 96 and C.sizeof(DownArgs) == 80 and C.sizeof(CombineArgs) == 48
+assert C.sizeof(DecPairArgs) == 192
 
 
 class Module:
@@ -228,4 +268,74 @@ def test_combine_object_launched_like_plowrt(T, H, k, res, shr):
     moe.exec_many([d], table)
     torch.cuda.synchronize()
     assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
+    moe.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,shrink", [(24, 1), (5, 1), (70, 3)])
+def test_decode_object_launched_like_plowrt(oracle, T, shrink):
+    """The decode pair (op 85 arm 6 + op 86 arm 2) through `moe_w8a8_dec_gfx950.elf`: GLU and DOWN back to
+    back on plowrt's grids (2 * tiles * I / 128 and 2 * tiles * H / 256 workgroups of 256 threads,
+    amd.rs:3519-3520; `shrink` divides them, any grid must serve), then both in one launch of the pair
+    kernel with its counter scratch. Same arithmetic as the library's streaming kernel: bit-identical to
+    the library's own ops on the same inputs, and within tolerance of the oracle."""
+    import torch
+    from gpu_harness import assert_output_close, assert_routing_equal, run_oracle
+    from plow_amd import abi, layer, synth
+    from plow_amd.lib import Moe
+    print(f"[case] plowrt decode object T={T} shrink={shrink}", flush=True)
+    cfg = layer.MoeConfig("dec-obj", H=1024, E=8, I=256, k=2, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          enc="fp8blk", arm="w8a8q", n_shared=1, shared_mode="fold")
+    plan = layer.plan_layer(cfg)
+    dev = synth.bind(plan, "cuda", seed=T)
+    host = synth.to_host(dev)
+    run_oracle(oracle, plan, host)
+    moe = Moe(0)
+    table = dev.table()
+    moe.exec_many(plan.insts, table)               # the library's own run: the bits to reproduce
+    torch.cuda.synchronize()
+    assert_routing_equal(plan, dev, host)
+    assert_output_close(dev.np("out"), host.np("out"))
+    want = {n: dev.t[n].clone() for n in ("fq", "fs", "part")}
+    Ea = cfg.E_all
+    tiles = int(dev.np("meta")[3 * Ea])             # 64-row tiles of this batch (plowrt passes a bound on it)
+    grid_glu = max(1, 2 * tiles * (cfg.I // 128) // shrink)
+    grid_down = max(1, 2 * tiles * ((cfg.H + 255) // 256) // shrink)
+    p = lambda name: dev.t[name].data_ptr()
+    ga = GluArgs(p("fq"), p("x"), p("wtab"), p("stab"), p("meta"), p("row_token"), 0, p("fs"),
+                 cfg.I, cfg.H, Ea, cfg.act, 0.0, 0.0, 0, 0)
+    da = DownArgs(p("part"), p("fq"), p("wtab"), p("stab"), p("meta"), p("row_partidx"), p("row_gate"), p("fs"),
+                  cfg.H, cfg.I, Ea, 0)
+    m = Module(ELF_DEC, (DEC_MARKER,))
+
+    def wipe():
+        dev.t["fq"].fill_(0x55)
+        dev.t["fs"].fill_(7.0)
+        dev.t["part"].fill_(float("nan"))
+        torch.cuda.synchronize()
+
+    def check(what):
+        live = dev.np("row_partidx")[:tiles * 64] != abi.EXPERT_UNUSED
+        for n in ("fq", "fs"):
+            got, ref = dev.t[n][:tiles * 64].cpu().numpy()[live], want[n][:tiles * 64].cpu().numpy()[live]
+            assert np.array_equal(got.view(np.uint8), ref.view(np.uint8)), (what, n)
+        assert torch.equal(dev.t["part"].view(torch.int32), want["part"].view(torch.int32)), (what, "part")
+
+    wipe()
+    print(f"[launch] dec_glu grid={grid_glu}, dec_down grid={grid_down}", flush=True)
+    m.launch("plow_moe_w8a8_dec_glu", ga, grid_glu, threads=256)
+    m.launch("plow_moe_w8a8_dec_down", da, grid_down, threads=256)
+    torch.cuda.synchronize()
+    check("back to back")
+
+    wipe()
+    ctr = torch.zeros(4 * max(tiles, 1), dtype=torch.int32, device="cuda")
+    pa = DecPairArgs(ga, da, ctr.data_ptr(), grid_glu, 0)
+    for rep in range(2):                            # the second launch finds the scratch the first left
+        print(f"[launch] dec_pair grid={grid_glu}+{grid_down} rep={rep}", flush=True)
+        m.launch("plow_moe_w8a8_dec_pair", pa, grid_glu + grid_down, threads=256)
+        torch.cuda.synchronize()
+        check(f"pair rep {rep}")
+        assert int(ctr.abs().sum().item()) == 0
+        wipe()
     moe.close()
