@@ -87,7 +87,20 @@ enum {
     PLOW_DOP_MOE_GLU_MX_PF                 = 152, /* the same on gathered rows (after 83 / 84)   */
     PLOW_DOP_MOE_DOWN_MX_PF                = 153,
     PLOW_DOP_GEMM_F32                      = 180, /* router score: bf16 x bf16 -> f32 logits     */
-    PLOW_DOP_QUANT_FP8_BLOCK128            = 184  /* 1x128 e4m3 activation quant                 */
+    PLOW_DOP_QUANT_FP8_BLOCK128            = 184, /* 1x128 e4m3 activation quant                 */
+    /* the block-fp8 chain with a bf16 intermediate and a slot-major quantized copy of it, reduced into
+     * the layer output with bf16 atomics (crates/packet/src/dev.rs:2171-2180,
+     * runtime/amd/op_moe_fp8_block128.h:7-88, runtime/amd/interp.hip:5282-5310):
+     * 188 t0=fu bf16[R][I] t1=xq t2=xscale f32[H/128][T] t3=wtab t4=stab t5=meta t6=row_token
+     *     i0=I i1=H i2=E i3=T, fj[1] > 0: clamped SwiGLU with that limit; pad rows of every tile zeroed
+     * 189 t0=hq u8[T*topk][I] t1=fu t2=hscale f32[I/128][T*topk] t3=meta t4=row_partidx t5=out bf16[T][H]
+     *     i0=I i1=E i2=topk i3=T i4=H: aligned rows quantized 1x128 into their slot's row; out zeroed
+     * 190 t0=out t1=hq t2=hscale t3=wtab t4=stab t5=meta t6=row_partidx t7=row_gate
+     *     i0=I i1=H i2=E i3=topk i4=T: out[slot / topk] += bf16(gate * (Wd . hq[slot])), bf16 atomics
+     *     (the order of the additions, and so the rounding, is not fixed) */
+    PLOW_DOP_MOE_GLU_FP8_BLOCK128          = 188,
+    PLOW_DOP_MOE_QUANT_FP8_BLOCK128        = 189,
+    PLOW_DOP_MOE_DOWN_FP8_BLOCK128         = 190
 };
 
 /* Weight encodings (i3 on ops 85/86, i6 on ops 48/49; dev_isa.h:442-461, :691-702). */

@@ -26,6 +26,10 @@
  *   op 85/86 enc 2 arm 8, and
  *   op 48/49 (all enc)         runtime/cpu/dev/golden/moe.c:21-174 with runtime/cpu/dev/
  *                              mxfp4_common.h:30-40 as the row dot; op_moe.h:1234-1399
+ *   op 85 enc 1 arm 6          runtime/amd/moe_pf_w8a8.h:118-121, :255-283 (quantizer + arm 2)
+ *   op 188/189/190             runtime/amd/op_moe_fp8_block128.h:7-88, op_gemm_common.h:1845-2010,
+ *                              :2582-2621 (SCATTER), interp.hip:5282-5310; op 190 adds in aligned-row
+ *                              order where the device adds atomically in no fixed order
  *   op 65/66                   runtime/cpu/dev/golden/fp8.c:33-41, :173-214
  *   op 81/82                   runtime/amd/op_moe.h:6655-6700 (per-row x per-channel epilogue)
  *   op 20 / op 8               runtime/cpu/dev/golden/gemm.c:45-96
@@ -1014,6 +1018,156 @@ static void op_down_mx_pf(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
     free(a); free(wf);
 }
 
+/* ---- ops 188 / 189 / 190: block-fp8 chain with a bf16 intermediate and atomic reduction ---------- */
+
+/* 188 (plow runtime/amd/op_moe_fp8_block128.h:7-47, op_gemm_common.h:1845-2010 with GLU, GATHER):
+ * t0=fu t1=xq t2=xscale[H/128][T] t3=wtab t4=stab t5=meta t6=row_token  i0=I i1=H i2=E i3=T, fj[1] =
+ * clamp limit (> 0: gate min, up both sides). fu[r][n] = bf16((g * (1 / (1 + expf(-g)))) * u) for the
+ * rows r0 .. r0 + cnt of every expert (a row whose token is out of range computes on zeros), zeros
+ * for the pad rows up to the next multiple of 64; an expert without gate or up weights zeroes all of
+ * its rows. */
+static void op_glu_fp8_block128(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* fu = TEN(in, T, 0);
+    const uint8_t* xq = TEN(in, T, 1);
+    const float* xs = TEN(in, T, 2);
+    const uint64_t* wtab = TEN(in, T, 3);
+    const uint64_t* stab = TEN(in, T, 4);
+    const int32_t* meta = TEN(in, T, 5);
+    const uint32_t* row_token = TEN(in, T, 6);
+    const uint32_t I = in->i[0], H = in->i[1], E = in->i[2], Tn = in->i[3];
+    const float limit = in->fj[1].f;
+    const uint32_t G = (I + 127u) / 128u, KB = (H + 127u) / 128u;
+    float* wg = malloc((size_t)H * 4u);
+    float* wu = malloc((size_t)H * 4u);
+    float* zero_scale = calloc(KB, 4u);
+    RowCache rc;
+    cache_init(&rc, H);
+    uint32_t lo, hi;
+    own_range(E * G, slice, nblk, &lo, &hi);
+    for (uint32_t it = lo; it < hi; it++) {
+        const uint32_t e = it / G, g0 = it % G;
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        if (cnt == 0u) continue;
+        const uint32_t padded = (cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM * PLOW_MPF_BM;
+        const uint32_t n0 = g0 * 128u, n1 = n0 + 128u < I ? n0 + 128u : I;
+        const void* Wg = (const void*)(uintptr_t)wtab[(size_t)e * 3u + 0u];
+        const void* Wu = (const void*)(uintptr_t)wtab[(size_t)e * 3u + 1u];
+        const uint32_t live_rows = (Wg && Wu) ? cnt : 0u;
+        for (uint32_t q = live_rows; q < padded; q++)
+            for (uint32_t n = n0; n < n1; n++) fu[(size_t)(r0 + q) * I + n] = 0;
+        if (!live_rows) continue;
+        const float* Sg = (const float*)(uintptr_t)stab[(size_t)e * 3u + 0u];
+        const float* Su = (const float*)(uintptr_t)stab[(size_t)e * 3u + 1u];
+        if (rc.expert != e) {
+            cache_fit(&rc, cnt);
+            for (uint32_t q = 0; q < cnt; q++) {
+                const uint32_t tok = row_token[r0 + q];
+                rc.live[q] = tok < Tn;
+                if (rc.live[q]) decode_e4m3_row(rc.a + (size_t)q * H, xq + (size_t)tok * H, H);
+                else memset(rc.a + (size_t)q * H, 0, (size_t)H * 4u);
+            }
+            rc.expert = e;
+        }
+        for (uint32_t n = n0; n < n1; n++) {
+            decode_e4m3_row(wg, (const uint8_t*)Wg + (size_t)n * H, H);
+            decode_e4m3_row(wu, (const uint8_t*)Wu + (size_t)n * H, H);
+            for (uint32_t q = 0; q < cnt; q++) {
+                const float* a = rc.a + (size_t)q * H;
+                const float* as = rc.live[q] ? xs + row_token[r0 + q] : zero_scale;
+                const size_t step = rc.live[q] ? Tn : 1u;
+                float g = dot_fp8blk_a8(wg, Sg + (size_t)g0 * KB, a, as, step, H);
+                float u = dot_fp8blk_a8(wu, Su + (size_t)g0 * KB, a, as, step, H);
+                if (limit > 0.0f) {
+                    g = fminf(g, limit);
+                    u = fminf(fmaxf(u, -limit), limit);
+                }
+                fu[(size_t)(r0 + q) * I + n] = orc_f2bf((g * (1.0f / (1.0f + expf(-g)))) * u);
+            }
+        }
+    }
+    free(wg); free(wu); free(zero_scale);
+    cache_free(&rc);
+}
+
+/* 189 (op_moe_fp8_block128.h:49-55, op_gemm_common.h:2582-2621 with SCATTER; interp.hip:5291-5300):
+ * t0=hq[T*topk][I] t1=fu t2=hscale[I/128][T*topk] t3=meta t4=row_partidx t5=out bf16[T][H]
+ * i0=I i1=E i2=topk i3=T i4=H. Every aligned row of the tilep[E] * 64 whose slot is in range is
+ * quantized 1x128 into its slot's row; out is zeroed. */
+static void op_moe_quant_block128(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    uint8_t* hq = TEN(in, T, 0);
+    const orc_bf16* fu = TEN(in, T, 1);
+    float* hscale = TEN(in, T, 2);
+    const int32_t* meta = TEN(in, T, 3);
+    const uint32_t* row_partidx = TEN(in, T, 4);
+    orc_bf16* out = TEN(in, T, 5);
+    const uint32_t I = in->i[0], E = in->i[1], topk = in->i[2], Tn = in->i[3], H = in->i[4];
+    const uint32_t rows = (uint32_t)meta[3u * E] * PLOW_MPF_BM, slots = Tn * topk, G = I / 128u;
+    uint32_t lo, hi;
+    own_range(rows, slice, nblk, &lo, &hi);
+    for (uint32_t r = lo; r < hi; r++) {
+        const uint32_t dst = row_partidx[r];
+        if (dst >= slots) continue;
+        for (uint32_t g = 0; g < G; g++) {
+            const orc_bf16* src = fu + (size_t)r * I + g * 128u;
+            float amax = 1e-10f;
+            for (uint32_t j = 0; j < 128u; j++) amax = fmaxf(amax, fabsf(orc_bf2f(src[j])));
+            const float sc = amax * (1.0f / 448.0f), inv = 1.0f / sc;
+            hscale[(size_t)g * slots + dst] = sc;
+            for (uint32_t j = 0; j < 128u; j++)
+                hq[(size_t)dst * I + g * 128u + j] = orc_f32_to_e4m3(orc_bf2f(src[j]) * inv);
+        }
+    }
+    own_range(Tn, slice, nblk, &lo, &hi);
+    if (hi > lo) memset(out + (size_t)lo * H, 0, (size_t)(hi - lo) * H * 2u);
+}
+
+/* 190 (op_moe_fp8_block128.h:57-88 with ATOMIC, op_gemm_common.h:1845-2010 with GATHER, WEIGHTED,
+ * SCATTER, ATOMIC): t0=out t1=hq t2=hscale t3=wtab t4=stab t5=meta t6=row_partidx t7=row_gate
+ * i0=I i1=H i2=E i3=topk i4=T. out[slot / topk][h] += bf16(gate * (Wd[h] . hq[slot])), each addition
+ * rounded to bf16. The device adds with atomics in no fixed order; this restatement adds in aligned-row
+ * order (one of the orders the device may take), on slice 0 alone. */
+static void op_moe_down_block128(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    (void)nblk;
+    if (slice != 0u) return;
+    orc_bf16* out = TEN(in, T, 0);
+    const uint8_t* hq = TEN(in, T, 1);
+    const float* hscale = TEN(in, T, 2);
+    const uint64_t* wtab = TEN(in, T, 3);
+    const uint64_t* stab = TEN(in, T, 4);
+    const int32_t* meta = TEN(in, T, 5);
+    const uint32_t* row_partidx = TEN(in, T, 6);
+    const float* row_gate = TEN(in, T, 7);
+    const uint32_t I = in->i[0], H = in->i[1], E = in->i[2], topk = in->i[3], Tn = in->i[4];
+    const uint32_t slots = Tn * topk, KB = (I + 127u) / 128u;
+    float* wd = malloc((size_t)I * 4u);
+    RowCache rc;
+    cache_init(&rc, I);
+    for (uint32_t e = 0; e < E; e++) {
+        const uint32_t r0 = (uint32_t)meta[e], cnt = (uint32_t)meta[E + e];
+        const void* Wd = (const void*)(uintptr_t)wtab[(size_t)e * 3u + 2u];
+        if (cnt == 0u || !Wd) continue;
+        const float* Sd = (const float*)(uintptr_t)stab[(size_t)e * 3u + 2u];
+        cache_fit(&rc, cnt);
+        for (uint32_t q = 0; q < cnt; q++) {
+            const uint32_t dst = row_partidx[r0 + q];
+            rc.live[q] = dst < slots;
+            if (rc.live[q]) decode_e4m3_row(rc.a + (size_t)q * I, hq + (size_t)dst * I, I);
+        }
+        for (uint32_t h = 0; h < H; h++) {
+            decode_e4m3_row(wd, (const uint8_t*)Wd + (size_t)h * I, I);
+            for (uint32_t q = 0; q < cnt; q++) {
+                if (!rc.live[q]) continue;
+                const uint32_t dst = row_partidx[r0 + q];
+                const float acc = dot_fp8blk_a8(wd, Sd + (size_t)(h / 128u) * KB, rc.a + (size_t)q * I, hscale + dst, slots, I);
+                orc_bf16* o = out + (size_t)(dst / topk) * H + h;
+                *o = orc_f2bf(orc_bf2f(*o) + orc_bf2f(orc_f2bf(acc * row_gate[r0 + q])));
+            }
+        }
+    }
+    free(wd);
+    cache_free(&rc);
+}
+
 /* ---- dispatch ---------------------------------------------------------------------------------- */
 
 typedef void (*op_fn)(const PlowDevInst*, uint32_t, uint32_t, void* const*);
@@ -1044,6 +1198,9 @@ static op_fn resolve(uint16_t op) {
     case PLOW_DOP_MOE_DOWN_MX: return op_down_mx;
     case PLOW_DOP_MOE_GLU_MX_PF: return op_glu_mx_pf;
     case PLOW_DOP_MOE_DOWN_MX_PF: return op_down_mx_pf;
+    case PLOW_DOP_MOE_GLU_FP8_BLOCK128: return op_glu_fp8_block128;
+    case PLOW_DOP_MOE_QUANT_FP8_BLOCK128: return op_moe_quant_block128;
+    case PLOW_DOP_MOE_DOWN_FP8_BLOCK128: return op_moe_down_block128;
     default: return NULL;
     }
 }

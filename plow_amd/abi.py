@@ -36,6 +36,9 @@ OP_MOE_GLU_MX_PF = 152
 OP_MOE_DOWN_MX_PF = 153
 OP_GEMM_F32 = 180
 OP_QUANT_FP8_BLOCK128 = 184
+OP_MOE_GLU_FP8_BLOCK128 = 188
+OP_MOE_QUANT_FP8_BLOCK128 = 189
+OP_MOE_DOWN_FP8_BLOCK128 = 190
 
 ENC_BF16, ENC_FP8BLK, ENC_MXFP4 = 0, 1, 2
 ARM_A16, ARM_W8A8, ARM_W8A8_P16, ARM_W8A8_XQ, ARM_W4A16 = 0, 2, 3, 6, 8

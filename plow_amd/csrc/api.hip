@@ -193,6 +193,49 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         return launch_quant_row(ten(in, T, 0), ten(in, T, 1), (float*)ten(in, T, 2), ten(in, T, 3), ten(in, T, 4),
                                 i[2], i[0], i[1], st);
     }
+    case PLOW_DOP_MOE_GLU_FP8_BLOCK128: {
+        const uint32_t I = i[0], H = i[1], E = i[2], Tn = i[3];
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5) && ten(in, T, 6),
+             "op 188: t0 fu, t1 xq, t2 xscale, t3 wtab, t4 stab, t5 meta, t6 row_token must be bound");
+        NEED(c, I && H && E && Tn, "op 188: zero geometry");
+        NEED(c, I % 128u == 0u && H % 128u == 0u, "op 188: I %u and H %u must be multiples of 128", I, H);
+        if (!launch) return 0;
+        GroupW8A8 g = {};
+        g.out = ten(in, T, 0); g.out_bf16 = 1;
+        g.a = ten(in, T, 1); g.a_scale = (const float*)ten(in, T, 2);
+        g.wtab = (const uint64_t*)ten(in, T, 3); g.stab = (const uint64_t*)ten(in, T, 4);
+        g.meta = (const int32_t*)ten(in, T, 5); g.row_token = (const uint32_t*)ten(in, T, 6);
+        g.N = I; g.K = H; g.E = E; g.pitch = Tn; g.T = Tn;
+        /* SiLU, or the clamped SwiGLU when a limit is given (plow runtime/amd/op_gemm_common.h:1973-1981) */
+        g.f1 = in->fj[1].f; g.act = g.f1 > 0.0f ? PLOW_MOE_ACT_SWIGLU_CLAMP : PLOW_MOE_ACT_SILU;
+        return launch_group_glu_w8a8(g, st);
+    }
+    case PLOW_DOP_MOE_QUANT_FP8_BLOCK128: {
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5),
+             "op 189: t0 hq, t1 fu, t2 hscale, t3 meta, t4 row_partidx, t5 out must be bound");
+        NEED(c, i[0] && i[1] && i[2] && i[3] && i[4], "op 189: zero geometry");
+        NEED(c, i[0] % 128u == 0u && i[4] % 4u == 0u, "op 189: I %u must be a multiple of 128 and H %u of 4", i[0], i[4]);
+        if (!launch) return 0;
+        return launch_quant_block128_scatter(ten(in, T, 0), ten(in, T, 1), (float*)ten(in, T, 2), ten(in, T, 3),
+                                             ten(in, T, 4), ten(in, T, 5), i[0], i[1], i[2], i[3], i[4], st);
+    }
+    case PLOW_DOP_MOE_DOWN_FP8_BLOCK128: {
+        const uint32_t I = i[0], H = i[1], E = i[2], topk = i[3], Tn = i[4];
+        NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5) &&
+                    ten(in, T, 6) && ten(in, T, 7),
+             "op 190: t0 out, t1 hq, t2 hscale, t3 wtab, t4 stab, t5 meta, t6 row_partidx, t7 row_gate must be bound");
+        NEED(c, I && H && E && topk && Tn, "op 190: zero geometry");
+        NEED(c, I % 128u == 0u && H % 128u == 0u, "op 190: I %u and H %u must be multiples of 128", I, H);
+        if (!launch) return 0;
+        GroupW8A8 g = {};
+        g.out = ten(in, T, 0); g.acc_topk = topk;
+        g.a = ten(in, T, 1); g.a_scale = (const float*)ten(in, T, 2); g.a_slots = Tn * topk;
+        g.wtab = (const uint64_t*)ten(in, T, 3); g.stab = (const uint64_t*)ten(in, T, 4);
+        g.meta = (const int32_t*)ten(in, T, 5);
+        g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
+        g.N = H; g.K = I; g.E = E;
+        return launch_group_down_w8a8(g, st);
+    }
     case PLOW_DOP_MOE_GROUP_GLU_PF: {
         const uint32_t I = i[0], H = i[1], E = i[2], enc = i[3], arm = i[7];
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 4) && ten(in, T, 5),

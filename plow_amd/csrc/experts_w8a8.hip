@@ -43,6 +43,12 @@ __device__ __forceinline__ v4i ldg16_stream(const uint8_t* p) {
 #endif
 }
 
+typedef short sk_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void sk_atomic_add_bf16x2(bf16_t* p, float a, float b) {
+    const uint32_t pk = (uint32_t)f2bf(a) | ((uint32_t)f2bf(b) << 16);
+    __builtin_amdgcn_global_atomic_fadd_v2bf16((sk_bf16x2*)p, __builtin_bit_cast(sk_bf16x2, pk));
+}
+
 /* WIDE (DOWN, block mode only): a wave owns 32 channels as two 16-channel streams, a workgroup 256
  * channels; the short K loop of the down projection then amortises its prologue over twice the bytes.
  * NW: waves in the workgroup. The work item is always that of eight waves (128 channels, 256 WIDE);
@@ -82,7 +88,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
         valid[rt] = off < cnt;
         if (GLU) {
             const uint32_t tok = valid[rt] ? g.row_token[rowidx[rt]] : PLOW_EXPERT_UNUSED;
-            valid[rt] = tok != PLOW_EXPERT_UNUSED;
+            valid[rt] = tok != PLOW_EXPERT_UNUSED && (g.T == 0u || tok < g.T);
             const uint32_t t = valid[rt] ? tok : 0u;
             ap[rt] = (const uint8_t*)g.a + ((size_t)t * K + 16u * q) * (AQ ? 2u : 1u);
             asp[rt] = AQ ? nullptr : g.a_scale + t;
@@ -90,6 +96,12 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             const uint32_t pi = valid[rt] ? g.row_partidx[rowidx[rt]] : PLOW_EXPERT_UNUSED;
             valid[rt] = pi != PLOW_EXPERT_UNUSED;
             const uint32_t r = valid[rt] ? rowidx[rt] : r0;
+            ap[rt] = (const uint8_t*)g.a + (size_t)r * K + 16u * q;
+            asp[rt] = g.a_scale + r;
+        } else if (g.a_slots) { /* rows and scales stored by slot: [slot][K], [KB][a_slots] */
+            const uint32_t pi = valid[rt] ? g.row_partidx[rowidx[rt]] : PLOW_EXPERT_UNUSED;
+            valid[rt] = pi < g.a_slots;
+            const uint32_t r = valid[rt] ? pi : 0u;
             ap[rt] = (const uint8_t*)g.a + (size_t)r * K + 16u * q;
             asp[rt] = g.a_scale + r;
         } else {
@@ -100,7 +112,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             asp[rt] = g.a_scale + (size_t)r * KB;
         }
     }
-    as_stride = GLU ? g.pitch : 1u;
+    as_stride = GLU ? g.pitch : (!PC && g.a_slots ? g.a_slots : 1u);
 
     float vkeep[SUBS][RT][4]; /* block-mode GLU: a share's values until the group's amax is known */
 #pragma unroll
@@ -251,6 +263,22 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
                 *(float4*)((float*)g.out + (size_t)pidx * N + col) = make_float4(o[0], o[1], o[2], o[3]);
             }
         }
+    } else if (GLU && g.out_bf16) {
+        /* bf16 intermediate (op 188): bf16(act(g) * u) for live rows, zeros for the other rows of the tile */
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            const uint32_t off = rb + (uint32_t)rt * 16u + c;
+            uint2 pk = make_uint2(0u, 0u);
+            if (valid[rt]) {
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) o[i] = moe_glu(acc0[rt][i], acc1[rt][i], g.act, g.f0, g.f1);
+                pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
+                pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
+            }
+            if (off < ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM)
+                *(uint2*)((bf16_t*)g.out + (size_t)rowidx[rt] * N + col) = pk;
+        }
     } else if (GLU) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
@@ -271,6 +299,16 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             const uint32_t pidx = g.row_partidx[rowidx[rt]];
             const float gate = g.row_gate[rowidx[rt]];
             const float y0 = gate * acc0[rt][0], y1 = gate * acc0[rt][1], y2 = gate * acc0[rt][2], y3 = gate * acc0[rt][3];
+            if (g.acc_topk) { /* add into the layer output row of the slot's token, packed bf16 atomics */
+                bf16_t* orow = (bf16_t*)g.out + (size_t)(pidx / g.acc_topk) * N + col;
+                sk_atomic_add_bf16x2(orow, y0, y1);
+                sk_atomic_add_bf16x2(orow + 2, y2, y3);
+                if (WIDE) {
+                    sk_atomic_add_bf16x2(orow + 16, gate * acc1[rt][0], gate * acc1[rt][1]);
+                    sk_atomic_add_bf16x2(orow + 18, gate * acc1[rt][2], gate * acc1[rt][3]);
+                }
+                continue;
+            }
             if (g.part16) {
                 uint2 o;
                 o.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16);
@@ -294,7 +332,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
     }
     } /* sub */
 
-    if (GLU && !PC) {
+    if (GLU && !PC && !g.out_bf16) {
         __syncthreads();
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
@@ -326,15 +364,23 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles;
     const uint32_t cnt = (uint32_t)g.meta[g.E + e];
     if (cnt == 0u) return;
-    if (g.wtab[(size_t)e * (PC ? 2u : 3u) + (PC ? (GLU ? 0u : 1u) : (GLU ? 0u : 2u))] == 0ull) return; /* not resident */
     const uint32_t r0 = (uint32_t)g.meta[e];
+    const bool bf16_mid = GLU && (PC || g.out_bf16); /* the GLU owns every row of its 64-row tiles */
+    const uint32_t padded = ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
+    bool resident = g.wtab[(size_t)e * (PC ? 2u : 3u) + (PC ? (GLU ? 0u : 1u) : (GLU ? 0u : 2u))] != 0ull;
+    if (GLU && !PC && g.out_bf16) resident = resident && g.wtab[(size_t)e * 3u + 1u] != 0ull;
+    if (!resident) {
+        if (GLU && !PC && g.out_bf16) /* op 188 zeroes the rows of an expert it cannot compute */
+            for (uint32_t i = threadIdx.x; i < padded * (SK_BN / 4u); i += SK_THREADS)
+                *(uint2*)((bf16_t*)g.out + (size_t)(r0 + i / (SK_BN / 4u)) * g.N + ct * SK_BN + (i % (SK_BN / 4u)) * 4u) = make_uint2(0u, 0u);
+        return;
+    }
     /* 16 rows a pass; an expert with more rows streams its weights once per pass (the tiled
      * kernel, not this one, is the tool for many rows per expert) */
     for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D, PC, WIDE, SK_WAVES, AQ>(g, e, ct, r0, rb, cnt, s_red);
-    if (PC && GLU) {
-        /* the per-channel GLU zeroes the pad rows of its 64-row tile (the partial 16-row pass above
-         * did its own); the row quantizer that follows reads every aligned row */
-        const uint32_t padded = ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
+    if (bf16_mid) {
+        /* a GLU with a bf16 intermediate zeroes the pad rows of its 64-row tile (the partial 16-row pass
+         * above did its own); the row quantizer that follows reads every aligned row */
         const uint32_t first = ((cnt + 15u) / 16u) * 16u;
         for (uint32_t i = threadIdx.x; i < (padded - first) * (SK_BN / 4u); i += SK_THREADS) {
             const uint32_t r = r0 + first + i / (SK_BN / 4u), col = ct * SK_BN + (i % (SK_BN / 4u)) * 4u;
@@ -542,6 +588,10 @@ int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<true, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
+    if (g.out_bf16) { /* bf16 intermediate: the register form writes it */
+        k_group_w8a8_stream<true, 3, false><<<grid, SK_THREADS, 0, st>>>(g);
+        return 0;
+    }
     if (g.a_bf16) { /* bf16 rows, quantized where they are loaded */
         k_group_w8a8_stream<true, 3, false, false, true><<<grid, SK_THREADS, 0, st>>>(g);
         return 0;

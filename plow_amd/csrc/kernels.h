@@ -20,6 +20,9 @@ int launch_combine(void* out, const void* residual, const void* shared, const vo
 
 int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uint32_t K, uint32_t pitch,
                           hipStream_t st);
+int launch_quant_block128_scatter(void* hq, const void* fu, float* scale, const void* meta, const void* row_partidx,
+                                  void* out, uint32_t K, uint32_t E, uint32_t topk, uint32_t T, uint32_t H,
+                                  hipStream_t st);
 int launch_quant_row(void* xq, void* x, float* scale, const void* gate, const void* up, uint32_t act,
                      uint32_t M, uint32_t K, hipStream_t st);
 
@@ -47,6 +50,12 @@ struct GroupW8A8 {
     /* GLU, block mode: when non-zero, `a` holds the bf16 rows [T][K] themselves and the kernel quantizes
      * every 1x128 group as it loads it (a_scale and pitch unused; plow's arm i7 = 6) */
     uint32_t a_bf16;
+    /* GLU, block mode: write bf16(act(g) * u) rows [R][N] instead of quantized ones, zeros in the pad
+     * rows of every 64-row tile and in all rows of an expert without weights (op 188) */
+    uint32_t out_bf16;
+    /* DOWN, block mode: when non-zero, `a` and `a_scale` are stored by routing slot ([a_slots][K] and
+     * [K/128][a_slots]) and aligned row r reads slot row_partidx[r]; slots >= a_slots are skipped (op 190) */
+    uint32_t a_slots;
 };
 int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);

@@ -48,6 +48,60 @@ int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uin
     return 0;
 }
 
+/* Op 189 (plow runtime/amd/op_moe_fp8_block128.h:49-55, op_gemm_common.h:2582-2621 with SCATTER,
+ * interp.hip:5291-5300): the tilep[E] * 64 aligned bf16 rows, each quantized 1x128 into the row of its
+ * routing slot (hq[slot][K], scale[g][slot]; rows whose slot is out of range are skipped), and the bf16
+ * layer output [T][H] zeroed for the atomic reduction that follows. 16 lanes per (row, group). */
+__global__ __launch_bounds__(256) void k_quant_block128_scatter(uint8_t* __restrict__ hq, const bf16_t* __restrict__ fu,
+                                                                float* __restrict__ scale, const int32_t* __restrict__ meta,
+                                                                const uint32_t* __restrict__ row_partidx,
+                                                                uint2* __restrict__ out, uint32_t K, uint32_t E,
+                                                                uint32_t slots, size_t out_words) {
+    const uint32_t groups = K / 128u, sub = threadIdx.x & 15u;
+    const size_t ngroup = (size_t)((uint32_t)meta[3u * E] * PLOW_MPF_BM) * groups;
+    for (size_t grp = ((size_t)blockIdx.x * 256u + threadIdx.x) / 16u; grp < ngroup; grp += (size_t)gridDim.x * 16u) {
+        const uint32_t row = (uint32_t)(grp / groups), g = (uint32_t)(grp % groups);
+        const uint32_t dst = row_partidx[row];
+        if (dst >= slots) continue; /* the same for all 16 lanes of the group */
+        const uint4 raw = *(const uint4*)(fu + (size_t)row * K + g * 128u + sub * 8u);
+        const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+        float f[8];
+        float amax = 1e-10f; /* the amax is floored, not the scale */
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            f[2 * j] = __uint_as_float(v[j] << 16);
+            f[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+            amax = fmaxf(amax, fmaxf(fabsf(f[2 * j]), fabsf(f[2 * j + 1])));
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 16));
+        const float s = amax * (1.0f / 448.0f);
+        const float inv = 1.0f / s;
+        if (sub == 0) scale[(size_t)g * slots + dst] = s;
+        uint2 q;
+        q.x = cvt4_e4m3(f[0] * inv, f[1] * inv, f[2] * inv, f[3] * inv);
+        q.y = cvt4_e4m3(f[4] * inv, f[5] * inv, f[6] * inv, f[7] * inv);
+        *(uint2*)(hq + (size_t)dst * K + g * 128u + sub * 8u) = q;
+    }
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < out_words; i += (size_t)gridDim.x * 256u)
+        out[i] = make_uint2(0u, 0u);
+}
+
+int launch_quant_block128_scatter(void* hq, const void* fu, float* scale, const void* meta, const void* row_partidx,
+                                  void* out, uint32_t K, uint32_t E, uint32_t topk, uint32_t T, uint32_t H,
+                                  hipStream_t st) {
+    if (K % 128u || H % 4u || T == 0 || topk == 0 || E == 0) return PLOW_MOE_EINVAL;
+    /* the row count lives on the device (meta[3E]); size the grid for its upper bound */
+    const size_t rows_max = (size_t)T * topk + (size_t)E * (PLOW_MPF_BM - 1u);
+    const size_t ngroup = rows_max * (K / 128u), out_words = (size_t)T * H / 4u;
+    size_t want = (ngroup + 15u) / 16u;
+    if (want < (out_words + 255u) / 256u) want = (out_words + 255u) / 256u;
+    const uint32_t blocks = (uint32_t)(want > 8192u ? 8192u : want);
+    k_quant_block128_scatter<<<blocks, 256, 0, st>>>((uint8_t*)hq, (const bf16_t*)fu, scale, (const int32_t*)meta,
+                                                     (const uint32_t*)row_partidx, (uint2*)out, K, E, T * topk, out_words);
+    return 0;
+}
+
 /* e4m3 byte of plow's plow_f32_to_e4m3 (runtime/cpu/dev/fp8_common.h:16-33) for EVERY product
  * prod = x * inv: NaN keeps its sign (0x7f / 0xff), anything at or above 448 in magnitude saturates to
  * the signed 0x7e; in range the hardware conversion rounds as the reference does. A NaN that the

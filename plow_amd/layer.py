@@ -33,7 +33,10 @@ class MoeConfig:
     route_scale: float = 1.0
     enc: str = "fp8blk"             # "bf16" | "fp8blk" | "mxfp4" | "fp8pc" (per-channel)
     arm: str = "w8a8"               # "a16" (bf16 activations) | "w8a8" | "w8a8q" (block-fp8 only: the GLU
-                                    # quantizes the bf16 rows itself, plow's arm 6; no quantizer op)
+                                    # quantizes the bf16 rows itself, plow's arm 6; no quantizer op) |
+                                    # "w8a8atomic" (block-fp8 only: ops 184, 188, 189, 190 - bf16
+                                    # intermediate, slot-major quantized copy, bf16 atomic reduction into
+                                    # the output; no combine op, no residual / dense shared expert)
     n_shared: int = 0
     shared_mode: Optional[str] = None  # "fold" (slot {E, 1.0}) | "dense" (ops 20 + 8) | None
     act: int = abi.ACT_SILU
@@ -180,6 +183,22 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
         enc = {"bf16": abi.ENC_BF16, "fp8blk": abi.ENC_FP8BLK, "mxfp4": abi.ENC_MXFP4}[cfg.enc]
         wtab = p._t("wtab", "u64", (Ea, 3), "table")
         stab = p._t("stab", "u64", (Ea, 3), "table") if enc != abi.ENC_BF16 else None
+        if enc == abi.ENC_FP8BLK and cfg.arm == "w8a8atomic":
+            assert cfg.shared_mode != "dense" and not cfg.residual, "the atomic chain has no combine op"
+            xq = p._t("xq", "u8", (T, H), "scratch")
+            xs = p._t("xs", "f32", (H // 128, T), "scratch")
+            fu = p._t("fu", "bf16", (R, I), "scratch")
+            hq = p._t("hq", "u8", (T * ka, I), "scratch")
+            hs = p._t("hs", "f32", (I // 128, T * ka), "scratch")
+            p._emit("quant_x", abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[xq, x, xs], i=[T, H]))
+            p._emit("glu", abi.inst(abi.OP_MOE_GLU_FP8_BLOCK128, t=[fu, xq, xs, wtab, stab, meta, row_token],
+                                    i=[I, H, Ea, T], f=[0.0, cfg.act_f[1] if cfg.act == 4 else 0.0]))
+            p._emit("quant_fu", abi.inst(abi.OP_MOE_QUANT_FP8_BLOCK128, t=[hq, fu, hs, meta, row_partidx, out],
+                                         i=[I, Ea, ka, T, H]))
+            p._emit("down", abi.inst(abi.OP_MOE_DOWN_FP8_BLOCK128,
+                                     t=[out, hq, hs, wtab, stab, meta, row_partidx, row_gate],
+                                     i=[I, H, Ea, ka, T]))
+            return p
         if enc == abi.ENC_FP8BLK and cfg.arm in ("w8a8", "w8a8q"):
             fq = p._t("fq", "u8", (R, I), "scratch")
             fs = p._t("fs", "f32", (R, I // 128), "scratch")

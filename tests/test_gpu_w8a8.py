@@ -64,6 +64,38 @@ def test_glu_quantizes_bf16_rows_itself(moe, oracle, T):
     check_layer(plan, dev, host)
 
 
+@pytest.mark.parametrize("T,limit", [(1, 0.0), (19, 0.0), (100, 0.02), (333, 0.0)])
+def test_atomic_chain_ops_188_189_190(moe, oracle, T, limit):
+    """The block-fp8 chain with a bf16 intermediate (op 188), a slot-major quantized copy of it (op 189)
+    and a bf16 atomic reduction straight into the layer output (op 190), no combine op
+    (plow runtime/amd/op_moe_fp8_block128.h:7-88). The additions of op 190 come in no fixed order, each
+    rounded to bf16: the output is held to a few bf16 roundings of the oracle's, everything before it to
+    the usual bars."""
+    print(f"[case] w8a8 atomic chain T={T} limit={limit}", flush=True)
+    cfg = layer.MoeConfig("mini-atomic", H=512, E=32, I=256, k=4, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          n_group=4, topk_group=2, route_scale=2.5, enc="fp8blk", arm="w8a8atomic", n_shared=1,
+                          shared_mode="fold", act=4 if limit > 0 else 1, act_f=(0.0, limit))
+    plan, dev, host = both(moe, oracle, cfg, seed=T)
+    assert "combine" not in plan.names
+    rows = assert_routing_equal(plan, dev, host)
+    assert np.array_equal(dev.np("xq"), host.np("xq"))
+    fd, fh = ol.bf2f(dev.np("fu")[:rows]), ol.bf2f(host.np("fu")[:rows])
+    live = host.np("row_partidx")[:rows] != abi.EXPERT_UNUSED
+    assert not dev.np("fu")[:rows][~live].any()                  # pad rows of every tile are zeroed
+    same = (dev.np("fu")[:rows] == host.np("fu")[:rows]).mean()
+    print(f"[parity] fu bf16 identical on {same * 100:.3f} % of elements", flush=True)
+    assert same > 0.98 and np.abs(fd - fh).max() <= 2.0 ** -7 * np.abs(fh).max()
+    # the slot-major copy: dequantized values agree to fp8 precision
+    deq = lambda h: (torch.from_numpy(h.np("hq")).view(torch.float8_e4m3fn).float().numpy() *
+                     np.repeat(h.np("hs").T, 128, axis=1))
+    hd, hh = deq(dev), deq(host)
+    assert np.abs(hd - hh).max() <= 2.0 ** -3 * np.abs(hh).max()
+    got, want = ol.bf2f(dev.np("out")), ol.bf2f(host.np("out"))
+    assert np.all(np.isfinite(got))
+    assert np.abs(got - want).max() <= 3e-2 * np.abs(want).max()
+    assert np.abs(got - want).mean() <= 1e-2 * np.abs(want).mean()
+
+
 @pytest.mark.parametrize("T,act,f", [(24, 2, (2.0, 1.5)), (24, 4, (0.0, 0.75)), (600, 2, (3.0, 0.0)), (600, 4, (0.0, 0.75))])
 def test_pair_form_activations(moe, oracle, T, act, f):
     """Activations that transform the up branch too on op 85's block-fp8 W8A8 arm: 2 situ (beta, linear

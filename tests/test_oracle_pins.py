@@ -398,6 +398,75 @@ def test_fp8blk_inline_quant_arm_equals_quantizer_plus_plain_arm(oracle):
     assert (fq6 != 0x55).any()
 
 
+def test_fp8blk_atomic_chain_against_f64_and_the_plain_quantizer(oracle):
+    """Ops 188 / 189 / 190 (bf16 intermediate, slot-major quantized copy, bf16 reduction into the output;
+    plow runtime/amd/op_moe_fp8_block128.h:7-88): the GLU against an f64 evaluation of the same quantized
+    operands with the pad rows of every tile zeroed, the scatter quantizer bit for bit against the plain
+    1x128 quantizer applied to the rows put in slot order by hand, the reduction against f64 within the
+    rounding of k bf16 additions; the clamp limit of fj[1] acts on gate (above) and up (both sides)."""
+    r = cases.rng_of(31)
+    E, T, H, I, k = 4, 11, 256, 256, 2
+    W, S, wtab, stab = build_fp8(oracle, r, E, T, H, I, False, False)
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    for t in range(T):
+        tab["eid"][t * k:(t + 1) * k] = r.choice(E, k, replace=False)
+    tab["gate"] = (r.random(T * k) + 0.1).astype(np.float32)
+    al = cases.align_arrays(tab, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    meta, row_token, row_partidx, row_gate = al[0], al[2], al[3], al[4]
+    R = row_token.shape[0]
+    ntile = int(meta[3 * E])
+    x = cases.randn_bf16(r, (T, H), 1.0)
+    xq, xs = np.zeros((T, H), np.uint8), np.zeros((H // 128, T), np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[T, H]), [xq, x, xs])
+    xa = torch.from_numpy(xq).view(torch.float8_e4m3fn).double().numpy() * np.repeat(xs.T.astype(np.float64), 128, axis=1)
+    silu = lambda g: g / (1.0 + np.exp(-g))
+    for limit in (0.0, 0.05):
+        fu = np.full((R, I), 0x7FC0, np.uint16)
+        run(oracle, abi.inst(abi.OP_MOE_GLU_FP8_BLOCK128, t=[0, 1, 2, 3, 4, 5, 6], i=[I, H, E, T], f=[0.0, limit]),
+            [fu, xq, xs, wtab, stab, meta, row_token], 3)
+        fa = ol.bf2f(fu).astype(np.float64)
+        clamped = 0
+        for row in range(ntile * 64):
+            s_ = row_partidx[row]
+            if s_ == abi.EXPERT_UNUSED:
+                assert not fu[row].any()                        # pad rows of a tile are zeroed
+                continue
+            e, t = tab["eid"][s_], s_ // k
+            g = dequant(W["g"][e][1], S["g"][e]) @ xa[t]
+            u = dequant(W["u"][e][1], S["u"][e]) @ xa[t]
+            if limit > 0:
+                clamped += int((g > limit).sum() + (np.abs(u) > limit).sum())
+                g, u = np.minimum(g, limit), np.clip(u, -limit, limit)
+            v = silu(g) * u
+            assert np.all(np.abs(fa[row] - v) <= 2.0 ** -8 * np.abs(v).max() + 1e-6)
+        assert (fu[ntile * 64:] == 0x7FC0).all()                # nothing beyond the last tile is touched
+        assert limit == 0.0 or clamped > 0
+    # (fu now holds the clamped run) scatter quantizer == plain quantizer over the rows in slot order
+    slots = T * k
+    hq, hs = np.full((slots, I), 0x55, np.uint8), np.full((I // 128, slots), 7.0, np.float32)
+    out = np.full((T, H), 0x7FC0, np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_QUANT_FP8_BLOCK128, t=[0, 1, 2, 3, 4, 5], i=[I, E, k, T, H]),
+        [hq, fu, hs, meta, row_partidx, out], 3)
+    assert not out.any()
+    by_slot = np.zeros((slots, I), np.uint16)
+    for row in range(ntile * 64):
+        if row_partidx[row] != abi.EXPERT_UNUSED:
+            by_slot[row_partidx[row]] = fu[row]
+    hq2, hs2 = np.zeros((slots, I), np.uint8), np.zeros((I // 128, slots), np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[slots, I]), [hq2, by_slot, hs2])
+    assert np.array_equal(hq, hq2) and np.array_equal(hs.view(np.uint32), hs2.view(np.uint32))
+    # the reduction
+    run(oracle, abi.inst(abi.OP_MOE_DOWN_FP8_BLOCK128, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[I, H, E, k, T]),
+        [out, hq, hs, wtab, stab, meta, row_partidx, row_gate], 2)
+    ha = torch.from_numpy(hq).view(torch.float8_e4m3fn).double().numpy() * np.repeat(hs.T.astype(np.float64), 128, axis=1)
+    want = np.zeros((T, H))
+    for s_ in range(slots):
+        want[s_ // k] += float(tab["gate"][s_]) * (dequant(W["d"][tab["eid"][s_]][1], S["d"][tab["eid"][s_]]) @ ha[s_])
+    got = ol.bf2f(out).astype(np.float64)
+    assert np.abs(got - want).max() <= k * 2.0 ** -8 * np.abs(want).max()
+
+
 def test_fp8blk_constant_block_scale_factors_out(oracle):
     """A constant scale grid c equals c times the unit-scale result (c a power of two: exactly)."""
     r = cases.rng_of(12)
