@@ -437,8 +437,14 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     const uint32_t cnt = (uint32_t)g.meta[g.E + e];
     if (cnt == 0u) return;
     const uint64_t wp0 = g.wtab[(size_t)e * 3u], wp1 = g.wtab[(size_t)e * 3u + 1u];
-    if (wp0 == 0ull) return; /* not resident */
     const uint32_t r0 = (uint32_t)g.meta[e];
+    const uint32_t padded = ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
+    if (wp0 == 0ull || (g.out_bf16 && wp1 == 0ull)) { /* not resident; the bf16 form zeroes what it cannot compute */
+        if (g.out_bf16)
+            for (uint32_t i = threadIdx.x; i < padded * (SK_BN / 4u); i += SK_THREADS)
+                *(uint2*)((bf16_t*)g.out + (size_t)(r0 + i / (SK_BN / 4u)) * g.N + ct * SK_BN + (i % (SK_BN / 4u)) * 4u) = make_uint2(0u, 0u);
+        return;
+    }
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, 32-byte chunk q */
@@ -470,13 +476,14 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
 
     for (uint32_t rb = 0; rb < cnt; rb += 16u) {
         /* activation rows of the pass: load i covers rows 8i .. 8i + 7 */
-        const uint32_t tok0 = g.row_token[r0 + rb];
+        uint32_t tok0 = g.row_token[r0 + rb];
+        if (g.T != 0u && tok0 >= g.T) tok0 = 0u; /* any readable row: its scale is zeroed below */
         const uint8_t* xsrc[2];
 #pragma unroll
         for (uint32_t i = 0; i < 2u; i++) {
             const uint32_t row = 8u * i + lr, off = rb + row;
             uint32_t tok = off < cnt ? g.row_token[r0 + off] : PLOW_EXPERT_UNUSED;
-            if (tok == PLOW_EXPERT_UNUSED) tok = tok0;
+            if (tok == PLOW_EXPERT_UNUSED || (g.T != 0u && tok >= g.T)) tok = tok0;
             xsrc[i] = (const uint8_t*)g.a + (size_t)tok * K + ((p ^ ((row >> 1) & 7u)) << 4);
         }
         const float* ssrc;
@@ -484,11 +491,15 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
         {
             const uint32_t off = rb + c;
             const uint32_t tok = off < cnt ? g.row_token[r0 + off] : PLOW_EXPERT_UNUSED;
-            const bool ok = tok != PLOW_EXPERT_UNUSED;
+            const bool ok = tok != PLOW_EXPERT_UNUSED && (g.T == 0u || tok < g.T);
             ssrc = ok ? g.a_scale + tok : (const float*)(g.meta + 2u * g.E); /* tilep[0] = 0 */
             sstep = ok ? g.pitch : 0u;
         }
-        const bool valid = rb + c < cnt && g.row_token[r0 + rb + c] != PLOW_EXPERT_UNUSED;
+        bool valid = rb + c < cnt;
+        if (valid) {
+            const uint32_t tok = g.row_token[r0 + rb + c];
+            valid = tok != PLOW_EXPERT_UNUSED && (g.T == 0u || tok < g.T);
+        }
         auto issue = [&](uint32_t kb) {
             SdSlot* s = ring + kb % SD_STAGES;
             __builtin_amdgcn_global_load_lds((const void*)(ssrc + (size_t)kb * sstep), (sd_lds_void*)&s->xs[0], 4, 0, 0);
@@ -532,6 +543,18 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
             }
         }
         /* ---- epilogue: lane holds channels chw + 4q + i (i = 0..3) of row rb + c ---- */
+        if (g.out_bf16) { /* bf16 intermediate: live rows get bf16(act(g) * u), the tile's other rows zeros */
+            uint2 pk = make_uint2(0u, 0u);
+            if (valid) {
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) o[i] = moe_glu(acc0[i], acc1[i], g.act, g.f0, g.f1);
+                pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
+                pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
+            }
+            if (rb + c < padded) *(uint2*)((bf16_t*)g.out + (size_t)(r0 + rb + c) * N + chw + 4u * q) = pk;
+            continue;
+        }
         float v[4], m = 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -552,6 +575,11 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
             if (wv == 0 && q == 0) g.out_scale[(size_t)row * (N / 128u) + ct] = s;
         }
         __syncthreads(); /* L.red is reused by the next pass */
+    }
+    if (g.out_bf16) { /* pad rows of the last 64-row tile that no 16-row pass covered */
+        const uint32_t first = ((cnt + 15u) / 16u) * 16u;
+        for (uint32_t i = threadIdx.x; i < (padded - first) * (SK_BN / 4u); i += SK_THREADS)
+            *(uint2*)((bf16_t*)g.out + (size_t)(r0 + first + i / (SK_BN / 4u)) * N + ct * SK_BN + (i % (SK_BN / 4u)) * 4u) = make_uint2(0u, 0u);
     }
 }
 
@@ -588,7 +616,7 @@ int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<true, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
-    if (g.out_bf16) { /* bf16 intermediate: the register form writes it */
+    if (g.out_bf16 && !glu_dma_form()) { /* bf16 intermediate on the register form */
         k_group_w8a8_stream<true, 3, false><<<grid, SK_THREADS, 0, st>>>(g);
         return 0;
     }

@@ -514,7 +514,157 @@ __global__ __launch_bounds__(128) void k_router_score_wave(float* __restrict__ o
     if (m < M && n < N) out[(size_t)m * N + n] = acc;
 }
 
-/* PLOW_MOE_SCORE_KERNEL=valu keeps the prefill score on the vector unit (for comparison) */
+/* Few outputs (decode): TOK tokens x 64 experts per workgroup, one consumer wave per token. Every output
+ * is a chain of K dependent multiply-adds (2 ns a step on this chip), so the kernel's time is the chain's
+ * and the job is to keep everything else off the consumer waves' instruction streams:
+ *  - four stager waves (16 weight rows each) own every global load. They widen the weight rows to f32
+ *    into a double-buffered LDS tile shared by the consumers and copy the tokens' bf16 rows beside it.
+ *    Their loads are written by hand (uniform chunk base + a per-lane byte offset that never changes)
+ *    and waited for by count, RSR_PF - 1 chunks (about 100 KB a workgroup) in flight: at the chain's pace
+ *    a chunk lasts half a microsecond, less than one trip to memory, and loads the compiler issues in a
+ *    loop like this one end up waited for in full at every chunk;
+ *  - a consumer lane (one expert) reads 4 k of its weight row per 16-byte LDS read, and its token's x
+ *    sixteen steps at a time: lane l holds x[16 g + l % 16] and the multiply-add takes its x operand
+ *    from lane i of the lane's row of 16 (row broadcast), so one register serves 16 steps and the chain
+ *    is one instruction a step.
+ * K must be a multiple of RSR_KC and the weight tensor smaller than 2 GiB (32-bit lane offsets). */
+#define RSR_KC 256
+#define RSR_LD (RSR_KC + 4) /* floats per LDS row: consecutive rows start 4 banks apart */
+#define RSR_PF 4
+#define RSR_STAGERS 4u
+#define RSR_WS_BYTES (2u * 64u * RSR_LD * 4u)
+template <uint32_t TOK>
+__global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(float* __restrict__ out,
+                                                                                const bf16_t* __restrict__ x,
+                                                                                const bf16_t* __restrict__ w,
+                                                                                uint32_t M, uint32_t N, uint32_t K) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t rsr_raw[];
+    float* const rsr_ws = (float*)rsr_raw;                        /* [2][64][RSR_LD] f32 weights */
+    bf16_t* const rsr_xs = (bf16_t*)(rsr_raw + RSR_WS_BYTES);     /* [2][TOK][RSR_KC] bf16 tokens */
+    constexpr int KC = RSR_KC, LD = RSR_LD;
+    constexpr int NL = 8 + (int)TOK; /* loads per stager and chunk */
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t n0 = blockIdx.x * 64u, m0 = blockIdx.y * TOK;
+    const uint32_t NC = K / KC;
+    if (wv >= TOK) {
+        /* a row of a chunk is 32 16-byte pieces; lane l loads piece l % 32 of rows base + l / 32, + 2, ...
+         * (8 rows of this stager's 16) and of every token's row (only the first stager stores those) */
+        const uint32_t pc = lane & 31u, sidx = wv - TOK, rbase = sidx * 16u + (lane >> 5);
+        v4i wr[RSR_PF][8], xr[RSR_PF][TOK];
+        uint32_t voff[8], xoff[TOK];
+#pragma unroll
+        for (int i = 0; i < 8; i++) { /* a row past N repeats the last row (never stored) */
+            const uint32_t r = n0 + rbase + 2u * i;
+            voff[i] = ((r < N ? r : N - 1u) * K + pc * 8u) * 2u;
+        }
+#pragma unroll
+        for (uint32_t t = 0; t < TOK; t++) xoff[t] = ((m0 + t < M ? m0 + t : M - 1u) * K + pc * 8u) * 2u;
+        auto fetch = [&](int st, uint32_t c) { /* a chunk past the end repeats the last chunk (never read) */
+            const size_t off = (size_t)(c < NC ? c : NC - 1u) * (KC * 2u);
+            const char* wb = (const char*)w + off;
+            const char* xb = (const char*)x + off;
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(wr[st][i]) : "v"(voff[i]), "s"(wb) : "memory");
+#pragma unroll
+            for (uint32_t t = 0; t < TOK; t++)
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(xr[st][t]) : "v"(xoff[t]), "s"(xb) : "memory");
+        };
+        auto commit = [&](int st, uint32_t buf) {
+            /* loads return in order: this stage's have landed once at most those of the RSR_PF - 1
+             * younger stages are outstanding */
+            asm volatile("s_waitcnt vmcnt(%8)"
+                         : "+v"(wr[st][0]), "+v"(wr[st][1]), "+v"(wr[st][2]), "+v"(wr[st][3]), "+v"(wr[st][4]),
+                           "+v"(wr[st][5]), "+v"(wr[st][6]), "+v"(wr[st][7])
+                         : "n"((RSR_PF - 1) * NL)
+                         : "memory");
+#pragma unroll
+            for (uint32_t t = 0; t < TOK; t++) asm volatile("" : "+v"(xr[st][t]));
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const uint32_t r = rbase + 2u * i;
+                float* d = rsr_ws + ((size_t)buf * 64u + r) * LD + pc * 8u;
+                const v4i a = wr[st][i];
+                *(float4*)d = make_float4(__uint_as_float((uint32_t)a[0] << 16), __uint_as_float((uint32_t)a[0] & 0xFFFF0000u),
+                                          __uint_as_float((uint32_t)a[1] << 16), __uint_as_float((uint32_t)a[1] & 0xFFFF0000u));
+                *(float4*)(d + 4) = make_float4(__uint_as_float((uint32_t)a[2] << 16), __uint_as_float((uint32_t)a[2] & 0xFFFF0000u),
+                                                __uint_as_float((uint32_t)a[3] << 16), __uint_as_float((uint32_t)a[3] & 0xFFFF0000u));
+            }
+            if (sidx == 0u && lane < 32u) {
+#pragma unroll
+                for (uint32_t t = 0; t < TOK; t++) *(v4i*)(rsr_xs + ((size_t)buf * TOK + t) * KC + pc * 8u) = xr[st][t];
+            }
+        };
+#pragma unroll
+        for (int st = 0; st < RSR_PF; st++) fetch(st, (uint32_t)st);
+        commit(0, 0);
+        for (uint32_t c0 = 0; c0 < NC; c0 += RSR_PF) {
+#pragma unroll
+            for (int st = 0; st < RSR_PF; st++) {
+                const uint32_t c = c0 + (uint32_t)st;
+                if (c < NC) {
+                    lds_barrier(); /* chunk c is published; the consumers are done with chunk c - 1 */
+                    fetch(st, c + RSR_PF); /* register stage st held chunk c, already in LDS */
+                    if (c + 1u < NC) commit((st + 1) % RSR_PF, (c + 1u) & 1u);
+                }
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* nothing in flight into dead registers at the end */
+        return;
+    }
+    const uint32_t m = m0 + wv, l16 = lane & 15u;
+    float acc = 0.0f;
+/* four steps in one statement (no filler between them): x from lanes I .. I + 3 of the row, w = one float4 */
+#define RSR_FMAC4(I0, I1, I2, I3, W)                                                                       \
+    asm volatile("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #I0 " row_mask:0xf bank_mask:0xf\n\t"            \
+                 "v_fmac_f32_dpp %0, %1, %3 row_newbcast:" #I1 " row_mask:0xf bank_mask:0xf\n\t"            \
+                 "v_fmac_f32_dpp %0, %1, %4 row_newbcast:" #I2 " row_mask:0xf bank_mask:0xf\n\t"            \
+                 "v_fmac_f32_dpp %0, %1, %5 row_newbcast:" #I3 " row_mask:0xf bank_mask:0xf"                 \
+                 : "+v"(acc)                                                                               \
+                 : "v"(xv), "v"((W).x), "v"((W).y), "v"((W).z), "v"((W).w))
+    for (uint32_t c = 0; c < NC; c++) {
+        const uint32_t buf = c & 1u;
+        lds_barrier(); /* chunk c is in buffer c & 1 */
+        const float* wp = rsr_ws + ((size_t)buf * 64u + lane) * LD;
+        const bf16_t* xp = rsr_xs + ((size_t)buf * TOK + wv) * KC + l16;
+        float xf[KC / 16];
+#pragma unroll
+        for (int g = 0; g < KC / 16; g++) xf[g] = __uint_as_float((uint32_t)xp[16 * g] << 16);
+        /* operand reads run one 16-k group ahead of the multiply-adds */
+        float4 b[2][4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) b[0][u] = *(const float4*)(wp + 4 * u);
+        asm volatile("s_nop 1" ::: "memory"); /* the row-broadcast operand was written by vector instructions */
+#pragma unroll
+        for (int gq = 0; gq < KC / 16; gq++) {
+            const int cur = gq & 1, nxt = cur ^ 1;
+            if (gq + 1 < KC / 16) {
+#pragma unroll
+                for (int u = 0; u < 4; u++) b[nxt][u] = *(const float4*)(wp + 16 * (gq + 1) + 4 * u);
+            }
+            const float xv = xf[gq];
+            RSR_FMAC4(0, 1, 2, 3, b[cur][0]);
+            RSR_FMAC4(4, 5, 6, 7, b[cur][1]);
+            RSR_FMAC4(8, 9, 10, 11, b[cur][2]);
+            RSR_FMAC4(12, 13, 14, 15, b[cur][3]);
+        }
+    }
+#undef RSR_FMAC4
+    const uint32_t n = n0 + lane;
+    if (m < M && n < N) out[(size_t)m * N + n] = acc;
+}
+
+/* PLOW_MOE_SCORE_KERNEL=tile8 keeps the few-output score on the 8 x 8 tile kernel (for comparison) */
+static bool score_row_form() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = getenv("PLOW_MOE_SCORE_KERNEL");
+        v = (e && !strcmp(e, "tile8")) ? 0 : 1;
+    }
+    return v == 1;
+}
+
 static bool score_mfma_form() {
     static int v = -1;
     if (v < 0) {
@@ -574,6 +724,25 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
             dim3 g((N + 63) / 64, (M + 63) / 64);
             k_router_score_tile<4><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
         }
+    } else if (score_row_form() && K % RSR_KC == 0u && (uint64_t)N * K * 2u < (1ull << 31) && (uint64_t)M * K * 2u < (1ull << 31) &&
+               (M < 16u || (uint64_t)M * N <= 2048u)) {
+        /* measured against the 8 x 8 tile kernel below: ahead with one or two tokens per workgroup (6 of
+         * 38 us at 1 x 384 x 7168) and with four on small score matrices (16 x 64 x 2048: 17 against
+         * 25 us); with four tokens on a large one the shared LDS tile is the limit and the two are level */
+        /* tokens per workgroup: as many as keep the weight rows' re-reads (once per workgroup row) low */
+        static bool attr_set = false;
+        const uint32_t lds = RSR_WS_BYTES + 2u * 4u * RSR_KC * 2u;
+        if (!attr_set) {
+            if (hipFuncSetAttribute((const void*)k_router_score_row<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
+                hipFuncSetAttribute((const void*)k_router_score_row<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
+                hipFuncSetAttribute((const void*)k_router_score_row<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+                return PLOW_MOE_EDEVICE;
+            attr_set = true;
+        }
+        const uint32_t nx = (N + 63) / 64;
+        if (M >= 16u) k_router_score_row<4><<<dim3(nx, (M + 3u) / 4u), (4u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        else if (M >= 4u) k_router_score_row<2><<<dim3(nx, (M + 1u) / 2u), (2u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        else k_router_score_row<1><<<dim3(nx, M), (1u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else {
         dim3 g((N + 7) / 8, (M + 7) / 8);
         k_router_score_wave<<<g, 128, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);

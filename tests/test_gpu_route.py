@@ -101,7 +101,11 @@ def test_route_and_align_match_oracle(moe, oracle, E, k, T, flags, ng, tg, tail)
 # K a multiple of 64 and 2^17 outputs or more: the matrix-unit forms. 16 x 32 tiles with 4, 2, 1, 16 and 3
 # chunks (the fifth is ragged in both directions); the last two fill the SIMDs evenly with 32 x 32 tiles and
 # take that form (2 and 3 chunks)
-@pytest.mark.parametrize("M,N,K", [(6, 40, 768), (64, 256, 7168), (1, 384, 7168), (700, 1000, 264),
+# Few outputs and K a multiple of 256: one token x 64 experts per consumer wave, 1 / 2 / 4 tokens per
+# workgroup (ragged in tokens and experts: (3, 100), (15, 130), (17, 100)); (6, 40, 768) etc. on the 8 x 8 tiles
+@pytest.mark.parametrize("M,N,K", [(3, 100, 512), (2, 64, 256), (5, 64, 1280), (15, 130, 1024), (16, 64, 2048),
+                                   (17, 100, 512), (1, 128, 4096), (8, 128, 4096),
+                                   (6, 40, 768), (64, 256, 7168), (1, 384, 7168), (700, 1000, 264),
                                    (700, 1000, 256), (520, 520, 128), (1030, 300, 64), (1500, 288, 1024),
                                    (413, 331, 192), (1024, 1024, 128), (2048, 512, 192)])
 def test_router_score_bit_exact(moe, oracle, M, N, K):
