@@ -208,7 +208,11 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.N = I; g.K = H; g.E = E; g.pitch = Tn; g.T = Tn;
         /* SiLU, or the clamped SwiGLU when a limit is given (plow runtime/amd/op_gemm_common.h:1973-1981) */
         g.f1 = in->fj[1].f; g.act = g.f1 > 0.0f ? PLOW_MOE_ACT_SWIGLU_CLAMP : PLOW_MOE_ACT_SILU;
-        return launch_group_glu_w8a8(g, st);
+        /* many rows per expert (16 or more on average at the last align): tiled form, which leaves the
+         * rows of an expert without weights unwritten where the streaming form zeroes them (op 190 skips
+         * such an expert either way) */
+        c->tiled = (c->forced >= 0 ? c->forced : (c->rows_hint >= 16u ? 1 : 0)) && H >= 256u && I >= 256u;
+        return c->tiled ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
     }
     case PLOW_DOP_MOE_QUANT_FP8_BLOCK128: {
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5),
@@ -234,7 +238,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 5);
         g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
         g.N = H; g.K = I; g.E = E;
-        return launch_group_down_w8a8(g, st);
+        const int tiled = (c->forced >= 0 ? c->forced : c->tiled) && g.K >= 256u && g.N >= 256u;
+        return tiled ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_PF: {
         const uint32_t I = i[0], H = i[1], E = i[2], enc = i[3], arm = i[7];

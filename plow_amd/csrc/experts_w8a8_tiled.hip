@@ -363,7 +363,15 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
 #pragma unroll
             for (uint32_t i = 0; i < 4u; i++) { /* token rows 32 * cw + 8 * i + lr; a pad row reads the first row */
                 const uint32_t row = 32u * cw + 8u * i + lr;
-                P.tok[i] = GLU ? g.row_token[r0 + (row < rows ? row : 0u)] : r0 + (row < rows ? row : 0u);
+                const uint32_t ar = r0 + (row < rows ? row : 0u);
+                if (GLU) {
+                    P.tok[i] = g.row_token[ar];
+                } else if (!PC && g.a_slots) { /* rows stored by routing slot: read the slot's row */
+                    const uint32_t slot = g.row_partidx[ar];
+                    P.tok[i] = slot < g.a_slots ? slot : 0u;
+                } else {
+                    P.tok[i] = ar;
+                }
             }
             {
                 const uint32_t row = (cw & 1u) * 64u + lane; /* the row whose activation scale this lane loads */
@@ -415,6 +423,10 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 if (GLU) {
                     S.ssrc = ok ? g.a_scale + P.stok : (const float*)(g.meta + 2u * g.E);
                     S.sstep = ok ? g.pitch : 0u;
+                } else if (!PC && g.a_slots) { /* scales [KB][a_slots], by slot */
+                    const bool in = ok && P.stok < g.a_slots;
+                    S.ssrc = in ? g.a_scale + P.stok : (const float*)(g.meta + 2u * g.E);
+                    S.sstep = in ? g.a_slots : 0u;
                 } else {
                     S.ssrc = ok ? g.a_scale + (size_t)(r0 + row) * KB : (const float*)(g.meta + 2u * g.E);
                     S.sstep = ok ? 1u : 0u;
@@ -552,7 +564,36 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
              *      group 0 and up in group 1; DOWN channel = ch0 + 16 * x + 4q + i ---- */
             const uint32_t stl = st >= 1u ? st - 1u : 2u; /* the ring stage the tile has just left */
-            if (!PC && GLU) {
+            if (!PC && GLU && g.out_bf16) {
+                /* bf16 intermediate (op 188): bf16(act(g) * u) for live rows, zeros for the pad rows of the
+                 * expert's last 64-row tile */
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); /* pairs with the loaders' */
+                const uint32_t cnt_e = (uint32_t)g.meta[g.E + t.e], erow0 = r0 - (uint32_t)g.meta[t.e];
+                const uint32_t padded = ((cnt_e + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
+#pragma unroll
+                for (uint32_t sub = 0; sub < SUBS; sub++) {
+                    const uint32_t cw = cw0 + sub, ch0 = nt * 128u + 16u * cw;
+                    v4f(&acc)[8][2] = accs[sub];
+#pragma unroll
+                    for (int rg = 0; rg < 8; rg++) {
+                        const uint32_t row = 16u * (uint32_t)rg + r16;
+                        bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
+                        if (row >= rows) {
+                            if (erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u);
+                            continue;
+                        }
+                        uint2 pk = make_uint2(0u, 0u);
+                        if (L.epi_idx[par][row] != PLOW_EXPERT_UNUSED) {
+                            float o[4];
+#pragma unroll
+                            for (int i = 0; i < 4; i++) o[i] = t5_glu(acc[rg][0][i], acc[rg][1][i], g.act, g.f0, g.f1);
+                            pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
+                            pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
+                        }
+                        *(uint2*)orow = pk;
+                    }
+                }
+            } else if (!PC && GLU) {
                 float v[SUBS][8][4];
 #pragma unroll
                 for (uint32_t sub = 0; sub < SUBS; sub++) {

@@ -64,7 +64,7 @@ def test_glu_quantizes_bf16_rows_itself(moe, oracle, T):
     check_layer(plan, dev, host)
 
 
-@pytest.mark.parametrize("T,limit", [(1, 0.0), (19, 0.0), (100, 0.02), (333, 0.0)])
+@pytest.mark.parametrize("T,limit", [(1, 0.0), (19, 0.0), (100, 0.02), (333, 0.0), (700, 0.02)])  # from 16 rows per expert: tiled form
 def test_atomic_chain_ops_188_189_190(moe, oracle, T, limit):
     """The block-fp8 chain with a bf16 intermediate (op 188), a slot-major quantized copy of it (op 189)
     and a bf16 atomic reduction straight into the layer output (op 190), no combine op
