@@ -62,6 +62,13 @@ typedef struct {
 
 /* ---- opcodes served (numbers from runtime/common/dev_isa.h) ---------------------------------- */
 enum {
+    PLOW_DOP_RMSNORM                       = 1,   /* the step before the path: t0=out t1=x t2=gamma?
+                                                     t3=xq? t4=scale? i0=rows i1=feat i2=out_row0 f0=eps;
+                                                     t3 bound: also quantize the rounded row, per row
+                                                     (scale f32[rows], as op 32) or, with i4 = 128, per
+                                                     1x128 group (scale f32[feat/128][rows], as op 184)
+                                                     (runtime/cpu/dev/golden/norm.c:15-43,
+                                                     runtime/amd/op_norm.h:486-551)                 */
     PLOW_DOP_GEMM                          = 8,   /* dense bf16 GEMM (shared-expert down)        */
     PLOW_DOP_GEMM_GLU                      = 20,  /* dense bf16 gate|up + GLU (shared expert)    */
     PLOW_DOP_QUANT_FP8                     = 32,  /* per-row e4m3 activation quant; any K; with

@@ -16,6 +16,7 @@
  *   op 84 align                runtime/cpu/dev/golden/moe_route.c:91-127
  *   op 87/43 combine           runtime/cpu/dev/golden/moe_route.c:130-147; t_row0 / part16
  *                              runtime/amd/interp.hip:6605-6635
+ *   op 1 RMSNorm (+ quant)     runtime/cpu/dev/golden/norm.c:6-43; 1x128 form runtime/amd/op_norm.h:486-551
  *   op 184 1x128 quant         runtime/amd/op_gemm_common.h:2582-2621
  *   op 32 per-row quant        runtime/cpu/dev/golden/fp8.c:9-30
  *   op 85/86 enc 0 (bf16)      runtime/cpu/dev/golden/moe_gemma.c:244-302 through the wtab[E][3]
@@ -1018,6 +1019,48 @@ static void op_down_mx_pf(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
     free(a); free(wf);
 }
 
+/* ---- op 1: RMSNorm with its fused quantizers ------------------------------------------------------ */
+
+/* t0=out t1=x t2=gamma? t3=xq? t4=scale? i0=rows i1=feat i2=out_row0 i4=128: 1x128 groups  f0=eps
+ * (plow runtime/cpu/dev/golden/norm.c:6-43: sum of squares in index order, inv = 1 / sqrtf, out =
+ * bf16(x * inv * gamma), per-row quant of the ROUNDED row with scale = max(amax / 448, 1e-12); the
+ * 1x128 form of runtime/amd/op_norm.h:486-551 quantizes the rounded row like op 184). */
+static void op_rmsnorm(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
+    orc_bf16* out = TEN(in, T, 0);
+    const orc_bf16* x = TEN(in, T, 1);
+    const orc_bf16* gamma = TEN(in, T, 2);
+    uint8_t* q = TEN(in, T, 3);
+    float* scale = TEN(in, T, 4);
+    const uint32_t rows = in->i[0], feat = in->i[1], out_row0 = in->i[2], blk = in->i[4] == 128u;
+    const float eps = in->fj[0].f;
+    uint32_t lo, hi;
+    own_range(rows, slice, nblk, &lo, &hi);
+    for (uint32_t row = lo; row < hi; row++) {
+        const orc_bf16* xr = x + (size_t)row * feat;
+        orc_bf16* o = out + (size_t)(out_row0 + row) * feat;
+        float ss = 0.0f;
+        for (uint32_t i = 0; i < feat; i++) { const float v = orc_bf2f(xr[i]); ss += v * v; }
+        const float inv = 1.0f / sqrtf(ss / (float)feat + eps);
+        for (uint32_t i = 0; i < feat; i++) o[i] = orc_f2bf(orc_bf2f(xr[i]) * inv * (gamma ? orc_bf2f(gamma[i]) : 1.0f));
+        if (!q) continue;
+        if (blk) {
+            for (uint32_t g = 0; g < feat / 128u; g++) {
+                float amax = 1e-10f;
+                for (uint32_t j = 0; j < 128u; j++) amax = fmaxf(amax, fabsf(orc_bf2f(o[g * 128u + j])));
+                const float sc = amax * (1.0f / 448.0f), qi = 1.0f / sc;
+                scale[(size_t)g * rows + row] = sc;
+                for (uint32_t j = 0; j < 128u; j++) q[(size_t)row * feat + g * 128u + j] = orc_f32_to_e4m3(orc_bf2f(o[g * 128u + j]) * qi);
+            }
+        } else {
+            float amax = 0.0f;
+            for (uint32_t i = 0; i < feat; i++) amax = fmaxf(amax, fabsf(orc_bf2f(o[i])));
+            scale[row] = fmaxf(amax * (1.0f / 448.0f), 1e-12f);
+            const float qi = 1.0f / scale[row];
+            for (uint32_t i = 0; i < feat; i++) q[(size_t)row * feat + i] = orc_f32_to_e4m3(orc_bf2f(o[i]) * qi);
+        }
+    }
+}
+
 /* ---- ops 188 / 189 / 190: block-fp8 chain with a bf16 intermediate and atomic reduction ---------- */
 
 /* 188 (plow runtime/amd/op_moe_fp8_block128.h:7-47, op_gemm_common.h:1845-2010 with GLU, GATHER):
@@ -1198,6 +1241,7 @@ static op_fn resolve(uint16_t op) {
     case PLOW_DOP_MOE_DOWN_MX: return op_down_mx;
     case PLOW_DOP_MOE_GLU_MX_PF: return op_glu_mx_pf;
     case PLOW_DOP_MOE_DOWN_MX_PF: return op_down_mx_pf;
+    case PLOW_DOP_RMSNORM: return op_rmsnorm;
     case PLOW_DOP_MOE_GLU_FP8_BLOCK128: return op_glu_fp8_block128;
     case PLOW_DOP_MOE_QUANT_FP8_BLOCK128: return op_moe_quant_block128;
     case PLOW_DOP_MOE_DOWN_FP8_BLOCK128: return op_moe_down_block128;

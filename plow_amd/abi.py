@@ -12,6 +12,7 @@ MPF_BM = 64
 ROUTE_MAX_TOPK = 16
 
 # opcodes (runtime/common/dev_isa.h)
+OP_RMSNORM = 1
 OP_GEMM = 8
 OP_GEMM_GLU = 20
 OP_QUANT_FP8 = 32

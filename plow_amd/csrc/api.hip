@@ -193,6 +193,18 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         return launch_quant_row(ten(in, T, 0), ten(in, T, 1), (float*)ten(in, T, 2), ten(in, T, 3), ten(in, T, 4),
                                 i[2], i[0], i[1], st);
     }
+    case PLOW_DOP_RMSNORM: {
+        NEED(c, ten(in, T, 0) && ten(in, T, 1), "op 1: t0 out and t1 x must be bound");
+        NEED(c, !ten(in, T, 3) == !ten(in, T, 4), "op 1: quantized row (t3) and scale (t4) must be bound together");
+        NEED(c, i[0] && i[1] && i[1] % 8u == 0u && i[1] <= 16384u, "op 1: rows %u, feat %u (a multiple of 8, at most 16384)", i[0], i[1]);
+        const uint32_t mode = !ten(in, T, 3) ? 0u : (i[4] == 128u ? 2u : 1u);
+        NEED(c, mode != 2u || i[1] % 128u == 0u, "op 1: 1x128 quantization needs feat %u to be a multiple of 128", i[1]);
+        NEED(c, mode == 0u || i[2] == 0u, "op 1: the quantizing forms take no output row offset");
+        NEED(c, i[3] == 0u && i[7] == 0u, "op 1: i3 / i7 variants are not served");
+        if (!launch) return 0;
+        return launch_rmsnorm(ten(in, T, 0), ten(in, T, 1), ten(in, T, 2), ten(in, T, 3), (float*)ten(in, T, 4), i[0], i[1],
+                              i[2], in->fj[0].f, mode, st);
+    }
     case PLOW_DOP_MOE_GLU_FP8_BLOCK128: {
         const uint32_t I = i[0], H = i[1], E = i[2], Tn = i[3];
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5) && ten(in, T, 6),

@@ -23,6 +23,8 @@ int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uin
 int launch_quant_block128_scatter(void* hq, const void* fu, float* scale, const void* meta, const void* row_partidx,
                                   void* out, uint32_t K, uint32_t E, uint32_t topk, uint32_t T, uint32_t H,
                                   hipStream_t st);
+int launch_rmsnorm(void* out, const void* x, const void* gamma, void* xq, float* scale, uint32_t rows, uint32_t feat,
+                   uint32_t out_row0, float eps, uint32_t mode, hipStream_t st);
 int launch_quant_row(void* xq, void* x, float* scale, const void* gate, const void* up, uint32_t act,
                      uint32_t M, uint32_t K, hipStream_t st);
 

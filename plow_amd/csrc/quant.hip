@@ -224,3 +224,123 @@ int launch_quant_row(void* xq, void* x, float* scale, const void* gate, const vo
         k_quant_row<false><<<M, 256, 0, st>>>((uint8_t*)xq, (bf16_t*)x, scale, (const bf16_t*)gate, (const bf16_t*)up, act, K);
     return 0;
 }
+
+
+/* Op 1, RMSNorm with its fused activation quantizers (plow runtime/cpu/dev/golden/norm.c:15-43,
+ * runtime/amd/op_norm.h:486-551): out[row0 + r] = bf16(x[r] * inv * gamma) with
+ * inv = 1 / sqrt(mean(x^2) + eps) in f32 (the sum of squares in a fixed tree order, as plow's GPU kernel
+ * does; its CPU kernel sums in index order, a difference of rounding only), gamma optional. MODE 1: the
+ * rounded row is also quantized per row like op 32 (scale = max(amax / 448, 1e-12)); MODE 2: per 1x128
+ * group like op 184 (amax floored at 1e-10, scale [feat / 128][rows]) - in both cases exactly what the
+ * separate quantizer produces from `out`. One workgroup per row; a thread keeps its share of the row
+ * (8 elements per 256-thread stride, feat <= 16384) in registers between the passes. */
+#define RN_MAXV 8
+template <int MODE>
+__global__ __launch_bounds__(256) void k_rmsnorm(bf16_t* __restrict__ out, const bf16_t* __restrict__ x,
+                                                 const bf16_t* __restrict__ gamma, uint8_t* __restrict__ xq,
+                                                 float* __restrict__ scale, uint32_t rows, uint32_t feat,
+                                                 uint32_t out_row0, float eps) {
+    __shared__ float red[4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
+    auto block_reduce = [&](float v, bool is_max) -> float {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float other = __shfl_xor(v, o, 64);
+            v = is_max ? fmaxf(v, other) : v + other;
+        }
+        __syncthreads(); /* the previous reduction's values have been read */
+        if (lane == 0) red[wv] = v;
+        __syncthreads();
+        return is_max ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : (red[0] + red[1]) + (red[2] + red[3]);
+    };
+    for (uint32_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const bf16_t* xr = x + (size_t)row * feat;
+        bf16_t* orow = out + (size_t)(out_row0 + row) * feat;
+        float f[RN_MAXV][8];
+        float ss = 0.0f;
+#pragma unroll
+        for (int c = 0; c < RN_MAXV; c++) {
+            const uint32_t i = ((uint32_t)c * 256u + tid) * 8u;
+#pragma unroll
+            for (int j = 0; j < 8; j++) f[c][j] = 0.0f;
+            if (i < feat) {
+                const uint4 raw = *(const uint4*)(xr + i);
+                const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    f[c][2 * j] = __uint_as_float(v[j] << 16);
+                    f[c][2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++) ss += f[c][j] * f[c][j];
+            }
+        }
+        ss = block_reduce(ss, false);
+        const float inv = 1.0f / sqrtf(ss / (float)feat + eps);
+        float amax_row = 0.0f;
+#pragma unroll
+        for (int c = 0; c < RN_MAXV; c++) {
+            const uint32_t i = ((uint32_t)c * 256u + tid) * 8u;
+            float amax = 1e-10f; /* MODE 2: the amax is floored, not the scale */
+            if (i < feat) {
+                uint4 graw = make_uint4(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u); /* ones */
+                if (gamma) graw = *(const uint4*)(gamma + i);
+                const uint32_t gv[4] = {graw.x, graw.y, graw.z, graw.w};
+                uint32_t o[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float g = (j & 1) ? __uint_as_float(gv[j >> 1] & 0xFFFF0000u) : __uint_as_float(gv[j >> 1] << 16);
+                    o[j] = f2bf(gamma ? f[c][j] * inv * g : f[c][j] * inv * 1.0f);
+                    f[c][j] = bf2f((bf16_t)o[j]); /* the quantizers read the rounded row */
+                    amax = fmaxf(amax, fabsf(f[c][j]));
+                }
+                *(uint4*)(orow + i) = make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
+            }
+            if (MODE == 2) { /* a 128-group is 16 consecutive threads' 8 elements; feat % 128 == 0 keeps groups whole */
+#pragma unroll
+                for (int o2 = 8; o2 > 0; o2 >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o2, 16));
+                if (i < feat) {
+                    const float sc = amax * (1.0f / 448.0f), qi = 1.0f / sc;
+                    if ((tid & 15u) == 0u) scale[(size_t)(i / 128u) * rows + row] = sc;
+                    uint2 q;
+                    q.x = cvt4_e4m3(f[c][0] * qi, f[c][1] * qi, f[c][2] * qi, f[c][3] * qi);
+                    q.y = cvt4_e4m3(f[c][4] * qi, f[c][5] * qi, f[c][6] * qi, f[c][7] * qi);
+                    *(uint2*)(xq + (size_t)row * feat + i) = q;
+                }
+            }
+            if (MODE == 1 && i < feat) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) amax_row = fmaxf(amax_row, fabsf(f[c][j]));
+            }
+        }
+        if (MODE == 1) {
+            amax_row = block_reduce(amax_row, true);
+            const float sc = fmaxf(amax_row * (1.0f / 448.0f), 1e-12f), qi = 1.0f / sc;
+            if (tid == 0) scale[row] = sc;
+#pragma unroll
+            for (int c = 0; c < RN_MAXV; c++) {
+                const uint32_t i = ((uint32_t)c * 256u + tid) * 8u;
+                if (i < feat) {
+                    uint2 q = make_uint2(0u, 0u);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        q.x |= e4m3_any(f[c][j] * qi, f[c][j]) << (8 * j);
+                        q.y |= e4m3_any(f[c][4 + j] * qi, f[c][4 + j]) << (8 * j);
+                    }
+                    *(uint2*)(xq + (size_t)row * feat + i) = q;
+                }
+            }
+        }
+    }
+}
+
+int launch_rmsnorm(void* out, const void* x, const void* gamma, void* xq, float* scale, uint32_t rows, uint32_t feat,
+                   uint32_t out_row0, float eps, uint32_t mode, hipStream_t st) {
+    if (rows == 0 || feat == 0 || feat % 8u || feat > RN_MAXV * 256u * 8u) return PLOW_MOE_EINVAL;
+    if (mode == 2u && feat % 128u) return PLOW_MOE_EINVAL;
+    const uint32_t blocks = rows < 65535u ? rows : 65535u;
+    if (mode == 2u) k_rmsnorm<2><<<blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)gamma, (uint8_t*)xq, scale, rows, feat, out_row0, eps);
+    else if (mode == 1u) k_rmsnorm<1><<<blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)gamma, (uint8_t*)xq, scale, rows, feat, out_row0, eps);
+    else k_rmsnorm<0><<<blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)gamma, nullptr, nullptr, rows, feat, out_row0, eps);
+    return 0;
+}

@@ -5,7 +5,7 @@ Run where the plow tree is mounted:   make -C oracle ref && python tests/golden/
 The fixtures hold inputs and expected outputs only; tests/test_golden.py replays them through the
 in-repo oracle on any machine. Reference op numbers used: 83/84/87 routing, 180 router score,
 75/76 bf16 grouped experts, 150-153 flat mxfp4 experts, 65/66 per-channel fp8 decode
-experts, 32 per-row activation quant, 20/8 dense GLU / GEMM.
+experts, 32 per-row activation quant, 20/8 dense GLU / GEMM, 1 RMSNorm.
 """
 import os
 import sys
@@ -204,6 +204,20 @@ def main():
     fug = np.zeros((rows, I), np.uint16)
     run(abi.inst(152, t=[0, 1, 2, 3, 4, 5, 6], i=[I, K, E, 0, 0, 3], f=(1.702, 7.0)), [fug, x, Wgu, Sgu, al[0], al[2], bgu], nblk=3)
     out["mxflat/pf_fu_act3"] = fug
+
+    # --- RMSNorm op 1 (its own generator, after everything above): plain with gamma and a row offset,
+    # weightless, and with the per-row quantizer fused
+    rn = cases.rng_of(1001)
+    rows, feat = 5, 384
+    xn, gam = cases.randn_bf16(rn, (rows, feat), 1.5), cases.randn_bf16(rn, (feat,), 1.0)
+    o1 = np.zeros((rows + 2, feat), np.uint16)
+    run(abi.inst(1, t=[0, 1, 2], i=[rows, feat, 2], f=[1e-6]), [o1, xn, gam], nblk=2)
+    o2 = np.zeros((rows, feat), np.uint16)
+    run(abi.inst(1, t=[0, 1], i=[rows, feat, 0], f=[1e-5]), [o2, xn], nblk=1)
+    o3, q3, s3 = np.zeros((rows, feat), np.uint16), np.zeros((rows, feat), np.uint8), np.zeros(rows, np.float32)
+    run(abi.inst(1, t=[0, 1, 2, 3, 4], i=[rows, feat, 0], f=[1e-6]), [o3, xn, gam, q3, s3], nblk=3)
+    out.update({"rmsnorm/x": xn, "rmsnorm/gamma": gam, "rmsnorm/out_row2": o1, "rmsnorm/out_plain": o2,
+                "rmsnorm/out_q": o3, "rmsnorm/xq": q3, "rmsnorm/scale": s3})
 
     path = os.path.join(HERE, "plow_cpu_golden.npz")
     np.savez_compressed(path, **out)

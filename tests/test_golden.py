@@ -259,3 +259,26 @@ def test_dense_shared_expert(oracle):
     y = np.zeros((M, K), np.uint16)
     run(oracle, abi.inst(abi.OP_GEMM, t=[0, 1, 2], i=[M, K, N]), [y, fu, wd], 2)
     assert np.array_equal(y, G["dense/y"])
+
+
+def test_rmsnorm_and_its_per_row_quantizer(oracle):
+    """Op 1 against plow's CPU kernel (runtime/cpu/dev/golden/norm.c:15-43): gamma with an output row
+    offset, weightless, and with the per-row quantizer of the rounded row."""
+    x, gam = G["rmsnorm/x"], G["rmsnorm/gamma"]
+    rows, feat = x.shape
+    o1 = np.zeros((rows + 2, feat), np.uint16)
+    run(oracle, abi.inst(abi.OP_RMSNORM, t=[0, 1, 2], i=[rows, feat, 2], f=[1e-6]), [o1, x, gam], 2)
+    assert np.array_equal(o1, G["rmsnorm/out_row2"]) and not o1[:2].any()
+    o2 = np.zeros((rows, feat), np.uint16)
+    run(oracle, abi.inst(abi.OP_RMSNORM, t=[0, 1], i=[rows, feat, 0], f=[1e-5]), [o2, x], 1)
+    assert np.array_equal(o2, G["rmsnorm/out_plain"])
+    o3, q3, s3 = np.zeros((rows, feat), np.uint16), np.zeros((rows, feat), np.uint8), np.zeros(rows, np.float32)
+    run(oracle, abi.inst(abi.OP_RMSNORM, t=[0, 1, 2, 3, 4], i=[rows, feat, 0], f=[1e-6]), [o3, x, gam, q3, s3], 3)
+    assert np.array_equal(o3, G["rmsnorm/out_q"]) and np.array_equal(q3, G["rmsnorm/xq"])
+    assert np.array_equal(s3.view(np.uint32), G["rmsnorm/scale"].view(np.uint32))
+    # the 1x128 form (AMD only): by definition the 1x128 quantizer op over the rounded row
+    o4, q4, s4 = np.zeros((rows, feat), np.uint16), np.zeros((rows, feat), np.uint8), np.zeros((feat // 128, rows), np.float32)
+    run(oracle, abi.inst(abi.OP_RMSNORM, t=[0, 1, 2, 3, 4], i=[rows, feat, 0, 0, 128], f=[1e-6]), [o4, x, gam, q4, s4], 2)
+    q5, s5 = np.zeros((rows, feat), np.uint8), np.zeros((feat // 128, rows), np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[rows, feat]), [q5, o4, s5], 1)
+    assert np.array_equal(o4, o3) and np.array_equal(q4, q5) and np.array_equal(s4.view(np.uint32), s5.view(np.uint32))

@@ -206,3 +206,42 @@ def test_refusals(moe):
     assert moe.check(abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[4, 100]), t) == abi.E_INVAL
     with pytest.raises(Exception):
         moe.exec(abi.inst(abi.OP_MOE_ALIGN_PF, t=[0, 1, 2, 3], i=[4, 8, 2]), t)
+
+
+@pytest.mark.parametrize("rows,feat,gamma", [(5, 384, True), (64, 7168, True), (3, 16384, False), (7, 8, True), (300, 2048, True)])
+def test_rmsnorm_with_fused_quantizers(moe, oracle, rows, feat, gamma):
+    """Op 1, the step before the path (plow runtime/cpu/dev/golden/norm.c:15-43, runtime/amd/op_norm.h:
+    486-551). The sum of squares is a tree here and an index-order loop in the oracle (as in plow's GPU
+    and CPU kernels): the normalized row may differ in the last bf16 bit now and then, no more. The fused
+    quantizers must produce exactly what the separate quantizer ops produce from the row this kernel
+    wrote: per row (as op 32) and per 1x128 group (as op 184)."""
+    print(f"[case] rmsnorm rows={rows} feat={feat} gamma={gamma}", flush=True)
+    r = cases.rng_of(rows + feat)
+    x = cases.randn_bf16(r, (rows, feat), 1.5)
+    g = cases.randn_bf16(r, (feat,), 1.0) if gamma else None
+    want = np.zeros((rows, feat), np.uint16)
+    ol.run(oracle.plow_oracle_exec, abi.inst(abi.OP_RMSNORM, t=[0, 1, 2 if gamma else None], i=[rows, feat], f=[1e-6]),
+           ol.table_of([want, x, g]), 4)
+    dx, dg = to_dev(x), (to_dev(g) if gamma else None)
+    for mode in (0, 1, 2):
+        if mode == 2 and feat % 128:
+            continue
+        out = torch.zeros((rows, feat), dtype=torch.int16, device="cuda")
+        xq = torch.zeros((rows, feat), dtype=torch.uint8, device="cuda")
+        sc = torch.zeros((feat // 128, rows) if mode == 2 else (rows,), dtype=torch.float32, device="cuda")
+        t = [0, 1, 2 if gamma else None] + ([3, 4] if mode else [])
+        moe.exec(abi.inst(abi.OP_RMSNORM, t=t, i=[rows, feat, 0, 0, 128 if mode == 2 else 0], f=[1e-6]),
+                 dev_table([out, dx, dg, xq, sc]))
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(np.uint16)
+        a, b = ol.bf2f(got), ol.bf2f(want)
+        assert (got == want).mean() > 0.99
+        assert np.all(np.abs(a - b) <= 2.0 ** -7 * np.abs(b) + 1e-30)          # one bf16 step at most
+        if mode:
+            q2 = np.zeros((rows, feat), np.uint8)
+            s2 = np.zeros(tuple(sc.shape), np.float32)
+            op = abi.OP_QUANT_FP8 if mode == 1 else abi.OP_QUANT_FP8_BLOCK128
+            row_in = np.ascontiguousarray(got)          # held here: the table keeps nothing alive
+            ol.run(oracle.plow_oracle_exec, abi.inst(op, t=[0, 1, 2], i=[rows, feat]), ol.table_of([q2, row_in, s2]), 2)
+            assert np.array_equal(xq.cpu().numpy(), q2)
+            assert np.array_equal(sc.cpu().numpy().view(np.uint32), s2.view(np.uint32))
