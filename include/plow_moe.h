@@ -38,7 +38,14 @@ typedef union {
 typedef struct {
     uint16_t op;
     uint16_t blocks; /* workgroups the producer sliced the op across; advisory for this library */
-    PlowFJ   fj[3];
+    PlowFJ   fj[3];  /* fj[2].u on a grouped expert op (75, 76, 81, 82, 85, 86, 152, 153, 188, 190): the
+                      * routed slots T * k of the batch if the producer states them, 0 = not stated. An
+                      * extension of this library (no MoE op of the reference uses the third immediate):
+                      * these ops carry no row count, and the kernel form that serves them best depends on
+                      * it. Without it the count is taken from the align op (84) of the same
+                      * plow_moe_exec_many / segment run, then from what the op's own operands imply;
+                      * unknown means few rows. It never changes a result, and nothing is remembered
+                      * between calls. */
     uint16_t t[8];   /* handles into the tensor table; PLOW_TENSOR_NONE = absent => NULL */
     uint32_t i[8];
 } PlowDevInst;

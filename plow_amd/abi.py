@@ -75,9 +75,10 @@ def max_rows(T, k, n_exp):
     return T * k + n_exp * (MPF_BM - 1)
 
 
-def inst(op, t=(), i=(), f=(), blocks=1):
+def inst(op, t=(), i=(), f=(), blocks=1, slots=0):
     """Build one descriptor. ``t``: up to 8 handles (None = absent); ``i``: up to 8 ints;
-    ``f``: up to 3 floats placed in fj[n].f."""
+    ``f``: up to 3 floats placed in fj[n].f; ``slots``: the routed slots (T * k) of the batch in
+    fj[2].u, this library's row-count statement on the grouped expert ops (0 = not stated)."""
     d = PlowDevInst()
     d.op, d.blocks = op, blocks
     for n in range(8):
@@ -87,6 +88,8 @@ def inst(op, t=(), i=(), f=(), blocks=1):
         d.i[n] = int(v) & 0xFFFFFFFF
     for n, v in enumerate(f):
         d.fj[n].f = float(v)
+    if slots:
+        d.fj[2].u = int(slots)
     return d
 
 

@@ -29,6 +29,7 @@ SOURCES = {
     "experts_a16.hip": [],
     "experts_w8a8_tiled.hip": [],
     "api.hip": [],
+    "device.hip": [],
 }
 
 

@@ -14,34 +14,51 @@
 
 #include "../../include/plow_moe.h"
 #include "kernels.h"
+#include "tuning.h"
 
-/* Slot-major ops (48 / 49 / 65 / 66) are served by sorting their slots by expert into this
- * context-owned workspace first, so that every hit expert streams its weights once. */
+/* Slot-major ops (48 / 49 / 65 / 66, 150 / 151) are served by sorting their slots by expert into a
+ * workspace first, so that every hit expert streams its weights once; the flat-tensor ops (150 - 153)
+ * build their per-expert pointer tables there. A context owns one sized for WS_MAX_SLOTS slots. Nothing in a
+ * workspace has to start at zero: every word a kernel reads was written earlier in the same call. */
 #define WS_MAX_E 1056u
 #define WS_MAX_SLOTS (1u << 18)
-#define WS_MAX_ROWS (WS_MAX_SLOTS + WS_MAX_E * (PLOW_MPF_BM - 1u))
-#define WS_MAX_CHUNKS (WS_MAX_SLOTS / 1024u)
+
+struct Workspace {
+    uint32_t max_e, max_slots, max_chunks;
+    int32_t* meta;        /* [3 * max_e + 1] */
+    uint32_t* row_token;  /* [max_slots + max_e * (PLOW_MPF_BM - 1)] */
+    uint32_t* row_partidx;
+    float* row_gate;
+    uint32_t* chunk_hist; /* [max_chunks][max_e] scratch of the multi-workgroup align */
+    uint64_t* ftab;       /* [2][max_e][3] pointer tables built for the flat-tensor ops (150 - 153) */
+};
+static constexpr size_t ws_up(size_t v) { return (v + 255u) & ~(size_t)255u; }
+static constexpr size_t ws_rows(uint32_t max_e, uint32_t max_slots) { return (size_t)max_slots + (size_t)max_e * (PLOW_MPF_BM - 1u); }
+/* bytes of one workspace laid out in a single 256-byte aligned block */
+static constexpr size_t ws_bytes(uint32_t max_e, uint32_t max_slots) {
+    return ws_up((3u * (size_t)max_e + 1u) * 4u) + 3u * ws_up(ws_rows(max_e, max_slots) * 4u) +
+           ws_up((size_t)((max_slots + 1023u) / 1024u) * max_e * 4u) + ws_up((size_t)2u * max_e * 3u * 8u);
+}
+static Workspace ws_carve(void* base, uint32_t max_e, uint32_t max_slots) {
+    Workspace w = {};
+    char* p = (char*)base;
+    w.max_e = max_e, w.max_slots = max_slots, w.max_chunks = (max_slots + 1023u) / 1024u;
+    w.meta = (int32_t*)p, p += ws_up((3u * (size_t)max_e + 1u) * 4u);
+    const size_t rb = ws_up(ws_rows(max_e, max_slots) * 4u);
+    w.row_token = (uint32_t*)p, p += rb;
+    w.row_partidx = (uint32_t*)p, p += rb;
+    w.row_gate = (float*)p, p += rb;
+    w.chunk_hist = (uint32_t*)p, p += ws_up((size_t)w.max_chunks * max_e * 4u);
+    w.ftab = (uint64_t*)p;
+    return w;
+}
 
 struct PlowMoeCtx {
     int device;
     int min_rows[2]; /* [0] prefill, [1] decode; < 0 unset */
     char err[256];
-    /* which form of the block-fp8 x fp8 kernels serves ops 85 / 86: 0 weight-streaming (few rows per
-     * expert), 1 tiled (many). Decided at the GLU from its row pitch (op 86 carries no row count and
-     * follows the GLU before it on this context); the segment entry points set it from their variant;
-     * PLOW_MOE_W8A8_KERNEL=stream|tiled forces it. */
-    int tiled;
-    /* slots per expert of the last align (op 84) on this context: ops 81 / 82 carry no row count and
-     * pick their kernel form from it (0 = unknown: streaming form) */
-    uint32_t rows_hint;
-    uint32_t slots_hint; /* T * k of the last align (op 84) on this context, 0 = unknown */
-    int forced; /* -1 none, 0 stream, 1 tiled (segment entry point or environment) */
-    int32_t* ws_meta;        /* [3 * WS_MAX_E + 1] */
-    uint32_t* ws_row_token;  /* [WS_MAX_ROWS] */
-    uint32_t* ws_row_partidx;
-    float* ws_row_gate;
-    uint32_t* ws_chunk_hist; /* [WS_MAX_CHUNKS][n_exp] scratch of the multi-workgroup align */
-    uint64_t* ws_ftab;       /* [2][WS_MAX_E][3] pointer tables built for the flat-tensor ops (150 - 153) */
+    void* ws_base;   /* the context's own allocation behind `ws` (NULL when `ws` is borrowed) */
+    Workspace ws;
 };
 
 static int fail(PlowMoeCtx* c, int code, const char* fmt, ...) {
@@ -66,46 +83,34 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
     *out = nullptr;
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) return PLOW_MOE_EDEVICE;
-    hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return PLOW_MOE_EDEVICE;
-    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return PLOW_MOE_EUNSUPPORTED; /* CDNA4 only */
     PlowMoeCtx* c = new (std::nothrow) PlowMoeCtx();
     if (c) memset(c, 0, sizeof *c);
     if (!c) return PLOW_MOE_ENOMEM;
     c->device = device;
     c->min_rows[0] = c->min_rows[1] = -1;
     c->err[0] = 0;
-    c->forced = -1;
-    if (const char* k = getenv("PLOW_MOE_W8A8_KERNEL")) {
-        if (!strcmp(k, "stream")) c->forced = 0;
-        if (!strcmp(k, "tiled")) c->forced = 1;
+    const int src = plow_moe_device_setup(device); /* CU count, kernel attributes: once per device */
+    if (src) {
+        delete c;
+        return src;
     }
     int prev = 0;
     (void)hipGetDevice(&prev);
     (void)hipSetDevice(device);
-    const bool ok = hipMalloc(&c->ws_meta, (3u * WS_MAX_E + 1u) * 4u) == hipSuccess &&
-                    hipMalloc(&c->ws_row_token, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
-                    hipMalloc(&c->ws_row_partidx, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
-                    hipMalloc(&c->ws_row_gate, (size_t)WS_MAX_ROWS * 4u) == hipSuccess &&
-                    hipMalloc(&c->ws_chunk_hist, (size_t)WS_MAX_CHUNKS * WS_MAX_E * 4u) == hipSuccess &&
-                    hipMalloc(&c->ws_ftab, (size_t)2u * WS_MAX_E * 3u * 8u) == hipSuccess;
+    const bool ok = hipMalloc(&c->ws_base, ws_bytes(WS_MAX_E, WS_MAX_SLOTS)) == hipSuccess;
     (void)hipSetDevice(prev);
     if (!ok) {
         plow_moe_destroy(c);
         return PLOW_MOE_ENOMEM;
     }
+    c->ws = ws_carve(c->ws_base, WS_MAX_E, WS_MAX_SLOTS);
     *out = c;
     return 0;
 }
 
 extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) {
     if (!ctx) return;
-    (void)hipFree(ctx->ws_meta);
-    (void)hipFree(ctx->ws_row_token);
-    (void)hipFree(ctx->ws_row_partidx);
-    (void)hipFree(ctx->ws_row_gate);
-    (void)hipFree(ctx->ws_chunk_hist);
-    (void)hipFree(ctx->ws_ftab);
+    (void)hipFree(ctx->ws_base);
     delete ctx;
 }
 
@@ -122,7 +127,35 @@ extern "C" int plow_moe_set_min_rows(PlowMoeCtx* ctx, int variant, int min_rows)
 #define NEED(c, cond, ...) \
     do { if (!(cond)) return fail(c, PLOW_MOE_EINVAL, __VA_ARGS__); } while (0)
 
-static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStream_t st, bool launch) {
+/* What a call knows about the batch beyond the descriptor in hand. Nothing of it outlives the call: the
+ * kernel form of an op never depends on what ran on the context before.
+ *   form   0 / 1: the segment entry points' variant (decode: weight-streaming kernels, prefill: tiled
+ *          kernels), -1: decide per op from its row count
+ *   slots  routed slots (T * k) of the align op of the same run, 0 = the run has none */
+struct Hint {
+    int form;
+    uint32_t slots;
+};
+
+/* Routed slots of the batch as far as this op can know them: the descriptor's own statement (fj[2].u,
+ * an extension of this library: no MoE op of the reference uses the third immediate), else the align op
+ * of the same run, else what the op's own operands imply (`own`, 0 = nothing). */
+static uint32_t slots_of(const PlowDevInst* in, const Hint& h, uint32_t own) {
+    if (in->fj[2].u) return in->fj[2].u;
+    if (h.slots) return h.slots;
+    return own;
+}
+
+/* Tiled or weight-streaming form of the fp8 x fp8 grouped GEMMs: the tiled one from 16 rows per expert on
+ * average (the measured crossover), when it serves the shape; unknown row counts take the streaming form,
+ * which is right at every size and fast at small ones. */
+static bool want_tiled(const Hint& h, uint32_t slots, const GroupW8A8& g) {
+    const int env = plow_moe_tuning().w8a8_kernel;
+    const bool tiled = env >= 0 ? env == 1 : h.form >= 0 ? h.form == 1 : slots >= 16u * g.E;
+    return tiled && group_w8a8_tiled_serves(g);
+}
+
+static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStream_t st, bool launch, const Hint& h) {
     const uint32_t* i = in->i;
     switch (in->op) {
     case PLOW_DOP_GEMM_F32: {
@@ -157,11 +190,9 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, i[1] >= 1u && i[1] <= 1056u && i[2] >= 1u, "op 84: n_exp %u outside 1..1056 or k = 0", i[1]);
         NEED(c, (uint64_t)i[0] * i[2] < (1ull << 31), "op 84: T * k overflows");
         if (!launch) return 0;
-        c->rows_hint = (uint32_t)(((uint64_t)i[0] * i[2]) / i[1]);
-        c->slots_hint = i[0] * i[2];
         return launch_align((int32_t*)ten(in, T, 0), ten(in, T, 1), (uint32_t*)ten(in, T, 2),
                             (uint32_t*)ten(in, T, 3), (float*)ten(in, T, 4), i[0], i[1], i[2],
-                            c->ws_chunk_hist, WS_MAX_CHUNKS, st);
+                            c->ws.chunk_hist, c->ws.max_chunks, st);
     }
     case PLOW_DOP_MOE_COMBINE:
     case PLOW_DOP_MOE_COMBINE_PF: {
@@ -220,11 +251,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.N = I; g.K = H; g.E = E; g.pitch = Tn; g.T = Tn;
         /* SiLU, or the clamped SwiGLU when a limit is given (plow runtime/amd/op_gemm_common.h:1973-1981) */
         g.f1 = in->fj[1].f; g.act = g.f1 > 0.0f ? PLOW_MOE_ACT_SWIGLU_CLAMP : PLOW_MOE_ACT_SILU;
-        /* many rows per expert (16 or more on average at the last align): tiled form, which leaves the
-         * rows of an expert without weights unwritten where the streaming form zeroes them (op 190 skips
-         * such an expert either way) */
-        c->tiled = (c->forced >= 0 ? c->forced : (c->rows_hint >= 16u ? 1 : 0)) && H >= 256u && I >= 256u;
-        return c->tiled ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
+        /* without a stated slot count: eight slots per token */
+        return want_tiled(h, slots_of(in, h, 8u * Tn), g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
     }
     case PLOW_DOP_MOE_QUANT_FP8_BLOCK128: {
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5),
@@ -250,8 +278,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 5);
         g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
         g.N = H; g.K = I; g.E = E;
-        const int tiled = (c->forced >= 0 ? c->forced : c->tiled) && g.K >= 256u && g.N >= 256u;
-        return tiled ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
+        return want_tiled(h, slots_of(in, h, Tn * topk), g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_PF: {
         const uint32_t I = i[0], H = i[1], E = i[2], enc = i[3], arm = i[7];
@@ -271,10 +298,9 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.pitch = i[4]; g.act = i[5];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
-            /* many rows per expert (row pitch >= 2 rows per expert per routed slot): tiled form */
-            c->tiled = c->forced >= 0 ? c->forced : (i[4] >= 2u * E ? 1 : 0);
-            if (H < 256u || I < 256u) c->tiled = 0; /* the tiled form needs two 128-k blocks in both GEMMs */
-            return c->tiled ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
+            /* without a stated slot count: the row pitch of the activation scales as the token count,
+             * eight slots per token */
+            return want_tiled(h, slots_of(in, h, 8u * i[4]), g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
         }
         if (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ) {
             NEED(c, ten(in, T, 3) && ten(in, T, 7), "op 85 W8A8 (bf16 rows): t3 stab, t7 fs must be bound");
@@ -288,9 +314,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.act = i[5];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
-            /* the streaming form serves this arm at every row count; the DOWN that follows reads plain
-             * fq / fs rows and takes the tiled form when the last align saw 16 or more rows per expert */
-            c->tiled = (c->forced >= 0 ? c->forced : (c->rows_hint >= 16u ? 1 : 0)) && H >= 256u && I >= 256u;
+            /* the streaming form serves this arm at every row count */
             return launch_group_glu_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
@@ -309,7 +333,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.N = I; g.K = H; g.E = E; g.enc = enc; g.act = i[5];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
             g.wcols = 3; g.wsel0 = 0; g.wsel1 = 1;
-            g.slots_hint = c->slots_hint;
+            g.slots_hint = slots_of(in, h, 0u);
             return launch_group_glu_a16(g, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85: encoding %u arm %u is not served", enc, arm);
@@ -330,8 +354,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4);
             g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_W8A8_P16;
-            const int tiled = (c->forced >= 0 ? c->forced : c->tiled) && g.K >= 256u && g.N >= 256u;
-            return tiled ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
+            return want_tiled(h, slots_of(in, h, 0u), g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
                          (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
@@ -348,7 +371,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.o_idx = (const uint32_t*)ten(in, T, 6); g.gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.enc = enc;
             g.wcols = 3; g.wsel0 = 2; g.wsel1 = 2;
-            g.slots_hint = c->slots_hint;
+            g.slots_hint = slots_of(in, h, 0u);
             return launch_group_down_a16(g, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 86: encoding %u arm %u is not served", enc, arm);
@@ -365,9 +388,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 6);
         g.meta = (const int32_t*)ten(in, T, 3); g.row_token = (const uint32_t*)ten(in, T, 4);
         g.N = I; g.K = H; g.E = E; g.act = i[5]; g.per_channel = 1;
-        /* many rows per expert (16 or more on average): tiled form, as for the block-fp8 pair */
-        c->tiled = (c->forced >= 0 ? c->forced : (c->rows_hint >= 16u ? 1 : 0)) && H >= 256u && I >= 256u;
-        return c->tiled ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
+        return want_tiled(h, slots_of(in, h, 0u), g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
     }
     case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8: {
         const uint32_t H = i[0], I = i[1], E = i[2];
@@ -381,8 +402,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 3);
         g.row_partidx = (const uint32_t*)ten(in, T, 4); g.row_gate = (const float*)ten(in, T, 5);
         g.N = H; g.K = I; g.E = E; g.per_channel = 1;
-        const int tiled = (c->forced >= 0 ? c->forced : c->tiled) && g.K >= 256u && g.N >= 256u;
-        return tiled ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
+        return want_tiled(h, slots_of(in, h, 0u), g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_FP8_BLK:
     case PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8:
@@ -405,28 +425,28 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, !pc || i[4] == 0u, "op %u: a non-zero slot offset (i4) is not served", (unsigned)in->op);
         NEED(c, (enc == PLOW_MOE_ENC_BF16 || ten(in, T, 4)), "op %u: scale table t4 must be bound for encoding %u", (unsigned)in->op, enc);
         NEED(c, nslot && kx && N && K && E && N % 128u == 0u && K % 128u == 0u, "op %u: N %u and K %u must be non-zero multiples of 128", (unsigned)in->op, N, K);
-        NEED(c, E <= WS_MAX_E && nslot <= WS_MAX_SLOTS, "op %u: %u slots / %u experts exceed the context workspace", (unsigned)in->op, nslot, E);
+        NEED(c, E <= c->ws.max_e && nslot <= c->ws.max_slots, "op %u: %u slots / %u experts exceed the workspace (%u slots, %u experts)", (unsigned)in->op, nslot, E, c->ws.max_slots, c->ws.max_e);
         NEED(c, act <= 1u, "op %u: activation %u is not served", (unsigned)in->op, act);
         if (!launch) return 0;
         /* align with k = slots per input row: row_token = slot / kx, row_partidx = slot */
-        int rc = launch_align(c->ws_meta, ten(in, T, 2), c->ws_row_token, c->ws_row_partidx, c->ws_row_gate,
-                              (nslot + kx - 1u) / kx, E, kx, c->ws_chunk_hist, WS_MAX_CHUNKS, st);
+        int rc = launch_align(c->ws.meta, ten(in, T, 2), c->ws.row_token, c->ws.row_partidx, c->ws.row_gate,
+                              (nslot + kx - 1u) / kx, E, kx, c->ws.chunk_hist, c->ws.max_chunks, st);
         if (rc) return rc;
         GroupA16 g = {};
         g.out = ten(in, T, 0); g.a = ten(in, T, 1);
         g.wtab = (const uint64_t*)ten(in, T, 3);
         g.stab = enc == PLOW_MOE_ENC_BF16 ? nullptr : (const uint64_t*)ten(in, T, 4);
-        g.meta = c->ws_meta;
+        g.meta = c->ws.meta;
         g.N = N; g.K = K; g.E = E; g.enc = enc; g.act = act;
         g.wcols = pc ? 2u : 3u;
         g.slots_hint = nslot;
-        g.o_idx = c->ws_row_partidx;
+        g.o_idx = c->ws.row_partidx;
         if (glu) {
-            g.a_idx = c->ws_row_token;
+            g.a_idx = c->ws.row_token;
             g.wsel0 = 0; g.wsel1 = pc ? 0u : 1u; g.wrow1 = pc ? N : 0u;
             return launch_group_glu_a16(g, st);
         }
-        g.a_idx = c->ws_row_partidx; g.gate = c->ws_row_gate;
+        g.a_idx = c->ws.row_partidx; g.gate = c->ws.row_gate;
         g.wsel0 = g.wsel1 = pc ? 1u : 2u;
         rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), g.wtab, g.stab, g.wcols, g.wsel0, nslot, E, N, st);
         if (rc) return rc;
@@ -449,7 +469,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.wtab = (const uint64_t*)ten(in, T, 2); g.wcols = 2;
         g.meta = (const int32_t*)ten(in, T, 3);
         g.N = N; g.K = K; g.E = E; g.enc = PLOW_MOE_ENC_BF16; g.act = glu ? i[5] : 0u;
-        g.slots_hint = c->slots_hint;
+        g.slots_hint = slots_of(in, h, 0u);
         if (glu) {
             g.a_idx = (const uint32_t*)ten(in, T, 4);
             g.wsel0 = g.wsel1 = 0; g.wrow1 = N;
@@ -481,13 +501,13 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, pf ? ten(in, T, 4) != nullptr : ten(in, T, 2) != nullptr, "op %u: %s must be bound", (unsigned)in->op, pf ? "t4 meta" : "t2 table");
         NEED(c, !pf || (glu ? ten(in, T, 5) != nullptr : (ten(in, T, 6) && ten(in, T, 7))), "op %u: the row maps must be bound", (unsigned)in->op);
         NEED(c, N && K && E && N % 128u == 0u && K % 128u == 0u, "op %u: N %u and K %u must be non-zero multiples of 128", (unsigned)in->op, N, K);
-        NEED(c, E <= WS_MAX_E && nslot <= WS_MAX_SLOTS && (pf || nslot), "op %u: %u slots / %u experts exceed the context workspace", (unsigned)in->op, nslot, E);
+        NEED(c, E <= c->ws.max_e && nslot <= c->ws.max_slots && (pf || nslot), "op %u: %u slots / %u experts exceed the workspace (%u slots, %u experts)", (unsigned)in->op, nslot, E, c->ws.max_slots, c->ws.max_e);
         NEED(c, layout <= 1u, "op %u: layout %u is neither interleaved (0) nor blocked (1)", (unsigned)in->op, layout);
         if (act > PLOW_MOE_ACT_SWIGLU_OAI) return fail(c, PLOW_MOE_EUNSUPPORTED, "op %u: activation %u is not served", (unsigned)in->op, act);
         if (!launch) return 0;
         const uint32_t rows = glu ? 2u * N : N; /* weight rows per expert */
-        uint64_t* wtab = c->ws_ftab;
-        uint64_t* stab = c->ws_ftab + (size_t)WS_MAX_E * 3u;
+        uint64_t* wtab = c->ws.ftab;
+        uint64_t* stab = c->ws.ftab + (size_t)c->ws.max_e * 3u;
         int rc = launch_flat_tables(wtab, stab, W, S, E, (size_t)rows * (K / 2u), (size_t)rows * (K / 32u), st);
         if (rc) return rc;
         GroupA16 g = {};
@@ -499,18 +519,18 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         if (glu) { g.wmul = layout ? 1u : 2u; g.wrow0 = 0; g.wrow1 = layout ? N : 1u; }
         if (pf) {
             g.meta = (const int32_t*)ten(in, T, 4);
-            g.slots_hint = c->slots_hint;
+            g.slots_hint = slots_of(in, h, 0u);
             if (glu) { g.a_idx = (const uint32_t*)ten(in, T, 5); return launch_group_glu_a16(g, st); }
             g.o_idx = (const uint32_t*)ten(in, T, 6); g.gate = (const float*)ten(in, T, 7);
             return launch_group_down_a16(g, st);
         }
         /* slot-major: sort the slots by expert into the context workspace (row_token = slot / k) */
-        rc = launch_align(c->ws_meta, ten(in, T, 2), c->ws_row_token, c->ws_row_partidx, c->ws_row_gate,
-                          nslot / kx, E, kx, c->ws_chunk_hist, WS_MAX_CHUNKS, st);
+        rc = launch_align(c->ws.meta, ten(in, T, 2), c->ws.row_token, c->ws.row_partidx, c->ws.row_gate,
+                          nslot / kx, E, kx, c->ws.chunk_hist, c->ws.max_chunks, st);
         if (rc) return rc;
-        g.meta = c->ws_meta; g.slots_hint = nslot; g.o_idx = c->ws_row_partidx;
-        if (glu) { g.a_idx = c->ws_row_token; return launch_group_glu_a16(g, st); }
-        g.a_idx = c->ws_row_partidx; g.gate = c->ws_row_gate;
+        g.meta = c->ws.meta; g.slots_hint = nslot; g.o_idx = c->ws.row_partidx;
+        if (glu) { g.a_idx = c->ws.row_token; return launch_group_glu_a16(g, st); }
+        g.a_idx = c->ws.row_partidx; g.gate = c->ws.row_gate;
         rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), wtab, stab, 3u, 0u, nslot, E, N, st);
         if (rc) return rc;
         return launch_group_down_a16(g, st);
@@ -550,31 +570,48 @@ static int finish(PlowMoeCtx* c, int rc, const PlowDevInst* in) {
     return 0;
 }
 
+/* the align op of a run states its routed slots (T * k) for the ops that follow it in the same run */
+static Hint hint_of_run(const PlowDevInst* insts, uint32_t n_inst, int form) {
+    Hint h = {form, 0u};
+    for (uint32_t n = 0; n < n_inst; n++)
+        if (insts[n].op == PLOW_DOP_MOE_ALIGN_PF) {
+            const uint64_t slots = (uint64_t)insts[n].i[0] * insts[n].i[2];
+            h.slots = slots < 0xFFFFFFFFull ? (uint32_t)slots : 0xFFFFFFFFu;
+        }
+    return h;
+}
+
+static int exec_run(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, void* const* tensors, void* stream,
+                    int form) {
+    const Hint h = hint_of_run(insts, n_inst, form);
+    for (uint32_t n = 0; n < n_inst; n++) { /* refuse the whole run before launching any of it */
+        const int rc = run_op(ctx, &insts[n], tensors, nullptr, false, h);
+        if (rc) return rc;
+    }
+    for (uint32_t n = 0; n < n_inst; n++) {
+        const int rc = finish(ctx, run_op(ctx, &insts[n], tensors, (hipStream_t)stream, true, h), &insts[n]);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
 extern "C" int plow_moe_check(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors) {
     if (!ctx || !inst || !tensors) return PLOW_MOE_EINVAL;
     ctx->err[0] = 0;
-    return run_op(ctx, inst, tensors, nullptr, false);
+    return run_op(ctx, inst, tensors, nullptr, false, Hint{-1, 0u});
 }
 
 extern "C" int plow_moe_exec(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors, void* stream) {
     if (!ctx || !inst || !tensors) return PLOW_MOE_EINVAL;
     ctx->err[0] = 0;
-    return finish(ctx, run_op(ctx, inst, tensors, (hipStream_t)stream, true), inst);
+    return finish(ctx, run_op(ctx, inst, tensors, (hipStream_t)stream, true, Hint{-1, 0u}), inst);
 }
 
 extern "C" int plow_moe_exec_many(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst,
                                   void* const* tensors, void* stream) {
     if (!ctx || !insts || !tensors) return PLOW_MOE_EINVAL;
     ctx->err[0] = 0;
-    for (uint32_t n = 0; n < n_inst; n++) { /* refuse the whole run before launching any of it */
-        const int rc = run_op(ctx, &insts[n], tensors, nullptr, false);
-        if (rc) return rc;
-    }
-    for (uint32_t n = 0; n < n_inst; n++) {
-        const int rc = finish(ctx, run_op(ctx, &insts[n], tensors, (hipStream_t)stream, true), &insts[n]);
-        if (rc) return rc;
-    }
-    return 0;
+    return exec_run(ctx, insts, n_inst, tensors, stream, -1);
 }
 
 /* ---- segment entry points ---------------------------------------------------------------------- */
@@ -627,11 +664,9 @@ static int run_segment(PlowMoeCtx* ctx, int variant, const PlowDevInst* insts, u
     if (mr == 0 || (mr > 0 && rows < (uint32_t)mr)) return PLOW_MOE_ROLLBACK;
     int rc = check_segment(ctx, insts, n_inst);
     if (rc) return rc;
-    const int saved = ctx->forced;
-    if (saved < 0) ctx->forced = variant == 0 ? 1 : 0; /* prefill: tiled form, decode: streaming form */
-    rc = plow_moe_exec_many(ctx, insts, n_inst, tensors, stream);
-    ctx->forced = saved;
-    return rc;
+    /* prefill: tiled kernels (the streaming ones where a shape is outside the tiled form's limits);
+     * decode: weight-streaming kernels */
+    return exec_run(ctx, insts, n_inst, tensors, stream, variant == 0 ? 1 : 0);
 }
 
 extern "C" int plow_moe_pf(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst,

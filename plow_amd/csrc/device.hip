@@ -1,0 +1,65 @@
+/* device.hip — process-wide state of the library: the environment knobs (read once) and the table of
+ * devices that have been set up. Host code only. */
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+#include "../../include/plow_moe.h"
+#include "tuning.h"
+
+const PlowMoeTuning& plow_moe_tuning() {
+    static PlowMoeTuning t;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        auto is = [](const char* name, const char* value) {
+            const char* e = getenv(name);
+            return e && !strcmp(e, value);
+        };
+        t.w8a8_kernel = is("PLOW_MOE_W8A8_KERNEL", "stream") ? 0 : is("PLOW_MOE_W8A8_KERNEL", "tiled") ? 1 : -1;
+        t.tile_waves4 = is("PLOW_MOE_W8A8_TILE_WAVES", "4");
+        const char* d = getenv("PLOW_MOE_SK_DEPTH");
+        t.sk_depth = d ? atoi(d) : 3;
+        if (t.sk_depth < 2 || t.sk_depth > 4) t.sk_depth = 3;
+        t.sk_glu_regs = is("PLOW_MOE_SK_GLU", "regs");
+        t.sk_down_regs = is("PLOW_MOE_SK_DOWN", "regs");
+        t.sk_narrow = getenv("PLOW_MOE_SK_NARROW") != nullptr;
+        t.a16_regs = is("PLOW_MOE_A16_KERNEL", "regs");
+        t.score_tile8 = is("PLOW_MOE_SCORE_KERNEL", "tile8");
+        t.score_valu = is("PLOW_MOE_SCORE_KERNEL", "valu");
+        const char* f = getenv("PLOW_MOE_SCORE_MFMA32_FROM");
+        t.score_mfma32_from = f ? strtoull(f, nullptr, 10) : 0ull;
+        t.router_fused = !is("PLOW_MOE_ROUTER_FUSED", "0");
+    });
+    return t;
+}
+
+#define MAX_DEVICES 64
+static std::mutex g_dev_mutex;
+static uint32_t g_n_cu[MAX_DEVICES]; /* 0 = not set up; written once under the mutex */
+
+int plow_moe_device_setup(int device) {
+    if (device < 0 || device >= MAX_DEVICES) return PLOW_MOE_EINVAL;
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    if (g_n_cu[device]) return 0;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return PLOW_MOE_EDEVICE;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return PLOW_MOE_EUNSUPPORTED; /* CDNA4 only */
+    int prev = 0;
+    if (hipGetDevice(&prev) != hipSuccess || hipSetDevice(device) != hipSuccess) return PLOW_MOE_EDEVICE;
+    int rc = plow_moe_route_setup();
+    if (!rc) rc = plow_moe_w8a8_setup();
+    if (!rc) rc = plow_moe_w8a8_tiled_setup();
+    if (!rc) rc = plow_moe_a16_setup();
+    (void)hipSetDevice(prev);
+    if (rc) return rc;
+    __atomic_store_n(&g_n_cu[device], (uint32_t)prop.multiProcessorCount, __ATOMIC_RELEASE);
+    return 0;
+}
+
+uint32_t plow_moe_n_cu() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 0u;
+    return __atomic_load_n(&g_n_cu[dev], __ATOMIC_ACQUIRE);
+}

@@ -30,6 +30,7 @@
  */
 #include "common.h"
 #include "kernels.h"
+#include "tuning.h"
 #include <string.h>
 
 #define AK_WAVES 8u
@@ -669,26 +670,9 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     a16_dma_body<ENC, GLU, RG>(g, dm_raw, blockIdx.x);
 }
 
-/* PLOW_MOE_A16_KERNEL=regs selects the first form */
-static bool a16_dma_form() {
-    static int v = -1;
-    if (v < 0) {
-        const char* e = getenv("PLOW_MOE_A16_KERNEL");
-        v = (e && !strcmp(e, "regs")) ? 0 : 1;
-    }
-    return v == 1;
-}
-
 template <int ENC, bool GLU, int RG>
 static int launch_a16_dma_rg(const GroupA16& g, dim3 grid, hipStream_t st) {
-    static bool attr_set = false;
     static_assert(sizeof(DmLds<ENC, RG>) <= 160u * 1024u, "the rings must fit the CU's LDS");
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)k_group_a16_dma<ENC, GLU, RG>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)sizeof(DmLds<ENC, RG>)) != hipSuccess)
-            return PLOW_MOE_EDEVICE;
-        attr_set = true;
-    }
     k_group_a16_dma<ENC, GLU, RG><<<grid, AK_THREADS, sizeof(DmLds<ENC, RG>), st>>>(g);
     return 0;
 }
@@ -708,20 +692,15 @@ static int launch_a16(const GroupA16& g, hipStream_t st) {
     const dim3 grid(g.E * (g.N / AK_BN));
     /* second form: needs whole steps of K (one 128-byte line per weight row) and the block scales of a
      * tile to fit its LDS table */
-    bool dma = a16_dma_form() && !g.bias && g.K <= 16384u &&
+    bool dma = !plow_moe_tuning().a16_regs && !g.bias && g.K <= 16384u &&
                g.K % (g.enc == AENC_MXFP4 ? 256u : 128u) == 0u && (g.enc == AENC_BF16 || g.stab);
     if (dma && g.slots_hint) {
         /* The second form fills a CU with one workgroup. With a short K loop and between one and three
          * workgroups per CU in all, the start-up chains of dependent loads (tables, row maps, first steps)
          * run one after the other on a CU, and the first form, four workgroups to a CU, hides them
          * better (mxfp4 DOWN at one token: 39 against 62 microseconds). */
-        static int n_cu = 0;
-        if (!n_cu) {
-            int dev = 0;
-            hipDeviceProp_t prop;
-            if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return PLOW_MOE_EDEVICE;
-            n_cu = prop.multiProcessorCount;
-        }
+        const uint32_t n_cu = plow_moe_n_cu();
+        if (!n_cu) return PLOW_MOE_EDEVICE;
         const uint64_t wgs = (uint64_t)(g.slots_hint < g.E ? g.slots_hint : g.E) * (g.N / AK_BN);
         const uint32_t steps = g.K / (g.enc == AENC_MXFP4 ? 256u : (g.enc == AENC_BF16 ? 64u : 128u));
         if (steps <= 16u && wgs > (uint64_t)n_cu && wgs < 3ull * (uint64_t)n_cu) dma = false;
@@ -746,6 +725,23 @@ static int launch_a16(const GroupA16& g, hipStream_t st) {
     default: return PLOW_MOE_EUNSUPPORTED;
     }
     return 0;
+}
+
+/* dynamic-LDS limits of every instance of the direct-to-LDS form, once per device (plow_moe_device_setup) */
+template <int ENC, bool GLU, int RG>
+static bool a16_set_attr() {
+    return hipFuncSetAttribute((const void*)k_group_a16_dma<ENC, GLU, RG>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)sizeof(DmLds<ENC, RG>)) == hipSuccess;
+}
+template <int ENC>
+static bool a16_set_attrs() {
+    constexpr int RGM = ENC == AENC_MXFP4 ? 2 : 4;
+    return a16_set_attr<ENC, true, 1>() && a16_set_attr<ENC, false, 1>() && a16_set_attr<ENC, true, RGM>() &&
+           a16_set_attr<ENC, false, RGM>();
+}
+int plow_moe_a16_setup() {
+    return a16_set_attrs<AENC_BF16>() && a16_set_attrs<AENC_FP8BLK>() && a16_set_attrs<AENC_MXFP4>() &&
+                   a16_set_attrs<AENC_FP8PC>() ? 0 : PLOW_MOE_EDEVICE;
 }
 
 int launch_group_glu_a16(const GroupA16& g, hipStream_t st) { return launch_a16<true>(g, st); }

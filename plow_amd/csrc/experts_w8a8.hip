@@ -21,6 +21,7 @@
  */
 #include "common.h"
 #include "kernels.h"
+#include "tuning.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -34,14 +35,8 @@
 
 
 __device__ __forceinline__ v4i ldg16(const uint8_t* p) { return *(const v4i*)p; }
-/* weight bytes are read exactly once per launch: stream them past the caches */
-__device__ __forceinline__ v4i ldg16_stream(const uint8_t* p) {
-#ifdef SK_NT_WEIGHTS
-    return __builtin_nontemporal_load((const v4i*)p);
-#else
-    return *(const v4i*)p;
-#endif
-}
+/* weight bytes (a non-temporal load measured no faster than a plain one here) */
+__device__ __forceinline__ v4i ldg16_stream(const uint8_t* p) { return *(const v4i*)p; }
 
 typedef short sk_bf16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void sk_atomic_add_bf16x2(bf16_t* p, float a, float b) {
@@ -583,25 +578,10 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     }
 }
 
-/* k-steps of weight loads a wave keeps in flight; PLOW_MOE_SK_DEPTH (2..4) overrides for tuning */
-static int stream_depth() {
-    static int d = 0;
-    if (!d) {
-        const char* e = getenv("PLOW_MOE_SK_DEPTH");
-        d = e ? atoi(e) : SK_DEPTH;
-        if (d < 2 || d > 4) d = SK_DEPTH;
-    }
-    return d;
-}
-
-/* PLOW_MOE_SK_GLU=regs selects the first form of the block-mode GLU (weights straight into registers) */
-static bool glu_dma_form() {
-    static int v = -1;
-    if (v < 0) {
-        const char* e = getenv("PLOW_MOE_SK_GLU");
-        v = (e && !strcmp(e, "regs")) ? 0 : 1;
-    }
-    return v == 1;
+/* dynamic-LDS limit of the direct-to-LDS form, once per device (plow_moe_device_setup) */
+int plow_moe_w8a8_setup() {
+    return hipFuncSetAttribute((const void*)k_group_glu_w8a8_dma, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)sizeof(SdLds)) == hipSuccess ? 0 : PLOW_MOE_EDEVICE;
 }
 
 static int check_w8a8(const GroupW8A8& g) {
@@ -616,7 +596,8 @@ int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<true, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
-    if (g.out_bf16 && !glu_dma_form()) { /* bf16 intermediate on the register form */
+    const PlowMoeTuning& tune = plow_moe_tuning();
+    if (g.out_bf16 && tune.sk_glu_regs) { /* bf16 intermediate on the register form */
         k_group_w8a8_stream<true, 3, false><<<grid, SK_THREADS, 0, st>>>(g);
         return 0;
     }
@@ -624,18 +605,11 @@ int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
         k_group_w8a8_stream<true, 3, false, false, true><<<grid, SK_THREADS, 0, st>>>(g);
         return 0;
     }
-    if (glu_dma_form()) {
-        static bool attr_set = false;
-        if (!attr_set) {
-            if (hipFuncSetAttribute((const void*)k_group_glu_w8a8_dma, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)sizeof(SdLds)) != hipSuccess)
-                return PLOW_MOE_EDEVICE;
-            attr_set = true;
-        }
+    if (!tune.sk_glu_regs) {
         k_group_glu_w8a8_dma<<<grid, SK_THREADS, sizeof(SdLds), st>>>(g);
         return 0;
     }
-    switch (stream_depth()) {
+    switch (plow_moe_tuning().sk_depth) {
     case 2: k_group_w8a8_stream<true, 2, false><<<grid, SK_THREADS, 0, st>>>(g); break;
     case 4: k_group_w8a8_stream<true, 4, false><<<grid, SK_THREADS, 0, st>>>(g); break;
     default: k_group_w8a8_stream<true, 3, false><<<grid, SK_THREADS, 0, st>>>(g); break;
@@ -648,16 +622,16 @@ int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<false, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
-    if (g.N % 256u == 0u && !getenv("PLOW_MOE_SK_NARROW")) {
+    if (g.N % 256u == 0u && !plow_moe_tuning().sk_narrow) {
         const dim3 wgrid(g.E * (g.N / 256u));
-        switch (stream_depth()) {
+        switch (plow_moe_tuning().sk_depth) {
         case 2: k_group_w8a8_stream<false, 2, false, true><<<wgrid, SK_THREADS, 0, st>>>(g); break;
         case 4: k_group_w8a8_stream<false, 4, false, true><<<wgrid, SK_THREADS, 0, st>>>(g); break;
         default: k_group_w8a8_stream<false, 3, false, true><<<wgrid, SK_THREADS, 0, st>>>(g); break;
         }
         return 0;
     }
-    switch (stream_depth()) {
+    switch (plow_moe_tuning().sk_depth) {
     case 2: k_group_w8a8_stream<false, 2, false><<<grid, SK_THREADS, 0, st>>>(g); break;
     case 4: k_group_w8a8_stream<false, 4, false><<<grid, SK_THREADS, 0, st>>>(g); break;
     default: k_group_w8a8_stream<false, 3, false><<<grid, SK_THREADS, 0, st>>>(g); break;

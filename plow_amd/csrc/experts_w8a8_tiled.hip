@@ -36,12 +36,16 @@
 #include <string.h>
 #include "common.h"
 #include "kernels.h"
+#include "tuning.h"
 
 /* SiLU(g) * u for the tile epilogue, where 128 x 128 of them per tile run on the waves that should be
  * multiplying: hardware exp2 and reciprocal (about 1 ulp each) instead of the library's expf and an
- * IEEE division, a third of the instructions. The result is rounded to fp8 (block mode) or bf16
- * (per-channel mode) right after, far above this error. Limits agree with g / (1 + expf(-g)):
- * g -> -inf gives -0, +inf gives +inf, NaN stays NaN. */
+ * IEEE division, a third of the instructions. The result is rounded to fp8 (block mode) or bf16 (op 188,
+ * per-channel mode) right after, far above this error: against the expf form over the same accumulators
+ * the bf16 result differs in about one element in 10^4, by one bf16 step (measured by the GPU test that
+ * runs op 188 on both forms). Limits: +inf gives +inf and NaN stays NaN as with g / (1 + expf(-g));
+ * g = -inf gives NaN here (-inf * rcp(inf)) where the library form gives -0, which only an accumulator
+ * that has already overflowed can reach. */
 __device__ __forceinline__ float t5_glu(float gt, float up, uint32_t act, float f0, float f1) {
     if (act == PLOW_MOE_ACT_SILU) {
         const float e = __builtin_amdgcn_exp2f(gt * -1.4426950408889634f);
@@ -116,12 +120,6 @@ __device__ __forceinline__ void ds_read_group(uint32_t live, uint32_t alo, uint3
 /* wait until at most n of this wave's loads are outstanding, then the workgroup barrier */
 #define LOADER_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory")
 
-#ifdef T5_PROF
-__device__ unsigned long long t5_prof[2][256][8];
-#define PROF_STAMP(v) const unsigned long long v = __builtin_readcyclecounter()
-#else
-#define PROF_STAMP(v)
-#endif
 
 /* ---- one 128-k block of a consumer wave (names are those of the kernel body) -------------------- */
 #define T5_BLOCK_HEAD()                                                                                      \
@@ -270,10 +268,17 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             __syncthreads();
         }
     }
-#ifdef T5_PROF
-    unsigned long long pf_setup = 0, pf_ramp = 0, pf_loop = 0, pf_epi = 0, pf_tiles = 0;
-    const unsigned long long pf_begin = __builtin_readcyclecounter();
-#endif
+    if (GLU && !PC && g.out_bf16) {
+        /* bf16 intermediate: the padded rows of an expert whose gate or up weights are not resident are
+         * zero-filled (the tile walk below skips such an expert), as in the streaming form */
+        for (uint32_t e = blockIdx.x; e < g.E; e += gridDim.x) {
+            if (g.wtab[(size_t)e * 3u] != 0ull && g.wtab[(size_t)e * 3u + 1u] != 0ull) continue;
+            const uint32_t cnt = (uint32_t)g.meta[g.E + e], r0 = (uint32_t)g.meta[e];
+            const uint32_t padded = ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
+            for (uint32_t i = tid; i < padded * (g.N / 4u); i += NTHR)
+                *(uint2*)((bf16_t*)g.out + (size_t)(r0 + i / (g.N / 4u)) * g.N + (i % (g.N / 4u)) * 4u) = make_uint2(0u, 0u);
+        }
+    }
     const uint32_t total = L.prefix[g.E - 1u] * NT;
     const uint32_t K = g.K, KB = K / 128u;
     const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]);
@@ -323,6 +328,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         t.rows = cnt - mt * T5_BM < T5_BM ? cnt - mt * T5_BM : T5_BM; /* live rows of the tile */
         /* block mode: {gate, up, down} tables; per-channel mode: {gate_up fused [2N][K], down} */
         t.wp0 = PC ? g.wtab[(size_t)t.e * 2u + (GLU ? 0u : 1u)] : g.wtab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
+        if (GLU && !PC && g.wtab[(size_t)t.e * 3u + 1u] == 0ull) t.wp0 = 0ull; /* gate without up: not resident */
         return t;
     };
     /* this workgroup's next tile at or after `from` whose expert is resident (`total` if none); loaders
@@ -445,9 +451,6 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             }
         };
         auto issue = [&](const Src& S, uint32_t kb, uint32_t st) {
-#ifdef T5_NOSTREAM
-            kb &= 1u;
-#endif
             __builtin_amdgcn_global_load_lds((const void*)(S.ssrc + (size_t)kb * S.sstep),
                                              (lds_void*)&L.as[st][(cw & 1u) * 64u], 4, 0, 0);
             const uint8_t* const ak = A0 + (size_t)kb * 128u;
@@ -508,7 +511,6 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         uint32_t par = 0, st = 0;
         const uint32_t cw0 = SUBS * cw;
         for (uint32_t tile = next_tile(wg, t); tile < total; tile = next_tile(tile + G, t), par ^= 1u) {
-            PROF_STAMP(ts0);
             const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
             const uint32_t ngrp = (rows + 15u) / 16u; /* live 16-row groups */
             /* DOWN: N may end mid-tile (N is a multiple of 128, so a wave's consumers are in or out together) */
@@ -521,19 +523,12 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 for (int rg = 0; rg < 8; rg++)
 #pragma unroll
                     for (int x = 0; x < 2; x++) accs[sub][rg][x] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-            PROF_STAMP(ts1);
-#ifdef T5_PROF
-            unsigned long long ts2 = 0;
-#endif
             /* Two forms of the block loop: tiles whose eight row groups are all live (the common case) run
              * code without a condition in it, which lets the scaled adds of a group be issued after the
              * matrix instructions of the next group; the other tiles skip their dead groups. */
             if (ngrp_w == 8u) {
                 for (uint32_t kb = 0; kb < KB; kb++) {
                     WG_BARRIER(); /* block kb is in LDS */
-#ifdef T5_PROF
-                    if (kb == 0) ts2 = __builtin_readcyclecounter();
-#endif
 #pragma unroll
                     for (uint32_t sub = 0; sub < SUBS; sub++) {
                         const uint32_t cw = cw0 + sub;
@@ -546,9 +541,6 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             } else {
                 for (uint32_t kb = 0; kb < KB; kb++) {
                     WG_BARRIER(); /* block kb is in LDS */
-#ifdef T5_PROF
-                    if (kb == 0) ts2 = __builtin_readcyclecounter();
-#endif
 #pragma unroll
                     for (uint32_t sub = 0; sub < SUBS; sub++) {
                         const uint32_t cw = cw0 + sub;
@@ -559,7 +551,6 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     LDS_WAIT_ALL();
                 }
             }
-            PROF_STAMP(ts3);
 
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
              *      group 0 and up in group 1; DOWN channel = ch0 + 16 * x + 4q + i ---- */
@@ -766,21 +757,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     }
                 }
             }
-#ifdef T5_PROF
-            {
-                const unsigned long long ts4 = __builtin_readcyclecounter();
-                pf_setup += ts1 - ts0, pf_ramp += ts2 - ts1, pf_loop += ts3 - ts2, pf_epi += ts4 - ts3, pf_tiles++;
-            }
-#endif
         }
     }
-#ifdef T5_PROF
-    if (tid == 0 && blockIdx.x < 256u) {
-        unsigned long long* o = t5_prof[GLU][blockIdx.x];
-        o[0] = pf_setup, o[1] = pf_ramp, o[2] = pf_loop, o[3] = pf_epi, o[4] = pf_tiles;
-        o[5] = __builtin_readcyclecounter() - pf_begin;
-    }
-#endif
 }
 template <bool GLU, bool PC, uint32_t NCW>
 __global__ __launch_bounds__((NCW + 4u) * 64u) void k_group_w8a8_tiled(GroupW8A8 g) {
@@ -788,50 +766,40 @@ __global__ __launch_bounds__((NCW + 4u) * 64u) void k_group_w8a8_tiled(GroupW8A8
     t5_body<GLU, PC, NCW>(g, lds_raw);
 }
 
-#ifdef T5_PROF
-extern "C" int plow_moe_debug_prof(unsigned long long* out) {
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(t5_prof), sizeof(t5_prof));
-}
-#endif
 
-/* PLOW_MOE_W8A8_TILE_WAVES=4 runs the 512-thread form (four consumer waves) instead of the 768-thread one */
-static bool tiled_four_consumers() {
-    static int v = -1;
-    if (v < 0) {
-        const char* e = getenv("PLOW_MOE_W8A8_TILE_WAVES");
-        v = (e && !strcmp(e, "4")) ? 1 : 0;
-    }
-    return v == 1;
+/* dynamic-LDS limits, once per device (plow_moe_device_setup) */
+template <bool GLU, bool PC, uint32_t NCW>
+static bool t5_set_attr() {
+    return hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU, PC, NCW>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)sizeof(T5Lds)) == hipSuccess;
+}
+int plow_moe_w8a8_tiled_setup() {
+    const bool ok = t5_set_attr<true, false, 8u>() && t5_set_attr<false, false, 8u>() && t5_set_attr<true, true, 8u>() &&
+                    t5_set_attr<false, true, 8u>() && t5_set_attr<true, false, 4u>() && t5_set_attr<false, false, 4u>() &&
+                    t5_set_attr<true, true, 4u>() && t5_set_attr<false, true, 4u>();
+    return ok ? 0 : PLOW_MOE_EDEVICE;
 }
 
 /* Persistent launch: one workgroup per CU; the tile count is computed on the device from meta. */
 template <bool GLU, bool PC, uint32_t NCW>
 static int launch_tiled_t(const GroupW8A8& g, hipStream_t st) {
-    static bool attr_set = false;
-    static int n_cu = 0;
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU, PC, NCW>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)sizeof(T5Lds)) != hipSuccess)
-            return PLOW_MOE_EDEVICE;
-        attr_set = true;
-    }
-    if (!n_cu) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return PLOW_MOE_EDEVICE;
-        n_cu = prop.multiProcessorCount;
-    }
-    k_group_w8a8_tiled<GLU, PC, NCW><<<(uint32_t)n_cu, (NCW + 4u) * 64u, sizeof(T5Lds), st>>>(g);
+    const uint32_t n_cu = plow_moe_n_cu();
+    if (!n_cu) return PLOW_MOE_EDEVICE;
+    k_group_w8a8_tiled<GLU, PC, NCW><<<n_cu, (NCW + 4u) * 64u, sizeof(T5Lds), st>>>(g);
     return 0;
 }
 
-/* Persistent launch: one workgroup per CU; the tile count is computed on the device from meta. */
+/* The shapes the tiled form serves: the tile keeps K / 128 block scales in LDS and the load ring runs
+ * two blocks ahead. Callers fall back to the streaming form otherwise. */
+bool group_w8a8_tiled_serves(const GroupW8A8& g) {
+    return g.N != 0u && g.E != 0u && g.E <= 1056u && g.N % 128u == 0u && g.K % 128u == 0u && g.K >= 256u &&
+           g.K <= 128u * 128u && g.N >= 256u;
+}
+
 template <bool GLU>
 static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
-    if (g.N == 0 || g.K == 0 || g.E == 0 || g.E > 1056u || g.N % 128u || g.K % 128u) return PLOW_MOE_EINVAL;
-    /* the tile keeps K / 128 block scales in LDS; the load ring runs two blocks ahead */
-    if (g.K > 128u * 128u || g.K < 256u) return PLOW_MOE_EINVAL;
-    if (tiled_four_consumers()) return g.per_channel ? launch_tiled_t<GLU, true, 4u>(g, st) : launch_tiled_t<GLU, false, 4u>(g, st);
+    if (!group_w8a8_tiled_serves(g)) return PLOW_MOE_EINVAL;
+    if (plow_moe_tuning().tile_waves4) return g.per_channel ? launch_tiled_t<GLU, true, 4u>(g, st) : launch_tiled_t<GLU, false, 4u>(g, st);
     return g.per_channel ? launch_tiled_t<GLU, true, 8u>(g, st) : launch_tiled_t<GLU, false, 8u>(g, st);
 }
 

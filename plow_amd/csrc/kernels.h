@@ -64,6 +64,8 @@ int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);
 /* the many-rows-per-expert form of the same two ops (block mode only) */
 int launch_group_glu_w8a8_tiled(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8_tiled(const GroupW8A8& g, hipStream_t st);
+/* whether the tiled form serves this shape (callers take the streaming form otherwise) */
+bool group_w8a8_tiled_serves(const GroupW8A8& g);
 
 
 /* Grouped experts with bf16 activations (see experts_a16.hip). */

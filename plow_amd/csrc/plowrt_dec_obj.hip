@@ -18,6 +18,8 @@
  * bound) and 86 (arm 2). Shapes the kernel cannot serve make it return without writing, as plow's own do
  * (runtime/amd/moe_w8a8_dec.hip:486-487). */
 #include "experts_w8a8.hip"
+#define DP_FN __device__ __forceinline__
+#include "dec_pair_protocol.h"
 
 extern "C" __device__ __attribute__((used)) unsigned plow_moe_w8a8_dec_abi_1 = 1;
 
@@ -62,18 +64,19 @@ __device__ __forceinline__ bool dec_down_ok(const DecDownArgs& a) {
            (unsigned long long)a.experts * (a.hidden / 256u) <= 0x7FFFFFFFull;
 }
 
-/* The pair kernel's counters: expert e owns the words ctr[4 * t] (GLU items done) and ctr[4 * t + 1]
- * (DOWN items done) with t = tilep[e], its first 64-row tile, which is unique among experts that have
- * rows and below the tile bound that sizes the scratch. A DOWN item waits until all N / 128 GLU items of
- * its expert are counted; the expert's last DOWN item zeroes both words. The wait is bounded
- * (DEC_SPIN_LIMIT polls, seconds): an item that gives up is skipped, so a broken dependency shows as
- * missing output, never as a kernel that does not return. */
-#define DEC_SPIN_LIMIT (1u << 21)
+/* The pair kernel's counters and its bounded wait: dec_pair_protocol.h. */
+__device__ __forceinline__ void dec_item_done(unsigned* mine, uint32_t glu_items, uint32_t down_items) {
+    const uint32_t before = __hip_atomic_fetch_add(mine + DP_ITEMS_DONE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (dp_is_last(before, glu_items, down_items)) { /* every other item of the expert has made its last access */
+        __hip_atomic_store(mine + DP_GLU_DONE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + DP_ITEMS_DONE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
 
 /* GLU work items first, first + stride, ...: (expert, 128 channels), heavy (folded shared) expert first */
 template <bool AQ, bool FUSED>
 __device__ __forceinline__ void dec_glu_items(const DecGluArgs& a, uint32_t first, uint32_t stride, float* s_red,
-                                              unsigned* ctr) {
+                                              unsigned* ctr, uint32_t down_items) {
     GroupW8A8 g = {};
     g.out = a.out; g.out_scale = a.out_scale; g.a = a.x; g.a_scale = a.x_scale;
     g.wtab = (const uint64_t*)a.wtab; g.stab = (const uint64_t*)a.stab; g.meta = a.meta; g.row_token = a.row_token;
@@ -89,8 +92,11 @@ __device__ __forceinline__ void dec_glu_items(const DecGluArgs& a, uint32_t firs
         if (FUSED) {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent"); /* this thread's fq / fs stores, device-wide */
             __syncthreads();
-            if (threadIdx.x == 0)
-                __hip_atomic_fetch_add(&ctr[4u * (uint32_t)g.meta[2u * g.E + e]], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (threadIdx.x == 0) {
+                unsigned* const mine = ctr + dp_expert_words((uint32_t)g.meta[2u * g.E + e]);
+                __hip_atomic_fetch_add(mine + DP_GLU_DONE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                dec_item_done(mine, tiles, down_items);
+            }
         }
     }
 }
@@ -98,7 +104,7 @@ __device__ __forceinline__ void dec_glu_items(const DecGluArgs& a, uint32_t firs
 /* DOWN work items: (expert, 256 channels) */
 template <bool FUSED>
 __device__ __forceinline__ void dec_down_items(const DecDownArgs& a, uint32_t first, uint32_t stride, float* s_red,
-                                               unsigned* ctr, uint32_t* s_go) {
+                                               unsigned* ctr, uint32_t* s_go, uint32_t spin_limit) {
     GroupW8A8 g = {};
     g.out = a.part; g.a = a.fu; g.a_scale = a.fu_scale;
     g.wtab = (const uint64_t*)a.wtab; g.stab = (const uint64_t*)a.stab; g.meta = a.meta;
@@ -111,42 +117,46 @@ __device__ __forceinline__ void dec_down_items(const DecDownArgs& a, uint32_t fi
         /* the GLU's own test: what it skipped is not counted and must not be waited for */
         if (cnt == 0u || g.wtab[(size_t)e * 3u] == 0ull) continue;
         bool go = g.wtab[(size_t)e * 3u + 2u] != 0ull;
-        unsigned* const mine = FUSED ? ctr + 4u * (uint32_t)g.meta[2u * g.E + e] : nullptr;
+        const uint32_t glu_items = g.K / SK_BN; /* GLU items of this expert */
+        unsigned* const mine = FUSED ? ctr + dp_expert_words((uint32_t)g.meta[2u * g.E + e]) : nullptr;
+        const uint32_t r0 = (uint32_t)g.meta[e];
         if (FUSED) {
             if (threadIdx.x == 0) {
-                const uint32_t need = g.K / SK_BN; /* GLU items of this expert */
                 uint32_t ok = 0u;
-                for (uint32_t spin = 0; spin < DEC_SPIN_LIMIT; spin++) {
-                    if (__hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= need) { ok = 1u; break; }
+                for (uint32_t spin = 0; spin < spin_limit; spin++) {
+                    if (dp_down_ready(__hip_atomic_load(mine + DP_GLU_DONE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), glu_items)) { ok = 1u; break; }
                     __builtin_amdgcn_s_sleep(32);
                 }
                 *s_go = ok;
             }
             __syncthreads();
-            go = go && *s_go != 0u;
+            const bool ready = *s_go != 0u;
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); /* every wave reads fq / fs fresh */
-        }
-        if (go) {
-            const uint32_t r0 = (uint32_t)g.meta[e];
-            for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, false, 3, false, true, 4u, false>(g, e, ct, r0, rb, cnt, s_red);
-        }
-        if (FUSED) {
-            __syncthreads(); /* s_go is free again; every wave is past its reads of fq / fs */
-            if (threadIdx.x == 0) {
-                const uint32_t done = __hip_atomic_fetch_add(mine + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (done == tiles - 1u) { /* the expert's other DOWN items are all past their wait */
-                    __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(mine + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (go && !ready) {
+                /* the wait gave up: the rows this item owns say so (NaN), they do not keep stale data */
+                const float poison = __builtin_nanf("");
+                for (uint32_t i = threadIdx.x; i < cnt * 64u; i += 256u) {
+                    const uint32_t pidx = g.row_partidx[r0 + i / 64u];
+                    if (pidx != PLOW_EXPERT_UNUSED)
+                        *(float4*)((float*)g.out + (size_t)pidx * g.N + ct * 256u + (i % 64u) * 4u) = make_float4(poison, poison, poison, poison);
                 }
             }
+            go = go && ready;
+        }
+        if (go)
+            for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, false, 3, false, true, 4u, false>(g, e, ct, r0, rb, cnt, s_red);
+        if (FUSED) {
+            __syncthreads(); /* s_go is free again; every wave is past its reads of fq / fs */
+            if (threadIdx.x == 0) dec_item_done(mine, glu_items, tiles);
         }
     }
 }
 
 template <bool FUSED>
-__device__ __forceinline__ void dec_glu(const DecGluArgs& a, uint32_t first, uint32_t stride, float* s_red, unsigned* ctr) {
-    if (a.x_scale) dec_glu_items<false, FUSED>(a, first, stride, s_red, ctr); /* e4m3 rows with their scales (arm 2) */
-    else dec_glu_items<true, FUSED>(a, first, stride, s_red, ctr);            /* bf16 rows (arm 6) */
+__device__ __forceinline__ void dec_glu(const DecGluArgs& a, uint32_t first, uint32_t stride, float* s_red, unsigned* ctr,
+                                        uint32_t down_items) {
+    if (a.x_scale) dec_glu_items<false, FUSED>(a, first, stride, s_red, ctr, down_items); /* e4m3 rows with their scales (arm 2) */
+    else dec_glu_items<true, FUSED>(a, first, stride, s_red, ctr, down_items);            /* bf16 rows (arm 6) */
 }
 
 extern "C" __global__ __launch_bounds__(256) void plow_moe_w8a8_dec_glu(
@@ -158,7 +168,7 @@ extern "C" __global__ __launch_bounds__(256) void plow_moe_w8a8_dec_glu(
     const DecGluArgs a = {out, x, wtab, stab, meta, row_token, x_scale, out_scale, inter, hidden, experts, act,
                           beta, lbeta, x_pitch, reserved};
     if (!dec_glu_ok(a)) return;
-    dec_glu<false>(a, blockIdx.x, gridDim.x, s_red, nullptr);
+    dec_glu<false>(a, blockIdx.x, gridDim.x, s_red, nullptr, 0u);
 }
 
 extern "C" __global__ __launch_bounds__(256) void plow_moe_w8a8_dec_down(
@@ -169,7 +179,7 @@ extern "C" __global__ __launch_bounds__(256) void plow_moe_w8a8_dec_down(
     __shared__ float s_red[SK_WAVES * 64u];
     const DecDownArgs a = {part, fu, wtab, stab, meta, row_partidx, row_gate, fu_scale, hidden, inter, experts, reserved};
     if (!dec_down_ok(a)) return;
-    dec_down_items<false>(a, blockIdx.x, gridDim.x, s_red, nullptr, nullptr);
+    dec_down_items<false>(a, blockIdx.x, gridDim.x, s_red, nullptr, nullptr, 0u);
 }
 
 /* Both grids in one launch: workgroups [0, grid_glu) walk the GLU items, the others the DOWN items, each
@@ -182,6 +192,7 @@ extern "C" __global__ __launch_bounds__(256) void plow_moe_w8a8_dec_pair(DecPair
     if (!dec_glu_ok(a.g) || !dec_down_ok(a.d) || a.d.inter != a.g.inter || a.d.experts != a.g.experts ||
         a.d.meta != a.g.meta || a.d.wtab != a.g.wtab || a.ctr == nullptr || ng == 0u || ng >= nb)
         return;
-    if (blockIdx.x < ng) dec_glu<true>(a.g, blockIdx.x, ng, s_red, a.ctr);
-    else dec_down_items<true>(a.d, blockIdx.x - ng, nb - ng, s_red, a.ctr, &s_go);
+    /* a.reserved: polls before a DOWN item gives up its wait (0 = the default, seconds) */
+    if (blockIdx.x < ng) dec_glu<true>(a.g, blockIdx.x, ng, s_red, a.ctr, a.d.hidden / 256u);
+    else dec_down_items<true>(a.d, blockIdx.x - ng, nb - ng, s_red, a.ctr, &s_go, dp_spin_limit(a.reserved));
 }

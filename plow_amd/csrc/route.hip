@@ -12,6 +12,7 @@
 #include "common.h"
 #include "kernels.h"
 #include "pm_expf.h"
+#include "tuning.h"
 
 /* ============================ op 180: router score ============================================= */
 /* logit[m][n] = sum_k bf(x[m][k]) * bf(w[n][k]) with ONE f32 accumulator per output walking k in
@@ -655,34 +656,19 @@ __global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(
     if (m < M && n < N) out[(size_t)m * N + n] = acc;
 }
 
-/* PLOW_MOE_SCORE_KERNEL=tile8 keeps the few-output score on the 8 x 8 tile kernel (for comparison) */
-static bool score_row_form() {
-    static int v = -1;
-    if (v < 0) {
-        const char* e = getenv("PLOW_MOE_SCORE_KERNEL");
-        v = (e && !strcmp(e, "tile8")) ? 0 : 1;
-    }
-    return v == 1;
-}
+#define RS16_LDS (4u * RSM_STAGES * (uint32_t)sizeof(Rs16Stage))
+#define RSM_LDS (4u * RSM_STAGES * (uint32_t)sizeof(RsmStage))
+#define RSR_LDS (RSR_WS_BYTES + 2u * 4u * RSR_KC * 2u)
 
-static bool score_mfma_form() {
-    static int v = -1;
-    if (v < 0) {
-        const char* e = getenv("PLOW_MOE_SCORE_KERNEL");
-        v = !(e && !strcmp(e, "valu"));
-    }
-    return v != 0;
-}
-
-/* PLOW_MOE_SCORE_MFMA32_FROM = number of outputs from which the 32 x 32 tiles are forced (0 / unset: the
- * rule in launch_router_score decides) */
-static uint64_t score_mfma32_from() {
-    static uint64_t v = ~0ull;
-    if (v == ~0ull) {
-        const char* e = getenv("PLOW_MOE_SCORE_MFMA32_FROM");
-        v = e ? strtoull(e, nullptr, 10) : 0ull;
-    }
-    return v;
+/* dynamic-LDS limits of the score kernels, once per device (plow_moe_device_setup) */
+int plow_moe_route_setup() {
+    const bool ok =
+        hipFuncSetAttribute((const void*)k_router_score_mfma16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RS16_LDS) == hipSuccess &&
+        hipFuncSetAttribute((const void*)k_router_score_mfma, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSM_LDS) == hipSuccess &&
+        hipFuncSetAttribute((const void*)k_router_score_row<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess &&
+        hipFuncSetAttribute((const void*)k_router_score_row<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess &&
+        hipFuncSetAttribute((const void*)k_router_score_row<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess;
+    return ok ? 0 : PLOW_MOE_EDEVICE;
 }
 
 int launch_router_score(float* out, const void* x, const void* w, uint32_t M, uint32_t N, uint32_t K,
@@ -691,54 +677,37 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
     /* 32 x 32 tiles (fewer operand bytes per output) when they fill the SIMDs evenly: a whole number of
      * tiles per SIMD, or at least four; otherwise, from 2^17 outputs, the 16 x 32 tiles */
     const uint64_t t32 = (uint64_t)((N + 31) / 32) * ((M + 31) / 32);
-    const uint64_t n_simd = 1024; /* 256 CUs x 4 */
-    const uint64_t outputs = (uint64_t)M * N, force32 = score_mfma32_from();
-    const bool mfma_ok = K % 64u == 0u && score_mfma_form();
+    const PlowMoeTuning& tune = plow_moe_tuning();
+    const uint64_t n_cu = plow_moe_n_cu();
+    if (!n_cu) return PLOW_MOE_EDEVICE;
+    const uint64_t n_simd = 4u * n_cu;
+    const uint64_t outputs = (uint64_t)M * N, force32 = tune.score_mfma32_from;
+    const bool mfma_ok = K % 64u == 0u && !tune.score_valu;
     const bool use32 = mfma_ok && outputs >= (1u << 18) && (force32 ? outputs >= force32 : (t32 % n_simd == 0u || t32 >= 4u * n_simd));
     const bool use16 = mfma_ok && !use32 && outputs >= (1u << 17);
     if (use16) {
-        static bool attr_set = false;
-        const uint32_t lds = 4u * RSM_STAGES * (uint32_t)sizeof(Rs16Stage);
-        if (!attr_set) {
-            if (hipFuncSetAttribute((const void*)k_router_score_mfma16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-                return PLOW_MOE_EDEVICE;
-            attr_set = true;
-        }
+        const uint32_t lds = RS16_LDS;
         const uint32_t waves = ((N + 16u * RS16_NB - 1u) / (16u * RS16_NB)) * ((M + 15u) / 16u);
         k_router_score_mfma16<<<(waves + 3u) / 4u, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else if (use32) {
-        static bool attr_set = false;
-        const uint32_t lds = 4u * RSM_STAGES * (uint32_t)sizeof(RsmStage);
-        if (!attr_set) {
-            if (hipFuncSetAttribute((const void*)k_router_score_mfma, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-                return PLOW_MOE_EDEVICE;
-            attr_set = true;
-        }
+        const uint32_t lds = RSM_LDS;
         const uint32_t g = ((N + 63) / 64) * ((M + 63) / 64);
         k_router_score_mfma<<<g, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else if ((uint64_t)M * N >= (1u << 19)) {
-        if ((uint64_t)((N + 63) / 64) * ((M + 63) / 64) < 512u) { /* fewer than two 64-row workgroups per CU */
+        if ((uint64_t)((N + 63) / 64) * ((M + 63) / 64) < 2u * n_cu) { /* fewer than two 64-row workgroups per CU */
             dim3 g((N + 63) / 64, (M + 31) / 32);
             k_router_score_tile<2><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
         } else {
             dim3 g((N + 63) / 64, (M + 63) / 64);
             k_router_score_tile<4><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
         }
-    } else if (score_row_form() && K % RSR_KC == 0u && (uint64_t)N * K * 2u < (1ull << 31) && (uint64_t)M * K * 2u < (1ull << 31) &&
+    } else if (!tune.score_tile8 && K % RSR_KC == 0u && (uint64_t)N * K * 2u < (1ull << 31) && (uint64_t)M * K * 2u < (1ull << 31) &&
                (M < 16u || (uint64_t)M * N <= 2048u)) {
         /* measured against the 8 x 8 tile kernel below: ahead with one or two tokens per workgroup (6 of
          * 38 us at 1 x 384 x 7168) and with four on small score matrices (16 x 64 x 2048: 17 against
          * 25 us); with four tokens on a large one the shared LDS tile is the limit and the two are level */
         /* tokens per workgroup: as many as keep the weight rows' re-reads (once per workgroup row) low */
-        static bool attr_set = false;
-        const uint32_t lds = RSR_WS_BYTES + 2u * 4u * RSR_KC * 2u;
-        if (!attr_set) {
-            if (hipFuncSetAttribute((const void*)k_router_score_row<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
-                hipFuncSetAttribute((const void*)k_router_score_row<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
-                hipFuncSetAttribute((const void*)k_router_score_row<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-                return PLOW_MOE_EDEVICE;
-            attr_set = true;
-        }
+        const uint32_t lds = RSR_LDS;
         const uint32_t nx = (N + 63) / 64;
         if (M >= 16u) k_router_score_row<4><<<dim3(nx, (M + 3u) / 4u), (4u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
         else if (M >= 4u) k_router_score_row<2><<<dim3(nx, (M + 1u) / 2u), (2u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);

@@ -1,0 +1,52 @@
+/* tuning.h — the registry of the library's environment knobs and the per-device facts its launchers
+ * use. Every knob is read exactly once per process (thread-safe), here; nothing else in the library
+ * calls getenv. Every knob only selects between kernels that compute the same results: they exist for
+ * A/B timing, and the defaults are what the measurements chose.
+ *
+ *   PLOW_MOE_W8A8_KERNEL      stream | tiled   force one form of the fp8 x fp8 grouped GEMMs
+ *                                              (default: chosen per op from its row count)
+ *   PLOW_MOE_W8A8_TILE_WAVES  4                512-thread form of the tiled kernel (default 768 threads)
+ *   PLOW_MOE_SK_DEPTH         2..4             k-steps of weight loads in flight, register form (default 3)
+ *   PLOW_MOE_SK_GLU           regs             block-mode decode GLU on the register form (default: direct-to-LDS form)
+ *   PLOW_MOE_SK_DOWN          regs             decode DOWN on the register form (default: direct-to-LDS form)
+ *   PLOW_MOE_SK_NARROW        (any)            decode DOWN register form with 128-channel workgroups (default 256)
+ *   PLOW_MOE_A16_KERNEL       regs             bf16-activation kernels on their register form (default: direct-to-LDS form)
+ *   PLOW_MOE_SCORE_KERNEL     tile8 | valu     router score: keep the 8 x 8 tile kernel for few outputs / keep
+ *                                              the vector-unit kernels at prefill sizes
+ *   PLOW_MOE_SCORE_MFMA32_FROM  n              number of outputs from which the 32 x 32 matrix-unit tiles are forced
+ *   PLOW_MOE_ROUTER_FUSED     0                keep score, top-k and align as separate launches at decode sizes
+ */
+#ifndef PLOW_MOE_TUNING_H
+#define PLOW_MOE_TUNING_H
+
+#include <stdint.h>
+
+struct PlowMoeTuning {
+    int w8a8_kernel;      /* -1 auto, 0 stream, 1 tiled */
+    bool tile_waves4;
+    int sk_depth;         /* 2..4 */
+    bool sk_glu_regs;
+    bool sk_down_regs;
+    bool sk_narrow;
+    bool a16_regs;
+    bool score_tile8;
+    bool score_valu;
+    uint64_t score_mfma32_from;
+    bool router_fused;
+};
+const PlowMoeTuning& plow_moe_tuning();
+
+/* Per-device set-up, done once per device by plow_moe_create with that device current: the CU count
+ * and the dynamic-LDS attribute of every kernel that needs more than the default. Returns 0 or a
+ * negative PLOW_MOE_E* code. Launchers read the CU count of the current device with plow_moe_n_cu()
+ * (0 if the device was never set up: the launchers then refuse). */
+int plow_moe_device_setup(int device);
+uint32_t plow_moe_n_cu();
+
+/* one per translation unit with kernels that use dynamic LDS beyond the default limit */
+int plow_moe_route_setup();
+int plow_moe_w8a8_setup();
+int plow_moe_w8a8_tiled_setup();
+int plow_moe_a16_setup();
+
+#endif

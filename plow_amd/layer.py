@@ -167,11 +167,11 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
             p._emit("quant_x", abi.inst(abi.OP_QUANT_FP8, t=[xq, x, ascale], i=[T, H]))
             p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_GEMMA_PF_W8A8,
                                     t=[fu, xq, ewt, meta, row_token, ascale, est],
-                                    i=[I, H, Ea, 0, 0, cfg.act]))
+                                    i=[I, H, Ea, 0, 0, cfg.act], slots=T * ka))
             p._emit("quant_fu", abi.inst(abi.OP_QUANT_FP8, t=[fu8, fu, fscale], i=[R, I]))
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_GEMMA_PF_W8A8,
                                      t=[part, fu8, ewt, meta, row_partidx, row_gate, est, fscale],
-                                     i=[H, I, Ea]))
+                                     i=[H, I, Ea], slots=T * ka))
         else:
             # per-channel fp8 weights with bf16 activations: the decode ops 65/66, table driven.
             fu = p._t("fu", "bf16", (T * ka, I), "scratch")
@@ -192,12 +192,12 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
             hs = p._t("hs", "f32", (I // 128, T * ka), "scratch")
             p._emit("quant_x", abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[xq, x, xs], i=[T, H]))
             p._emit("glu", abi.inst(abi.OP_MOE_GLU_FP8_BLOCK128, t=[fu, xq, xs, wtab, stab, meta, row_token],
-                                    i=[I, H, Ea, T], f=[0.0, cfg.act_f[1] if cfg.act == 4 else 0.0]))
+                                    i=[I, H, Ea, T], f=[0.0, cfg.act_f[1] if cfg.act == 4 else 0.0], slots=T * ka))
             p._emit("quant_fu", abi.inst(abi.OP_MOE_QUANT_FP8_BLOCK128, t=[hq, fu, hs, meta, row_partidx, out],
                                          i=[I, Ea, ka, T, H]))
             p._emit("down", abi.inst(abi.OP_MOE_DOWN_FP8_BLOCK128,
                                      t=[out, hq, hs, wtab, stab, meta, row_partidx, row_gate],
-                                     i=[I, H, Ea, ka, T]))
+                                     i=[I, H, Ea, ka, T], slots=T * ka))
             return p
         if enc == abi.ENC_FP8BLK and cfg.arm in ("w8a8", "w8a8q"):
             fq = p._t("fq", "u8", (R, I), "scratch")
@@ -205,26 +205,26 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
             if cfg.arm == "w8a8q":
                 p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
                                         t=[fq, x, wtab, stab, meta, row_token, None, fs],
-                                        i=[I, H, Ea, enc, 0, cfg.act, 0, abi.ARM_W8A8_XQ], f=cfg.act_f))
+                                        i=[I, H, Ea, enc, 0, cfg.act, 0, abi.ARM_W8A8_XQ], f=cfg.act_f, slots=T * ka))
             else:
                 xq = p._t("xq", "u8", (T, H), "scratch")
                 xs = p._t("xs", "f32", (H // 128, T), "scratch")
                 p._emit("quant_x", abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[xq, x, xs], i=[T, H, T]))
                 p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
                                         t=[fq, xq, wtab, stab, meta, row_token, xs, fs],
-                                        i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8], f=cfg.act_f))
+                                        i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8], f=cfg.act_f, slots=T * ka))
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
                                      t=[part, fq, wtab, stab, meta, fs, row_partidx, row_gate],
-                                     i=[H, I, Ea, enc, 0, 0, 0, abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8]))
+                                     i=[H, I, Ea, enc, 0, 0, 0, abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8], slots=T * ka))
         else:
             arm = abi.ARM_W4A16 if enc == abi.ENC_MXFP4 else abi.ARM_A16
             fu = p._t("fu", "bf16", (R, I), "scratch")
             p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
                                     t=[fu, x, wtab, stab, meta, row_token],
-                                    i=[I, H, Ea, enc, 0, cfg.act, 0, arm], f=cfg.act_f))
+                                    i=[I, H, Ea, enc, 0, cfg.act, 0, arm], f=cfg.act_f, slots=T * ka))
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
                                      t=[part, fu, wtab, stab, meta, None, row_partidx, row_gate],
-                                     i=[H, I, Ea, enc, 0, 0, 0, arm]))
+                                     i=[H, I, Ea, enc, 0, 0, 0, arm], slots=T * ka))
 
     shared = None
     if cfg.shared_mode == "dense":

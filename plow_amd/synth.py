@@ -147,11 +147,14 @@ def zipf_bias(E: int, s: float, device, seed: int, alpha: float = 0.01) -> torch
 
 
 def bind(plan: LayerPlan, device, seed: int = 0, x_std: float = 1.0, w_std: float = 0.02,
-         hot_expert: float = 0.0, experts_alias: int = 0, zipf: float = 0.0) -> Bound:
+         hot_expert: float = 0.0, experts_alias: int = 0, zipf: float = 0.0,
+         share: Optional[Bound] = None) -> Bound:
     """Allocate and fill every tensor of ``plan`` on ``device``.
 
     ``experts_alias`` > 0 generates only that many distinct expert weight sets and lets the pointer
     tables cycle through them (for memory-limited CPU tests; 0 = every expert distinct).
+    ``share``: a binding of the same layer (same seed, same expert geometry, any batch size) on the same
+    device whose router and expert weights and pointer tables are reused instead of generated again.
     """
     cfg: MoeConfig = plan.cfg
     b = Bound(plan, device)
@@ -160,7 +163,10 @@ def bind(plan: LayerPlan, device, seed: int = 0, x_std: float = 1.0, w_std: floa
         if sp.role in ("scratch", "out", "table"):
             b.alloc(name)
     b.t["x"] = randn_bf16((cfg.T, cfg.H), x_std, dev, seed * 1000 + 1)
-    b.t["Wr"] = randn_bf16((cfg.E, cfg.H), w_std, dev, seed * 1000 + 2)
+    if share is not None:
+        sc = share.plan.cfg
+        assert (sc.H, sc.E, sc.I, sc.enc, sc.E_all) == (cfg.H, cfg.E, cfg.I, cfg.enc, cfg.E_all) and share.device == dev
+    b.t["Wr"] = share.t["Wr"] if share is not None else randn_bf16((cfg.E, cfg.H), w_std, dev, seed * 1000 + 2)
     if cfg.bias:
         b.t["bias"] = (zipf_bias(cfg.E, zipf, dev, seed * 1000 + 3) if zipf
                        else skewed_bias(cfg.E, hot_expert, dev, seed * 1000 + 3) if hot_expert
@@ -174,6 +180,14 @@ def bind(plan: LayerPlan, device, seed: int = 0, x_std: float = 1.0, w_std: floa
         b.t["Ws_down"] = randn_bf16((cfg.H, Is), w_std, dev, seed * 1000 + 7)
 
     Ea = cfg.E_all
+    wname, sname = ("ewt", "est") if cfg.enc == "fp8pc" else ("wtab", "stab")
+    if share is not None:
+        b.experts = share.experts
+        b.t[wname] = share.t[wname]
+        if sname in plan.slots:
+            b.t[sname] = share.t[sname]
+        b._table = None
+        return b
     n_distinct = min(Ea, experts_alias) if experts_alias else Ea
     sets = []
     for e in range(n_distinct):
@@ -197,7 +211,6 @@ def bind(plan: LayerPlan, device, seed: int = 0, x_std: float = 1.0, w_std: floa
             raise ValueError(cfg.enc)
         del g, u, d
     b.experts = sets
-    wname, sname = ("ewt", "est") if cfg.enc == "fp8pc" else ("wtab", "stab")
     width = 2 if cfg.enc == "fp8pc" else 3
     wt = torch.zeros((Ea, width), dtype=torch.int64)
     st = torch.zeros((Ea, width), dtype=torch.int64)

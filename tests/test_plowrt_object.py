@@ -338,4 +338,31 @@ def test_decode_object_launched_like_plowrt(oracle, T, shrink):
         check(f"pair rep {rep}")
         assert int(ctr.abs().sum().item()) == 0
         wipe()
+
+    # A DOWN item whose bounded wait gives up: forced from the host with a poll limit of 1 (the pair block's
+    # `reserved` word) and a GLU share of one workgroup, so most DOWN items poll before their expert's GLU
+    # items are done. Every kernel still runs to its end. Each 256-channel block of each live slot row must
+    # then hold either the right values or NaN (the item said it could not compute), never what was there
+    # before; the scratch must come back zeroed; and a normal launch on that scratch must be exact again.
+    dev.t["fq"].fill_(0x55)
+    dev.t["fs"].fill_(7.0)
+    dev.t["part"].fill_(123.0)
+    torch.cuda.synchronize()
+    pa1 = DecPairArgs(ga, da, ctr.data_ptr(), 1, 1)
+    print(f"[launch] dec_pair grid=1+{grid_down} poll limit 1", flush=True)
+    m.launch("plow_moe_w8a8_dec_pair", pa1, 1 + grid_down, threads=256)
+    torch.cuda.synchronize()
+    assert int(ctr.abs().sum().item()) == 0
+    got = dev.t["part"].cpu().numpy().reshape(-1, cfg.H // 256, 256)
+    ref = want["part"].cpu().numpy().reshape(-1, cfg.H // 256, 256)
+    live_slots = host.np("table")["eid"] < Ea
+    blk_nan = np.isnan(got).all(axis=2)
+    blk_ok = (got.view(np.uint32) == ref.view(np.uint32)).all(axis=2)
+    assert (blk_nan | blk_ok)[live_slots].all(), "a block holds neither the result nor the poison"
+    print(f"[pair] {int(blk_nan[live_slots].sum())} of {int(live_slots.sum()) * (cfg.H // 256)} blocks poisoned, the rest exact", flush=True)
+    wipe()
+    m.launch("plow_moe_w8a8_dec_pair", pa, grid_glu + grid_down, threads=256)
+    torch.cuda.synchronize()
+    check("pair after a launch whose waits gave up")
+    assert int(ctr.abs().sum().item()) == 0
     moe.close()
