@@ -204,6 +204,21 @@ int plow_moe_dec(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, voi
  * returns PLOW_MOE_ROLLBACK; N > 0: segments with rows < N return PLOW_MOE_ROLLBACK. */
 int plow_moe_set_min_rows(PlowMoeCtx* ctx, int variant, int min_rows);
 
+/* plow_moe_exec for callers that cannot allocate. It has no counterpart in the reference: it is for code
+ * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc, where even creating a
+ * context (which allocates its workspace) is not possible. It takes no context and calls no allocating
+ * routine. Every op of plow_moe_exec is served; the ops that need a workspace (slot-major decode experts 48 /
+ * 49 / 65 / 66, flat mxfp4 150 - 153) take it from a static device array inside the library (1 MiB per GPU,
+ * held until the process ends), which limits them to PLOW_MOE_NOALLOC_MAX_SLOTS routed slots and
+ * PLOW_MOE_NOALLOC_MAX_EXPERTS experts: larger calls are refused with PLOW_MOE_EINVAL and a text in `err`
+ * (err may be NULL). The op runs on the CURRENT device. All calls on one GPU share that GPU's array: calls
+ * that overlap there (two streams, two threads) race; calls on one stream are safe. Nothing in the array
+ * has to start at zero and nothing is kept in it between calls. The first call on a device sets the device
+ * up (no stream work); inst == NULL does only that, e.g. before a capture begins. */
+#define PLOW_MOE_NOALLOC_MAX_SLOTS 4096u
+#define PLOW_MOE_NOALLOC_MAX_EXPERTS 1056u
+int plow_moe_exec_noalloc(const PlowDevInst* inst, void* const* tensors, void* stream, char* err, size_t err_len);
+
 /* Validate one descriptor against this library's contract without launching (0 = would run). */
 int plow_moe_check(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors);
 

@@ -18,7 +18,8 @@
 
 /* Slot-major ops (48 / 49 / 65 / 66, 150 / 151) are served by sorting their slots by expert into a
  * workspace first, so that every hit expert streams its weights once; the flat-tensor ops (150 - 153)
- * build their per-expert pointer tables there. A context owns one sized for WS_MAX_SLOTS slots. Nothing in a
+ * build their per-expert pointer tables there. A context owns one sized for WS_MAX_SLOTS slots;
+ * plow_moe_exec_noalloc carves a smaller one out of the library's static device array. Nothing in a
  * workspace has to start at zero: every word a kernel reads was written earlier in the same call. */
 #define WS_MAX_E 1056u
 #define WS_MAX_SLOTS (1u << 18)
@@ -39,6 +40,8 @@ static constexpr size_t ws_bytes(uint32_t max_e, uint32_t max_slots) {
     return ws_up((3u * (size_t)max_e + 1u) * 4u) + 3u * ws_up(ws_rows(max_e, max_slots) * 4u) +
            ws_up((size_t)((max_slots + 1023u) / 1024u) * max_e * 4u) + ws_up((size_t)2u * max_e * 3u * 8u);
 }
+static_assert(ws_bytes(PLOW_MOE_NOALLOC_MAX_EXPERTS, PLOW_MOE_NOALLOC_MAX_SLOTS) <= PLOW_MOE_STATIC_BYTES,
+              "the static device array must hold the workspace of the largest call plow_moe_exec_noalloc accepts");
 static Workspace ws_carve(void* base, uint32_t max_e, uint32_t max_slots) {
     Workspace w = {};
     char* p = (char*)base;
@@ -612,6 +615,39 @@ extern "C" int plow_moe_exec_many(PlowMoeCtx* ctx, const PlowDevInst* insts, uin
     if (!ctx || !insts || !tensors) return PLOW_MOE_EINVAL;
     ctx->err[0] = 0;
     return exec_run(ctx, insts, n_inst, tensors, stream, -1);
+}
+
+/* One op with no allocation anywhere on its path: no context (creating one allocates its workspace), the
+ * slot-major and flat-tensor ops take their workspace from the library's static device array instead.
+ * The first call on a device sets that device up (kernel attributes, the array's address there); inst ==
+ * NULL does only that. */
+extern "C" int plow_moe_exec_noalloc(const PlowDevInst* inst, void* const* tensors, void* stream, char* err,
+                                     size_t err_len) {
+    if (err && err_len) err[0] = 0;
+    auto say = [&](const char* text) {
+        if (err && err_len) snprintf(err, err_len, "%s", text);
+    };
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return PLOW_MOE_EDEVICE;
+    void* base = plow_moe_static_scratch();
+    if (!base) {
+        const int rc = plow_moe_device_setup(dev);
+        if (rc) {
+            say(rc == PLOW_MOE_EUNSUPPORTED ? "the current device is not gfx950" : "device set-up failed");
+            return rc;
+        }
+        base = plow_moe_static_scratch();
+        if (!base) return PLOW_MOE_EDEVICE;
+    }
+    if (!inst) return 0;
+    if (!tensors) return PLOW_MOE_EINVAL;
+    PlowMoeCtx c = {};
+    c.device = dev;
+    c.min_rows[0] = c.min_rows[1] = -1;
+    c.ws = ws_carve(base, PLOW_MOE_NOALLOC_MAX_EXPERTS, PLOW_MOE_NOALLOC_MAX_SLOTS); /* borrowed: ws_base stays NULL */
+    const int rc = finish(&c, run_op(&c, inst, tensors, (hipStream_t)stream, true, Hint{-1, 0u}), inst);
+    if (rc) say(c.err);
+    return rc;
 }
 
 /* ---- segment entry points ---------------------------------------------------------------------- */

@@ -35,9 +35,15 @@ const PlowMoeTuning& plow_moe_tuning() {
     return t;
 }
 
+/* Workspace of the entry point that allocates nothing (plow_moe_exec_noalloc). In host code this name
+ * is only a handle for hipGetSymbolAddress, never a device address: each GPU holds its own copy, whose
+ * address plow_moe_device_setup resolves once per device and keeps in g_scratch_ptr. */
+static __device__ __align__(256) unsigned char scratch[PLOW_MOE_STATIC_BYTES];
+
 #define MAX_DEVICES 64
 static std::mutex g_dev_mutex;
 static uint32_t g_n_cu[MAX_DEVICES]; /* 0 = not set up; written once under the mutex */
+static void* g_scratch_ptr[MAX_DEVICES];
 
 int plow_moe_device_setup(int device) {
     if (device < 0 || device >= MAX_DEVICES) return PLOW_MOE_EINVAL;
@@ -52,10 +58,20 @@ int plow_moe_device_setup(int device) {
     if (!rc) rc = plow_moe_w8a8_setup();
     if (!rc) rc = plow_moe_w8a8_tiled_setup();
     if (!rc) rc = plow_moe_a16_setup();
+    void* ptr = nullptr;
+    if (!rc && (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr)) rc = PLOW_MOE_EDEVICE;
     (void)hipSetDevice(prev);
     if (rc) return rc;
+    g_scratch_ptr[device] = ptr; /* this device's copy of the array */
     __atomic_store_n(&g_n_cu[device], (uint32_t)prop.multiProcessorCount, __ATOMIC_RELEASE);
     return 0;
+}
+
+void* plow_moe_static_scratch() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+    if (!__atomic_load_n(&g_n_cu[dev], __ATOMIC_ACQUIRE)) return nullptr; /* not set up */
+    return g_scratch_ptr[dev];
 }
 
 uint32_t plow_moe_n_cu() {

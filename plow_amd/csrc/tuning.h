@@ -43,6 +43,12 @@ const PlowMoeTuning& plow_moe_tuning();
 int plow_moe_device_setup(int device);
 uint32_t plow_moe_n_cu();
 
+/* The library's static device array: workspace of plow_moe_exec_noalloc, one copy per GPU at its own
+ * address, held from the moment the library's code is loaded on that GPU until the process ends. Its
+ * address on the current device (resolved by plow_moe_device_setup), or NULL. */
+#define PLOW_MOE_STATIC_BYTES (1u << 20)
+void* plow_moe_static_scratch();
+
 /* one per translation unit with kernels that use dynamic LDS beyond the default limit */
 int plow_moe_route_setup();
 int plow_moe_w8a8_setup();

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(HERE, "libplow_moe_gfx950.so")
 
 EXPORTS = ["plow_moe_abi", "plow_moe_create", "plow_moe_destroy", "plow_moe_last_error",
            "plow_moe_exec", "plow_moe_exec_many", "plow_moe_pf", "plow_moe_dec",
-           "plow_moe_set_min_rows", "plow_moe_check"]
+           "plow_moe_set_min_rows", "plow_moe_check", "plow_moe_exec_noalloc"]
 
 _lib = None
 
@@ -47,6 +47,8 @@ def load():
     for name in ("plow_moe_pf", "plow_moe_dec"):
         getattr(lib, name).argtypes = [C.c_void_p, I, C.c_uint32, P(C.c_void_p), C.c_uint32, C.c_void_p]
     lib.plow_moe_set_min_rows.argtypes = [C.c_void_p, C.c_int, C.c_int]
+    lib.plow_moe_exec_noalloc.argtypes = [I, P(C.c_void_p), C.c_void_p, C.c_char_p, C.c_size_t]
+    lib.plow_moe_exec_noalloc.restype = C.c_int
     _lib = lib
     return lib
 
