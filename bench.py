@@ -72,7 +72,9 @@ def make_cfg(layer, a, name, tokens):
         # from 128 tokens on, the decode ops (65 / 66 semantics, bf16 activations) below
         cfg.bias = True
         cfg.arm = "w8a8" if cfg.T >= 128 else "a16"
-    if a.arm:
+    if a.arm == "w8a8det":      # the deterministic fused down -> combine on the block-fp8 W8A8 arm
+        cfg.arm, cfg.det_combine = "w8a8", True
+    elif a.arm:
         cfg.arm = a.arm
     return cfg
 
@@ -219,7 +221,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="", help="one configuration only (c1..c6); default: c2 with c3 under prefill_4k")
     ap.add_argument("--tokens", type=int, default=0)
-    ap.add_argument("--arm", default="", help="override the configuration's arm (a16 | w8a8 | w8a8q | w8a8atomic)")
+    ap.add_argument("--arm", default="", help="override the configuration's arm (a16 | w8a8 | w8a8q | w8a8atomic | w8a8det)")
     ap.add_argument("--zipf", type=float, default=-1.0, help="override the expert popularity exponent")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib", action="store_true",

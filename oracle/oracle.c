@@ -186,6 +186,14 @@ static void op_router_topk(const PlowDevInst* in, uint32_t slice, uint32_t nblk,
     const size_t esz = (flags & PLOW_ROUTE_F32_LOGIT) ? 4u : 2u;
     float* score = malloc((size_t)n_exp * 4u);
     uint64_t* key = malloc((size_t)n_exp * 8u);
+    /* op 83 with t2 bound: the [T][i0] f64 accumulator of the deterministic fused combine is zeroed here
+     * (plow runtime/amd/op_moe.h:2329-2340, runtime/amd/interp.hip:6479-6483) */
+    double* det_acc = in->op == PLOW_DOP_MOE_ROUTER_TOPK_PF ? TEN(in, T, 2) : NULL;
+    if (det_acc) {
+        uint32_t lo, hi;
+        own_range(nt, slice, nblk, &lo, &hi);
+        for (size_t q = (size_t)lo * in->i[0]; q < (size_t)hi * in->i[0]; q++) det_acc[q] = 0.0;
+    }
     for (uint32_t tok = slice; tok < nt; tok += nblk) {
         PlowMoeRoute* row = table + (size_t)tok * (k + tail);
         route_one(row, logit + (size_t)tok * n_exp * esz, bias, n_exp, k, flags, in->fj[0].f,
@@ -251,10 +259,18 @@ static void op_combine(const PlowDevInst* in, uint32_t slice, uint32_t nblk, voi
     part += r0 * k * H * (part16 ? 2u : 4u);
     uint32_t lo, hi;
     own_range(nt * H, slice, nblk, &lo, &hi);
+    /* i4: `part` is the f64 [T][H] fixed-point accumulator op 86 summed in place (k == 1): one stream,
+     * scaled by 2^-32 on the way out (plow runtime/amd/op_moe.h:5510-5520) */
+    const int det = pf && in->i[4];
     for (uint32_t i = lo; i < hi; i++) {
         const uint32_t tok = i / H, h = i - tok * H;
         float acc = residual ? orc_bf2f(residual[i]) : 0.0f;
         if (shared) acc += orc_bf2f(shared[i]);
+        if (det) {
+            acc += (float)(((const double*)TEN(in, T, 3) + r0 * H)[i] * 2.3283064365386962890625e-10);
+            out[i] = orc_f2bf(acc);
+            continue;
+        }
         for (uint32_t j = 0; j < k; j++) {
             const size_t at = ((size_t)tok * k + j) * H + h;
             acc += part16 ? orc_bf2f(((const orc_bf16*)part)[at]) : ((const float*)part)[at];
@@ -533,6 +549,24 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
 
 /* 86: t0=part t1=fu_g|fq t2=wtab t3=stab t4=meta t5=fs t6=row_partidx t7=row_gate  i0=H i1=I i2=E
  * i3=enc i7=arm (2: f32 part, 3: bf16 part; enc 0/1 arm 0 and enc 2 arm 8: f32 part). */
+/* One contribution of the deterministic fused combine in the fixed-point domain and its order-independent
+ * add (plow runtime/amd/op_moe.h:2153-2163, :3855-3880): rint(clamp(v, +-2^17) * 2^32) is an integer below
+ * 2^49, sums of up to 16 of them are exact in f64, so the slices may add in any order (a compare-and-swap
+ * loop here; a device-scope f64 atomic on the GPU). */
+static double det_q(float v) { return rint((double)fminf(fmaxf(v, -131072.0f), 131072.0f) * 4294967296.0); }
+static void det_add(double* p, double q) {
+    uint64_t* u = (uint64_t*)p;
+    uint64_t old = __atomic_load_n(u, __ATOMIC_RELAXED);
+    for (;;) {
+        double d;
+        memcpy(&d, &old, 8);
+        d += q;
+        uint64_t nw;
+        memcpy(&nw, &d, 8);
+        if (__atomic_compare_exchange_n(u, &old, nw, 0, __ATOMIC_RELAXED, __ATOMIC_RELAXED)) return;
+    }
+}
+
 static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, void* const* T) {
     const uint64_t* wtab = TEN(in, T, 2);
     const uint64_t* stab = TEN(in, T, 3);
@@ -543,6 +577,8 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
     const int w8a8 = enc == PLOW_MOE_ENC_FP8BLK &&
                      (arm == PLOW_MOE_ARM_W8A8 || arm == PLOW_MOE_ARM_W8A8_P16);
     const int part16 = w8a8 && arm == PLOW_MOE_ARM_W8A8_P16;
+    /* i5: t0 is the f64 [T][H] accumulator of the deterministic fused combine; log2(k) + 1, or 256 + k */
+    const uint32_t det_k = !in->i[5] ? 0u : in->i[5] > 256u ? in->i[5] - 256u : 1u << (in->i[5] - 1u);
     const float* fs = TEN(in, T, 5);
     const uint32_t G = (H + 127u) / 128u, KB = (I + 127u) / 128u;
     float* wd = malloc((size_t)I * 4u);
@@ -579,7 +615,8 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
                                                        fs + (size_t)r * KB, 1u, I)
                                        : enc_dot(enc, wd, rs, a, I);
                 const float val = row_gate[r] * acc;
-                if (part16) ((orc_bf16*)TEN(in, T, 0))[(size_t)pidx * H + h] = orc_f2bf(val);
+                if (det_k) det_add((double*)TEN(in, T, 0) + (size_t)(pidx / det_k) * H + h, det_q(val));
+                else if (part16) ((orc_bf16*)TEN(in, T, 0))[(size_t)pidx * H + h] = orc_f2bf(val);
                 else ((float*)TEN(in, T, 0))[(size_t)pidx * H + h] = val;
             }
         }

@@ -183,7 +183,15 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
                         (uint64_t)i[7] * (E / i[6]) >= (k < 16u ? k : 16u),
                  "router top-k: group shape n_group=%u topk_group=%u is not selectable for n_exp=%u k=%u",
                  i[6], i[7], E, k);
+        /* op 83 with t2 bound: the [T][i0] f64 accumulator of the deterministic fused combine, zeroed here
+         * ahead of the chain that adds into it (plow runtime/amd/interp.hip:6479-6483) */
+        double* const det_acc = pf ? (double*)ten(in, T, 2) : nullptr;
+        NEED(c, !det_acc || (i[0] != 0u && (uintptr_t)det_acc % 16u == 0u), "op 83: the accumulator (t2) needs its width in i0 and 16-byte alignment");
         if (!launch) return 0;
+        if (det_acc) {
+            const int zrc = launch_zero_f64(det_acc, (size_t)rows * i[0], st);
+            if (zrc) return zrc;
+        }
         return launch_router_topk(ten(in, T, 0), ten(in, T, 1), (const float*)ten(in, T, 3), E, k, flags,
                                   rows, pf && i[5] ? 1u : 0u, i[6], i[7], in->fj[0].f, in->fj[1].f, st);
     }
@@ -205,9 +213,14 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         const uint32_t p16 = pf && i[7] ? 1u : 0u;
         NEED(c, ten(in, T, 0) && ten(in, T, 3), "combine: t0 out and t3 part must be bound");
         NEED(c, H && H % 4u == 0u, "combine: H %u must be a non-zero multiple of 4", H);
+        const bool det = pf && i[4] != 0u; /* part is the f64 [T][H] accumulator of the deterministic fused combine */
+        NEED(c, !det || (k == 1u && !p16), "op 87: the f64 accumulator form (i4) takes k = 1 and no bf16 partials");
         if (!launch) return 0;
         const char* res = (const char*)ten(in, T, 1);
         const char* sh = (const char*)ten(in, T, 2);
+        if (det)
+            return launch_combine_det((char*)ten(in, T, 0) + r0 * H * 2u, res ? res + r0 * H * 2u : nullptr,
+                                      sh ? sh + r0 * H * 2u : nullptr, (const double*)ten(in, T, 3) + r0 * H, H, rows, st);
         return launch_combine((char*)ten(in, T, 0) + r0 * H * 2u, res ? res + r0 * H * 2u : nullptr,
                               sh ? sh + r0 * H * 2u : nullptr,
                               (const char*)ten(in, T, 3) + r0 * k * H * (p16 ? 2u : 4u), H, k, rows, p16, st);
@@ -346,6 +359,16 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 4) && ten(in, T, 6) && ten(in, T, 7),
              "op 86: t0 part, t1 fu, t2 wtab, t4 meta, t6 row_partidx, t7 row_gate must be bound");
         NEED(c, I && H && E, "op 86: zero geometry");
+        /* i5: the deterministic fused combine. t0 is then the f64 [T][H] fixed-point accumulator (zeroed by
+         * op 83) and every live row adds into row slot / k of it. The reference's encoding is log2(k) + 1
+         * for a power-of-two k (plow runtime/amd/interp.hip:6596-6600); 256 + k states any k (an extension of
+         * this library: a folded shared expert makes k = 9). */
+        uint32_t det_k = 0u;
+        if (i[5]) {
+            NEED(c, i[5] <= 5u || (i[5] > 256u && i[5] <= 256u + 16u), "op 86: i5 = %u is neither log2(k) + 1 for k <= 16 nor 256 + k", i[5]);
+            det_k = i[5] > 256u ? i[5] - 256u : 1u << (i[5] - 1u);
+            NEED(c, enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8, "op 86: the deterministic fused combine (i5) is served on the block-fp8 W8A8 arm only");
+        }
         if (enc == PLOW_MOE_ENC_FP8BLK && (arm == PLOW_MOE_ARM_W8A8 || arm == PLOW_MOE_ARM_W8A8_P16)) {
             NEED(c, ten(in, T, 3) && ten(in, T, 5), "op 86 W8A8: t3 stab and t5 fs must be bound");
             NEED(c, I % 128u == 0u && H % 128u == 0u, "op 86 W8A8: I %u and H %u must be multiples of 128", I, H);
@@ -357,6 +380,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4);
             g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_W8A8_P16;
+            g.det_k = det_k;
             return want_tiled(h, slots_of(in, h, 0u), g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||

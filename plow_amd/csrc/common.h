@@ -76,6 +76,21 @@ __device__ __forceinline__ float moe_glu(float g, float u, uint32_t act, float f
     return __builtin_nanf("");
 }
 
+/* The order-independent form of the fused down -> combine (plow runtime/amd/op_moe.h:2110-2165): a
+ * contribution crosses into the [T][H] accumulator as the integer-valued double rint(clamp(v, +-2^17) *
+ * 2^32), added with a device-scope f64 atomic. Every partial sum of up to 16 such values is an integer
+ * below 2^53, so every addition is exact and the total does not depend on the order of arrival. A NaN
+ * clamps to -2^17 (fmaxf returns its other operand), as in the reference. */
+#define PLOW_DET_SCALE 4294967296.0
+#define PLOW_DET_UNSCALE 2.3283064365386962890625e-10
+#define PLOW_DET_CLAMP 131072.0f
+__device__ __forceinline__ double det_q(float v) {
+    return __builtin_rint((double)fminf(fmaxf(v, -PLOW_DET_CLAMP), PLOW_DET_CLAMP) * PLOW_DET_SCALE);
+}
+__device__ __forceinline__ void det_add(double* p, float v) {
+    (void)__builtin_amdgcn_global_atomic_fadd_f64((__attribute__((address_space(1))) double*)p, det_q(v));
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));

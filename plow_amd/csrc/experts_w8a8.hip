@@ -294,6 +294,15 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             const uint32_t pidx = g.row_partidx[rowidx[rt]];
             const float gate = g.row_gate[rowidx[rt]];
             const float y0 = gate * acc0[rt][0], y1 = gate * acc0[rt][1], y2 = gate * acc0[rt][2], y3 = gate * acc0[rt][3];
+            if (g.det_k) { /* order-independent: fixed-point f64 atomics into the token's accumulator row */
+                double* arow = (double*)g.out + (size_t)(pidx / g.det_k) * N + col;
+                det_add(arow, y0), det_add(arow + 1, y1), det_add(arow + 2, y2), det_add(arow + 3, y3);
+                if (WIDE) {
+                    det_add(arow + 16, gate * acc1[rt][0]), det_add(arow + 17, gate * acc1[rt][1]);
+                    det_add(arow + 18, gate * acc1[rt][2]), det_add(arow + 19, gate * acc1[rt][3]);
+                }
+                continue;
+            }
             if (g.acc_topk) { /* add into the layer output row of the slot's token, packed bf16 atomics */
                 bf16_t* orow = (bf16_t*)g.out + (size_t)(pidx / g.acc_topk) * N + col;
                 sk_atomic_add_bf16x2(orow, y0, y1);

@@ -650,6 +650,19 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                                      : "=&v"(oa), "=&v"(ob)
                                      : "v"(wr0), "v"(wr1), "v"(y0), "v"(y1), "v"(rd)
                                      : "memory");
+                        if (g.det_k) {
+                            /* deterministic fused combine: fixed-point f64 atomics into the token's accumulator
+                             * row; 8 lanes cover 256 consecutive bytes of it */
+                            if (rowa < rows && pa != PLOW_EXPERT_UNUSED) {
+                                double* o = (double*)g.out + (size_t)(pa / g.det_k) * g.N + ch0 + 4u * lp;
+                                det_add(o, oa[0]), det_add(o + 1, oa[1]), det_add(o + 2, oa[2]), det_add(o + 3, oa[3]);
+                            }
+                            if (rowb < rows && pb != PLOW_EXPERT_UNUSED) {
+                                double* o = (double*)g.out + (size_t)(pb / g.det_k) * g.N + ch0 + 4u * lp;
+                                det_add(o, ob[0]), det_add(o + 1, ob[1]), det_add(o + 2, ob[2]), det_add(o + 3, ob[3]);
+                            }
+                            return;
+                        }
                         float* const ocol = (float*)g.out + ch0 + 4u * lp;
                         if (rowa < rows && pa != PLOW_EXPERT_UNUSED)
                             *(float4*)(ocol + (size_t)pa * g.N) = make_float4(oa[0], oa[1], oa[2], oa[3]);
@@ -728,7 +741,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                                                                                __builtin_bit_cast(bf16x2_t, pk));
                                 }
                         }
-                    } else if (wave_on && !g.part16) {
+                    } else if (wave_on && (g.det_k || !g.part16)) {
 #pragma unroll
                         for (int rg = 0; rg < 8; rg++) {
                             if (16u * (uint32_t)rg >= rows) break; /* uniform */

@@ -17,6 +17,10 @@ int launch_align(int32_t* meta, const void* table, uint32_t* row_token, uint32_t
                  uint32_t chunk_cap, hipStream_t st);
 int launch_combine(void* out, const void* residual, const void* shared, const void* part, uint32_t H,
                    uint32_t k, uint32_t T, uint32_t part16, hipStream_t st);
+/* the deterministic fused combine: acc is the f64 [T][H] fixed-point accumulator the DOWN op summed in place */
+int launch_combine_det(void* out, const void* residual, const void* shared, const double* acc, uint32_t H, uint32_t T,
+                       hipStream_t st);
+int launch_zero_f64(double* p, size_t n, hipStream_t st);
 
 int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uint32_t K, uint32_t pitch,
                           hipStream_t st);
@@ -49,6 +53,10 @@ struct GroupW8A8 {
      * gate * acc into row (row_partidx / acc_topk) with packed bf16 atomics (order-dependent rounding;
      * plow's fused-combine variant, runtime/amd/moe_fp8_pf.hip:1219-1230) */
     uint32_t acc_topk;
+    /* DOWN: when non-zero (= routing slots per token), `out` is the f64 [T][N] fixed-point accumulator of
+     * the deterministic fused combine: every live row adds rint(clamp(gate * acc) * 2^32) into row
+     * (row_partidx / det_k) with f64 atomics (order-independent; plow runtime/amd/op_moe.h:2110-2165) */
+    uint32_t det_k;
     /* GLU, block mode: when non-zero, `a` holds the bf16 rows [T][K] themselves and the kernel quantizes
      * every 1x128 group as it loads it (a_scale and pitch unused; plow's arm i7 = 6) */
     uint32_t a_bf16;

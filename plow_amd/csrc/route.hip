@@ -1177,6 +1177,63 @@ __global__ __launch_bounds__(256) void k_combine(CombineArgs a) {
     combine_body<KT>(a);
 }
 
+/* The deterministic fused combine (plow runtime/amd/op_moe.h:5380-5520): the DOWN op has summed the k
+ * contributions of every token in place as integer-valued doubles (fixed point, 2^-32), so this reads one
+ * contiguous f64 stream: out = bf16(residual? + shared? + (float)(acc * 2^-32)), four h per thread. */
+__global__ __launch_bounds__(256) void k_combine_det(bf16_t* __restrict__ out, const bf16_t* __restrict__ residual,
+                                                     const bf16_t* __restrict__ shared, const double* __restrict__ acc64,
+                                                     uint32_t H, uint32_t T) {
+    const size_t total = (size_t)T * (H / 4u);
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < total; i += (size_t)gridDim.x * 256u) {
+        const size_t o = i * 4u;
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const double4 v = *(const double4*)(acc64 + o);
+        if (residual) {
+            const uint2 r = *(const uint2*)(residual + o);
+            acc[0] = __uint_as_float(r.x << 16); acc[1] = __uint_as_float(r.x & 0xFFFF0000u);
+            acc[2] = __uint_as_float(r.y << 16); acc[3] = __uint_as_float(r.y & 0xFFFF0000u);
+        }
+        if (shared) {
+            const uint2 r = *(const uint2*)(shared + o);
+            acc[0] += __uint_as_float(r.x << 16); acc[1] += __uint_as_float(r.x & 0xFFFF0000u);
+            acc[2] += __uint_as_float(r.y << 16); acc[3] += __uint_as_float(r.y & 0xFFFF0000u);
+        }
+        acc[0] += (float)(v.x * PLOW_DET_UNSCALE); acc[1] += (float)(v.y * PLOW_DET_UNSCALE);
+        acc[2] += (float)(v.z * PLOW_DET_UNSCALE); acc[3] += (float)(v.w * PLOW_DET_UNSCALE);
+        uint2 w;
+        w.x = (uint32_t)f2bf(acc[0]) | ((uint32_t)f2bf(acc[1]) << 16);
+        w.y = (uint32_t)f2bf(acc[2]) | ((uint32_t)f2bf(acc[3]) << 16);
+        *(uint2*)(out + o) = w;
+    }
+}
+
+int launch_combine_det(void* out, const void* residual, const void* shared, const double* acc, uint32_t H, uint32_t T,
+                       hipStream_t st) {
+    if (H % 4u || T == 0) return PLOW_MOE_EINVAL;
+    const size_t total = (size_t)T * (H / 4u);
+    uint32_t blocks = (uint32_t)((total + 255u) / 256u);
+    if (blocks > 4096u) blocks = 4096u;
+    k_combine_det<<<blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)residual, (const bf16_t*)shared, acc, H, T);
+    return 0;
+}
+
+/* zero-fill of the f64 accumulator (a kernel, not a memset: the call may be captured into a graph) */
+__global__ __launch_bounds__(256) void k_zero_f64(double2* __restrict__ p, size_t n2, double* __restrict__ tail, uint32_t ntail) {
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n2; i += (size_t)gridDim.x * 256u) p[i] = make_double2(0.0, 0.0);
+    if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0.0;
+}
+
+int launch_zero_f64(double* p, size_t n, hipStream_t st) {
+    if (n == 0) return 0;
+    if ((uintptr_t)p % 16u) return PLOW_MOE_EINVAL;
+    const size_t n2 = n / 2u;
+    uint32_t blocks = (uint32_t)((n2 + 255u) / 256u);
+    if (blocks > 4096u) blocks = 4096u;
+    if (blocks == 0u) blocks = 1u;
+    k_zero_f64<<<blocks, 256, 0, st>>>((double2*)p, n2, p + 2u * n2, (uint32_t)(n & 1u));
+    return 0;
+}
+
 int launch_combine(void* out, const void* residual, const void* shared, const void* part, uint32_t H,
                    uint32_t k, uint32_t T, uint32_t part16, hipStream_t st) {
     if (H % 4u || T == 0) return PLOW_MOE_EINVAL;

@@ -43,6 +43,9 @@ class MoeConfig:
     act_f: Tuple[float, float] = (0.0, 0.0)  # the activation's immediates (fj[0], fj[1]) for the pair forms 2 / 3 / 4
     residual: bool = False
     part_bf16: bool = False         # block-fp8 W8A8 only: bf16 partials (arm 3) instead of f32
+    det_combine: bool = False       # block-fp8 W8A8 only: the deterministic fused down -> combine (op 83 zeroes a
+                                    # [T][H] f64 fixed-point accumulator, op 86 adds into it, op 87 reads it as
+                                    # one stream; plow runtime/amd/op_moe.h:2110-2165); no part tensor
 
     @property
     def tail(self) -> int:
@@ -143,14 +146,17 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
     row_partidx = p._t("row_partidx", "u32", (R,), "scratch")
     row_gate = p._t("row_gate", "f32", (R,), "scratch")
     p16 = cfg.part_bf16 and cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q")
-    part = p._t("part", "bf16" if p16 else "f32", (T * ka, H), "scratch")
+    det = cfg.det_combine and cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q")
+    assert not (det and p16)
+    part = (p._t("acc64", "f64", (T, H), "scratch") if det
+            else p._t("part", "bf16" if p16 else "f32", (T * ka, H), "scratch"))
     out = p._t("out", "bf16", (T, H), "out")
     residual = p._t("residual", "bf16", (T, H), "in") if cfg.residual else None
 
     if with_router_score:
         p._emit("score", abi.inst(abi.OP_GEMM_F32, t=[logit, x, wr], i=[T, E, H]))
-    p._emit("topk", abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[table, logit, None, bias],
-                             i=[0, E, k, cfg.flags, T, cfg.tail, cfg.n_group, cfg.topk_group],
+    p._emit("topk", abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[table, logit, part if det else None, bias],
+                             i=[H if det else 0, E, k, cfg.flags, T, cfg.tail, cfg.n_group, cfg.topk_group],
                              f=[cfg.route_scale, 0.0]))
     p._emit("align", abi.inst(abi.OP_MOE_ALIGN_PF, t=[meta, table, row_token, row_partidx, row_gate],
                               i=[T, Ea, ka]))
@@ -215,7 +221,8 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
                                         i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8], f=cfg.act_f, slots=T * ka))
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
                                      t=[part, fq, wtab, stab, meta, fs, row_partidx, row_gate],
-                                     i=[H, I, Ea, enc, 0, 0, 0, abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8], slots=T * ka))
+                                     i=[H, I, Ea, enc, 0, (256 + ka) if det else 0, 0,
+                                        abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8], slots=T * ka))
         else:
             arm = abi.ARM_W4A16 if enc == abi.ENC_MXFP4 else abi.ARM_A16
             fu = p._t("fu", "bf16", (R, I), "scratch")
@@ -238,5 +245,5 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
                                        i=[T, Is, H, 0, 0, cfg.act]))
         p._emit("shared_down", abi.inst(abi.OP_GEMM, t=[shared, sfu, wsd], i=[T, H, Is]))
     p._emit("combine", abi.inst(abi.OP_MOE_COMBINE_PF, t=[out, residual, shared, part],
-                                i=[H, ka, T, 0, 0, 0, 0, 1 if p16 else 0]))
+                                i=[H, 1 if det else ka, T, 0, 1 if det else 0, 0, 0, 1 if p16 else 0]))
     return p

@@ -23,8 +23,8 @@ import torch
 from . import abi
 from .layer import LayerPlan, MoeConfig
 
-_TORCH_DT = {"bf16": torch.bfloat16, "f32": torch.float32, "u8": torch.uint8, "i32": torch.int32,
-             "u32": torch.int32, "u64": torch.int64}
+_TORCH_DT = {"bf16": torch.bfloat16, "f32": torch.float32, "f64": torch.float64, "u8": torch.uint8,
+             "i32": torch.int32, "u32": torch.int32, "u64": torch.int64}
 
 E4M3_MAX = 448.0
 

@@ -197,3 +197,37 @@ def test_segment_entry_points(moe, oracle):
     with pytest.raises(Exception) as ei:
         moe.pf(bad, dev.table(), cfg.T)
     assert "disagree" in str(ei.value)
+
+
+@pytest.mark.parametrize("T", [24, 700])   # weight-streaming form, tiled form
+def test_deterministic_fused_combine(moe, oracle, T):
+    """Op 83 zeroes a [T][H] f64 accumulator, op 86 (i5) adds every live row's gate * acc into its token's
+    row as an integer-valued double, op 87 (i4) reads it as one stream (plow runtime/amd/op_moe.h:2110-2165).
+    The accumulator must equal, exactly, the integer sum of the quantized partials the plain chain of the
+    same kernels writes (closed form over the device's own `part`), two runs must agree bit for bit
+    (the additions commute), and the output must meet the layer tolerance against the oracle's."""
+    import dataclasses
+    from gpu_harness import run_device, run_oracle
+    from plow_amd import synth
+    from test_oracle_pins import det_closed_form
+    print(f"[case] deterministic fused combine T={T}", flush=True)
+    cfg = layer.MoeConfig("det", H=512, E=32, I=256, k=4, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          n_group=4, topk_group=2, route_scale=2.5, enc="fp8blk", arm="w8a8", n_shared=1,
+                          shared_mode="fold", residual=True)
+    plain = layer.plan_layer(cfg)
+    dp = synth.bind(plain, "cuda", seed=T)
+    run_device(moe, plain, dp)
+    want = det_closed_form(dp.t["part"].cpu().numpy(), cfg.T, cfg.k_all, cfg.H)
+    det = layer.plan_layer(dataclasses.replace(cfg, det_combine=True))
+    runs = []
+    for rep in range(2):
+        dd = synth.bind(det, "cuda", seed=T)
+        dd.t["acc64"].fill_(float(rep + 1))          # op 83 must zero it
+        run_device(moe, det, dd)
+        runs.append((dd.t["acc64"].cpu().numpy(), dd.np("out")))
+    assert np.array_equal(runs[0][0].view(np.uint64), runs[1][0].view(np.uint64))
+    assert np.array_equal(runs[0][1], runs[1][1])
+    assert np.array_equal(runs[0][0], want.astype(np.float64)), "accumulator differs from the integer sum of the partials"
+    host = synth.to_host(dd)
+    run_oracle(oracle, det, host)
+    assert_output_close(runs[0][1], host.np("out"), f"det combine T={T} out")

@@ -562,3 +562,68 @@ def test_per_channel_w8a8_against_f64(oracle):
         assert np.all(np.abs(ol.bf2f(fu[row]) - v) <= 2.0 ** -8 * np.abs(v) + 1e-7)
         y = tab["gate"][s] * ((dec(d8[e]) @ dec(fu8[row])) * fsc[row] * sd[e])
         assert np.allclose(part[s], y, rtol=1e-5, atol=1e-6)
+
+
+def det_closed_form(part, T, k, H):
+    """The deterministic fused combine's accumulator from the f32 partials of the plain chain, in exact
+    integer arithmetic: acc[t][h] = sum_j rint(clamp(part[t*k+j][h], +-2^17) * 2^32) (Python integers)."""
+    p = np.clip(part.astype(np.float64).reshape(T, k, H), -131072.0, 131072.0) * 4294967296.0
+    q = np.rint(p)                                  # |q| <= 2^49: exact in f64 and in int64
+    return q.astype(np.int64).sum(axis=1)
+
+
+def test_deterministic_fused_combine_closed_form_and_thread_independence(oracle):
+    """Op 86 with i5 (plow runtime/amd/op_moe.h:2110-2165): the [T][H] f64 accumulator must hold, exactly,
+    the integer sum of the quantized contributions the plain arm writes to `part` (closed form in integer
+    arithmetic), whatever the number of workers (the additions commute); op 83 zeroes it; op 87 with i4
+    reads it as one stream: out = bf16(residual + (float)(acc * 2^-32)). The clamp at +-2^17 is reached
+    with a huge gate."""
+    import dataclasses
+    from gpu_harness import run_oracle
+    from plow_amd import layer, synth
+    cfg = layer.MoeConfig("det", H=256, E=6, I=128, k=3, T=21, scoring="sigmoid", norm_topk=True, bias=True,
+                          enc="fp8blk", arm="w8a8", n_shared=1, shared_mode="fold", residual=True)
+    plain = layer.plan_layer(cfg)
+    hp = synth.bind(plain, "cpu", seed=5)
+    run_oracle(oracle, plain, hp)
+    det = layer.plan_layer(dataclasses.replace(cfg, det_combine=True))
+    assert "part" not in det.slots and det.insts[det.index("down")].i[5] == 256 + cfg.k_all
+    outs = []
+    for nthreads in (1, 7, 16):
+        hd = synth.bind(det, "cpu", seed=5)
+        hd.t["acc64"].fill_(123.0)                  # op 83 must zero it
+        run_oracle(oracle, det, hd, nthreads=nthreads)
+        outs.append((hd.t["acc64"].numpy().copy(), hd.np("out").copy()))
+    want = det_closed_form(hp.t["part"].numpy(), cfg.T, cfg.k_all, cfg.H)
+    for acc, out in outs:
+        assert np.array_equal(acc, want.astype(np.float64)) and np.all(acc == np.rint(acc))
+        assert np.array_equal(out, outs[0][1])
+    res = ol.bf2f(hp.np("residual")).astype(np.float32)
+    expect = ol.f2bf(res + (want.astype(np.float64) * 2.0 ** -32).astype(np.float32))
+    assert np.array_equal(outs[0][1], expect)
+    # against the plain chain's output: same values up to the order of the f32 additions and 2^-32 steps
+    a, b = ol.bf2f(outs[0][1]).astype(np.float64), ol.bf2f(hp.np("out")).astype(np.float64)
+    assert np.abs(a - b).max() <= 2.0 ** -7 * np.abs(b).max()
+    # the clamp: a gate of 1e9 drives every contribution to +-2^17 * 2^32 = +-2^49
+    big = synth.bind(det, "cpu", seed=5)
+    run_oracle(oracle, det, big, labels=["score", "topk", "align", "quant_x", "glu"])
+    big.t["row_gate"].fill_(1e9)
+    run_oracle(oracle, det, big, labels=["down"])
+    acc = big.t["acc64"].numpy()
+    assert np.abs(acc).max() <= cfg.k_all * 2.0 ** 49 and (np.abs(acc) >= 2.0 ** 49).any()
+
+
+def test_deterministic_fused_combine_reference_shift_encoding(oracle):
+    """i5 = log2(k) + 1 (the reference's encoding, power-of-two k) selects the same rows as 256 + k."""
+    import dataclasses
+    from gpu_harness import run_oracle
+    from plow_amd import layer, synth
+    cfg = layer.MoeConfig("det4", H=128, E=5, I=128, k=4, T=9, scoring="softmax", norm_topk=True,
+                          enc="fp8blk", arm="w8a8", det_combine=True)
+    plan = layer.plan_layer(cfg)
+    a = synth.bind(plan, "cpu", seed=2)
+    run_oracle(oracle, plan, a)
+    plan.insts[plan.index("down")].i[5] = 3         # log2(4) + 1
+    b = synth.bind(plan, "cpu", seed=2)
+    run_oracle(oracle, plan, b)
+    assert np.array_equal(a.t["acc64"].numpy(), b.t["acc64"].numpy()) and np.abs(a.t["acc64"].numpy()).max() > 0
