@@ -89,32 +89,7 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
     asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
     return r;
 }
-/* The B operand (and scale) of a row group, requested only when `live` (wave-uniform): the reads
- * execute with EXEC = 0 otherwise, which skips them in hardware. For the compiler the statement is
- * unconditional, so a register written by these asynchronous reads never passes a control-flow merge
- * on its way to its wait (a copy placed at a merge would run before the data has arrived). EXEC is
- * all ones wherever this is used. */
-template <uint32_t OFF, uint32_t SOFF, bool WITH_SCALE>
-__device__ __forceinline__ void ds_read_group(uint32_t live, uint32_t alo, uint32_t ahi, uint32_t asc, v4i& lo,
-                                              v4i& hi, float& sc) {
-    if (WITH_SCALE)
-        asm volatile("s_cmp_lg_u32 %6, 0\n\ts_cselect_b64 exec, -1, 0\n\t"
-                     "ds_read_b128 %0, %3 offset:%7\n\tds_read_b128 %1, %4 offset:%7\n\tds_read_b32 %2, %5 offset:%8\n\t"
-                     "s_mov_b64 exec, -1"
-                     : "=v"(lo), "=v"(hi), "=v"(sc)
-                     : "v"(alo), "v"(ahi), "v"(asc), "s"(live), "n"(OFF), "n"(SOFF)
-                     : "memory", "scc");
-    else
-        asm volatile("s_cmp_lg_u32 %4, 0\n\ts_cselect_b64 exec, -1, 0\n\t"
-                     "ds_read_b128 %0, %2 offset:%5\n\tds_read_b128 %1, %3 offset:%5\n\t"
-                     "s_mov_b64 exec, -1"
-                     : "=v"(lo), "=v"(hi)
-                     : "v"(alo), "v"(ahi), "s"(live), "n"(OFF)
-                     : "memory", "scc");
-}
-/* all ds_reads issued so far have returned; the operands are tied so no use is hoisted above */
-#define LDS_WAIT2(a, b) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b))
-#define LDS_WAIT_F(a) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a))
+/* all ds_reads issued so far have returned */
 #define LDS_WAIT_ALL() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
 #define WG_BARRIER() asm volatile("s_barrier" ::: "memory")
 /* wait until at most n of this wave's loads are outstanding, then the workgroup barrier */
@@ -129,84 +104,30 @@ __device__ __forceinline__ void ds_read_group(uint32_t live, uint32_t alo, uint3
     const uint32_t sl = s_base + st * (T5_BM * 4u) + r16 * 4u;                                               \
     const uint32_t cl = c_base + par * 1024u + kb * 4u;
 #define T5_ADVANCE() st = st == 2u ? 0u : st + 1u
-#define T5_BLOCK_OPERANDS()                                                                                  \
-    float ws0 = 0.0f, ws1 = 0.0f;                                                                            \
-    if (!PC) {                                                                                               \
-        ws0 = ds_read4<0>(cl);                                                                               \
-        ws1 = ds_read4<512>(cl);                                                                             \
-    }                                                                                                        \
-    v4i al[2], ah[2];                                                                                        \
-    al[0] = ds_read16<0>(alo), ah[0] = ds_read16<0>(ahi);                                                    \
-    al[1] = ds_read16<2048>(alo), ah[1] = ds_read16<2048>(ahi);                                              \
-    v4i bl[2], bh[2];                                                                                        \
-    float as_[2];                                                                                            \
-    bl[0] = ds_read16<0>(blo), bh[0] = ds_read16<0>(bhi);                                                    \
-    as_[0] = as_[1] = 0.0f;                                                                                  \
-    if (!PC) as_[0] = ds_read4<0>(sl);                                                                       \
-    if (!PC) LDS_WAIT2(ws0, ws1);                                                                            \
-    LDS_WAIT2(al[0], ah[0]);                                                                                 \
-    LDS_WAIT2(al[1], ah[1]);                                                                                 \
-    if (!GLU && !PC) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);                                                    \
-    v8i aop[2];                                                                                              \
-    _Pragma("unroll") for (int x = 0; x < 2; x++) aop[x] = __builtin_shufflevector(al[x], ah[x], 0, 1, 2, 3, 4, 5, 6, 7);
-
-/* Tiles with dead row groups. Per-channel mode: the scales are outside the K reduction, so the matrix
- * unit accumulates straight through; block mode: one scaled add per 128-k block. The read of group
- * RG + 1 is in flight while group RG multiplies. */
-#define T5_GROUP_PARTIAL(RG)                                                                                 \
-    LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                                   \
-    if (!PC) LDS_WAIT_F(as_[(RG) & 1]);                                                                      \
-    if ((RG) + 1 < 8)                                                                                        \
-        ds_read_group<(((RG) + 1) & 7) * 2048u, (((RG) + 1) & 7) * 64u, !PC>(                                \
-            (uint32_t)__builtin_amdgcn_readfirstlane((RG) + 1u < ngrp_w ? 1 : 0), blo, bhi, sl, bl[((RG) + 1) & 1], bh[((RG) + 1) & 1], as_[((RG) + 1) & 1]); \
-    if ((RG) < ngrp_w) {                                                                                     \
-        const v8i b = __builtin_shufflevector(bl[(RG) & 1], bh[(RG) & 1], 0, 1, 2, 3, 4, 5, 6, 7);           \
-        if (PC) {                                                                                            \
-            acc[RG][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, acc[RG][0], 0, 0, 0, 0, 0, 0); \
-            acc[RG][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, acc[RG][1], 0, 0, 0, 0, 0, 0); \
-        } else {                                                                                             \
-            const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};                                                          \
-            const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, z, 0, 0, 0, 0, 0, 0); \
-            const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, z, 0, 0, 0, 0, 0, 0); \
-            const float sc0 = as_[(RG) & 1] * ws0, sc1 = as_[(RG) & 1] * ws1;                                \
-            _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                  \
-                acc[RG][0][i] = fmaf(t0[i], sc0, acc[RG][0][i]);                                             \
-                acc[RG][1][i] = fmaf(t1[i], sc1, acc[RG][1][i]);                                             \
-            }                                                                                                \
+/* A block of a consumer with N live row groups (N a constant, 1..8): straight-line code without a
+ * condition in it, so no value is ever copied between registers. Per-channel mode: the scales are outside
+ * the K reduction, so the matrix unit accumulates straight through; block mode: one scaled add per 128-k
+ * block, and the scaled adds of group RG follow the matrix instructions of group RG + 1, never wait for
+ * a result and overlap with the matrix unit.
+ * LDS reads return in issue order: with the reads of group RG + 1 (two operand halves, and the scale in
+ * block mode) issued behind those of group RG, "at most that many outstanding" means group RG has
+ * arrived. Three operand buffers rotate, so a group's reads are issued two groups before its multiply. */
+#define T5_GROUP_N(RG, N)                                                                                    \
+    if ((RG) < (N)) {                                                                                        \
+        asm volatile("s_waitcnt lgkmcnt(%2)"                                                                 \
+                     : "+v"(bl[(RG) % 3]), "+v"(bh[(RG) % 3])                                                \
+                     : "n"((RG) + 1 < (N) ? (PC ? 2 : 3) : 0));                                              \
+        if (!PC) {                                                                                           \
+            asm volatile("" : "+v"(as_[(RG) % 3]));                                                          \
+            sc[(RG) & 1][0] = as_[(RG) % 3] * ws0;                                                           \
+            sc[(RG) & 1][1] = as_[(RG) % 3] * ws1;                                                           \
         }                                                                                                    \
-    }
-#define T5_BLOCK_PARTIAL()                                                                                   \
-    T5_BLOCK_HEAD()                                                                                          \
-    if (ngrp_w != 0u) {                                                                                      \
-        T5_BLOCK_OPERANDS()                                                                                  \
-        T5_GROUP_PARTIAL(0) T5_GROUP_PARTIAL(1) T5_GROUP_PARTIAL(2) T5_GROUP_PARTIAL(3)                      \
-        T5_GROUP_PARTIAL(4) T5_GROUP_PARTIAL(5) T5_GROUP_PARTIAL(6) T5_GROUP_PARTIAL(7)                      \
-    }
-
-/* Tiles with all eight row groups live: no condition anywhere, so no value is ever copied between
- * registers; in block mode the scaled adds of group RG follow the matrix instructions of group RG + 1,
- * never wait for a result and overlap with the matrix unit. */
-#define T5_SCALE_FULL(RG)                                                                                    \
-    if (!PC) {                                                                                               \
-        _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                      \
-            acc[RG][0][i] = fmaf(t[(RG) & 1][0][i], sc[(RG) & 1][0], acc[RG][0][i]);                         \
-            acc[RG][1][i] = fmaf(t[(RG) & 1][1][i], sc[(RG) & 1][1], acc[RG][1][i]);                         \
+        if ((RG) + 2 < (N)) {                                                                                \
+            bl[((RG) + 2) % 3] = ds_read16<(((RG) + 2) & 7) * 2048u>(blo);                                   \
+            bh[((RG) + 2) % 3] = ds_read16<(((RG) + 2) & 7) * 2048u>(bhi);                                   \
+            if (!PC) as_[((RG) + 2) % 3] = ds_read4<(((RG) + 2) & 7) * 64u>(sl);                             \
         }                                                                                                    \
-    }
-#define T5_GROUP_FULL(RG)                                                                                    \
-    LDS_WAIT2(bl[(RG) & 1], bh[(RG) & 1]);                                                                   \
-    if (!PC) {                                                                                               \
-        LDS_WAIT_F(as_[(RG) & 1]);                                                                           \
-        sc[(RG) & 1][0] = as_[(RG) & 1] * ws0;                                                               \
-        sc[(RG) & 1][1] = as_[(RG) & 1] * ws1;                                                               \
-    }                                                                                                        \
-    if ((RG) + 1 < 8) {                                                                                      \
-        bl[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(blo);                                       \
-        bh[((RG) + 1) & 1] = ds_read16<(((RG) + 1) & 7) * 2048u>(bhi);                                       \
-        if (!PC) as_[((RG) + 1) & 1] = ds_read4<(((RG) + 1) & 7) * 64u>(sl);                                 \
-    }                                                                                                        \
-    {                                                                                                        \
-        const v8i b = __builtin_shufflevector(bl[(RG) & 1], bh[(RG) & 1], 0, 1, 2, 3, 4, 5, 6, 7);           \
+        const v8i b = __builtin_shufflevector(bl[(RG) % 3], bh[(RG) % 3], 0, 1, 2, 3, 4, 5, 6, 7);           \
         if (PC) {                                                                                            \
             acc[RG][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[0], b, acc[RG][0], 0, 0, 0, 0, 0, 0); \
             acc[RG][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, acc[RG][1], 0, 0, 0, 0, 0, 0); \
@@ -216,20 +137,67 @@ __device__ __forceinline__ void ds_read_group(uint32_t live, uint32_t alo, uint3
             t[(RG) & 1][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aop[1], b, z, 0, 0, 0, 0, 0, 0); \
         }                                                                                                    \
     }
-#define T5_BLOCK_FULL()                                                                                      \
+#define T5_SCALE_N(RG, N)                                                                                    \
+    if (!PC && (RG) < (N)) {                                                                                 \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                      \
+            acc[RG][0][i] = fmaf(t[(RG) & 1][0][i], sc[(RG) & 1][0], acc[RG][0][i]);                         \
+            acc[RG][1][i] = fmaf(t[(RG) & 1][1][i], sc[(RG) & 1][1], acc[RG][1][i]);                         \
+        }                                                                                                    \
+    }
+/* the operands of the block: weight scales, the two weight operands, then the token operands of groups 0
+ * and 1; the weight operands are waited for with those groups still in flight */
+#define T5_BLOCK_OPERANDS_N(N)                                                                               \
+    float ws0 = 0.0f, ws1 = 0.0f;                                                                            \
+    if (!PC) {                                                                                               \
+        ws0 = ds_read4<0>(cl);                                                                               \
+        ws1 = ds_read4<512>(cl);                                                                             \
+    }                                                                                                        \
+    v4i al[2], ah[2];                                                                                        \
+    al[0] = ds_read16<0>(alo), ah[0] = ds_read16<0>(ahi);                                                    \
+    al[1] = ds_read16<2048>(alo), ah[1] = ds_read16<2048>(ahi);                                              \
+    v4i bl[3], bh[3];                                                                                        \
+    float as_[3];                                                                                            \
+    as_[0] = as_[1] = as_[2] = 0.0f;                                                                         \
+    bl[0] = ds_read16<0>(blo), bh[0] = ds_read16<0>(bhi);                                                    \
+    if (!PC) as_[0] = ds_read4<0>(sl);                                                                       \
+    if ((N) > 1) {                                                                                           \
+        bl[1] = ds_read16<2048u>(blo), bh[1] = ds_read16<2048u>(bhi);                                        \
+        if (!PC) as_[1] = ds_read4<64u>(sl);                                                                 \
+    }                                                                                                        \
+    asm volatile("s_waitcnt lgkmcnt(%6)"                                                                     \
+                 : "+v"(al[0]), "+v"(ah[0]), "+v"(al[1]), "+v"(ah[1]), "+v"(ws0), "+v"(ws1)                  \
+                 : "n"((PC ? 2 : 3) * ((N) > 1 ? 2 : 1)));                                                   \
+    if (!GLU && !PC) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);                                                    \
+    v8i aop[2];                                                                                              \
+    _Pragma("unroll") for (int x = 0; x < 2; x++) aop[x] = __builtin_shufflevector(al[x], ah[x], 0, 1, 2, 3, 4, 5, 6, 7);
+#define T5_BLOCK_N(N)                                                                                        \
     T5_BLOCK_HEAD()                                                                                          \
-    T5_BLOCK_OPERANDS()                                                                                      \
+    T5_BLOCK_OPERANDS_N(N)                                                                                   \
     v4f t[2][2];                                                                                             \
     float sc[2][2];                                                                                          \
-    T5_GROUP_FULL(0)                                                                                         \
-    T5_GROUP_FULL(1) T5_SCALE_FULL(0)                                                                        \
-    T5_GROUP_FULL(2) T5_SCALE_FULL(1)                                                                        \
-    T5_GROUP_FULL(3) T5_SCALE_FULL(2)                                                                        \
-    T5_GROUP_FULL(4) T5_SCALE_FULL(3)                                                                        \
-    T5_GROUP_FULL(5) T5_SCALE_FULL(4)                                                                        \
-    T5_GROUP_FULL(6) T5_SCALE_FULL(5)                                                                        \
-    T5_GROUP_FULL(7) T5_SCALE_FULL(6)                                                                        \
-    T5_SCALE_FULL(7)
+    T5_GROUP_N(0, N)                                                                                         \
+    T5_GROUP_N(1, N) T5_SCALE_N(0, N)                                                                        \
+    T5_GROUP_N(2, N) T5_SCALE_N(1, N)                                                                        \
+    T5_GROUP_N(3, N) T5_SCALE_N(2, N)                                                                        \
+    T5_GROUP_N(4, N) T5_SCALE_N(3, N)                                                                        \
+    T5_GROUP_N(5, N) T5_SCALE_N(4, N)                                                                        \
+    T5_GROUP_N(6, N) T5_SCALE_N(5, N)                                                                        \
+    T5_GROUP_N(7, N) T5_SCALE_N(6, N)                                                                        \
+    T5_SCALE_N(7, N)
+/* the K loop of a tile for a consumer wave with N live groups (BODY empty: it only keeps the barriers) */
+#define T5_RUN_BLOCKS(BODY)                                                                                  \
+    for (uint32_t kb = 0; kb < KB; kb++) {                                                                   \
+        WG_BARRIER(); /* block kb is in LDS */                                                               \
+        _Pragma("unroll") for (uint32_t sub = 0; sub < SUBS; sub++) {                                        \
+            const uint32_t cw = cw0 + sub;                                                                   \
+            (void)cw;                                                                                        \
+            v4f(&acc)[8][2] = accs[sub];                                                                     \
+            (void)acc;                                                                                       \
+            BODY                                                                                             \
+        }                                                                                                    \
+        T5_ADVANCE();                                                                                        \
+        LDS_WAIT_ALL(); /* nothing of this block is still being read when the next barrier is passed */      \
+    }
 
 /* NCW = consumer waves: 8 (768 threads, the library's own launch) or 4 (512 threads: a wave then runs
  * two of the eight consumers' shares one after the other in every block, for callers whose launch shape
@@ -523,33 +491,20 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 for (int rg = 0; rg < 8; rg++)
 #pragma unroll
                     for (int x = 0; x < 2; x++) accs[sub][rg][x] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-            /* Two forms of the block loop: tiles whose eight row groups are all live (the common case) run
-             * code without a condition in it, which lets the scaled adds of a group be issued after the
-             * matrix instructions of the next group; the other tiles skip their dead groups. */
-            if (ngrp_w == 8u) {
-                for (uint32_t kb = 0; kb < KB; kb++) {
-                    WG_BARRIER(); /* block kb is in LDS */
-#pragma unroll
-                    for (uint32_t sub = 0; sub < SUBS; sub++) {
-                        const uint32_t cw = cw0 + sub;
-                        v4f(&acc)[8][2] = accs[sub];
-                        T5_BLOCK_FULL()
-                    }
-                    T5_ADVANCE();
-                    LDS_WAIT_ALL(); /* nothing of this block is still being read when the next barrier is passed */
-                }
-            } else {
-                for (uint32_t kb = 0; kb < KB; kb++) {
-                    WG_BARRIER(); /* block kb is in LDS */
-#pragma unroll
-                    for (uint32_t sub = 0; sub < SUBS; sub++) {
-                        const uint32_t cw = cw0 + sub;
-                        v4f(&acc)[8][2] = accs[sub];
-                        T5_BLOCK_PARTIAL()
-                    }
-                    T5_ADVANCE();
-                    LDS_WAIT_ALL();
-                }
+            /* One form of the block loop per count of live row groups: each is straight-line code. The
+             * wait the compiler can see (everything the LDS was asked for has arrived) keeps it from
+             * placing waits of its own inside the loops, whose LDS reads it does not see. */
+            __builtin_amdgcn_s_waitcnt(0xc07f); /* lgkmcnt(0) */
+            switch (ngrp_w) {
+                case 8u: { T5_RUN_BLOCKS(T5_BLOCK_N(8)) } break;
+                case 7u: { T5_RUN_BLOCKS(T5_BLOCK_N(7)) } break;
+                case 6u: { T5_RUN_BLOCKS(T5_BLOCK_N(6)) } break;
+                case 5u: { T5_RUN_BLOCKS(T5_BLOCK_N(5)) } break;
+                case 4u: { T5_RUN_BLOCKS(T5_BLOCK_N(4)) } break;
+                case 3u: { T5_RUN_BLOCKS(T5_BLOCK_N(3)) } break;
+                case 2u: { T5_RUN_BLOCKS(T5_BLOCK_N(2)) } break;
+                case 1u: { T5_RUN_BLOCKS(T5_BLOCK_N(1)) } break;
+                default: { T5_RUN_BLOCKS() } break;
             }
 
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
