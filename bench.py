@@ -144,6 +144,9 @@ def run_cell(a, name, tokens, steps, warmup, share=None, cpu_mode="full"):
             "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
             "traffic_over_algorithmic": round(traffic / dom_bytes, 3) if traffic else None,
             "bytes_per_launch": int(dom_bytes), "us_per_launch": round(op_us[dom], 2),
+            # the time each roof allows this launch: the larger one is the roof that binds
+            "roof_us": {"hbm": round(dom_bytes / (HBM_PEAK_GBS * 1e9) * 1e6, 1),
+                        "mfma": round(dom_flops / (FP8_PEAK_TFLOPS * 1e12) * 1e6, 1)},
             "mfma": {"achieved": round(achieved_tf, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved_tf / FP8_PEAK_TFLOPS, 4), "flops_per_launch": dom_flops}}
     rec = {

@@ -53,7 +53,7 @@ __device__ __forceinline__ void sk_atomic_add_bf16x2(bf16_t* p, float a, float b
  * is loaded: amax floored at 1e-10, scale amax / 448, e4m3 of x * (1 / scale), the arithmetic of the
  * separate quantizer op, so the result equals quantizer + plain GLU bit for bit
  * (plow runtime/amd/moe_pf_w8a8.h:118-121, :255-283). */
-template <int RT, bool GLU, int D, bool PC, bool WIDE, uint32_t NW = SK_WAVES, bool AQ = false>
+template <int RT, bool GLU, int D, bool PC, bool WIDE, uint32_t NW = SK_WAVES, bool AQ = false, bool DET = false>
 __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t ct, uint32_t r0,
                                         uint32_t rb, uint32_t cnt, float* s_red) {
     static_assert(NW == 8u || NW == 4u, "eight waves, or four running two shares each");
@@ -294,7 +294,7 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
             const uint32_t pidx = g.row_partidx[rowidx[rt]];
             const float gate = g.row_gate[rowidx[rt]];
             const float y0 = gate * acc0[rt][0], y1 = gate * acc0[rt][1], y2 = gate * acc0[rt][2], y3 = gate * acc0[rt][3];
-            if (g.det_k) { /* order-independent: fixed-point f64 atomics into the token's accumulator row */
+            if (DET && g.det_k) { /* order-independent: fixed-point f64 atomics into the token's accumulator row */
                 double* arow = (double*)g.out + (size_t)(pidx / g.det_k) * N + col;
                 det_add(arow, y0), det_add(arow + 1, y1), det_add(arow + 2, y2), det_add(arow + 3, y3);
                 if (WIDE) {
@@ -359,7 +359,9 @@ __device__ __forceinline__ void sk_body(const GroupW8A8& g, uint32_t e, uint32_t
     }
 }
 
-template <bool GLU, int D, bool PC, bool WIDE = false, bool AQ = false>
+/* DET: the deterministic accumulate epilogue (g.det_k) is compiled only into the launches that ask for
+ * it; in the plain kernel its f64 address arithmetic costs the registers of a fourth wave per SIMD */
+template <bool GLU, int D, bool PC, bool WIDE = false, bool AQ = false, bool DET = false>
 __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     __shared__ float s_red[SK_WAVES * 64u];
     const uint32_t tiles = g.N / (WIDE ? 256u : SK_BN);
@@ -381,7 +383,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
     }
     /* 16 rows a pass; an expert with more rows streams its weights once per pass (the tiled
      * kernel, not this one, is the tool for many rows per expert) */
-    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D, PC, WIDE, SK_WAVES, AQ>(g, e, ct, r0, rb, cnt, s_red);
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) sk_body<1, GLU, D, PC, WIDE, SK_WAVES, AQ, DET>(g, e, ct, r0, rb, cnt, s_red);
     if (bf16_mid) {
         /* a GLU with a bf16 intermediate zeroes the pad rows of its 64-row tile (the partial 16-row pass
          * above did its own); the row quantizer that follows reads every aligned row */
@@ -631,6 +633,14 @@ int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<false, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
+    if (g.det_k) { /* deterministic accumulate: its own instantiations */
+        if (g.N % 256u == 0u && !plow_moe_tuning().sk_narrow) {
+            k_group_w8a8_stream<false, 3, false, true, false, true><<<dim3(g.E * (g.N / 256u)), SK_THREADS, 0, st>>>(g);
+        } else {
+            k_group_w8a8_stream<false, 3, false, false, false, true><<<grid, SK_THREADS, 0, st>>>(g);
+        }
+        return 0;
+    }
     if (g.N % 256u == 0u && !plow_moe_tuning().sk_narrow) {
         const dim3 wgrid(g.E * (g.N / 256u));
         switch (plow_moe_tuning().sk_depth) {
