@@ -42,7 +42,7 @@
  * multiplying: hardware exp2 and reciprocal (about 1 ulp each) instead of the library's expf and an
  * IEEE division, a third of the instructions. The result is rounded to fp8 (block mode) or bf16 (op 188,
  * per-channel mode) right after, far above this error: against the expf form over the same accumulators
- * the bf16 result differs in about one element in 10^4, by one bf16 step (measured by the GPU test that
+ * the bf16 result differs in about one element in 10^5, by one bf16 step (measured by the GPU test that
  * runs op 188 on both forms). Limits: +inf gives +inf and NaN stays NaN as with g / (1 + expf(-g));
  * g = -inf gives NaN here (-inf * rcp(inf)) where the library form gives -0, which only an accumulator
  * that has already overflowed can reach. */
@@ -54,20 +54,22 @@ __device__ __forceinline__ float t5_glu(float gt, float up, uint32_t act, float 
     return moe_glu(gt, up, act, f0, f1);
 }
 
-#define T5_BM 128u
+#define T5_BM 144u /* rows the LDS plan holds per tile: nine 16-row groups (kernels built for eight use 128) */
+#define T5_AS 192u /* row slots of a stage's scale array (three loaders x 64 lanes) */
 #define T5_STAGES 3u
-#define T5_NLOAD 13 /* direct loads per loader and block: 1 scale, 4 token-row, 8 weight-row */
+#define T5_NLOAD 13 /* direct loads per loader and block: 1 scale, 4 token-row, 8 weight-row; loaders 0 and 1 one more
+                     * token-row load (the ninth group) */
 
 struct T5Lds {
     uint8_t a[T5_STAGES][T5_BM * 128u]; /* token rows of a 128-k block, swizzled */
     uint8_t w[T5_STAGES][256u * 128u];  /* weight rows, swizzled; row = 32 * consumer + 16 * group + r */
-    float as[T5_STAGES][T5_BM];         /* activation scales of the block */
+    float as[T5_STAGES][T5_AS];         /* activation scales of the block */
     float wsc[2][2][128];               /* [tile parity][gate|down, up] weight block scales, all of K */
-    float red[8][T5_BM];                /* GLU: per-row amax of each consumer's 16 channels */
-    uint32_t epi_idx[2][T5_BM];         /* [tile parity] GLU: row_token, DOWN: row_partidx of the tile's rows */
-    float epi_gate[2][T5_BM];           /* [tile parity] DOWN: row_gate */
-    uint32_t prefix[1056];
+    uint32_t epi_idx[2][T5_AS];         /* [tile parity] GLU: row_token, DOWN: row_partidx of the tile's rows */
+    float epi_gate[2][T5_AS];           /* [tile parity] DOWN: row_gate */
+    uint16_t prefix[1056];              /* inclusive tile count over experts: at most 2^18 slots / 144 + 1056 */
 };
+static_assert(sizeof(T5Lds) <= 160u * 1024u, "the tile's LDS plan must fit one CU");
 
 typedef __attribute__((address_space(3))) void lds_void;
 
@@ -101,10 +103,10 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
     const uint32_t ab = a_base + st * (T5_BM * 128u), wb = w_base + st * (256u * 128u) + cw * (32u * 128u);  \
     const uint32_t blo = ab + op_lo, bhi = ab + op_hi;                                                       \
     const uint32_t alo = wb + op_lo, ahi = wb + op_hi;                                                       \
-    const uint32_t sl = s_base + st * (T5_BM * 4u) + r16 * 4u;                                               \
+    const uint32_t sl = s_base + st * (T5_AS * 4u) + r16 * 4u;                                               \
     const uint32_t cl = c_base + par * 1024u + kb * 4u;
 #define T5_ADVANCE() st = st == 2u ? 0u : st + 1u
-/* A block of a consumer with N live row groups (N a constant, 1..8): straight-line code without a
+/* A block of a consumer with N live row groups (N a constant, 1..9): straight-line code without a
  * condition in it, so no value is ever copied between registers. Per-channel mode: the scales are outside
  * the K reduction, so the matrix unit accumulates straight through; block mode: one scaled add per 128-k
  * block, and the scaled adds of group RG follow the matrix instructions of group RG + 1, never wait for
@@ -123,9 +125,9 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
             sc[(RG) & 1][1] = as_[(RG) % 3] * ws1;                                                           \
         }                                                                                                    \
         if ((RG) + 2 < (N)) {                                                                                \
-            bl[((RG) + 2) % 3] = ds_read16<(((RG) + 2) & 7) * 2048u>(blo);                                   \
-            bh[((RG) + 2) % 3] = ds_read16<(((RG) + 2) & 7) * 2048u>(bhi);                                   \
-            if (!PC) as_[((RG) + 2) % 3] = ds_read4<(((RG) + 2) & 7) * 64u>(sl);                             \
+            bl[((RG) + 2) % 3] = ds_read16<((RG) + 2) * 2048u>(blo);                                         \
+            bh[((RG) + 2) % 3] = ds_read16<((RG) + 2) * 2048u>(bhi);                                         \
+            if (!PC) as_[((RG) + 2) % 3] = ds_read4<((RG) + 2) * 64u>(sl);                                   \
         }                                                                                                    \
         const v8i b = __builtin_shufflevector(bl[(RG) % 3], bh[(RG) % 3], 0, 1, 2, 3, 4, 5, 6, 7);           \
         if (PC) {                                                                                            \
@@ -183,7 +185,8 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
     T5_GROUP_N(5, N) T5_SCALE_N(4, N)                                                                        \
     T5_GROUP_N(6, N) T5_SCALE_N(5, N)                                                                        \
     T5_GROUP_N(7, N) T5_SCALE_N(6, N)                                                                        \
-    T5_SCALE_N(7, N)
+    T5_GROUP_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0) T5_SCALE_N(7, N)                                          \
+    T5_SCALE_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0)
 /* the K loop of a tile for a consumer wave with N live groups (BODY empty: it only keeps the barriers) */
 #define T5_RUN_BLOCKS(BODY)                                                                                  \
     for (uint32_t kb = 0; kb < KB; kb++) {                                                                   \
@@ -191,7 +194,7 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
         _Pragma("unroll") for (uint32_t sub = 0; sub < SUBS; sub++) {                                        \
             const uint32_t cw = cw0 + sub;                                                                   \
             (void)cw;                                                                                        \
-            v4f(&acc)[8][2] = accs[sub];                                                                     \
+            v4f(&acc)[NG][2] = accs[sub];                                                                 \
             (void)acc;                                                                                       \
             BODY                                                                                             \
         }                                                                                                    \
@@ -203,8 +206,10 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
  * two of the eight consumers' shares one after the other in every block, for callers whose launch shape
  * is fixed at 512 threads). The body takes its LDS as a pointer so that it can also sit in a kernel
  * with static LDS. */
-template <bool GLU, bool PC, uint32_t NCW>
+/* NG: 16-row groups a tile may hold, 8 or 9 (see t5_nine_groups below). */
+template <bool GLU, bool PC, uint32_t NCW, int NG = 8>
 __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
+    static_assert(NG == 8 || NG == 9, "a tile is eight or nine 16-row groups");
     T5Lds& L = *(T5Lds*)lds_raw;
     constexpr uint32_t BN = GLU ? 128u : 256u; /* output channels per tile */
     constexpr uint32_t NTHR = (NCW + 4u) * 64u, SUBS = 8u / NCW;
@@ -215,14 +220,16 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     const uint32_t NT = (g.N + BN - 1u) / BN;
     const uint32_t r16 = lane & 15u, q = lane >> 4;
 
-    /* ---- tile directory: inclusive prefix of ceil(cnt / 128) over experts, in LDS (the scan
+    /* rows a tile may hold */
+    const uint32_t cap = 16u * (uint32_t)NG;
+    /* ---- tile directory: inclusive prefix of ceil(cnt / cap) over experts, in LDS (the scan
      *      scratch borrows the ring, which is idle here) ---- */
     {
         uint32_t* scan = (uint32_t*)&L.a[0][0];
         uint32_t carry = 0;
         for (uint32_t e0 = 0; e0 < g.E; e0 += NTHR) {
             const uint32_t e = e0 + tid;
-            const uint32_t t = e < g.E ? ((uint32_t)g.meta[g.E + e] + T5_BM - 1u) / T5_BM : 0u;
+            const uint32_t t = e < g.E ? ((uint32_t)g.meta[g.E + e] + cap - 1u) / cap : 0u;
             scan[tid] = t;
             __syncthreads();
             for (uint32_t o = 1; o < NTHR; o <<= 1) {
@@ -231,7 +238,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 scan[tid] += v;
                 __syncthreads();
             }
-            if (e < g.E) L.prefix[e] = carry + scan[tid];
+            if (e < g.E) L.prefix[e] = (uint16_t)(carry + scan[tid]);
             carry += scan[NTHR - 1u];
             __syncthreads();
         }
@@ -247,7 +254,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 *(uint2*)((bf16_t*)g.out + (size_t)(r0 + i / (g.N / 4u)) * g.N + (i % (g.N / 4u)) * 4u) = make_uint2(0u, 0u);
         }
     }
-    const uint32_t total = L.prefix[g.E - 1u] * NT;
+    const uint32_t total = (uint32_t)L.prefix[g.E - 1u] * NT;
     const uint32_t K = g.K, KB = K / 128u;
     const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]);
     const uint32_t s_base = lds_off(&L.as[0][0]), c_base = lds_off(&L.wsc[0][0][0]);
@@ -275,11 +282,11 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         uint32_t lo = 0, hi = g.E - 1u; /* first expert whose inclusive prefix exceeds mt_global */
         while (lo < hi) {
             const uint32_t mid = (lo + hi) >> 1;
-            if (L.prefix[mid] > mt_global) hi = mid; else lo = mid + 1u;
+            if ((uint32_t)L.prefix[mid] > mt_global) hi = mid; else lo = mid + 1u;
         }
         Tile t;
         t.e = (uint32_t)__builtin_amdgcn_readfirstlane((int)lo);
-        const uint32_t pbase = t.e ? L.prefix[t.e - 1u] : 0u, Me = L.prefix[t.e] - pbase;
+        const uint32_t pbase = t.e ? (uint32_t)L.prefix[t.e - 1u] : 0u, Me = (uint32_t)L.prefix[t.e] - pbase;
         const uint32_t idx = tile - pbase * NT;
         uint32_t mt_v, nt_v;
         if (idx < FC * Me * 16u) {
@@ -292,8 +299,13 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         const uint32_t mt = (uint32_t)__builtin_amdgcn_readfirstlane((int)mt_v);
         t.nt = (uint32_t)__builtin_amdgcn_readfirstlane((int)nt_v);
         const uint32_t cnt = (uint32_t)g.meta[g.E + t.e];
-        t.r0 = (uint32_t)g.meta[t.e] + mt * T5_BM;
-        t.rows = cnt - mt * T5_BM < T5_BM ? cnt - mt * T5_BM : T5_BM; /* live rows of the tile */
+        /* nine-group kernels split the expert's rows evenly over its Me = ceil(cnt / cap) tiles, in whole 16-row
+         * groups: a tile takes nine groups only where that saves a tile; eight-group kernels fill 128-row tiles
+         * and leave the rest to the last one */
+        const uint32_t Mu = (uint32_t)__builtin_amdgcn_readfirstlane((int)Me);
+        const uint32_t h = NG == 8 ? 128u : (((cnt + Mu - 1u) / Mu + 15u) / 16u) * 16u; /* <= cap since cnt <= cap * Me */
+        t.r0 = (uint32_t)g.meta[t.e] + mt * h;
+        t.rows = cnt - mt * h < h ? cnt - mt * h : h; /* live rows of the tile */
         /* block mode: {gate, up, down} tables; per-channel mode: {gate_up fused [2N][K], down} */
         t.wp0 = PC ? g.wtab[(size_t)t.e * 2u + (GLU ? 0u : 1u)] : g.wtab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
         if (GLU && !PC && g.wtab[(size_t)t.e * 3u + 1u] == 0ull) t.wp0 = 0ull; /* gate without up: not resident */
@@ -320,7 +332,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         struct Src {
             /* per-lane 32-bit byte offsets from uniform bases: the loads take (scalar base + k offset,
              * vector offset) */
-            uint32_t aoff[4], woff[8], sstep;
+            uint32_t aoff[5], woff[8], sstep;
+            uint32_t nine; /* this loader has a ninth-group load in this tile (loaders 0 and 1, tiles of more than 128 rows) */
             const float* ssrc;
             const uint8_t *W0, *W1;
         };
@@ -329,14 +342,16 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
          * flight while the loader keeps feeding the tile before: fetch() only issues loads, finish()
          * uses them a few blocks later. Rows below the live count always hold a token. */
         struct Pre {
-            uint32_t tok[4], stok, eidx;
+            uint32_t tok[5], stok, eidx;
             float w0, w1, egate;
         };
         auto fetch = [&](const Tile& t, Pre& P) {
             const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
 #pragma unroll
-            for (uint32_t i = 0; i < 4u; i++) { /* token rows 32 * cw + 8 * i + lr; a pad row reads the first row */
-                const uint32_t row = 32u * cw + 8u * i + lr;
+            for (uint32_t i = 0; i < 5u; i++) { /* token rows 32 * cw + 8 * i + lr, and for loaders 0 and 1 rows
+                                                 * 128 + 8 * cw + lr of the ninth group; a pad row reads the first row */
+                if (i == 4u && cw >= 2u) { P.tok[i] = 0u; continue; }
+                const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * cw + lr;
                 const uint32_t ar = r0 + (row < rows ? row : 0u);
                 if (GLU) {
                     P.tok[i] = g.row_token[ar];
@@ -348,7 +363,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 }
             }
             {
-                const uint32_t row = (cw & 1u) * 64u + lane; /* the row whose activation scale this lane loads */
+                const uint32_t row = (cw < 3u ? cw : 0u) * 64u + lane; /* the row whose activation scale this lane loads */
                 /* per-channel mode has one activation scale per row, applied in the epilogue: its ring slot
                  * carries zeros */
                 P.eidx = row < rows ? (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
@@ -369,11 +384,12 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         auto finish = [&](const Tile& t, const Pre& P, uint32_t par, Src& S) {
             const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
             S.W0 = (const uint8_t*)(uintptr_t)t.wp0;
+            S.nine = (cw < 2u && rows > 128u) ? 1u : 0u;
             S.W1 = !GLU ? S.W0 : PC ? S.W0 + (size_t)g.N * K /* up rows follow the N gate rows */
                                : (const uint8_t*)(uintptr_t)g.wtab[(size_t)t.e * 3u + 1u];
 #pragma unroll
-            for (uint32_t i = 0; i < 4u; i++) {
-                const uint32_t row = 32u * cw + 8u * i + lr;
+            for (uint32_t i = 0; i < 5u; i++) {
+                const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * (cw & 1u) + lr;
                 const uint32_t src = (GLU && P.tok[i] == PLOW_EXPERT_UNUSED) ? 0u : P.tok[i];
                 S.aoff[i] = src * K + ((p ^ ((row >> 1) & 7u)) << 4);
             }
@@ -389,10 +405,10 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 }
                 S.woff[i] = ch * K + ((p ^ ((R >> 1) & 7u)) << 4);
             }
-            /* activation scale of row (cw & 1) * 64 + lane (loaders 0, 2 and 1, 3 load the same 64
-             * values); a pad row reads tilep[0], which is always 0 */
+            /* activation scale of row 64 * cw + lane (loader 3 repeats loader 0's 64 values); a pad row
+             * reads tilep[0], which is always 0 */
             {
-                const uint32_t row = (cw & 1u) * 64u + lane;
+                const uint32_t row = (cw < 3u ? cw : 0u) * 64u + lane;
                 const bool ok = P.stok != PLOW_EXPERT_UNUSED;
                 if (GLU) {
                     S.ssrc = ok ? g.a_scale + P.stok : (const float*)(g.meta + 2u * g.E);
@@ -412,15 +428,15 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 L.wsc[par][1][i] = P.w1;
             }
             /* what the consumers' epilogue needs per row, so that it does not start with a round trip to
-             * memory: loaders 0 and 1 hold rows 0..63 and 64..127 */
-            if (cw < 2u) {
+             * memory: loaders 0, 1 and 2 hold rows 0..63, 64..127 and 128..191 */
+            if (cw < 3u) {
                 L.epi_idx[par][cw * 64u + lane] = P.eidx;
                 if (!GLU) L.epi_gate[par][cw * 64u + lane] = P.egate;
             }
         };
         auto issue = [&](const Src& S, uint32_t kb, uint32_t st) {
             __builtin_amdgcn_global_load_lds((const void*)(S.ssrc + (size_t)kb * S.sstep),
-                                             (lds_void*)&L.as[st][(cw & 1u) * 64u], 4, 0, 0);
+                                             (lds_void*)&L.as[st][(cw < 3u ? cw : 0u) * 64u], 4, 0, 0);
             const uint8_t* const ak = A0 + (size_t)kb * 128u;
             const uint8_t* const wk0 = S.W0 + (size_t)kb * 128u;
             const uint8_t* const wk1 = S.W1 + (size_t)kb * 128u;
@@ -428,6 +444,9 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             for (uint32_t i = 0; i < 4u; i++)
                 __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[i]),
                                                  (lds_void*)&L.a[st][(32u * cw + 8u * i) * 128u], 16, 0, 0);
+            if (S.nine) /* the ninth group's rows */
+                __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[4]),
+                                                 (lds_void*)&L.a[st][(128u + 8u * cw) * 128u], 16, 0, 0);
 #pragma unroll
             for (uint32_t i = 0; i < 8u; i++)
                 __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + S.woff[i]),
@@ -456,7 +475,11 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 /* loads return in order: block kb has landed once at most the next block's loads (of this
                  * tile or the next) are outstanding. After the barrier the consumers are done with the
                  * block before kb, whose slot takes the block two ahead. */
-                if (kb + 1u < KB || more) LOADER_BARRIER(T5_NLOAD); else LOADER_BARRIER(0);
+                if (kb + 1u < KB || more) { /* the loads that may stay outstanding are those of the block after kb */
+                    if (kb + 1u < KB ? cur.nine : nxt.nine) LOADER_BARRIER(T5_NLOAD + 1); else LOADER_BARRIER(T5_NLOAD);
+                } else {
+                    LOADER_BARRIER(0);
+                }
                 const uint32_t st2 = st >= 1u ? st - 1u : 2u; /* (st + 2) % 3 */
                 /* not before this barrier: until it, the consumers may still be in the epilogue of the tile
                  * before, reading the L.epi_* half that finish() overwrites */
@@ -484,11 +507,11 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             /* DOWN: N may end mid-tile (N is a multiple of 128, so a wave's consumers are in or out together) */
             const bool wave_on = (GLU ? nt * 128u + 16u * cw0 : nt * 256u + 32u * cw0) < g.N;
             const uint32_t ngrp_w = wave_on ? ngrp : 0u;
-            v4f accs[SUBS][8][2];
+            v4f accs[SUBS][NG][2];
 #pragma unroll
             for (uint32_t sub = 0; sub < SUBS; sub++)
 #pragma unroll
-                for (int rg = 0; rg < 8; rg++)
+                for (int rg = 0; rg < NG; rg++)
 #pragma unroll
                     for (int x = 0; x < 2; x++) accs[sub][rg][x] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             /* One form of the block loop per count of live row groups: each is straight-line code. The
@@ -496,6 +519,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
              * placing waits of its own inside the loops, whose LDS reads it does not see. */
             __builtin_amdgcn_s_waitcnt(0xc07f); /* lgkmcnt(0) */
             switch (ngrp_w) {
+                case 9u: if constexpr (NG == 9) { T5_RUN_BLOCKS(T5_BLOCK_N(9)) } break;
                 case 8u: { T5_RUN_BLOCKS(T5_BLOCK_N(8)) } break;
                 case 7u: { T5_RUN_BLOCKS(T5_BLOCK_N(7)) } break;
                 case 6u: { T5_RUN_BLOCKS(T5_BLOCK_N(6)) } break;
@@ -519,13 +543,13 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
 #pragma unroll
                 for (uint32_t sub = 0; sub < SUBS; sub++) {
                     const uint32_t cw = cw0 + sub, ch0 = nt * 128u + 16u * cw;
-                    v4f(&acc)[8][2] = accs[sub];
+                    v4f(&acc)[NG][2] = accs[sub];
 #pragma unroll
-                    for (int rg = 0; rg < 8; rg++) {
+                    for (int rg = 0; rg < NG; rg++) {
                         const uint32_t row = 16u * (uint32_t)rg + r16;
                         bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
                         if (row >= rows) {
-                            if (erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u);
+                            if (erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
                             continue;
                         }
                         uint2 pk = make_uint2(0u, 0u);
@@ -540,13 +564,18 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     }
                 }
             } else if (!PC && GLU) {
-                float v[SUBS][8][4];
+                float v[SUBS][NG][4];
+                /* The row maxima of the eight consumers meet in the ring stage the tile has just left: consumer
+                 * x writes its own into the head of its own weight slice there (nobody else reads that slice,
+                 * and it is done with it), everyone reads all eight after the barrier; the loaders refill the
+                 * stage only after the next tile's first barrier. */
+                auto red = [&](uint32_t x) -> float* { return (float*)&L.w[stl][x * (32u * 128u)]; };
 #pragma unroll
                 for (uint32_t sub = 0; sub < SUBS; sub++) {
                     const uint32_t cw = cw0 + sub;
-                    v4f(&acc)[8][2] = accs[sub];
+                    v4f(&acc)[NG][2] = accs[sub];
 #pragma unroll
-                    for (int rg = 0; rg < 8; rg++) {
+                    for (int rg = 0; rg < NG; rg++) {
                         float m = 0.0f;
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
@@ -555,9 +584,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                         }
                         m = fmaxf(m, __shfl_xor(m, 16, 64));
                         m = fmaxf(m, __shfl_xor(m, 32, 64));
-                        /* L.red of the tile before has been read by everyone: its readers have passed this
-                         * tile's block barriers since */
-                        if (q == 0) L.red[cw][16u * (uint32_t)rg + r16] = m;
+                        if (q == 0) red(cw)[16u * (uint32_t)rg + r16] = m;
                     }
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -565,12 +592,12 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 for (uint32_t sub = 0; sub < SUBS; sub++) {
                     const uint32_t cw = cw0 + sub, ch0 = nt * 128u + 16u * cw;
 #pragma unroll
-                    for (int rg = 0; rg < 8; rg++) {
+                    for (int rg = 0; rg < NG; rg++) {
                         const uint32_t row = 16u * (uint32_t)rg + r16;
                         if (row >= rows || L.epi_idx[par][row] == PLOW_EXPERT_UNUSED) continue;
                         float amax = 1e-10f;
 #pragma unroll
-                        for (int x = 0; x < 8; x++) amax = fmaxf(amax, L.red[x][row]);
+                        for (int x = 0; x < 8; x++) amax = fmaxf(amax, red((uint32_t)x)[row]);
                         const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
                         uint8_t* orow = (uint8_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
                         *(uint32_t*)orow = cvt4_e4m3(v[sub][rg][0] * inv, v[sub][rg][1] * inv, v[sub][rg][2] * inv, v[sub][rg][3] * inv);
@@ -583,7 +610,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 for (uint32_t sub = 0; sub < SUBS; sub++) {
                     const uint32_t cw = cw0 + sub;
                     const uint32_t ch0 = GLU ? nt * 128u + 16u * cw : nt * 256u + 32u * cw; /* first channel */
-                    v4f(&acc)[8][2] = accs[sub];
+                    v4f(&acc)[NG][2] = accs[sub];
                     /* DOWN, f32 partials: a row's 32 channels of this consumer are one 128-byte line. A 16-row
                      * group goes through LDS once so that it leaves as two stores of 8 whole lines (8 consecutive
                      * lanes per line) instead of two stores that touch 16 half lines each. The staging area is
@@ -633,7 +660,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                         const uint32_t padded = ((cnt_e + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
                         if (wave_on && !GLU) {
 #pragma unroll
-                            for (int rg = 0; rg < 8; rg++) {
+                            for (int rg = 0; rg < NG; rg++) {
                                 if (16u * (uint32_t)rg >= rows) break; /* uniform */
                                 const uint32_t row = 16u * (uint32_t)rg + r16;
                                 const float gate = L.epi_gate[par][row]; /* 0 for pad rows */
@@ -652,11 +679,11 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                             }
                         } else if (wave_on) {
 #pragma unroll
-                            for (int rg = 0; rg < 8; rg++) {
+                            for (int rg = 0; rg < NG; rg++) {
                                 const uint32_t row = 16u * (uint32_t)rg + r16;
                                 bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
                                 if (row >= rows) {
-                                    if (erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u);
+                                    if (erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
                                     continue;
                                 }
                                 const uint32_t tok = L.epi_idx[par][row];
@@ -680,7 +707,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                         /* fused combine: add into the bf16 output row of the slot's token */
                         typedef short bf16x2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
-                        for (int rg = 0; rg < 8; rg++) {
+                        for (int rg = 0; rg < NG; rg++) {
                             const uint32_t row = 16u * (uint32_t)rg + r16;
                             if (row >= rows) continue;
                             const uint32_t pidx = L.epi_idx[par][row];
@@ -698,14 +725,14 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                         }
                     } else if (wave_on && (g.det_k || !g.part16)) {
 #pragma unroll
-                        for (int rg = 0; rg < 8; rg++) {
+                        for (int rg = 0; rg < NG; rg++) {
                             if (16u * (uint32_t)rg >= rows) break; /* uniform */
                             const float gate = L.epi_gate[par][16u * (uint32_t)rg + r16]; /* 0 for pad rows */
                             down_store_f32(rg, acc[rg][0] * gate, acc[rg][1] * gate);
                         }
                     } else if (wave_on) {
 #pragma unroll
-                        for (int rg = 0; rg < 8; rg++) {
+                        for (int rg = 0; rg < NG; rg++) {
                             const uint32_t row = 16u * (uint32_t)rg + r16;
                             if (row >= rows) continue;
                             const uint32_t pidx = L.epi_idx[par][row];
@@ -728,32 +755,35 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         }
     }
 }
-template <bool GLU, bool PC, uint32_t NCW>
+template <bool GLU, bool PC, uint32_t NCW, int NG>
 __global__ __launch_bounds__((NCW + 4u) * 64u) void k_group_w8a8_tiled(GroupW8A8 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    t5_body<GLU, PC, NCW>(g, lds_raw);
+    t5_body<GLU, PC, NCW, NG>(g, lds_raw);
 }
 
 
 /* dynamic-LDS limits, once per device (plow_moe_device_setup) */
-template <bool GLU, bool PC, uint32_t NCW>
+template <bool GLU, bool PC, uint32_t NCW, int NG>
 static bool t5_set_attr() {
-    return hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU, PC, NCW>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    return hipFuncSetAttribute((const void*)k_group_w8a8_tiled<GLU, PC, NCW, NG>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)sizeof(T5Lds)) == hipSuccess;
 }
+template <uint32_t NCW, int NG>
+static bool t5_set_attrs() {
+    return t5_set_attr<true, false, NCW, NG>() && t5_set_attr<false, false, NCW, NG>() && t5_set_attr<true, true, NCW, NG>() &&
+           t5_set_attr<false, true, NCW, NG>();
+}
 int plow_moe_w8a8_tiled_setup() {
-    const bool ok = t5_set_attr<true, false, 8u>() && t5_set_attr<false, false, 8u>() && t5_set_attr<true, true, 8u>() &&
-                    t5_set_attr<false, true, 8u>() && t5_set_attr<true, false, 4u>() && t5_set_attr<false, false, 4u>() &&
-                    t5_set_attr<true, true, 4u>() && t5_set_attr<false, true, 4u>();
+    const bool ok = t5_set_attrs<8u, 8>() && t5_set_attrs<8u, 9>() && t5_set_attrs<4u, 8>();
     return ok ? 0 : PLOW_MOE_EDEVICE;
 }
 
 /* Persistent launch: one workgroup per CU; the tile count is computed on the device from meta. */
-template <bool GLU, bool PC, uint32_t NCW>
+template <bool GLU, bool PC, uint32_t NCW, int NG>
 static int launch_tiled_t(const GroupW8A8& g, hipStream_t st) {
     const uint32_t n_cu = plow_moe_n_cu();
     if (!n_cu) return PLOW_MOE_EDEVICE;
-    k_group_w8a8_tiled<GLU, PC, NCW><<<n_cu, (NCW + 4u) * 64u, sizeof(T5Lds), st>>>(g);
+    k_group_w8a8_tiled<GLU, PC, NCW, NG><<<n_cu, (NCW + 4u) * 64u, sizeof(T5Lds), st>>>(g);
     return 0;
 }
 
@@ -764,11 +794,22 @@ bool group_w8a8_tiled_serves(const GroupW8A8& g) {
            g.K <= 128u * 128u && g.N >= 256u;
 }
 
+/* Tiles of nine 16-row groups (144 rows) instead of eight: the ninth group saves an expert with 129..144
+ * rows (257..288, ...) a whole second tile, i.e. a second pass over its weight rows. That pays when the
+ * weights are the traffic: an expert's matrix of this op is larger than an XCD's 4 MB L2, so a second row
+ * tile fetches it again (DeepSeek-V3 shape at 4096 tokens, 128 rows per expert on average: GLU 2030 ->
+ * 1818 us). Where they are not (plow's own prefill bench shape: 1 - 2 MB per expert) the larger
+ * accumulator only costs registers (+5 %), so those shapes keep eight groups. */
+static bool t5_nine_groups(const GroupW8A8& g, bool glu) {
+    return (uint64_t)(glu ? 2u : 1u) * g.N * g.K > (4ull << 20);
+}
+
 template <bool GLU>
 static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
     if (!group_w8a8_tiled_serves(g)) return PLOW_MOE_EINVAL;
-    if (plow_moe_tuning().tile_waves4) return g.per_channel ? launch_tiled_t<GLU, true, 4u>(g, st) : launch_tiled_t<GLU, false, 4u>(g, st);
-    return g.per_channel ? launch_tiled_t<GLU, true, 8u>(g, st) : launch_tiled_t<GLU, false, 8u>(g, st);
+    if (plow_moe_tuning().tile_waves4) return g.per_channel ? launch_tiled_t<GLU, true, 4u, 8>(g, st) : launch_tiled_t<GLU, false, 4u, 8>(g, st);
+    if (t5_nine_groups(g, GLU)) return g.per_channel ? launch_tiled_t<GLU, true, 8u, 9>(g, st) : launch_tiled_t<GLU, false, 8u, 9>(g, st);
+    return g.per_channel ? launch_tiled_t<GLU, true, 8u, 8>(g, st) : launch_tiled_t<GLU, false, 8u, 8>(g, st);
 }
 
 int launch_group_glu_w8a8_tiled(const GroupW8A8& g, hipStream_t st) { return launch_tiled<true>(g, st); }

@@ -231,3 +231,37 @@ def test_deterministic_fused_combine(moe, oracle, T):
     host = synth.to_host(dd)
     run_oracle(oracle, det, host)
     assert_output_close(runs[0][1], host.np("out"), f"det combine T={T} out")
+
+
+def test_tiled_glu_silu_against_the_streaming_form(moe, oracle):
+    """The tiled form's GLU epilogue takes SiLU from the hardware exp2 / reciprocal, the streaming form from
+    expf and an IEEE division (plow's choice, runtime/amd/op_moe.h:209-215). Both forms accumulate the same
+    matrix products in the same order, so running op 188 (bf16 intermediate) once per form over the same
+    rows isolates that difference: how many bf16 values differ, and by how many steps. The form is picked
+    through the routed-slot count in the descriptor (many slots: tiled; one slot: streaming, which is correct
+    at every row count)."""
+    T = 700
+    print(f"[case] tiled vs streaming SiLU T={T}", flush=True)
+    cfg = layer.MoeConfig("mini-atomic", H=512, E=32, I=256, k=4, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          n_group=4, topk_group=2, route_scale=2.5, enc="fp8blk", arm="w8a8atomic", n_shared=1,
+                          shared_mode="fold", act=1)
+    plan, dev, host = both(moe, oracle, cfg, seed=5)
+    rows = assert_routing_equal(plan, dev, host)
+    glu = plan.insts[plan.index("glu")]
+    assert glu.fj[2].u >= 16 * (cfg.E + 1)                       # the run above took the tiled form
+    tiled = dev.np("fu")[:rows].copy()
+    dev.t["fu"].zero_()
+    one = abi.PlowDevInst.from_buffer_copy(glu)
+    one.fj[2].u = 1
+    moe.exec(one, dev.table())
+    torch.cuda.synchronize()
+    stream = dev.np("fu")[:rows].copy()
+    live = host.np("row_partidx")[:rows] != abi.EXPERT_UNUSED
+    a, b = tiled[live].astype(np.int32), stream[live].astype(np.int32)
+    # bf16 bit patterns of one sign are ordered like the values: the difference of the patterns counts steps
+    same_sign = (a >> 15) == (b >> 15)
+    steps = np.where(same_sign, np.abs(a - b), (a & 0x7FFF) + (b & 0x7FFF))
+    frac = float((steps != 0).mean())
+    print(f"[parity] tiled vs streaming bf16 intermediate: {frac * 100:.4f} % of {steps.size} values differ, "
+          f"max {int(steps.max())} step(s)", flush=True)
+    assert frac <= 1e-3 and steps.max() <= 1
