@@ -685,10 +685,50 @@ static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
     return launch_a16_dma_rg<ENC, GLU, 1>(g, grid, st);
 }
 
+/* Many rows per expert (16 and more on average): the fp8-weight arms run on the tiled kernel (loader and
+ * consumer waves, 128-row tiles, weights decoded to bf16 in registers), which reads an expert's weights
+ * once per 128 rows instead of once per 64 and each operand from LDS once per tile. It serves the table
+ * layouts plow's ops use: block fp8 {gate, up, down} and per-channel fp8 {gate_up fused, down}; GLU gathers
+ * its rows through a_idx (and may scatter through o_idx in per-channel mode: the slot-major ops), DOWN
+ * reads aligned rows or, slot-major, the rows a_idx = o_idx names. Returns false when the call is not
+ * of that kind (the streaming forms then serve it). */
+template <bool GLU>
+static bool a16_tiled_try(const GroupA16& g, hipStream_t st, int* rc) {
+    if (!plow_moe_tuning().a16_tiled || !g.meta || g.bias || g.wmul > 1u || !g.stab || g.dense_rows) return false;
+    if (g.slots_hint < 16u * g.E) return false;
+    const bool pc = g.enc == AENC_FP8PC;
+    if (!pc && g.enc != AENC_FP8BLK) return false;
+    if (g.wrow0) return false;
+    if (pc) {
+        if (g.wcols != 2u || (GLU ? (g.wsel0 != 0u || g.wsel1 != 0u || g.wrow1 != g.N) : g.wsel0 != 1u)) return false;
+    } else {
+        if (g.wcols != 3u || g.wrow1 || (GLU ? (g.wsel0 != 0u || g.wsel1 != 1u) : g.wsel0 != 2u)) return false;
+    }
+    GroupW8A8 w = {};
+    w.out = g.out, w.a = g.a, w.wtab = g.wtab, w.stab = g.stab, w.meta = g.meta;
+    w.N = g.N, w.K = g.K, w.E = g.E, w.act = g.act, w.f0 = g.f0, w.f1 = g.f1;
+    w.per_channel = pc ? 1u : 0u;
+    if (GLU) {
+        if (!g.a_idx || (g.o_idx && !pc)) return false;
+        w.row_token = g.a_idx, w.row_partidx = g.o_idx, w.out_bf16 = 1u;
+    } else {
+        if (!g.o_idx || !g.gate || (g.a_idx && g.a_idx != g.o_idx)) return false;
+        w.row_partidx = g.o_idx, w.row_gate = g.gate, w.part16 = g.out_bf16;
+        w.a_slots = g.a_idx ? g.slots_hint : 0u;
+    }
+    if (!group_w8a8_tiled_serves(w)) return false;
+    *rc = launch_group_a16_tiled(w, GLU, st);
+    return true;
+}
+
 template <bool GLU>
 static int launch_a16(const GroupA16& g, hipStream_t st) {
     if (g.N == 0 || g.K == 0 || g.E == 0 || g.N % AK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
     if ((uint64_t)g.E * (g.N / AK_BN) > 0x7FFFFFFFull) return PLOW_MOE_EINVAL;
+    {
+        int rc = 0;
+        if (a16_tiled_try<GLU>(g, st, &rc)) return rc;
+    }
     const dim3 grid(g.E * (g.N / AK_BN));
     /* second form: needs whole steps of K (one 128-byte line per weight row) and the block scales of a
      * tile to fit its LDS table */

@@ -91,6 +91,12 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
     asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
     return r;
 }
+template <uint32_t OFF>
+__device__ __forceinline__ v2i ds_read8(uint32_t addr) {
+    v2i r;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+    return r;
+}
 /* all ds_reads issued so far have returned */
 #define LDS_WAIT_ALL() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
 #define WG_BARRIER() asm volatile("s_barrier" ::: "memory")
@@ -187,6 +193,87 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
     T5_GROUP_N(7, N) T5_SCALE_N(6, N)                                                                        \
     T5_GROUP_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0) T5_SCALE_N(7, N)                                          \
     T5_SCALE_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0)
+/* ---- the same block with bf16 activations (A16): a block is 64 k. Token rows are 128 bytes of bf16
+ *      (same stage geometry and swizzle as the fp8 rows), weight rows 64 bytes of e4m3 decoded to bf16 in
+ *      registers (exact: e4m3 fits bf16), v_mfma_f32_16x16x32_bf16 twice per operand pair. No activation
+ *      scales; block mode scales the block's product by the weight block scale (one per two blocks),
+ *      per-channel mode accumulates straight through. Weight row r16 of an operand holds its 8-byte piece
+ *      j at (j ^ 4 * ((r16 >> 2) & 1)): the 64 lanes of a read then touch every bank twice, the minimum
+ *      for 512 bytes. ---- */
+#define T5A_BLOCK_HEAD()                                                                                     \
+    const uint32_t ab = a_base + st * (T5_BM * 128u), wb = w_base + st * (256u * 128u) + cw * (32u * 64u);   \
+    const uint32_t b0 = ab + opb0, b1 = ab + opb1;                                                           \
+    const uint32_t cl = c_base + par * 1024u + (kb >> 1) * 4u;
+#define T5A_DECODE(R) t5a_decode(R)
+#define T5A_GROUP_N(RG, N)                                                                                   \
+    if ((RG) < (N)) {                                                                                        \
+        asm volatile("s_waitcnt lgkmcnt(%2)"                                                                 \
+                     : "+v"(bx[(RG) % 3][0]), "+v"(bx[(RG) % 3][1])                                          \
+                     : "n"((RG) + 1 < (N) ? 2 : 0));                                                         \
+        if ((RG) + 2 < (N)) {                                                                                \
+            bx[((RG) + 2) % 3][0] = ds_read16<((RG) + 2) * 2048u>(b0);                                       \
+            bx[((RG) + 2) % 3][1] = ds_read16<((RG) + 2) * 2048u>(b1);                                       \
+        }                                                                                                    \
+        const v8bf B0 = __builtin_bit_cast(v8bf, bx[(RG) % 3][0]), B1 = __builtin_bit_cast(v8bf, bx[(RG) % 3][1]); \
+        if (PC) {                                                                                            \
+            acc[RG][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[0][0], B0, acc[RG][0], 0, 0, 0);        \
+            acc[RG][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[1][0], B0, acc[RG][1], 0, 0, 0);        \
+            acc[RG][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[0][1], B1, acc[RG][0], 0, 0, 0);        \
+            acc[RG][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[1][1], B1, acc[RG][1], 0, 0, 0);        \
+        } else {                                                                                             \
+            const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};                                                          \
+            t[(RG) & 1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[0][0], B0, z, 0, 0, 0);             \
+            t[(RG) & 1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[1][0], B0, z, 0, 0, 0);             \
+            t[(RG) & 1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[0][1], B1, t[(RG) & 1][0], 0, 0, 0); \
+            t[(RG) & 1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[1][1], B1, t[(RG) & 1][1], 0, 0, 0); \
+        }                                                                                                    \
+    }
+#define T5A_SCALE_N(RG, N)                                                                                   \
+    if (!PC && (RG) < (N)) {                                                                                 \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                      \
+            acc[RG][0][i] = fmaf(t[(RG) & 1][0][i], ws0, acc[RG][0][i]);                                     \
+            acc[RG][1][i] = fmaf(t[(RG) & 1][1][i], ws1, acc[RG][1][i]);                                     \
+        }                                                                                                    \
+    }
+#define T5A_BLOCK_N(N)                                                                                       \
+    T5A_BLOCK_HEAD()                                                                                         \
+    float ws0 = 0.0f, ws1 = 0.0f;                                                                            \
+    if (!PC) {                                                                                               \
+        ws0 = ds_read4<0>(cl);                                                                               \
+        ws1 = ds_read4<512>(cl);                                                                             \
+    }                                                                                                        \
+    v2i ar[2][2];                                                                                            \
+    ar[0][0] = ds_read8<0>(wb + opa0), ar[0][1] = ds_read8<0>(wb + opa1);                                    \
+    ar[1][0] = ds_read8<1024>(wb + opa0), ar[1][1] = ds_read8<1024>(wb + opa1);                              \
+    v4i bx[3][2];                                                                                            \
+    bx[0][0] = ds_read16<0>(b0), bx[0][1] = ds_read16<0>(b1);                                                \
+    if ((N) > 1) bx[1][0] = ds_read16<2048u>(b0), bx[1][1] = ds_read16<2048u>(b1);                           \
+    asm volatile("s_waitcnt lgkmcnt(%6)"                                                                     \
+                 : "+v"(ar[0][0]), "+v"(ar[0][1]), "+v"(ar[1][0]), "+v"(ar[1][1]), "+v"(ws0), "+v"(ws1)      \
+                 : "n"((N) > 1 ? 4 : 2));                                                                    \
+    if (!GLU && !PC) ws0 = ws1 = ((cw & 4u) ? ws1 : ws0);                                                    \
+    v8bf aop[2][2];                                                                                          \
+    _Pragma("unroll") for (int x = 0; x < 2; x++)                                                            \
+        _Pragma("unroll") for (int k2 = 0; k2 < 2; k2++) aop[x][k2] = T5A_DECODE(ar[x][k2]);                 \
+    v4f t[2][2];                                                                                             \
+    T5A_GROUP_N(0, N)                                                                                        \
+    T5A_GROUP_N(1, N) T5A_SCALE_N(0, N)                                                                      \
+    T5A_GROUP_N(2, N) T5A_SCALE_N(1, N)                                                                      \
+    T5A_GROUP_N(3, N) T5A_SCALE_N(2, N)                                                                      \
+    T5A_GROUP_N(4, N) T5A_SCALE_N(3, N)                                                                      \
+    T5A_GROUP_N(5, N) T5A_SCALE_N(4, N)                                                                      \
+    T5A_GROUP_N(6, N) T5A_SCALE_N(5, N)                                                                      \
+    T5A_GROUP_N(7, N) T5A_SCALE_N(6, N)                                                                      \
+    T5A_GROUP_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0) T5A_SCALE_N(7, N)                                        \
+    T5A_SCALE_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0)
+/* eight e4m3 bytes -> eight bf16 (the hardware conversion is exact) */
+__device__ __forceinline__ v8bf t5a_decode(v2i r) {
+    const v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((uint32_t)r[0], 1.0f, false);
+    const v2bf p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((uint32_t)r[0], 1.0f, true);
+    const v2bf p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((uint32_t)r[1], 1.0f, false);
+    const v2bf p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((uint32_t)r[1], 1.0f, true);
+    return (v8bf){p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
 /* the K loop of a tile for a consumer wave with N live groups (BODY empty: it only keeps the barriers) */
 #define T5_RUN_BLOCKS(BODY)                                                                                  \
     for (uint32_t kb = 0; kb < KB; kb++) {                                                                   \
@@ -207,7 +294,9 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
  * is fixed at 512 threads). The body takes its LDS as a pointer so that it can also sit in a kernel
  * with static LDS. */
 /* NG: 16-row groups a tile may hold, 8 or 9 (see t5_nine_groups below). */
-template <bool GLU, bool PC, uint32_t NCW, int NG = 8>
+/* A16: `a` holds bf16 rows [..][K] (no activation scales) and a block is 64 k: the bf16-activation arms
+ * (block-fp8 weights: ops 85 / 86 arm 0; per-channel fp8 weights: ops 65 / 66). */
+template <bool GLU, bool PC, uint32_t NCW, int NG = 8, bool A16 = false>
 __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     static_assert(NG == 8 || NG == 9, "a tile is eight or nine 16-row groups");
     T5Lds& L = *(T5Lds*)lds_raw;
@@ -255,12 +344,20 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         }
     }
     const uint32_t total = (uint32_t)L.prefix[g.E - 1u] * NT;
-    const uint32_t K = g.K, KB = K / 128u;
+    const uint32_t K = g.K, KB = K / (A16 ? 64u : 128u); /* blocks of the K loop */
+    const uint32_t KS = K / 128u;                         /* weight block scales along K */
+    const uint32_t KA = A16 ? 2u * K : K;                 /* bytes of a token row */
     const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]);
     const uint32_t s_base = lds_off(&L.as[0][0]), c_base = lds_off(&L.wsc[0][0][0]);
     /* consumer: this lane's operand pieces 2q, 2q + 1 of row (16 * group + r16) */
     const uint32_t sw = (r16 >> 1) & 7u;
     const uint32_t op_lo = r16 * 128u + (((2u * q) ^ sw) << 4), op_hi = r16 * 128u + (((2u * q + 1u) ^ sw) << 4);
+    /* A16: this lane's 16-byte token pieces q and 4 + q (k 8q.. and 32 + 8q.. of the 64-k block), and its
+     * 8-byte weight pieces of row r16 */
+    const uint32_t opb0 = r16 * 128u + ((q ^ sw) << 4), opb1 = r16 * 128u + (((4u + q) ^ sw) << 4);
+    const uint32_t swa = ((r16 >> 2) & 1u) * 4u;
+    const uint32_t opa0 = r16 * 64u + ((q ^ swa) << 3), opa1 = r16 * 64u + (((4u + q) ^ swa) << 3);
+    (void)op_lo, (void)op_hi, (void)opb0, (void)opb1, (void)opa0, (void)opa1;
 
     /* Workgroup w runs on XCD w % 8 (round-robin dispatch), and each XCD has its own L2. The logical
      * index below makes the 32 workgroups of one XCD take 32 consecutive tiles of every sweep, and the
@@ -355,7 +452,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 const uint32_t ar = r0 + (row < rows ? row : 0u);
                 if (GLU) {
                     P.tok[i] = g.row_token[ar];
-                } else if (!PC && g.a_slots) { /* rows stored by routing slot: read the slot's row */
+                } else if (g.a_slots && (!PC || A16)) { /* rows stored by routing slot: read the slot's row */
                     const uint32_t slot = g.row_partidx[ar];
                     P.tok[i] = slot < g.a_slots ? slot : 0u;
                 } else {
@@ -367,7 +464,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 /* per-channel mode has one activation scale per row, applied in the epilogue: its ring slot
                  * carries zeros */
                 P.eidx = row < rows ? (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
-                P.stok = PC ? PLOW_EXPERT_UNUSED : P.eidx;
+                P.stok = (PC || A16) ? PLOW_EXPERT_UNUSED : P.eidx;
                 P.egate = (!GLU && row < rows) ? g.row_gate[r0 + row] : 0.0f;
             }
             /* weight block scales of the tile: GLU gate | up of channel block nt; DOWN blocks 2nt, 2nt + 1 */
@@ -376,9 +473,9 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
                 const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : S0;
                 const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
-                const uint32_t i = tid - NCW * 64u; /* 0..255 over the four loaders; KB <= 128 */
-                P.w0 = i < KB ? S0[(size_t)nb0 * KB + i] : 0.0f;
-                P.w1 = i < KB ? S1[(size_t)nb1 * KB + i] : 0.0f;
+                const uint32_t i = tid - NCW * 64u; /* 0..255 over the four loaders; KS <= 128 */
+                P.w0 = i < KS ? S0[(size_t)nb0 * KS + i] : 0.0f;
+                P.w1 = i < KS ? S1[(size_t)nb1 * KS + i] : 0.0f;
             }
         };
         auto finish = [&](const Tile& t, const Pre& P, uint32_t par, Src& S) {
@@ -391,11 +488,13 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             for (uint32_t i = 0; i < 5u; i++) {
                 const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * (cw & 1u) + lr;
                 const uint32_t src = (GLU && P.tok[i] == PLOW_EXPERT_UNUSED) ? 0u : P.tok[i];
-                S.aoff[i] = src * K + ((p ^ ((row >> 1) & 7u)) << 4);
+                S.aoff[i] = src * KA + ((p ^ ((row >> 1) & 7u)) << 4);
             }
 #pragma unroll
             for (uint32_t i = 0; i < 8u; i++) { /* LDS weight rows R = 64 * cw + 8 * i + lr: consumer R / 32, group (R / 16) & 1 */
-                const uint32_t R = 64u * cw + 8u * i + lr;
+                if (A16 && i >= 4u) { S.woff[i] = 0u; continue; }
+                /* A16: a load covers 16 rows x 64 B, lane -> (row l >> 2, 16-byte slot l & 3) */
+                const uint32_t R = A16 ? 64u * cw + 16u * i + (lane >> 2) : 64u * cw + 8u * i + lr;
                 uint32_t ch;
                 if (GLU) {
                     ch = nt * 128u + 16u * (R >> 5) + (R & 15u);
@@ -403,7 +502,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     ch = nt * 256u + R;
                     if (ch >= g.N) ch = 0; /* past the last channel: any valid row, never stored */
                 }
-                S.woff[i] = ch * K + ((p ^ ((R >> 1) & 7u)) << 4);
+                S.woff[i] = A16 ? ch * K + (((lane & 3u) ^ (((R >> 2) & 1u) << 1)) << 4) : ch * K + ((p ^ ((R >> 1) & 7u)) << 4);
             }
             /* activation scale of row 64 * cw + lane (loader 3 repeats loader 0's 64 values); a pad row
              * reads tilep[0], which is always 0 */
@@ -413,7 +512,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 if (GLU) {
                     S.ssrc = ok ? g.a_scale + P.stok : (const float*)(g.meta + 2u * g.E);
                     S.sstep = ok ? g.pitch : 0u;
-                } else if (!PC && g.a_slots) { /* scales [KB][a_slots], by slot */
+                } else if (!PC && !A16 && g.a_slots) { /* scales [KB][a_slots], by slot */
                     const bool in = ok && P.stok < g.a_slots;
                     S.ssrc = in ? g.a_scale + P.stok : (const float*)(g.meta + 2u * g.E);
                     S.sstep = in ? g.a_slots : 0u;
@@ -423,7 +522,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 }
             }
             const uint32_t i = tid - NCW * 64u;
-            if (i < KB) {
+            if (i < KS) {
                 L.wsc[par][0][i] = P.w0;
                 L.wsc[par][1][i] = P.w1;
             }
@@ -435,11 +534,12 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             }
         };
         auto issue = [&](const Src& S, uint32_t kb, uint32_t st) {
-            __builtin_amdgcn_global_load_lds((const void*)(S.ssrc + (size_t)kb * S.sstep),
-                                             (lds_void*)&L.as[st][(cw < 3u ? cw : 0u) * 64u], 4, 0, 0);
+            if (!A16)
+                __builtin_amdgcn_global_load_lds((const void*)(S.ssrc + (size_t)kb * S.sstep),
+                                                 (lds_void*)&L.as[st][(cw < 3u ? cw : 0u) * 64u], 4, 0, 0);
             const uint8_t* const ak = A0 + (size_t)kb * 128u;
-            const uint8_t* const wk0 = S.W0 + (size_t)kb * 128u;
-            const uint8_t* const wk1 = S.W1 + (size_t)kb * 128u;
+            const uint8_t* const wk0 = S.W0 + (size_t)kb * (A16 ? 64u : 128u);
+            const uint8_t* const wk1 = S.W1 + (size_t)kb * (A16 ? 64u : 128u);
 #pragma unroll
             for (uint32_t i = 0; i < 4u; i++)
                 __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[i]),
@@ -447,10 +547,17 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             if (S.nine) /* the ninth group's rows */
                 __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[4]),
                                                  (lds_void*)&L.a[st][(128u + 8u * cw) * 128u], 16, 0, 0);
+            if (A16) {
 #pragma unroll
-            for (uint32_t i = 0; i < 8u; i++)
-                __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + S.woff[i]),
-                                                 (lds_void*)&L.w[st][(64u * cw + 8u * i) * 128u], 16, 0, 0);
+                for (uint32_t i = 0; i < 4u; i++) /* 16 weight rows of 64 bytes each */
+                    __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 1u)) ? wk1 : wk0) + S.woff[i]),
+                                                     (lds_void*)&L.w[st][(64u * cw + 16u * i) * 64u], 16, 0, 0);
+            } else {
+#pragma unroll
+                for (uint32_t i = 0; i < 8u; i++)
+                    __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + S.woff[i]),
+                                                     (lds_void*)&L.w[st][(64u * cw + 8u * i) * 128u], 16, 0, 0);
+            }
         };
         Tile tcur, tnxt;
         Src cur, nxt;
@@ -476,7 +583,11 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                  * tile or the next) are outstanding. After the barrier the consumers are done with the
                  * block before kb, whose slot takes the block two ahead. */
                 if (kb + 1u < KB || more) { /* the loads that may stay outstanding are those of the block after kb */
-                    if (kb + 1u < KB ? cur.nine : nxt.nine) LOADER_BARRIER(T5_NLOAD + 1); else LOADER_BARRIER(T5_NLOAD);
+                    if (A16) { /* 4 token-row and 4 weight-row loads, no scales */
+                        if (kb + 1u < KB ? cur.nine : nxt.nine) LOADER_BARRIER(9); else LOADER_BARRIER(8);
+                    } else {
+                        if (kb + 1u < KB ? cur.nine : nxt.nine) LOADER_BARRIER(T5_NLOAD + 1); else LOADER_BARRIER(T5_NLOAD);
+                    }
                 } else {
                     LOADER_BARRIER(0);
                 }
@@ -518,17 +629,33 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
              * wait the compiler can see (everything the LDS was asked for has arrived) keeps it from
              * placing waits of its own inside the loops, whose LDS reads it does not see. */
             __builtin_amdgcn_s_waitcnt(0xc07f); /* lgkmcnt(0) */
+            if constexpr (A16) {
+                switch (ngrp_w) {
+                    case 9u: if constexpr (NG == 9) { T5_RUN_BLOCKS(T5A_BLOCK_N(9)) } break;
+                    case 8u: { T5_RUN_BLOCKS(T5A_BLOCK_N(8)) } break;
+                    case 7u: { T5_RUN_BLOCKS(T5A_BLOCK_N(7)) } break;
+                    case 6u: { T5_RUN_BLOCKS(T5A_BLOCK_N(6)) } break;
+                    case 5u: { T5_RUN_BLOCKS(T5A_BLOCK_N(5)) } break;
+                    case 4u: { T5_RUN_BLOCKS(T5A_BLOCK_N(4)) } break;
+                    case 3u: { T5_RUN_BLOCKS(T5A_BLOCK_N(3)) } break;
+                    case 2u: { T5_RUN_BLOCKS(T5A_BLOCK_N(2)) } break;
+                    case 1u: { T5_RUN_BLOCKS(T5A_BLOCK_N(1)) } break;
+                    default: { T5_RUN_BLOCKS() } break;
+                }
+            } else {
             switch (ngrp_w) {
-                case 9u: if constexpr (NG == 9) { T5_RUN_BLOCKS(T5_BLOCK_N(9)) } break;
-                case 8u: { T5_RUN_BLOCKS(T5_BLOCK_N(8)) } break;
-                case 7u: { T5_RUN_BLOCKS(T5_BLOCK_N(7)) } break;
-                case 6u: { T5_RUN_BLOCKS(T5_BLOCK_N(6)) } break;
-                case 5u: { T5_RUN_BLOCKS(T5_BLOCK_N(5)) } break;
-                case 4u: { T5_RUN_BLOCKS(T5_BLOCK_N(4)) } break;
-                case 3u: { T5_RUN_BLOCKS(T5_BLOCK_N(3)) } break;
-                case 2u: { T5_RUN_BLOCKS(T5_BLOCK_N(2)) } break;
-                case 1u: { T5_RUN_BLOCKS(T5_BLOCK_N(1)) } break;
-                default: { T5_RUN_BLOCKS() } break;
+                    case 9u: if constexpr (NG == 9) { T5_RUN_BLOCKS(T5_BLOCK_N(9)) } break;
+                    case 8u: { T5_RUN_BLOCKS(T5_BLOCK_N(8)) } break;
+                    case 7u: { T5_RUN_BLOCKS(T5_BLOCK_N(7)) } break;
+                    case 6u: { T5_RUN_BLOCKS(T5_BLOCK_N(6)) } break;
+                    case 5u: { T5_RUN_BLOCKS(T5_BLOCK_N(5)) } break;
+                    case 4u: { T5_RUN_BLOCKS(T5_BLOCK_N(4)) } break;
+                    case 3u: { T5_RUN_BLOCKS(T5_BLOCK_N(3)) } break;
+                    case 2u: { T5_RUN_BLOCKS(T5_BLOCK_N(2)) } break;
+                    case 1u: { T5_RUN_BLOCKS(T5_BLOCK_N(1)) } break;
+                    default: { T5_RUN_BLOCKS() } break;
+                }
+
             }
 
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
@@ -664,7 +791,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                                 if (16u * (uint32_t)rg >= rows) break; /* uniform */
                                 const uint32_t row = 16u * (uint32_t)rg + r16;
                                 const float gate = L.epi_gate[par][row]; /* 0 for pad rows */
-                                const float as = row < rows ? g.a_scale[r0 + row] : 0.0f;
+                                const float as = row < rows ? (A16 ? 1.0f : g.a_scale[r0 + row]) : 0.0f;
                                 v4f y[2];
 #pragma unroll
                                 for (int x = 0; x < 2; x++) {
@@ -681,17 +808,24 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
 #pragma unroll
                             for (int rg = 0; rg < NG; rg++) {
                                 const uint32_t row = 16u * (uint32_t)rg + r16;
+                                /* A16 with a row -> output row map (slot-major ops): rows leave by that map and
+                                 * nothing else of the output is touched */
+                                const bool mapped = A16 && g.row_partidx != nullptr;
                                 bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
                                 if (row >= rows) {
-                                    if (erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
+                                    if (!mapped && erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
                                     continue;
                                 }
                                 const uint32_t tok = L.epi_idx[par][row];
-                                if (tok == PLOW_EXPERT_UNUSED) {
+                                if (mapped) {
+                                    const uint32_t orow_i = g.row_partidx[r0 + row];
+                                    if (tok == PLOW_EXPERT_UNUSED || orow_i == PLOW_EXPERT_UNUSED) continue;
+                                    orow = (bf16_t*)g.out + (size_t)orow_i * g.N + ch0 + 4u * q;
+                                } else if (tok == PLOW_EXPERT_UNUSED) {
                                     *(uint2*)orow = make_uint2(0u, 0u);
                                     continue;
                                 }
-                                const float as = g.a_scale[tok];
+                                const float as = A16 ? 1.0f : g.a_scale[tok];
                                 float o[4];
 #pragma unroll
                                 for (int i = 0; i < 4; i++)
@@ -760,6 +894,12 @@ __global__ __launch_bounds__((NCW + 4u) * 64u) void k_group_w8a8_tiled(GroupW8A8
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     t5_body<GLU, PC, NCW, NG>(g, lds_raw);
 }
+/* the same tiles with bf16 activations */
+template <bool GLU, bool PC>
+__global__ __launch_bounds__(12u * 64u) void k_group_a16_tiled(GroupW8A8 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    t5_body<GLU, PC, 8u, 8, true>(g, lds_raw);
+}
 
 
 /* dynamic-LDS limits, once per device (plow_moe_device_setup) */
@@ -774,7 +914,12 @@ static bool t5_set_attrs() {
            t5_set_attr<false, true, NCW, NG>();
 }
 int plow_moe_w8a8_tiled_setup() {
-    const bool ok = t5_set_attrs<8u, 8>() && t5_set_attrs<8u, 9>() && t5_set_attrs<4u, 8>();
+    auto a16 = [](const void* f) {
+        return hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(T5Lds)) == hipSuccess;
+    };
+    const bool ok = t5_set_attrs<8u, 8>() && t5_set_attrs<8u, 9>() && t5_set_attrs<4u, 8>() &&
+                    a16((const void*)k_group_a16_tiled<true, false>) && a16((const void*)k_group_a16_tiled<false, false>) &&
+                    a16((const void*)k_group_a16_tiled<true, true>) && a16((const void*)k_group_a16_tiled<false, true>);
     return ok ? 0 : PLOW_MOE_EDEVICE;
 }
 
@@ -810,6 +955,21 @@ static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
     if (plow_moe_tuning().tile_waves4) return g.per_channel ? launch_tiled_t<GLU, true, 4u, 8>(g, st) : launch_tiled_t<GLU, false, 4u, 8>(g, st);
     if (t5_nine_groups(g, GLU)) return g.per_channel ? launch_tiled_t<GLU, true, 8u, 9>(g, st) : launch_tiled_t<GLU, false, 8u, 9>(g, st);
     return g.per_channel ? launch_tiled_t<GLU, true, 8u, 8>(g, st) : launch_tiled_t<GLU, false, 8u, 8>(g, st);
+}
+
+/* bf16 activations: `g.a` bf16 [..][K], no activation scales; g.per_channel picks the weight layout */
+int launch_group_a16_tiled(const GroupW8A8& g, bool glu, hipStream_t st) {
+    if (!group_w8a8_tiled_serves(g)) return PLOW_MOE_EINVAL;
+    const uint32_t n_cu = plow_moe_n_cu();
+    if (!n_cu) return PLOW_MOE_EDEVICE;
+    if (glu) {
+        if (g.per_channel) k_group_a16_tiled<true, true><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
+        else k_group_a16_tiled<true, false><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
+    } else {
+        if (g.per_channel) k_group_a16_tiled<false, true><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
+        else k_group_a16_tiled<false, false><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
+    }
+    return 0;
 }
 
 int launch_group_glu_w8a8_tiled(const GroupW8A8& g, hipStream_t st) { return launch_tiled<true>(g, st); }

@@ -74,6 +74,11 @@ int launch_group_glu_w8a8_tiled(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8_tiled(const GroupW8A8& g, hipStream_t st);
 /* whether the tiled form serves this shape (callers take the streaming form otherwise) */
 bool group_w8a8_tiled_serves(const GroupW8A8& g);
+/* the tiled form with bf16 activations (`a` bf16 [..][K], no activation scales): block-fp8 weights
+ * (wtab / stab [E][3]; GLU writes bf16 rows, out_bf16 set) or per-channel fp8 weights (per_channel set,
+ * tables [E][2]); GLU gathers rows by row_token and, per-channel mode only, may scatter them by
+ * row_partidx; DOWN reads aligned rows, or slot rows when a_slots is set */
+int launch_group_a16_tiled(const GroupW8A8& g, bool glu, hipStream_t st);
 
 
 /* Grouped experts with bf16 activations (see experts_a16.hip). */

@@ -14,7 +14,7 @@
  *   PLOW_MOE_SCORE_KERNEL     tile8 | valu     router score: keep the 8 x 8 tile kernel for few outputs / keep
  *                                              the vector-unit kernels at prefill sizes
  *   PLOW_MOE_SCORE_MFMA32_FROM  n              number of outputs from which the 32 x 32 matrix-unit tiles are forced
- *   PLOW_MOE_ROUTER_FUSED     0                keep score, top-k and align as separate launches at decode sizes
+ *   PLOW_MOE_A16_TILED        0                keep the bf16-activation arms on the streaming kernels at every row count
  */
 #ifndef PLOW_MOE_TUNING_H
 #define PLOW_MOE_TUNING_H
@@ -26,13 +26,12 @@ struct PlowMoeTuning {
     bool tile_waves4;
     int sk_depth;         /* 2..4 */
     bool sk_glu_regs;
-    bool sk_down_regs;
     bool sk_narrow;
     bool a16_regs;
     bool score_tile8;
     bool score_valu;
     uint64_t score_mfma32_from;
-    bool router_fused;
+    bool a16_tiled;
 };
 const PlowMoeTuning& plow_moe_tuning();
 

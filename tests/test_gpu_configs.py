@@ -86,6 +86,20 @@ def test_c5_qwen3_per_channel_fp8_prefill_sizes(moe, oracle, T):
     assert cnt.max() >= 0.9 * T          # Zipf(1.2): the most popular expert is chosen by (nearly) every token
 
 
+def test_c5_qwen3_per_channel_fp8_bf16_activations_prefill(moe, oracle):
+    """The same layer on ops 65 / 66 (bf16 activations, slot-major intermediate) at 512 tokens: from 16
+    rows per expert on average these run the tiled kernels too (rows gathered by token, scattered by slot;
+    DOWN reads the slot rows)."""
+    T = 512
+    print(f"[case] c5 T={T} arm=a16 zipf=1.2", flush=True)
+    cfg = c5_config(T, "a16")
+    plan = layer.plan_layer(cfg)
+    dev = synth.bind(plan, "cuda", seed=0, zipf=1.2)
+    run_device(moe, plan, dev)
+    cnt = check_prefill_sampled(oracle, cfg, plan, dev)
+    assert cnt.max() >= 0.9 * T
+
+
 def test_c3_dsv3_prefill_4k(moe, oracle):
     print("[case] c3", flush=True)
     cfg = layer.config("c3")
@@ -99,7 +113,7 @@ def test_c3_dsv3_prefill_4k(moe, oracle):
 @pytest.mark.parametrize("arm", ["w8a8", "a16"])
 def test_c6_glm_tp8_slice_prefill_8k(moe, oracle, arm):
     """The shape of plow's own gfx950 prefill bench (288 experts, top-8, H 4096, I 256 per rank, 8192
-    tokens), fp8 activations on the tiled kernels and bf16 activations on the four-row-group passes."""
+    tokens), fp8 activations and bf16 activations, both on the tiled kernels."""
     print(f"[case] c6 arm={arm}", flush=True)
     cfg = layer.config("c6")
     cfg.arm = arm
@@ -235,8 +249,11 @@ def check_prefill_sampled(oracle, cfg, plan, dev):
         fq_s = e4m3_to_f32(sh.np("fq")[rs]) * np.repeat(sh.np("fs")[rs], 128, axis=1)
         report_rows(f"{cfg.name} fq*fs (dequantized intermediate)", fq_d, fq_s, REL_L2_MID)
     else:
-        fu_d = ol.bf2f(gather("fu", rd_t).view(torch.int16).numpy().view(np.uint16))
-        fu_s = ol.bf2f(sh.np("fu")[rs])
+        # ops 65 / 66 (per-channel weights, bf16 activations) keep the intermediate by routing slot
+        slot_major = pc and not w8a8
+        fu_d = ol.bf2f(gather("fu", torch.from_numpy(slots_d).to(dev.device) if slot_major else rd_t)
+                       .view(torch.int16).numpy().view(np.uint16))
+        fu_s = ol.bf2f(sh.np("fu")[slots_s if slot_major else rs])
         report_rows(f"{cfg.name} fu (bf16 intermediate)", fu_d, fu_s, REL_L2_MID)
         if pc and w8a8:
             f8_d = e4m3_to_f32(gather("fu8", rd_t).numpy()) * gather("fscale", rd_t).numpy()[:, None]
