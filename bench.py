@@ -27,6 +27,8 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0          # MI355X datasheet
 FP8_PEAK_TFLOPS = 5000.0       # dense fp8 MFMA
+FP4_PEAK_TFLOPS = 10100.0      # dense fp4 MFMA
+BF16_PEAK_TFLOPS = 2500.0      # dense bf16 MFMA
 CPU_THREADS_CAP = 16           # the GPU box's CPU share for one GPU
 
 
@@ -133,7 +135,12 @@ def run_cell(a, name, tokens, steps, warmup, share=None, cpu_mode="full"):
     layer_bytes = hit * eb + cfg.E * H * 2 + (cfg.E * 4 if cfg.bias else 0) + 2 * T * H * 2
     dom = max(("glu", "down"), key=lambda n: op_us[n])
     frac_w = 2.0 / 3.0 if dom == "glu" else 1.0 / 3.0
-    act_in = T * H * (1 if cfg.arm == "w8a8" else 2) if dom == "glu" else rows * cfg.I
+    # bytes of an element of the intermediate the DOWN reads: e4m3 + a scale per 128, e2m1 + a byte per 32, bf16
+    mid = {"w8a8": 1.0 + 4.0 / 128.0, "w8a8q": 1.0 + 4.0 / 128.0, "a4w4": 0.5 + 1.0 / 32.0}.get(cfg.arm, 2.0)
+    act_in = T * H * (1 if cfg.arm == "w8a8" else 2) if dom == "glu" else rows * cfg.I * mid
+    # the matrix unit's peak in the type the arm multiplies in
+    mfma_peak = (FP4_PEAK_TFLOPS if cfg.arm == "a4w4" else
+                 FP8_PEAK_TFLOPS if cfg.arm.startswith("w8a8") else BF16_PEAK_TFLOPS)
     dom_bytes = hit * eb * frac_w + act_in
     dom_flops = 2.0 * rows * (2 if dom == "glu" else 1) * cfg.I * H
     achieved = dom_bytes / (op_us[dom] * 1e-6) / 1e9
@@ -146,9 +153,9 @@ def run_cell(a, name, tokens, steps, warmup, share=None, cpu_mode="full"):
             "bytes_per_launch": int(dom_bytes), "us_per_launch": round(op_us[dom], 2),
             # the time each roof allows this launch: the larger one is the roof that binds
             "roof_us": {"hbm": round(dom_bytes / (HBM_PEAK_GBS * 1e9) * 1e6, 1),
-                        "mfma": round(dom_flops / (FP8_PEAK_TFLOPS * 1e12) * 1e6, 1)},
-            "mfma": {"achieved": round(achieved_tf, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved_tf / FP8_PEAK_TFLOPS, 4), "flops_per_launch": dom_flops}}
+                        "mfma": round(dom_flops / (mfma_peak * 1e12) * 1e6, 1)},
+            "mfma": {"achieved": round(achieved_tf, 1), "peak": mfma_peak, "unit": "TFLOP/s",
+                     "frac": round(achieved_tf / mfma_peak, 4), "flops_per_launch": dom_flops}}
     rec = {
         "value": round(ms * 1e3, 2), "unit": "us/layer", "ms_per_step": round(ms, 4), "steps": steps, "warmup": warmup,
         "dtype": {"fp8blk": "fp8_e4m3", "mxfp4": "fp4_e2m1", "fp8pc": "fp8_e4m3", "bf16": "bf16"}[cfg.enc],
@@ -161,7 +168,7 @@ def run_cell(a, name, tokens, steps, warmup, share=None, cpu_mode="full"):
                                        "pad_frac": round(float(((cnt + 63) // 64 * 64).sum() / max(1, cnt.sum()) - 1.0), 4)}},
         "tokens_per_s": round(T / (ms * 1e-3), 1),
         "layer": {"algorithmic_bytes": int(layer_bytes), "hbm_frac": round(layer_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                  "flops": flops, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / FP8_PEAK_TFLOPS, 4)},
+                  "flops": flops, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / mfma_peak, 4)},
         "op_us": {n: round(v, 2) for n, v in op_us.items()},
         "roofline": roof,
     }
@@ -224,7 +231,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="", help="one configuration only (c1..c6); default: c2 with c3 under prefill_4k")
     ap.add_argument("--tokens", type=int, default=0)
-    ap.add_argument("--arm", default="", help="override the configuration's arm (a16 | w8a8 | w8a8q | w8a8atomic | w8a8det)")
+    ap.add_argument("--arm", default="", help="override the configuration's arm (a16 | w8a8 | w8a8q | w8a8atomic | w8a8det | a4w4)")
     ap.add_argument("--zipf", type=float, default=-1.0, help="override the expert popularity exponent")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib", action="store_true",

@@ -120,12 +120,19 @@ enum {
 /* Weight encodings (i3 on ops 85/86, i6 on ops 48/49; dev_isa.h:442-461, :691-702). */
 enum { PLOW_MOE_ENC_BF16 = 0, PLOW_MOE_ENC_FP8BLK = 1, PLOW_MOE_ENC_MXFP4 = 2 };
 
-/* Arms of ops 85/86 (i7; runtime/amd/interp.hip:6500-6604). 0 and 2/3 are the reference's; 8 is
+/* Arms of ops 85/86 (i7; runtime/amd/interp.hip:6500-6604). 0, 1 and 2/3 are the reference's; 8 is
  * this library's name for "mxfp4 weights, bf16 activations" on gathered rows (the arithmetic of the
- * reference's decode ops 48/49 at enc 2); the reference's enc-2 default (fp4 on both operands) is
- * refused with PLOW_MOE_EUNSUPPORTED. */
+ * reference's decode ops 48/49 at enc 2).
+ * At enc 2 arm 0 is the reference's default there, fp4 on both operands (runtime/amd/op_moe.h:3948-4720):
+ *   85: t0=fu mxfp4 [R][I/2] (out) t1=x bf16 [T][H] t2=wtab t3=stab (E8M0 rows [N][K/32]) t4=meta
+ *       t5=row_token t6=row_partidx (rows it marks unused are skipped) t7=E8M0 rows [R][I/32] (out)
+ *       i4 = T, the rows of t1 (an extension of this library, which quantizes every token row once ahead
+ *       of the GEMM; needs a context); I and H multiples of 256, at least 512
+ *   86: t0=part (arm 0: f32, arm 1: bf16) t1=fu mxfp4 t5=its E8M0 rows, the rest as on the other arms */
 enum {
     PLOW_MOE_ARM_A16       = 0, /* bf16 activations (enc 0 bf16 weights, enc 1 W8A16)             */
+    PLOW_MOE_ARM_A4W4      = 0, /* enc 2: mxfp4 activations, quantized per 32 values by the GLU op  */
+    PLOW_MOE_ARM_A4W4_P16  = 1, /* DOWN only, enc 2: as 0 with a bf16 part                         */
     PLOW_MOE_ARM_W8A8      = 2, /* enc 1: e4m3 activations with 1x128 scales; DOWN writes f32 part */
     PLOW_MOE_ARM_W8A8_P16  = 3, /* DOWN only: as 2 with a bf16 part                                */
     PLOW_MOE_ARM_W8A8_XQ   = 6, /* GLU only, enc 1: t1 holds the bf16 rows, quantized 1x128 where they

@@ -396,6 +396,61 @@ static float dot_mxfp4(const float* wf, const uint8_t* s, const float* a, uint32
     return acc;
 }
 
+/* ---- the activation quantizer of the fp4 x fp4 arm (A4W4) ------------------------------------------
+ * E8M0 byte of a 32-block from its amax, mapping the amax onto e2m1's top code 6 (plow
+ * runtime/amd/amd_common.h:1073-1111): 127 for amax not above zero, for +inf / NaN and for the three
+ * smallest subnormals; else E - 1 - (M < 2^22) of the float's exponent and mantissa fields, clamped to
+ * 1..254. */
+static uint8_t mx_act_e8m0(float amax) {
+    if (!(amax > 0.0f)) return 127u;
+    uint32_t bits;
+    memcpy(&bits, &amax, 4);
+    const uint32_t E = bits >> 23;
+    if (E == 0xFFu || bits < 4u) return 127u;
+    int e = (int)E - 1 - (int)((bits & 0x7FFFFFu) < 0x400000u);
+    if (e < 1) e = 1;
+    if (e > 254) e = 254;
+    return (uint8_t)e;
+}
+/* 1 / 2^(b - 127) (amd_common.h:731-741): exact; b = 254 gives the subnormal 2^-127 */
+static float mx_act_inv(uint8_t b) {
+    if (b == 254u) return orc_from_bits(0x00400000u);
+    return orc_from_bits((uint32_t)(254u - b) << 23);
+}
+/* f32 -> e2m1 code on the ladder 0, .5, 1, 1.5, 2, 3, 4, 6: nearest, an exact midpoint goes AWAY from
+ * zero, saturating at 6; NaN gives 7 with a clear sign, -0 a clear sign (amd_common.h:1031-1068) */
+static uint8_t mx_act_fp4(float v) {
+    const uint8_t sign = (v < 0.0f) ? 8u : 0u;
+    const float a = fabsf(v);
+    const uint8_t n = (uint8_t)(!(a < 0.25f) + !(a < 0.75f) + !(a < 1.25f) + !(a < 1.75f) + !(a < 2.5f) + !(a < 3.5f) +
+                                !(a < 5.0f));
+    return sign | n;
+}
+/* one 32-block: 16 bytes (element 2i in the low nibble of byte i) and its E8M0 byte
+ * (plow runtime/amd/op_moe.h:4132-4179: amax over the block, then every value times the inverse scale) */
+static void mx_act_quant32(const float* v, uint8_t* out16, uint8_t* sb_out) {
+    float amax = 0.0f;
+    for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(v[i]));
+    const uint8_t sb = mx_act_e8m0(amax);
+    const float inv = mx_act_inv(sb);
+    for (int i = 0; i < 16; i++)
+        out16[i] = (uint8_t)(mx_act_fp4(v[2 * i] * inv) | (mx_act_fp4(v[2 * i + 1] * inv) << 4));
+    *sb_out = sb;
+}
+/* fp4 x fp4 dot of two decoded rows (raw e2m1 values) with their E8M0 rows: every 32-block's sum of
+ * products is exact (multiples of 1/4 below 2^11), scaled by the exact power of two 2^(sa + sw - 254);
+ * the order in which the matrix instruction adds the blocks is not specified, so the blocks are added
+ * in f64 and rounded once */
+static float dot_a4w4(const float* wf, const uint8_t* sw, const float* af, const uint8_t* sa, uint32_t K) {
+    double acc = 0.0;
+    for (uint32_t k0 = 0; k0 < K; k0 += 32u) {
+        float blk = 0.0f;
+        for (uint32_t k = k0; k < k0 + 32u; k++) blk += wf[k] * af[k];
+        acc += (double)blk * (double)orc_e8m0(sw[k0 / 32u]) * (double)orc_e8m0(sa[k0 / 32u]);
+    }
+    return (float)acc;
+}
+
 /* One weight row of an expert matrix under `enc`, decoded to f32 without its scales. */
 typedef struct {
     const float* sf;   /* enc 1: scale row [ceil(K/128)] */
@@ -457,6 +512,12 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
      * rest is arm 2 (plow runtime/amd/moe_pf_w8a8.h:118-121, :255-283) */
     const int xq_inline = enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ;
     const int w8a8 = (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8) || xq_inline;
+    /* enc 2, arm 0 (the reference's default for mxfp4): fp4 on both operands. t1 = bf16 rows, quantized per
+     * 32 with mx_act_quant32; t0 = fu as mxfp4 [R][I/2]; t6 = row_partidx (pad rows are skipped);
+     * t7 = the E8M0 rows [R][I/32] it writes (plow runtime/amd/interp.hip:6496-6499, op_moe.h:4183-4632) */
+    const int a4w4 = enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_A16;
+    uint8_t* rowsa = NULL; /* a4w4: [cached row][H/32] E8M0 bytes of the rows quantized here */
+    uint32_t rowsa_cap = 0;
     const float* xs = TEN(in, T, 6);
     const uint32_t G = (I + 127u) / 128u, KB = (H + 127u) / 128u;
     float* rowxs = NULL; /* arm 6: [cached row][KB] scales of the rows quantized here */
@@ -480,6 +541,7 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
         if (rc.expert != e) {
             cache_fit(&rc, cnt);
             if (xq_inline && rowxs_cap < cnt) { free(rowxs); rowxs = malloc((size_t)cnt * KB * 4u); rowxs_cap = cnt; }
+            if (a4w4 && rowsa_cap < cnt) { free(rowsa); rowsa = malloc((size_t)cnt * (H / 32u)); rowsa_cap = cnt; }
             for (uint32_t q = 0; q < cnt; q++) {
                 const uint32_t tok = row_token[r0 + q];
                 rc.live[q] = tok != PLOW_EXPERT_UNUSED;
@@ -495,13 +557,46 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
                             rc.a[(size_t)q * H + kb * 128u + j] =
                                 e4m3_lut[orc_f32_to_e4m3(orc_bf2f(src[kb * 128u + j]) * inv)];
                     }
+                } else if (a4w4) { /* the row as raw e2m1 values plus its E8M0 bytes */
+                    const orc_bf16* src = (const orc_bf16*)TEN(in, T, 1) + (size_t)tok * H;
+                    for (uint32_t b = 0; b < H / 32u; b++) {
+                        float v32[32];
+                        uint8_t q16[16];
+                        for (uint32_t j = 0; j < 32u; j++) v32[j] = orc_bf2f(src[b * 32u + j]);
+                        mx_act_quant32(v32, q16, &rowsa[(size_t)q * (H / 32u) + b]);
+                        for (uint32_t j = 0; j < 32u; j++)
+                            rc.a[(size_t)q * H + b * 32u + j] = orc_e2m1((j & 1u) ? (uint8_t)(q16[j >> 1] >> 4) : (uint8_t)(q16[j >> 1] & 15u));
+                    }
                 } else if (w8a8) decode_e4m3_row(rc.a + (size_t)q * H, (const uint8_t*)TEN(in, T, 1) + (size_t)tok * H, H);
                 else decode_bf16_row(rc.a + (size_t)q * H, (const orc_bf16*)TEN(in, T, 1) + (size_t)tok * H, H);
             }
             rc.expert = e;
         }
         const uint32_t n0 = g0 * 128u, n1 = n0 + 128u < I ? n0 + 128u : I;
-        if (!w8a8) {
+        if (a4w4) {
+            /* SwiGLU in f32, then every (row, 32 channels) block quantized to mxfp4 with its E8M0 byte */
+            uint8_t* fq = TEN(in, T, 0);
+            uint8_t* cs = TEN(in, T, 7);
+            const uint32_t* rpi = TEN(in, T, 6);
+            if (vcap < cnt) { free(v); v = malloc((size_t)cnt * 128u * 4u); vcap = cnt; }
+            for (uint32_t n = n0; n < n1; n++) {
+                const RowScale sg = enc_row(enc, Wg, Sg, n, H, wg);
+                const RowScale su = enc_row(enc, Wu, Su, n, H, wu);
+                for (uint32_t q = 0; q < cnt; q++) {
+                    if (!rc.live[q]) continue;
+                    const float* a = rc.a + (size_t)q * H;
+                    const uint8_t* sa = rowsa + (size_t)q * (H / 32u);
+                    v[(size_t)q * 128u + (n - n0)] =
+                        glu_pair(dot_a4w4(wg, sg.sb, a, sa, H), dot_a4w4(wu, su.sb, a, sa, H), act, in->fj[0].f, in->fj[1].f);
+                }
+            }
+            for (uint32_t q = 0; q < cnt; q++) {
+                if (!rc.live[q] || (rpi && rpi[r0 + q] == PLOW_EXPERT_UNUSED)) continue;
+                for (uint32_t c0 = 0; c0 < n1 - n0; c0 += 32u)
+                    mx_act_quant32(v + (size_t)q * 128u + c0, fq + (size_t)(r0 + q) * (I / 2u) + (n0 + c0) / 2u,
+                                   cs + (size_t)(r0 + q) * (I / 32u) + (n0 + c0) / 32u);
+            }
+        } else if (!w8a8) {
             orc_bf16* fu = TEN(in, T, 0);
             for (uint32_t n = n0; n < n1; n++) {
                 const RowScale sg = enc_row(enc, Wg, Sg, n, H, wg);
@@ -543,7 +638,7 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
             }
         }
     }
-    free(wg); free(wu); free(v); free(rowxs);
+    free(wg); free(wu); free(v); free(rowxs); free(rowsa);
     cache_free(&rc);
 }
 
@@ -576,7 +671,10 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
     const uint32_t H = in->i[0], I = in->i[1], E = in->i[2], enc = in->i[3], arm = in->i[7];
     const int w8a8 = enc == PLOW_MOE_ENC_FP8BLK &&
                      (arm == PLOW_MOE_ARM_W8A8 || arm == PLOW_MOE_ARM_W8A8_P16);
-    const int part16 = w8a8 && arm == PLOW_MOE_ARM_W8A8_P16;
+    /* enc 2, arm 0 / 1: fp4 on both operands; t1 = fu as mxfp4 [R][I/2], t5 = its E8M0 rows [R][I/32];
+     * arm 1 = bf16 part (plow runtime/amd/interp.hip:6581-6589: i7 = part16 on the generic body) */
+    const int a4w4 = enc == PLOW_MOE_ENC_MXFP4 && (arm == PLOW_MOE_ARM_A16 || arm == 1u);
+    const int part16 = (w8a8 && arm == PLOW_MOE_ARM_W8A8_P16) || (a4w4 && arm == 1u);
     /* i5: t0 is the f64 [T][H] accumulator of the deterministic fused combine; log2(k) + 1, or 256 + k */
     const uint32_t det_k = !in->i[5] ? 0u : in->i[5] > 256u ? in->i[5] - 256u : 1u << (in->i[5] - 1u);
     const float* fs = TEN(in, T, 5);
@@ -598,6 +696,7 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
                 rc.live[q] = row_partidx[r0 + q] != PLOW_EXPERT_UNUSED;
                 if (!rc.live[q]) continue;
                 if (w8a8) decode_e4m3_row(rc.a + (size_t)q * I, (const uint8_t*)TEN(in, T, 1) + (size_t)(r0 + q) * I, I);
+                else if (a4w4) decode_mxfp4_row(rc.a + (size_t)q * I, (const uint8_t*)TEN(in, T, 1) + (size_t)(r0 + q) * (I / 2u), I);
                 else decode_bf16_row(rc.a + (size_t)q * I, (const orc_bf16*)TEN(in, T, 1) + (size_t)(r0 + q) * I, I);
             }
             rc.expert = e;
@@ -613,7 +712,8 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
                 const float* a = rc.a + (size_t)q * I;
                 const float acc = w8a8 ? dot_fp8blk_a8(wd, (const float*)Sd + (size_t)g0 * KB, a,
                                                        fs + (size_t)r * KB, 1u, I)
-                                       : enc_dot(enc, wd, rs, a, I);
+                                  : a4w4 ? dot_a4w4(wd, rs.sb, a, (const uint8_t*)TEN(in, T, 5) + (size_t)r * (I / 32u), I)
+                                         : enc_dot(enc, wd, rs, a, I);
                 const float val = row_gate[r] * acc;
                 if (det_k) det_add((double*)TEN(in, T, 0) + (size_t)(pidx / det_k) * H + h, det_q(val));
                 else if (part16) ((orc_bf16*)TEN(in, T, 0))[(size_t)pidx * H + h] = orc_f2bf(val);
@@ -1353,6 +1453,12 @@ int plow_oracle_exec_many(const PlowDevInst* insts, uint32_t n, void* const* ten
 
 /* ---- codec exports for the tests --------------------------------------------------------------- */
 
+/* the fp4 x fp4 arm's activation quantizer over n_blocks 32-blocks of f32 values */
+void plow_oracle_mx_act_quant(uint8_t* out, uint8_t* scales, const float* v, size_t n_blocks) {
+    for (size_t b = 0; b < n_blocks; b++) mx_act_quant32(v + b * 32u, out + b * 16u, scales + b);
+}
+uint8_t plow_oracle_mx_act_e8m0(float amax) { return mx_act_e8m0(amax); }
+uint8_t plow_oracle_mx_act_fp4(float v) { return mx_act_fp4(v); }
 uint16_t plow_oracle_f2bf(float f) { return orc_f2bf(f); }
 float plow_oracle_bf2f(uint16_t h) { return orc_bf2f(h); }
 uint8_t plow_oracle_f32_to_e4m3(float f) { return orc_f32_to_e4m3(f); }

@@ -24,6 +24,11 @@ float    plow_oracle_e2m1(uint8_t nib);
 float    plow_oracle_e8m0(uint8_t s);
 void     plow_oracle_f2bf_n(uint16_t* dst, const float* src, size_t n);
 void     plow_oracle_e4m3_encode_n(uint8_t* dst, const float* src, size_t n);
+/* the activation quantizer of the fp4 x fp4 arm (ops 85 / 86, enc 2, arm 0): n_blocks 32-blocks of f32 ->
+ * 16 bytes and one E8M0 byte each; its two primitives */
+void     plow_oracle_mx_act_quant(uint8_t* out, uint8_t* scales, const float* v, size_t n_blocks);
+uint8_t  plow_oracle_mx_act_e8m0(float amax);
+uint8_t  plow_oracle_mx_act_fp4(float v);
 
 #ifdef __cplusplus
 }

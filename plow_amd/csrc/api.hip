@@ -62,7 +62,31 @@ struct PlowMoeCtx {
     char err[256];
     void* ws_base;   /* the context's own allocation behind `ws` (NULL when `ws` is borrowed) */
     Workspace ws;
+    /* token rows of the fp4 x fp4 arm's GLU, quantized ahead of its GEMM: grown on demand, kept until
+     * the context is destroyed */
+    void* stage;
+    size_t stage_bytes;
 };
+
+/* Room for `bytes` of staging on the context's device. Growing frees the old block first, which waits for
+ * the device: work already queued that reads it finishes before it goes. */
+static int stage_reserve(PlowMoeCtx* c, size_t bytes) {
+    if (bytes <= c->stage_bytes) return 0;
+    int prev = 0;
+    (void)hipGetDevice(&prev);
+    (void)hipSetDevice(c->device);
+    (void)hipFree(c->stage);
+    c->stage = nullptr, c->stage_bytes = 0;
+    const bool ok = hipMalloc(&c->stage, bytes) == hipSuccess;
+    (void)hipSetDevice(prev);
+    if (!ok) {
+        c->stage = nullptr;
+        (void)hipGetLastError();
+        return PLOW_MOE_ENOMEM;
+    }
+    c->stage_bytes = bytes;
+    return 0;
+}
 
 static int fail(PlowMoeCtx* c, int code, const char* fmt, ...) {
     if (c) {
@@ -114,6 +138,7 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
 extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) {
     if (!ctx) return;
     (void)hipFree(ctx->ws_base);
+    (void)hipFree(ctx->stage);
     delete ctx;
 }
 
@@ -352,6 +377,34 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.slots_hint = slots_of(in, h, 0u);
             return launch_group_glu_a16(g, st);
         }
+        if (enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_A4W4) {
+            /* fp4 on both operands (plow runtime/amd/op_moe.h:3948-4720): the token rows are quantized to
+             * mxfp4 once each, ahead of the GEMM, into the context's staging block (the reference quantizes
+             * every gathered row inside its kernel: the same values, k times); the GLU's output leaves as
+             * mxfp4 rows (t0) with their E8M0 rows (t7) */
+            NEED(c, ten(in, T, 3) && ten(in, T, 6) && ten(in, T, 7), "op 85 A4W4: t3 stab, t6 row_partidx, t7 E8M0 rows must be bound");
+            NEED(c, I % 256u == 0u && H % 256u == 0u && I >= 512u && H >= 512u, "op 85 A4W4: I %u and H %u must be multiples of 256, at least 512", I, H);
+            NEED(c, i[4] != 0u, "op 85 A4W4: i4 (the number of token rows in t1) is zero");
+            NEED(c, i[5] <= 2u || i[5] == PLOW_MOE_ACT_SWIGLU_CLAMP, "op 85: activation %u is not served", i[5]);
+            if (!c->ws_base) return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85 A4W4: needs a context (its staging block)");
+            if (!launch) return 0;
+            const size_t qbytes = ws_up((size_t)i[4] * (H / 2u)), sbytes = ws_up((size_t)i[4] * (H / 32u));
+            const int src = stage_reserve(c, qbytes + sbytes);
+            if (src) return fail(c, src, "op 85 A4W4: %zu bytes of staging could not be allocated", qbytes + sbytes);
+            uint8_t* const xq4 = (uint8_t*)c->stage;
+            uint8_t* const xs = xq4 + qbytes;
+            const int qrc = launch_quant_mx_act(xq4, xs, ten(in, T, 1), i[4], H, st);
+            if (qrc) return qrc;
+            GroupW8A8 g = {};
+            g.out = ten(in, T, 0); g.out_e8m0 = (uint8_t*)ten(in, T, 7);
+            g.a = xq4; g.a_e8m0 = xs;
+            g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 3);
+            g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
+            g.row_partidx = (const uint32_t*)ten(in, T, 6);
+            g.N = I; g.K = H; g.E = E; g.act = i[5];
+            g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
+            return launch_group_a4w4_tiled(g, true, st);
+        }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85: encoding %u arm %u is not served", enc, arm);
     }
     case PLOW_DOP_MOE_GROUP_DOWN_PF: {
@@ -400,6 +453,20 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.wcols = 3; g.wsel0 = 2; g.wsel1 = 2;
             g.slots_hint = slots_of(in, h, 0u);
             return launch_group_down_a16(g, st);
+        }
+        if (enc == PLOW_MOE_ENC_MXFP4 && (arm == PLOW_MOE_ARM_A4W4 || arm == PLOW_MOE_ARM_A4W4_P16)) {
+            /* fp4 on both operands: t1 the mxfp4 rows and t5 the E8M0 rows that op 85 wrote */
+            NEED(c, ten(in, T, 3) && ten(in, T, 5), "op 86 A4W4: t3 stab and t5 E8M0 rows must be bound");
+            NEED(c, I % 256u == 0u && H % 256u == 0u && I >= 512u && H >= 512u, "op 86 A4W4: I %u and H %u must be multiples of 256, at least 512", I, H);
+            if (!launch) return 0;
+            GroupW8A8 g = {};
+            g.out = ten(in, T, 0);
+            g.a = ten(in, T, 1); g.a_e8m0 = (const uint8_t*)ten(in, T, 5);
+            g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 3);
+            g.meta = (const int32_t*)ten(in, T, 4);
+            g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
+            g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_A4W4_P16;
+            return launch_group_a4w4_tiled(g, false, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 86: encoding %u arm %u is not served", enc, arm);
     }
@@ -703,7 +770,9 @@ static int check_segment(PlowMoeCtx* c, const PlowDevInst* insts, uint32_t n) {
         NEED(c, g.t[2] == d.t[2] && g.t[3] == d.t[3] && g.t[4] == d.t[4], "segment: wtab / stab / meta handles differ");
         const bool quantized_mid = g.i[7] == PLOW_MOE_ARM_W8A8;
         NEED(c, g.t[0] == d.t[1], "segment: DOWN does not read the GLU's output");
-        if (quantized_mid) NEED(c, g.t[7] == d.t[5], "segment: DOWN does not read the GLU's output scales");
+        const bool a4w4 = g.i[3] == PLOW_MOE_ENC_MXFP4 && g.i[7] == PLOW_MOE_ARM_A4W4;
+        if (quantized_mid || a4w4) NEED(c, g.t[7] == d.t[5], "segment: DOWN does not read the GLU's output scales");
+        if (a4w4) NEED(c, d.i[7] == PLOW_MOE_ARM_A4W4 || d.i[7] == PLOW_MOE_ARM_A4W4_P16, "segment: GLU arm %u and DOWN arm %u disagree", g.i[7], d.i[7]);
         NEED(c, (g.i[7] == PLOW_MOE_ARM_W8A8) == (d.i[7] == PLOW_MOE_ARM_W8A8 || d.i[7] == PLOW_MOE_ARM_W8A8_P16),
              "segment: GLU arm %u and DOWN arm %u disagree", g.i[7], d.i[7]);
     } else if (g.op == PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF_W8A8) {

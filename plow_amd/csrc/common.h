@@ -91,6 +91,30 @@ __device__ __forceinline__ void det_add(double* p, float v) {
     (void)__builtin_amdgcn_global_atomic_fadd_f64((__attribute__((address_space(1))) double*)p, det_q(v));
 }
 
+/* The activation quantizer of the fp4 x fp4 arm (plow runtime/amd/amd_common.h:1073-1111, :731-741,
+ * :1031-1068): the E8M0 byte that maps a 32-block's amax onto e2m1's top code, its exact inverse scale,
+ * and the e2m1 code of a scaled value (nearest on the ladder, exact midpoints away from zero, saturating
+ * at 6; NaN gives code 7). */
+__device__ __forceinline__ uint32_t mxq_e8m0(float amax) {
+    if (!(amax > 0.0f)) return 127u;
+    const uint32_t bits = __float_as_uint(amax), E = bits >> 23;
+    if (E == 0xFFu || bits < 4u) return 127u;
+    int e = (int)E - 1 - (int)((bits & 0x7FFFFFu) < 0x400000u);
+    e = e < 1 ? 1 : e;
+    e = e > 254 ? 254 : e;
+    return (uint32_t)e;
+}
+__device__ __forceinline__ float mxq_inv(uint32_t b) {
+    return b == 254u ? __uint_as_float(0x00400000u) : __uint_as_float((254u - b) << 23);
+}
+__device__ __forceinline__ uint32_t mxq_fp4(float v) {
+    const uint32_t sign = (v < 0.0f) ? 8u : 0u;
+    const float a = fabsf(v);
+    const uint32_t n = (uint32_t)!(a < 0.25f) + (uint32_t)!(a < 0.75f) + (uint32_t)!(a < 1.25f) + (uint32_t)!(a < 1.75f) +
+                       (uint32_t)!(a < 2.5f) + (uint32_t)!(a < 3.5f) + (uint32_t)!(a < 5.0f);
+    return sign | n;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));

@@ -34,6 +34,7 @@
  * token rows and weight rows on one XCD at the same time (see the tile loop). */
 #include <stdlib.h>
 #include <string.h>
+#include <type_traits>
 #include "common.h"
 #include "kernels.h"
 #include "tuning.h"
@@ -70,6 +71,18 @@ struct T5Lds {
     uint16_t prefix[1056];              /* inclusive tile count over experts: at most 2^18 slots / 144 + 1056 */
 };
 static_assert(sizeof(T5Lds) <= 160u * 1024u, "the tile's LDS plan must fit one CU");
+/* the plan of the fp4 x fp4 arm: 128-row tiles, a block is 256 k (128 bytes of nibbles per row, so the
+ * ring has the geometry of the fp8 one), and every row of a stage brings its eight E8M0 bytes */
+struct T5LdsA4 {
+    uint8_t a[T5_STAGES][128u * 128u];
+    uint8_t w[T5_STAGES][256u * 128u];
+    uint8_t ts[T5_STAGES][128u][8]; /* token-row scales of the block */
+    uint8_t ws[T5_STAGES][256u][8]; /* weight-row scales of the block */
+    uint32_t epi_idx[2][T5_AS];
+    float epi_gate[2][T5_AS];
+    uint16_t prefix[1056];
+};
+static_assert(sizeof(T5LdsA4) <= 160u * 1024u, "the tile's LDS plan must fit one CU");
 
 typedef __attribute__((address_space(3))) void lds_void;
 
@@ -92,6 +105,12 @@ __device__ __forceinline__ float ds_read4(uint32_t addr) {
     return r;
 }
 template <uint32_t OFF>
+__device__ __forceinline__ int ds_read1(uint32_t addr) {
+    int r;
+    asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+    return r;
+}
+template <uint32_t OFF>
 __device__ __forceinline__ v2i ds_read8(uint32_t addr) {
     v2i r;
     asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
@@ -106,7 +125,7 @@ __device__ __forceinline__ v2i ds_read8(uint32_t addr) {
 
 /* ---- one 128-k block of a consumer wave (names are those of the kernel body) -------------------- */
 #define T5_BLOCK_HEAD()                                                                                      \
-    const uint32_t ab = a_base + st * (T5_BM * 128u), wb = w_base + st * (256u * 128u) + cw * (32u * 128u);  \
+    const uint32_t ab = a_base + st * (uint32_t)sizeof(L.a[0]), wb = w_base + st * (256u * 128u) + cw * (32u * 128u);  \
     const uint32_t blo = ab + op_lo, bhi = ab + op_hi;                                                       \
     const uint32_t alo = wb + op_lo, ahi = wb + op_hi;                                                       \
     const uint32_t sl = s_base + st * (T5_AS * 4u) + r16 * 4u;                                               \
@@ -201,7 +220,7 @@ __device__ __forceinline__ v2i ds_read8(uint32_t addr) {
  *      j at (j ^ 4 * ((r16 >> 2) & 1)): the 64 lanes of a read then touch every bank twice, the minimum
  *      for 512 bytes. ---- */
 #define T5A_BLOCK_HEAD()                                                                                     \
-    const uint32_t ab = a_base + st * (T5_BM * 128u), wb = w_base + st * (256u * 128u) + cw * (32u * 64u);   \
+    const uint32_t ab = a_base + st * (uint32_t)sizeof(L.a[0]), wb = w_base + st * (256u * 128u) + cw * (32u * 64u);   \
     const uint32_t b0 = ab + opb0, b1 = ab + opb1;                                                           \
     const uint32_t cl = c_base + par * 1024u + (kb >> 1) * 4u;
 #define T5A_DECODE(R) t5a_decode(R)
@@ -266,6 +285,57 @@ __device__ __forceinline__ v2i ds_read8(uint32_t addr) {
     T5A_GROUP_N(7, N) T5A_SCALE_N(6, N)                                                                      \
     T5A_GROUP_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0) T5A_SCALE_N(7, N)                                        \
     T5A_SCALE_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0)
+/* ---- the block of the fp4 x fp4 arm: 256 k as two matrix instructions of 128 k, both operands e2m1 with
+ *      their E8M0 bytes applied by the instruction itself (a lane's 32 k are one scale block, its byte goes
+ *      in as a register: with constant scale arguments the compiler would pick the unscaled instruction).
+ *      The accumulator runs straight through K. ---- */
+#define T5Q_BLOCK_HEAD()                                                                                     \
+    const uint32_t ab = a_base + st * (uint32_t)sizeof(L.a[0]), wb = w_base + st * (256u * 128u) + cw * (32u * 128u); \
+    const uint32_t b0 = ab + opb0, b1 = ab + opb1;                                                           \
+    const uint32_t tsl = ts_base + st * (128u * 8u) + r16 * 8u + q;                                          \
+    const uint32_t wsl = wsb_base + st * (256u * 8u) + (cw * 32u + r16) * 8u + q;
+#define T5Q_MFMA(A, B, C, SA, SB)                                                                            \
+    __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(__builtin_shufflevector(A, zero4, 0, 1, 2, 3, 4, 5, 6, 7), \
+                                                     __builtin_shufflevector(B, zero4, 0, 1, 2, 3, 4, 5, 6, 7), C, 4, 4, 0, SA, 0, SB)
+#define T5Q_GROUP_N(RG, N)                                                                                   \
+    if ((RG) < (N)) {                                                                                        \
+        asm volatile("s_waitcnt lgkmcnt(%4)"                                                                 \
+                     : "+v"(bx[(RG) % 3][0]), "+v"(bx[(RG) % 3][1]), "+v"(bs[(RG) % 3][0]), "+v"(bs[(RG) % 3][1]) \
+                     : "n"((RG) + 1 < (N) ? 4 : 0));                                                         \
+        if ((RG) + 2 < (N)) {                                                                                \
+            bx[((RG) + 2) % 3][0] = ds_read16<((RG) + 2) * 2048u>(b0);                                       \
+            bx[((RG) + 2) % 3][1] = ds_read16<((RG) + 2) * 2048u>(b1);                                       \
+            bs[((RG) + 2) % 3][0] = ds_read1<((RG) + 2) * 128u>(tsl);                                        \
+            bs[((RG) + 2) % 3][1] = ds_read1<((RG) + 2) * 128u + 4u>(tsl);                                   \
+        }                                                                                                    \
+        acc[RG][0] = T5Q_MFMA(ax[0][0], bx[(RG) % 3][0], acc[RG][0], as4[0][0], bs[(RG) % 3][0]);            \
+        acc[RG][1] = T5Q_MFMA(ax[1][0], bx[(RG) % 3][0], acc[RG][1], as4[1][0], bs[(RG) % 3][0]);            \
+        acc[RG][0] = T5Q_MFMA(ax[0][1], bx[(RG) % 3][1], acc[RG][0], as4[0][1], bs[(RG) % 3][1]);            \
+        acc[RG][1] = T5Q_MFMA(ax[1][1], bx[(RG) % 3][1], acc[RG][1], as4[1][1], bs[(RG) % 3][1]);            \
+    }
+#define T5Q_BLOCK_N(N)                                                                                       \
+    T5Q_BLOCK_HEAD()                                                                                         \
+    const v4i zero4 = {0, 0, 0, 0};                                                                          \
+    v4i ax[2][2];                                                                                            \
+    int as4[2][2];                                                                                           \
+    ax[0][0] = ds_read16<0>(wb + opb0), ax[0][1] = ds_read16<0>(wb + opb1);                                  \
+    ax[1][0] = ds_read16<2048>(wb + opb0), ax[1][1] = ds_read16<2048>(wb + opb1);                            \
+    as4[0][0] = ds_read1<0>(wsl), as4[0][1] = ds_read1<4>(wsl);                                              \
+    as4[1][0] = ds_read1<128>(wsl), as4[1][1] = ds_read1<132>(wsl);                                          \
+    v4i bx[3][2];                                                                                            \
+    int bs[3][2];                                                                                            \
+    bx[0][0] = ds_read16<0>(b0), bx[0][1] = ds_read16<0>(b1);                                                \
+    bs[0][0] = ds_read1<0>(tsl), bs[0][1] = ds_read1<4>(tsl);                                                \
+    if ((N) > 1) {                                                                                           \
+        bx[1][0] = ds_read16<2048u>(b0), bx[1][1] = ds_read16<2048u>(b1);                                    \
+        bs[1][0] = ds_read1<128u>(tsl), bs[1][1] = ds_read1<132u>(tsl);                                      \
+    }                                                                                                        \
+    asm volatile("s_waitcnt lgkmcnt(%8)"                                                                     \
+                 : "+v"(ax[0][0]), "+v"(ax[0][1]), "+v"(ax[1][0]), "+v"(ax[1][1]), "+v"(as4[0][0]),          \
+                   "+v"(as4[0][1]), "+v"(as4[1][0]), "+v"(as4[1][1])                                         \
+                 : "n"((N) > 1 ? 8 : 4));                                                                    \
+    T5Q_GROUP_N(0, N) T5Q_GROUP_N(1, N) T5Q_GROUP_N(2, N) T5Q_GROUP_N(3, N)                                  \
+    T5Q_GROUP_N(4, N) T5Q_GROUP_N(5, N) T5Q_GROUP_N(6, N) T5Q_GROUP_N(7, N)
 /* eight e4m3 bytes -> eight bf16 (the hardware conversion is exact) */
 __device__ __forceinline__ v8bf t5a_decode(v2i r) {
     const v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((uint32_t)r[0], 1.0f, false);
@@ -296,10 +366,16 @@ __device__ __forceinline__ v8bf t5a_decode(v2i r) {
 /* NG: 16-row groups a tile may hold, 8 or 9 (see t5_nine_groups below). */
 /* A16: `a` holds bf16 rows [..][K] (no activation scales) and a block is 64 k: the bf16-activation arms
  * (block-fp8 weights: ops 85 / 86 arm 0; per-channel fp8 weights: ops 65 / 66). */
-template <bool GLU, bool PC, uint32_t NCW, int NG = 8, bool A16 = false>
+/* AM: what the activation rows are. 0: e4m3 with scales (the W8A8 pairs); 1 (A16): bf16; 2 (A4): mxfp4 rows
+ * [..][K / 2] with E8M0 rows [..][K / 32] against mxfp4 weights, a block is 256 k, scales applied by the
+ * matrix instruction (ops 85 / 86 with enc 2, arm 0). */
+template <bool GLU, bool PC, uint32_t NCW, int NG = 8, int AM = 0>
 __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     static_assert(NG == 8 || NG == 9, "a tile is eight or nine 16-row groups");
-    T5Lds& L = *(T5Lds*)lds_raw;
+    constexpr bool A16 = AM == 1, A4 = AM == 2;
+    static_assert(!A4 || (NG == 8 && !PC), "the fp4 arm has 128-row tiles and no per-channel mode");
+    typedef typename std::conditional<A4, T5LdsA4, T5Lds>::type Lds;
+    Lds& L = *(Lds*)lds_raw;
     constexpr uint32_t BN = GLU ? 128u : 256u; /* output channels per tile */
     constexpr uint32_t NTHR = (NCW + 4u) * 64u, SUBS = 8u / NCW;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -344,11 +420,20 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         }
     }
     const uint32_t total = (uint32_t)L.prefix[g.E - 1u] * NT;
-    const uint32_t K = g.K, KB = K / (A16 ? 64u : 128u); /* blocks of the K loop */
-    const uint32_t KS = K / 128u;                         /* weight block scales along K */
-    const uint32_t KA = A16 ? 2u * K : K;                 /* bytes of a token row */
+    const uint32_t K = g.K, KB = K / (A16 ? 64u : A4 ? 256u : 128u); /* blocks of the K loop */
+    const uint32_t KS = K / 128u;                                    /* weight block scales along K */
+    const uint32_t KA = A16 ? 2u * K : A4 ? K / 2u : K;              /* bytes of a token row */
+    const uint32_t KW = A4 ? K / 2u : K;                             /* bytes of a weight row */
+    const uint32_t K32 = K / 32u;                                    /* A4: E8M0 bytes of a row */
+    (void)KS, (void)K32;
     const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]);
-    const uint32_t s_base = lds_off(&L.as[0][0]), c_base = lds_off(&L.wsc[0][0][0]);
+    uint32_t s_base = 0, c_base = 0, ts_base = 0, wsb_base = 0;
+    if constexpr (A4) {
+        ts_base = lds_off(&L.ts[0][0][0]), wsb_base = lds_off(&L.ws[0][0][0]);
+    } else {
+        s_base = lds_off(&L.as[0][0]), c_base = lds_off(&L.wsc[0][0][0]);
+    }
+    (void)s_base, (void)c_base, (void)ts_base, (void)wsb_base;
     /* consumer: this lane's operand pieces 2q, 2q + 1 of row (16 * group + r16) */
     const uint32_t sw = (r16 >> 1) & 7u;
     const uint32_t op_lo = r16 * 128u + (((2u * q) ^ sw) << 4), op_hi = r16 * 128u + (((2u * q + 1u) ^ sw) << 4);
@@ -431,6 +516,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
              * vector offset) */
             uint32_t aoff[5], woff[8], sstep;
             uint32_t nine; /* this loader has a ninth-group load in this tile (loaders 0 and 1, tiles of more than 128 rows) */
+            /* A4: this lane's dword of the E8M0 rows: token row 32 * cw + l / 2 and weight rows 64 * cw + 32 * j + l / 2 */
+            const uint8_t *tsp, *wsp[2];
             const float* ssrc;
             const uint8_t *W0, *W1;
         };
@@ -440,6 +527,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
          * uses them a few blocks later. Rows below the live count always hold a token. */
         struct Pre {
             uint32_t tok[5], stok, eidx;
+            uint32_t tsrow; /* A4: the row of `a` whose scale dword this lane loads */
             float w0, w1, egate;
         };
         auto fetch = [&](const Tile& t, Pre& P) {
@@ -463,13 +551,24 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 const uint32_t row = (cw < 3u ? cw : 0u) * 64u + lane; /* the row whose activation scale this lane loads */
                 /* per-channel mode has one activation scale per row, applied in the epilogue: its ring slot
                  * carries zeros */
-                P.eidx = row < rows ? (GLU ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
-                P.stok = (PC || A16) ? PLOW_EXPERT_UNUSED : P.eidx;
+                /* the fp4 arm's GLU skips the rows its row_partidx operand marks unused */
+                P.eidx = row < rows ? ((GLU && !A4) ? g.row_token[r0 + row] : g.row_partidx[r0 + row]) : PLOW_EXPERT_UNUSED;
+                P.stok = (PC || A16 || A4) ? PLOW_EXPERT_UNUSED : P.eidx;
                 P.egate = (!GLU && row < rows) ? g.row_gate[r0 + row] : 0.0f;
             }
             /* weight block scales of the tile: GLU gate | up of channel block nt; DOWN blocks 2nt, 2nt + 1 */
+            if (A4) { /* the token row 32 * cw + lane / 2 of the tile, as a row of `a` */
+                const uint32_t row = 32u * cw + (lane >> 1);
+                const uint32_t ar = r0 + (row < rows ? row : 0u);
+                if (GLU) {
+                    const uint32_t tk = g.row_token[ar];
+                    P.tsrow = tk == PLOW_EXPERT_UNUSED ? 0u : tk;
+                } else {
+                    P.tsrow = ar;
+                }
+            }
             P.w0 = P.w1 = 0.0f;
-            if (!PC) {
+            if (!PC && !A4) {
                 const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
                 const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : S0;
                 const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
@@ -502,7 +601,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     ch = nt * 256u + R;
                     if (ch >= g.N) ch = 0; /* past the last channel: any valid row, never stored */
                 }
-                S.woff[i] = A16 ? ch * K + (((lane & 3u) ^ (((R >> 2) & 1u) << 1)) << 4) : ch * K + ((p ^ ((R >> 1) & 7u)) << 4);
+                S.woff[i] = A16 ? ch * K + (((lane & 3u) ^ (((R >> 2) & 1u) << 1)) << 4) : ch * KW + ((p ^ ((R >> 1) & 7u)) << 4);
             }
             /* activation scale of row 64 * cw + lane (loader 3 repeats loader 0's 64 values); a pad row
              * reads tilep[0], which is always 0 */
@@ -521,10 +620,23 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     S.sstep = ok ? 1u : 0u;
                 }
             }
-            const uint32_t i = tid - NCW * 64u;
-            if (i < KS) {
-                L.wsc[par][0][i] = P.w0;
-                L.wsc[par][1][i] = P.w1;
+            if constexpr (A4) {
+                S.tsp = g.a_e8m0 + (size_t)P.tsrow * K32 + (lane & 1u) * 4u;
+                const uint8_t* const SW0 = (const uint8_t*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
+                const uint8_t* const SW1 = GLU ? (const uint8_t*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : SW0;
+#pragma unroll
+                for (uint32_t j = 0; j < 2u; j++) {
+                    const uint32_t R = 64u * cw + 32u * j + (lane >> 1);
+                    uint32_t ch = GLU ? nt * 128u + 16u * (R >> 5) + (R & 15u) : nt * 256u + R;
+                    if (ch >= g.N) ch = 0;
+                    S.wsp[j] = ((GLU && (R & 16u)) ? SW1 : SW0) + (size_t)ch * K32 + (lane & 1u) * 4u;
+                }
+            } else {
+                const uint32_t i = tid - NCW * 64u;
+                if (i < KS) {
+                    L.wsc[par][0][i] = P.w0;
+                    L.wsc[par][1][i] = P.w1;
+                }
             }
             /* what the consumers' epilogue needs per row, so that it does not start with a round trip to
              * memory: loaders 0, 1 and 2 hold rows 0..63, 64..127 and 128..191 */
@@ -534,9 +646,14 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             }
         };
         auto issue = [&](const Src& S, uint32_t kb, uint32_t st) {
-            if (!A16)
+            if constexpr (A4) { /* eight E8M0 bytes per row and block, a dword per lane */
+                __builtin_amdgcn_global_load_lds((const void*)(S.tsp + (size_t)kb * 8u), (lds_void*)&L.ts[st][32u * cw][0], 4, 0, 0);
+                __builtin_amdgcn_global_load_lds((const void*)(S.wsp[0] + (size_t)kb * 8u), (lds_void*)&L.ws[st][64u * cw][0], 4, 0, 0);
+                __builtin_amdgcn_global_load_lds((const void*)(S.wsp[1] + (size_t)kb * 8u), (lds_void*)&L.ws[st][64u * cw + 32u][0], 4, 0, 0);
+            } else if constexpr (!A16) {
                 __builtin_amdgcn_global_load_lds((const void*)(S.ssrc + (size_t)kb * S.sstep),
                                                  (lds_void*)&L.as[st][(cw < 3u ? cw : 0u) * 64u], 4, 0, 0);
+            }
             const uint8_t* const ak = A0 + (size_t)kb * 128u;
             const uint8_t* const wk0 = S.W0 + (size_t)kb * (A16 ? 64u : 128u);
             const uint8_t* const wk1 = S.W1 + (size_t)kb * (A16 ? 64u : 128u);
@@ -585,6 +702,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 if (kb + 1u < KB || more) { /* the loads that may stay outstanding are those of the block after kb */
                     if (A16) { /* 4 token-row and 4 weight-row loads, no scales */
                         if (kb + 1u < KB ? cur.nine : nxt.nine) LOADER_BARRIER(9); else LOADER_BARRIER(8);
+                    } else if (A4) { /* 3 scale, 4 token-row, 8 weight-row loads */
+                        LOADER_BARRIER(15);
                     } else {
                         if (kb + 1u < KB ? cur.nine : nxt.nine) LOADER_BARRIER(T5_NLOAD + 1); else LOADER_BARRIER(T5_NLOAD);
                     }
@@ -629,7 +748,19 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
              * wait the compiler can see (everything the LDS was asked for has arrived) keeps it from
              * placing waits of its own inside the loops, whose LDS reads it does not see. */
             __builtin_amdgcn_s_waitcnt(0xc07f); /* lgkmcnt(0) */
-            if constexpr (A16) {
+            if constexpr (A4) {
+                switch (ngrp_w) {
+                    case 8u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(8)) } break;
+                    case 7u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(7)) } break;
+                    case 6u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(6)) } break;
+                    case 5u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(5)) } break;
+                    case 4u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(4)) } break;
+                    case 3u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(3)) } break;
+                    case 2u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(2)) } break;
+                    case 1u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(1)) } break;
+                    default: { T5_RUN_BLOCKS() } break;
+                }
+            } else if constexpr (A16) {
                 switch (ngrp_w) {
                     case 9u: if constexpr (NG == 9) { T5_RUN_BLOCKS(T5A_BLOCK_N(9)) } break;
                     case 8u: { T5_RUN_BLOCKS(T5A_BLOCK_N(8)) } break;
@@ -661,7 +792,47 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             /* ---- epilogue. Lane: row = 16 * rg + r16; GLU channel = ch0 + 4q + i with gate in weight
              *      group 0 and up in group 1; DOWN channel = ch0 + 16 * x + 4q + i ---- */
             const uint32_t stl = st >= 1u ? st - 1u : 2u; /* the ring stage the tile has just left */
-            if (!PC && GLU && g.out_bf16) {
+            if constexpr (A4 && GLU) {
+                /* SwiGLU in f32, then every (row, 32 channels) block to mxfp4 with its E8M0 byte (plow
+                 * runtime/amd/op_moe.h:4595-4632). A block is the 16 channels of consumer 2j and those of
+                 * consumer 2j + 1: the row maxima meet as in the fp8 epilogue below. */
+                float v[SUBS][NG][4];
+                auto red = [&](uint32_t x) -> float* { return (float*)&L.w[stl][x * (32u * 128u)]; };
+#pragma unroll
+                for (uint32_t sub = 0; sub < SUBS; sub++) {
+                    const uint32_t cw = cw0 + sub;
+                    v4f(&acc)[NG][2] = accs[sub];
+#pragma unroll
+                    for (int rg = 0; rg < NG; rg++) {
+                        float m = 0.0f;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            v[sub][rg][i] = moe_glu(acc[rg][0][i], acc[rg][1][i], g.act, g.f0, g.f1);
+                            m = fmaxf(m, fabsf(v[sub][rg][i]));
+                        }
+                        m = fmaxf(m, __shfl_xor(m, 16, 64));
+                        m = fmaxf(m, __shfl_xor(m, 32, 64));
+                        if (q == 0) red(cw)[16u * (uint32_t)rg + r16] = m;
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); /* pairs with the loaders' */
+#pragma unroll
+                for (uint32_t sub = 0; sub < SUBS; sub++) {
+                    const uint32_t cw = cw0 + sub, ch0 = nt * 128u + 16u * cw;
+#pragma unroll
+                    for (int rg = 0; rg < NG; rg++) {
+                        const uint32_t row = 16u * (uint32_t)rg + r16;
+                        if (row >= rows || L.epi_idx[par][row] == PLOW_EXPERT_UNUSED) continue;
+                        const float amax = fmaxf(red(cw & ~1u)[row], red(cw | 1u)[row]);
+                        const uint32_t sb = mxq_e8m0(amax);
+                        const float inv = mxq_inv(sb);
+                        const uint32_t code = mxq_fp4(v[sub][rg][0] * inv) | (mxq_fp4(v[sub][rg][1] * inv) << 4) |
+                                              (mxq_fp4(v[sub][rg][2] * inv) << 8) | (mxq_fp4(v[sub][rg][3] * inv) << 12);
+                        *(uint16_t*)((uint8_t*)g.out + (size_t)(r0 + row) * (g.N / 2u) + (ch0 + 4u * q) / 2u) = (uint16_t)code;
+                        if (!(cw & 1u) && q == 0) g.out_e8m0[(size_t)(r0 + row) * (g.N / 32u) + (ch0 >> 5)] = (uint8_t)sb;
+                    }
+                }
+            } else if (!PC && GLU && g.out_bf16) {
                 /* bf16 intermediate (op 188): bf16(act(g) * u) for live rows, zeros for the pad rows of the
                  * expert's last 64-row tile */
                 asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); /* pairs with the loaders' */
@@ -898,7 +1069,7 @@ __global__ __launch_bounds__((NCW + 4u) * 64u) void k_group_w8a8_tiled(GroupW8A8
 template <bool GLU, bool PC>
 __global__ __launch_bounds__(12u * 64u) void k_group_a16_tiled(GroupW8A8 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    t5_body<GLU, PC, 8u, 8, true>(g, lds_raw);
+    t5_body<GLU, PC, 8u, 8, 1>(g, lds_raw);
 }
 
 
@@ -913,13 +1084,23 @@ static bool t5_set_attrs() {
     return t5_set_attr<true, false, NCW, NG>() && t5_set_attr<false, false, NCW, NG>() && t5_set_attr<true, true, NCW, NG>() &&
            t5_set_attr<false, true, NCW, NG>();
 }
+/* mxfp4 on both operands */
+template <bool GLU>
+__global__ __launch_bounds__(12u * 64u) void k_group_a4w4_tiled(GroupW8A8 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    t5_body<GLU, false, 8u, 8, 2>(g, lds_raw);
+}
 int plow_moe_w8a8_tiled_setup() {
     auto a16 = [](const void* f) {
         return hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(T5Lds)) == hipSuccess;
     };
     const bool ok = t5_set_attrs<8u, 8>() && t5_set_attrs<8u, 9>() && t5_set_attrs<4u, 8>() &&
                     a16((const void*)k_group_a16_tiled<true, false>) && a16((const void*)k_group_a16_tiled<false, false>) &&
-                    a16((const void*)k_group_a16_tiled<true, true>) && a16((const void*)k_group_a16_tiled<false, true>);
+                    a16((const void*)k_group_a16_tiled<true, true>) && a16((const void*)k_group_a16_tiled<false, true>) &&
+                    hipFuncSetAttribute((const void*)k_group_a4w4_tiled<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)sizeof(T5LdsA4)) == hipSuccess &&
+                    hipFuncSetAttribute((const void*)k_group_a4w4_tiled<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)sizeof(T5LdsA4)) == hipSuccess;
     return ok ? 0 : PLOW_MOE_EDEVICE;
 }
 
@@ -955,6 +1136,16 @@ static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
     if (plow_moe_tuning().tile_waves4) return g.per_channel ? launch_tiled_t<GLU, true, 4u, 8>(g, st) : launch_tiled_t<GLU, false, 4u, 8>(g, st);
     if (t5_nine_groups(g, GLU)) return g.per_channel ? launch_tiled_t<GLU, true, 8u, 9>(g, st) : launch_tiled_t<GLU, false, 8u, 9>(g, st);
     return g.per_channel ? launch_tiled_t<GLU, true, 8u, 8>(g, st) : launch_tiled_t<GLU, false, 8u, 8>(g, st);
+}
+
+int launch_group_a4w4_tiled(const GroupW8A8& g, bool glu, hipStream_t st) {
+    if (!g.N || !g.E || g.E > 1056u || g.N % 128u || g.N < 256u || g.K % 256u || g.K < 512u || g.K > 256u * 128u)
+        return PLOW_MOE_EINVAL;
+    const uint32_t n_cu = plow_moe_n_cu();
+    if (!n_cu) return PLOW_MOE_EDEVICE;
+    if (glu) k_group_a4w4_tiled<true><<<n_cu, 768, sizeof(T5LdsA4), st>>>(g);
+    else k_group_a4w4_tiled<false><<<n_cu, 768, sizeof(T5LdsA4), st>>>(g);
+    return 0;
 }
 
 /* bf16 activations: `g.a` bf16 [..][K], no activation scales; g.per_channel picks the weight layout */

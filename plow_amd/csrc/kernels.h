@@ -66,6 +66,10 @@ struct GroupW8A8 {
     /* DOWN, block mode: when non-zero, `a` and `a_scale` are stored by routing slot ([a_slots][K] and
      * [K/128][a_slots]) and aligned row r reads slot row_partidx[r]; slots >= a_slots are skipped (op 190) */
     uint32_t a_slots;
+    /* fp4 x fp4 arm (launch_group_a4w4_tiled): `a` holds mxfp4 rows [..][K / 2] and a_e8m0 their E8M0 rows
+     * [..][K / 32]; the GLU writes its output the same way into out / out_e8m0; stab holds E8M0 rows */
+    const uint8_t* a_e8m0;
+    uint8_t* out_e8m0;
 };
 int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);
@@ -79,6 +83,11 @@ bool group_w8a8_tiled_serves(const GroupW8A8& g);
  * tables [E][2]); GLU gathers rows by row_token and, per-channel mode only, may scatter them by
  * row_partidx; DOWN reads aligned rows, or slot rows when a_slots is set */
 int launch_group_a16_tiled(const GroupW8A8& g, bool glu, hipStream_t st);
+/* the tiled form with mxfp4 on both operands (K a multiple of 256, at least 512) */
+int launch_group_a4w4_tiled(const GroupW8A8& g, bool glu, hipStream_t st);
+/* bf16 rows [rows][K] -> mxfp4 rows [rows][K / 2] + E8M0 rows [rows][K / 32], the fp4 x fp4 arm's activation
+ * quantizer (K a multiple of 32) */
+int launch_quant_mx_act(uint8_t* out, uint8_t* scales, const void* x, uint32_t rows, uint32_t K, hipStream_t st);
 
 
 /* Grouped experts with bf16 activations (see experts_a16.hip). */

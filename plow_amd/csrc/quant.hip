@@ -48,6 +48,43 @@ int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uin
     return 0;
 }
 
+/* bf16 rows -> mxfp4 rows with one E8M0 byte per 32 values: the activation quantizer of the fp4 x fp4 arm
+ * of ops 85 / 86 (plow runtime/amd/op_moe.h:4132-4179, amd_common.h:1031-1111). Four lanes per 32-block,
+ * eight values each; value 2i sits in the low nibble of byte i. */
+__global__ __launch_bounds__(256) void k_quant_mx_act(uint8_t* __restrict__ out, uint8_t* __restrict__ scales,
+                                                      const bf16_t* __restrict__ x, size_t n_blocks) {
+    const uint32_t sub = threadIdx.x & 3u;
+    for (size_t b = ((size_t)blockIdx.x * 256u + threadIdx.x) / 4u; b < n_blocks; b += (size_t)gridDim.x * 64u) {
+        const uint4 raw = *(const uint4*)(x + b * 32u + sub * 8u);
+        const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+        float f[8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            f[2 * j] = __uint_as_float(v[j] << 16);
+            f[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+            amax = fmaxf(amax, fmaxf(fabsf(f[2 * j]), fabsf(f[2 * j + 1])));
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 4));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 4));
+        const uint32_t sb = mxq_e8m0(amax);
+        const float inv = mxq_inv(sb);
+        uint32_t code = 0u;
+#pragma unroll
+        for (int j = 0; j < 8; j++) code |= mxq_fp4(f[j] * inv) << (4 * j);
+        *(uint32_t*)(out + b * 16u + sub * 4u) = code;
+        if (sub == 0) scales[b] = (uint8_t)sb;
+    }
+}
+
+int launch_quant_mx_act(uint8_t* out, uint8_t* scales, const void* x, uint32_t rows, uint32_t K, hipStream_t st) {
+    if (K % 32u || rows == 0 || !out || !scales || !x) return PLOW_MOE_EINVAL;
+    const size_t n_blocks = (size_t)rows * (K / 32u);
+    uint32_t blocks = (uint32_t)((n_blocks + 63u) / 64u > 16384u ? 16384u : (n_blocks + 63u) / 64u);
+    k_quant_mx_act<<<blocks, 256, 0, st>>>(out, scales, (const bf16_t*)x, n_blocks);
+    return 0;
+}
+
 /* Op 189 (plow runtime/amd/op_moe_fp8_block128.h:49-55, op_gemm_common.h:2582-2621 with SCATTER,
  * interp.hip:5291-5300): the tilep[E] * 64 aligned bf16 rows, each quantized 1x128 into the row of its
  * routing slot (hq[slot][K], scale[g][slot]; rows whose slot is out of range are skipped), and the bf16

@@ -145,7 +145,8 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
     row_token = p._t("row_token", "u32", (R,), "scratch")
     row_partidx = p._t("row_partidx", "u32", (R,), "scratch")
     row_gate = p._t("row_gate", "f32", (R,), "scratch")
-    p16 = cfg.part_bf16 and cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q")
+    p16 = cfg.part_bf16 and ((cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q")) or
+                             (cfg.enc == "mxfp4" and cfg.arm == "a4w4"))
     det = cfg.det_combine and cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q")
     assert not (det and p16)
     part = (p._t("acc64", "f64", (T, H), "scratch") if det
@@ -223,6 +224,18 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
                                      t=[part, fq, wtab, stab, meta, fs, row_partidx, row_gate],
                                      i=[H, I, Ea, enc, 0, (256 + ka) if det else 0, 0,
                                         abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8], slots=T * ka))
+        elif enc == abi.ENC_MXFP4 and cfg.arm == "a4w4":
+            # fp4 on both operands: the GLU quantizes its bf16 rows per 32 and writes the intermediate as
+            # mxfp4 with E8M0 rows; i4 = T (the rows of x) is what this library's quantizer pass needs
+            fu4 = p._t("fu4", "u8", (R, I // 2), "scratch")
+            fsc = p._t("fsc", "u8", (R, I // 32), "scratch")
+            p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
+                                    t=[fu4, x, wtab, stab, meta, row_token, row_partidx, fsc],
+                                    i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_A4W4], f=cfg.act_f, slots=T * ka))
+            p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
+                                     t=[part, fu4, wtab, stab, meta, fsc, row_partidx, row_gate],
+                                     i=[H, I, Ea, enc, 0, 0, 0, abi.ARM_A4W4_P16 if p16 else abi.ARM_A4W4],
+                                     slots=T * ka))
         else:
             arm = abi.ARM_W4A16 if enc == abi.ENC_MXFP4 else abi.ARM_A16
             fu = p._t("fu", "bf16", (R, I), "scratch")

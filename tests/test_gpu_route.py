@@ -202,7 +202,7 @@ def test_refusals(moe):
     assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 1, 2, 0, 8, 1]), t) == 0
     assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 60, 8, 1, 2, 0, 8, 4]), t) == abi.E_INVAL
     assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 1, 2, 0, 32, 2]), t) == abi.E_INVAL
-    assert moe.check(abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5], i=[256, 256, 4, 2, 0, 1, 0, 0]), t) == abi.E_UNSUPPORTED
+    assert moe.check(abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5], i=[256, 256, 4, 2, 0, 1, 0, 5]), t) == abi.E_UNSUPPORTED
     assert moe.check(abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[4, 100]), t) == abi.E_INVAL
     with pytest.raises(Exception):
         moe.exec(abi.inst(abi.OP_MOE_ALIGN_PF, t=[0, 1, 2, 3], i=[4, 8, 2]), t)

@@ -627,3 +627,144 @@ def test_deterministic_fused_combine_reference_shift_encoding(oracle):
     b = synth.bind(plan, "cpu", seed=2)
     run_oracle(oracle, plan, b)
     assert np.array_equal(a.t["acc64"].numpy(), b.t["acc64"].numpy()) and np.abs(a.t["acc64"].numpy()).max() > 0
+
+
+# ---- the fp4 x fp4 arm of ops 85 / 86: its activation quantizer and its GEMMs ---------------------
+
+E2M1 = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+
+
+def test_mx_act_e8m0_is_the_smallest_power_of_two_that_brings_the_amax_below_six(oracle):
+    """Exact rational arithmetic instead of the float's bit fields: 2^(b - 127) is the smallest power of two
+    s with amax / s < 6 (so the block's largest value lands on e2m1's 3, 4 or just under 6), clamped to the
+    bytes 1..254; zero, negative, infinite and NaN amax give 127."""
+    from fractions import Fraction
+    r = cases.rng_of(21)
+    vals = [np.float32(v) for v in r.integers(4, 0x7F800000, 4000, dtype=np.uint32).view(np.float32)]
+    for n in range(-140, 128):
+        for m in (1.0, 1.25, 1.5, 1.75):
+            v = np.float32(m * 2.0 ** n)
+            if v > 0 and np.isfinite(v):
+                vals += [v, np.nextafter(v, np.float32(0)), np.nextafter(v, np.float32(np.inf))]
+    for a in vals:
+        if not np.isfinite(a) or a.view(np.uint32) < 4:
+            continue
+        F = Fraction(float(a))
+        e = int(np.frexp(float(a))[1])
+        while F >= 6 * Fraction(2) ** e:
+            e += 1
+        while F < 6 * Fraction(2) ** (e - 1):
+            e -= 1
+        want = min(max(e + 127, 1), 254)
+        assert oracle.plow_oracle_mx_act_e8m0(float(a)) == want, (a, want)
+    for a in (0.0, -1.0, float("inf"), float("nan"), float(np.uint32(3).view(np.float32))):
+        assert oracle.plow_oracle_mx_act_e8m0(a) == 127
+
+
+def test_mx_act_fp4_is_the_nearest_e2m1_value_with_midpoints_away_from_zero(oracle):
+    from fractions import Fraction
+    r = cases.rng_of(22)
+    vals = list(r.uniform(-8, 8, 3000).astype(np.float32)) + list(r.standard_normal(500).astype(np.float32) * 1e-3)
+    for a, b in zip(E2M1[:-1], E2M1[1:]):
+        mid = np.float32((a + b) / 2)
+        for v in (mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(9)), np.float32(a), np.float32(b)):
+            vals += [v, -v]
+    vals += [np.float32(v) for v in (6.0, 6.5, 100.0, 3e38, float("inf"), -float("inf"), 1e-40, -1e-40)]
+    for v in vals:
+        F = Fraction(float(abs(v))) if np.isfinite(v) else Fraction(10)
+        best = min(range(8), key=lambda n: (abs(F - Fraction(float(E2M1[n]))), -n))   # ties: the larger magnitude
+        want = (8 if v < 0 else 0) | best
+        assert oracle.plow_oracle_mx_act_fp4(float(v)) == want, (v, want)
+    assert oracle.plow_oracle_mx_act_fp4(-0.0) == 0
+    assert oracle.plow_oracle_mx_act_fp4(float("nan")) == 7
+
+
+def mx_dequant(codes, scales):
+    c = np.stack([codes & 0xF, codes >> 4], axis=-1).reshape(codes.shape[0], -1)
+    v = E2M1[c & 7] * np.where(c & 8, -1.0, 1.0)
+    return v * np.repeat(np.exp2(scales.astype(np.float64) - 127.0), 32, axis=1)
+
+
+def mx_act_quant(oracle, v):
+    v = np.ascontiguousarray(v, np.float32)
+    out, sc = np.zeros((v.shape[0], v.shape[1] // 2), np.uint8), np.zeros((v.shape[0], v.shape[1] // 32), np.uint8)
+    oracle.plow_oracle_mx_act_quant(out.ctypes.data, sc.ctypes.data, v.ctypes.data, v.size // 32)
+    return out, sc
+
+
+def test_mx_act_quant_returns_representable_blocks_unchanged(oracle):
+    """A block of e2m1 values up to 4, times 2^s, with a 4 in it: the byte is s + 127 and the block survives
+    exactly. With a 6 as its amax the byte is one more (6 / 2^s is not below 6) and the block comes back as
+    its halves, rounded away from zero onto the ladder."""
+    r = cases.rng_of(23)
+    n = 64
+    s = r.integers(-20, 20, (n, 1))
+    v = E2M1[r.integers(0, 7, (n, 32))] * r.choice([-1.0, 1.0], (n, 32))
+    v[:, 5] = 4.0
+    x = (v * np.exp2(s)).astype(np.float32)
+    q, sc = mx_act_quant(oracle, x)
+    assert np.array_equal(sc[:, 0], (s[:, 0] + 127).astype(np.uint8))
+    assert np.array_equal(mx_dequant(q, sc), x.astype(np.float64))
+    v[:, 5] = -6.0
+    x = (v * np.exp2(s)).astype(np.float32)
+    q, sc = mx_act_quant(oracle, x)
+    assert np.array_equal(sc[:, 0], (s[:, 0] + 128).astype(np.uint8))
+    half = np.abs(v) / 2                                    # 0 .25 .5 .75 1 1.5 2 3: .25 -> .5 and .75 -> 1
+    want = np.where(half == 0.25, 0.5, np.where(half == 0.75, 1.0, half)) * np.sign(v) * 2 * np.exp2(s)
+    assert np.array_equal(mx_dequant(q, sc), want)
+
+
+@pytest.mark.parametrize("p16", [False, True])
+def test_a4w4_arm_against_f64_over_the_same_bytes(oracle, p16):
+    """Op 85 at enc 2 / arm 0 quantizes each gathered row per 32 values, multiplies in fp4 x fp4, applies the
+    GLU in f32 and leaves mxfp4 rows with E8M0 rows; op 86 reads them back. Against numpy f64 over the
+    dequantized bytes, with the pad rows left untouched."""
+    r = cases.rng_of(31)
+    E, T, H, I, k = 4, 9, 128, 64, 2
+    Wg = [r.integers(0, 256, (I, H // 2), dtype=np.uint8) for _ in range(E)]
+    Wu = [r.integers(0, 256, (I, H // 2), dtype=np.uint8) for _ in range(E)]
+    Wd = [r.integers(0, 256, (H, I // 2), dtype=np.uint8) for _ in range(E)]
+    Sg = [r.integers(118, 124, (I, H // 32), dtype=np.uint8) for _ in range(E)]
+    Su = [r.integers(118, 124, (I, H // 32), dtype=np.uint8) for _ in range(E)]
+    Sd = [r.integers(118, 124, (H, I // 32), dtype=np.uint8) for _ in range(E)]
+    wtab = np.array([[Wg[e].ctypes.data, Wu[e].ctypes.data, Wd[e].ctypes.data] for e in range(E)], dtype=np.uint64)
+    stab = np.array([[Sg[e].ctypes.data, Su[e].ctypes.data, Sd[e].ctypes.data] for e in range(E)], dtype=np.uint64)
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    for t in range(T):
+        tab["eid"][t * k:(t + 1) * k] = r.choice(E, k, replace=False)
+    tab["gate"] = r.random(T * k).astype(np.float32)
+    x = cases.randn_bf16(r, (T, H), 1.0)
+    al = cases.align_arrays(tab, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    meta, _, row_token, row_partidx, row_gate = al
+    R = row_token.shape[0]
+    fu4, fsc = np.full((R, I // 2), 0xAA, np.uint8), np.full((R, I // 32), 0x55, np.uint8)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[I, H, E, 2, T, 1, 0, abi.ARM_A4W4]),
+        [fu4, x, wtab, stab, meta, row_token, row_partidx, fsc], 2)
+    part = np.zeros((T * k, H), np.uint16 if p16 else np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, 5, 6, 7],
+                         i=[H, I, E, 2, 0, 0, 0, abi.ARM_A4W4_P16 if p16 else abi.ARM_A4W4]),
+        [part, fu4, wtab, stab, meta, fsc, row_partidx, row_gate], 2)
+
+    xq = mx_dequant(*mx_act_quant(oracle, ol.bf2f(x)))      # the quantizer is pinned by the three tests above
+    seen = 0
+    for e in range(E):
+        r0, cnt = int(meta[e]), int(meta[E + e])
+        g64, u64, d64 = mx_dequant(Wg[e], Sg[e]), mx_dequant(Wu[e], Su[e]), mx_dequant(Wd[e], Sd[e])
+        for row in range(r0, r0 + cnt):
+            a = xq[row_token[row]]
+            gt, up = (g64 @ a).astype(np.float32).astype(np.float64), (u64 @ a).astype(np.float32).astype(np.float64)
+            v = (gt / (1.0 + np.exp(-gt)) * up).astype(np.float32)
+            wq, ws = mx_act_quant(oracle, v[None, :])
+            # the oracle's f32 SiLU and this f64 one may differ in the last bit: a value on a rounding boundary
+            # may take the neighbouring code
+            got, want = mx_dequant(fu4[row:row + 1], fsc[row:row + 1])[0], mx_dequant(wq, ws)[0]
+            assert np.array_equal(fsc[row], ws[0]) and np.mean(got != want) <= 1 / 32, row
+            np.testing.assert_allclose(got, want, rtol=0, atol=0.5 * np.abs(want).max())
+            p = (d64 @ got) * float(row_gate[row])
+            have = ol.bf2f(part[row_partidx[row]]) if p16 else part[row_partidx[row]]
+            np.testing.assert_allclose(have, p, rtol=2 ** -8 if p16 else 1e-6, atol=1e-30)
+            seen += 1
+    assert seen == T * k
+    pad = row_partidx == abi.EXPERT_UNUSED
+    assert pad.any() and np.all(fu4[pad] == 0xAA) and np.all(fsc[pad] == 0x55)
