@@ -110,6 +110,19 @@ def test_c3_dsv3_prefill_4k(moe, oracle):
     assert cnt[:cfg.E].max() >= 2.0 * cnt[:cfg.E].mean()        # the skew the configuration asks for
 
 
+def test_c4_kimi_k2_mxfp4_prefill_fp4_activations(moe, oracle):
+    """The Kimi-K2 shape at prefill on the fp4 x fp4 arm (activations quantized to mxfp4 per 32 values), expert
+    popularity falling off like 1 / rank so that the hottest expert spans more than one 128-row tile."""
+    print("[case] c4 a4w4 T=2048", flush=True)
+    cfg = layer.config("c4", 2048)
+    cfg.arm = "a4w4"
+    plan = layer.plan_layer(cfg)
+    dev = synth.bind(plan, "cuda", seed=0, zipf=1.0)
+    run_device(moe, plan, dev)
+    cnt = check_prefill_sampled(oracle, cfg, plan, dev)
+    assert cnt[:cfg.E].max() > 128      # more than one row tile
+
+
 @pytest.mark.parametrize("arm", ["w8a8", "a16"])
 def test_c6_glm_tp8_slice_prefill_8k(moe, oracle, arm):
     """The shape of plow's own gfx950 prefill bench (288 experts, top-8, H 4096, I 256 per rank, 8192
@@ -175,6 +188,14 @@ def report_rows(what, a, b, bar):
 
 def e4m3_to_f32(u8):
     return torch.from_numpy(np.ascontiguousarray(u8)).view(torch.float8_e4m3fn).float().numpy()
+
+
+def mxfp4_to_f64(codes, scales):
+    """mxfp4 rows [R][n / 2] (element 2i in the low nibble of byte i) with E8M0 rows [R][n / 32]"""
+    ladder = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+    c = np.stack([codes & 0xF, codes >> 4], axis=-1).reshape(codes.shape[0], -1)
+    v = ladder[c & 7] * np.where(c & 8, -1.0, 1.0)
+    return v * np.repeat(np.exp2(scales.astype(np.float64) - 127.0), 32, axis=1)
 
 
 def check_prefill_sampled(oracle, cfg, plan, dev):
@@ -244,7 +265,11 @@ def check_prefill_sampled(oracle, cfg, plan, dev):
     def gather(name, idx_t):
         return dev.t[name][idx_t].cpu()
 
-    if w8a8 and not pc:
+    if cfg.arm == "a4w4":
+        fu_d = mxfp4_to_f64(gather("fu4", rd_t).numpy(), gather("fsc", rd_t).numpy())
+        fu_s = mxfp4_to_f64(sh.np("fu4")[rs], sh.np("fsc")[rs])
+        report_rows(f"{cfg.name} fu4*fsc (dequantized intermediate)", fu_d, fu_s, REL_L2_MID)
+    elif w8a8 and not pc:
         fq_d = e4m3_to_f32(gather("fq", rd_t).numpy()) * np.repeat(gather("fs", rd_t).numpy(), 128, axis=1)
         fq_s = e4m3_to_f32(sh.np("fq")[rs]) * np.repeat(sh.np("fs")[rs], 128, axis=1)
         report_rows(f"{cfg.name} fq*fs (dequantized intermediate)", fq_d, fq_s, REL_L2_MID)
