@@ -117,6 +117,16 @@ enum {
     PLOW_DOP_MOE_DOWN_FP8_BLOCK128         = 190
 };
 
+/* Op 180 with i7 = PLOW_ROUTER_RAW_MARK: the decode router's score with its top-k in one launch
+ * (crates/packet/src/dev.rs:90-94, runtime/amd/router_decode.hip:1-63; plowrt routes such an op to
+ * router_decode_gfx950.elf). On top of the score's operands (t0 logits f32 [rows][n_exp], t1 x, t2 W,
+ * i0 rows, i1 n_exp, i2 K): t3 = routing table, t4 = selection bias, t5 = arrival counters (u32, one per
+ * row, 32 words apart, zero between launches: the kernel leaves them zero), i3 = k, i4 = router flags
+ * (PLOW_ROUTE_F32_LOGIT set), i5 bit 0 = shared tail slot, i6 = n_group | topk_group << 16, f0 = route
+ * scale. Logits and table are the bytes of op 180 followed by op 83. i5 bit 1 (signal the interpreter's
+ * counters) is refused. */
+#define PLOW_ROUTER_RAW_MARK 0x52545241u
+
 /* Weight encodings (i3 on ops 85/86, i6 on ops 48/49; dev_isa.h:442-461, :691-702). */
 enum { PLOW_MOE_ENC_BF16 = 0, PLOW_MOE_ENC_FP8BLK = 1, PLOW_MOE_ENC_MXFP4 = 2 };
 

@@ -1438,7 +1438,22 @@ int plow_oracle_exec(const PlowDevInst* inst, void* const* tensors, uint32_t nth
         e4m3_lut_ready = 1;
     }
     const unsigned mode = fp_mode_enter();
-    const int rc = exec_one(fn, inst, tensors, nthreads);
+    int rc = exec_one(fn, inst, tensors, nthreads);
+    if (!rc && inst->op == PLOW_DOP_GEMM_F32 && inst->i[7] == PLOW_ROUTER_RAW_MARK) {
+        /* the score op that carries its top-k (plow crates/packet/src/dev.rs:90-94,
+         * runtime/amd/router_decode.hip:1-63): the table bytes are those of the op pair, so the top-k is
+         * op 83 over the logits just written: t3 table, t4 bias, i3 k, i4 flags, i5 bit 0 shared tail,
+         * i6 = n_group | topk_group << 16, f0 route scale; the counters (t5) are left as they were */
+        PlowDevInst tk;
+        memset(&tk, 0, sizeof tk);
+        tk.op = PLOW_DOP_MOE_ROUTER_TOPK_PF;
+        tk.t[0] = inst->t[3], tk.t[1] = inst->t[0], tk.t[2] = PLOW_TENSOR_NONE, tk.t[3] = inst->t[4];
+        for (int q = 4; q < 8; q++) tk.t[q] = PLOW_TENSOR_NONE;
+        tk.i[1] = inst->i[1], tk.i[2] = inst->i[3], tk.i[3] = inst->i[4], tk.i[4] = inst->i[0];
+        tk.i[5] = inst->i[5] & 1u, tk.i[6] = inst->i[6] & 0xFFFFu, tk.i[7] = inst->i[6] >> 16;
+        tk.fj[0].f = inst->fj[0].f;
+        rc = exec_one(op_router_topk, &tk, tensors, nthreads);
+    }
     fp_mode_leave(mode);
     return rc;
 }

@@ -189,6 +189,29 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
     case PLOW_DOP_GEMM_F32: {
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2), "op 180: t0 logits, t1 x, t2 W must be bound");
         NEED(c, i[0] && i[1] && i[2] && i[2] % 8u == 0u, "op 180: M, N, K must be non-zero and K a multiple of 8");
+        if (i[7] == PLOW_ROUTER_RAW_MARK) {
+            /* the score carries its top-k (plow crates/packet/src/dev.rs:90-94): one launch where the few-token
+             * score kernel serves the shape, the two launches otherwise; the same bytes either way */
+            const uint32_t E = i[1], k = i[3], flags = i[4], ng = i[6] & 0xFFFFu, tg = i[6] >> 16;
+            NEED(c, ten(in, T, 3) && ten(in, T, 5), "op 180 (router): t3 table and t5 counters must be bound");
+            NEED(c, E <= 1024u && k >= 1u, "op 180 (router): n_exp %u above 1024 or k = 0", E);
+            NEED(c, (flags & PLOW_ROUTE_F32_LOGIT) != 0u, "op 180 (router): the top-k reads the f32 logits, flag bit 3 must be set");
+            NEED(c, ((flags & PLOW_ROUTE_BIAS) != 0u) == (ten(in, T, 4) != nullptr), "op 180 (router): bias flag (bit 2) and the t4 binding disagree");
+            if (ng > 1u && tg > 0u && tg < ng)
+                NEED(c, ng <= PLOW_ROUTE_MAX_GROUPS && E % ng == 0u && E / ng >= 2u && (uint64_t)tg * (E / ng) >= (k < 16u ? k : 16u),
+                     "op 180 (router): group shape n_group=%u topk_group=%u is not selectable for n_exp=%u k=%u", ng, tg, E, k);
+            if (i[5] & ~1u) return fail(c, PLOW_MOE_EUNSUPPORTED, "op 180 (router): i5 = %u asks for a signal to the interpreter's counters", i[5]);
+            if (!launch) return 0;
+            RouterRun r = {};
+            r.logit = ten(in, T, 0), r.x = ten(in, T, 1), r.w = ten(in, T, 2), r.M = i[0], r.N = E, r.K = i[2];
+            r.table = ten(in, T, 3), r.bias = (const float*)ten(in, T, 4), r.row_ctr = (uint32_t*)ten(in, T, 5);
+            r.k = k, r.flags = flags, r.tail = i[5] & 1u, r.n_group = ng, r.topk_group = tg;
+            r.route_scale = in->fj[0].f;
+            if (router_decode_serves(r)) return launch_router_decode(r, st);
+            const int src = launch_router_score((float*)r.logit, r.x, r.w, r.M, r.N, r.K, st);
+            if (src) return src;
+            return launch_router_topk(r.table, r.logit, r.bias, E, k, flags, r.M, r.tail, ng, tg, r.route_scale, 0.0f, st);
+        }
         if (!launch) return 0;
         return launch_router_score((float*)ten(in, T, 0), ten(in, T, 1), ten(in, T, 2), i[0], i[1], i[2], st);
     }

@@ -15,6 +15,24 @@ int launch_router_topk(void* table, const void* logit, const float* bias, uint32
 int launch_align(int32_t* meta, const void* table, uint32_t* row_token, uint32_t* row_partidx,
                  float* row_gate, uint32_t T, uint32_t E, uint32_t k, uint32_t* chunk_hist,
                  uint32_t chunk_cap, hipStream_t st);
+
+/* The decode router's score with its top-k in one launch (op 180 with the router mark). Every field has
+ * the meaning it has on the separate launchers above; `logit` is f32 [M][N] and PLOW_ROUTE_F32_LOGIT is set
+ * in flags. `row_ctr`: the caller's arrival counters, one word per row, 32 words apart, zero between
+ * launches (the kernel leaves them zero) and used by one launch at a time. */
+struct RouterRun {
+    void* logit;
+    const void* x;
+    const void* w;
+    uint32_t M, N, K;
+    void* table;
+    const float* bias;
+    uint32_t k, flags, tail, n_group, topk_group;
+    float route_scale, logit_scale;
+    uint32_t* row_ctr;
+};
+bool router_decode_serves(const RouterRun& r);
+int launch_router_decode(const RouterRun& r, hipStream_t st);
 int launch_combine(void* out, const void* residual, const void* shared, const void* part, uint32_t H,
                    uint32_t k, uint32_t T, uint32_t part16, hipStream_t st);
 /* the deterministic fused combine: acc is the f64 [T][H] fixed-point accumulator the DOWN op summed in place */

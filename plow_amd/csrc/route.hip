@@ -534,19 +534,20 @@ __global__ __launch_bounds__(128) void k_router_score_wave(float* __restrict__ o
 #define RSR_PF 4
 #define RSR_STAGERS 4u
 #define RSR_WS_BYTES (2u * 64u * RSR_LD * 4u)
+/* The body takes its workgroup coordinates (expert tile bx, token group by) and its LDS as arguments, so
+ * that the fused decode router below can run it and carry on. Every wave returns from it (the stagers
+ * early), after the same number of barriers. */
 template <uint32_t TOK>
-__global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(float* __restrict__ out,
-                                                                                const bf16_t* __restrict__ x,
-                                                                                const bf16_t* __restrict__ w,
-                                                                                uint32_t M, uint32_t N, uint32_t K) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t rsr_raw[];
+__device__ __forceinline__ void router_score_row_body(float* __restrict__ out, const bf16_t* __restrict__ x,
+                                                      const bf16_t* __restrict__ w, uint32_t M, uint32_t N, uint32_t K,
+                                                      uint32_t bx, uint32_t by, uint8_t* rsr_raw) {
     float* const rsr_ws = (float*)rsr_raw;                        /* [2][64][RSR_LD] f32 weights */
     bf16_t* const rsr_xs = (bf16_t*)(rsr_raw + RSR_WS_BYTES);     /* [2][TOK][RSR_KC] bf16 tokens */
     constexpr int KC = RSR_KC, LD = RSR_LD;
     constexpr int NL = 8 + (int)TOK; /* loads per stager and chunk */
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const uint32_t n0 = blockIdx.x * 64u, m0 = blockIdx.y * TOK;
+    const uint32_t n0 = bx * 64u, m0 = by * TOK;
     const uint32_t NC = K / KC;
     if (wv >= TOK) {
         /* a row of a chunk is 32 16-byte pieces; lane l loads piece l % 32 of rows base + l / 32, + 2, ...
@@ -655,14 +656,23 @@ __global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(
     const uint32_t n = n0 + lane;
     if (m < M && n < N) out[(size_t)m * N + n] = acc;
 }
+template <uint32_t TOK>
+__global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(float* __restrict__ out,
+                                                                                const bf16_t* __restrict__ x,
+                                                                                const bf16_t* __restrict__ w,
+                                                                                uint32_t M, uint32_t N, uint32_t K) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t rsr_raw[];
+    router_score_row_body<TOK>(out, x, w, M, N, K, blockIdx.x, blockIdx.y, rsr_raw);
+}
 
 #define RS16_LDS (4u * RSM_STAGES * (uint32_t)sizeof(Rs16Stage))
 #define RSM_LDS (4u * RSM_STAGES * (uint32_t)sizeof(RsmStage))
 #define RSR_LDS (RSR_WS_BYTES + 2u * 4u * RSR_KC * 2u)
 
 /* dynamic-LDS limits of the score kernels, once per device (plow_moe_device_setup) */
+static bool rf_setup();
 int plow_moe_route_setup() {
-    const bool ok =
+    const bool ok = rf_setup() &&
         hipFuncSetAttribute((const void*)k_router_score_mfma16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RS16_LDS) == hipSuccess &&
         hipFuncSetAttribute((const void*)k_router_score_mfma, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSM_LDS) == hipSuccess &&
         hipFuncSetAttribute((const void*)k_router_score_row<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess &&
@@ -748,13 +758,10 @@ __device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
     return ab > cd ? ab : cd;
 }
 
+/* one token by one wave; `score` is the wave's own 64 * RT_EPL floats of LDS */
 template <uint32_t RT_EPL> /* experts per lane: n_exp <= 64 * RT_EPL */
-__global__ __launch_bounds__(RT_WAVES* WAVE) void k_router_topk(RouterArgs a) {
-    __shared__ float s_score[RT_WAVES][64u * RT_EPL];
-    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
-    const uint32_t tok = blockIdx.x * RT_WAVES + wv;
-    if (tok >= a.T) return; /* whole wave leaves together; no block-level barrier below */
-    float* score = s_score[wv];
+__device__ __forceinline__ void router_topk_token(const RouterArgs& a, uint32_t tok, float* score) {
+    const uint32_t lane = threadIdx.x & 63u;
     const uint32_t E = a.n_exp;
     const bool sigmoid = a.flags & PLOW_ROUTE_SIGMOID, norm = a.flags & PLOW_ROUTE_NORM_TOPK;
     const bool f32l = a.flags & PLOW_ROUTE_F32_LOGIT;
@@ -903,6 +910,21 @@ __global__ __launch_bounds__(RT_WAVES* WAVE) void k_router_topk(RouterArgs a) {
         row[a.k].gate = 1.0f;
     }
 }
+template <uint32_t RT_EPL>
+__global__ __launch_bounds__(RT_WAVES* WAVE) void k_router_topk(RouterArgs a) {
+    __shared__ float s_score[RT_WAVES][64u * RT_EPL];
+    const uint32_t wv = threadIdx.x >> 6;
+    const uint32_t tok = blockIdx.x * RT_WAVES + wv;
+    if (tok >= a.T) return; /* whole wave leaves together; no block-level barrier below */
+    router_topk_token<RT_EPL>(a, tok, s_score[wv]);
+}
+/* the same with the form picked inside the kernel (the fused decode routers) */
+__device__ __forceinline__ void router_topk_token_any(const RouterArgs& a, uint32_t tok, float* score) {
+    if (a.n_exp <= 128u) router_topk_token<2>(a, tok, score);
+    else if (a.n_exp <= 256u) router_topk_token<4>(a, tok, score);
+    else if (a.n_exp <= 512u) router_topk_token<8>(a, tok, score);
+    else router_topk_token<16>(a, tok, score);
+}
 
 int launch_router_topk(void* table, const void* logit, const float* bias, uint32_t n_exp, uint32_t k,
                        uint32_t flags, uint32_t T, uint32_t tail, uint32_t n_group, uint32_t topk_group,
@@ -940,28 +962,30 @@ struct AlignArgs {
     uint32_t T, E, k;
 };
 
-__global__ __launch_bounds__(AL_WAVES* WAVE) void k_align(AlignArgs a) {
-    __shared__ uint32_t hist[AL_WAVES][AL_MAX_E];
-    __shared__ uint32_t s_rowoff[AL_MAX_E];
-    __shared__ uint32_t s_cnt[AL_MAX_E];
-    __shared__ uint32_t s_carry;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
+/* LDS words the single-workgroup align needs with nw waves */
+#define AL_LDS_WORDS(nw) (((nw) + 2u) * AL_MAX_E + 1u)
+/* The whole workgroup (nw waves) calls this; lds: AL_LDS_WORDS(nw) words. */
+__device__ __forceinline__ void align_body(const AlignArgs& a, uint32_t* lds, uint32_t nw) {
+    uint32_t(*hist)[AL_MAX_E] = (uint32_t(*)[AL_MAX_E])lds;
+    uint32_t* const s_rowoff = lds + nw * AL_MAX_E;
+    uint32_t* const s_cnt = s_rowoff + AL_MAX_E;
+    uint32_t& s_carry = s_cnt[AL_MAX_E];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6, nthr = nw * WAVE;
     const uint32_t E = a.E, nslot = a.T * a.k;
     /* slots per wave, a multiple of 64 so that every step of phase C is a whole wave */
-    const uint32_t per = ((nslot + AL_WAVES * WAVE - 1u) / (AL_WAVES * WAVE)) * WAVE;
-    const uint32_t lo = wv * per, hi = lo + per < nslot ? lo + per : nslot;
+    const uint32_t per = ((nslot + nthr - 1u) / nthr) * WAVE;
+    const uint32_t lo = wv * per < nslot ? wv * per : nslot, hi = lo + per < nslot ? lo + per : nslot;
 
-    for (uint32_t i = tid; i < AL_WAVES * E; i += AL_WAVES * WAVE) hist[i / E][i % E] = 0u;
+    for (uint32_t i = tid; i < nw * E; i += nthr) hist[i / E][i % E] = 0u;
     __syncthreads();
     for (uint32_t s = lo + lane; s < hi; s += WAVE) {
         const uint32_t e = a.table[s].eid;
         if (e < E) atomicAdd(&hist[wv][e], 1u);
     }
     __syncthreads();
-    for (uint32_t e = tid; e < E; e += AL_WAVES * WAVE) {
+    for (uint32_t e = tid; e < E; e += nthr) {
         uint32_t run = 0;
-#pragma unroll
-        for (uint32_t w = 0; w < AL_WAVES; w++) {
+        for (uint32_t w = 0; w < nw; w++) {
             const uint32_t c = hist[w][e];
             hist[w][e] = run;
             run += c;
@@ -997,7 +1021,7 @@ __global__ __launch_bounds__(AL_WAVES* WAVE) void k_align(AlignArgs a) {
     }
     __syncthreads();
     /* pad rows: [rowoff + cnt, rowoff + 64 * ceil(cnt / 64)) */
-    for (uint32_t i = tid; i < E * PLOW_MPF_BM; i += AL_WAVES * WAVE) {
+    for (uint32_t i = tid; i < E * PLOW_MPF_BM; i += nthr) {
         const uint32_t e = i / PLOW_MPF_BM, j = i % PLOW_MPF_BM;
         const uint32_t c = s_cnt[e], r = s_rowoff[e] + c + j;
         if (c + j < ((c + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM) {
@@ -1033,6 +1057,80 @@ __global__ __launch_bounds__(AL_WAVES* WAVE) void k_align(AlignArgs a) {
             a.row_gate[pos] = g;
         }
     }
+}
+__global__ __launch_bounds__(AL_WAVES* WAVE) void k_align(AlignArgs a) {
+    __shared__ uint32_t al_lds[AL_LDS_WORDS(AL_WAVES)];
+    align_body(a, al_lds, AL_WAVES);
+}
+
+/* ============================ the decode router's score with its top-k in one launch ============ */
+/* Op 180 marked as carrying its top-k (plow crates/packet/src/dev.rs:90-94, runtime/amd/
+ * router_decode.hip:1-63). The score workgroups of a token group count themselves off on the group's
+ * arrival counter; the last to arrive runs the top-k of the group's tokens, one wave per token. The
+ * bodies are those of the separate kernels: same logits, same table. A counter is zero between launches
+ * (the last arrival puts it back); launches that share counters must not overlap. */
+struct RouterFuse {
+    uint32_t* ctr;       /* token group g counts itself off on ctr[g * stride] */
+    uint32_t stride;
+    RouterArgs topk;
+};
+/* this workgroup was the last of `n` to add itself to *ctr (every thread gets the answer); what the
+ * workgroup wrote before is visible to whoever comes last, and the last sees everyone's writes */
+__device__ __forceinline__ bool rf_last_arrival(uint32_t* ctr, uint32_t n, uint32_t* s_flag) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t last = old == n - 1u ? 1u : 0u;
+        if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_flag = last;
+    }
+    __syncthreads();
+    const bool last = *s_flag != 0u;
+    if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return last;
+}
+template <uint32_t TOK>
+__global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_decode(float* __restrict__ out,
+                                                                             const bf16_t* __restrict__ x,
+                                                                             const bf16_t* __restrict__ w,
+                                                                             uint32_t M, uint32_t N, uint32_t K, RouterFuse f) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t rsr_raw[];
+    __shared__ uint32_t s_flag;
+    router_score_row_body<TOK>(out, x, w, M, N, K, blockIdx.x, blockIdx.y, rsr_raw);
+    if (!rf_last_arrival(f.ctr + (size_t)blockIdx.y * f.stride, gridDim.x, &s_flag)) return;
+    const uint32_t wv = threadIdx.x >> 6, tok = blockIdx.y * TOK + wv;
+    if (wv < TOK && tok < M) router_topk_token_any(f.topk, tok, (float*)rsr_raw + wv * RT_MAX_E);
+}
+static_assert(RSR_LDS >= 4u * RT_MAX_E * 4u, "the top-k borrows the score kernel's LDS");
+
+static bool rf_setup() {
+    return hipFuncSetAttribute((const void*)k_router_decode<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess &&
+           hipFuncSetAttribute((const void*)k_router_decode<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess;
+}
+
+/* The one-launch form serves the shapes the few-token score kernel above serves (below 16 tokens, K a
+ * multiple of its chunk, 32-bit lane offsets). */
+bool router_decode_serves(const RouterRun& r) {
+    return r.row_ctr && r.table && r.logit && r.x && r.w && r.M >= 1u && r.M < 16u && r.N >= 1u && r.N <= RT_MAX_E &&
+           r.k >= 1u && !plow_moe_tuning().score_tile8 && r.K % RSR_KC == 0u && (uint64_t)r.N * r.K * 2u < (1ull << 31) &&
+           (uint64_t)r.M * r.K * 2u < (1ull << 31);
+}
+int launch_router_decode(const RouterRun& r, hipStream_t st) {
+    if (!router_decode_serves(r)) return PLOW_MOE_EINVAL;
+    RouterFuse f = {};
+    const uint32_t tok = r.M >= 4u ? 2u : 1u;
+    f.ctr = r.row_ctr, f.stride = tok * 32u; /* one counter per row, 32 words apart: a group takes its first row's */
+    f.topk = {(PlowMoeRoute*)r.table, r.logit, r.bias, r.N, r.k, r.flags, r.M, r.tail, r.n_group, r.topk_group,
+              r.route_scale, r.logit_scale};
+    const uint32_t nx = (r.N + 63u) / 64u;
+    if (tok == 2u)
+        k_router_decode<2><<<dim3(nx, (r.M + 1u) / 2u), (2u + RSR_STAGERS) * 64u, RSR_LDS, st>>>(
+            (float*)r.logit, (const bf16_t*)r.x, (const bf16_t*)r.w, r.M, r.N, r.K, f);
+    else
+        k_router_decode<1><<<dim3(nx, r.M), (1u + RSR_STAGERS) * 64u, RSR_LDS, st>>>(
+            (float*)r.logit, (const bf16_t*)r.x, (const bf16_t*)r.w, r.M, r.N, r.K, f);
+    return 0;
 }
 
 /* Many slots (prefill): the same counting sort spread over the chip in three launches.

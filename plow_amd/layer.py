@@ -43,6 +43,7 @@ class MoeConfig:
     act_f: Tuple[float, float] = (0.0, 0.0)  # the activation's immediates (fj[0], fj[1]) for the pair forms 2 / 3 / 4
     residual: bool = False
     part_bf16: bool = False         # block-fp8 W8A8 only: bf16 partials (arm 3) instead of f32
+    router_raw: bool = False        # the score op carries its top-k (op 180 with the router mark): one launch at decode
     det_combine: bool = False       # block-fp8 W8A8 only: the deterministic fused down -> combine (op 83 zeroes a
                                     # [T][H] f64 fixed-point accumulator, op 86 adds into it, op 87 reads it as
                                     # one stream; plow runtime/amd/op_moe.h:2110-2165); no part tensor
@@ -154,11 +155,19 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
     out = p._t("out", "bf16", (T, H), "out")
     residual = p._t("residual", "bf16", (T, H), "in") if cfg.residual else None
 
-    if with_router_score:
+    if cfg.router_raw:
+        # plow's raw router segment (crates/devgen/src/mla.rs:3294-3312): per-row arrival counters, 128 bytes apart
+        assert with_router_score and not det
+        ctr = p._t("router_ctr", "u32", (T * 32,), "scratch")
+        p._emit("score", abi.inst(abi.OP_GEMM_F32, t=[logit, x, wr, table, bias, ctr],
+                                  i=[T, E, H, k, cfg.flags, cfg.tail, cfg.n_group | (cfg.topk_group << 16),
+                                     abi.ROUTER_RAW_MARK], f=[cfg.route_scale, 0.0]))
+    elif with_router_score:
         p._emit("score", abi.inst(abi.OP_GEMM_F32, t=[logit, x, wr], i=[T, E, H]))
-    p._emit("topk", abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[table, logit, part if det else None, bias],
-                             i=[H if det else 0, E, k, cfg.flags, T, cfg.tail, cfg.n_group, cfg.topk_group],
-                             f=[cfg.route_scale, 0.0]))
+    if not cfg.router_raw:
+        p._emit("topk", abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[table, logit, part if det else None, bias],
+                                 i=[H if det else 0, E, k, cfg.flags, T, cfg.tail, cfg.n_group, cfg.topk_group],
+                                 f=[cfg.route_scale, 0.0]))
     p._emit("align", abi.inst(abi.OP_MOE_ALIGN_PF, t=[meta, table, row_token, row_partidx, row_gate],
                               i=[T, Ea, ka]))
 

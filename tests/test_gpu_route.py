@@ -1,5 +1,6 @@
 """Routing on the GPU (ops 180, 83, 84, 87, 184, 32) against golden vectors from plow's CPU kernels
 and against the oracle: everything bit-exact."""
+import ctypes as C
 import os
 
 import numpy as np
@@ -245,3 +246,59 @@ def test_rmsnorm_with_fused_quantizers(moe, oracle, rows, feat, gamma):
             ol.run(oracle.plow_oracle_exec, abi.inst(op, t=[0, 1, 2], i=[rows, feat]), ol.table_of([q2, row_in, s2]), 2)
             assert np.array_equal(xq.cpu().numpy(), q2)
             assert np.array_equal(sc.cpu().numpy().view(np.uint32), s2.view(np.uint32))
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 5, 15, 16, 40])
+@pytest.mark.parametrize("shape", ["dsv3", "qwen", "kimi"])
+def test_router_score_that_carries_its_topk_equals_the_op_pair(moe, oracle, T, shape):
+    """Op 180 with the router mark (plow's raw router segment): below 16 tokens one launch in which the
+    score's workgroups count themselves off and the last arrival of a token group runs its top-k, two
+    launches from there. Logits and table are the bytes of op 180 followed by op 83, on the device and in
+    the oracle; also on a second run (the counters are back at zero), with the counters left zero."""
+    from plow_amd import layer, synth
+    kw = {"dsv3": dict(H=1024, E=256, I=256, k=8, scoring="sigmoid", norm_topk=True, bias=True, n_group=8, topk_group=4,
+                       route_scale=2.5, n_shared=1, shared_mode="fold"),
+          "qwen": dict(H=512, E=128, I=256, k=8, scoring="softmax", norm_topk=True),
+          "kimi": dict(H=768, E=384, I=256, k=8, scoring="sigmoid", norm_topk=True, bias=True, route_scale=2.827,
+                       n_shared=1, shared_mode="fold")}[shape]
+    pair = layer.plan_layer(layer.MoeConfig(f"router-{shape}", T=T, enc="bf16", arm="a16", **kw))
+    raw = layer.plan_layer(layer.MoeConfig(f"router-raw-{shape}", T=T, enc="bf16", arm="a16", router_raw=True, **kw))
+    assert "topk" not in raw.names
+    ref = synth.bind(pair, "cuda", seed=T)
+    moe.exec_many([pair.insts[pair.index(l)] for l in ("score", "topk")], ref.table())
+    torch.cuda.synchronize()
+    dev = synth.bind(raw, "cuda", seed=T)
+    host = synth.to_host(dev)
+    for rep in range(2):
+        dev.t["logit"].fill_(float("nan"))
+        dev.t["table"].fill_(-1)
+        moe.exec(raw.insts[raw.index("score")], dev.table())
+        torch.cuda.synchronize()
+        assert np.array_equal(dev.np("logit").view(np.uint32), ref.np("logit").view(np.uint32)), rep
+        assert np.array_equal(dev.np("table"), ref.np("table")), rep
+        assert not dev.np("router_ctr").any()
+    ol.run(oracle.plow_oracle_exec, raw.insts[raw.index("score")], host.table(), 4)
+    assert np.array_equal(host.np("logit").view(np.uint32), ref.np("logit").view(np.uint32))
+    assert np.array_equal(host.np("table"), ref.np("table"))
+
+
+def test_router_score_that_carries_its_topk_refusals(moe):
+    from plow_amd import layer, synth
+    plan = layer.plan_layer(layer.MoeConfig("router-raw", T=2, H=512, E=64, I=256, k=4, scoring="sigmoid", bias=True,
+                                            enc="bf16", arm="a16", router_raw=True))
+    dev = synth.bind(plan, "cuda", seed=1)
+    good = plan.insts[plan.index("score")]
+    assert moe.check(good, dev.table()) == 0
+
+    def variant(**kw):
+        c = abi.PlowDevInst()
+        C.memmove(C.byref(c), C.byref(good), C.sizeof(c))
+        for name, (idx, val) in kw.items():
+            getattr(c, name)[idx] = val
+        return c
+    assert moe.check(variant(t=(5, abi.TENSOR_NONE)), dev.table()) == abi.E_INVAL          # no counters
+    assert moe.check(variant(t=(3, abi.TENSOR_NONE)), dev.table()) == abi.E_INVAL          # no table
+    assert moe.check(variant(t=(4, abi.TENSOR_NONE)), dev.table()) == abi.E_INVAL          # bias flag without a bias
+    assert moe.check(variant(i=(4, good.i[4] & ~abi.ROUTE_F32_LOGIT)), dev.table()) == abi.E_INVAL
+    assert moe.check(variant(i=(3, 0)), dev.table()) == abi.E_INVAL                          # k = 0
+    assert moe.check(variant(i=(5, 2)), dev.table()) == abi.E_UNSUPPORTED                   # interpreter signal

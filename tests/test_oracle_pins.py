@@ -768,3 +768,24 @@ def test_a4w4_arm_against_f64_over_the_same_bytes(oracle, p16):
     assert seen == T * k
     pad = row_partidx == abi.EXPERT_UNUSED
     assert pad.any() and np.all(fu4[pad] == 0xAA) and np.all(fsc[pad] == 0x55)
+
+
+def test_router_score_that_carries_its_topk_is_the_op_pair(oracle):
+    """Op 180 with the router mark writes the logits of op 180 and the table of op 83 over them (the pair is
+    pinned above and by plow's golden vectors); the counters stay as they were."""
+    r = cases.rng_of(41)
+    T, E, H, k = 5, 64, 256, 4
+    x, w = cases.randn_bf16(r, (T, H), 1.0), cases.randn_bf16(r, (E, H), 0.05)
+    bias = (r.standard_normal(E) * 0.01).astype(np.float32)
+    flags = abi.ROUTE_SIGMOID | abi.ROUTE_NORM_TOPK | abi.ROUTE_BIAS | abi.ROUTE_F32_LOGIT
+    logit = np.zeros((T, E), np.float32)
+    table = np.zeros(T * (k + 1), dtype=ol.ROUTE_DT)
+    run(oracle, abi.inst(abi.OP_GEMM_F32, t=[0, 1, 2], i=[T, E, H]), [logit, x, w], 3)
+    run(oracle, abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1, None, 3], i=[0, E, k, flags, T, 1, 8, 4], f=[2.5, 0.0]),
+        [table, logit, None, bias], 3)
+    logit2, table2 = np.zeros_like(logit), np.zeros_like(table)
+    ctr = np.full(T * 32, 7, np.uint32)
+    run(oracle, abi.inst(abi.OP_GEMM_F32, t=[0, 1, 2, 3, 4, 5], i=[T, E, H, k, flags, 1, 8 | (4 << 16), abi.ROUTER_RAW_MARK],
+                         f=[2.5, 0.0]), [logit2, x, w, table2, bias, ctr], 3)
+    assert np.array_equal(logit.view(np.uint32), logit2.view(np.uint32))
+    assert np.array_equal(table, table2) and table["eid"].max() == E and np.all(ctr == 7)
