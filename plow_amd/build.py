@@ -27,6 +27,7 @@ SOURCES = {
     "quant.hip": ["-ffp-contract=off"],
     "experts_w8a8.hip": [],
     "experts_a16.hip": [],
+    "experts_gemv.hip": [],
     "experts_w8a8_tiled.hip": [],
     "api.hip": [],
     "device.hip": [],

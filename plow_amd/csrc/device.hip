@@ -30,6 +30,7 @@ const PlowMoeTuning& plow_moe_tuning() {
         const char* f = getenv("PLOW_MOE_SCORE_MFMA32_FROM");
         t.score_mfma32_from = f ? strtoull(f, nullptr, 10) : 0ull;
         t.a16_tiled = !is("PLOW_MOE_A16_TILED", "0");
+        t.a16_gemv = !is("PLOW_MOE_A16_GEMV", "0");
     });
     return t;
 }

@@ -725,6 +725,7 @@ template <bool GLU>
 static int launch_a16(const GroupA16& g, hipStream_t st) {
     if (g.N == 0 || g.K == 0 || g.E == 0 || g.N % AK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
     if ((uint64_t)g.E * (g.N / AK_BN) > 0x7FFFFFFFull) return PLOW_MOE_EINVAL;
+    if (group_a16_gemv_serves(g)) return launch_group_a16_gemv(g, GLU, st); /* a handful of rows in all */
     {
         int rc = 0;
         if (a16_tiled_try<GLU>(g, st, &rc)) return rc;

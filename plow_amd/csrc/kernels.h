@@ -133,6 +133,9 @@ struct GroupA16 {
     uint32_t bias_rows;
     const void* wdirect[2]; /* used when wtab is NULL: the two weight tensors themselves (dense ops) */
 };
+/* the matrix-vector form of the same ops for batches that route a handful of rows in all (slots_hint says so) */
+bool group_a16_gemv_serves(const GroupA16& g);
+int launch_group_a16_gemv(const GroupA16& g, bool glu, hipStream_t st);
 int launch_group_glu_a16(const GroupA16& g, hipStream_t st);
 int launch_group_down_a16(const GroupA16& g, hipStream_t st);
 /* wtab / stab rows {p, p, p} for the experts of one flat tensor: p = W + e * w_stride, S + e * s_stride */

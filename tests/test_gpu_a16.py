@@ -10,8 +10,9 @@ import torch
 
 import cases
 import oracle_lib as ol
-from gpu_harness import (assert_output_close, assert_routing_equal, both, dev_table, from_dev, to_dev)
-from plow_amd import abi, layer
+from gpu_harness import (assert_output_close, assert_routing_equal, both, dev_table, from_dev, run_device, run_oracle,
+                         to_dev)
+from plow_amd import abi, layer, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -373,3 +374,32 @@ def test_bf16_grouped_fused_table_ops(moe, oracle, act):
     touched = part_h != 9.0
     assert np.array_equal(part_g != 9.0, touched)
     close(part_g[touched], part_h[touched], "part", mean_rel=1e-4, max_frac=1e-4)
+
+
+@pytest.mark.parametrize("enc,H,I", [("bf16", 384, 256), ("bf16", 2048, 1408), ("fp8blk", 640, 384), ("fp8blk", 7168, 256),
+                                     ("mxfp4", 768, 256), ("mxfp4", 3584, 512), ("fp8pc", 1536, 640)])
+@pytest.mark.parametrize("T,k", [(1, 8), (2, 3), (1, 1)])
+def test_matrix_vector_form_at_one_and_two_tokens(moe, oracle, enc, H, I, T, k):
+    """Batches that route a handful of rows in all run the bf16-activation ops as matrix-vector products
+    (every wave a share of one row's channels, weight rows of 16-byte pieces per lane): row lengths that
+    are not whole kilobytes, rows of one to eight pieces, every encoding, gate folded into the DOWN."""
+    print(f"[case] gemv enc={enc} H={H} I={I} T={T} k={k}", flush=True)
+    cfg = layer.MoeConfig("gemv", T=T, H=H, E=16, I=I, k=k, scoring="sigmoid", norm_topk=True, bias=True,
+                          route_scale=2.5, enc=enc, arm="a16", n_shared=1, shared_mode="fold")
+    assert T * cfg.k_all <= 9
+    check_chain(*both(moe, oracle, cfg, seed=H + T))
+
+
+def test_matrix_vector_form_is_right_when_the_slot_count_is_understated(moe, oracle):
+    """The form is chosen from the routed-slot count the descriptor states. A count that is far too small
+    still gives the layer's result: live rows are walked in windows, an expert's rows one after the other."""
+    cfg = layer.MoeConfig("gemv-lie", T=40, H=512, E=8, I=256, k=4, scoring="softmax", norm_topk=True, enc="mxfp4",
+                          arm="a16", n_shared=1, shared_mode="fold")
+    plan = layer.plan_layer(cfg)
+    for name in ("glu", "down"):
+        plan.insts[plan.index(name)].fj[2].u = 5          # 200 slots in truth
+    dev = synth.bind(plan, "cuda", seed=3)
+    host = synth.to_host(dev)
+    run_device(moe, plan, dev)
+    run_oracle(oracle, plan, host)
+    check_chain(plan, dev, host)
