@@ -16,6 +16,7 @@ LIB = os.path.join(HERE, "libplow_moe_gfx950.so")
 ELF = os.path.join(HERE, "moe_fp8_pf_gfx950.elf")
 ELF_COMBINE = os.path.join(HERE, "moe_combine_gfx950.elf")   # amd.rs:11666-11716
 ELF_DEC = os.path.join(HERE, "moe_w8a8_dec_gfx950.elf")      # amd.rs:10799-10852
+ELF_ROUTER = os.path.join(HERE, "router_decode_gfx950.elf")  # amd.rs:10755-10800
 
 COMMON = ["--offload-arch=gfx950", "-O3", *os.environ.get("PLOW_MOE_EXTRA_FLAGS", "").split(), "-std=c++17", "-fPIC", "-fno-fast-math",
           # packed-FP32 VALU forms are kept out of every kernel
@@ -61,7 +62,8 @@ def build(verbose=True):
     os.makedirs(OBJ, exist_ok=True)
     with cf.ThreadPoolExecutor(max_workers=8) as ex:
         elfs = [ex.submit(_code_object), ex.submit(_code_object, "plowrt_combine_obj.hip", ELF_COMBINE, ("-ffp-contract=off",)),
-                ex.submit(_code_object, "plowrt_dec_obj.hip", ELF_DEC)]
+                ex.submit(_code_object, "plowrt_dec_obj.hip", ELF_DEC),
+                ex.submit(_code_object, "plowrt_router_obj.hip", ELF_ROUTER, ("-ffp-contract=off",))]
         results = list(ex.map(lambda kv: _compile(*kv), SOURCES.items()))
         for f in elfs:
             _, elf_err = f.result()
@@ -80,6 +82,7 @@ def build(verbose=True):
         print("built", ELF)
         print("built", ELF_COMBINE)
         print("built", ELF_DEC)
+        print("built", ELF_ROUTER)
     return LIB
 
 

@@ -1,5 +1,6 @@
 """The device code objects for an unmodified plowrt (plow_amd/moe_fp8_pf_gfx950.elf, the expert GEMMs;
-plow_amd/moe_combine_gfx950.elf, the combine): each ELF carries the kernel symbols, the ABI markers and a
+plow_amd/moe_w8a8_dec_gfx950.elf, the decode pair; plow_amd/moe_combine_gfx950.elf, the combine;
+plow_amd/router_decode_gfx950.elf, the decode router): each ELF carries the kernel symbols, the ABI markers and a
 launch shape plowrt can use (CPU tests); launched the way plowrt launches them (1-D grid, 512 / 256
 threads, no dynamic LDS, one by-value argument block) they match the oracle (GPU tests)."""
 import ctypes as C
@@ -19,6 +20,8 @@ COMBINE_MARKERS = ["plow_moe_combine_fixed_order_abi_1", "plow_moe_combine_fixed
 ELF_DEC = os.path.join(ROOT, "plow_amd", "moe_w8a8_dec_gfx950.elf")
 DEC_MARKER = "plow_moe_w8a8_dec_abi_1"                                            # amd.rs:10810
 DEC_KERNELS = {"plow_moe_w8a8_dec_glu": 96, "plow_moe_w8a8_dec_down": 80, "plow_moe_w8a8_dec_pair": 192}  # amd.rs:10827-10840
+ELF_ROUTER = os.path.join(ROOT, "plow_amd", "router_decode_gfx950.elf")
+ROUTER_MARKER, ROUTER_KERNEL = "plow_router_decode_abi_3", "plow_router_decode"  # amd.rs:10765-10767
 KERNELS = ["plow_moe_fp8_glu_pf_gfx950", "plow_moe_fp8_down_pf_gfx950", "plow_moe_w8a8_glu_pf_gfx950",
            "plow_moe_w8a8_down_pf_gfx950", "plow_moe_w8a8_down_acc_pf_gfx950"]   # amd.rs:11720-11740
 
@@ -120,6 +123,29 @@ def test_decode_object_symbols_and_launch_shape():
         assert seen == 3
 
 
+def test_router_object_symbols_and_launch_shape():
+    """plowrt takes the router object only with its marker, its kernel, a 104-byte argument segment (or 104 +
+    256 bytes of hidden arguments) and no private memory; it launches 512 threads with no dynamic LDS
+    (plow crates/plowrt/src/exec/amd.rs:10755-10800, :17811-17832)."""
+    if not os.path.exists(ELF_ROUTER):
+        pytest.fail(f"{ELF_ROUTER} is not built; run `python -m plow_amd.build`")
+    names, _ = elf_symbols(ELF_ROUTER)
+    assert ROUTER_MARKER in names and ROUTER_KERNEL in names and ROUTER_KERNEL + ".kd" in names
+    import re
+    import subprocess
+    readelf = "/opt/rocm/llvm/bin/llvm-readelf"
+    if os.path.exists(readelf):
+        notes = subprocess.run([readelf, "--notes", ELF_ROUTER], capture_output=True, text=True).stdout
+        assert re.findall(r"\.name:\s+(plow_\S+)\n", notes) == [ROUTER_KERNEL]
+        field = lambda f: int(re.search(r"\." + f + r":\s+(\d+)", notes).group(1))
+        assert field("kernarg_segment_size") in (104, 104 + 256)
+        assert field("private_segment_fixed_size") == 0
+        assert field("sgpr_spill_count") == 0 and field("vgpr_spill_count") == 0
+        assert field("max_flat_workgroup_size") >= 512
+        assert field("group_segment_fixed_size") <= 160 * 1024
+        assert field("wavefront_size") == 64
+
+
 # ---- GPU: launch it the way plowrt does --------------------------------------------------------------
 
 class GluArgs(C.Structure):       # plow crates/plowrt/src/exec/amd.rs:1784-1807, 96 bytes
@@ -142,6 +168,13 @@ class DecPairArgs(C.Structure):   # amd.rs:3420-3430, 192 bytes
     _fields_ = [("glu", GluArgs), ("down", DownArgs), ("ctr", C.c_uint64), ("grid_glu", C.c_uint32), ("reserved", C.c_uint32)]
 
 
+class RouterDecodeArgs(C.Structure):   # amd.rs:955-982, 104 bytes
+    _fields_ = [(n, C.c_uint64) for n in ("logit", "x", "w", "table", "bias", "ctr", "signal")] + \
+               [(n, C.c_uint32) for n in ("rows", "n_exp", "k_dim", "topk", "flags", "shared_tail", "n_group", "topk_group")] + \
+               [("route_scale", C.c_float), ("per_row", C.c_uint32), ("signal_add", C.c_uint32), ("pad", C.c_uint32)]
+
+
+assert C.sizeof(RouterDecodeArgs) == 104
 assert C.sizeof(GluArgs) == 96 and C.sizeof(DownArgs) == 80 and C.sizeof(CombineArgs) == 48
 assert C.sizeof(DecPairArgs) == 192
 
@@ -366,3 +399,49 @@ def test_decode_object_launched_like_plowrt(oracle, T, shrink):
     check("pair after a launch whose waits gave up")
     assert int(ctr.abs().sum().item()) == 0
     moe.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,E,H,k,tail,groups", [(1, 256, 1024, 8, 1, (8, 4)), (3, 384, 768, 8, 1, (1, 1)), (7, 128, 512, 6, 0, (1, 1)),
+                                                    (1, 72, 520, 4, 0, (1, 1)), (20, 512, 256, 8, 1, (4, 2))])
+def test_router_object_launched_like_plowrt(rows, E, H, k, tail, groups):
+    """rows * ceil(n_exp / 8) workgroups of 512 threads, no dynamic LDS (amd.rs:1009, :17811-17832): logits and
+    table are the bytes of the library's op 180 followed by op 83, the arrival counters are back at zero, a
+    second launch gives the same, and a launch that signals adds its increment to the counter it names.
+    H = 520 is a row length the few-token score kernel does not serve (the object's plain loop runs)."""
+    import torch
+    from plow_amd import abi
+    from plow_amd.lib import Moe
+    print(f"[case] plowrt router object rows={rows} E={E} H={H} k={k} tail={tail} groups={groups}", flush=True)
+    g = torch.Generator(device="cpu").manual_seed(rows * 1000 + E)
+    x = torch.randn((rows, H), generator=g).bfloat16().cuda()
+    w = (torch.randn((E, H), generator=g) * 0.05).bfloat16().cuda()
+    bias = (torch.randn(E, generator=g) * 0.01).float().cuda()
+    flags = abi.ROUTE_SIGMOID | abi.ROUTE_NORM_TOPK | abi.ROUTE_BIAS | abi.ROUTE_F32_LOGIT
+    ng, tg = groups
+    # the library's two ops
+    moe = Moe(0)
+    logit_ref = torch.zeros((rows, E), dtype=torch.float32, device="cuda")
+    table_ref = torch.zeros((rows * (k + tail), 2), dtype=torch.int32, device="cuda")
+    tab = (C.c_void_p * 5)(logit_ref.data_ptr(), x.data_ptr(), w.data_ptr(), table_ref.data_ptr(), bias.data_ptr())
+    moe.exec_many([abi.inst(abi.OP_GEMM_F32, t=[0, 1, 2], i=[rows, E, H]),
+                   abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[3, 0, None, 4], i=[0, E, k, flags, rows, tail, ng, tg], f=[2.5, 0.0])], tab)
+    torch.cuda.synchronize()
+    moe.close()
+    m = Module(ELF_ROUTER, (ROUTER_MARKER,))
+    per_row = (E + 7) // 8
+    ctr = torch.zeros(rows * 32, dtype=torch.int32, device="cuda")
+    signal = torch.zeros(64, dtype=torch.int32, device="cuda")
+    for rep, add in enumerate((0, 0, 5)):
+        if add and rows != 1:
+            break                                   # plowrt signals from one-row routers only
+        logit = torch.full((rows, E), float("nan"), dtype=torch.float32, device="cuda")
+        table = torch.full((rows * (k + tail), 2), -1, dtype=torch.int32, device="cuda")
+        a = RouterDecodeArgs(logit.data_ptr(), x.data_ptr(), w.data_ptr(), table.data_ptr(), bias.data_ptr(), ctr.data_ptr(),
+                             signal.data_ptr() + 16 * 4, rows, E, H, k, flags, tail, ng, tg, 2.5, per_row, add, 0)
+        m.launch(ROUTER_KERNEL, a, rows * per_row, threads=512)
+        torch.cuda.synchronize()
+        assert torch.equal(logit.view(torch.int32), logit_ref.view(torch.int32)), rep
+        assert torch.equal(table, table_ref), rep
+        assert not ctr.any()
+        assert int(signal[16]) == add and int(signal.sum()) == add
