@@ -424,7 +424,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 3);
             g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
             g.row_partidx = (const uint32_t*)ten(in, T, 6);
-            g.N = I; g.K = H; g.E = E; g.act = i[5];
+            g.N = I; g.K = H; g.E = E; g.act = i[5]; g.T = i[4];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
             return launch_group_a4w4_tiled(g, true, st);
         }

@@ -440,10 +440,15 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     SdLds& L = *(SdLds*)sd_raw;
     const uint32_t tiles = g.N / SK_BN;
     const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
+    /* A workgroup fills its CU alone, so every trip to memory before its first block is time the CU streams
+     * nothing. Everything that depends on the expert alone is asked for at once, before the first of it is
+     * used (count, row offset, weight and scale pointers: one trip) ... */
     const uint32_t cnt = (uint32_t)g.meta[g.E + e];
-    if (cnt == 0u) return;
-    const uint64_t wp0 = g.wtab[(size_t)e * 3u], wp1 = g.wtab[(size_t)e * 3u + 1u];
     const uint32_t r0 = (uint32_t)g.meta[e];
+    const uint64_t wp0 = g.wtab[(size_t)e * 3u], wp1 = g.wtab[(size_t)e * 3u + 1u];
+    const uint64_t sp0 = g.stab[(size_t)e * 3u], sp1 = g.stab[(size_t)e * 3u + 1u];
+    asm volatile("" ::"s"(r0), "s"(wp0), "s"(wp1), "s"(sp0), "s"(sp1)); /* the loads stay above the branch */
+    if (cnt == 0u) return;
     const uint32_t padded = ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
     if (wp0 == 0ull || (g.out_bf16 && wp1 == 0ull)) { /* not resident; the bf16 form zeroes what it cannot compute */
         if (g.out_bf16)
@@ -457,8 +462,11 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     const uint32_t lr = lane >> 3, p = lane & 7u; /* load layout: row lr of a group of 8, piece p */
     const uint32_t K = g.K, KB = K / 128u, N = g.N;
     const uint32_t chw = ct * SK_BN + wv * 16u;   /* this wave's first channel */
-    const float* s0 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u] + (size_t)ct * KB;
-    const float* s1 = (const float*)(uintptr_t)g.stab[(size_t)e * 3u + 1u] + (size_t)ct * KB;
+    const float* s0 = (const float*)(uintptr_t)sp0 + (size_t)ct * KB;
+    const float* s1 = (const float*)(uintptr_t)sp1 + (size_t)ct * KB;
+    /* ... and what depends on those — the tile's weight block scales and the tokens of the first pass's 16
+     * rows (lane l: row l & 15) — in a second trip, together */
+    const uint32_t tok_first = (lane & 15u) < cnt ? g.row_token[r0 + (lane & 15u)] : PLOW_EXPERT_UNUSED;
 
     /* weight rows: load j covers LDS rows 8j .. 8j + 7 (j < 2 gate, else up) */
     const uint8_t* wsrc[4];
@@ -481,31 +489,29 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     const uint32_t o_lo = c * 128u + (((2u * q) ^ swz) << 4), o_hi = c * 128u + (((2u * q + 1u) ^ swz) << 4);
 
     for (uint32_t rb = 0; rb < cnt; rb += 16u) {
+        /* the token of row `idx` of the pass (PLOW_EXPERT_UNUSED past the expert's rows): the first pass has
+         * them in registers already, a later pass (an expert with more than 16 rows) reads them now */
+        auto tok_at = [&](uint32_t idx) -> uint32_t {
+            if (rb == 0u) return (uint32_t)__shfl((int)tok_first, (int)idx, 64);
+            return rb + idx < cnt ? g.row_token[r0 + rb + idx] : PLOW_EXPERT_UNUSED;
+        };
         /* activation rows of the pass: load i covers rows 8i .. 8i + 7 */
-        uint32_t tok0 = g.row_token[r0 + rb];
+        uint32_t tok0 = tok_at(0u);
         if (g.T != 0u && tok0 >= g.T) tok0 = 0u; /* any readable row: its scale is zeroed below */
         const uint8_t* xsrc[2];
 #pragma unroll
         for (uint32_t i = 0; i < 2u; i++) {
-            const uint32_t row = 8u * i + lr, off = rb + row;
-            uint32_t tok = off < cnt ? g.row_token[r0 + off] : PLOW_EXPERT_UNUSED;
+            const uint32_t row = 8u * i + lr;
+            uint32_t tok = tok_at(row);
             if (tok == PLOW_EXPERT_UNUSED || (g.T != 0u && tok >= g.T)) tok = tok0;
             xsrc[i] = (const uint8_t*)g.a + (size_t)tok * K + ((p ^ ((row >> 1) & 7u)) << 4);
         }
         const float* ssrc;
         uint32_t sstep;
-        {
-            const uint32_t off = rb + c;
-            const uint32_t tok = off < cnt ? g.row_token[r0 + off] : PLOW_EXPERT_UNUSED;
-            const bool ok = tok != PLOW_EXPERT_UNUSED && (g.T == 0u || tok < g.T);
-            ssrc = ok ? g.a_scale + tok : (const float*)(g.meta + 2u * g.E); /* tilep[0] = 0 */
-            sstep = ok ? g.pitch : 0u;
-        }
-        bool valid = rb + c < cnt;
-        if (valid) {
-            const uint32_t tok = g.row_token[r0 + rb + c];
-            valid = tok != PLOW_EXPERT_UNUSED && (g.T == 0u || tok < g.T);
-        }
+        const uint32_t tok_c = tok_at(c);
+        const bool valid = tok_c != PLOW_EXPERT_UNUSED && (g.T == 0u || tok_c < g.T);
+        ssrc = valid ? g.a_scale + tok_c : (const float*)(g.meta + 2u * g.E); /* tilep[0] = 0 */
+        sstep = valid ? g.pitch : 0u;
         auto issue = [&](uint32_t kb) {
             SdSlot* s = ring + kb % SD_STAGES;
             __builtin_amdgcn_global_load_lds((const void*)(ssrc + (size_t)kb * sstep), (sd_lds_void*)&s->xs[0], 4, 0, 0);

@@ -562,7 +562,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 const uint32_t ar = r0 + (row < rows ? row : 0u);
                 if (GLU) {
                     const uint32_t tk = g.row_token[ar];
-                    P.tsrow = tk == PLOW_EXPERT_UNUSED ? 0u : tk;
+                    P.tsrow = (tk == PLOW_EXPERT_UNUSED || (g.T != 0u && tk >= g.T)) ? 0u : tk;
                 } else {
                     P.tsrow = ar;
                 }
@@ -586,7 +586,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
 #pragma unroll
             for (uint32_t i = 0; i < 5u; i++) {
                 const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * (cw & 1u) + lr;
-                const uint32_t src = (GLU && P.tok[i] == PLOW_EXPERT_UNUSED) ? 0u : P.tok[i];
+                /* a pad row, or (fp4 arm: the staged rows end at g.T) a token past the rows that exist, reads row 0 */
+                const uint32_t src = (GLU && (P.tok[i] == PLOW_EXPERT_UNUSED || (A4 && g.T != 0u && P.tok[i] >= g.T))) ? 0u : P.tok[i];
                 S.aoff[i] = src * KA + ((p ^ ((row >> 1) & 7u)) << 4);
             }
 #pragma unroll

@@ -156,3 +156,34 @@ def test_a4w4_refusals(moe):
     err = C.create_string_buffer(256)
     rc = moe.lib.plow_moe_exec_noalloc(C.byref(glu), dev.table(), None, err, 256)
     assert rc == abi.E_UNSUPPORTED and b"context" in err.value, (rc, err.value)
+
+
+def test_a4w4_skips_a_non_resident_expert_and_survives_a_token_past_the_batch(moe, oracle):
+    """A null weight-table row (expert not resident on this rank): both ops leave its rows alone. A row whose
+    token lies past the rows the op was told of (i4) is read from row 0 of the staged batch instead of from
+    memory that was never staged: the layer's other rows are unaffected."""
+    cfg = layer.MoeConfig("a4w4-null", H=512, E=4, I=512, k=2, T=150, scoring="softmax", norm_topk=True,
+                          enc="mxfp4", arm="a4w4", n_shared=1, shared_mode="fold")
+    plan = layer.plan_layer(cfg)
+    dev = synth.bind(plan, "cuda", seed=11)
+    dev.t["wtab"][1].zero_()                       # expert 1 is elsewhere
+    dev.t["part"].fill_(0.25)                      # untouched rows must keep this
+    dev.t["fu4"].fill_(0x77)
+    host = synth.to_host(dev)
+    host.t["wtab"][1].zero_()                      # (the host table holds host pointers of its own)
+    run_device(moe, plan, dev)
+    run_oracle(oracle, plan, host)
+    rows = assert_routing_equal(plan, dev, host)
+    pd, ph = dev.np("part"), host.np("part")
+    untouched = (ph == 0.25).all(axis=1)
+    assert untouched.any() and np.array_equal(pd[untouched], ph[untouched])
+    assert_output_close(dev.np("out"), host.np("out"))
+    # the GLU told of fewer rows than the row map names
+    glu = clone(plan.insts[plan.index("glu")])
+    glu.i[4] = 100
+    want = dev.np("fu4").copy()
+    moe.exec(glu, dev.table())
+    torch.cuda.synchronize()
+    tok = dev.np("row_token")[:rows]
+    fine = (tok < 100) & (dev.np("row_partidx")[:rows] != abi.EXPERT_UNUSED)
+    assert fine.any() and np.array_equal(dev.np("fu4")[:rows][fine], want[:rows][fine])
