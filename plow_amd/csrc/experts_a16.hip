@@ -283,7 +283,10 @@ __global__ __launch_bounds__(AK_THREADS, GLU ? 2 : 4) void k_group_a16_stream(Gr
  *             activation rows of 128 B; piece p of a longer activation row r holds global piece
  *             (p & ~15) | ((p ^ r) & 15).
  * Same arithmetic and the same order of additions as the first form. */
-#define DM_STAGES 3u
+/* ring depth: four steps (loads three ahead) where the rings leave room in the CU's 160 KB — one row group per
+ * pass and 4 KB of weight rows per wave and step — three steps otherwise (mxfp4's step carries 8 KB of
+ * activation rows and the E8M0 bytes; several row groups per pass multiply the activation ring) */
+template <int ENC, int RG> struct DmDepth { static constexpr uint32_t v = (ENC != AENC_MXFP4 && RG == 1) ? 4u : 3u; };
 template <int ENC> struct DmGeom;
 template <> struct DmGeom<AENC_MXFP4> { static constexpr uint32_t KSTEP = 256u; };
 template <> struct DmGeom<AENC_FP8PC> { static constexpr uint32_t KSTEP = 128u; };
@@ -297,13 +300,13 @@ template <> struct DmWSlot<true> {
 template <> struct DmWSlot<false> {
     uint8_t w[2][16u * 128u];
 };
-/* RG = 16-row groups of activation rows per pass over the weights (1 for decode; 4, mxfp4 2, when
- * experts have many rows: the weights are then streamed a quarter as often and every weight operand
- * read from LDS feeds four matrix instructions) */
+/* RG = 16-row groups of activation rows per pass over the weights: 1, 2 or 4 (mxfp4: 1 or 2), picked per
+ * workgroup from its expert's row count: with more groups the weights are streamed less often and every
+ * weight operand read from LDS feeds that many matrix instructions */
 template <int ENC, int RG>
 struct DmLds {
-    uint8_t x[DM_STAGES][RG * 16u * DmGeom<ENC>::KSTEP * 2u];
-    DmWSlot<ENC == AENC_MXFP4> ring[AK_WAVES][DM_STAGES];
+    uint8_t x[DmDepth<ENC, RG>::v][RG * 16u * DmGeom<ENC>::KSTEP * 2u];
+    DmWSlot<ENC == AENC_MXFP4> ring[AK_WAVES][DmDepth<ENC, RG>::v];
     float bsc[4][2][128]; /* block-fp8: the weight block scales of the workgroup's tiles, all of K (K <= 16384) */
 };
 typedef __attribute__((address_space(3))) void dm_lds_void;
@@ -329,11 +332,39 @@ __device__ __forceinline__ float dm_read4(uint32_t addr) {
  * workgroup barrier */
 #define DM_WAIT_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory")
 
-/* The body works on workgroup index `bid` of a logical grid of E * N / 128 and takes its LDS as a pointer,
- * so that a kernel with a fixed launch shape (any 1-D grid, static LDS) can walk that grid itself. */
+/* What workgroup index `bid` of a logical grid of E * N / 128 works on: expert e (cnt rows), TPW channel tiles
+ * from tile ct. False when it has nothing to do. */
+struct DmWork {
+    uint32_t e, ct, TPW, cnt;
+};
+template <int ENC>
+__device__ __forceinline__ bool a16_dma_work(const GroupA16& g, uint32_t bid, DmWork& w) {
+    const uint32_t tiles = g.N / AK_BN;
+    /* With plenty of tiles to go round and a short K loop, a workgroup takes TPW consecutive channel tiles
+     * of its expert and keeps the load rings running across them, which hides the ramp of the loop. meta[3E], the
+     * number of 64-row tiles, is at least the number of experts with rows. The grid has one workgroup per
+     * tile; the first E * tiles / TPW of them do the work (consecutive indices, so that they spread over
+     * all XCDs) and the rest leave at once. */
+    const uint32_t busy = (g.meta ? (uint32_t)g.meta[3u * g.E] : 1u) * tiles;
+    const bool short_k = g.K / DmGeom<ENC>::KSTEP <= 16u; /* a long K loop amortises its ramp by itself */
+    w.TPW = !short_k ? 1u
+            : (ENC == AENC_MXFP4 && busy >= 8192u && tiles % 8u == 0u) ? 8u /* no per-tile tables to hold */
+            : (busy >= 4096u && tiles % 4u == 0u) ? 4u : ((busy >= 2048u && tiles % 2u == 0u) ? 2u : 1u);
+    const uint32_t wpe = tiles / w.TPW; /* workgroups per expert */
+    if (bid >= g.E * wpe) return false;
+    w.e = g.E - 1u - bid / wpe, w.ct = (bid % wpe) * w.TPW; /* heavy (folded shared) expert first */
+    w.cnt = g.meta ? (uint32_t)g.meta[g.E + w.e] : g.dense_rows;
+    return w.cnt != 0u;
+}
+
+/* The body takes its LDS as a pointer, so that a kernel with a fixed launch shape (any 1-D grid, static LDS) can
+ * walk the logical grid itself. */
 template <int ENC, bool GLU, int RG>
-__device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw, uint32_t bid) {
+__device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw, const DmWork& work) {
     DmLds<ENC, RG>& L = *(DmLds<ENC, RG>*)dm_raw;
+    /* ring slots in use; steps of loads in flight. The GLU's two weight streams already keep twice the bytes in
+     * flight per step and measured no faster at the fourth slot (the DOWN gained 3 %), so it stays at three */
+    constexpr uint32_t DM_STAGES = GLU ? 3u : DmDepth<ENC, RG>::v, AH = DM_STAGES - 1u;
     typedef DmWSlot<ENC == AENC_MXFP4> Slot;
     constexpr uint32_t KSTEP = DmGeom<ENC>::KSTEP, XROW = KSTEP * 2u; /* activation bytes per row and step */
     constexpr uint32_t NP = XROW / 16u;                              /* 16-byte pieces per activation row */
@@ -344,22 +375,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
     constexpr int NS = GLU ? 2 : 1;
     /* direct loads per wave and step: weights 2 per stream, mxfp4 scales 1 per stream, rows NXI (waves below XL) */
     constexpr int NLW = NS * (ENC == AENC_MXFP4 ? 3 : 2);
-    const uint32_t tiles = g.N / AK_BN;
-    /* With plenty of tiles to go round and a short K loop, a workgroup takes TPW consecutive channel tiles
-     * of its expert and keeps the load rings running across them, which hides the ramp of the loop. meta[3E], the
-     * number of 64-row tiles, is at least the number of experts with rows. The grid has one workgroup per
-     * tile; the first E * tiles / TPW of them do the work (consecutive indices, so that they spread over
-     * all XCDs) and the rest leave at once. */
-    const uint32_t busy = (g.meta ? (uint32_t)g.meta[3u * g.E] : 1u) * tiles;
-    const bool short_k = g.K / DmGeom<ENC>::KSTEP <= 16u; /* a long K loop amortises its ramp by itself */
-    const uint32_t TPW = !short_k ? 1u
-                         : (ENC == AENC_MXFP4 && busy >= 8192u && tiles % 8u == 0u) ? 8u /* no per-tile tables to hold */
-                         : (busy >= 4096u && tiles % 4u == 0u) ? 4u : ((busy >= 2048u && tiles % 2u == 0u) ? 2u : 1u);
-    const uint32_t wpe = tiles / TPW; /* workgroups per expert */
-    if (bid >= g.E * wpe) return;
-    const uint32_t e = g.E - 1u - bid / wpe, ct = (bid % wpe) * TPW; /* heavy (folded shared) expert first */
-    const uint32_t cnt = g.meta ? (uint32_t)g.meta[g.E + e] : g.dense_rows;
-    if (cnt == 0u) return;
+    const uint32_t e = work.e, ct = work.ct, TPW = work.TPW, cnt = work.cnt;
     const uint64_t* wt = g.wtab ? g.wtab + (size_t)e * g.wcols : nullptr;
     const uint64_t* stt = g.stab ? g.stab + (size_t)e * g.wcols : nullptr;
     if (wt && wt[g.wsel0] == 0ull) return; /* expert not resident: skipped */
@@ -494,14 +510,18 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
         DM_WAIT_BARRIER(0);
         issue();
         if (GS > 1u) issue();
+        if (AH > 2u && GS > 2u) issue();
         uint32_t st = 0;
         for (uint32_t G = 0, t = 0, S = 0; G < GS; G++) {
-            /* loads return in order: step G has landed once at most step G + 1's are outstanding; after the
-             * barrier every wave's share of the rows is there and nobody reads step G - 1 any more */
-            if (G + 1u >= GS) DM_WAIT_BARRIER(0);
-            else if (XL >= AK_WAVES || wv < XL) DM_WAIT_BARRIER(NLW + (int)NXI);
-            else DM_WAIT_BARRIER(NLW);
-            if (G + 2u < GS) issue();
+            /* loads return in order: step G has landed once at most the steps after it that were issued (AH - 1
+             * of them, fewer at the end) are outstanding; after the barrier every wave's share of the rows is
+             * there and nobody reads step G - 1 any more */
+            const uint32_t after = GS - 1u - G < AH - 1u ? GS - 1u - G : AH - 1u; /* steps in flight behind step G */
+            const bool loads_x = XL >= AK_WAVES || wv < XL;
+            if (after == 0u) DM_WAIT_BARRIER(0);
+            else if (after == 1u) { if (loads_x) DM_WAIT_BARRIER(NLW + (int)NXI); else DM_WAIT_BARRIER(NLW); }
+            else { if (loads_x) DM_WAIT_BARRIER(2 * (NLW + (int)NXI)); else DM_WAIT_BARRIER(2 * NLW); }
+            if (G + AH < GS) issue();
             const uint32_t wb = w_base + st * (uint32_t)sizeof(Slot), xb0 = x_base + st * (RG * 16u * XROW) + c * XROW;
             /* the weight operands of the step are read once and multiply every row group of the pass */
             if constexpr (ENC == AENC_MXFP4) {
@@ -664,25 +684,31 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
     }
 }
 
-template <int ENC, bool GLU, int RG>
+/* One kernel, three instances of the body: a workgroup takes the one that covers its expert's rows in the fewest
+ * passes over the weights (16, 32 or 64 rows per pass; mxfp4 16 or 32, its rings fill the LDS at 32). Routing is
+ * skewed: at 4 rows per expert on average the hot experts hold 30 to 60, and a second pass re-reads the weights
+ * from memory (Qwen3 shape, 64 tokens: GLU 325 us with 16-row passes for all, 289 us with 32-row passes for
+ * all, which in turn costs the few-row experts 3 % in row loads and multiplies they do not need). */
+template <int ENC, bool GLU>
 __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
-    a16_dma_body<ENC, GLU, RG>(g, dm_raw, blockIdx.x);
+    DmWork w;
+    if (!a16_dma_work<ENC>(g, blockIdx.x, w)) return;
+    if (w.cnt <= 16u) a16_dma_body<ENC, GLU, 1>(g, dm_raw, w);
+    else if (ENC == AENC_MXFP4 || w.cnt <= 32u) a16_dma_body<ENC, GLU, 2>(g, dm_raw, w);
+    else a16_dma_body<ENC, GLU, ENC == AENC_MXFP4 ? 2 : 4>(g, dm_raw, w);
 }
 
-template <int ENC, bool GLU, int RG>
-static int launch_a16_dma_rg(const GroupA16& g, dim3 grid, hipStream_t st) {
-    static_assert(sizeof(DmLds<ENC, RG>) <= 160u * 1024u, "the rings must fit the CU's LDS");
-    k_group_a16_dma<ENC, GLU, RG><<<grid, AK_THREADS, sizeof(DmLds<ENC, RG>), st>>>(g);
-    return 0;
-}
-/* Experts with many rows (two dozen or more on average, from the slot count the host knows) take four
- * 16-row groups per pass over their weights; mxfp4 two (its rings then fill the CU's LDS exactly). */
+template <int ENC> struct DmLdsMax {
+    static constexpr size_t a = sizeof(DmLds<ENC, 1>), b = sizeof(DmLds<ENC, 2>),
+                            c = sizeof(DmLds<ENC, ENC == AENC_MXFP4 ? 2 : 4>);
+    static constexpr size_t v = a > b ? (a > c ? a : c) : (b > c ? b : c);
+};
 template <int ENC, bool GLU>
 static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
-    const bool many = g.meta ? g.slots_hint >= 24u * g.E : g.dense_rows >= 24u; /* a dense op is one expert of dense_rows rows */
-    if (many) return launch_a16_dma_rg<ENC, GLU, ENC == AENC_MXFP4 ? 2 : 4>(g, grid, st);
-    return launch_a16_dma_rg<ENC, GLU, 1>(g, grid, st);
+    static_assert(DmLdsMax<ENC>::v <= 160u * 1024u, "the rings must fit the CU's LDS");
+    k_group_a16_dma<ENC, GLU><<<grid, AK_THREADS, DmLdsMax<ENC>::v, st>>>(g);
+    return 0;
 }
 
 /* Many rows per expert (16 and more on average): the fp8-weight arms run on the tiled kernel (loader and
@@ -769,16 +795,14 @@ static int launch_a16(const GroupA16& g, hipStream_t st) {
 }
 
 /* dynamic-LDS limits of every instance of the direct-to-LDS form, once per device (plow_moe_device_setup) */
-template <int ENC, bool GLU, int RG>
+template <int ENC, bool GLU>
 static bool a16_set_attr() {
-    return hipFuncSetAttribute((const void*)k_group_a16_dma<ENC, GLU, RG>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)sizeof(DmLds<ENC, RG>)) == hipSuccess;
+    return hipFuncSetAttribute((const void*)k_group_a16_dma<ENC, GLU>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)DmLdsMax<ENC>::v) == hipSuccess;
 }
 template <int ENC>
 static bool a16_set_attrs() {
-    constexpr int RGM = ENC == AENC_MXFP4 ? 2 : 4;
-    return a16_set_attr<ENC, true, 1>() && a16_set_attr<ENC, false, 1>() && a16_set_attr<ENC, true, RGM>() &&
-           a16_set_attr<ENC, false, RGM>();
+    return a16_set_attr<ENC, true>() && a16_set_attr<ENC, false>();
 }
 int plow_moe_a16_setup() {
     return a16_set_attrs<AENC_BF16>() && a16_set_attrs<AENC_FP8BLK>() && a16_set_attrs<AENC_MXFP4>() &&

@@ -89,7 +89,8 @@ extern "C" __global__ __launch_bounds__(512) void plow_moe_fp8_glu_pf_gfx950(PLO
     g.wcols = 3; g.wsel0 = 0; g.wsel1 = 1;
     const uint32_t nwg = experts * (inter / 128u);
     for (uint32_t b = blockIdx.x; b < nwg; b += gridDim.x) {
-        a16_dma_body<AENC_FP8BLK, true, 4>(g, lds, b);
+        DmWork w;
+        if (a16_dma_work<AENC_FP8BLK>(g, b, w)) a16_dma_body<AENC_FP8BLK, true, 4>(g, lds, w);
         __syncthreads();
     }
 }
@@ -105,7 +106,8 @@ extern "C" __global__ __launch_bounds__(512) void plow_moe_fp8_down_pf_gfx950(PL
     g.wcols = 3; g.wsel0 = 2; g.wsel1 = 2;
     const uint32_t nwg = experts * (hidden / 128u);
     for (uint32_t b = blockIdx.x; b < nwg; b += gridDim.x) {
-        a16_dma_body<AENC_FP8BLK, false, 4>(g, lds, b);
+        DmWork w;
+        if (a16_dma_work<AENC_FP8BLK>(g, b, w)) a16_dma_body<AENC_FP8BLK, false, 4>(g, lds, w);
         __syncthreads();
     }
 }
