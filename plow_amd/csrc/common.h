@@ -29,6 +29,24 @@ __device__ __forceinline__ bf16_t f2bf(float f) {
     return (bf16_t)(u >> 16);
 }
 
+/* Swizzles of LDS operand rows. Direct loads write 64 lanes' 16-byte pieces to consecutive LDS addresses, so rows
+ * sit unpadded, and bank conflicts are avoided by permuting the pieces of a row on the GLOBAL side of the load;
+ * the reader applies the same permutation. What must not collide is what one clock serves, measured on this
+ * part (two lanes of one set on the same banks cost a clock each):
+ *   ds_read_b128  16 lanes per clock, not consecutive ones: {0-3, 12-15, 20-23, 24-27}, then
+ *                 {4-7, 8-11, 16-19, 28-31}, then the same of lanes 32-63;
+ *   ds_read_b64   32 consecutive lanes per clock.
+ * In the matrix operand layout (row = lane & 15, k-chunk = lane >> 4) a b128 set therefore holds rows
+ * {0-3, 12-15} of one k-chunk and rows {4-11} of the next: the swizzles send those two classes of rows to
+ * disjoint halves of the piece range, and an XOR with the k-chunk's piece offset keeps them disjoint.
+ * lds_swz8: XOR for the 16-byte piece index (0..7) of row r, rows of 128 bytes (rows r and r ^ 1 differ in
+ * bank bit 5 already). lds_swz16: the same for rows of 256 bytes or a multiple (piece index & 15). */
+__device__ __forceinline__ uint32_t lds_swz8(uint32_t r) {
+    const uint32_t t = (r >> 1) & 7u;
+    return t ^ ((t & 2u) << 1);
+}
+__device__ __forceinline__ uint32_t lds_swz16(uint32_t r) { return (r ^ ((r & 4u) << 1)) & 15u; }
+
 /* Monotone f32 -> u32 (plow runtime/common/moe_route_key.h:35-39). */
 __device__ __forceinline__ uint32_t route_ord(float x) {
     const uint32_t b = __float_as_uint(x);

@@ -279,9 +279,9 @@ __global__ __launch_bounds__(AK_THREADS, GLU ? 2 : 4) void k_group_a16_stream(Gr
  *   sync      rings of three steps, loads two steps ahead; per step each wave waits for its own loads
  *             (s_waitcnt vmcnt) and all meet at one barrier, after which the step before is free;
  *   swizzle   direct loads write LDS contiguously, so bank conflicts are avoided on the global side:
- *             LDS piece p of weight row r holds global piece p ^ ((r >> 1) & 7), and likewise for
+ *             LDS piece p of weight row r holds global piece p ^ lds_swz8(r), and likewise for
  *             activation rows of 128 B; piece p of a longer activation row r holds global piece
- *             (p & ~15) | ((p ^ r) & 15).
+ *             (p & ~15) | ((p ^ lds_swz16(r)) & 15).
  * Same arithmetic and the same order of additions as the first form. */
 /* ring depth: four steps (loads three ahead) where the rings leave room in the CU's 160 KB — one row group per
  * pass and 4 KB of weight rows per wave and step — three steps otherwise (mxfp4's step carries 8 KB of
@@ -403,7 +403,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
 #pragma unroll
         for (uint32_t j = 0; j < 2u; j++) {
             const uint32_t R = 8u * j + lr;
-            wsrc[sidx][j] = wbase + (size_t)((chw + R) * wmul + wr0) * wrow + ((p ^ ((R >> 1) & 7u)) << 4);
+            wsrc[sidx][j] = wbase + (size_t)((chw + R) * wmul + wr0) * wrow + ((p ^ lds_swz8(R)) << 4);
         }
         /* mxfp4 scales: lane -> (row (lane & 31) >> 1, dword lane & 1) of the step's 8 bytes per row */
         if (ENC == AENC_MXFP4)
@@ -416,12 +416,12 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
             }
         }
     }
-    const uint32_t swz = (c >> 1) & 7u;
+    const uint32_t swz = lds_swz8(c), swx = lds_swz16(c);
     const uint32_t x_base = dm_lds_off(&L.x[0][0]);
     const uint32_t w_base = dm_lds_off(&L.ring[wv][0]);
     const uint32_t b_base = dm_lds_off(&L.bsc[0][0][0]);
     /* LDS position of logical piece P of activation row c */
-    auto xpos = [&](uint32_t P) -> uint32_t { return NP >= 16u ? ((P & ~15u) | ((P ^ c) & 15u)) : (P ^ swz); };
+    auto xpos = [&](uint32_t P) -> uint32_t { return NP >= 16u ? ((P & ~15u) | ((P ^ swx) & 15u)) : (P ^ swz); };
 
     for (uint32_t rb = 0; rb < cnt; rb += 16u * RG) {
         /* this wave's share of the pass's rows: load i covers rows XRPL * (wv + 8 i) .., NP lanes each; a pad
@@ -438,7 +438,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                     const uint32_t off = rb + xrow;
                     uint32_t ai = off < cnt ? (g.a_idx ? g.a_idx[r0 + off] : r0 + off) : PLOW_EXPERT_UNUSED;
                     if (ai == PLOW_EXPERT_UNUSED) ai = first == PLOW_EXPERT_UNUSED ? 0u : first;
-                    const uint32_t gp = NP >= 16u ? ((pc & ~15u) | ((pc ^ xrow) & 15u)) : (pc ^ ((xrow >> 1) & 7u));
+                    const uint32_t gp = NP >= 16u ? ((pc & ~15u) | ((pc ^ lds_swz16(xrow)) & 15u)) : (pc ^ lds_swz8(xrow));
                     xsrc[i] = (const uint8_t*)g.a + (size_t)ai * K * 2u + (gp << 4);
                 }
             }

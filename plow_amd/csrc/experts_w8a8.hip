@@ -403,7 +403,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
  * the vector memory pipeline four times as much per instruction, which shows at the gate|up shape
  * (two matrices, rows 7 KB apart). No workgroup barrier in the K loop: a wave waits for its own loads
  * (s_waitcnt vmcnt) and nobody else's. Pad rows read the pass's first row and carry a zero scale.
- * LDS pieces are swizzled on the global side: piece p of row r holds global piece p ^ ((r >> 1) & 7). */
+ * LDS pieces are swizzled on the global side: piece p of row r holds global piece p ^ lds_swz8(r). */
 #ifndef SD_STAGES
 #define SD_STAGES 3
 #endif
@@ -474,7 +474,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     for (uint32_t j = 0; j < 4u; j++) {
         const uint32_t R = 8u * j + lr;
         const uint8_t* base = (const uint8_t*)(uintptr_t)(j < 2u ? wp0 : wp1);
-        wsrc[j] = base + (size_t)(chw + (R & 15u)) * K + ((p ^ ((R >> 1) & 7u)) << 4);
+        wsrc[j] = base + (size_t)(chw + (R & 15u)) * K + ((p ^ lds_swz8(R)) << 4);
     }
     /* the weight block scales go to LDS once: an ordinary load inside the K loop would make the
      * compiler wait for every outstanding load of the ring */
@@ -485,7 +485,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     __syncthreads();
     const uint32_t wsc_base = sd_lds_off(&L.wsc[0][0]);
     SdSlot* const ring = L.ring[wv];
-    const uint32_t swz = (c >> 1) & 7u;
+    const uint32_t swz = lds_swz8(c);
     const uint32_t o_lo = c * 128u + (((2u * q) ^ swz) << 4), o_hi = c * 128u + (((2u * q + 1u) ^ swz) << 4);
 
     for (uint32_t rb = 0; rb < cnt; rb += 16u) {
@@ -504,7 +504,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
             const uint32_t row = 8u * i + lr;
             uint32_t tok = tok_at(row);
             if (tok == PLOW_EXPERT_UNUSED || (g.T != 0u && tok >= g.T)) tok = tok0;
-            xsrc[i] = (const uint8_t*)g.a + (size_t)tok * K + ((p ^ ((row >> 1) & 7u)) << 4);
+            xsrc[i] = (const uint8_t*)g.a + (size_t)tok * K + ((p ^ lds_swz8(row)) << 4);
         }
         const float* ssrc;
         uint32_t sstep;

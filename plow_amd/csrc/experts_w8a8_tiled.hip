@@ -27,7 +27,7 @@
  *
  * A direct load writes the 64 lanes' 16-byte pieces to consecutive LDS addresses, so rows sit
  * unpadded (128 B); bank conflicts are avoided by swizzling on the GLOBAL side: LDS piece p of row r
- * holds global piece p ^ ((r >> 1) & 7), and the operand reads of 16 consecutive rows then cover all
+ * holds global piece p ^ lds_swz8(r), and the lanes an operand read serves in one clock then cover all
  * 64 banks. Rows of the tile beyond the expert's live rows read the tile's first row and carry a
  * zero activation scale; 16-row groups with no live row are skipped by the consumers.
  * Tiles are walked by persistent workgroups (one per CU) in an order that puts the tiles sharing
@@ -217,8 +217,8 @@ __device__ __forceinline__ v2i ds_read8(uint32_t addr) {
  *      registers (exact: e4m3 fits bf16), v_mfma_f32_16x16x32_bf16 twice per operand pair. No activation
  *      scales; block mode scales the block's product by the weight block scale (one per two blocks),
  *      per-channel mode accumulates straight through. Weight row r16 of an operand holds its 8-byte piece
- *      j at (j ^ 4 * ((r16 >> 2) & 1)): the 64 lanes of a read then touch every bank twice, the minimum
- *      for 512 bytes. ---- */
+ *      j at (j ^ 2 * ((r16 >> 2) & 3)): a ds_read_b64 serves 32 consecutive lanes per clock (16 rows x two
+ *      k-chunks), and rows 4 apart start on the same bank. ---- */
 #define T5A_BLOCK_HEAD()                                                                                     \
     const uint32_t ab = a_base + st * (uint32_t)sizeof(L.a[0]), wb = w_base + st * (256u * 128u) + cw * (32u * 64u);   \
     const uint32_t b0 = ab + opb0, b1 = ab + opb1;                                                           \
@@ -435,12 +435,12 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     }
     (void)s_base, (void)c_base, (void)ts_base, (void)wsb_base;
     /* consumer: this lane's operand pieces 2q, 2q + 1 of row (16 * group + r16) */
-    const uint32_t sw = (r16 >> 1) & 7u;
+    const uint32_t sw = lds_swz8(r16);
     const uint32_t op_lo = r16 * 128u + (((2u * q) ^ sw) << 4), op_hi = r16 * 128u + (((2u * q + 1u) ^ sw) << 4);
     /* A16: this lane's 16-byte token pieces q and 4 + q (k 8q.. and 32 + 8q.. of the 64-k block), and its
      * 8-byte weight pieces of row r16 */
     const uint32_t opb0 = r16 * 128u + ((q ^ sw) << 4), opb1 = r16 * 128u + (((4u + q) ^ sw) << 4);
-    const uint32_t swa = ((r16 >> 2) & 1u) * 4u;
+    const uint32_t swa = ((r16 >> 2) & 3u) * 2u;
     const uint32_t opa0 = r16 * 64u + ((q ^ swa) << 3), opa1 = r16 * 64u + (((4u + q) ^ swa) << 3);
     (void)op_lo, (void)op_hi, (void)opb0, (void)opb1, (void)opa0, (void)opa1;
 
@@ -588,7 +588,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * (cw & 1u) + lr;
                 /* a pad row, or (fp4 arm: the staged rows end at g.T) a token past the rows that exist, reads row 0 */
                 const uint32_t src = (GLU && (P.tok[i] == PLOW_EXPERT_UNUSED || (A4 && g.T != 0u && P.tok[i] >= g.T))) ? 0u : P.tok[i];
-                S.aoff[i] = src * KA + ((p ^ ((row >> 1) & 7u)) << 4);
+                S.aoff[i] = src * KA + ((p ^ lds_swz8(row)) << 4);
             }
 #pragma unroll
             for (uint32_t i = 0; i < 8u; i++) { /* LDS weight rows R = 64 * cw + 8 * i + lr: consumer R / 32, group (R / 16) & 1 */
@@ -602,7 +602,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     ch = nt * 256u + R;
                     if (ch >= g.N) ch = 0; /* past the last channel: any valid row, never stored */
                 }
-                S.woff[i] = A16 ? ch * K + (((lane & 3u) ^ (((R >> 2) & 1u) << 1)) << 4) : ch * KW + ((p ^ ((R >> 1) & 7u)) << 4);
+                S.woff[i] = A16 ? ch * K + (((lane & 3u) ^ ((R >> 2) & 3u)) << 4) : ch * KW + ((p ^ lds_swz8(R)) << 4);
             }
             /* activation scale of row 64 * cw + lane (loader 3 repeats loader 0's 64 values); a pad row
              * reads tilep[0], which is always 0 */
