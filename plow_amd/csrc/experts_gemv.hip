@@ -1,5 +1,5 @@
 /* experts_gemv.hip — the bf16-activation expert ops (85 / 86 arms 0 and 8, 48 / 49, 65 / 66, 75 / 76) when
- * the batch routes a handful of rows in all (decode at one or two tokens).
+ * the batch routes few rows in all (decode at a few tokens).
  *
  * With one row per expert the matrix unit has nothing to amortise: the op is a set of matrix-vector
  * products, bound by how many weight bytes the chip keeps in flight. The tile kernels give a workgroup
@@ -18,7 +18,7 @@
 
 enum { GV_BF16 = 0, GV_FP8BLK = 1, GV_MXFP4 = 2, GV_FP8PC = 3 };
 #define GV_WAVES 4u
-#define GV_WINDOW 64u /* live rows handled per pass (the form is chosen for far fewer) */
+#define GV_WINDOW 256u /* live rows handled per pass (the form is chosen for fewer) */
 #define GV_MAX_E 1088u
 #define GV_ECHUNKS (GV_MAX_E / WAVE)
 
@@ -132,6 +132,7 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
             uint32_t seen = 0; /* live rows of the experts before this chunk */
 #pragma unroll
             for (uint32_t j = 0; j < GV_ECHUNKS; j++) {
+                if (j * WAVE >= E) continue; /* the same in every lane: chunks past the last expert cost nothing */
                 const uint32_t e = j * WAVE + lane;
                 const uint32_t c = cnt_r[j];
                 uint32_t inc = c;
@@ -185,6 +186,18 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
                         x[it][j] = p < pieces ? *(const v4i*)(xsrc + ((size_t)p * XQ + j) * 16u) : (v4i){0, 0, 0, 0};
                 }
                 const float gate = (!GLU && g.gate) ? g.gate[row] : 1.0f;
+                /* per-channel scales: lane l applies the scale of channel c0 + l when the 64 results of a group are
+                 * stored; those of the wave's first group (usually its only one) are asked for here, with the
+                 * activations, and not one by one inside the loop */
+                auto pc_scale = [&](uint32_t c0, int s_) -> float {
+                    const uint32_t ch = c0 + lane < c_hi ? c0 + lane : c_hi - 1u;
+                    return ((const float*)sbase[s_])[(size_t)ch * wmul + wr[s_]];
+                };
+                float pcs0 = 1.0f, pcs1 = 1.0f;
+                if (ENC == GV_FP8PC) {
+                    pcs0 = pc_scale(c_lo, 0);
+                    if (GLU) pcs1 = pc_scale(c_lo, 1);
+                }
                 auto row_ptrs = [&](uint32_t ch, int s, const uint8_t*& wp, const uint8_t*& sp) {
                     const size_t wrow = (size_t)ch * wmul + wr[s];
                     wp = wbase[s] + wrow * wrow_bytes;
@@ -206,7 +219,8 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
                 };
 #pragma unroll
                 for (int u = 0; u < AHEAD; u++) fetch(ring[u], (uint32_t)u, u % NS);
-                float keep = 0.0f; /* lane l keeps the result of channel c_lo + 64 j + l until the 64 are stored */
+                /* lane l keeps the sums of channel c_lo + 64 j + l until the 64 are finished and stored at once */
+                float keep_a = 0.0f, keep_b = 0.0f;
                 float v0 = 0.0f;
                 for (uint32_t i0 = 0; i0 < units; i0 += (uint32_t)D) {
 #pragma unroll
@@ -219,20 +233,24 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
                             v0 = v;
                             continue;
                         }
-                        float va = GLU ? v0 : v, vb = v;
                         const uint32_t ch = c_lo + unit / (uint32_t)NS;
-                        if (ENC == GV_FP8PC) {
-                            va *= ((const float*)sbase[0])[(size_t)ch * wmul + wr[0]];
-                            if (GLU) vb *= ((const float*)sbase[1])[(size_t)ch * wmul + wr[1]];
-                        }
-                        const float res = GLU ? moe_glu(va, vb, g.act, g.f0, g.f1) : gate * va;
                         const uint32_t rel = ch - c_lo;
-                        if ((rel & 63u) == lane) keep = res;
-                        if ((rel & 63u) == 63u || ch + 1u == c_hi) { /* 64 results (or the tail): one store */
+                        if ((rel & 63u) == lane) keep_a = GLU ? v0 : v, keep_b = v;
+                        if ((rel & 63u) == 63u || ch + 1u == c_hi) { /* 64 sums (or the tail): finished and stored at once */
                             const uint32_t c0 = c_lo + (rel & ~63u);
+                            if (ENC == GV_FP8PC && c0 != c_lo) { /* a later group of a wave with many channels */
+                                pcs0 = pc_scale(c0, 0);
+                                if (GLU) pcs1 = pc_scale(c0, 1);
+                            }
+                            float va = keep_a, vb = keep_b;
+                            if (ENC == GV_FP8PC) {
+                                va *= pcs0;
+                                if (GLU) vb *= pcs1;
+                            }
+                            const float res = GLU ? moe_glu(va, vb, g.act, g.f0, g.f1) : gate * va;
                             if (c0 + lane <= ch) {
-                                if (GLU || g.out_bf16) ((bf16_t*)g.out)[(size_t)orow * N + c0 + lane] = f2bf(keep);
-                                else ((float*)g.out)[(size_t)orow * N + c0 + lane] = keep;
+                                if (GLU || g.out_bf16) ((bf16_t*)g.out)[(size_t)orow * N + c0 + lane] = f2bf(res);
+                                else ((float*)g.out)[(size_t)orow * N + c0 + lane] = res;
                             }
                         }
                     }
@@ -255,7 +273,8 @@ static int launch_gemv_iter(const GroupA16& g, uint32_t n_cu, hipStream_t st) {
         if (nb > 3) nb = 3;
         __atomic_store_n(&per_cu, nb, __ATOMIC_RELAXED);
     }
-    const uint32_t grid = n_cu * (uint32_t)nb < 16u ? 16u : n_cu * (uint32_t)nb; /* never fewer waves than a window has rows */
+    const uint32_t min_grid = GV_WINDOW / GV_WAVES; /* never fewer waves than a window has rows */
+    const uint32_t grid = n_cu * (uint32_t)nb < min_grid ? min_grid : n_cu * (uint32_t)nb;
     k_group_a16_gemv<ENC, GLU, ITER><<<grid, GV_WAVES * WAVE, 0, st>>>(g);
     return 0;
 }
@@ -269,15 +288,21 @@ static int launch_gemv_enc(const GroupA16& g, uint32_t row_bytes, uint32_t n_cu,
     return PLOW_MOE_EINVAL;
 }
 
-/* Rows a batch may route in all for this form to be chosen: two tokens' worth at nine slots each. */
-#define GV_MAX_SLOTS 18u
+/* Rows a batch may route in all for this form to be chosen, measured against the tile kernels per layer (a
+ * routed row streams its expert's weights by itself here, an expert's rows share them there):
+ *   mxfp4 (Kimi-K2 shape)             ahead up to about 28 tokens of 9 slots: 1 token 139 -> 106 us, 4 tokens 305 -> 220,
+ *                                     16 tokens 725 -> 637, 24 tokens 938 -> 858, 32 tokens 1006 -> 1037
+ *   block fp8 (DeepSeek-V3 shape)     ahead up to 4 tokens: 2 tokens 233 -> 202, 4 tokens 346 -> 328, 5 tokens 361 -> 384
+ *   per-channel fp8 (Qwen3 shape)     1 token 87 -> 80, 2 tokens 95 -> 90, mixed from 3 tokens on (skewed routing)
+ *   bf16 weights                      level at 1 token, behind at 2 (90 -> 98): twice the bytes per row */
+static uint32_t gv_max_slots(uint32_t enc) {
+    return enc == GV_MXFP4 ? 240u : enc == GV_FP8BLK ? 36u : enc == GV_FP8PC ? 18u : 9u;
+}
 
 bool group_a16_gemv_serves(const GroupA16& g) {
-    if (!plow_moe_tuning().a16_gemv || !g.meta || !g.wtab || g.bias || g.slots_hint == 0u || g.slots_hint > GV_MAX_SLOTS) return false;
-    /* measured against the tile kernels: at one token ahead on mxfp4 (Kimi-K2 shape 139 -> 110 us per layer) and
-     * level to a few percent ahead on the other encodings; at two tokens ahead on mxfp4 (221 -> 150 us) and level
-     * or behind on the others, whose tile kernels fill the chip better there */
-    if (g.slots_hint > GV_MAX_SLOTS / 2u && g.enc != GV_MXFP4) return false;
+    if (!plow_moe_tuning().a16_gemv || !g.meta || !g.wtab || g.bias || g.slots_hint == 0u || g.enc > GV_FP8PC ||
+        g.slots_hint > gv_max_slots(g.enc))
+        return false;
     if (g.enc != GV_BF16 && !g.stab) return false;
     const uint32_t row_bytes = g.enc == GV_BF16 ? g.K * 2u : (g.enc == GV_MXFP4 ? g.K / 2u : g.K);
     const uint32_t max_bytes = g.enc == GV_MXFP4 ? 4096u : 8192u;

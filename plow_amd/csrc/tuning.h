@@ -15,7 +15,7 @@
  *                                              the vector-unit kernels at prefill sizes
  *   PLOW_MOE_SCORE_MFMA32_FROM  n              number of outputs from which the 32 x 32 matrix-unit tiles are forced
  *   PLOW_MOE_A16_TILED        0                keep the bf16-activation arms on the streaming kernels at every row count
- *   PLOW_MOE_A16_GEMV         0                keep the bf16-activation arms off the matrix-vector form at one or two tokens
+ *   PLOW_MOE_A16_GEMV         0                keep the bf16-activation arms off the matrix-vector form at a few tokens
  */
 #ifndef PLOW_MOE_TUNING_H
 #define PLOW_MOE_TUNING_H

@@ -390,14 +390,31 @@ def test_matrix_vector_form_at_one_and_two_tokens(moe, oracle, enc, H, I, T, k):
     check_chain(*both(moe, oracle, cfg, seed=H + T))
 
 
-def test_matrix_vector_form_is_right_when_the_slot_count_is_understated(moe, oracle):
+@pytest.mark.parametrize("enc,H,I,T,k", [("mxfp4", 768, 256, 24, 8), ("mxfp4", 3584, 512, 26, 8), ("fp8blk", 640, 384, 4, 8),
+                                         ("fp8pc", 1536, 640, 2, 8)])
+def test_matrix_vector_form_at_a_few_tokens(moe, oracle, enc, H, I, T, k):
+    """The largest batches the matrix-vector form is chosen for, per encoding (mxfp4 up to 240 routed rows,
+    block fp8 36, per-channel fp8 18): 16 experts, so every expert holds several rows and streams its weights
+    once per row."""
+    print(f"[case] gemv few tokens enc={enc} H={H} I={I} T={T} k={k}", flush=True)
+    cfg = layer.MoeConfig("gemv-few", T=T, H=H, E=16, I=I, k=k, scoring="sigmoid", norm_topk=True, bias=True,
+                          route_scale=2.5, enc=enc, arm="a16", n_shared=1, shared_mode="fold")
+    check_chain(*both(moe, oracle, cfg, seed=H + T))
+
+
+@pytest.mark.parametrize("enc,H,I,T", [("mxfp4", 512, 256, 40), ("mxfp4", 512, 256, 72), ("fp8pc", 256, 4096, 40)])
+def test_matrix_vector_form_is_right_when_the_slot_count_is_understated(moe, oracle, enc, H, I, T):
     """The form is chosen from the routed-slot count the descriptor states. A count that is far too small
-    still gives the layer's result: live rows are walked in windows, an expert's rows one after the other."""
-    cfg = layer.MoeConfig("gemv-lie", T=40, H=512, E=8, I=256, k=4, scoring="softmax", norm_topk=True, enc="mxfp4",
+    still gives the layer's result: live rows are walked in windows of 256 (72 tokens route 360 rows: two
+    windows), an expert's rows one after the other. With 200 rows in the window a wave's share of the
+    per-channel case's 4096 GLU channels is more than the 64 whose sums (and channel scales) a wave holds
+    at a time."""
+    print(f"[case] gemv understated enc={enc} H={H} I={I} T={T}", flush=True)
+    cfg = layer.MoeConfig("gemv-lie", T=T, H=H, E=8, I=I, k=4, scoring="softmax", norm_topk=True, enc=enc,
                           arm="a16", n_shared=1, shared_mode="fold")
     plan = layer.plan_layer(cfg)
     for name in ("glu", "down"):
-        plan.insts[plan.index(name)].fj[2].u = 5          # 200 slots in truth
+        plan.insts[plan.index(name)].fj[2].u = 5          # 200 or 360 slots in truth
     dev = synth.bind(plan, "cuda", seed=3)
     host = synth.to_host(dev)
     run_device(moe, plan, dev)
