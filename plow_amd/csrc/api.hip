@@ -177,6 +177,9 @@ static uint32_t slots_of(const PlowDevInst* in, const Hint& h, uint32_t own) {
 /* Tiled or weight-streaming form of the fp8 x fp8 grouped GEMMs: the tiled one from 16 rows per expert on
  * average (the measured crossover), when it serves the shape; unknown row counts take the streaming form,
  * which is right at every size and fast at small ones. */
+/* Routed rows up to which the fp8 x fp8 DOWN runs as matrix-vector products (measured against the streaming
+ * kernel, DeepSeek-V3 shape) */
+#define W8A8_GEMV_MAX_SLOTS 36u
 static bool want_tiled(const Hint& h, uint32_t slots, const GroupW8A8& g) {
     const int env = plow_moe_tuning().w8a8_kernel;
     const bool tiled = env >= 0 ? env == 1 : h.form >= 0 ? h.form == 1 : slots >= 16u * g.E;
@@ -457,6 +460,14 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_W8A8_P16;
             g.det_k = det_k;
+            if (!det_k) { /* a batch of a few rows: the matrix-vector form, every row spread over the whole chip */
+                GroupA16 v = {};
+                v.out = g.out; v.a = g.a; v.a_f8scale = g.a_scale; v.wtab = g.wtab; v.stab = g.stab; v.meta = g.meta;
+                v.o_idx = g.row_partidx; v.gate = g.row_gate;
+                v.N = H; v.K = I; v.E = E; v.enc = 1u /* block fp8 */; v.wcols = 3u; v.wsel0 = v.wsel1 = 2u;
+                v.out_bf16 = g.part16; v.slots_hint = slots_of(in, h, 0u);
+                if (v.slots_hint <= W8A8_GEMV_MAX_SLOTS && group_a16_gemv_serves(v)) return launch_group_a16_gemv(v, false, st);
+            }
             return want_tiled(h, slots_of(in, h, 0u), g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||

@@ -67,9 +67,11 @@ __device__ __forceinline__ void gv_load(GvRow<ENC, ITER>& r, const uint8_t* wrow
     }
 }
 
-/* the lane's share of <row, x> */
-template <int ENC, int ITER>
-__device__ __forceinline__ float gv_dot(const GvRow<ENC, ITER>& r, const v4i (&x)[ITER][GvGeom<ENC>::XQ]) {
+/* the lane's share of <row, x>; xs (block fp8 with quantized activations only): the 1x128 activation scale of
+ * each piece's block, multiplied into the weight block scale as the tile kernels do */
+template <int ENC, int ITER, bool XF8 = false>
+__device__ __forceinline__ float gv_dot(const GvRow<ENC, ITER>& r, const v4i (&x)[ITER][GvGeom<ENC>::XQ],
+                                        const float (&xs)[ITER]) {
     float acc = 0.0f;
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
@@ -96,14 +98,17 @@ __device__ __forceinline__ float gv_dot(const GvRow<ENC, ITER>& r, const v4i (&x
                 part = gv_dot2(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd, 1.0f, true)),
                                (uint32_t)x[it][j >> 1][(j & 1) * 2 + 1], part);
             }
-            acc = ENC == GV_FP8BLK ? fmaf(part, r.sf[it], acc) : acc + part;
+            acc = ENC == GV_FP8BLK ? fmaf(part, XF8 ? xs[it] * r.sf[it] : r.sf[it], acc) : acc + part;
         }
     }
     return acc;
 }
 
-template <int ENC, bool GLU, int ITER>
+/* XF8 (block-fp8 weights, DOWN): the activations are e4m3 rows [rows][K] with one f32 scale per row and 128 k
+ * (g.a_f8scale), the intermediate of the fp8 x fp8 arm; they are widened to bf16 once, exactly. */
+template <int ENC, bool GLU, int ITER, bool XF8 = false>
 __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
+    static_assert(!XF8 || (ENC == GV_FP8BLK && !GLU), "quantized activations: the block-fp8 DOWN only");
     constexpr uint32_t KL = GvGeom<ENC>::KL, XQ = GvGeom<ENC>::XQ;
     constexpr int NS = GLU ? 2 : 1;
     __shared__ uint32_t l_row[GV_WINDOW], l_exp[GV_WINDOW];
@@ -194,14 +199,26 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
             if (resident && orow != PLOW_EXPERT_UNUSED && c_lo < c_hi) {
                 /* the row of activations: the lane's slice of every piece */
                 const uint32_t arow = g.a_idx ? g.a_idx[row] : row;
-                const uint8_t* xsrc = (const uint8_t*)g.a + (size_t)arow * K * 2u;
+                const uint8_t* xsrc = (const uint8_t*)g.a + (size_t)arow * K * (XF8 ? 1u : 2u);
                 v4i x[ITER][XQ];
+                float xs[ITER];
 #pragma unroll
                 for (int it = 0; it < ITER; it++) {
                     const uint32_t p = (uint32_t)it * 64u + lane;
+                    xs[it] = 1.0f;
+                    if constexpr (XF8) { /* 16 e4m3 values -> the 16 bf16 values the weight pieces meet, same order */
+                        const v4i q8 = p < pieces ? *(const v4i*)(xsrc + (size_t)p * 16u) : (v4i){0, 0, 0, 0};
+                        xs[it] = p < pieces ? g.a_f8scale[(size_t)arow * (K / 128u) + (p >> 3)] : 0.0f;
 #pragma unroll
-                    for (uint32_t j = 0; j < XQ; j++)
-                        x[it][j] = p < pieces ? *(const v4i*)(xsrc + ((size_t)p * XQ + j) * 16u) : (v4i){0, 0, 0, 0};
+                        for (int j = 0; j < 4; j++) {
+                            x[it][j >> 1][(j & 1) * 2] = (int)__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((uint32_t)q8[j], 1.0f, false));
+                            x[it][j >> 1][(j & 1) * 2 + 1] = (int)__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((uint32_t)q8[j], 1.0f, true));
+                        }
+                    } else {
+#pragma unroll
+                        for (uint32_t j = 0; j < XQ; j++)
+                            x[it][j] = p < pieces ? *(const v4i*)(xsrc + ((size_t)p * XQ + j) * 16u) : (v4i){0, 0, 0, 0};
+                    }
                 }
                 const float gate = (!GLU && g.gate) ? g.gate[row] : 1.0f;
                 /* per-channel scales: lane l applies the scale of channel c0 + l when the 64 results of a group are
@@ -246,7 +263,7 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
                         const uint32_t unit = i0 + (uint32_t)u;
                         fetch(ring[(u + AHEAD) % D], unit + (uint32_t)AHEAD, (u + AHEAD) % NS);
                         if (unit >= units) continue;
-                        const float v = gv_wave_sum(gv_dot<ENC, ITER>(ring[u], x));
+                        const float v = gv_wave_sum(gv_dot<ENC, ITER, XF8>(ring[u], x, xs));
                         if (GLU && (u % NS) == 0) { /* the gate row: its up row comes next */
                             v0 = v;
                             continue;
@@ -281,28 +298,28 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
 
 /* Every wave must be resident at once (a row's share of the waves is fixed when the kernel starts): the
  * grid is what the kernel's registers let a CU hold, asked of the runtime once per kernel. */
-template <int ENC, bool GLU, int ITER>
+template <int ENC, bool GLU, int ITER, bool XF8 = false>
 static int launch_gemv_iter(const GroupA16& g, uint32_t n_cu, hipStream_t st) {
     static int per_cu = 0; /* written once with the same value by whoever comes first */
     int nb = __atomic_load_n(&per_cu, __ATOMIC_RELAXED);
     if (nb == 0) {
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void*)k_group_a16_gemv<ENC, GLU, ITER>, (int)(GV_WAVES * WAVE), 0) != hipSuccess || nb < 1)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void*)k_group_a16_gemv<ENC, GLU, ITER, XF8>, (int)(GV_WAVES * WAVE), 0) != hipSuccess || nb < 1)
             return PLOW_MOE_EDEVICE;
         if (nb > 3) nb = 3;
         __atomic_store_n(&per_cu, nb, __ATOMIC_RELAXED);
     }
     const uint32_t min_grid = GV_WINDOW / GV_WAVES; /* never fewer waves than a window has rows */
     const uint32_t grid = n_cu * (uint32_t)nb < min_grid ? min_grid : n_cu * (uint32_t)nb;
-    k_group_a16_gemv<ENC, GLU, ITER><<<grid, GV_WAVES * WAVE, 0, st>>>(g);
+    k_group_a16_gemv<ENC, GLU, ITER, XF8><<<grid, GV_WAVES * WAVE, 0, st>>>(g);
     return 0;
 }
-template <int ENC, bool GLU>
+template <int ENC, bool GLU, bool XF8 = false>
 static int launch_gemv_enc(const GroupA16& g, uint32_t row_bytes, uint32_t n_cu, hipStream_t st) {
     const uint32_t iters = (row_bytes + 1023u) / 1024u;
-    if (iters <= 1u) return launch_gemv_iter<ENC, GLU, 1>(g, n_cu, st);
-    if (iters <= 2u) return launch_gemv_iter<ENC, GLU, 2>(g, n_cu, st);
-    if (iters <= 4u) return launch_gemv_iter<ENC, GLU, 4>(g, n_cu, st);
-    if (ENC != GV_MXFP4 && iters <= 8u) return launch_gemv_iter<ENC, GLU, (ENC != GV_MXFP4 ? 8 : 4)>(g, n_cu, st);
+    if (iters <= 1u) return launch_gemv_iter<ENC, GLU, 1, XF8>(g, n_cu, st);
+    if (iters <= 2u) return launch_gemv_iter<ENC, GLU, 2, XF8>(g, n_cu, st);
+    if (iters <= 4u) return launch_gemv_iter<ENC, GLU, 4, XF8>(g, n_cu, st);
+    if (ENC != GV_MXFP4 && iters <= 8u) return launch_gemv_iter<ENC, GLU, (ENC != GV_MXFP4 ? 8 : 4), XF8>(g, n_cu, st);
     return PLOW_MOE_EINVAL;
 }
 
@@ -322,8 +339,12 @@ bool group_a16_gemv_serves(const GroupA16& g) {
         g.slots_hint > gv_max_slots(g.enc))
         return false;
     if (g.enc != GV_BF16 && !g.stab) return false;
+    if (g.a_f8scale && (g.enc != GV_FP8BLK || g.a_idx)) return false; /* quantized activations: block-fp8 DOWN on aligned rows */
     const uint32_t row_bytes = g.enc == GV_BF16 ? g.K * 2u : (g.enc == GV_MXFP4 ? g.K / 2u : g.K);
     const uint32_t max_bytes = g.enc == GV_MXFP4 ? 4096u : 8192u;
+    /* against the streaming fp8 x fp8 DOWN the form wins from rows of a kilobyte on (DeepSeek-V3 shape, one token
+     * 44.7 -> 33.0 us); with 256-byte rows a quarter of a wave's lanes have a piece to load (11.3 -> 14.9 us) */
+    if (g.a_f8scale && row_bytes < 1024u) return false;
     return g.N != 0u && g.K != 0u && g.K % 128u == 0u && row_bytes <= max_bytes && g.enc <= GV_FP8PC && g.E <= GV_MAX_E;
 }
 
@@ -334,7 +355,9 @@ int launch_group_a16_gemv(const GroupA16& g, bool glu, hipStream_t st) {
     const uint32_t row_bytes = g.enc == GV_BF16 ? g.K * 2u : (g.enc == GV_MXFP4 ? g.K / 2u : g.K);
     switch (g.enc) {
     case GV_BF16: return glu ? launch_gemv_enc<GV_BF16, true>(g, row_bytes, n_cu, st) : launch_gemv_enc<GV_BF16, false>(g, row_bytes, n_cu, st);
-    case GV_FP8BLK: return glu ? launch_gemv_enc<GV_FP8BLK, true>(g, row_bytes, n_cu, st) : launch_gemv_enc<GV_FP8BLK, false>(g, row_bytes, n_cu, st);
+    case GV_FP8BLK:
+        if (g.a_f8scale) return glu ? PLOW_MOE_EINVAL : launch_gemv_enc<GV_FP8BLK, false, true>(g, row_bytes, n_cu, st);
+        return glu ? launch_gemv_enc<GV_FP8BLK, true>(g, row_bytes, n_cu, st) : launch_gemv_enc<GV_FP8BLK, false>(g, row_bytes, n_cu, st);
     case GV_MXFP4: return glu ? launch_gemv_enc<GV_MXFP4, true>(g, row_bytes, n_cu, st) : launch_gemv_enc<GV_MXFP4, false>(g, row_bytes, n_cu, st);
     case GV_FP8PC: return glu ? launch_gemv_enc<GV_FP8PC, true>(g, row_bytes, n_cu, st) : launch_gemv_enc<GV_FP8PC, false>(g, row_bytes, n_cu, st);
     default: return PLOW_MOE_EUNSUPPORTED;

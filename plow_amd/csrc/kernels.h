@@ -132,6 +132,9 @@ struct GroupA16 {
     const void* bias;
     uint32_t bias_rows;
     const void* wdirect[2]; /* used when wtab is NULL: the two weight tensors themselves (dense ops) */
+    /* matrix-vector form, DOWN with block-fp8 weights only: when set, `a` holds e4m3 rows [rows][K] and this their
+     * f32 scales [rows][K / 128] (the intermediate of the fp8 x fp8 arm) */
+    const float* a_f8scale;
 };
 /* the matrix-vector form of the same ops for batches that route a handful of rows in all (slots_hint says so) */
 bool group_a16_gemv_serves(const GroupA16& g);

@@ -50,6 +50,26 @@ def test_small_dsv3_like_layer(moe, oracle, T):
     check_layer(*both(moe, oracle, cfg, seed=T))
 
 
+@pytest.mark.parametrize("T,k,I,arm", [(1, 8, 1024, "w8a8"), (2, 8, 2048, "w8a8"), (4, 8, 1408 + 128, "w8a8"), (3, 4, 1024, "w8a8_p16")])
+def test_down_as_matrix_vector_products_at_a_few_tokens(moe, oracle, T, k, I, arm):
+    """With at most 36 routed rows and intermediate rows of a kilobyte or more the fp8 x fp8 DOWN runs as
+    matrix-vector products (e4m3 rows widened to bf16 exactly, activation and weight block scales multiplied
+    as in the streaming kernel): f32 and bf16 partials, rows of one and of several 1 KB pieces, experts with
+    several rows."""
+    print(f"[case] w8a8 down gemv T={T} k={k} I={I} arm={arm}", flush=True)
+    p16 = arm == "w8a8_p16"
+    cfg = layer.MoeConfig("w8a8-gemv", H=512, E=16, I=I, k=k, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          route_scale=2.5, enc="fp8blk", arm="w8a8", part_bf16=p16, n_shared=1, shared_mode="fold")
+    assert T * cfg.k_all <= 36
+    plan, dev, host = both(moe, oracle, cfg, seed=11 * T + k)
+    if p16:
+        assert_routing_equal(plan, dev, host)
+        assert_output_close(dev.np("part").reshape(-1), host.np("part").reshape(-1), "part (bf16)")
+        assert_output_close(dev.np("out"), host.np("out"))
+    else:
+        check_layer(plan, dev, host)
+
+
 @pytest.mark.parametrize("T", [1, 19, 100, 333])
 def test_glu_quantizes_bf16_rows_itself(moe, oracle, T):
     """Op 85 arm 6: bf16 rows in, quantized 1x128 where the kernel loads them, no quantizer op and no
