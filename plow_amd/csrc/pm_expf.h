@@ -45,37 +45,60 @@ PM_FN uint64_t pm_exp2_tab(uint32_t i) {
     }
 }
 
-PM_FN float pm_expf(float x) {
-    uint32_t xb;
-    __builtin_memcpy(&xb, &x, 4);
-    const uint32_t abstop = (xb >> 20) & 0x7ffu;
-    if (abstop >= 0x42bu) { /* |x| >= 88 or NaN */
-        if (xb == 0xff800000u) return 0.0f;
-        if (abstop >= 0x7f8u) return x + x;
-        if (x > 0x1.62e42ep6f) return __builtin_inff();
-        if (x < -0x1.9fe368p6f) return 0.0f;
-    }
-    const double xd = (double)x;
-    const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;
-    const double shift = 0x1.8p+52;
-    const double z = inv_ln2_n * xd;
-    double kd = z + shift;
-    uint64_t ki;
-    __builtin_memcpy(&ki, &kd, 8);
-    kd -= shift;
-    const double r = __builtin_fma(inv_ln2_n, xd, -kd);
-    uint64_t t = pm_exp2_tab((uint32_t)ki) + (ki << 47);
-    double s;
-    __builtin_memcpy(&s, &t, 8);
-    const double c0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
-    const double c1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;
-    const double c2 = 0x1.62e42ff0c52d6p-1 / 32.0;
-    const double p = __builtin_fma(c0, r, c1);
-    const double r2 = r * r;
-    double y = __builtin_fma(c2, r, 1.0);
-    y = __builtin_fma(p, r2, y);
-    y = y * s;
-    return (float)y;
+/* The body, with the table access as a parameter (TAB(i): entry i & 31) so that the device's second form
+ * below is the same arithmetic by construction. The special inputs are decided first and selected last:
+ * no lane leaves early, which the second form needs. */
+#define PM_EXPF_BODY(x, TAB)                                                                        \
+    uint32_t xb;                                                                                    \
+    __builtin_memcpy(&xb, &(x), 4);                                                                 \
+    const uint32_t abstop = (xb >> 20) & 0x7ffu;                                                    \
+    int special = 0;                                                                                \
+    float special_value = 0.0f;                                                                     \
+    if (abstop >= 0x42bu) { /* |x| >= 88 or NaN */                                                  \
+        if (xb == 0xff800000u) special = 1, special_value = 0.0f;                                   \
+        else if (abstop >= 0x7f8u) special = 1, special_value = (x) + (x);                          \
+        else if ((x) > 0x1.62e42ep6f) special = 1, special_value = __builtin_inff();                \
+        else if ((x) < -0x1.9fe368p6f) special = 1, special_value = 0.0f;                           \
+    }                                                                                               \
+    const double xd = (double)(x);                                                                  \
+    const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;                                           \
+    const double shift = 0x1.8p+52;                                                                 \
+    const double z = inv_ln2_n * xd;                                                                \
+    double kd = z + shift;                                                                          \
+    uint64_t ki;                                                                                    \
+    __builtin_memcpy(&ki, &kd, 8);                                                                  \
+    kd -= shift;                                                                                    \
+    const double r = __builtin_fma(inv_ln2_n, xd, -kd);                                             \
+    uint64_t t = TAB((uint32_t)ki) + (ki << 47);                                                    \
+    double s;                                                                                       \
+    __builtin_memcpy(&s, &t, 8);                                                                    \
+    const double c0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;                                    \
+    const double c1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;                                           \
+    const double c2 = 0x1.62e42ff0c52d6p-1 / 32.0;                                                  \
+    const double p = __builtin_fma(c0, r, c1);                                                      \
+    const double r2 = r * r;                                                                        \
+    double y = __builtin_fma(c2, r, 1.0);                                                           \
+    y = __builtin_fma(p, r2, y);                                                                    \
+    y = y * s;                                                                                      \
+    return special ? special_value : (float)y;
+
+PM_FN float pm_expf(float x) { PM_EXPF_BODY(x, pm_exp2_tab) }
+
+#if defined(__HIPCC__)
+/* Second form for code in which a whole wave evaluates the function together: lane l keeps entry l & 31 of
+ * the table in registers and an entry is fetched from the lane that holds it (two lane permutes), instead
+ * of through the 32-way selection above, which the lanes of a wave take one case after the other. Every lane
+ * of the wave must be active at the call (a permute reads nothing from an inactive lane). */
+struct PmExpLanes {
+    uint32_t lo, hi;
+};
+__device__ static inline PmExpLanes pm_exp_lanes() {
+    const uint64_t t = pm_exp2_tab(threadIdx.x & 31u);
+    return PmExpLanes{(uint32_t)t, (uint32_t)(t >> 32)};
 }
+#define PM_TAB_LANES(i)                                                                             \
+    (((uint64_t)(uint32_t)__shfl((int)tab.hi, (int)((i) & 31u), 64) << 32) | (uint64_t)(uint32_t)__shfl((int)tab.lo, (int)((i) & 31u), 64))
+__device__ static inline float pm_expf_lanes(float x, const PmExpLanes& tab) { PM_EXPF_BODY(x, PM_TAB_LANES) }
+#endif
 
 #endif

@@ -194,7 +194,8 @@ __device__ __forceinline__ void router_topk_token(const RouterArgs& a, uint32_t 
     }
     if (k > PLOW_ROUTE_MAX_TOPK) k = PLOW_ROUTE_MAX_TOPK;
 
-    /* --- score transform --- */
+    /* --- score transform (the whole wave is here: the exponential takes its table entries from the lanes) --- */
+    const PmExpLanes tab = pm_exp_lanes();
     float sc[RT_EPL];
 #pragma unroll
     for (uint32_t j = 0; j < RT_EPL; j++) {
@@ -206,7 +207,7 @@ __device__ __forceinline__ void router_topk_token(const RouterArgs& a, uint32_t 
     }
     if (sigmoid) {
 #pragma unroll
-        for (uint32_t j = 0; j < RT_EPL; j++) sc[j] = 1.0f / (1.0f + pm_expf(-sc[j]));
+        for (uint32_t j = 0; j < RT_EPL; j++) sc[j] = 1.0f / (1.0f + pm_expf_lanes(-sc[j], tab));
     } else {
         float m = -1e30f; /* the maximum is the same value in any visiting order */
 #pragma unroll
@@ -216,7 +217,8 @@ __device__ __forceinline__ void router_topk_token(const RouterArgs& a, uint32_t 
 #pragma unroll
         for (uint32_t j = 0; j < RT_EPL; j++) {
             const uint32_t e = lane + WAVE * j;
-            if (e < E) score[e] = pm_expf(sc[j] - m);
+            const float ex = pm_expf_lanes(sc[j] - m, tab); /* every lane, also those past the last expert */
+            if (e < E) score[e] = ex;
         }
         __builtin_amdgcn_wave_barrier();
         float s = 0.0f; /* the sum IS order dependent: ascending expert id, one accumulator */
@@ -306,7 +308,13 @@ __device__ __forceinline__ void router_topk_token(const RouterArgs& a, uint32_t 
             if (cand && (bi == 0u || ordv[j] > bo || (ordv[j] == bo && inv > bi))) { bo = ordv[j]; bi = inv; }
         }
         const uint32_t mo = wave_umax(bi ? bo : 0u);
-        const uint32_t mi = wave_umax((bi && bo == mo) ? bi : 0u);
+        /* the lanes whose best candidate has the winning key: almost always one, whose id is then read
+         * straight from it; several (equal keys in different lanes) take the second maximum, over ids */
+        const bool top = bi != 0u && bo == mo;
+        const unsigned long long tops = __ballot(top);
+        uint32_t mi;
+        if (__builtin_popcountll(tops) == 1) mi = (uint32_t)__builtin_amdgcn_readlane((int)bi, (int)__builtin_ctzll(tops));
+        else mi = tops ? wave_umax(top ? bi : 0u) : 0u;
         const uint32_t ew = mi ? E - mi : E - 1u; /* nothing left: the reference's pre-filled E - 1 */
         const uint32_t wl = ew & 63u, ws = ew >> 6;
         float cand_score = sc[0];
