@@ -635,20 +635,82 @@ struct AlignArgs {
 };
 
 /* LDS words the single-workgroup align needs with nw waves */
-#define AL_LDS_WORDS(nw) (((nw) + 2u) * AL_MAX_E + 1u)
+#define AL_LDS_WORDS(nw) (((nw) + 2u) * AL_MAX_E + 64u)
+#define AL_MAX_CHUNKS ((AL_MAX_E + WAVE - 1u) / WAVE) /* 64-expert chunks of the padded prefix: 17 */
+
+/* How many lower lanes of the wave hold the same expert as this lane: the lane's position among its
+ * expert's slots in this step (slots are in lane order). nl: lanes of the step that hold a slot (they are
+ * the first nl). One permute and compare per distance, none of them waiting for another, instead of one
+ * round of ballots per distinct expert of the step (some fifty rounds for 64 slots over 256 experts). */
+__device__ __forceinline__ uint32_t al_rank_below(uint32_t e, uint32_t lane, uint32_t nl) {
+    uint32_t rank = 0;
+    for (uint32_t d = 1; d < nl; d++) {
+        const uint32_t o = (uint32_t)__shfl_up((int)e, d, 64);
+        rank += (lane >= d && o == e) ? 1u : 0u;
+    }
+    return rank;
+}
+
+/* Padded exclusive prefix over the experts' row counts, by all the waves of the workgroup: every wave scans
+ * 64-expert chunks of tile counts, one wave scans the chunk totals, every thread finishes its experts.
+ * In: s_cnt[e]. Out: s_rowoff[e], meta (rowoff | cnt | tilep | total tiles). s_chunk: 2 * AL_MAX_CHUNKS words.
+ * Every thread of the workgroup calls this (three barriers inside; s_cnt must be complete before). */
+__device__ __forceinline__ void al_padded_prefix(const AlignArgs& a, uint32_t* s_rowoff, const uint32_t* s_cnt,
+                                                 uint32_t* s_chunk, uint32_t nthr) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6, nw = nthr >> 6, E = a.E;
+    const uint32_t chunks = (E + WAVE - 1u) / WAVE;
+    for (uint32_t ch = wv; ch < chunks; ch += nw) {
+        const uint32_t e = ch * WAVE + lane;
+        const uint32_t tiles = e < E ? (s_cnt[e] + PLOW_MPF_BM - 1u) / PLOW_MPF_BM : 0u;
+        uint32_t inc = tiles;
+#pragma unroll
+        for (uint32_t o = 1; o < WAVE; o <<= 1) {
+            const uint32_t v = __shfl_up(inc, o, 64);
+            if (lane >= o) inc += v;
+        }
+        if (e < E) s_rowoff[e] = inc - tiles; /* tiles before this expert inside its chunk */
+        if (lane == WAVE - 1u) s_chunk[ch] = inc;
+    }
+    __syncthreads();
+    if (wv == 0) {
+        const uint32_t v = lane < chunks ? s_chunk[lane] : 0u;
+        uint32_t inc = v;
+#pragma unroll
+        for (uint32_t o = 1; o < WAVE; o <<= 1) {
+            const uint32_t u = __shfl_up(inc, o, 64);
+            if (lane >= o) inc += u;
+        }
+        if (lane < chunks) s_chunk[AL_MAX_CHUNKS + lane] = inc - v; /* tiles before the chunk */
+        if (lane == WAVE - 1u) a.meta[3u * E] = (int32_t)inc;
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < E; e += nthr) {
+        const uint32_t excl = s_rowoff[e] + s_chunk[AL_MAX_CHUNKS + e / WAVE];
+        s_rowoff[e] = excl * PLOW_MPF_BM;
+        a.meta[e] = (int32_t)(excl * PLOW_MPF_BM);
+        a.meta[E + e] = (int32_t)s_cnt[e];
+        a.meta[2u * E + e] = (int32_t)excl;
+    }
+    __syncthreads();
+}
 /* The whole workgroup (nw waves) calls this; lds: AL_LDS_WORDS(nw) words. */
 __device__ __forceinline__ void align_body(const AlignArgs& a, uint32_t* lds, uint32_t nw) {
     uint32_t(*hist)[AL_MAX_E] = (uint32_t(*)[AL_MAX_E])lds;
     uint32_t* const s_rowoff = lds + nw * AL_MAX_E;
     uint32_t* const s_cnt = s_rowoff + AL_MAX_E;
-    uint32_t& s_carry = s_cnt[AL_MAX_E];
+    uint32_t* const s_chunk = s_cnt + AL_MAX_E;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6, nthr = nw * WAVE;
     const uint32_t E = a.E, nslot = a.T * a.k;
     /* slots per wave, a multiple of 64 so that every step of phase C is a whole wave */
     const uint32_t per = ((nslot + nthr - 1u) / nthr) * WAVE;
     const uint32_t lo = wv * per < nslot ? wv * per : nslot, hi = lo + per < nslot ? lo + per : nslot;
 
-    for (uint32_t i = tid; i < nw * E; i += nthr) hist[i / E][i % E] = 0u;
+    /* the histograms of all waves sit in one run of words (rows of AL_MAX_E, a multiple of four): 16 bytes a store */
+    {
+        uint4* const z = (uint4*)lds;
+        const uint32_t n4 = ((nw - 1u) * AL_MAX_E + E + 3u) / 4u;
+        for (uint32_t i = tid; i < n4; i += nthr) z[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
     __syncthreads();
     for (uint32_t s = lo + lane; s < hi; s += WAVE) {
         const uint32_t e = a.table[s].eid;
@@ -664,35 +726,10 @@ __device__ __forceinline__ void align_body(const AlignArgs& a, uint32_t* lds, ui
         }
         s_cnt[e] = run;
     }
-    if (tid == 0) s_carry = 0u;
     __syncthreads();
-    if (wv == 0) { /* padded exclusive prefix over experts, 64 at a time */
-        for (uint32_t e0 = 0; e0 < E; e0 += WAVE) {
-            const uint32_t e = e0 + lane;
-            const uint32_t c = e < E ? s_cnt[e] : 0u;
-            const uint32_t tiles = (c + PLOW_MPF_BM - 1u) / PLOW_MPF_BM;
-            uint32_t inc = tiles;
-#pragma unroll
-            for (uint32_t o = 1; o < WAVE; o <<= 1) {
-                const uint32_t v = __shfl_up(inc, o, 64);
-                if (lane >= o) inc += v;
-            }
-            const uint32_t carry = s_carry;
-            const uint32_t excl = carry + inc - tiles;
-            if (e < E) {
-                s_rowoff[e] = excl * PLOW_MPF_BM;
-                a.meta[e] = (int32_t)(excl * PLOW_MPF_BM);
-                a.meta[E + e] = (int32_t)c;
-                a.meta[2u * E + e] = (int32_t)excl;
-            }
-            __builtin_amdgcn_wave_barrier();
-            if (lane == WAVE - 1u) s_carry = carry + inc;
-            __builtin_amdgcn_wave_barrier();
-        }
-        if (lane == 0) a.meta[3u * E] = (int32_t)s_carry;
-    }
-    __syncthreads();
+    al_padded_prefix(a, s_rowoff, s_cnt, s_chunk, nthr);
     /* pad rows: [rowoff + cnt, rowoff + 64 * ceil(cnt / 64)) */
+#pragma unroll 4
     for (uint32_t i = tid; i < E * PLOW_MPF_BM; i += nthr) {
         const uint32_t e = i / PLOW_MPF_BM, j = i % PLOW_MPF_BM;
         const uint32_t c = s_cnt[e], r = s_rowoff[e] + c + j;
@@ -702,28 +739,20 @@ __device__ __forceinline__ void align_body(const AlignArgs& a, uint32_t* lds, ui
             a.row_gate[r] = 0.0f;
         }
     }
-    /* stable scatter, each wave on its own range and its own cursors (no block barrier needed) */
+    /* stable scatter, each wave on its own range and its own cursors (no block barrier needed): a slot goes
+     * to its expert's first row + the wave's cursor + its position among the step's slots of that expert;
+     * the cursors advance after every lane has read its own (a wave's LDS operations run in order) */
     for (uint32_t s0 = lo; s0 < hi; s0 += WAVE) {
         const uint32_t s = s0 + lane;
         const bool in = s < hi;
         const uint32_t e = in ? a.table[s].eid : PLOW_EXPERT_UNUSED;
         const float g = in ? a.table[s].gate : 0.0f;
         const bool live = e < E;
-        unsigned long long todo = __ballot(live);
-        uint32_t pos = 0;
-        while (todo) {
-            const uint32_t leader = (uint32_t)__builtin_ctzll(todo);
-            const uint32_t e0 = (uint32_t)__shfl((int)e, (int)leader, 64);
-            const unsigned long long same = __ballot(live && e == e0);
-            const uint32_t cursor = hist[wv][e0];
-            if (live && e == e0)
-                pos = s_rowoff[e0] + cursor + (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
-            __builtin_amdgcn_wave_barrier();
-            if (lane == leader) hist[wv][e0] = cursor + (uint32_t)__builtin_popcountll(same);
-            __builtin_amdgcn_wave_barrier();
-            todo &= ~same;
-        }
+        const uint32_t nl = hi - s0 < WAVE ? hi - s0 : WAVE;
+        const uint32_t rank = al_rank_below(e, lane, nl);
         if (live) {
+            const uint32_t pos = s_rowoff[e] + hist[wv][e] + rank;
+            atomicAdd(&hist[wv][e], 1u);
             a.row_token[pos] = s / a.k;
             a.row_partidx[pos] = s;
             a.row_gate[pos] = g;
@@ -731,7 +760,7 @@ __device__ __forceinline__ void align_body(const AlignArgs& a, uint32_t* lds, ui
     }
 }
 __global__ __launch_bounds__(AL_WAVES* WAVE) void k_align(AlignArgs a) {
-    __shared__ uint32_t al_lds[AL_LDS_WORDS(AL_WAVES)];
+    __shared__ __attribute__((aligned(16))) uint32_t al_lds[AL_LDS_WORDS(AL_WAVES)];
     align_body(a, al_lds, AL_WAVES);
 }
 
@@ -817,45 +846,26 @@ __global__ __launch_bounds__(AL_CHUNK) void k_align_scan(AlignArgs a, uint32_t* 
                                                          uint32_t nchunk) {
     __shared__ uint32_t s_rowoff[AL_MAX_E];
     __shared__ uint32_t s_cnt[AL_MAX_E];
-    __shared__ uint32_t s_carry;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6, E = a.E;
+    __shared__ uint32_t s_chunk[2u * AL_MAX_CHUNKS];
+    const uint32_t tid = threadIdx.x, E = a.E;
     for (uint32_t e = tid; e < E; e += AL_CHUNK) {
         uint32_t run = 0;
-        for (uint32_t c = 0; c < nchunk; c++) {
-            const uint32_t v = chunk_hist[(size_t)c * E + e];
-            chunk_hist[(size_t)c * E + e] = run;
-            run += v;
+        /* eight chunks' counts are asked for together: one trip to memory per eight, not one per chunk */
+        for (uint32_t c0 = 0; c0 < nchunk; c0 += 8u) {
+            uint32_t v[8];
+#pragma unroll
+            for (uint32_t j = 0; j < 8u; j++) v[j] = c0 + j < nchunk ? chunk_hist[(size_t)(c0 + j) * E + e] : 0u;
+#pragma unroll
+            for (uint32_t j = 0; j < 8u; j++) {
+                if (c0 + j < nchunk) chunk_hist[(size_t)(c0 + j) * E + e] = run;
+                run += v[j];
+            }
         }
         s_cnt[e] = run;
     }
-    if (tid == 0) s_carry = 0u;
     __syncthreads();
-    if (wv == 0) {
-        for (uint32_t e0 = 0; e0 < E; e0 += WAVE) {
-            const uint32_t e = e0 + lane;
-            const uint32_t c = e < E ? s_cnt[e] : 0u;
-            const uint32_t tiles = (c + PLOW_MPF_BM - 1u) / PLOW_MPF_BM;
-            uint32_t inc = tiles;
-#pragma unroll
-            for (uint32_t o = 1; o < WAVE; o <<= 1) {
-                const uint32_t v = __shfl_up(inc, o, 64);
-                if (lane >= o) inc += v;
-            }
-            const uint32_t carry = s_carry;
-            const uint32_t excl = carry + inc - tiles;
-            if (e < E) {
-                s_rowoff[e] = excl * PLOW_MPF_BM;
-                a.meta[e] = (int32_t)(excl * PLOW_MPF_BM);
-                a.meta[E + e] = (int32_t)c;
-                a.meta[2u * E + e] = (int32_t)excl;
-            }
-            __builtin_amdgcn_wave_barrier();
-            if (lane == WAVE - 1u) s_carry = carry + inc;
-            __builtin_amdgcn_wave_barrier();
-        }
-        if (lane == 0) a.meta[3u * E] = (int32_t)s_carry;
-    }
-    __syncthreads();
+    al_padded_prefix(a, s_rowoff, s_cnt, s_chunk, AL_CHUNK);
+#pragma unroll 4
     for (uint32_t i = tid; i < E * PLOW_MPF_BM; i += AL_CHUNK) {
         const uint32_t e = i / PLOW_MPF_BM, j = i % PLOW_MPF_BM;
         const uint32_t c = s_cnt[e], r = s_rowoff[e] + c + j;
@@ -868,11 +878,15 @@ __global__ __launch_bounds__(AL_CHUNK) void k_align_scan(AlignArgs a, uint32_t* 
 }
 
 __global__ __launch_bounds__(AL_CHUNK) void k_align_scatter(AlignArgs a, const uint32_t* __restrict__ chunk_hist) {
-    __shared__ uint32_t hist[AL_WAVES][AL_MAX_E];
+    __shared__ __attribute__((aligned(16))) uint32_t hist[AL_WAVES][AL_MAX_E];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
     const uint32_t E = a.E, nslot = a.T * a.k;
     const uint32_t s = blockIdx.x * AL_CHUNK + tid;
-    for (uint32_t i = tid; i < AL_WAVES * E; i += AL_CHUNK) hist[i / E][i % E] = 0u;
+    {
+        uint4* const z = (uint4*)&hist[0][0];
+        const uint32_t n4 = ((AL_WAVES - 1u) * AL_MAX_E + E + 3u) / 4u;
+        for (uint32_t i = tid; i < n4; i += AL_CHUNK) z[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
     __syncthreads();
     const bool in = s < nslot;
     const uint32_t e = in ? a.table[s].eid : PLOW_EXPERT_UNUSED;
@@ -891,16 +905,11 @@ __global__ __launch_bounds__(AL_CHUNK) void k_align_scatter(AlignArgs a, const u
         }
     }
     __syncthreads();
-    unsigned long long todo = __ballot(live);
-    uint32_t pos = 0;
-    while (todo) {
-        const uint32_t leader = (uint32_t)__builtin_ctzll(todo);
-        const uint32_t e0 = (uint32_t)__shfl((int)e, (int)leader, 64);
-        const unsigned long long same = __ballot(live && e == e0);
-        if (live && e == e0) pos = hist[wv][e0] + (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
-        todo &= ~same;
-    }
+    const uint32_t s0 = blockIdx.x * AL_CHUNK + wv * WAVE; /* the wave's first slot */
+    const uint32_t nl = s0 >= nslot ? 0u : (nslot - s0 < WAVE ? nslot - s0 : WAVE);
+    const uint32_t rank = al_rank_below(e, lane, nl);
     if (live) {
+        const uint32_t pos = hist[wv][e] + rank;
         a.row_token[pos] = s / a.k;
         a.row_partidx[pos] = s;
         a.row_gate[pos] = g;
