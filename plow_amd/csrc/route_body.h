@@ -9,7 +9,8 @@
 #include "pm_expf.h"
 
 /* Few outputs (decode): TOK tokens x 64 experts per workgroup, one consumer wave per token. Every output
- * is a chain of K dependent multiply-adds (2 ns a step on this chip), so the kernel's time is the chain's
+ * is a chain of K dependent multiply-adds (9.3 cycles, 3.9 ns, a step on this chip whatever the operands:
+ * register, scalar or DPP), so the kernel's time is the chain's
  * and the job is to keep everything else off the consumer waves' instruction streams:
  *  - four stager waves (16 weight rows each) own every global load. They widen the weight rows to f32
  *    into a double-buffered LDS tile shared by the consumers and copy the tokens' bf16 rows beside it.
