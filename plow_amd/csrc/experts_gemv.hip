@@ -121,7 +121,6 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
     const uint32_t wrow_bytes = ENC == GV_BF16 ? K * 2u : (ENC == GV_MXFP4 ? K / 2u : K);
     const uint32_t srow_bytes = ENC == GV_MXFP4 ? K / 32u : (ENC == GV_FP8BLK ? (K / 128u) * 4u : 0u);
     const uint32_t wmul = g.wmul ? g.wmul : 1u;
-    const uint32_t total = (uint32_t)g.meta[3u * E] * PLOW_MPF_BM; /* aligned rows, pads included: an upper bound */
 
     /* live rows in windows of GV_WINDOW, by their ordinal among the live rows */
     for (uint32_t base = 0;; base += GV_WINDOW) {
@@ -161,7 +160,7 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
         }
         __syncthreads();
         const uint32_t n = l_n;
-        if (n == 0u || base >= total) break;
+        if (n == 0u) break; /* no live row at or past `base` */
 
         /* the waves are dealt out evenly over the window's rows; a row's waves split its channels evenly */
         constexpr uint32_t RING = ITER == 1 ? 8u : (ITER == 8 ? 2u : 4u);
