@@ -22,6 +22,9 @@ enum { GV_BF16 = 0, GV_FP8BLK = 1, GV_MXFP4 = 2, GV_FP8PC = 3 };
 #define GV_QUADS_FROM 32u /* rows from which a workgroup's waves take neighbouring rows */
 #define GV_MAX_E 1088u
 #define GV_ECHUNKS (GV_MAX_E / WAVE)
+/* A pointer made from a table word is generic to the compiler, which then emits flat loads (they count on
+ * both memory counters); this says what it is: global memory. */
+typedef const __attribute__((address_space(1))) uint8_t* gv_gptr;
 
 /* k values a lane's 16 bytes of a weight row hold, and the 16-byte pieces of its activation slice */
 template <int ENC> struct GvGeom;
@@ -61,9 +64,9 @@ __device__ __forceinline__ void gv_load(GvRow<ENC, ITER>& r, const uint8_t* wrow
     for (int it = 0; it < ITER; it++) {
         const uint32_t p = (uint32_t)it * 64u + lane; /* the lane's 16-byte piece of the row */
         const bool in = p < pieces;
-        r.w[it] = in ? *(const v4i*)(wrow + (size_t)p * 16u) : (v4i){0, 0, 0, 0};
-        if (ENC == GV_MXFP4) r.sb[it] = in ? (uint32_t)srow[p] : 0u;
-        if (ENC == GV_FP8BLK) r.sf[it] = in ? ((const float*)srow)[p >> 3] : 0.0f; /* 8 pieces of 16 k per 128-k block */
+        r.w[it] = in ? *(const __attribute__((address_space(1))) v4i*)((gv_gptr)wrow + (size_t)p * 16u) : (v4i){0, 0, 0, 0};
+        if (ENC == GV_MXFP4) r.sb[it] = in ? (uint32_t)((gv_gptr)srow)[p] : 0u;
+        if (ENC == GV_FP8BLK) r.sf[it] = in ? ((const __attribute__((address_space(1))) float*)(gv_gptr)srow)[p >> 3] : 0.0f; /* 8 pieces of 16 k per 128-k block */
     }
 }
 
