@@ -177,30 +177,46 @@ __global__ __launch_bounds__(256) void k_quant_row(uint8_t* __restrict__ xq, bf1
     const uint32_t row = blockIdx.x, tid = threadIdx.x;
     bf16_t* xr = x + (size_t)row * K;
     float amax = 0.0f;
-    if (VEC) {
-        for (uint32_t k = tid * 8u; k < K; k += 2048u) {
-            uint4 raw;
-            if (gate) {
-                const uint4 g4 = *(const uint4*)(gate + (size_t)row * K + k);
-                const uint4 u4 = *(const uint4*)(up + (size_t)row * K + k);
-                const uint32_t gv[4] = {g4.x, g4.y, g4.z, g4.w}, uv[4] = {u4.x, u4.y, u4.z, u4.w};
-                uint32_t o[4];
+    /* eight elements at k: produced (act(gate) * up, stored) or loaded; their |max| joins amax */
+    auto first_pass = [&](uint32_t k) -> uint4 {
+        uint4 raw;
+        if (gate) {
+            const uint4 g4 = *(const uint4*)(gate + (size_t)row * K + k);
+            const uint4 u4 = *(const uint4*)(up + (size_t)row * K + k);
+            const uint32_t gv[4] = {g4.x, g4.y, g4.z, g4.w}, uv[4] = {u4.x, u4.y, u4.z, u4.w};
+            uint32_t o[4];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const float lo = act_gate_only(__uint_as_float(gv[j] << 16), act) * __uint_as_float(uv[j] << 16);
-                    const float hi = act_gate_only(__uint_as_float(gv[j] & 0xFFFF0000u), act) *
-                                     __uint_as_float(uv[j] & 0xFFFF0000u);
-                    o[j] = (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
-                }
-                raw = make_uint4(o[0], o[1], o[2], o[3]);
-                *(uint4*)(xr + k) = raw;
-            } else {
-                raw = *(const uint4*)(xr + k);
+            for (int j = 0; j < 4; j++) {
+                const float lo = act_gate_only(__uint_as_float(gv[j] << 16), act) * __uint_as_float(uv[j] << 16);
+                const float hi = act_gate_only(__uint_as_float(gv[j] & 0xFFFF0000u), act) *
+                                 __uint_as_float(uv[j] & 0xFFFF0000u);
+                o[j] = (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
             }
-            const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+            raw = make_uint4(o[0], o[1], o[2], o[3]);
+            *(uint4*)(xr + k) = raw;
+        } else {
+            raw = *(const uint4*)(xr + k);
+        }
+        const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(v[j] << 16)), fabsf(__uint_as_float(v[j] & 0xFFFF0000u))));
+        for (int j = 0; j < 4; j++)
+            amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(v[j] << 16)), fabsf(__uint_as_float(v[j] & 0xFFFF0000u))));
+        return raw;
+    };
+    /* VEC: a thread's pieces of the row stay in registers between the two passes when the row has at most four
+     * per thread (K <= 8192): the second pass then starts without another trip to memory */
+    const bool hold = VEC && K <= 8192u;
+    uint4 held[4];
+    if (VEC) {
+        if (hold) {
+#pragma unroll
+            for (uint32_t it = 0; it < 4u; it++) {
+                const uint32_t k = tid * 8u + it * 2048u;
+                held[it] = make_uint4(0u, 0u, 0u, 0u);
+                if (k < K) held[it] = first_pass(k);
+            }
+        } else {
+            for (uint32_t k = tid * 8u; k < K; k += 2048u) (void)first_pass(k);
         }
     } else {
         for (uint32_t k = tid; k < K; k += 256u) {
@@ -216,38 +232,104 @@ __global__ __launch_bounds__(256) void k_quant_row(uint8_t* __restrict__ xq, bf1
     const float s = fmaxf(amax * (1.0f / 448.0f), 1e-12f);
     const float inv = 1.0f / s;
     if (tid == 0) scale[row] = s;
-    if (VEC) {
-        for (uint32_t k = tid * 8u; k < K; k += 2048u) {
-            const uint4 raw = *(const uint4*)(xr + k);
-            const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
-            float xf[8], f[8];
-            bool plain = true;
+    auto second_pass = [&](uint32_t k, const uint4 raw) {
+        const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+        float xf[8], f[8];
+        bool plain = true;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            xf[2 * j] = __uint_as_float(v[j] << 16);
+            xf[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            f[j] = xf[j] * inv;
+            plain = plain && e4m3_in_range(f[j]);
+        }
+        uint2 q;
+        if (plain) {
+            q.x = cvt4_e4m3(f[0], f[1], f[2], f[3]);
+            q.y = cvt4_e4m3(f[4], f[5], f[6], f[7]);
+        } else { /* NaN or infinities among the eight: every byte by the total rule */
+            q.x = q.y = 0u;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                xf[2 * j] = __uint_as_float(v[j] << 16);
-                xf[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+                q.x |= e4m3_any(f[j], xf[j]) << (8 * j);
+                q.y |= e4m3_any(f[4 + j], xf[4 + j]) << (8 * j);
             }
+        }
+        *(uint2*)(xq + (size_t)row * K + k) = q;
+    };
+    if (VEC) {
+        if (hold) {
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                f[j] = xf[j] * inv;
-                plain = plain && e4m3_in_range(f[j]);
+            for (uint32_t it = 0; it < 4u; it++) {
+                const uint32_t k = tid * 8u + it * 2048u;
+                if (k < K) second_pass(k, held[it]);
             }
-            uint2 q;
-            if (plain) {
-                q.x = cvt4_e4m3(f[0], f[1], f[2], f[3]);
-                q.y = cvt4_e4m3(f[4], f[5], f[6], f[7]);
-            } else { /* NaN or infinities among the eight: every byte by the total rule */
-                q.x = q.y = 0u;
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    q.x |= e4m3_any(f[j], xf[j]) << (8 * j);
-                    q.y |= e4m3_any(f[4 + j], xf[4 + j]) << (8 * j);
-                }
-            }
-            *(uint2*)(xq + (size_t)row * K + k) = q;
+        } else {
+            for (uint32_t k = tid * 8u; k < K; k += 2048u) second_pass(k, *(const uint4*)(xr + k));
         }
     } else {
         for (uint32_t k = tid; k < K; k += 256u) xq[(size_t)row * K + k] = (uint8_t)e4m3_any(bf2f(xr[k]) * inv, bf2f(xr[k]));
+    }
+}
+
+/* Rows of at most 2048 elements that only need quantizing (no gate / up): one wave per row, four rows per
+ * workgroup. A lane holds its up to four 8-element pieces between the two passes, the row's maximum is a wave
+ * reduction, and there is no barrier and no LDS: the same values in the same order as k_quant_row<true>
+ * (a maximum does not depend on the order of its operands). */
+__global__ __launch_bounds__(256) void k_quant_row_wave(uint8_t* __restrict__ xq, const bf16_t* __restrict__ x,
+                                                        float* __restrict__ scale, uint32_t M, uint32_t K) {
+    const uint32_t lane = threadIdx.x & 63u, row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= M) return; /* the whole wave */
+    const bf16_t* xr = x + (size_t)row * K;
+    uint4 held[4];
+    float amax = 0.0f;
+#pragma unroll
+    for (uint32_t it = 0; it < 4u; it++) {
+        const uint32_t k = lane * 8u + it * 512u;
+        held[it] = make_uint4(0u, 0u, 0u, 0u);
+        if (k < K) held[it] = *(const uint4*)(xr + k);
+        const uint32_t v[4] = {held[it].x, held[it].y, held[it].z, held[it].w};
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(v[j] << 16)), fabsf(__uint_as_float(v[j] & 0xFFFF0000u))));
+    }
+    amax = wave_max(amax);
+    const float s = fmaxf(amax * (1.0f / 448.0f), 1e-12f);
+    const float inv = 1.0f / s;
+    if (lane == 0) scale[row] = s;
+#pragma unroll
+    for (uint32_t it = 0; it < 4u; it++) {
+        const uint32_t k = lane * 8u + it * 512u;
+        if (k >= K) continue;
+        const uint32_t v[4] = {held[it].x, held[it].y, held[it].z, held[it].w};
+        float xf[8], f[8];
+        bool plain = true;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            xf[2 * j] = __uint_as_float(v[j] << 16);
+            xf[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            f[j] = xf[j] * inv;
+            plain = plain && e4m3_in_range(f[j]);
+        }
+        uint2 q;
+        if (plain) {
+            q.x = cvt4_e4m3(f[0], f[1], f[2], f[3]);
+            q.y = cvt4_e4m3(f[4], f[5], f[6], f[7]);
+        } else { /* NaN or infinities among the eight: every byte by the total rule */
+            q.x = q.y = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                q.x |= e4m3_any(f[j], xf[j]) << (8 * j);
+                q.y |= e4m3_any(f[4 + j], xf[4 + j]) << (8 * j);
+            }
+        }
+        *(uint2*)(xq + (size_t)row * K + k) = q;
     }
 }
 
@@ -255,6 +337,10 @@ int launch_quant_row(void* xq, void* x, float* scale, const void* gate, const vo
                      uint32_t M, uint32_t K, hipStream_t st) {
     if (K == 0 || M == 0 || (gate == nullptr) != (up == nullptr)) return PLOW_MOE_EINVAL;
     const uintptr_t al = (uintptr_t)x | (uintptr_t)gate | (uintptr_t)up;
+    if (!gate && K % 8u == 0u && K <= 2048u && al % 16u == 0u && (uintptr_t)xq % 8u == 0u && M >= 64u) {
+        k_quant_row_wave<<<(M + 3u) / 4u, 256, 0, st>>>((uint8_t*)xq, (const bf16_t*)x, scale, M, K);
+        return 0;
+    }
     if (K % 8u == 0u && al % 16u == 0u && (uintptr_t)xq % 8u == 0u)
         k_quant_row<true><<<M, 256, 0, st>>>((uint8_t*)xq, (bf16_t*)x, scale, (const bf16_t*)gate, (const bf16_t*)up, act, K);
     else
