@@ -50,15 +50,17 @@ def test_small_dsv3_like_layer(moe, oracle, T):
     check_layer(*both(moe, oracle, cfg, seed=T))
 
 
-@pytest.mark.parametrize("T,k,I,arm", [(1, 8, 1024, "w8a8"), (2, 8, 2048, "w8a8"), (4, 8, 1408 + 128, "w8a8"), (3, 4, 1024, "w8a8_p16")])
-def test_down_as_matrix_vector_products_at_a_few_tokens(moe, oracle, T, k, I, arm):
+@pytest.mark.parametrize("T,k,H,I,arm", [(1, 8, 512, 1024, "w8a8"), (2, 8, 512, 2048, "w8a8"), (4, 8, 512, 1408 + 128, "w8a8"),
+                                         (3, 4, 512, 1024, "w8a8_p16"), (1, 8, 1024, 1024, "w8a8"), (4, 8, 2048 + 512, 1280, "w8a8"),
+                                         (2, 6, 7168, 256, "w8a8")])
+def test_few_tokens_as_matrix_vector_products(moe, oracle, T, k, H, I, arm):
     """With at most 36 routed rows and intermediate rows of a kilobyte or more the fp8 x fp8 DOWN runs as
     matrix-vector products (e4m3 rows widened to bf16 exactly, activation and weight block scales multiplied
     as in the streaming kernel): f32 and bf16 partials, rows of one and of several 1 KB pieces, experts with
-    several rows."""
-    print(f"[case] w8a8 down gemv T={T} k={k} I={I} arm={arm}", flush=True)
+    several rows, hidden sizes from 512 to 7168 (the GLU stays on its tile kernel at every one of them)."""
+    print(f"[case] w8a8 gemv T={T} k={k} H={H} I={I} arm={arm}", flush=True)
     p16 = arm == "w8a8_p16"
-    cfg = layer.MoeConfig("w8a8-gemv", H=512, E=16, I=I, k=k, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+    cfg = layer.MoeConfig("w8a8-gemv", H=H, E=16, I=I, k=k, T=T, scoring="sigmoid", norm_topk=True, bias=True,
                           route_scale=2.5, enc="fp8blk", arm="w8a8", part_bf16=p16, n_shared=1, shared_mode="fold")
     assert T * cfg.k_all <= 36
     plan, dev, host = both(moe, oracle, cfg, seed=11 * T + k)
