@@ -705,6 +705,10 @@ __device__ __forceinline__ void align_body(const AlignArgs& a, uint32_t* lds, ui
     const uint32_t per = ((nslot + nthr - 1u) / nthr) * WAVE;
     const uint32_t lo = wv * per < nslot ? wv * per : nslot, hi = lo + per < nslot ? lo + per : nslot;
 
+    /* the wave's first 64 slots are asked for before anything else and kept: the trip to memory runs under the
+     * clearing of the histograms, and the scatter's first step (the only one up to 1024 slots) needs no second */
+    const uint32_t e_first = lo + lane < hi ? a.table[lo + lane].eid : PLOW_EXPERT_UNUSED;
+    const float g_first = lo + lane < hi ? a.table[lo + lane].gate : 0.0f;
     /* the histograms of all waves sit in one run of words (rows of AL_MAX_E, a multiple of four): 16 bytes a store */
     {
         uint4* const z = (uint4*)lds;
@@ -713,7 +717,7 @@ __device__ __forceinline__ void align_body(const AlignArgs& a, uint32_t* lds, ui
     }
     __syncthreads();
     for (uint32_t s = lo + lane; s < hi; s += WAVE) {
-        const uint32_t e = a.table[s].eid;
+        const uint32_t e = s < lo + WAVE ? e_first : a.table[s].eid;
         if (e < E) atomicAdd(&hist[wv][e], 1u);
     }
     __syncthreads();
@@ -745,8 +749,8 @@ __device__ __forceinline__ void align_body(const AlignArgs& a, uint32_t* lds, ui
     for (uint32_t s0 = lo; s0 < hi; s0 += WAVE) {
         const uint32_t s = s0 + lane;
         const bool in = s < hi;
-        const uint32_t e = in ? a.table[s].eid : PLOW_EXPERT_UNUSED;
-        const float g = in ? a.table[s].gate : 0.0f;
+        const uint32_t e = s0 == lo ? e_first : (in ? a.table[s].eid : PLOW_EXPERT_UNUSED);
+        const float g = s0 == lo ? g_first : (in ? a.table[s].gate : 0.0f);
         const bool live = e < E;
         const uint32_t nl = hi - s0 < WAVE ? hi - s0 : WAVE;
         const uint32_t rank = al_rank_below(e, lane, nl);
