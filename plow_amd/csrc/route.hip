@@ -183,7 +183,9 @@ __global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ o
     float af[2][4], bf[2][4];
     auto read_piece = [&](uint32_t stage, uint32_t pc) {
         const uint32_t addr = obase + stage * (uint32_t)sizeof(RsmStage) + ((pc ^ osw) << 4);
-        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:4096" : "=v"(xa), "=v"(wb) : "v"(addr) : "memory");
+        /* early-clobber outputs: the first read's destination must not be the register the second takes its
+         * address from (the data may land before the second instruction issues) */
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:4096" : "=&v"(xa), "=&v"(wb) : "v"(addr) : "memory");
     };
     auto widen = [&](uint32_t h, int d0, int d1) {
         if (d0 == 0) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa), "+v"(wb));
