@@ -131,20 +131,25 @@ struct RsmStage {
     uint8_t w[32u * 128u];
 };
 typedef __attribute__((address_space(3))) void rsm_lds_void;
-__global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ out, const bf16_t* __restrict__ x,
-                                                           const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
-                                                           uint32_t K) {
-    /* four independent waves per workgroup (a 2 x 2 block of tiles): 96 KB of LDS makes it one workgroup
-     * per CU, which puts exactly one wave on every SIMD */
+/* NWV waves per workgroup, rings of ST chunks: 4 x 3 (one wave per SIMD, two chunks ahead), or 8 x 2 (two waves
+ * per SIMD, one chunk ahead: a wave's matrix instructions fill the other's issue gaps) when there are tiles
+ * enough for two per SIMD. */
+template <uint32_t NWV, uint32_t ST>
+__global__ __launch_bounds__(NWV * 64u) void k_router_score_mfma(float* __restrict__ out, const bf16_t* __restrict__ x,
+                                                                 const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
+                                                                 uint32_t K) {
+    static_assert((NWV == 4u && ST == 3u) || (NWV == 8u && ST == 2u), "4 waves x 3 chunks or 8 waves x 2 chunks");
+    /* independent waves (a 2 x 2 or 4 x 2 block of tiles): 96 / 128 KB of LDS makes it one workgroup per CU,
+     * which puts exactly one (two) waves on every SIMD */
     extern __shared__ __attribute__((aligned(16))) uint8_t rsm_raw[];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    RsmStage* const ring = (RsmStage*)rsm_raw + wv * RSM_STAGES;
+    RsmStage* const ring = (RsmStage*)rsm_raw + wv * ST;
     /* Workgroup b runs on XCD b % 8 and each XCD has its own L2: the logical index gives one XCD
      * consecutive workgroups, which share their token rows (the expert-tile index runs fastest) */
     const uint32_t G = gridDim.x, gx = (N + 63u) / 64u;
     const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
-    const uint32_t m0 = ((wg / gx) * 2u + (wv >> 1)) * 32u, n0 = ((wg % gx) * 2u + (wv & 1u)) * 32u;
+    const uint32_t m0 = ((wg / gx) * (NWV / 2u) + (wv >> 1)) * 32u, n0 = ((wg % gx) * 2u + (wv & 1u)) * 32u;
     if (m0 >= M || n0 >= N) return; /* whole wave; there is no barrier below */
     const uint32_t NC = K / 64u;
     /* load j covers rows 8j .. 8j + 7: lane -> (row lane >> 3, LDS piece lane & 7); rows past the end
@@ -159,7 +164,7 @@ __global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ o
         wsrc[j] = (const uint8_t*)(w + (size_t)nr * K) + ((lp ^ ((row >> 1) & 7u)) << 4);
     }
     auto issue = [&](uint32_t c) {
-        RsmStage* s = &ring[c % RSM_STAGES];
+        RsmStage* s = &ring[c % ST];
 #pragma unroll
         for (uint32_t j = 0; j < 4u; j++)
             __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
@@ -197,8 +202,8 @@ __global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ o
     };
     issue(0u);
     if (NC > 1u) issue(1u);
-    if (NC > 2u) issue(2u);
-    if (NC > 2u) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    if (ST > 2u && NC > 2u) issue(2u);
+    if (ST > 2u && NC > 2u) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     else if (NC > 1u) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     read_piece(0u, 0u);
@@ -207,7 +212,7 @@ __global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ o
 #define RSM_MFMA(d) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][d], bf[cur][d], acc, 0, 0, 0)
 #define RSM_FENCE() __builtin_amdgcn_sched_barrier(0)
     for (uint32_t c = 0; c < NC; c++) {
-        const uint32_t stn = st == RSM_STAGES - 1u ? 0u : st + 1u;
+        const uint32_t stn = st == ST - 1u ? 0u : st + 1u;
 #pragma unroll
         for (uint32_t pc = 0; pc < 8u; pc++) {
             const uint32_t cur = pc & 1u, nxt = cur ^ 1u;
@@ -218,8 +223,9 @@ __global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ o
             RSM_FENCE();
             if (pc == 7u) {
                 /* every piece of chunk c has been read: chunk c + 1 must have landed before its first
-                 * piece is read, and chunk c's stage takes chunk c + 3 */
-                if (c + 2u < NC) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                 * piece is read (with three stages chunk c + 2's loads may stay outstanding), and chunk c's
+                 * stage takes chunk c + ST */
+                if (ST > 2u && c + 2u < NC) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
                 else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 read_piece(stn, 0u); /* past the last chunk: stale bytes, never used */
             } else {
@@ -228,20 +234,20 @@ __global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ o
             RSM_FENCE();
             RSM_MFMA(1);
             RSM_FENCE();
-            if (pc == 7u && c + 3u < NC) {
-                RsmStage* s = &ring[(c + 3u) % RSM_STAGES];
+            if (pc == 7u && c + ST < NC) {
+                RsmStage* s = &ring[(c + ST) % ST];
 #pragma unroll
                 for (uint32_t j = 0; j < 4u; j++)
-                    __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)(c + 3u) * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)(c + ST) * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
             }
             RSM_FENCE();
             RSM_MFMA(2);
             RSM_FENCE();
-            if (pc == 7u && c + 3u < NC) {
-                RsmStage* s = &ring[(c + 3u) % RSM_STAGES];
+            if (pc == 7u && c + ST < NC) {
+                RsmStage* s = &ring[(c + ST) % ST];
 #pragma unroll
                 for (uint32_t j = 0; j < 4u; j++)
-                    __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)(c + 3u) * 128u), (rsm_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)(c + ST) * 128u), (rsm_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
             }
             RSM_FENCE();
             widen(nxt, 0, 2);
@@ -529,13 +535,15 @@ __global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(
 
 #define RS16_LDS (4u * RSM_STAGES * (uint32_t)sizeof(Rs16Stage))
 #define RSM_LDS (4u * RSM_STAGES * (uint32_t)sizeof(RsmStage))
+#define RSM_LDS8 (8u * 2u * (uint32_t)sizeof(RsmStage))
 
 /* dynamic-LDS limits of the score kernels, once per device (plow_moe_device_setup) */
 static bool rf_setup();
 int plow_moe_route_setup() {
     const bool ok = rf_setup() &&
         hipFuncSetAttribute((const void*)k_router_score_mfma16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RS16_LDS) == hipSuccess &&
-        hipFuncSetAttribute((const void*)k_router_score_mfma, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSM_LDS) == hipSuccess &&
+        hipFuncSetAttribute((const void*)k_router_score_mfma<4u, 3u>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSM_LDS) == hipSuccess &&
+        hipFuncSetAttribute((const void*)k_router_score_mfma<8u, 2u>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSM_LDS8) == hipSuccess &&
         hipFuncSetAttribute((const void*)k_router_score_row<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess &&
         hipFuncSetAttribute((const void*)k_router_score_row<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess &&
         hipFuncSetAttribute((const void*)k_router_score_row<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess;
@@ -561,9 +569,17 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
         const uint32_t waves = ((N + 16u * RS16_NB - 1u) / (16u * RS16_NB)) * ((M + 15u) / 16u);
         k_router_score_mfma16<<<(waves + 3u) / 4u, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else if (use32) {
+        /* two waves per SIMD when the tiles fill both slots of every SIMD a whole number of times (DeepSeek-V3
+         * router at 8192 tokens 360 -> 330 us, at 16384 655 -> 591; at 4096, one tile per SIMD, it would leave half
+         * the SIMDs idle: 174 -> 298) */
+        if (t32 % (2u * n_simd) == 0u) {
+            const uint32_t g = ((N + 63) / 64) * ((M + 127) / 128);
+            k_router_score_mfma<8u, 2u><<<g, 512, RSM_LDS8, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+            return 0;
+        }
         const uint32_t lds = RSM_LDS;
         const uint32_t g = ((N + 63) / 64) * ((M + 63) / 64);
-        k_router_score_mfma<<<g, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        k_router_score_mfma<4u, 3u><<<g, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else if ((uint64_t)M * N >= (1u << 19)) {
         if ((uint64_t)((N + 63) / 64) * ((M + 63) / 64) < 2u * n_cu) { /* fewer than two 64-row workgroups per CU */
             dim3 g((N + 63) / 64, (M + 31) / 32);

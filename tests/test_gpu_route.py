@@ -108,7 +108,8 @@ def test_route_and_align_match_oracle(moe, oracle, E, k, T, flags, ng, tg, tail)
                                    (17, 100, 512), (1, 128, 4096), (8, 128, 4096),
                                    (6, 40, 768), (64, 256, 7168), (1, 384, 7168), (700, 1000, 264),
                                    (700, 1000, 256), (520, 520, 128), (1030, 300, 64), (1500, 288, 1024),
-                                   (413, 331, 192), (1024, 1024, 128), (2048, 512, 192)])
+                                   (413, 331, 192), (1024, 1024, 128), (2048, 512, 192),
+                                       (2048, 1024, 192), (4096, 512, 320)])  # the last two: two 32 x 32 tiles per SIMD
 def test_router_score_bit_exact(moe, oracle, M, N, K):
     print(f"[case] score {M}x{N}x{K}", flush=True)
     if (M, N, K) == (6, 40, 768):
