@@ -99,6 +99,39 @@ def test_route_and_align_match_oracle(moe, oracle, E, k, T, flags, ng, tg, tail)
     assert np.array_equal(dev[3][:rows].view(np.uint32), al[4][:rows].view(np.uint32))
 
 
+@pytest.mark.parametrize("flags", [1 | 8, 1 | 2 | 8, 2 | 8, 8], ids=["sigmoid", "sigmoid-renorm", "softmax-renorm", "softmax"])
+def test_route_on_logits_at_the_ends_of_the_exponential(moe, oracle, flags):
+    """Logits that drive the score transform's exponential through its special inputs: overflow and underflow
+    thresholds (88.72, -103.97) and their neighbours, the |x| >= 88 test, infinities (sigmoid only: a softmax
+    row with +inf has no defined scores), zeros of both signs, denormals. The oracle calls the C library."""
+    print(f"[case] route-extreme flags={flags}", flush=True)
+    E, k, T = 160, 8, 96
+    r = cases.rng_of(flags + 77)
+    edge = np.array([88.0, 88.5, 88.72, 88.7228, 88.73, 89.0, 100.0, 103.9, 103.97, 103.9721, 104.0, 126.0, 150.0,
+                     87.9999, 1e-45, 1e-38, 1e-20, 0.0, 3e38], np.float32)
+    for v in list(edge[:13]):
+        edge = np.append(edge, [np.nextafter(v, np.float32(0)), np.nextafter(v, np.float32(1e9))])
+    edge = np.concatenate([edge, -edge]).astype(np.float32)
+    sigmoid = bool(flags & 1)
+    if sigmoid:
+        edge = np.concatenate([edge, np.array([np.inf, -np.inf], np.float32)])
+    logit = (r.standard_normal((T, E)) * 2.0).astype(np.float32)
+    for t in range(T):
+        n = 1 + t % 12                                   # a few special values a row, at moving places
+        pos = r.choice(E, n, replace=False)
+        vals = edge[(np.arange(n) * 7 + t * 5) % len(edge)]
+        if not sigmoid:                                  # softmax subtracts the row maximum: keep x - max finite and
+            vals = -np.abs(vals)                         # let it reach the underflow side instead
+        logit[t, pos] = vals
+    kw = dict(n_group=0, topk_group=0, tail=0, route_scale=1.0)
+    got = gpu_route(moe, logit, None, E, k, T, flags, **kw)
+    want = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    ol.run(oracle.plow_oracle_exec, cases.route_inst(E, k, T, flags, False, **kw),
+           ol.table_of([want, logit, None, None]), 8)
+    assert np.array_equal(got["eid"], want["eid"])
+    assert np.array_equal(got["gate"].view(np.uint32), want["gate"].view(np.uint32))
+
+
 # K a multiple of 64 and 2^17 outputs or more: the matrix-unit forms. 16 x 32 tiles with 4, 2, 1, 16 and 3
 # chunks (the fifth is ragged in both directions); the last two fill the SIMDs evenly with 32 x 32 tiles and
 # take that form (2 and 3 chunks)
