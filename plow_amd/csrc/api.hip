@@ -22,7 +22,7 @@
  * plow_moe_exec_noalloc carves a smaller one out of the library's static device array. Nothing in a
  * workspace has to start at zero: every word a kernel reads was written earlier in the same call. */
 #define WS_MAX_E 1056u
-#define WS_MAX_SLOTS (1u << 18)
+#define WS_MAX_SLOTS (1u << 20)
 
 struct Workspace {
     uint32_t max_e, max_slots, max_chunks;

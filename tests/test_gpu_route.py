@@ -99,6 +99,28 @@ def test_route_and_align_match_oracle(moe, oracle, E, k, T, flags, ng, tg, tail)
     assert np.array_equal(dev[3][:rows].view(np.uint32), al[4][:rows].view(np.uint32))
 
 
+@pytest.mark.parametrize("T,E,k", [(32768, 257, 9), (50000, 64, 8), (2049, 1056, 1), (116508, 9, 9)])
+def test_align_of_long_tables(moe, oracle, T, E, k):
+    """The align alone on tables of 2^18 slots and more (the multi-workgroup form with hundreds of slot chunks),
+    with a skewed expert popularity, unused slots and one expert that nobody picks."""
+    print(f"[case] align-long T={T} E={E} k={k}", flush=True)
+    r = cases.rng_of(T + E)
+    table = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    pop = 1.0 / (1.0 + np.arange(E)) ** 0.7
+    pop[E // 2] = 0.0
+    table["eid"] = r.choice(E, size=T * k, p=pop / pop.sum()).astype(np.uint32)
+    table["eid"][r.integers(0, T * k, size=T * k // 50)] = 0xFFFFFFFF
+    table["gate"] = r.random(T * k, dtype=np.float32)
+    dev = gpu_align(moe, table, T, E, k)
+    al = cases.align_arrays(table, T, E, k)
+    ol.run(oracle.plow_oracle_exec, cases.align_inst(T, E, k), ol.table_of(al), 1)
+    rows = int(al[0][3 * E]) * abi.MPF_BM
+    assert np.array_equal(dev[0], al[0])
+    assert np.array_equal(dev[1][:rows], al[2][:rows]) and np.array_equal(dev[2][:rows], al[3][:rows])
+    assert np.array_equal(dev[3][:rows].view(np.uint32), al[4][:rows].view(np.uint32))
+    assert np.all(dev[1][rows:] == 7)
+
+
 @pytest.mark.parametrize("flags", [1 | 8, 1 | 2 | 8, 2 | 8, 8], ids=["sigmoid", "sigmoid-renorm", "softmax-renorm", "softmax"])
 def test_route_on_logits_at_the_ends_of_the_exponential(moe, oracle, flags):
     """Logits that drive the score transform's exponential through its special inputs: overflow and underflow
