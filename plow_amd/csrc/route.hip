@@ -9,6 +9,7 @@
  */
 #include <stdlib.h>
 #include <string.h>
+#include <type_traits>
 #include "common.h"
 #include "kernels.h"
 #include "pm_expf.h"
@@ -257,6 +258,169 @@ __global__ __launch_bounds__(NWV * 64u) void k_router_score_mfma(float* __restri
             widen(nxt, 2, 4);
         }
         st = stn;
+    }
+#undef RSM_MFMA
+#undef RSM_FENCE
+    /* acc[r] = out[m0 + 8 * (r / 4) + 4 * (lane / 32) + r % 4][n0 + lane % 32] */
+    const uint32_t n = n0 + (lane & 31u);
+#pragma unroll
+    for (uint32_t r = 0; r < 16u; r++) {
+        const uint32_t m = m0 + 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
+        if (m < M && n < N) out[(size_t)m * N + n] = acc[r];
+    }
+}
+
+/* The 32 x 32 form as it runs by default. Two facts of the part shape it. (1) The f32 matrix instructions
+ * execute on the vector unit's own multiply-add lanes (the f32 matrix peak equals the vector f32 peak): vector
+ * instructions between two of them do not hide behind them, they add (measured: the eight byte permutes that
+ * widened a piece's bf16 operands cost 9 cycles each, 29 of 173 us at T = 4096, E = 256, K = 7168). So operands
+ * are widened by the LDS read itself: ds_read_u16_d16_hi puts a bf16 into the high half of a register whose
+ * low half is zero, which is the f32; the per-lane addresses of the eight pieces are computed once (the XOR
+ * swizzle makes them lane-dependent) and the stage and element are immediate offsets, so the loop issues no
+ * vector instruction at all next to its matrix instructions except a chunk's four load addresses.
+ * (2) The operand rows of a workgroup's four tiles (64 tokens x 64 experts) are loaded once: a stage holds
+ * 64 + 64 rows (16 KB), each wave loads a quarter of it and the four waves meet at one barrier per chunk,
+ * after a wave's last LDS read of chunk c has landed and its own loads of chunk c + 1 have: behind the barrier
+ * chunk c + 1 is complete and chunk c's stage is free for chunk c + 3. 48 KB of LDS: a CU takes up to three
+ * workgroups when the grid has them. */
+struct RssStage {
+    uint8_t x[64u * 128u];
+    uint8_t w[64u * 128u];
+};
+static_assert(sizeof(RssStage) == 16384u, "the stage size is an immediate of the LDS reads below");
+/* eight 2-byte reads: elements 0, 2, 4, 6 of the lane's half of a 16-byte piece (the lane's address already
+ * holds its even / odd byte), of its token row and of its expert row; stage STG of the ring */
+template <uint32_t STG>
+__device__ __forceinline__ void rss_read(float (&a)[4], float (&b)[4], uint32_t ax, uint32_t aw) {
+    asm volatile("ds_read_u16_d16_hi %0, %8 offset:%10\n\t"
+                 "ds_read_u16_d16_hi %4, %9 offset:%10\n\t"
+                 "ds_read_u16_d16_hi %1, %8 offset:%11\n\t"
+                 "ds_read_u16_d16_hi %5, %9 offset:%11\n\t"
+                 "ds_read_u16_d16_hi %2, %8 offset:%12\n\t"
+                 "ds_read_u16_d16_hi %6, %9 offset:%12\n\t"
+                 "ds_read_u16_d16_hi %3, %8 offset:%13\n\t"
+                 "ds_read_u16_d16_hi %7, %9 offset:%13"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3])
+                 : "v"(ax), "v"(aw), "n"(STG * 16384u), "n"(STG * 16384u + 4u), "n"(STG * 16384u + 8u), "n"(STG * 16384u + 12u)
+                 : "memory");
+}
+__device__ __forceinline__ void rss_wait_reads(float (&a)[4], float (&b)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+}
+__global__ __launch_bounds__(256) void k_router_score_mfma_shared(float* __restrict__ out, const bf16_t* __restrict__ x,
+                                                                  const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
+                                                                  uint32_t K) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t rss_raw[];
+    constexpr uint32_t ST = RSM_STAGES;
+    static_assert(ST == 3u, "the chunk loop below is written out for three stages");
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    RssStage* const ring = (RssStage*)rss_raw;
+    const uint32_t G = gridDim.x, gx = (N + 63u) / 64u;
+    const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const uint32_t M0 = (wg / gx) * 64u, N0 = (wg % gx) * 64u;          /* the workgroup's block */
+    const uint32_t m0 = M0 + (wv >> 1) * 32u, n0 = N0 + (wv & 1u) * 32u; /* this wave's tile */
+    const uint32_t NC = K / 64u;
+    /* this wave's share of a stage: rows 16 wv .. 16 wv + 15 of both operands, two loads of eight rows each;
+     * rows past the end of a matrix read its last row and are never stored. No wave leaves early: every wave
+     * loads for the others and takes part in the barriers. A load's address is a base the whole wave shares
+     * (the block's first row, advanced by the chunk) plus a 32-bit lane offset. */
+    const uint32_t lr = lane >> 3, lp = lane & 7u;
+    const uint8_t* const xblk = (const uint8_t*)(x + (size_t)M0 * K);
+    const uint8_t* const wblk = (const uint8_t*)(w + (size_t)N0 * K);
+    uint32_t xoff[2], woff[2];
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; j++) {
+        const uint32_t row = 16u * wv + 8u * j + lr;
+        const uint32_t mr = M0 + row < M ? row : M - 1u - M0, nr = N0 + row < N ? row : N - 1u - N0;
+        xoff[j] = mr * K * 2u + ((lp ^ ((row >> 1) & 7u)) << 4);
+        woff[j] = nr * K * 2u + ((lp ^ ((row >> 1) & 7u)) << 4);
+    }
+    auto issue = [&](uint32_t c, uint32_t stage) {
+        RssStage* s = &ring[stage];
+        uint64_t xcb = (uint64_t)(uintptr_t)(xblk + (size_t)c * 128u), wcb = (uint64_t)(uintptr_t)(wblk + (size_t)c * 128u);
+        asm volatile("" : "+s"(xcb), "+s"(wcb));
+        const uint8_t* const xc = (const uint8_t*)(uintptr_t)xcb;
+        const uint8_t* const wc = (const uint8_t*)(uintptr_t)wcb;
+        /* the chunk's base addresses and the lane offsets are made opaque here so that an address stays "scalar
+         * base + 32-bit lane offset" (two scalar additions per chunk) instead of four 64-bit per-lane pointers
+         * advanced on the vector unit */
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; j++) {
+            uint32_t o = xoff[j];
+            asm volatile("" : "+v"(o));
+            __builtin_amdgcn_global_load_lds((const void*)(xc + o), (rsm_lds_void*)&s->x[(16u * wv + 8u * j) * 128u], 16, 0, 0);
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; j++) {
+            uint32_t o = woff[j];
+            asm volatile("" : "+v"(o));
+            __builtin_amdgcn_global_load_lds((const void*)(wc + o), (rsm_lds_void*)&s->w[(16u * wv + 8u * j) * 128u], 16, 0, 0);
+        }
+    };
+    /* operand reads: lanes 0..31 take the even k of a pair, lanes 32..63 the odd k; row lane & 31 of the wave's
+     * token rows and of its expert rows (32 is a multiple of 16: the swizzle of row 32 h + r is that of r) */
+    const uint32_t orow = lane & 31u, osw = (orow >> 1) & 7u;
+    const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)&ring[0];
+    const uint32_t xrow = ring0 + ((wv >> 1) * 32u + orow) * 128u + (lane >> 5) * 2u;
+    const uint32_t wrow = ring0 + 64u * 128u + ((wv & 1u) * 32u + orow) * 128u + (lane >> 5) * 2u;
+    uint32_t ax[8], aw[8];
+#pragma unroll
+    for (uint32_t pc = 0; pc < 8u; pc++) ax[pc] = xrow + ((pc ^ osw) << 4), aw[pc] = wrow + ((pc ^ osw) << 4);
+    v16f acc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+    float af[2][4], bf[2][4]; /* the low halves stay zero: the reads write high halves only */
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int d = 0; d < 4; d++) af[h][d] = 0.0f, bf[h][d] = 0.0f;
+    issue(0u, 0u);
+    if (NC > 1u) issue(1u, 1u);
+    if (NC > 2u) issue(2u, 2u);
+    if (NC > 2u) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if (NC > 1u) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_barrier" ::: "memory"); /* chunk 0 is complete */
+    rss_read<0u>(af[0], bf[0], ax[0], aw[0]);
+    rss_wait_reads(af[0], bf[0]);
+#define RSM_MFMA(d) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][d], bf[cur][d], acc, 0, 0, 0)
+#define RSM_FENCE() __builtin_amdgcn_sched_barrier(0)
+    /* one chunk in stage STG (a constant: the reads' offsets are immediates) */
+    auto chunk = [&](auto stg_, uint32_t c) {
+        constexpr uint32_t STG = decltype(stg_)::value, STN = (STG + 1u) % ST;
+#pragma unroll
+        for (uint32_t pc = 0; pc < 8u; pc++) {
+            const uint32_t cur = pc & 1u, nxt = cur ^ 1u;
+            RSM_FENCE();
+            RSM_MFMA(0);
+            RSM_FENCE();
+            if (pc == 7u) {
+                /* this wave's reads of chunk c have all landed (piece 7 was waited for a piece ago); once its loads
+                 * of chunk c + 1 have landed too, the barrier says both of every wave */
+                if (c + 2u < NC) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                asm volatile("s_barrier" ::: "memory");
+                rss_read<STN>(af[nxt], bf[nxt], ax[0], aw[0]); /* past the last chunk: stale bytes, never used */
+            } else {
+                rss_read<STG>(af[nxt], bf[nxt], ax[(pc + 1u) & 7u], aw[(pc + 1u) & 7u]);
+            }
+            RSM_FENCE();
+            RSM_MFMA(1);
+            RSM_FENCE();
+            if (pc == 7u && c + ST < NC) issue(c + ST, STG); /* into the stage chunk c has left */
+            RSM_FENCE();
+            RSM_MFMA(2);
+            RSM_FENCE();
+            RSM_MFMA(3);
+            RSM_FENCE();
+            rss_wait_reads(af[nxt], bf[nxt]);
+        }
+    };
+    for (uint32_t c = 0; c < NC; c += 3u) {
+        chunk(std::integral_constant<uint32_t, 0u>{}, c);
+        if (c + 1u < NC) chunk(std::integral_constant<uint32_t, 1u>{}, c + 1u);
+        if (c + 2u < NC) chunk(std::integral_constant<uint32_t, 2u>{}, c + 2u);
     }
 #undef RSM_MFMA
 #undef RSM_FENCE
@@ -536,6 +700,7 @@ __global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(
 #define RS16_LDS (4u * RSM_STAGES * (uint32_t)sizeof(Rs16Stage))
 #define RSM_LDS (4u * RSM_STAGES * (uint32_t)sizeof(RsmStage))
 #define RSM_LDS8 (8u * 2u * (uint32_t)sizeof(RsmStage))
+#define RSS_LDS (RSM_STAGES * (uint32_t)sizeof(RssStage))
 
 /* dynamic-LDS limits of the score kernels, once per device (plow_moe_device_setup) */
 static bool rf_setup();
@@ -572,6 +737,11 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
         /* two waves per SIMD when the tiles fill both slots of every SIMD a whole number of times (DeepSeek-V3
          * router at 8192 tokens 360 -> 330 us, at 16384 655 -> 591; at 4096, one tile per SIMD, it would leave half
          * the SIMDs idle: 174 -> 298) */
+        if (!tune.score_private) {
+            const uint32_t g = ((N + 63) / 64) * ((M + 63) / 64);
+            k_router_score_mfma_shared<<<g, 256, RSS_LDS, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+            return 0;
+        }
         if (t32 % (2u * n_simd) == 0u) {
             const uint32_t g = ((N + 63) / 64) * ((M + 127) / 128);
             k_router_score_mfma<8u, 2u><<<g, 512, RSM_LDS8, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
