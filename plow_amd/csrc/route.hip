@@ -697,10 +697,163 @@ __global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(
     router_score_row_body<TOK>(out, x, w, M, N, K, blockIdx.x, blockIdx.y, rsr_raw);
 }
 
+/* The 16 x 32 form as it runs by default: like k_router_score_mfma_shared, operands widened by the LDS read
+ * (no vector instruction next to the matrix instructions) and operand rows shared by the workgroup. Four waves
+ * stacked over 64 tokens share one block of 32 experts: a stage holds 64 + 32 rows (12 KB), a wave loads a
+ * quarter of it (16 token rows, 8 expert rows). A piece is only four short matrix instructions, so the reads run
+ * two pieces ahead into four sets of operand registers (set = piece % 4: the same in every chunk). The barrier of
+ * chunk c sits in its seventh piece, before the first read of chunk c + 1: every wave has then landed its loads
+ * of chunk c + 1 and its reads of chunk c - 1, whose stage takes chunk c + 3 (four stages, 48 KB). */
+#define RS16S_STAGES 4u
+struct Rs16sStage {
+    uint8_t x[64u * 128u];
+    uint8_t w[32u * 128u];
+};
+static_assert(sizeof(Rs16sStage) == 12288u, "the stage size is an immediate of the LDS reads below");
+/* six 2-byte reads of a piece: k = ks and 4 + ks (the lane's address holds 2 ks) of the lane's token row and of
+ * its expert row in both 16-row blocks */
+template <uint32_t STG>
+__device__ __forceinline__ void rs16s_read(float (&a)[2], float (&b)[2][2], uint32_t ax, uint32_t aw) {
+    asm volatile("ds_read_u16_d16_hi %0, %6 offset:%8\n\t"
+                 "ds_read_u16_d16_hi %2, %7 offset:%8\n\t"
+                 "ds_read_u16_d16_hi %4, %7 offset:%10\n\t"
+                 "ds_read_u16_d16_hi %1, %6 offset:%9\n\t"
+                 "ds_read_u16_d16_hi %3, %7 offset:%9\n\t"
+                 "ds_read_u16_d16_hi %5, %7 offset:%11"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[1][0]), "+v"(b[1][1])
+                 : "v"(ax), "v"(aw), "n"(STG * 12288u), "n"(STG * 12288u + 8u), "n"(STG * 12288u + 2048u), "n"(STG * 12288u + 2056u)
+                 : "memory");
+}
+/* all but the newest piece's six reads have landed (LDS answers in order) */
+__device__ __forceinline__ void rs16s_wait_older(float (&a)[2], float (&b)[2][2]) {
+    asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[1][0]), "+v"(b[1][1]));
+}
+__global__ __launch_bounds__(256) void k_router_score_mfma16_shared(float* __restrict__ out, const bf16_t* __restrict__ x,
+                                                                    const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
+                                                                    uint32_t K) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t rs16s_raw[];
+    constexpr uint32_t ST = RS16S_STAGES, NLD = 3u; /* direct loads per wave and chunk */
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    Rs16sStage* const ring = (Rs16sStage*)rs16s_raw;
+    const uint32_t G = gridDim.x, gx = (N + 31u) / 32u;
+    const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const uint32_t M0 = (wg / gx) * 64u, N0 = (wg % gx) * 32u; /* the workgroup's block */
+    const uint32_t m0 = M0 + 16u * wv, n0 = N0;                /* this wave's tile */
+    const uint32_t NC = K / 64u;
+    /* this wave's share of a stage: token rows 16 wv .. 16 wv + 15 (two loads) and expert rows 8 wv .. 8 wv + 7;
+     * rows past the end of a matrix read its last row and are never stored; no wave leaves early */
+    const uint32_t lr = lane >> 3, lp = lane & 7u;
+    const uint8_t* const xblk = (const uint8_t*)(x + (size_t)M0 * K);
+    const uint8_t* const wblk = (const uint8_t*)(w + (size_t)N0 * K);
+    uint32_t xoff[2], woff;
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; j++) {
+        const uint32_t row = 16u * wv + 8u * j + lr;
+        const uint32_t mr = M0 + row < M ? row : M - 1u - M0;
+        xoff[j] = mr * K * 2u + ((lp ^ ((row >> 1) & 7u)) << 4);
+    }
+    {
+        const uint32_t row = 8u * wv + lr;
+        const uint32_t nr = N0 + row < N ? row : N - 1u - N0;
+        woff = nr * K * 2u + ((lp ^ ((row >> 1) & 7u)) << 4);
+    }
+    auto issue = [&](uint32_t c, uint32_t stage) {
+        Rs16sStage* s = &ring[stage];
+        /* opaque scalar bases and lane offsets: an address stays "scalar base + 32-bit lane offset" */
+        uint64_t xcb = (uint64_t)(uintptr_t)(xblk + (size_t)c * 128u), wcb = (uint64_t)(uintptr_t)(wblk + (size_t)c * 128u);
+        asm volatile("" : "+s"(xcb), "+s"(wcb));
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; j++) {
+            uint32_t o = xoff[j];
+            asm volatile("" : "+v"(o));
+            __builtin_amdgcn_global_load_lds((const void*)((const uint8_t*)(uintptr_t)xcb + o), (rsm_lds_void*)&s->x[(16u * wv + 8u * j) * 128u], 16, 0, 0);
+        }
+        uint32_t o = woff;
+        asm volatile("" : "+v"(o));
+        __builtin_amdgcn_global_load_lds((const void*)((const uint8_t*)(uintptr_t)wcb + o), (rsm_lds_void*)&s->w[(8u * wv) * 128u], 16, 0, 0);
+    };
+    /* operand reads: lane = (row lane & 15, k lane >> 4); 16 is a multiple of 16: the swizzle of row 16 h + r is that of r */
+    const uint32_t orow = lane & 15u, ks = lane >> 4, osw = (orow >> 1) & 7u;
+    const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)&ring[0];
+    const uint32_t xrow = ring0 + (16u * wv + orow) * 128u + 2u * ks;
+    const uint32_t wrow = ring0 + 64u * 128u + orow * 128u + 2u * ks;
+    uint32_t ax[8], aw[8];
+#pragma unroll
+    for (uint32_t pc = 0; pc < 8u; pc++) ax[pc] = xrow + ((pc ^ osw) << 4), aw[pc] = wrow + ((pc ^ osw) << 4);
+    v4f acc[2];
+    acc[0] = (v4f){0.0f, 0.0f, 0.0f, 0.0f}, acc[1] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    float af[4][2], bf[4][2][2]; /* [set][k half] and [set][block][k half]; the low halves stay zero */
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) af[q][h] = 0.0f, bf[q][0][h] = 0.0f, bf[q][1][h] = 0.0f;
+    issue(0u, 0u);
+    if (NC > 1u) issue(1u, 1u);
+    if (NC > 2u) issue(2u, 2u);
+    if (NC > 2u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
+    else if (NC > 1u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_barrier" ::: "memory"); /* chunk 0 is complete */
+    rs16s_read<0u>(af[0], bf[0], ax[0], aw[0]);
+    rs16s_read<0u>(af[1], bf[1], ax[1], aw[1]);
+    rs16s_wait_older(af[0], bf[0]);
+#define RS16_FENCE() __builtin_amdgcn_sched_barrier(0)
+    auto chunk = [&](auto stg_, uint32_t c) {
+        constexpr uint32_t STG = decltype(stg_)::value, STN = (STG + 1u) % ST, STF = (STG + 3u) % ST;
+#pragma unroll
+        for (uint32_t pc = 0; pc < 8u; pc++) {
+            const uint32_t cur = pc & 3u, n1 = (pc + 1u) & 3u, n2 = (pc + 2u) & 3u;
+            RS16_FENCE();
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][0], bf[cur][0][0], acc[0], 0, 0, 0);
+            RS16_FENCE();
+            if (pc == 6u) {
+                /* this wave's loads of chunk c + 1 have landed and so have its reads of chunk c - 1 (its last piece was
+                 * waited for seven pieces ago): behind the barrier that holds for every wave */
+                if (c + 2u < NC) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                asm volatile("s_barrier" ::: "memory");
+            }
+            /* piece p + 2 into the set piece p - 2 used; past the last chunk: stale bytes, never used */
+            if (pc < 6u) rs16s_read<STG>(af[n2], bf[n2], ax[(pc + 2u) & 7u], aw[(pc + 2u) & 7u]);
+            else rs16s_read<STN>(af[n2], bf[n2], ax[(pc + 2u) & 7u], aw[(pc + 2u) & 7u]);
+            RS16_FENCE();
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][0], bf[cur][1][0], acc[1], 0, 0, 0);
+            RS16_FENCE();
+            if (pc == 6u && c + 3u < NC) issue(c + 3u, STF); /* into the stage chunk c - 1 has left */
+            RS16_FENCE();
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][1], bf[cur][0][1], acc[0], 0, 0, 0);
+            RS16_FENCE();
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][1], bf[cur][1][1], acc[1], 0, 0, 0);
+            RS16_FENCE();
+            rs16s_wait_older(af[n1], bf[n1]); /* piece p + 1 */
+        }
+    };
+    for (uint32_t c = 0; c < NC; c += 4u) {
+        chunk(std::integral_constant<uint32_t, 0u>{}, c);
+        if (c + 1u < NC) chunk(std::integral_constant<uint32_t, 1u>{}, c + 1u);
+        if (c + 2u < NC) chunk(std::integral_constant<uint32_t, 2u>{}, c + 2u);
+        if (c + 3u < NC) chunk(std::integral_constant<uint32_t, 3u>{}, c + 3u);
+    }
+#undef RS16_FENCE
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stale reads of the last two pieces */
+    /* acc[b][r] = out[m0 + 4 * (lane / 16) + r][n0 + 16 b + lane % 16] */
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+        const uint32_t n = n0 + 16u * (uint32_t)b + (lane & 15u);
+#pragma unroll
+        for (uint32_t r = 0; r < 4u; r++) {
+            const uint32_t m = m0 + 4u * (lane >> 4) + r;
+            if (m < M && n < N) out[(size_t)m * N + n] = acc[b][r];
+        }
+    }
+}
+
 #define RS16_LDS (4u * RSM_STAGES * (uint32_t)sizeof(Rs16Stage))
 #define RSM_LDS (4u * RSM_STAGES * (uint32_t)sizeof(RsmStage))
 #define RSM_LDS8 (8u * 2u * (uint32_t)sizeof(RsmStage))
 #define RSS_LDS (RSM_STAGES * (uint32_t)sizeof(RssStage))
+#define RS16S_LDS (RS16S_STAGES * (uint32_t)sizeof(Rs16sStage))
 
 /* dynamic-LDS limits of the score kernels, once per device (plow_moe_device_setup) */
 static bool rf_setup();
@@ -729,7 +882,10 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
     const bool mfma_ok = K % 64u == 0u && !tune.score_valu;
     const bool use32 = mfma_ok && outputs >= (1u << 18) && (force32 ? outputs >= force32 : (t32 % n_simd == 0u || t32 >= 4u * n_simd));
     const bool use16 = mfma_ok && !use32 && outputs >= (1u << 17);
-    if (use16) {
+    if (use16 && !tune.score_private) {
+        const uint32_t g = ((N + 31) / 32) * ((M + 63) / 64);
+        k_router_score_mfma16_shared<<<g, 256, RS16S_LDS, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+    } else if (use16) {
         const uint32_t lds = RS16_LDS;
         const uint32_t waves = ((N + 16u * RS16_NB - 1u) / (16u * RS16_NB)) * ((M + 15u) / 16u);
         k_router_score_mfma16<<<(waves + 3u) / 4u, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
