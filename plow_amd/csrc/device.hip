@@ -27,9 +27,6 @@ const PlowMoeTuning& plow_moe_tuning() {
         t.a16_regs = is("PLOW_MOE_A16_KERNEL", "regs");
         t.score_tile8 = is("PLOW_MOE_SCORE_KERNEL", "tile8");
         t.score_valu = is("PLOW_MOE_SCORE_KERNEL", "valu");
-        t.score_private = is("PLOW_MOE_SCORE_KERNEL", "private");
-        const char* f = getenv("PLOW_MOE_SCORE_MFMA32_FROM");
-        t.score_mfma32_from = f ? strtoull(f, nullptr, 10) : 0ull;
         t.a16_tiled = !is("PLOW_MOE_A16_TILED", "0");
         t.a16_gemv = !is("PLOW_MOE_A16_GEMV", "0");
     });

@@ -114,469 +114,7 @@ __global__ __launch_bounds__(256) void k_router_score_tile(float* __restrict__ o
         }
 }
 
-/* Large problems with K a multiple of 64: the same sums on the matrix unit. v_mfma_f32_32x32x2_f32
- * adds a[i][k] * b[k][j], then a[i][k + 1] * b[k + 1][j], to its f32 accumulator, each step rounded
- * to nearest even and denormals kept (measured against the fmaf chain, bit for bit, normal and
- * denormal ranges), so a chain of K / 2 of them IS the reference's sum in the reference's order, at
- * twice the rate of the vector unit and without an operand broadcast through LDS.
- * One wave per workgroup computes 32 tokens x 32 experts. Operand rows (bf16, 64 k = one 128-byte line
- * per row and chunk) come in by direct global -> LDS loads in the coalesced shape into a wave-private
- * ring of three chunks, two chunks ahead; no barrier anywhere. A lane reads 16 bytes (8 k) of its
- * token row and of its expert row per piece; lanes 0..31 feed the even k of a pair to the instruction
- * and lanes 32..63 the odd k (one byte permute each widens bf16 to f32). The next piece's LDS reads
- * are issued before the four matrix instructions of this piece and waited for after them. LDS piece p
- * of row r holds global piece p ^ ((r >> 1) & 7): 16 consecutive rows of a piece cover all 64 banks. */
-#define RSM_STAGES 3
-struct RsmStage {
-    uint8_t x[32u * 128u];
-    uint8_t w[32u * 128u];
-};
 typedef __attribute__((address_space(3))) void rsm_lds_void;
-/* NWV waves per workgroup, rings of ST chunks: 4 x 3 (one wave per SIMD, two chunks ahead), or 8 x 2 (two waves
- * per SIMD, one chunk ahead: a wave's matrix instructions fill the other's issue gaps) when there are tiles
- * enough for two per SIMD. */
-template <uint32_t NWV, uint32_t ST>
-__global__ __launch_bounds__(NWV * 64u) void k_router_score_mfma(float* __restrict__ out, const bf16_t* __restrict__ x,
-                                                                 const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
-                                                                 uint32_t K) {
-    static_assert((NWV == 4u && ST == 3u) || (NWV == 8u && ST == 2u), "4 waves x 3 chunks or 8 waves x 2 chunks");
-    /* independent waves (a 2 x 2 or 4 x 2 block of tiles): 96 / 128 KB of LDS makes it one workgroup per CU,
-     * which puts exactly one (two) waves on every SIMD */
-    extern __shared__ __attribute__((aligned(16))) uint8_t rsm_raw[];
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    RsmStage* const ring = (RsmStage*)rsm_raw + wv * ST;
-    /* Workgroup b runs on XCD b % 8 and each XCD has its own L2: the logical index gives one XCD
-     * consecutive workgroups, which share their token rows (the expert-tile index runs fastest) */
-    const uint32_t G = gridDim.x, gx = (N + 63u) / 64u;
-    const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
-    const uint32_t m0 = ((wg / gx) * (NWV / 2u) + (wv >> 1)) * 32u, n0 = ((wg % gx) * 2u + (wv & 1u)) * 32u;
-    if (m0 >= M || n0 >= N) return; /* whole wave; there is no barrier below */
-    const uint32_t NC = K / 64u;
-    /* load j covers rows 8j .. 8j + 7: lane -> (row lane >> 3, LDS piece lane & 7); rows past the end
-     * of the matrix read its last row and are never stored */
-    const uint32_t lr = lane >> 3, lp = lane & 7u;
-    const uint8_t *xsrc[4], *wsrc[4];
-#pragma unroll
-    for (uint32_t j = 0; j < 4u; j++) {
-        const uint32_t row = 8u * j + lr;
-        const uint32_t mr = m0 + row < M ? m0 + row : M - 1u, nr = n0 + row < N ? n0 + row : N - 1u;
-        xsrc[j] = (const uint8_t*)(x + (size_t)mr * K) + ((lp ^ ((row >> 1) & 7u)) << 4);
-        wsrc[j] = (const uint8_t*)(w + (size_t)nr * K) + ((lp ^ ((row >> 1) & 7u)) << 4);
-    }
-    auto issue = [&](uint32_t c) {
-        RsmStage* s = &ring[c % ST];
-#pragma unroll
-        for (uint32_t j = 0; j < 4u; j++)
-            __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
-#pragma unroll
-        for (uint32_t j = 0; j < 4u; j++)
-            __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
-    };
-    /* operand reads: row lane & 31 of the token rows (A) and of the expert rows (B) */
-    const uint32_t orow = lane & 31u, osw = (orow >> 1) & 7u;
-    const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)&ring[0];
-    const uint32_t obase = ring0 + orow * 128u;
-    const uint32_t sel = lane < 32u ? 0x01000c0cu : 0x03020c0cu; /* low / high bf16 of a dword -> f32 bits */
-    v16f acc;
-#pragma unroll
-    for (int i = 0; i < 16; i++) acc[i] = 0.0f;
-    /* Per piece: issue the next piece's LDS reads, run this piece's four matrix instructions, wait for
-     * the reads, widen them into the other half of the operand registers. An instruction's operands
-     * are never overwritten while it may still be reading them (the vector unit would wait for it), and
-     * the widening runs under the last matrix instruction of the piece. */
-    v4i xa, wb;
-    float af[2][4], bf[2][4];
-    auto read_piece = [&](uint32_t stage, uint32_t pc) {
-        const uint32_t addr = obase + stage * (uint32_t)sizeof(RsmStage) + ((pc ^ osw) << 4);
-        /* early-clobber outputs: the first read's destination must not be the register the second takes its
-         * address from (the data may land before the second instruction issues) */
-        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:4096" : "=&v"(xa), "=&v"(wb) : "v"(addr) : "memory");
-    };
-    auto widen = [&](uint32_t h, int d0, int d1) {
-        if (d0 == 0) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa), "+v"(wb));
-#pragma unroll
-        for (int d = d0; d < d1; d++) {
-            af[h][d] = __uint_as_float(__builtin_amdgcn_perm((uint32_t)xa[d], (uint32_t)xa[d], sel));
-            bf[h][d] = __uint_as_float(__builtin_amdgcn_perm((uint32_t)wb[d], (uint32_t)wb[d], sel));
-        }
-    };
-    issue(0u);
-    if (NC > 1u) issue(1u);
-    if (ST > 2u && NC > 2u) issue(2u);
-    if (ST > 2u && NC > 2u) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else if (NC > 1u) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    read_piece(0u, 0u);
-    widen(0u, 0, 4);
-    uint32_t st = 0;
-#define RSM_MFMA(d) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][d], bf[cur][d], acc, 0, 0, 0)
-#define RSM_FENCE() __builtin_amdgcn_sched_barrier(0)
-    for (uint32_t c = 0; c < NC; c++) {
-        const uint32_t stn = st == ST - 1u ? 0u : st + 1u;
-#pragma unroll
-        for (uint32_t pc = 0; pc < 8u; pc++) {
-            const uint32_t cur = pc & 1u, nxt = cur ^ 1u;
-            /* everything that is not a matrix instruction is issued behind one, so that the matrix unit
-             * is busy while the wave issues it */
-            RSM_FENCE();
-            RSM_MFMA(0);
-            RSM_FENCE();
-            if (pc == 7u) {
-                /* every piece of chunk c has been read: chunk c + 1 must have landed before its first
-                 * piece is read (with three stages chunk c + 2's loads may stay outstanding), and chunk c's
-                 * stage takes chunk c + ST */
-                if (ST > 2u && c + 2u < NC) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                read_piece(stn, 0u); /* past the last chunk: stale bytes, never used */
-            } else {
-                read_piece(st, pc + 1u);
-            }
-            RSM_FENCE();
-            RSM_MFMA(1);
-            RSM_FENCE();
-            if (pc == 7u && c + ST < NC) {
-                RsmStage* s = &ring[(c + ST) % ST];
-#pragma unroll
-                for (uint32_t j = 0; j < 4u; j++)
-                    __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)(c + ST) * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
-            }
-            RSM_FENCE();
-            RSM_MFMA(2);
-            RSM_FENCE();
-            if (pc == 7u && c + ST < NC) {
-                RsmStage* s = &ring[(c + ST) % ST];
-#pragma unroll
-                for (uint32_t j = 0; j < 4u; j++)
-                    __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)(c + ST) * 128u), (rsm_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
-            }
-            RSM_FENCE();
-            widen(nxt, 0, 2);
-            RSM_FENCE();
-            RSM_MFMA(3);
-            RSM_FENCE();
-            widen(nxt, 2, 4);
-        }
-        st = stn;
-    }
-#undef RSM_MFMA
-#undef RSM_FENCE
-    /* acc[r] = out[m0 + 8 * (r / 4) + 4 * (lane / 32) + r % 4][n0 + lane % 32] */
-    const uint32_t n = n0 + (lane & 31u);
-#pragma unroll
-    for (uint32_t r = 0; r < 16u; r++) {
-        const uint32_t m = m0 + 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
-        if (m < M && n < N) out[(size_t)m * N + n] = acc[r];
-    }
-}
-
-/* The 32 x 32 form as it runs by default. Two facts of the part shape it. (1) The f32 matrix instructions
- * execute on the vector unit's own multiply-add lanes (the f32 matrix peak equals the vector f32 peak): vector
- * instructions between two of them do not hide behind them, they add (measured: the eight byte permutes that
- * widened a piece's bf16 operands cost 9 cycles each, 29 of 173 us at T = 4096, E = 256, K = 7168). So operands
- * are widened by the LDS read itself: ds_read_u16_d16_hi puts a bf16 into the high half of a register whose
- * low half is zero, which is the f32; the per-lane addresses of the eight pieces are computed once (the XOR
- * swizzle makes them lane-dependent) and the stage and element are immediate offsets, so the loop issues no
- * vector instruction at all next to its matrix instructions except a chunk's four load addresses.
- * (2) The operand rows of a workgroup's four tiles (64 tokens x 64 experts) are loaded once: a stage holds
- * 64 + 64 rows (16 KB), each wave loads a quarter of it and the four waves meet at one barrier per chunk,
- * after a wave's last LDS read of chunk c has landed and its own loads of chunk c + 1 have: behind the barrier
- * chunk c + 1 is complete and chunk c's stage is free for chunk c + 3. 48 KB of LDS: a CU takes up to three
- * workgroups when the grid has them. */
-struct RssStage {
-    uint8_t x[64u * 128u];
-    uint8_t w[64u * 128u];
-};
-static_assert(sizeof(RssStage) == 16384u, "the stage size is an immediate of the LDS reads below");
-/* eight 2-byte reads: elements 0, 2, 4, 6 of the lane's half of a 16-byte piece (the lane's address already
- * holds its even / odd byte), of its token row and of its expert row; stage STG of the ring */
-template <uint32_t STG>
-__device__ __forceinline__ void rss_read(float (&a)[4], float (&b)[4], uint32_t ax, uint32_t aw) {
-    asm volatile("ds_read_u16_d16_hi %0, %8 offset:%10\n\t"
-                 "ds_read_u16_d16_hi %4, %9 offset:%10\n\t"
-                 "ds_read_u16_d16_hi %1, %8 offset:%11\n\t"
-                 "ds_read_u16_d16_hi %5, %9 offset:%11\n\t"
-                 "ds_read_u16_d16_hi %2, %8 offset:%12\n\t"
-                 "ds_read_u16_d16_hi %6, %9 offset:%12\n\t"
-                 "ds_read_u16_d16_hi %3, %8 offset:%13\n\t"
-                 "ds_read_u16_d16_hi %7, %9 offset:%13"
-                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3])
-                 : "v"(ax), "v"(aw), "n"(STG * 16384u), "n"(STG * 16384u + 4u), "n"(STG * 16384u + 8u), "n"(STG * 16384u + 12u)
-                 : "memory");
-}
-__device__ __forceinline__ void rss_wait_reads(float (&a)[4], float (&b)[4]) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-}
-__global__ __launch_bounds__(256) void k_router_score_mfma_shared(float* __restrict__ out, const bf16_t* __restrict__ x,
-                                                                  const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
-                                                                  uint32_t K) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t rss_raw[];
-    constexpr uint32_t ST = RSM_STAGES;
-    static_assert(ST == 3u, "the chunk loop below is written out for three stages");
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    RssStage* const ring = (RssStage*)rss_raw;
-    const uint32_t G = gridDim.x, gx = (N + 63u) / 64u;
-    const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
-    const uint32_t M0 = (wg / gx) * 64u, N0 = (wg % gx) * 64u;          /* the workgroup's block */
-    const uint32_t m0 = M0 + (wv >> 1) * 32u, n0 = N0 + (wv & 1u) * 32u; /* this wave's tile */
-    const uint32_t NC = K / 64u;
-    /* this wave's share of a stage: rows 16 wv .. 16 wv + 15 of both operands, two loads of eight rows each;
-     * rows past the end of a matrix read its last row and are never stored. No wave leaves early: every wave
-     * loads for the others and takes part in the barriers. A load's address is a base the whole wave shares
-     * (the block's first row, advanced by the chunk) plus a 32-bit lane offset. */
-    const uint32_t lr = lane >> 3, lp = lane & 7u;
-    const uint8_t* const xblk = (const uint8_t*)(x + (size_t)M0 * K);
-    const uint8_t* const wblk = (const uint8_t*)(w + (size_t)N0 * K);
-    uint32_t xoff[2], woff[2];
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; j++) {
-        const uint32_t row = 16u * wv + 8u * j + lr;
-        const uint32_t mr = M0 + row < M ? row : M - 1u - M0, nr = N0 + row < N ? row : N - 1u - N0;
-        xoff[j] = mr * K * 2u + ((lp ^ ((row >> 1) & 7u)) << 4);
-        woff[j] = nr * K * 2u + ((lp ^ ((row >> 1) & 7u)) << 4);
-    }
-    auto issue = [&](uint32_t c, uint32_t stage) {
-        RssStage* s = &ring[stage];
-        uint64_t xcb = (uint64_t)(uintptr_t)(xblk + (size_t)c * 128u), wcb = (uint64_t)(uintptr_t)(wblk + (size_t)c * 128u);
-        asm volatile("" : "+s"(xcb), "+s"(wcb));
-        const uint8_t* const xc = (const uint8_t*)(uintptr_t)xcb;
-        const uint8_t* const wc = (const uint8_t*)(uintptr_t)wcb;
-        /* the chunk's base addresses and the lane offsets are made opaque here so that an address stays "scalar
-         * base + 32-bit lane offset" (two scalar additions per chunk) instead of four 64-bit per-lane pointers
-         * advanced on the vector unit */
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; j++) {
-            uint32_t o = xoff[j];
-            asm volatile("" : "+v"(o));
-            __builtin_amdgcn_global_load_lds((const void*)(xc + o), (rsm_lds_void*)&s->x[(16u * wv + 8u * j) * 128u], 16, 0, 0);
-        }
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; j++) {
-            uint32_t o = woff[j];
-            asm volatile("" : "+v"(o));
-            __builtin_amdgcn_global_load_lds((const void*)(wc + o), (rsm_lds_void*)&s->w[(16u * wv + 8u * j) * 128u], 16, 0, 0);
-        }
-    };
-    /* operand reads: lanes 0..31 take the even k of a pair, lanes 32..63 the odd k; row lane & 31 of the wave's
-     * token rows and of its expert rows (32 is a multiple of 16: the swizzle of row 32 h + r is that of r) */
-    const uint32_t orow = lane & 31u, osw = (orow >> 1) & 7u;
-    const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)&ring[0];
-    const uint32_t xrow = ring0 + ((wv >> 1) * 32u + orow) * 128u + (lane >> 5) * 2u;
-    const uint32_t wrow = ring0 + 64u * 128u + ((wv & 1u) * 32u + orow) * 128u + (lane >> 5) * 2u;
-    uint32_t ax[8], aw[8];
-#pragma unroll
-    for (uint32_t pc = 0; pc < 8u; pc++) ax[pc] = xrow + ((pc ^ osw) << 4), aw[pc] = wrow + ((pc ^ osw) << 4);
-    v16f acc;
-#pragma unroll
-    for (int i = 0; i < 16; i++) acc[i] = 0.0f;
-    float af[2][4], bf[2][4]; /* the low halves stay zero: the reads write high halves only */
-#pragma unroll
-    for (int h = 0; h < 2; h++)
-#pragma unroll
-        for (int d = 0; d < 4; d++) af[h][d] = 0.0f, bf[h][d] = 0.0f;
-    issue(0u, 0u);
-    if (NC > 1u) issue(1u, 1u);
-    if (NC > 2u) issue(2u, 2u);
-    if (NC > 2u) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else if (NC > 1u) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    asm volatile("s_barrier" ::: "memory"); /* chunk 0 is complete */
-    rss_read<0u>(af[0], bf[0], ax[0], aw[0]);
-    rss_wait_reads(af[0], bf[0]);
-#define RSM_MFMA(d) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][d], bf[cur][d], acc, 0, 0, 0)
-#define RSM_FENCE() __builtin_amdgcn_sched_barrier(0)
-    /* one chunk in stage STG (a constant: the reads' offsets are immediates) */
-    auto chunk = [&](auto stg_, uint32_t c) {
-        constexpr uint32_t STG = decltype(stg_)::value, STN = (STG + 1u) % ST;
-#pragma unroll
-        for (uint32_t pc = 0; pc < 8u; pc++) {
-            const uint32_t cur = pc & 1u, nxt = cur ^ 1u;
-            RSM_FENCE();
-            RSM_MFMA(0);
-            RSM_FENCE();
-            if (pc == 7u) {
-                /* this wave's reads of chunk c have all landed (piece 7 was waited for a piece ago); once its loads
-                 * of chunk c + 1 have landed too, the barrier says both of every wave */
-                if (c + 2u < NC) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                asm volatile("s_barrier" ::: "memory");
-                rss_read<STN>(af[nxt], bf[nxt], ax[0], aw[0]); /* past the last chunk: stale bytes, never used */
-            } else {
-                rss_read<STG>(af[nxt], bf[nxt], ax[(pc + 1u) & 7u], aw[(pc + 1u) & 7u]);
-            }
-            RSM_FENCE();
-            RSM_MFMA(1);
-            RSM_FENCE();
-            if (pc == 7u && c + ST < NC) issue(c + ST, STG); /* into the stage chunk c has left */
-            RSM_FENCE();
-            RSM_MFMA(2);
-            RSM_FENCE();
-            RSM_MFMA(3);
-            RSM_FENCE();
-            rss_wait_reads(af[nxt], bf[nxt]);
-        }
-    };
-    for (uint32_t c = 0; c < NC; c += 3u) {
-        chunk(std::integral_constant<uint32_t, 0u>{}, c);
-        if (c + 1u < NC) chunk(std::integral_constant<uint32_t, 1u>{}, c + 1u);
-        if (c + 2u < NC) chunk(std::integral_constant<uint32_t, 2u>{}, c + 2u);
-    }
-#undef RSM_MFMA
-#undef RSM_FENCE
-    /* acc[r] = out[m0 + 8 * (r / 4) + 4 * (lane / 32) + r % 4][n0 + lane % 32] */
-    const uint32_t n = n0 + (lane & 31u);
-#pragma unroll
-    for (uint32_t r = 0; r < 16u; r++) {
-        const uint32_t m = m0 + 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
-        if (m < M && n < N) out[(size_t)m * N + n] = acc[r];
-    }
-}
-
-/* The same on v_mfma_f32_16x16x4_f32 (four k per instruction, a quarter of the chain latency per k of
- * the 32x32x2 form, also bit-identical to the sequential sum): a wave computes 16 tokens x 32 experts as
- * two independent chains that share the token operand. Half the outputs per operand byte, but twice as
- * many, shorter-lived waves: this is the form for problems too small to fill the chip with 32 x 32
- * tiles, where the chain latency is the time (from 2^17 outputs; below that the vector-unit form, whose
- * chain is shorter still, wins). Lane = (row lane & 15, k lane >> 4): a lane reads the two
- * dwords of its row's 16-byte piece that hold k = 4 h + (lane >> 4), h = 0, 1, with one ds_read2_b32. */
-#define RS16_NB 2
-struct Rs16Stage {
-    uint8_t x[16u * 128u];
-    uint8_t w[RS16_NB * 16u * 128u];
-};
-__global__ __launch_bounds__(256) void k_router_score_mfma16(float* __restrict__ out, const bf16_t* __restrict__ x,
-                                                             const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
-                                                             uint32_t K) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t rs16_raw[];
-    constexpr int NB = RS16_NB, NLD = 2 + 2 * NB; /* direct loads per chunk */
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    Rs16Stage* const ring = (Rs16Stage*)rs16_raw + wv * RSM_STAGES;
-    const uint32_t G = gridDim.x, tn_count = (N + 16u * NB - 1u) / (16u * NB), tm_count = (M + 15u) / 16u;
-    const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
-    const uint32_t wid = wg * 4u + wv;
-    if (wid >= tn_count * tm_count) return; /* whole wave; there is no barrier below */
-    const uint32_t m0 = (wid / tn_count) * 16u, n0 = (wid % tn_count) * (16u * NB);
-    const uint32_t NC = K / 64u;
-    const uint32_t lr = lane >> 3, lp = lane & 7u;
-    const uint8_t *xsrc[2], *wsrc[2 * NB];
-#pragma unroll
-    for (uint32_t j = 0; j < 2u * NB; j++) {
-        const uint32_t row = 8u * j + lr, sw = ((row & 15u) >> 1) & 7u;
-        const uint32_t nr = n0 + row < N ? n0 + row : N - 1u;
-        wsrc[j] = (const uint8_t*)(w + (size_t)nr * K) + ((lp ^ sw) << 4);
-        if (j < 2u) {
-            const uint32_t mr = m0 + row < M ? m0 + row : M - 1u;
-            xsrc[j] = (const uint8_t*)(x + (size_t)mr * K) + ((lp ^ sw) << 4);
-        }
-    }
-    auto issue = [&](uint32_t c) {
-        Rs16Stage* s = &ring[c % RSM_STAGES];
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; j++)
-            __builtin_amdgcn_global_load_lds((const void*)(xsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->x[8u * j * 128u], 16, 0, 0);
-#pragma unroll
-        for (uint32_t j = 0; j < 2u * NB; j++)
-            __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)c * 128u), (rsm_lds_void*)&s->w[8u * j * 128u], 16, 0, 0);
-    };
-    const uint32_t orow = lane & 15u, ks = lane >> 4, osw = (orow >> 1) & 7u;
-    const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)&ring[0];
-    const uint32_t obase = ring0 + orow * 128u + (ks >> 1) * 4u;
-    const uint32_t sel = (ks & 1u) ? 0x03020c0cu : 0x01000c0cu;
-    v4f acc[NB];
-#pragma unroll
-    for (int b = 0; b < NB; b++) acc[b] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
-    /* Software pipeline over the 8-k pieces: while piece p multiplies, the reads of piece p + 1 (issued
-     * during piece p - 1) are waited for and widened into the other half of the operand registers, and
-     * the reads of piece p + 2 are issued. Everything but matrix instructions is issued behind one. */
-    uint2 xa[2], wb[2][NB];
-    float af[2][2], bf[2][NB][2];
-    auto read_piece = [&](uint32_t stage, uint32_t pc, uint32_t buf) {
-        const uint32_t addr = obase + stage * (uint32_t)sizeof(Rs16Stage) + ((pc ^ osw) << 4);
-        asm volatile("ds_read2_b32 %0, %1 offset1:2" : "=v"(xa[buf]) : "v"(addr) : "memory");
-#pragma unroll
-        for (int b = 0; b < NB; b++)
-            asm volatile("ds_read2_b32 %0, %1 offset1:2" : "=v"(wb[buf][b]) : "v"(addr + 2048u + (uint32_t)b * 2048u) : "memory");
-    };
-    auto wait_reads = [&](uint32_t buf) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[buf]), "+v"(wb[buf][0]), "+v"(wb[buf][NB - 1])); };
-    auto widen_x = [&](uint32_t buf) {
-        af[buf][0] = __uint_as_float(__builtin_amdgcn_perm(xa[buf].x, xa[buf].x, sel));
-        af[buf][1] = __uint_as_float(__builtin_amdgcn_perm(xa[buf].y, xa[buf].y, sel));
-    };
-    auto widen_w = [&](uint32_t buf, int b) {
-        bf[buf][b][0] = __uint_as_float(__builtin_amdgcn_perm(wb[buf][b].x, wb[buf][b].x, sel));
-        bf[buf][b][1] = __uint_as_float(__builtin_amdgcn_perm(wb[buf][b].y, wb[buf][b].y, sel));
-    };
-    issue(0u);
-    if (NC > 1u) issue(1u);
-    if (NC > 2u) issue(2u);
-    if (NC > 2u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
-    else if (NC > 1u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    read_piece(0u, 0u, 0u);
-    wait_reads(0u);
-    widen_x(0u);
-#pragma unroll
-    for (int b = 0; b < NB; b++) widen_w(0u, b);
-    read_piece(0u, 1u, 1u);
-    wait_reads(1u); /* nothing is in flight across the loop's back edge */
-    uint32_t st = 0;
-#define RS16_FENCE() __builtin_amdgcn_sched_barrier(0)
-    for (uint32_t c = 0; c < NC; c++) {
-        const uint32_t stn = st == RSM_STAGES - 1u ? 0u : st + 1u;
-#pragma unroll
-        for (uint32_t pc = 0; pc < 8u; pc++) {
-            const uint32_t cur = pc & 1u, nxt = cur ^ 1u;
-            /* four matrix instructions per piece; the other work is spread over the gaps between them */
-            RS16_FENCE();
-            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][0], bf[cur][0][0], acc[0], 0, 0, 0);
-            RS16_FENCE();
-            wait_reads(nxt); /* piece p + 1, requested a piece ago */
-            /* piece p + 2 into the raw registers piece p came from (widened a piece ago) */
-            if (pc == 6u) {
-                /* every piece of chunk c has been read (piece 7 was waited for above): chunk c + 1 must have
-                 * landed before its first piece is read, and chunk c's stage takes chunk c + 3 */
-                if (c + 2u < NC) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                read_piece(stn, 0u, cur); /* past the last chunk: stale bytes, never used */
-            } else if (pc == 7u) {
-                read_piece(stn, 1u, cur);
-            } else {
-                read_piece(st, pc + 2u, cur);
-            }
-            RS16_FENCE();
-#pragma unroll
-            for (int b = 1; b < NB; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][0], bf[cur][b][0], acc[b], 0, 0, 0);
-            RS16_FENCE();
-            widen_x(nxt);
-            widen_w(nxt, 0);
-            RS16_FENCE();
-            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][1], bf[cur][0][1], acc[0], 0, 0, 0);
-            RS16_FENCE();
-#pragma unroll
-            for (int b = 1; b < NB; b++) widen_w(nxt, b);
-            RS16_FENCE();
-#pragma unroll
-            for (int b = 1; b < NB; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][1], bf[cur][b][1], acc[b], 0, 0, 0);
-            RS16_FENCE();
-            if (pc == 6u && c + 3u < NC) issue(c + 3u);
-            if (pc == 7u) wait_reads(cur); /* nothing in flight across the back edge */
-        }
-        st = stn;
-    }
-#undef RS16_FENCE
-    /* acc[b][r] = out[m0 + 4 * (lane / 16) + r][n0 + 16 b + lane % 16] */
-#pragma unroll
-    for (int b = 0; b < NB; b++) {
-        const uint32_t n = n0 + 16u * (uint32_t)b + (lane & 15u);
-#pragma unroll
-        for (uint32_t r = 0; r < 4u; r++) {
-            const uint32_t m = m0 + 4u * (lane >> 4) + r;
-            if (m < M && n < N) out[(size_t)m * N + n] = acc[b][r];
-        }
-    }
-}
 
 /* Small problems (decode). Two things bound this shape: the dependent chain of K multiply-adds per
  * output, and LDS bandwidth (every multiply-add of every lane reads a fresh operand pair). Both say
@@ -697,23 +235,43 @@ __global__ __launch_bounds__((TOK + RSR_STAGERS) * 64u) void k_router_score_row(
     router_score_row_body<TOK>(out, x, w, M, N, K, blockIdx.x, blockIdx.y, rsr_raw);
 }
 
-/* The 16 x 32 form as it runs by default: like k_router_score_mfma_shared, operands widened by the LDS read
- * (no vector instruction next to the matrix instructions) and operand rows shared by the workgroup. Four waves
- * stacked over 64 tokens share one block of 32 experts: a stage holds 64 + 32 rows (12 KB), a wave loads a
- * quarter of it (16 token rows, 8 expert rows). A piece is only four short matrix instructions, so the reads run
- * two pieces ahead into four sets of operand registers (set = piece % 4: the same in every chunk). The barrier of
- * chunk c sits in its seventh piece, before the first read of chunk c + 1: every wave has then landed its loads
- * of chunk c + 1 and its reads of chunk c - 1, whose stage takes chunk c + 3 (four stages, 48 KB). */
-#define RS16S_STAGES 4u
-struct Rs16sStage {
+/* Large problems with K a multiple of 64: the same sums on the matrix unit. v_mfma_f32_16x16x4_f32 adds
+ * a[i][k] * b[k][j] for four consecutive k to its f32 accumulator one after the other, each step rounded to
+ * nearest even and denormals kept (measured against the fmaf chain, bit for bit, normal and denormal ranges;
+ * v_mfma_f32_32x32x2_f32 does the same with two k), so a chain of K / 4 of them IS the reference's sum in the
+ * reference's order. A wave computes 16 tokens x 32 experts as two independent chains that share the token
+ * operand; lane = (row lane & 15, k lane >> 4).
+ * Two facts of the part shape the kernel. (1) The f32 matrix instructions execute on the vector unit's own
+ * multiply-add lanes (the f32 matrix peak equals the vector f32 peak): a vector instruction between two of
+ * them does not hide behind them, it adds its full time (measured on a 32 x 32 form of this kernel: the eight
+ * byte permutes that widened a piece's bf16 operands cost 9 cycles each, 29 of 173 us at T = 4096, E = 256,
+ * K = 7168). So an operand is widened by its LDS read: ds_read_u16_d16_hi puts a bf16 into the high half of a
+ * register whose low half is zero, which is the f32. The per-lane addresses of the eight 16-byte pieces of a
+ * row are computed once (LDS piece p of row r holds global piece p ^ ((r >> 1) & 7), so that the 16 rows of a
+ * read fall on distinct banks; that makes them lane-dependent) and stage, block and k half are immediate
+ * offsets: the loop issues no vector instruction next to its matrix instructions.
+ * (2) A CU's vector-memory path delivers about 38 KB/us whatever level answers, and wave-private operand rings
+ * (every token row loaded by each of the waves that use it) ask for more than that at the matrix unit's full
+ * rate. So the four waves of a workgroup, stacked over 64 tokens, share one block of 32 experts and one ring:
+ * a stage holds 64 + 32 rows (12 KB, direct global -> LDS loads, 8 lanes per 128-byte line), a wave loads a
+ * quarter of it (16 token rows, 8 expert rows). A piece (8 k) is only four short matrix instructions, so the
+ * reads run two pieces ahead into four sets of operand registers (set = piece % 4: the same in every chunk).
+ * The barrier of chunk c sits in its seventh piece, before the first read of chunk c + 1: every wave has then
+ * landed its loads of chunk c + 1 and its reads of chunk c - 1, whose stage takes chunk c + 3 (four stages,
+ * 48 KB: a CU takes three workgroups). Measured against the earlier forms (private rings, operands widened by
+ * permutes; 32 x 32 tiles where they filled the SIMDs evenly): DeepSeek-V3 router at 4096 tokens 176 -> 141 us
+ * (a shared-ring 32 x 32 form with the same reads: 147), GLM slice (E = 288, K = 4096) at 8192 tokens 243 -> 166,
+ * Qwen3 at 2048 tokens 60 -> 41. */
+#define RSM_STAGES 4u
+struct RsmStage {
     uint8_t x[64u * 128u];
     uint8_t w[32u * 128u];
 };
-static_assert(sizeof(Rs16sStage) == 12288u, "the stage size is an immediate of the LDS reads below");
+static_assert(sizeof(RsmStage) == 12288u, "the stage size is an immediate of the LDS reads below");
 /* six 2-byte reads of a piece: k = ks and 4 + ks (the lane's address holds 2 ks) of the lane's token row and of
  * its expert row in both 16-row blocks */
 template <uint32_t STG>
-__device__ __forceinline__ void rs16s_read(float (&a)[2], float (&b)[2][2], uint32_t ax, uint32_t aw) {
+__device__ __forceinline__ void rsm_read(float (&a)[2], float (&b)[2][2], uint32_t ax, uint32_t aw) {
     asm volatile("ds_read_u16_d16_hi %0, %6 offset:%8\n\t"
                  "ds_read_u16_d16_hi %2, %7 offset:%8\n\t"
                  "ds_read_u16_d16_hi %4, %7 offset:%10\n\t"
@@ -725,17 +283,17 @@ __device__ __forceinline__ void rs16s_read(float (&a)[2], float (&b)[2][2], uint
                  : "memory");
 }
 /* all but the newest piece's six reads have landed (LDS answers in order) */
-__device__ __forceinline__ void rs16s_wait_older(float (&a)[2], float (&b)[2][2]) {
+__device__ __forceinline__ void rsm_wait_older(float (&a)[2], float (&b)[2][2]) {
     asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[1][0]), "+v"(b[1][1]));
 }
-__global__ __launch_bounds__(256) void k_router_score_mfma16_shared(float* __restrict__ out, const bf16_t* __restrict__ x,
+__global__ __launch_bounds__(256) void k_router_score_mfma(float* __restrict__ out, const bf16_t* __restrict__ x,
                                                                     const bf16_t* __restrict__ w, uint32_t M, uint32_t N,
                                                                     uint32_t K) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t rs16s_raw[];
-    constexpr uint32_t ST = RS16S_STAGES, NLD = 3u; /* direct loads per wave and chunk */
+    extern __shared__ __attribute__((aligned(16))) uint8_t rsm_raw[];
+    constexpr uint32_t ST = RSM_STAGES, NLD = 3u; /* direct loads per wave and chunk */
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    Rs16sStage* const ring = (Rs16sStage*)rs16s_raw;
+    RsmStage* const ring = (RsmStage*)rsm_raw;
     const uint32_t G = gridDim.x, gx = (N + 31u) / 32u;
     const uint32_t wg = (G % 8u == 0u) ? (blockIdx.x % 8u) * (G / 8u) + blockIdx.x / 8u : blockIdx.x;
     const uint32_t M0 = (wg / gx) * 64u, N0 = (wg % gx) * 32u; /* the workgroup's block */
@@ -759,7 +317,7 @@ __global__ __launch_bounds__(256) void k_router_score_mfma16_shared(float* __res
         woff = nr * K * 2u + ((lp ^ ((row >> 1) & 7u)) << 4);
     }
     auto issue = [&](uint32_t c, uint32_t stage) {
-        Rs16sStage* s = &ring[stage];
+        RsmStage* s = &ring[stage];
         /* opaque scalar bases and lane offsets: an address stays "scalar base + 32-bit lane offset" */
         uint64_t xcb = (uint64_t)(uintptr_t)(xblk + (size_t)c * 128u), wcb = (uint64_t)(uintptr_t)(wblk + (size_t)c * 128u);
         asm volatile("" : "+s"(xcb), "+s"(wcb));
@@ -795,18 +353,18 @@ __global__ __launch_bounds__(256) void k_router_score_mfma16_shared(float* __res
     else if (NC > 1u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     asm volatile("s_barrier" ::: "memory"); /* chunk 0 is complete */
-    rs16s_read<0u>(af[0], bf[0], ax[0], aw[0]);
-    rs16s_read<0u>(af[1], bf[1], ax[1], aw[1]);
-    rs16s_wait_older(af[0], bf[0]);
-#define RS16_FENCE() __builtin_amdgcn_sched_barrier(0)
+    rsm_read<0u>(af[0], bf[0], ax[0], aw[0]);
+    rsm_read<0u>(af[1], bf[1], ax[1], aw[1]);
+    rsm_wait_older(af[0], bf[0]);
+#define RSM_FENCE() __builtin_amdgcn_sched_barrier(0)
     auto chunk = [&](auto stg_, uint32_t c) {
         constexpr uint32_t STG = decltype(stg_)::value, STN = (STG + 1u) % ST, STF = (STG + 3u) % ST;
 #pragma unroll
         for (uint32_t pc = 0; pc < 8u; pc++) {
             const uint32_t cur = pc & 3u, n1 = (pc + 1u) & 3u, n2 = (pc + 2u) & 3u;
-            RS16_FENCE();
+            RSM_FENCE();
             acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][0], bf[cur][0][0], acc[0], 0, 0, 0);
-            RS16_FENCE();
+            RSM_FENCE();
             if (pc == 6u) {
                 /* this wave's loads of chunk c + 1 have landed and so have its reads of chunk c - 1 (its last piece was
                  * waited for seven pieces ago): behind the barrier that holds for every wave */
@@ -815,18 +373,18 @@ __global__ __launch_bounds__(256) void k_router_score_mfma16_shared(float* __res
                 asm volatile("s_barrier" ::: "memory");
             }
             /* piece p + 2 into the set piece p - 2 used; past the last chunk: stale bytes, never used */
-            if (pc < 6u) rs16s_read<STG>(af[n2], bf[n2], ax[(pc + 2u) & 7u], aw[(pc + 2u) & 7u]);
-            else rs16s_read<STN>(af[n2], bf[n2], ax[(pc + 2u) & 7u], aw[(pc + 2u) & 7u]);
-            RS16_FENCE();
+            if (pc < 6u) rsm_read<STG>(af[n2], bf[n2], ax[(pc + 2u) & 7u], aw[(pc + 2u) & 7u]);
+            else rsm_read<STN>(af[n2], bf[n2], ax[(pc + 2u) & 7u], aw[(pc + 2u) & 7u]);
+            RSM_FENCE();
             acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][0], bf[cur][1][0], acc[1], 0, 0, 0);
-            RS16_FENCE();
+            RSM_FENCE();
             if (pc == 6u && c + 3u < NC) issue(c + 3u, STF); /* into the stage chunk c - 1 has left */
-            RS16_FENCE();
+            RSM_FENCE();
             acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][1], bf[cur][0][1], acc[0], 0, 0, 0);
-            RS16_FENCE();
+            RSM_FENCE();
             acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[cur][1], bf[cur][1][1], acc[1], 0, 0, 0);
-            RS16_FENCE();
-            rs16s_wait_older(af[n1], bf[n1]); /* piece p + 1 */
+            RSM_FENCE();
+            rsm_wait_older(af[n1], bf[n1]); /* piece p + 1 */
         }
     };
     for (uint32_t c = 0; c < NC; c += 4u) {
@@ -835,7 +393,7 @@ __global__ __launch_bounds__(256) void k_router_score_mfma16_shared(float* __res
         if (c + 2u < NC) chunk(std::integral_constant<uint32_t, 2u>{}, c + 2u);
         if (c + 3u < NC) chunk(std::integral_constant<uint32_t, 3u>{}, c + 3u);
     }
-#undef RS16_FENCE
+#undef RSM_FENCE
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stale reads of the last two pieces */
     /* acc[b][r] = out[m0 + 4 * (lane / 16) + r][n0 + 16 b + lane % 16] */
 #pragma unroll
@@ -849,19 +407,13 @@ __global__ __launch_bounds__(256) void k_router_score_mfma16_shared(float* __res
     }
 }
 
-#define RS16_LDS (4u * RSM_STAGES * (uint32_t)sizeof(Rs16Stage))
-#define RSM_LDS (4u * RSM_STAGES * (uint32_t)sizeof(RsmStage))
-#define RSM_LDS8 (8u * 2u * (uint32_t)sizeof(RsmStage))
-#define RSS_LDS (RSM_STAGES * (uint32_t)sizeof(RssStage))
-#define RS16S_LDS (RS16S_STAGES * (uint32_t)sizeof(Rs16sStage))
+#define RSM_LDS (RSM_STAGES * (uint32_t)sizeof(RsmStage))
 
 /* dynamic-LDS limits of the score kernels, once per device (plow_moe_device_setup) */
 static bool rf_setup();
 int plow_moe_route_setup() {
     const bool ok = rf_setup() &&
-        hipFuncSetAttribute((const void*)k_router_score_mfma16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RS16_LDS) == hipSuccess &&
-        hipFuncSetAttribute((const void*)k_router_score_mfma<4u, 3u>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSM_LDS) == hipSuccess &&
-        hipFuncSetAttribute((const void*)k_router_score_mfma<8u, 2u>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSM_LDS8) == hipSuccess &&
+        hipFuncSetAttribute((const void*)k_router_score_mfma, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSM_LDS) == hipSuccess &&
         hipFuncSetAttribute((const void*)k_router_score_row<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess &&
         hipFuncSetAttribute((const void*)k_router_score_row<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess &&
         hipFuncSetAttribute((const void*)k_router_score_row<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RSR_LDS) == hipSuccess;
@@ -871,41 +423,15 @@ int plow_moe_route_setup() {
 int launch_router_score(float* out, const void* x, const void* w, uint32_t M, uint32_t N, uint32_t K,
                         hipStream_t st) {
     if (K % 8u) return PLOW_MOE_EINVAL;
-    /* 32 x 32 tiles (fewer operand bytes per output) when they fill the SIMDs evenly: a whole number of
-     * tiles per SIMD, or at least four; otherwise, from 2^17 outputs, the 16 x 32 tiles */
-    const uint64_t t32 = (uint64_t)((N + 31) / 32) * ((M + 31) / 32);
+    /* the matrix-unit form from 2^17 outputs on (below that the vector-unit forms, whose chains are shorter still,
+     * win: 256 x 256 x 7168 takes 54 us there, 512 x 256 x 7168 takes 67 here and 128 there) */
     const PlowMoeTuning& tune = plow_moe_tuning();
     const uint64_t n_cu = plow_moe_n_cu();
     if (!n_cu) return PLOW_MOE_EDEVICE;
-    const uint64_t n_simd = 4u * n_cu;
-    const uint64_t outputs = (uint64_t)M * N, force32 = tune.score_mfma32_from;
-    const bool mfma_ok = K % 64u == 0u && !tune.score_valu;
-    const bool use32 = mfma_ok && outputs >= (1u << 18) && (force32 ? outputs >= force32 : (t32 % n_simd == 0u || t32 >= 4u * n_simd));
-    const bool use16 = mfma_ok && !use32 && outputs >= (1u << 17);
-    if (use16 && !tune.score_private) {
+    /* (a load's lane offset is 32 bits and spans 64 rows of a matrix) */
+    if (K % 64u == 0u && (uint64_t)K * 2u * 64u < (1ull << 32) && !tune.score_valu && (uint64_t)M * N >= (1u << 17)) {
         const uint32_t g = ((N + 31) / 32) * ((M + 63) / 64);
-        k_router_score_mfma16_shared<<<g, 256, RS16S_LDS, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
-    } else if (use16) {
-        const uint32_t lds = RS16_LDS;
-        const uint32_t waves = ((N + 16u * RS16_NB - 1u) / (16u * RS16_NB)) * ((M + 15u) / 16u);
-        k_router_score_mfma16<<<(waves + 3u) / 4u, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
-    } else if (use32) {
-        /* two waves per SIMD when the tiles fill both slots of every SIMD a whole number of times (DeepSeek-V3
-         * router at 8192 tokens 360 -> 330 us, at 16384 655 -> 591; at 4096, one tile per SIMD, it would leave half
-         * the SIMDs idle: 174 -> 298) */
-        if (!tune.score_private) {
-            const uint32_t g = ((N + 63) / 64) * ((M + 63) / 64);
-            k_router_score_mfma_shared<<<g, 256, RSS_LDS, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
-            return 0;
-        }
-        if (t32 % (2u * n_simd) == 0u) {
-            const uint32_t g = ((N + 63) / 64) * ((M + 127) / 128);
-            k_router_score_mfma<8u, 2u><<<g, 512, RSM_LDS8, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
-            return 0;
-        }
-        const uint32_t lds = RSM_LDS;
-        const uint32_t g = ((N + 63) / 64) * ((M + 63) / 64);
-        k_router_score_mfma<4u, 3u><<<g, 256, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        k_router_score_mfma<<<g, 256, RSM_LDS, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else if ((uint64_t)M * N >= (1u << 19)) {
         if ((uint64_t)((N + 63) / 64) * ((M + 63) / 64) < 2u * n_cu) { /* fewer than two 64-row workgroups per CU */
             dim3 g((N + 63) / 64, (M + 31) / 32);

@@ -10,10 +10,8 @@
  *   PLOW_MOE_SK_GLU           regs             block-mode decode GLU on the register form (default: direct-to-LDS form)
  *   PLOW_MOE_SK_NARROW        (any)            decode DOWN register form with 128-channel workgroups (default 256)
  *   PLOW_MOE_A16_KERNEL       regs             bf16-activation kernels on their register form (default: direct-to-LDS form)
- *   PLOW_MOE_SCORE_KERNEL     tile8 | valu | private   router score: keep the 8 x 8 tile kernel for few outputs / keep
- *                                              the vector-unit kernels at prefill sizes / matrix-unit forms with
- *                                              wave-private operand rings (default: operands shared by a workgroup)
- *   PLOW_MOE_SCORE_MFMA32_FROM  n              number of outputs from which the 32 x 32 matrix-unit tiles are forced
+ *   PLOW_MOE_SCORE_KERNEL     tile8 | valu     router score: keep the 8 x 8 tile kernel for few outputs / keep
+ *                                              the vector-unit kernels at prefill sizes
  *   PLOW_MOE_A16_TILED        0                keep the bf16-activation arms on the streaming kernels at every row count
  *   PLOW_MOE_A16_GEMV         0                keep the bf16-activation arms off the matrix-vector form at a few tokens
  */
@@ -31,8 +29,6 @@ struct PlowMoeTuning {
     bool a16_regs;
     bool score_tile8;
     bool score_valu;
-    bool score_private;
-    uint64_t score_mfma32_from;
     bool a16_tiled;
     bool a16_gemv;
 };

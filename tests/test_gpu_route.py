@@ -154,9 +154,8 @@ def test_route_on_logits_at_the_ends_of_the_exponential(moe, oracle, flags):
     assert np.array_equal(got["gate"].view(np.uint32), want["gate"].view(np.uint32))
 
 
-# K a multiple of 64 and 2^17 outputs or more: the matrix-unit forms. 16 x 32 tiles with 4, 2, 1, 16 and 3
-# chunks (the fifth is ragged in both directions); the last two fill the SIMDs evenly with 32 x 32 tiles and
-# take that form (2 and 3 chunks)
+# K a multiple of 64 and 2^17 outputs or more: the matrix-unit form (64 tokens x 32 experts per workgroup, a ring of
+# four 64-k chunks): 4, 2, 1, 16, 3, 5, 7 and 112 chunks, ragged in tokens and in experts
 # Few outputs and K a multiple of 256: one token x 64 experts per consumer wave, 1 / 2 / 4 tokens per
 # workgroup (ragged in tokens and experts: (3, 100), (15, 130), (17, 100)); (6, 40, 768) etc. on the 8 x 8 tiles
 @pytest.mark.parametrize("M,N,K", [(3, 100, 512), (2, 64, 256), (5, 64, 1280), (15, 130, 1024), (16, 64, 2048),
@@ -164,7 +163,7 @@ def test_route_on_logits_at_the_ends_of_the_exponential(moe, oracle, flags):
                                    (6, 40, 768), (64, 256, 7168), (1, 384, 7168), (700, 1000, 264),
                                    (700, 1000, 256), (520, 520, 128), (1030, 300, 64), (1500, 288, 1024),
                                    (413, 331, 192), (1024, 1024, 128), (2048, 512, 192),
-                                       (2048, 1024, 192), (4096, 512, 320)])  # the last two: two 32 x 32 tiles per SIMD
+                                   (2048, 1024, 192), (4096, 512, 320), (520, 260, 448), (512, 256, 7168)])
 def test_router_score_bit_exact(moe, oracle, M, N, K):
     print(f"[case] score {M}x{N}x{K}", flush=True)
     if (M, N, K) == (6, 40, 768):
