@@ -455,7 +455,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     const uint32_t nblk = g.N / 128u;
     struct Tile {
         uint32_t e, nt, r0, rows;
-        uint64_t wp0;
+        uint64_t wp0, wp1; /* weight rows (GLU block mode: gate, up) */
+        uint64_t sp0, sp1; /* block mode: their scale tables */
     };
     /* every value is the same in all lanes (made explicit with readfirstlane so that what is indexed
      * by them is read with scalar loads) */
@@ -480,17 +481,29 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         }
         const uint32_t mt = (uint32_t)__builtin_amdgcn_readfirstlane((int)mt_v);
         t.nt = (uint32_t)__builtin_amdgcn_readfirstlane((int)nt_v);
-        const uint32_t cnt = (uint32_t)g.meta[g.E + t.e];
+        /* meta and the pointer table were written by earlier kernels and the expert index is the same in every
+         * lane: read through the constant address space these are scalar loads, which a loader's direct loads in
+         * flight do not have to be waited for (a vector load's result would drain them, once per tile) */
+        const auto* const meta_c = (const __attribute__((address_space(4))) int32_t*)g.meta;
+        const auto* const wtab_c = (const __attribute__((address_space(4))) uint64_t*)g.wtab;
+        const uint32_t cnt = (uint32_t)meta_c[g.E + t.e];
         /* nine-group kernels split the expert's rows evenly over its Me = ceil(cnt / cap) tiles, in whole 16-row
          * groups: a tile takes nine groups only where that saves a tile; eight-group kernels fill 128-row tiles
          * and leave the rest to the last one */
         const uint32_t Mu = (uint32_t)__builtin_amdgcn_readfirstlane((int)Me);
         const uint32_t h = NG == 8 ? 128u : (((cnt + Mu - 1u) / Mu + 15u) / 16u) * 16u; /* <= cap since cnt <= cap * Me */
-        t.r0 = (uint32_t)g.meta[t.e] + mt * h;
+        t.r0 = (uint32_t)meta_c[t.e] + mt * h;
         t.rows = cnt - mt * h < h ? cnt - mt * h : h; /* live rows of the tile */
         /* block mode: {gate, up, down} tables; per-channel mode: {gate_up fused [2N][K], down} */
-        t.wp0 = PC ? g.wtab[(size_t)t.e * 2u + (GLU ? 0u : 1u)] : g.wtab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
-        if (GLU && !PC && g.wtab[(size_t)t.e * 3u + 1u] == 0ull) t.wp0 = 0ull; /* gate without up: not resident */
+        t.wp0 = PC ? wtab_c[(size_t)t.e * 2u + (GLU ? 0u : 1u)] : wtab_c[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
+        t.wp1 = (GLU && !PC) ? wtab_c[(size_t)t.e * 3u + 1u] : t.wp0;
+        if (t.wp1 == 0ull) t.wp0 = 0ull; /* gate without up: not resident */
+        t.sp0 = t.sp1 = 0ull;
+        if (!PC) {
+            const auto* const stab_c = (const __attribute__((address_space(4))) uint64_t*)g.stab;
+            t.sp0 = stab_c[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
+            t.sp1 = GLU ? stab_c[(size_t)t.e * 3u + 1u] : t.sp0;
+        }
         return t;
     };
     /* this workgroup's next tile at or after `from` whose expert is resident (`total` if none); loaders
@@ -569,8 +582,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             }
             P.w0 = P.w1 = 0.0f;
             if (!PC && !A4) {
-                const float* S0 = (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
-                const float* S1 = GLU ? (const float*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : S0;
+                const float* S0 = (const float*)(uintptr_t)t.sp0;
+                const float* S1 = (const float*)(uintptr_t)t.sp1;
                 const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
                 const uint32_t i = tid - NCW * 64u; /* 0..255 over the four loaders; KS <= 128 */
                 P.w0 = i < KS ? S0[(size_t)nb0 * KS + i] : 0.0f;
@@ -582,7 +595,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             S.W0 = (const uint8_t*)(uintptr_t)t.wp0;
             S.nine = (cw < 2u && rows > 128u) ? 1u : 0u;
             S.W1 = !GLU ? S.W0 : PC ? S.W0 + (size_t)g.N * K /* up rows follow the N gate rows */
-                               : (const uint8_t*)(uintptr_t)g.wtab[(size_t)t.e * 3u + 1u];
+                               : (const uint8_t*)(uintptr_t)t.wp1;
 #pragma unroll
             for (uint32_t i = 0; i < 5u; i++) {
                 const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * (cw & 1u) + lr;
@@ -623,8 +636,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             }
             if constexpr (A4) {
                 S.tsp = g.a_e8m0 + (size_t)P.tsrow * K32 + (lane & 1u) * 4u;
-                const uint8_t* const SW0 = (const uint8_t*)(uintptr_t)g.stab[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
-                const uint8_t* const SW1 = GLU ? (const uint8_t*)(uintptr_t)g.stab[(size_t)t.e * 3u + 1u] : SW0;
+                const uint8_t* const SW0 = (const uint8_t*)(uintptr_t)t.sp0;
+                const uint8_t* const SW1 = (const uint8_t*)(uintptr_t)t.sp1;
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; j++) {
                     const uint32_t R = 64u * cw + 32u * j + (lane >> 1);
@@ -715,10 +728,13 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 /* not before this barrier: until it, the consumers may still be in the epilogue of the tile
                  * before, reading the L.epi_* half that finish() overwrites */
                 if (more && early && kb == 0u) finish(tnxt, pre, par ^ 1u, nxt);
+                /* the next tile's set-up loads go out before this block's direct loads: behind them they would be
+                 * the youngest loads at the next barrier, whose count then makes it wait for as many loads of the
+                 * block after (in practice for that block: 1.3 us per tile) */
+                if (more && !early && kb == 0u) fetch(tnxt, pre);
                 if (kb + 2u < KB) issue(cur, kb + 2u, st2);
                 else if (more) issue(nxt, kb + 2u - KB, st2);
                 st = st == 2u ? 0u : st + 1u;
-                if (more && !early && kb == 0u) fetch(tnxt, pre);
                 if (more && !early && kb == KB - 3u) finish(tnxt, pre, par ^ 1u, nxt);
             }
             WG_BARRIER(); /* after the last block (the consumers' amax exchange) */
