@@ -30,7 +30,11 @@ __device__ __forceinline__ void combine_body(const CombineArgs& a) {
         if (KT && !a.part16) {
             float4 v[KT ? KT : 1u];
 #pragma unroll
-            for (uint32_t j = 0; j < KT; j++) v[j] = *(const float4*)((const float*)a.part + ((size_t)tok * KT + j) * a.H + h);
+            for (uint32_t j = 0; j < KT; j++) {
+                typedef float f4v __attribute__((ext_vector_type(4)));
+                const f4v t = __builtin_nontemporal_load((const f4v*)((const float*)a.part + ((size_t)tok * KT + j) * a.H + h));
+                v[j] = make_float4(t[0], t[1], t[2], t[3]);
+            }
             if (a.residual) {
                 acc[0] = __uint_as_float(rr.x << 16); acc[1] = __uint_as_float(rr.x & 0xFFFF0000u);
                 acc[2] = __uint_as_float(rr.y << 16); acc[3] = __uint_as_float(rr.y & 0xFFFF0000u);

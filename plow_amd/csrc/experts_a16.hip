@@ -489,10 +489,10 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; j++)
                     __builtin_amdgcn_global_load_lds((const void*)(wsrc[sidx][j] + wofs),
-                                                     (dm_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, 0);
+                                                     (dm_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, LOAD_NT);
                 if constexpr (ENC == AENC_MXFP4)
                     __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)ld_t * AK_BN * wmul * (K / 32u) + (size_t)ld_S * 8u),
-                                                     (dm_lds_void*)&slot->sc[sidx][0], 4, 0, 0);
+                                                     (dm_lds_void*)&slot->sc[sidx][0], 4, 0, 0); /* 8 bytes of a line per step: cached */
             }
 #pragma unroll
             for (uint32_t i = 0; i < NXI; i++)

@@ -64,7 +64,7 @@ __device__ __forceinline__ void gv_load(GvRow<ENC, ITER>& r, const uint8_t* wrow
     for (int it = 0; it < ITER; it++) {
         const uint32_t p = (uint32_t)it * 64u + lane; /* the lane's 16-byte piece of the row */
         const bool in = p < pieces;
-        r.w[it] = in ? *(const __attribute__((address_space(1))) v4i*)((gv_gptr)wrow + (size_t)p * 16u) : (v4i){0, 0, 0, 0};
+        r.w[it] = in ? __builtin_nontemporal_load((const __attribute__((address_space(1))) v4i*)((gv_gptr)wrow + (size_t)p * 16u)) : (v4i){0, 0, 0, 0}; /* read once */
         if (ENC == GV_MXFP4) r.sb[it] = in ? (uint32_t)((gv_gptr)srow)[p] : 0u;
         if (ENC == GV_FP8BLK) r.sf[it] = in ? ((const __attribute__((address_space(1))) float*)(gv_gptr)srow)[p >> 3] : 0.0f; /* 8 pieces of 16 k per 128-k block */
     }
