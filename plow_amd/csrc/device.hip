@@ -23,6 +23,7 @@ const PlowMoeTuning& plow_moe_tuning() {
         t.sk_depth = d ? atoi(d) : 3;
         if (t.sk_depth < 2 || t.sk_depth > 4) t.sk_depth = 3;
         t.sk_glu_regs = is("PLOW_MOE_SK_GLU", "regs");
+        t.sk_down_regs = is("PLOW_MOE_SK_DOWN", "regs");
         t.sk_narrow = getenv("PLOW_MOE_SK_NARROW") != nullptr;
         t.a16_regs = is("PLOW_MOE_A16_KERNEL", "regs");
         t.score_tile8 = is("PLOW_MOE_SCORE_KERNEL", "tile8");

@@ -596,10 +596,130 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     }
 }
 
+/* DOWN, block mode, the same direct-to-LDS form: a wave owns 32 output channels (two 16-row operands that share
+ * the activation operand and the weight block scale) and a private ring of the same slots; the weight rows are
+ * read once, whole 128-byte lines per row and block, with non-temporal loads (the register form reads a line as
+ * two halves a k-step apart and has to keep it cached: 5.7 TB/s against the 6.6 of the GLU above). Four waves
+ * and 128 channels per workgroup: 77 KB of LDS, so a CU holds two workgroups and one's set-up trips to memory
+ * (count and pointers, then row maps and block scales) pass under the other's stream. Plain arm only: e4m3 rows
+ * by aligned row, f32 or bf16 partials by row_partidx. Rows past the expert's count read its first row with a
+ * zero scale; a row whose slot is unused is computed and not stored. */
+#define SDD_WAVES 4u
+struct SddLds {
+    SdSlot ring[SDD_WAVES][SD_STAGES];
+    float wsc[128]; /* the tile's weight block scales, all of K: K <= 16384 */
+};
+__global__ __launch_bounds__(SDD_WAVES* WAVE) void k_group_down_w8a8_dma(GroupW8A8 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t sdd_raw[];
+    SddLds& L = *(SddLds*)sdd_raw;
+    const uint32_t tiles = g.N / 128u;
+    const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
+    const uint32_t cnt = (uint32_t)g.meta[g.E + e];
+    const uint32_t r0 = (uint32_t)g.meta[e];
+    const uint64_t wp = g.wtab[(size_t)e * 3u + 2u], sp = g.stab[(size_t)e * 3u + 2u];
+    asm volatile("" ::"s"(r0), "s"(wp), "s"(sp)); /* the loads stay above the branch */
+    if (cnt == 0u || wp == 0ull) return;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, 32-byte chunk q */
+    const uint32_t lr = lane >> 3, p = lane & 7u; /* load layout: row lr of a group of 8, piece p */
+    const uint32_t K = g.K, KB = K / 128u, N = g.N;
+    const uint32_t chw = ct * 128u + wv * 32u; /* this wave's first channel */
+    const float* const sc = (const float*)(uintptr_t)sp + (size_t)ct * KB;
+    /* weight rows: load j covers LDS rows 8j .. 8j + 7 = channels chw + 8j .. */
+    const uint8_t* wsrc[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4u; j++) {
+        const uint32_t R = 8u * j + lr;
+        wsrc[j] = (const uint8_t*)(uintptr_t)wp + (size_t)(chw + R) * K + ((p ^ lds_swz8(R)) << 4);
+    }
+    for (uint32_t i = threadIdx.x; i < KB; i += SDD_WAVES * WAVE) L.wsc[i] = sc[i];
+    __syncthreads();
+    const uint32_t wsc_base = sd_lds_off(&L.wsc[0]);
+    SdSlot* const ring = L.ring[wv];
+    const uint32_t swz = lds_swz8(c);
+    const uint32_t o_lo = c * 128u + (((2u * q) ^ swz) << 4), o_hi = c * 128u + (((2u * q + 1u) ^ swz) << 4);
+
+    for (uint32_t rb = 0; rb < cnt; rb += 16u) {
+        /* activation rows of the pass: load i covers rows 8i .. 8i + 7; aligned rows need no map */
+        const uint8_t* xsrc[2];
+#pragma unroll
+        for (uint32_t i = 0; i < 2u; i++) {
+            const uint32_t idx = 8u * i + lr;
+            const uint32_t row = rb + idx < cnt ? r0 + rb + idx : r0;
+            xsrc[i] = (const uint8_t*)g.a + (size_t)row * K + ((p ^ lds_swz8(idx)) << 4);
+        }
+        const bool live = rb + c < cnt;
+        const float* const ssrc = live ? g.a_scale + (size_t)(r0 + rb + c) * KB : (const float*)(g.meta + 2u * g.E); /* tilep[0] = 0 */
+        const uint32_t sstep = live ? 1u : 0u;
+        uint32_t pidx = live ? g.row_partidx[r0 + rb + c] : PLOW_EXPERT_UNUSED;
+        float gate = live ? g.row_gate[r0 + rb + c] : 0.0f;
+        auto issue = [&](uint32_t kb) {
+            SdSlot* s = ring + kb % SD_STAGES;
+            __builtin_amdgcn_global_load_lds((const void*)(ssrc + (size_t)kb * sstep), (sd_lds_void*)&s->xs[0], 4, 0, 0);
+#pragma unroll
+            for (uint32_t i = 0; i < 2u; i++)
+                __builtin_amdgcn_global_load_lds((const void*)(xsrc[i] + (size_t)kb * 128u),
+                                                 (sd_lds_void*)&s->x[8u * i * 128u], 16, 0, 0);
+#pragma unroll
+            for (uint32_t j = 0; j < 4u; j++)
+                __builtin_amdgcn_global_load_lds((const void*)(wsrc[j] + (size_t)kb * 128u),
+                                                 (sd_lds_void*)&s->w[8u * j * 128u], 16, 0, LOAD_NT);
+        };
+        v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(pidx), "+v"(gate) : : "memory"); /* the row maps are loaded; the count starts at zero */
+        issue(0);
+        if (KB > 1u) issue(1);
+        for (uint32_t kb = 0; kb < KB; kb++) {
+            /* loads return in order: block kb has landed once at most block kb + 1's are outstanding */
+            if (kb + 1u < KB) SD_WAIT_VM(SD_NLOAD); else SD_WAIT_VM(0);
+            const uint32_t base = sd_lds_off(ring + kb % SD_STAGES);
+            v4i a0l = sd_read16<0>(base + o_lo), a0h = sd_read16<0>(base + o_hi);
+            v4i a1l = sd_read16<2048>(base + o_lo), a1h = sd_read16<2048>(base + o_hi);
+            v4i bl = sd_read16<4096>(base + o_lo), bh = sd_read16<4096>(base + o_hi);
+            float xs = sd_read4(base + 6144u + c * 4u);
+            float sa = sd_read4(wsc_base + kb * 4u);
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0l), "+v"(a0h), "+v"(a1l), "+v"(a1h));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(bl), "+v"(bh), "+v"(xs), "+v"(sa));
+            /* block kb - 1's slot is free (its reads were waited for one iteration ago): refill it */
+            if (kb + 2u < KB) issue(kb + 2u);
+            const v8i A0 = __builtin_shufflevector(a0l, a0h, 0, 1, 2, 3, 4, 5, 6, 7);
+            const v8i A1 = __builtin_shufflevector(a1l, a1h, 0, 1, 2, 3, 4, 5, 6, 7);
+            const v8i B = __builtin_shufflevector(bl, bh, 0, 1, 2, 3, 4, 5, 6, 7);
+            const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
+            const v4f t0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A0, B, z, 0, 0, 0, 0, 0, 0);
+            const v4f t1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A1, B, z, 0, 0, 0, 0, 0, 0);
+            const float s01 = xs * sa;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                acc0[i] = fmaf(t0[i], s01, acc0[i]);
+                acc1[i] = fmaf(t1[i], s01, acc1[i]);
+            }
+        }
+        /* ---- epilogue: lane holds channels chw + 4q + i and chw + 16 + 4q + i (i = 0..3) of row rb + c ---- */
+        if (pidx == PLOW_EXPERT_UNUSED) continue;
+        const size_t o = (size_t)pidx * N + chw + 4u * q;
+        const float y0 = gate * acc0[0], y1 = gate * acc0[1], y2 = gate * acc0[2], y3 = gate * acc0[3];
+        const float z0 = gate * acc1[0], z1 = gate * acc1[1], z2 = gate * acc1[2], z3 = gate * acc1[3];
+        if (g.part16) {
+            uint2 a, b;
+            a.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16), a.y = (uint32_t)f2bf(y2) | ((uint32_t)f2bf(y3) << 16);
+            b.x = (uint32_t)f2bf(z0) | ((uint32_t)f2bf(z1) << 16), b.y = (uint32_t)f2bf(z2) | ((uint32_t)f2bf(z3) << 16);
+            *(uint2*)((bf16_t*)g.out + o) = a;
+            *(uint2*)((bf16_t*)g.out + o + 16u) = b;
+        } else {
+            *(float4*)((float*)g.out + o) = make_float4(y0, y1, y2, y3);
+            *(float4*)((float*)g.out + o + 16u) = make_float4(z0, z1, z2, z3);
+        }
+    }
+}
+
 /* dynamic-LDS limit of the direct-to-LDS form, once per device (plow_moe_device_setup) */
 int plow_moe_w8a8_setup() {
     return hipFuncSetAttribute((const void*)k_group_glu_w8a8_dma, hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)sizeof(SdLds)) == hipSuccess ? 0 : PLOW_MOE_EDEVICE;
+                               (int)sizeof(SdLds)) == hipSuccess &&
+           hipFuncSetAttribute((const void*)k_group_down_w8a8_dma, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)sizeof(SddLds)) == hipSuccess ? 0 : PLOW_MOE_EDEVICE;
 }
 
 static int check_w8a8(const GroupW8A8& g) {
@@ -646,6 +766,11 @@ int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
         } else {
             k_group_w8a8_stream<false, 3, false, false, false, true><<<grid, SK_THREADS, 0, st>>>(g);
         }
+        return 0;
+    }
+    /* the plain arm on the direct-to-LDS form (the block scales of all of K sit in LDS: K <= 16384) */
+    if (!g.acc_topk && !g.a_slots && !g.a_bf16 && g.K <= 16384u && !plow_moe_tuning().sk_down_regs) {
+        k_group_down_w8a8_dma<<<grid, SDD_WAVES * WAVE, sizeof(SddLds), st>>>(g);
         return 0;
     }
     if (g.N % 256u == 0u && !plow_moe_tuning().sk_narrow) {

@@ -8,6 +8,7 @@
  *   PLOW_MOE_W8A8_TILE_WAVES  4                512-thread form of the tiled kernel (default 768 threads)
  *   PLOW_MOE_SK_DEPTH         2..4             k-steps of weight loads in flight, register form (default 3)
  *   PLOW_MOE_SK_GLU           regs             block-mode decode GLU on the register form (default: direct-to-LDS form)
+ *   PLOW_MOE_SK_DOWN          regs             block-mode decode DOWN on the register form (default: direct-to-LDS form)
  *   PLOW_MOE_SK_NARROW        (any)            decode DOWN register form with 128-channel workgroups (default 256)
  *   PLOW_MOE_A16_KERNEL       regs             bf16-activation kernels on their register form (default: direct-to-LDS form)
  *   PLOW_MOE_SCORE_KERNEL     tile8 | valu     router score: keep the 8 x 8 tile kernel for few outputs / keep
@@ -25,6 +26,7 @@ struct PlowMoeTuning {
     bool tile_waves4;
     int sk_depth;         /* 2..4 */
     bool sk_glu_regs;
+    bool sk_down_regs;
     bool sk_narrow;
     bool a16_regs;
     bool score_tile8;
