@@ -163,7 +163,8 @@ def test_route_on_logits_at_the_ends_of_the_exponential(moe, oracle, flags):
                                    (6, 40, 768), (64, 256, 7168), (1, 384, 7168), (700, 1000, 264),
                                    (700, 1000, 256), (520, 520, 128), (1030, 300, 64), (1500, 288, 1024),
                                    (413, 331, 192), (1024, 1024, 128), (2048, 512, 192),
-                                   (2048, 1024, 192), (4096, 512, 320), (520, 260, 448), (512, 256, 7168)])
+                                   (2048, 1024, 192), (4096, 512, 320), (520, 260, 448), (512, 256, 7168),
+                                   (16, 8192, 256), (8200, 16, 128), (70, 1900, 64)])  # fewer rows than a block holds
 def test_router_score_bit_exact(moe, oracle, M, N, K):
     print(f"[case] score {M}x{N}x{K}", flush=True)
     if (M, N, K) == (6, 40, 768):
