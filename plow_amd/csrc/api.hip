@@ -180,6 +180,16 @@ static uint32_t slots_of(const PlowDevInst* in, const Hint& h, uint32_t own) {
 /* Routed rows up to which the fp8 x fp8 DOWN runs as matrix-vector products (measured against the streaming
  * kernel, DeepSeek-V3 shape) */
 #define W8A8_GEMV_MAX_SLOTS 36u
+/* Tiled forms: the weight rows of an expert with a single row tile are read once and may be loaded non-temporal
+ * (the kernel decides that per expert; this is the launch's permission). DOWN: always (measured better from
+ * 16 to 143 rows per expert on average: DeepSeek-V3 shape 512 tokens 750 -> 698 us, 4096: 1069 -> 1052; Qwen3
+ * 512: 192 -> 175). GLU: up to 80 rows per expert on average (DeepSeek-V3 shape 512 tokens 1301 -> 1179 us,
+ * 2048: 1386 -> 1334, 3072: 1577 -> 1618, not taken; fp4 x fp4 arm, Kimi-K2 shape, 3072: 1404 -> 1356) */
+static uint32_t tiled_w_nt(uint32_t slots, uint32_t E, bool glu) {
+    const int env = plow_moe_tuning().tiled_nt;
+    if (env >= 0) return (uint32_t)env;
+    return !glu || (slots != 0u && slots <= 80u * E) ? 1u : 0u;
+}
 static bool want_tiled(const Hint& h, uint32_t slots, const GroupW8A8& g) {
     const int env = plow_moe_tuning().w8a8_kernel;
     const bool tiled = env >= 0 ? env == 1 : h.form >= 0 ? h.form == 1 : slots >= 16u * g.E;
@@ -319,7 +329,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         /* SiLU, or the clamped SwiGLU when a limit is given (plow runtime/amd/op_gemm_common.h:1973-1981) */
         g.f1 = in->fj[1].f; g.act = g.f1 > 0.0f ? PLOW_MOE_ACT_SWIGLU_CLAMP : PLOW_MOE_ACT_SILU;
         /* without a stated slot count: eight slots per token */
-        return want_tiled(h, slots_of(in, h, 8u * Tn), g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
+        { const uint32_t slots_ = slots_of(in, h, 8u * Tn); g.w_nt = tiled_w_nt(slots_, g.E, true);
+          return want_tiled(h, slots_, g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st); }
     }
     case PLOW_DOP_MOE_QUANT_FP8_BLOCK128: {
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5),
@@ -345,7 +356,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 5);
         g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
         g.N = H; g.K = I; g.E = E;
-        return want_tiled(h, slots_of(in, h, Tn * topk), g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
+        { const uint32_t slots_ = slots_of(in, h, Tn * topk); g.w_nt = tiled_w_nt(slots_, g.E, false);
+          return want_tiled(h, slots_, g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st); }
     }
     case PLOW_DOP_MOE_GROUP_GLU_PF: {
         const uint32_t I = i[0], H = i[1], E = i[2], enc = i[3], arm = i[7];
@@ -367,7 +379,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
             /* without a stated slot count: the row pitch of the activation scales as the token count,
              * eight slots per token */
-            return want_tiled(h, slots_of(in, h, 8u * i[4]), g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
+            { const uint32_t slots_ = slots_of(in, h, 8u * i[4]); g.w_nt = tiled_w_nt(slots_, g.E, true);
+          return want_tiled(h, slots_, g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st); }
         }
         if (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ) {
             NEED(c, ten(in, T, 3) && ten(in, T, 7), "op 85 W8A8 (bf16 rows): t3 stab, t7 fs must be bound");
@@ -429,6 +442,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.row_partidx = (const uint32_t*)ten(in, T, 6);
             g.N = I; g.K = H; g.E = E; g.act = i[5]; g.T = i[4];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
+            g.w_nt = tiled_w_nt(slots_of(in, h, 0u), g.E, true);
             return launch_group_a4w4_tiled(g, true, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85: encoding %u arm %u is not served", enc, arm);
@@ -468,7 +482,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
                 v.out_bf16 = g.part16; v.slots_hint = slots_of(in, h, 0u);
                 if (v.slots_hint <= W8A8_GEMV_MAX_SLOTS && group_a16_gemv_serves(v)) return launch_group_a16_gemv(v, false, st);
             }
-            return want_tiled(h, slots_of(in, h, 0u), g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
+            { const uint32_t slots_ = slots_of(in, h, 0u); g.w_nt = tiled_w_nt(slots_, g.E, false);
+          return want_tiled(h, slots_, g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st); }
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
                          (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
@@ -500,6 +515,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4);
             g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_A4W4_P16;
+            g.w_nt = tiled_w_nt(slots_of(in, h, 0u), g.E, false);
             return launch_group_a4w4_tiled(g, false, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 86: encoding %u arm %u is not served", enc, arm);
@@ -516,7 +532,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 6);
         g.meta = (const int32_t*)ten(in, T, 3); g.row_token = (const uint32_t*)ten(in, T, 4);
         g.N = I; g.K = H; g.E = E; g.act = i[5]; g.per_channel = 1;
-        return want_tiled(h, slots_of(in, h, 0u), g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st);
+        { const uint32_t slots_ = slots_of(in, h, 0u); g.w_nt = tiled_w_nt(slots_, g.E, true);
+          return want_tiled(h, slots_, g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st); }
     }
     case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8: {
         const uint32_t H = i[0], I = i[1], E = i[2];
@@ -530,7 +547,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 3);
         g.row_partidx = (const uint32_t*)ten(in, T, 4); g.row_gate = (const float*)ten(in, T, 5);
         g.N = H; g.K = I; g.E = E; g.per_channel = 1;
-        return want_tiled(h, slots_of(in, h, 0u), g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st);
+        { const uint32_t slots_ = slots_of(in, h, 0u); g.w_nt = tiled_w_nt(slots_, g.E, false);
+          return want_tiled(h, slots_, g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st); }
     }
     case PLOW_DOP_MOE_GROUP_GLU_FP8_BLK:
     case PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8:

@@ -19,6 +19,7 @@ const PlowMoeTuning& plow_moe_tuning() {
         };
         t.w8a8_kernel = is("PLOW_MOE_W8A8_KERNEL", "stream") ? 0 : is("PLOW_MOE_W8A8_KERNEL", "tiled") ? 1 : -1;
         t.tile_waves4 = is("PLOW_MOE_W8A8_TILE_WAVES", "4");
+        t.tiled_nt = is("PLOW_MOE_TILED_NT", "0") ? 0 : is("PLOW_MOE_TILED_NT", "1") ? 1 : -1;
         const char* d = getenv("PLOW_MOE_SK_DEPTH");
         t.sk_depth = d ? atoi(d) : 3;
         if (t.sk_depth < 2 || t.sk_depth > 4) t.sk_depth = 3;

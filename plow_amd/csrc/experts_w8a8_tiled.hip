@@ -455,6 +455,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     const uint32_t nblk = g.N / 128u;
     struct Tile {
         uint32_t e, nt, r0, rows;
+        uint32_t single;   /* the expert's only row tile: its weight rows are read once */
         uint64_t wp0, wp1; /* weight rows (GLU block mode: gate, up) */
         uint64_t sp0, sp1; /* block mode: their scale tables */
     };
@@ -491,6 +492,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
          * groups: a tile takes nine groups only where that saves a tile; eight-group kernels fill 128-row tiles
          * and leave the rest to the last one */
         const uint32_t Mu = (uint32_t)__builtin_amdgcn_readfirstlane((int)Me);
+        t.single = Mu == 1u ? 1u : 0u;
         const uint32_t h = NG == 8 ? 128u : (((cnt + Mu - 1u) / Mu + 15u) / 16u) * 16u; /* <= cap since cnt <= cap * Me */
         t.r0 = (uint32_t)meta_c[t.e] + mt * h;
         t.rows = cnt - mt * h < h ? cnt - mt * h : h; /* live rows of the tile */
@@ -533,8 +535,10 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             const uint8_t *tsp, *wsp[2];
             const float* ssrc;
             const uint8_t *W0, *W1;
+            uint32_t nt; /* weight rows non-temporal: asked for by the launch and the expert has one row tile */
         };
         const uint8_t* const A0 = (const uint8_t*)g.a;
+        const bool w_nt = __builtin_amdgcn_readfirstlane((int)g.w_nt) != 0;
         /* Set-up of a tile's sources in two halves, so that its loads (row -> token, scales) are in
          * flight while the loader keeps feeding the tile before: fetch() only issues loads, finish()
          * uses them a few blocks later. Rows below the live count always hold a token. */
@@ -593,6 +597,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         auto finish = [&](const Tile& t, const Pre& P, uint32_t par, Src& S) {
             const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
             S.W0 = (const uint8_t*)(uintptr_t)t.wp0;
+            S.nt = (w_nt && t.single) ? 1u : 0u;
             S.nine = (cw < 2u && rows > 128u) ? 1u : 0u;
             S.W1 = !GLU ? S.W0 : PC ? S.W0 + (size_t)g.N * K /* up rows follow the N gate rows */
                                : (const uint8_t*)(uintptr_t)t.wp1;
@@ -684,10 +689,17 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 1u)) ? wk1 : wk0) + S.woff[i]),
                                                      (lds_void*)&L.w[st][(64u * cw + 16u * i) * 64u], 16, 0, 0);
             } else {
+                if (S.nt) { /* the same in every lane; the cache policy is an immediate of the instruction */
 #pragma unroll
-                for (uint32_t i = 0; i < 8u; i++)
-                    __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + S.woff[i]),
-                                                     (lds_void*)&L.w[st][(64u * cw + 8u * i) * 128u], 16, 0, 0);
+                    for (uint32_t i = 0; i < 8u; i++)
+                        __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + S.woff[i]),
+                                                         (lds_void*)&L.w[st][(64u * cw + 8u * i) * 128u], 16, 0, LOAD_NT);
+                } else {
+#pragma unroll
+                    for (uint32_t i = 0; i < 8u; i++)
+                        __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 2u)) ? wk1 : wk0) + S.woff[i]),
+                                                         (lds_void*)&L.w[st][(64u * cw + 8u * i) * 128u], 16, 0, 0);
+                }
             }
         };
         Tile tcur, tnxt;

@@ -88,6 +88,10 @@ struct GroupW8A8 {
      * [..][K / 32]; the GLU writes its output the same way into out / out_e8m0; stab holds E8M0 rows */
     const uint8_t* a_e8m0;
     uint8_t* out_e8m0;
+    /* tiled forms: when non-zero, the weight rows of an expert with a single row tile (read once) are loaded
+     * non-temporal. Right while the launch is bound by the weight stream; from about 64 rows per expert on
+     * average it is bound by what a CU's load path carries and the bit costs time */
+    uint32_t w_nt;
 };
 int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);

@@ -6,6 +6,7 @@
  *   PLOW_MOE_W8A8_KERNEL      stream | tiled   force one form of the fp8 x fp8 grouped GEMMs
  *                                              (default: chosen per op from its row count)
  *   PLOW_MOE_W8A8_TILE_WAVES  4                512-thread form of the tiled kernel (default 768 threads)
+ *   PLOW_MOE_TILED_NT         0 | 1            tiled kernels' weight rows never / always non-temporal (default: by rows per expert)
  *   PLOW_MOE_SK_DEPTH         2..4             k-steps of weight loads in flight, register form (default 3)
  *   PLOW_MOE_SK_GLU           regs             block-mode decode GLU on the register form (default: direct-to-LDS form)
  *   PLOW_MOE_SK_DOWN          regs             block-mode decode DOWN on the register form (default: direct-to-LDS form)
@@ -24,6 +25,7 @@
 struct PlowMoeTuning {
     int w8a8_kernel;      /* -1 auto, 0 stream, 1 tiled */
     bool tile_waves4;
+    int tiled_nt;         /* -1 auto, 0, 1 */
     int sk_depth;         /* 2..4 */
     bool sk_glu_regs;
     bool sk_down_regs;
