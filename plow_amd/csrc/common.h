@@ -148,10 +148,12 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-/* Cache-policy operand of a direct global -> LDS load for bytes that are read once (an expert's weights at
- * decode): non-temporal. Measured on the DeepSeek-V3 decode GLU, 6.37 GB of weights per launch: 1061 -> 967 us
- * (6.0 -> 6.6 TB/s). Not for bytes another workgroup reads again soon (token rows, the prefill kernels' weight
- * rows: there it costs 8 %). */
+/* Cache-policy operand of a direct global -> LDS load for bytes that are read once, in whole 128-byte lines (an
+ * expert's weight rows at decode; at prefill those of an expert whose rows fit one row tile): non-temporal.
+ * Measured on the DeepSeek-V3 decode GLU, 6.37 GB of weights per launch: 1061 -> 967 us (6.0 -> 6.6 TB/s). Not for
+ * bytes that are read again soon (token rows; weight rows that a second row tile of the expert reads: 8 % slower
+ * at 4096 tokens with the bit on all of them) and not for lines that come in piecewise (8 bytes of an E8M0 scale
+ * row a step: every line fetched sixteen times; 64-byte halves a k-step apart: 13 % slower). */
 #define LOAD_NT 2
 
 #endif
