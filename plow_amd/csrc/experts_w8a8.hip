@@ -601,8 +601,8 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
  * read once, whole 128-byte lines per row and block, with non-temporal loads (the register form reads a line as
  * two halves a k-step apart and has to keep it cached: 5.7 TB/s against the 6.6 of the GLU above). Four waves
  * and 128 channels per workgroup: 77 KB of LDS, so a CU holds two workgroups and one's set-up trips to memory
- * (count and pointers, then row maps and block scales) pass under the other's stream. Plain arm only: e4m3 rows
- * by aligned row, f32 or bf16 partials by row_partidx. Rows past the expert's count read its first row with a
+ * (count and pointers, then row maps and block scales) pass under the other's stream. e4m3 rows by aligned row;
+ * f32 or bf16 partials by row_partidx, or the deterministic accumulate. Rows past the expert's count read its first row with a
  * zero scale; a row whose slot is unused is computed and not stored. */
 #define SDD_WAVES 4u
 struct SddLds {
@@ -701,6 +701,12 @@ __global__ __launch_bounds__(SDD_WAVES* WAVE) void k_group_down_w8a8_dma(GroupW8
         const size_t o = (size_t)pidx * N + chw + 4u * q;
         const float y0 = gate * acc0[0], y1 = gate * acc0[1], y2 = gate * acc0[2], y3 = gate * acc0[3];
         const float z0 = gate * acc1[0], z1 = gate * acc1[1], z2 = gate * acc1[2], z3 = gate * acc1[3];
+        if (g.det_k) { /* order-independent: fixed-point f64 atomics into the token's accumulator row */
+            double* const arow = (double*)g.out + (size_t)(pidx / g.det_k) * N + chw + 4u * q;
+            det_add(arow, y0), det_add(arow + 1, y1), det_add(arow + 2, y2), det_add(arow + 3, y3);
+            det_add(arow + 16, z0), det_add(arow + 17, z1), det_add(arow + 18, z2), det_add(arow + 19, z3);
+            continue;
+        }
         if (g.part16) {
             uint2 a, b;
             a.x = (uint32_t)f2bf(y0) | ((uint32_t)f2bf(y1) << 16), a.y = (uint32_t)f2bf(y2) | ((uint32_t)f2bf(y3) << 16);
@@ -760,7 +766,8 @@ int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
     if (rc) return rc;
     const dim3 grid(g.E * (g.N / SK_BN));
     if (g.per_channel) { k_group_w8a8_stream<false, 3, true><<<grid, SK_THREADS, 0, st>>>(g); return 0; }
-    if (g.det_k) { /* deterministic accumulate: its own instantiations */
+    const bool dma_ok = !g.acc_topk && !g.a_slots && !g.a_bf16 && g.K <= 16384u && !plow_moe_tuning().sk_down_regs;
+    if (g.det_k && !dma_ok) { /* deterministic accumulate on the register form: its own instantiations */
         if (g.N % 256u == 0u && !plow_moe_tuning().sk_narrow) {
             k_group_w8a8_stream<false, 3, false, true, false, true><<<dim3(g.E * (g.N / 256u)), SK_THREADS, 0, st>>>(g);
         } else {
@@ -769,7 +776,7 @@ int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st) {
         return 0;
     }
     /* the plain arm on the direct-to-LDS form (the block scales of all of K sit in LDS: K <= 16384) */
-    if (!g.acc_topk && !g.a_slots && !g.a_bf16 && g.K <= 16384u && !plow_moe_tuning().sk_down_regs) {
+    if (dma_ok) {
         k_group_down_w8a8_dma<<<grid, SDD_WAVES * WAVE, sizeof(SddLds), st>>>(g);
         return 0;
     }
