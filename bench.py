@@ -188,7 +188,10 @@ def cpu_baseline(a, name, cfg, dev, mode):
     import oracle_lib as ol
     from plow_amd import abi, layer, synth
     oracle = ol.load_oracle()
-    cores = min(CPU_THREADS_CAP, os.cpu_count() or 1)
+    # worker threads: the CPUs this process may run on, capped at the box's share for one GPU; each worker pinned
+    avail = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(CPU_THREADS_CAP, avail)
+    oracle.plow_oracle_pin_workers(1)
     T = cfg.T
     Tc = T if mode == "full" else min(T, 32)
     ccfg = make_cfg(layer, a, name, Tc)
@@ -206,7 +209,7 @@ def cpu_baseline(a, name, cfg, dev, mode):
     chost.experts = full_host.experts
     cinsts = abi.inst_array(cplan.insts)
     times = []
-    reps = 3
+    reps = 5 if mode == "sample" else 3 if a.steps < 10 else 5
     for rep in range(reps):
         # rep 0: the batch the GPU ran (its first Tc tokens); later reps: fresh activations, fresh routing
         chost.t["x"] = (full_host.t["x"][:Tc].contiguous() if rep == 0
@@ -216,12 +219,16 @@ def cpu_baseline(a, name, cfg, dev, mode):
         rc = oracle.plow_oracle_exec_many(cinsts, len(cinsts), chost.table(), cores)
         times.append(time.perf_counter() - t0)
         assert rc == 0
+    oracle.plow_oracle_pin_workers(0)
     cpu_us = statistics.median(times) * 1e6
     sample = (f"the whole batch of {T} tokens through the whole chain, {reps} repetitions with fresh activations "
               f"and routing each, median" if Tc == T else
               f"first {Tc} of {T} tokens through the whole chain, {reps} repetitions with fresh activations and "
               f"routing, median {cpu_us:.0f} us, scaled by {T}/{Tc} (extrapolated: a sample streams more weight bytes per token)")
-    return {"value": round(cpu_us * T / Tc, 1), "unit": "us/layer", "cores": cores, "kind": "port", "sample": sample}
+    return {"value": round(cpu_us * T / Tc, 1), "unit": "us/layer", "cores": cores, "cores_available": os.cpu_count(),
+            "cores_allowed": avail, "kind": "port",
+            "tier": "scalar restatement of plow's golden CPU kernels (plow's AVX-512 / AMX tiers do not run the block-fp8 arm)",
+            "pinned": True, "reps": reps, "rep_us": [round(t * 1e6, 1) for t in times], "sample": sample}
 
 
 def main():

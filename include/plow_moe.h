@@ -43,9 +43,16 @@ typedef struct {
                       * extension of this library (no MoE op of the reference uses the third immediate):
                       * these ops carry no row count, and the kernel form that serves them best depends on
                       * it. Without it the count is taken from the align op (84) of the same
-                      * plow_moe_exec_many / segment run, then from what the op's own operands imply;
-                      * unknown means few rows. It never changes a result, and nothing is remembered
-                      * between calls. */
+                      * plow_moe_exec_many / segment run, then from what the op's own operands imply,
+                      * then (fp8 x fp8 arms) from the routing meta on the device. Nothing is remembered
+                      * between calls. The count only selects between kernel forms, which agree within
+                      * the layer tolerance but not bit for bit: the tiled GLU takes SiLU from the
+                      * hardware exp2 / reciprocal where the streaming form uses expf and an IEEE
+                      * division (at most one bf16 step on a bf16 intermediate); the matrix-vector DOWN
+                      * (at most 36 slots) adds a row's products in another order than the matrix
+                      * instruction forms; the tiled W8A8 GLU leaves the fq / fs rows of an expert
+                      * whose weights are not resident unwritten where the streaming form zeroes them
+                      * (the bf16 intermediate of op 188 is zero-filled by both). */
     uint16_t t[8];   /* handles into the tensor table; PLOW_TENSOR_NONE = absent => NULL */
     uint32_t i[8];
 } PlowDevInst;
@@ -185,11 +192,23 @@ typedef struct PlowMoeCtx PlowMoeCtx;
  * (crates/plowrt/src/exec/gpu/moe_lt.rs:713-724). */
 uint32_t plow_moe_abi(void);
 
-/* Create / destroy an operator context on HIP device `device`. The context owns a small fixed
- * workspace (routing scratch, the device copy of descriptors); per-call work allocates nothing.
- * Replaces the per-engine load step of moe_lt.rs:697-814. */
+/* Create / destroy an operator context on HIP device `device`. The context owns a fixed workspace
+ * (routing scratch of the slot-major ops) and PLOW_MOE_STAGE_DEFAULT_BYTES of staging for the fp4 x fp4
+ * arm; no op allocates, frees or waits for the device (the ownership contract of
+ * runtime/cpu/dev/cpu_dev.h:5-7). Replaces the per-engine load step of moe_lt.rs:697-814. */
 int  plow_moe_create(PlowMoeCtx** out, int device);
 void plow_moe_destroy(PlowMoeCtx* ctx);
+
+/* Staging of the fp4 x fp4 arm (op 85 at enc 2, arm 0 quantizes its token rows to mxfp4 once, ahead of the
+ * GEMM): rows * (H / 2 + H / 32) bytes, each part rounded up to 256. A context starts with
+ * PLOW_MOE_STAGE_DEFAULT_BYTES (8192 rows of width 7168); an op 85 whose i4 rows do not fit is refused with
+ * PLOW_MOE_EINVAL before anything of its run is launched. This call makes room for `token_rows` rows of
+ * width `hidden`: it allocates (call it at set-up, never under stream capture), keeps every earlier block
+ * until plow_moe_destroy (graphs captured before stay valid) and returns PLOW_MOE_ENOMEM after seven
+ * growths or when the device is out of memory. No counterpart in the reference, which quantizes every
+ * gathered row inside its GEMM kernel (runtime/amd/op_moe.h:3948-4720). */
+#define PLOW_MOE_STAGE_DEFAULT_BYTES (32u << 20)
+int plow_moe_reserve_staging(PlowMoeCtx* ctx, size_t token_rows, size_t hidden);
 
 /* Text of the last failure on this context (valid until the next call on it). */
 const char* plow_moe_last_error(const PlowMoeCtx* ctx);
@@ -224,7 +243,8 @@ int plow_moe_set_min_rows(PlowMoeCtx* ctx, int variant, int min_rows);
 /* plow_moe_exec for callers that cannot allocate. It has no counterpart in the reference: it is for code
  * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc, where even creating a
  * context (which allocates its workspace) is not possible. It takes no context and calls no allocating
- * routine. Every op of plow_moe_exec is served; the ops that need a workspace (slot-major decode experts 48 /
+ * routine. Every op of plow_moe_exec is served except op 85 on the fp4 x fp4 arm (enc 2, arm 0), whose
+ * staging block belongs to a context: it is refused with PLOW_MOE_EUNSUPPORTED. The ops that need a workspace (slot-major decode experts 48 /
  * 49 / 65 / 66, flat mxfp4 150 - 153) take it from a static device array inside the library (1 MiB per GPU,
  * held until the process ends), which limits them to PLOW_MOE_NOALLOC_MAX_SLOTS routed slots and
  * PLOW_MOE_NOALLOC_MAX_EXPERTS experts: larger calls are refused with PLOW_MOE_EINVAL and a text in `err`

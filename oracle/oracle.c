@@ -40,10 +40,12 @@
  * level only): the f32 summation order INSIDE one 128-K block of the fp8 x fp8 arms, which the
  * reference leaves to its MFMA; this file sums a block with eight interleaved f32 partials.
  */
+#define _GNU_SOURCE /* sched_getaffinity, pthread_setaffinity_np */
 #include "oracle.h"
 #include "codec.h"
 
 #include <pthread.h>
+#include <sched.h>
 #include <stdlib.h>
 
 #define TEN(in, T, k) ((in)->t[(k)] == PLOW_TENSOR_NONE ? (void*)0 : (T)[(in)->t[(k)]])
@@ -1393,8 +1395,29 @@ typedef struct {
     uint32_t slice, nblk;
 } Job;
 
+/* Timing runs pin worker s to the s-th CPU the process may run on, as plow's CPU benches do with their
+ * worker pool (runtime/tests/cpu_dev_moe_gemma_test.c:109-155); off by default (tests do not care). */
+static int g_pin_workers = 0;
+void plow_oracle_pin_workers(int on) { g_pin_workers = on; }
+
 static void* job_main(void* p) {
     Job* j = p;
+    if (g_pin_workers) {
+        cpu_set_t allowed, one;
+        if (sched_getaffinity(0, sizeof allowed, &allowed) == 0) {
+            const int n = CPU_COUNT(&allowed);
+            int want = n > 0 ? (int)(j->slice % (uint32_t)n) : -1;
+            for (int c = 0; c < CPU_SETSIZE && want >= 0; c++) {
+                if (!CPU_ISSET(c, &allowed)) continue;
+                if (want-- == 0) {
+                    CPU_ZERO(&one);
+                    CPU_SET(c, &one);
+                    (void)pthread_setaffinity_np(pthread_self(), sizeof one, &one);
+                    break;
+                }
+            }
+        }
+    }
     j->fn(j->in, j->slice, j->nblk, j->T);
     return NULL;
 }

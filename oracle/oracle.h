@@ -16,6 +16,9 @@ extern "C" {
 int plow_oracle_exec(const PlowDevInst* inst, void* const* tensors, uint32_t nthreads);
 int plow_oracle_exec_many(const PlowDevInst* insts, uint32_t n, void* const* tensors, uint32_t nthreads);
 
+/* timing runs: pin worker s to the s-th CPU the process may run on (0 = off, the default) */
+void plow_oracle_pin_workers(int on);
+
 uint16_t plow_oracle_f2bf(float f);
 float    plow_oracle_bf2f(uint16_t h);
 uint8_t  plow_oracle_f32_to_e4m3(float f);

@@ -32,13 +32,16 @@ struct Workspace {
     float* row_gate;
     uint32_t* chunk_hist; /* [max_chunks][max_e] scratch of the multi-workgroup align */
     uint64_t* ftab;       /* [2][max_e][3] pointer tables built for the flat-tensor ops (150 - 153) */
+    uint32_t* form_words; /* [WS_FORM_WORDS] device-side form choices of grouped ops issued without a row count */
 };
+#define WS_FORM_WORDS 64u
 static constexpr size_t ws_up(size_t v) { return (v + 255u) & ~(size_t)255u; }
 static constexpr size_t ws_rows(uint32_t max_e, uint32_t max_slots) { return (size_t)max_slots + (size_t)max_e * (PLOW_MPF_BM - 1u); }
 /* bytes of one workspace laid out in a single 256-byte aligned block */
 static constexpr size_t ws_bytes(uint32_t max_e, uint32_t max_slots) {
     return ws_up((3u * (size_t)max_e + 1u) * 4u) + 3u * ws_up(ws_rows(max_e, max_slots) * 4u) +
-           ws_up((size_t)((max_slots + 1023u) / 1024u) * max_e * 4u) + ws_up((size_t)2u * max_e * 3u * 8u);
+           ws_up((size_t)((max_slots + 1023u) / 1024u) * max_e * 4u) + ws_up((size_t)2u * max_e * 3u * 8u) +
+           ws_up(WS_FORM_WORDS * 4u);
 }
 static_assert(ws_bytes(PLOW_MOE_NOALLOC_MAX_EXPERTS, PLOW_MOE_NOALLOC_MAX_SLOTS) <= PLOW_MOE_STATIC_BYTES,
               "the static device array must hold the workspace of the largest call plow_moe_exec_noalloc accepts");
@@ -52,39 +55,50 @@ static Workspace ws_carve(void* base, uint32_t max_e, uint32_t max_slots) {
     w.row_partidx = (uint32_t*)p, p += rb;
     w.row_gate = (float*)p, p += rb;
     w.chunk_hist = (uint32_t*)p, p += ws_up((size_t)w.max_chunks * max_e * 4u);
-    w.ftab = (uint64_t*)p;
+    w.ftab = (uint64_t*)p, p += ws_up((size_t)2u * max_e * 3u * 8u);
+    w.form_words = (uint32_t*)p;
     return w;
 }
 
+/* Staging of the fp4 x fp4 arm (op 85 at enc 2, arm 0): its token rows, quantized to mxfp4 ahead of the
+ * GEMM. A context is created with PLOW_MOE_STAGE_DEFAULT_BYTES of it and plow_moe_reserve_staging grows it
+ * outside the op path; an op whose batch does not fit is refused before anything is launched. A block
+ * that kernels have been given is never freed before plow_moe_destroy: a graph captured earlier keeps
+ * pointing at memory that is still the context's. */
+#define STAGE_MAX_BLOCKS 8u
 struct PlowMoeCtx {
     int device;
     int min_rows[2]; /* [0] prefill, [1] decode; < 0 unset */
     char err[256];
     void* ws_base;   /* the context's own allocation behind `ws` (NULL when `ws` is borrowed) */
     Workspace ws;
-    /* token rows of the fp4 x fp4 arm's GLU, quantized ahead of its GEMM: grown on demand, kept until
-     * the context is destroyed */
+    uint32_t form_seq; /* the next of the workspace's form words to hand out (they rotate) */
+    void* stage_blocks[STAGE_MAX_BLOCKS]; /* every block ever allocated; the last one is in use */
+    uint32_t n_stage;
     void* stage;
     size_t stage_bytes;
 };
 
-/* Room for `bytes` of staging on the context's device. Growing frees the old block first, which waits for
- * the device: work already queued that reads it finishes before it goes. */
-static int stage_reserve(PlowMoeCtx* c, size_t bytes) {
+/* bytes of staging the fp4 x fp4 GLU needs for `rows` token rows of width H */
+static size_t stage_need(size_t rows, size_t H) { return ws_up(rows * (H / 2u)) + ws_up(rows * (H / 32u)); }
+
+/* A larger staging block on the context's device. Never called from an op: it allocates. The block in use so
+ * far stays allocated (work already queued, or a captured graph, may still read it). */
+static int stage_grow(PlowMoeCtx* c, size_t bytes) {
     if (bytes <= c->stage_bytes) return 0;
+    if (c->n_stage >= STAGE_MAX_BLOCKS) return PLOW_MOE_ENOMEM;
     int prev = 0;
     (void)hipGetDevice(&prev);
     (void)hipSetDevice(c->device);
-    (void)hipFree(c->stage);
-    c->stage = nullptr, c->stage_bytes = 0;
-    const bool ok = hipMalloc(&c->stage, bytes) == hipSuccess;
+    void* p = nullptr;
+    const bool ok = hipMalloc(&p, bytes) == hipSuccess;
     (void)hipSetDevice(prev);
     if (!ok) {
-        c->stage = nullptr;
         (void)hipGetLastError();
         return PLOW_MOE_ENOMEM;
     }
-    c->stage_bytes = bytes;
+    c->stage_blocks[c->n_stage++] = p;
+    c->stage = p, c->stage_bytes = bytes;
     return 0;
 }
 
@@ -131,14 +145,29 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
         return PLOW_MOE_ENOMEM;
     }
     c->ws = ws_carve(c->ws_base, WS_MAX_E, WS_MAX_SLOTS);
+    if (stage_grow(c, PLOW_MOE_STAGE_DEFAULT_BYTES)) {
+        plow_moe_destroy(c);
+        return PLOW_MOE_ENOMEM;
+    }
     *out = c;
+    return 0;
+}
+
+extern "C" int plow_moe_reserve_staging(PlowMoeCtx* ctx, size_t token_rows, size_t hidden) {
+    if (!ctx || !ctx->ws_base) return PLOW_MOE_EINVAL;
+    ctx->err[0] = 0;
+    const size_t need = stage_need(token_rows, hidden);
+    if (need <= ctx->stage_bytes) return 0;
+    const int rc = stage_grow(ctx, need);
+    if (rc) return fail(ctx, rc, "plow_moe_reserve_staging: %zu bytes could not be allocated (a context grows its staging at most %u times; "
+                                 "allocation is refused while a stream capture is active)", need, STAGE_MAX_BLOCKS - 1u);
     return 0;
 }
 
 extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) {
     if (!ctx) return;
     (void)hipFree(ctx->ws_base);
-    (void)hipFree(ctx->stage);
+    for (uint32_t n = 0; n < ctx->n_stage; n++) (void)hipFree(ctx->stage_blocks[n]);
     delete ctx;
 }
 
@@ -194,6 +223,31 @@ static bool want_tiled(const Hint& h, uint32_t slots, const GroupW8A8& g) {
     const int env = plow_moe_tuning().w8a8_kernel;
     const bool tiled = env >= 0 ? env == 1 : h.form >= 0 ? h.form == 1 : slots >= 16u * g.E;
     return tiled && group_w8a8_tiled_serves(g);
+}
+
+/* One fp8 x fp8 grouped op. With a row count (or a form stated by the segment entry points or the
+ * environment) the host picks the form. Without one - a caller that issues its ops one at a time and fills
+ * no fj[2], as plow's interpreter does (runtime/amd/interp.hip:6556-6604) - the count exists only on the
+ * device, in meta: a one-workgroup launch adds it up into a word of the workspace, and both forms are
+ * launched behind it; every workgroup of the form the word does not name returns at once (a few microseconds
+ * per op, where the wrong form costs up to twenty times the op). */
+static int launch_w8a8(PlowMoeCtx* c, const Hint& h, uint32_t slots, GroupW8A8& g, bool glu, hipStream_t st) {
+    g.slots_bound = slots;
+    g.w_nt = tiled_w_nt(slots, g.E, glu);
+    const bool open = slots == 0u && h.form < 0 && plow_moe_tuning().w8a8_kernel < 0 && plow_moe_tuning().form_on_device;
+    if (!open || !group_w8a8_tiled_serves(g)) {
+        if (want_tiled(h, slots, g)) return glu ? launch_group_glu_w8a8_tiled(g, st) : launch_group_down_w8a8_tiled(g, st);
+        return glu ? launch_group_glu_w8a8(g, st) : launch_group_down_w8a8(g, st);
+    }
+    uint32_t* const word = c->ws.form_words + (c->form_seq++ % WS_FORM_WORDS);
+    int rc = launch_pick_form(word, g.meta, g.E, st);
+    if (rc) return rc;
+    g.form_word = word;
+    g.form_want = 0u;
+    rc = glu ? launch_group_glu_w8a8(g, st) : launch_group_down_w8a8(g, st);
+    if (rc) return rc;
+    g.form_want = 1u;
+    return glu ? launch_group_glu_w8a8_tiled(g, st) : launch_group_down_w8a8_tiled(g, st);
 }
 
 static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStream_t st, bool launch, const Hint& h) {
@@ -329,8 +383,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         /* SiLU, or the clamped SwiGLU when a limit is given (plow runtime/amd/op_gemm_common.h:1973-1981) */
         g.f1 = in->fj[1].f; g.act = g.f1 > 0.0f ? PLOW_MOE_ACT_SWIGLU_CLAMP : PLOW_MOE_ACT_SILU;
         /* without a stated slot count: eight slots per token */
-        { const uint32_t slots_ = slots_of(in, h, 8u * Tn); g.w_nt = tiled_w_nt(slots_, g.E, true);
-          return want_tiled(h, slots_, g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st); }
+        return launch_w8a8(c, h, slots_of(in, h, 8u * Tn), g, true, st);
     }
     case PLOW_DOP_MOE_QUANT_FP8_BLOCK128: {
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5),
@@ -356,8 +409,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 5);
         g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
         g.N = H; g.K = I; g.E = E;
-        { const uint32_t slots_ = slots_of(in, h, Tn * topk); g.w_nt = tiled_w_nt(slots_, g.E, false);
-          return want_tiled(h, slots_, g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st); }
+        return launch_w8a8(c, h, slots_of(in, h, Tn * topk), g, false, st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_PF: {
         const uint32_t I = i[0], H = i[1], E = i[2], enc = i[3], arm = i[7];
@@ -379,8 +431,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
             /* without a stated slot count: the row pitch of the activation scales as the token count,
              * eight slots per token */
-            { const uint32_t slots_ = slots_of(in, h, 8u * i[4]); g.w_nt = tiled_w_nt(slots_, g.E, true);
-          return want_tiled(h, slots_, g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st); }
+            return launch_w8a8(c, h, slots_of(in, h, 8u * i[4]), g, true, st);
         }
         if (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ) {
             NEED(c, ten(in, T, 3) && ten(in, T, 7), "op 85 W8A8 (bf16 rows): t3 stab, t7 fs must be bound");
@@ -425,11 +476,14 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             NEED(c, I % 256u == 0u && H % 256u == 0u && I >= 512u && H >= 512u, "op 85 A4W4: I %u and H %u must be multiples of 256, at least 512", I, H);
             NEED(c, i[4] != 0u, "op 85 A4W4: i4 (the number of token rows in t1) is zero");
             NEED(c, i[5] <= 2u || i[5] == PLOW_MOE_ACT_SWIGLU_CLAMP, "op 85: activation %u is not served", i[5]);
+            NEED(c, (uint64_t)slots_of(in, h, 0u) / 128u + E <= 65535u, "op 85 A4W4: %u routed rows over %u experts exceed the 65535 row tiles the tiled kernel's directory counts", slots_of(in, h, 0u), E);
             if (!c->ws_base) return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85 A4W4: needs a context (its staging block)");
+            /* nothing is allocated here: the batch fits the context's staging or the op is refused */
+            NEED(c, stage_need(i[4], H) <= c->stage_bytes,
+                 "op 85 A4W4: %u token rows of width %u need %zu bytes of staging, the context holds %zu: call plow_moe_reserve_staging first",
+                 i[4], H, stage_need(i[4], H), c->stage_bytes);
             if (!launch) return 0;
-            const size_t qbytes = ws_up((size_t)i[4] * (H / 2u)), sbytes = ws_up((size_t)i[4] * (H / 32u));
-            const int src = stage_reserve(c, qbytes + sbytes);
-            if (src) return fail(c, src, "op 85 A4W4: %zu bytes of staging could not be allocated", qbytes + sbytes);
+            const size_t qbytes = ws_up((size_t)i[4] * (H / 2u));
             uint8_t* const xq4 = (uint8_t*)c->stage;
             uint8_t* const xs = xq4 + qbytes;
             const int qrc = launch_quant_mx_act(xq4, xs, ten(in, T, 1), i[4], H, st);
@@ -442,7 +496,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.row_partidx = (const uint32_t*)ten(in, T, 6);
             g.N = I; g.K = H; g.E = E; g.act = i[5]; g.T = i[4];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
-            g.w_nt = tiled_w_nt(slots_of(in, h, 0u), g.E, true);
+            g.slots_bound = slots_of(in, h, 0u);
+            g.w_nt = tiled_w_nt(g.slots_bound, g.E, true);
             return launch_group_a4w4_tiled(g, true, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 85: encoding %u arm %u is not served", enc, arm);
@@ -482,8 +537,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
                 v.out_bf16 = g.part16; v.slots_hint = slots_of(in, h, 0u);
                 if (v.slots_hint <= W8A8_GEMV_MAX_SLOTS && group_a16_gemv_serves(v)) return launch_group_a16_gemv(v, false, st);
             }
-            { const uint32_t slots_ = slots_of(in, h, 0u); g.w_nt = tiled_w_nt(slots_, g.E, false);
-          return want_tiled(h, slots_, g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st); }
+            return launch_w8a8(c, h, slots_of(in, h, 0u), g, false, st);
         }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
                          (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
@@ -507,6 +561,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             /* fp4 on both operands: t1 the mxfp4 rows and t5 the E8M0 rows that op 85 wrote */
             NEED(c, ten(in, T, 3) && ten(in, T, 5), "op 86 A4W4: t3 stab and t5 E8M0 rows must be bound");
             NEED(c, I % 256u == 0u && H % 256u == 0u && I >= 512u && H >= 512u, "op 86 A4W4: I %u and H %u must be multiples of 256, at least 512", I, H);
+            NEED(c, (uint64_t)slots_of(in, h, 0u) / 128u + E <= 65535u, "op 86 A4W4: %u routed rows over %u experts exceed the 65535 row tiles the tiled kernel's directory counts", slots_of(in, h, 0u), E);
             if (!launch) return 0;
             GroupW8A8 g = {};
             g.out = ten(in, T, 0);
@@ -515,7 +570,8 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4);
             g.row_partidx = (const uint32_t*)ten(in, T, 6); g.row_gate = (const float*)ten(in, T, 7);
             g.N = H; g.K = I; g.E = E; g.part16 = arm == PLOW_MOE_ARM_A4W4_P16;
-            g.w_nt = tiled_w_nt(slots_of(in, h, 0u), g.E, false);
+            g.slots_bound = slots_of(in, h, 0u);
+            g.w_nt = tiled_w_nt(g.slots_bound, g.E, false);
             return launch_group_a4w4_tiled(g, false, st);
         }
         return fail(c, PLOW_MOE_EUNSUPPORTED, "op 86: encoding %u arm %u is not served", enc, arm);
@@ -532,8 +588,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.wtab = (const uint64_t*)ten(in, T, 2); g.stab = (const uint64_t*)ten(in, T, 6);
         g.meta = (const int32_t*)ten(in, T, 3); g.row_token = (const uint32_t*)ten(in, T, 4);
         g.N = I; g.K = H; g.E = E; g.act = i[5]; g.per_channel = 1;
-        { const uint32_t slots_ = slots_of(in, h, 0u); g.w_nt = tiled_w_nt(slots_, g.E, true);
-          return want_tiled(h, slots_, g) ? launch_group_glu_w8a8_tiled(g, st) : launch_group_glu_w8a8(g, st); }
+        return launch_w8a8(c, h, slots_of(in, h, 0u), g, true, st);
     }
     case PLOW_DOP_MOE_GROUP_DOWN_GEMMA_PF_W8A8: {
         const uint32_t H = i[0], I = i[1], E = i[2];
@@ -547,8 +602,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 3);
         g.row_partidx = (const uint32_t*)ten(in, T, 4); g.row_gate = (const float*)ten(in, T, 5);
         g.N = H; g.K = I; g.E = E; g.per_channel = 1;
-        { const uint32_t slots_ = slots_of(in, h, 0u); g.w_nt = tiled_w_nt(slots_, g.E, false);
-          return want_tiled(h, slots_, g) ? launch_group_down_w8a8_tiled(g, st) : launch_group_down_w8a8(g, st); }
+        return launch_w8a8(c, h, slots_of(in, h, 0u), g, false, st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_FP8_BLK:
     case PLOW_DOP_MOE_EXPERT_GLU_GEMMA_FP8:

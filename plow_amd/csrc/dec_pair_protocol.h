@@ -13,7 +13,14 @@
  * adding 1 to word 2; the item that brings word 2 to the expert's total zeroes words 0 and 2. Nothing can
  * touch the words after that, because every other item of the expert has already made its last access
  * (its own add to word 2), so the scratch is left zeroed whether or not a wait gave up. Words 1 and 3 are
- * never written. */
+ * never written.
+ *
+ * Ordering. The argument above needs an item's add to word 0 to be performed before its add to word 2, and
+ * the last item's two reset stores after every other item's accesses; the words are different addresses, so
+ * relaxed atomics alone would not order them. The kernel's add to word 2 is therefore an acquire-release
+ * operation at device scope (release for every item, acquire for the one that resets). The CPU model walks
+ * the items with every access as one sequentially consistent step: it checks the counting, not the memory
+ * model. */
 #ifndef PLOW_DEC_PAIR_PROTOCOL_H
 #define PLOW_DEC_PAIR_PROTOCOL_H
 

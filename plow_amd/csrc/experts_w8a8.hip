@@ -370,7 +370,7 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_w8a8_stream(GroupW8A8 g) {
      * segment that needs several passes, so it must start early instead of forming the tail */
     const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles;
     const uint32_t cnt = (uint32_t)g.meta[g.E + e];
-    if (cnt == 0u) return;
+    if (cnt == 0u || !form_is_mine(g)) return;
     const uint32_t r0 = (uint32_t)g.meta[e];
     const bool bf16_mid = GLU && (PC || g.out_bf16); /* the GLU owns every row of its 64-row tiles */
     const uint32_t padded = ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
@@ -448,8 +448,9 @@ __global__ __launch_bounds__(SK_THREADS) void k_group_glu_w8a8_dma(GroupW8A8 g) 
     const uint32_t r0 = (uint32_t)g.meta[e];
     const uint64_t wp0 = g.wtab[(size_t)e * 3u], wp1 = g.wtab[(size_t)e * 3u + 1u];
     const uint64_t sp0 = g.stab[(size_t)e * 3u], sp1 = g.stab[(size_t)e * 3u + 1u];
+    const bool mine = form_is_mine(g);
     asm volatile("" ::"s"(r0), "s"(wp0), "s"(wp1), "s"(sp0), "s"(sp1)); /* the loads stay above the branch */
-    if (cnt == 0u) return;
+    if (cnt == 0u || !mine) return;
     const uint32_t padded = ((cnt + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
     if (wp0 == 0ull || (g.out_bf16 && wp1 == 0ull)) { /* not resident; the bf16 form zeroes what it cannot compute */
         if (g.out_bf16)
@@ -617,8 +618,9 @@ __global__ __launch_bounds__(SDD_WAVES* WAVE) void k_group_down_w8a8_dma(GroupW8
     const uint32_t cnt = (uint32_t)g.meta[g.E + e];
     const uint32_t r0 = (uint32_t)g.meta[e];
     const uint64_t wp = g.wtab[(size_t)e * 3u + 2u], sp = g.stab[(size_t)e * 3u + 2u];
+    const bool mine = form_is_mine(g);
     asm volatile("" ::"s"(r0), "s"(wp), "s"(sp)); /* the loads stay above the branch */
-    if (cnt == 0u || wp == 0ull) return;
+    if (cnt == 0u || wp == 0ull || !mine) return;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, 32-byte chunk q */
@@ -728,6 +730,24 @@ int plow_moe_w8a8_setup() {
                                (int)sizeof(SddLds)) == hipSuccess ? 0 : PLOW_MOE_EDEVICE;
 }
 
+/* The device-side choice between the streaming and the tiled form of a grouped op whose caller states no row
+ * count: one workgroup adds up the experts' row counts. */
+__global__ __launch_bounds__(256) void k_pick_form(uint32_t* word, const int32_t* meta, uint32_t E) {
+    __shared__ uint32_t part[4];
+    uint32_t s = 0;
+    for (uint32_t e = threadIdx.x; e < E; e += 256u) s += (uint32_t)meta[E + e];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    if ((threadIdx.x & 63u) == 0u) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0u) *word = (part[0] + part[1] + part[2] + part[3] >= 16u * E) ? 1u : 0u;
+}
+int launch_pick_form(uint32_t* word, const int32_t* meta, uint32_t E, hipStream_t st) {
+    if (!word || !meta || !E) return PLOW_MOE_EINVAL;
+    k_pick_form<<<1, 256, 0, st>>>(word, meta, E);
+    return 0;
+}
+
 static int check_w8a8(const GroupW8A8& g) {
     if (g.N == 0 || g.K == 0 || g.E == 0) return PLOW_MOE_EINVAL;
     if (g.N % SK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
@@ -749,7 +769,9 @@ int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st) {
         k_group_w8a8_stream<true, 3, false, false, true><<<grid, SK_THREADS, 0, st>>>(g);
         return 0;
     }
-    if (!tune.sk_glu_regs) {
+    /* the direct-to-LDS form keeps the block scales of all of K in LDS (K <= 16384); longer rows take the
+     * register form, which reads them as it goes */
+    if (!tune.sk_glu_regs && g.K <= 16384u) {
         k_group_glu_w8a8_dma<<<grid, SK_THREADS, sizeof(SdLds), st>>>(g);
         return 0;
     }

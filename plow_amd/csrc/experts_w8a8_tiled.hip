@@ -58,6 +58,7 @@ __device__ __forceinline__ float t5_glu(float gt, float up, uint32_t act, float 
 #define T5_BM 144u /* rows the LDS plan holds per tile: nine 16-row groups (kernels built for eight use 128) */
 #define T5_AS 192u /* row slots of a stage's scale array (three loaders x 64 lanes) */
 #define T5_STAGES 3u
+#define T5_MAX_ROW_TILES 65535u /* what the 16-bit tile directory counts */
 #define T5_NLOAD 13 /* direct loads per loader and block: 1 scale, 4 token-row, 8 weight-row; loaders 0 and 1 one more
                      * token-row load (the ninth group) */
 
@@ -385,6 +386,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     const uint32_t NT = (g.N + BN - 1u) / BN;
     const uint32_t r16 = lane & 15u, q = lane >> 4;
 
+    if (!form_is_mine(g)) return; /* the device-side choice named the streaming form: the same in every workgroup */
     /* rows a tile may hold */
     const uint32_t cap = 16u * (uint32_t)NG;
     /* ---- tile directory: inclusive prefix of ceil(cnt / cap) over experts, in LDS (the scan
@@ -407,6 +409,10 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             carry += scan[NTHR - 1u];
             __syncthreads();
         }
+        /* the directory holds 16-bit counts: a batch with more row tiles than that (some 8 million routed rows)
+         * is not served. The launchers refuse it where the host knows the row count; a count only the device
+         * knows ends every workgroup here, before anything is written. */
+        if (carry > T5_MAX_ROW_TILES) return;
     }
     if (GLU && !PC && g.out_bf16) {
         /* bf16 intermediate: the padded rows of an expert whose gate or up weights are not resident are
@@ -1142,11 +1148,16 @@ static int launch_tiled_t(const GroupW8A8& g, hipStream_t st) {
     return 0;
 }
 
+/* Row tiles of a batch of `slots_bound` routed rows never exceed slots / 128 + E (every expert's last tile may be
+ * partial); 0 = the host does not know the count and the kernel checks the real one. */
+static bool t5_row_tiles_fit(const GroupW8A8& g) {
+    return (uint64_t)g.slots_bound / 128u + g.E <= T5_MAX_ROW_TILES;
+}
 /* The shapes the tiled form serves: the tile keeps K / 128 block scales in LDS and the load ring runs
  * two blocks ahead. Callers fall back to the streaming form otherwise. */
 bool group_w8a8_tiled_serves(const GroupW8A8& g) {
     return g.N != 0u && g.E != 0u && g.E <= 1056u && g.N % 128u == 0u && g.K % 128u == 0u && g.K >= 256u &&
-           g.K <= 128u * 128u && g.N >= 256u;
+           g.K <= 128u * 128u && g.N >= 256u && t5_row_tiles_fit(g);
 }
 
 /* Tiles of nine 16-row groups (144 rows) instead of eight: the ninth group saves an expert with 129..144
@@ -1168,7 +1179,8 @@ static int launch_tiled(const GroupW8A8& g, hipStream_t st) {
 }
 
 int launch_group_a4w4_tiled(const GroupW8A8& g, bool glu, hipStream_t st) {
-    if (!g.N || !g.E || g.E > 1056u || g.N % 128u || g.N < 256u || g.K % 256u || g.K < 512u || g.K > 256u * 128u)
+    if (!g.N || !g.E || g.E > 1056u || g.N % 128u || g.N < 256u || g.K % 256u || g.K < 512u || g.K > 256u * 128u ||
+        !t5_row_tiles_fit(g))
         return PLOW_MOE_EINVAL;
     const uint32_t n_cu = plow_moe_n_cu();
     if (!n_cu) return PLOW_MOE_EDEVICE;

@@ -92,7 +92,26 @@ struct GroupW8A8 {
      * non-temporal. Right while the launch is bound by the weight stream; from about 64 rows per expert on
      * average it is bound by what a CU's load path carries and the bit costs time */
     uint32_t w_nt;
+    /* Form chosen on the device: when form_word is set, the launch runs only if *form_word == form_want and
+     * every workgroup of it returns at once otherwise. The host then launches both forms of the op behind
+     * launch_pick_form, which writes the word from the routed rows in meta (0 streaming, 1 tiled). */
+    const uint32_t* form_word;
+    uint32_t form_want;
+    /* tiled forms: an upper bound of the batch's routed rows when the host knows one (0 = unknown). Their tile
+     * directory counts row tiles in 16 bits; a batch that may exceed that is refused by the launcher */
+    uint32_t slots_bound;
 };
+#if defined(__HIPCC__)
+/* whether this launch is the form the device-side choice names (always, when the launch carries no choice) */
+__device__ __forceinline__ bool form_is_mine(const GroupW8A8& g) {
+    uint32_t form = g.form_want;
+    if (g.form_word) form = *(const __attribute__((address_space(4))) uint32_t*)g.form_word; /* written by an earlier kernel: a scalar load */
+    return form == g.form_want;
+}
+#endif
+/* *word = 1 when meta counts at least 16 routed rows per expert on average (the tiled forms' side of the
+ * measured crossover), else 0 */
+int launch_pick_form(uint32_t* word, const int32_t* meta, uint32_t E, hipStream_t st);
 int launch_group_glu_w8a8(const GroupW8A8& g, hipStream_t st);
 int launch_group_down_w8a8(const GroupW8A8& g, hipStream_t st);
 /* the many-rows-per-expert form of the same two ops (block mode only) */

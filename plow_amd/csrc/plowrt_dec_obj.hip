@@ -66,7 +66,9 @@ __device__ __forceinline__ bool dec_down_ok(const DecDownArgs& a) {
 
 /* The pair kernel's counters and its bounded wait: dec_pair_protocol.h. */
 __device__ __forceinline__ void dec_item_done(unsigned* mine, uint32_t glu_items, uint32_t down_items) {
-    const uint32_t before = __hip_atomic_fetch_add(mine + DP_ITEMS_DONE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    /* release: this item's earlier accesses to the words (its add to word 0, its polls) are ordered before the
+     * add; acquire: the item that sees the full count, and resets, is ordered after every other item's */
+    const uint32_t before = __hip_atomic_fetch_add(mine + DP_ITEMS_DONE, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     if (dp_is_last(before, glu_items, down_items)) { /* every other item of the expert has made its last access */
         __hip_atomic_store(mine + DP_GLU_DONE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(mine + DP_ITEMS_DONE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

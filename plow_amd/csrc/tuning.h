@@ -16,6 +16,8 @@
  *                                              the vector-unit kernels at prefill sizes
  *   PLOW_MOE_A16_TILED        0                keep the bf16-activation arms on the streaming kernels at every row count
  *   PLOW_MOE_A16_GEMV         0                keep the bf16-activation arms off the matrix-vector form at a few tokens
+ *   PLOW_MOE_FORM_ON_DEVICE   0                a grouped fp8 x fp8 op without a row count runs the streaming form
+ *                                              (default: both forms are launched behind a choice made on the device)
  */
 #ifndef PLOW_MOE_TUNING_H
 #define PLOW_MOE_TUNING_H
@@ -35,6 +37,7 @@ struct PlowMoeTuning {
     bool score_valu;
     bool a16_tiled;
     bool a16_gemv;
+    bool form_on_device;
 };
 const PlowMoeTuning& plow_moe_tuning();
 

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(HERE, "libplow_moe_gfx950.so")
 
 EXPORTS = ["plow_moe_abi", "plow_moe_create", "plow_moe_destroy", "plow_moe_last_error",
            "plow_moe_exec", "plow_moe_exec_many", "plow_moe_pf", "plow_moe_dec",
-           "plow_moe_set_min_rows", "plow_moe_check", "plow_moe_exec_noalloc"]
+           "plow_moe_set_min_rows", "plow_moe_check", "plow_moe_exec_noalloc", "plow_moe_reserve_staging"]
 
 _lib = None
 
@@ -49,6 +49,7 @@ def load():
     lib.plow_moe_set_min_rows.argtypes = [C.c_void_p, C.c_int, C.c_int]
     lib.plow_moe_exec_noalloc.argtypes = [I, P(C.c_void_p), C.c_void_p, C.c_char_p, C.c_size_t]
     lib.plow_moe_exec_noalloc.restype = C.c_int
+    lib.plow_moe_reserve_staging.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t]
     _lib = lib
     return lib
 
@@ -99,6 +100,10 @@ class Moe:
     def dec(self, insts, table, rows, stream=None):
         arr = abi.inst_array(insts)
         return self._ck(self.lib.plow_moe_dec(self.h, arr, len(arr), table, rows, stream), allow=(abi.ROLLBACK,))
+
+    def reserve_staging(self, token_rows, hidden):
+        """Room for the fp4 x fp4 arm's quantized token rows (allocates: set-up time only)."""
+        return self._ck(self.lib.plow_moe_reserve_staging(self.h, token_rows, hidden))
 
     def set_min_rows(self, variant, min_rows):
         return self._ck(self.lib.plow_moe_set_min_rows(self.h, variant, min_rows))

@@ -22,6 +22,8 @@ def load_oracle():
     lib.plow_oracle_exec_many.argtypes = [C.POINTER(abi.PlowDevInst), C.c_uint32,
                                           C.POINTER(C.c_void_p), C.c_uint32]
     lib.plow_oracle_exec_many.restype = C.c_int
+    lib.plow_oracle_pin_workers.argtypes = [C.c_int]
+    lib.plow_oracle_pin_workers.restype = None
     lib.plow_oracle_f2bf.argtypes = [C.c_float]
     lib.plow_oracle_f2bf.restype = C.c_uint16
     lib.plow_oracle_bf2f.argtypes = [C.c_uint16]

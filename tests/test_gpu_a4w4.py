@@ -152,6 +152,21 @@ def test_a4w4_refusals(moe):
     bad = clone(down)
     bad.i[7] = 2   # the block-fp8 arm's number under the mxfp4 encoding
     assert moe.check(bad, dev.table()) == abi.E_UNSUPPORTED
+    # the tiled kernel's directory counts row tiles in 16 bits: a stated row count that may exceed it is refused
+    for op in (glu, down):
+        bad = clone(op)
+        bad.fj[2].u = 128 * 65535
+        assert moe.check(bad, dev.table()) == abi.E_INVAL and "row tiles" in moe.last_error()
+    # the staging of the quantized token rows belongs to the context and no op grows it: a batch beyond it is
+    # refused before launch, and served once the caller has made room
+    from plow_amd.lib import Moe
+    own = Moe(0)
+    big = clone(glu)
+    big.i[1], big.i[4] = 7168, 20000                                # 76 MB of staging; a new context holds 32 MiB
+    assert own.check(big, dev.table()) == abi.E_INVAL and "plow_moe_reserve_staging" in own.last_error()
+    assert own.reserve_staging(20000, 7168) == 0
+    assert own.check(big, dev.table()) == 0
+    own.close()
     # the entry point that allocates nothing has no staging block
     err = C.create_string_buffer(256)
     rc = moe.lib.plow_moe_exec_noalloc(C.byref(glu), dev.table(), None, err, 256)

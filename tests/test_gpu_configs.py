@@ -54,6 +54,29 @@ def test_c4_kimi_k2_mxfp4_decode(moe, oracle, B):
     assert_output_close(dev.np("out"), host.np("out"), f"c4 B={B} out")
 
 
+def print_popularity(cnt, T, k, s=1.2):
+    """The realised expert popularity (share of the tokens that chose the expert, experts sorted by it) next to
+    what Zipf(s) gives: k experts drawn without replacement with weights rank^-s (10000 seeded draws by the
+    Gumbel top-k construction). The configuration reaches its popularity through a selection bias added to the
+    router's scores, not by sampling, so the two agree in shape (a hot head, a long thin tail), not in law."""
+    E = len(cnt)
+    r = np.random.default_rng(12)
+    w = np.log(np.arange(1, E + 1, dtype=np.float64) ** -s)
+    draws = np.argsort(-(w[None, :] + r.gumbel(size=(10000, E))), axis=1)[:, :k]
+    want = np.bincount(draws.reshape(-1), minlength=E) / 10000.0
+    got = np.sort(np.asarray(cnt, np.float64))[::-1] / T
+    ranks = [n for n in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128) if n <= E]
+    print(f"[popularity] T={T} k={k}: share of tokens per expert by popularity rank, realised | Zipf({s})", flush=True)
+    print("[popularity] " + "  ".join(f"r{n}: {got[n - 1]:.3f}|{want[n - 1]:.3f}" for n in ranks), flush=True)
+    live = got > 0
+    if live.sum() >= 8:
+        lr = np.log(np.arange(1, E + 1))[live]
+        slope = np.polyfit(lr[3:], np.log(got[live])[3:], 1)[0]
+        slope_w = np.polyfit(np.log(np.arange(1, E + 1))[3:], np.log(np.maximum(want, 1e-9))[3:], 1)[0]
+        print(f"[popularity] log-log slope beyond rank 3: realised {slope:.2f}, Zipf({s}) drawn without replacement {slope_w:.2f}; "
+              f"experts hit {int(live.sum())}/{E}", flush=True)
+
+
 def c5_config(T, arm):
     """Qwen3-shaped per-channel fp8 with the expert popularity the configuration asks for: a selection
     bias falling off like Zipf(1.2) over a seeded permutation of the experts."""
@@ -83,6 +106,7 @@ def test_c5_qwen3_per_channel_fp8_prefill_sizes(moe, oracle, T):
     dev = synth.bind(plan, "cuda", seed=0, zipf=1.2)
     run_device(moe, plan, dev)
     cnt = check_prefill_sampled(oracle, cfg, plan, dev)
+    print_popularity(cnt[:cfg.E], T, cfg.k)
     assert cnt.max() >= 0.9 * T          # Zipf(1.2): the most popular expert is chosen by (nearly) every token
 
 

@@ -19,6 +19,13 @@ def moe():
     m.close()
 
 
+# Share of the intermediate's e4m3 bytes that must equal the oracle's. A byte differs where the f32 sum of a
+# 128-k block, added in the matrix instruction's order here and in index order there, lands on the other side
+# of an e4m3 rounding boundary, or where the row's amax (and with it the scale) differs in its last bit. The
+# floor is set a little under the smallest share measured over this file's cases (printed by every case).
+FQ_SAME_FLOOR = 0.98
+
+
 def check_layer(plan, dev, host):
     cfg = plan.cfg
     rows = assert_routing_equal(plan, dev, host)
@@ -32,7 +39,7 @@ def check_layer(plan, dev, host):
     fsd, fsh = dev.np("fs")[:rows][live], host.np("fs")[:rows][live]
     same = (fqd == fqh).mean()
     print(f"[parity] fq bytes identical on {same * 100:.3f} % of live elements", flush=True)
-    assert same > 0.98
+    assert same > FQ_SAME_FLOOR
     assert np.allclose(fsd, fsh, rtol=1e-4)
     pd, ph = dev.np("part"), host.np("part")
     assert np.all(np.isfinite(pd))
@@ -126,6 +133,46 @@ def test_pair_form_activations(moe, oracle, T, act, f):
     cfg = layer.MoeConfig("mini-act", H=512, E=8, I=256, k=2, T=T, scoring="sigmoid", norm_topk=True,
                           bias=True, enc="fp8blk", arm="w8a8", n_shared=1, shared_mode="fold", act=act, act_f=f)
     check_layer(*both(moe, oracle, cfg, seed=T + act))
+
+
+def test_rows_longer_than_the_lds_scale_table(moe, oracle):
+    """H = 16512 (129 blocks of 128 k): the direct-to-LDS GLU keeps a tile's weight block scales of all of K in
+    an LDS table of 128 entries, so this shape must take the register form, which reads them as it goes (the
+    tiled form does not serve it either); streaming row counts and tiled ones."""
+    for T in (3, 80):
+        print(f"[case] w8a8 long rows T={T}", flush=True)
+        cfg = layer.MoeConfig("long-k", H=16512, E=4, I=256, k=2, T=T, scoring="sigmoid", norm_topk=True,
+                              bias=True, enc="fp8blk", arm="w8a8", n_shared=1, shared_mode="fold")
+        check_layer(*both(moe, oracle, cfg, seed=T))
+
+
+@pytest.mark.parametrize("enc,T,E,k", [("fp8blk", 600, 8, 2), ("fp8blk", 24, 8, 2), ("fp8pc", 640, 8, 4), ("fp8pc", 20, 8, 4)])
+def test_ops_issued_alone_pick_their_form_on_the_device(moe, enc, T, E, k):
+    """A caller that issues the ops one at a time and states no row count (plow's interpreter,
+    runtime/amd/interp.hip:6556-6604): ops 86 / 81 / 82 know their rows only from meta, on the device. Both
+    forms are launched behind a choice made there; the bytes must be those of the run that states the count
+    (same form, same kernel), at tiled and at streaming row counts."""
+    from plow_amd import synth
+    print(f"[case] form on device enc={enc} T={T}", flush=True)
+    shared = dict(n_shared=1, shared_mode="fold") if enc == "fp8blk" else {}
+    cfg = layer.MoeConfig("alone", H=512, E=E, I=256, k=k, T=T, scoring="softmax", norm_topk=True, enc=enc, arm="w8a8", **shared)
+    plan = layer.plan_layer(cfg)
+    assert T * cfg.k_all > 36                                     # beyond the matrix-vector form, which only a stated count selects
+    want = synth.bind(plan, "cuda", seed=T)
+    moe.exec_many(plan.insts, want.table())
+    torch.cuda.synchronize()
+    got = synth.bind(plan, "cuda", seed=T)
+    for d in plan.insts:
+        d.fj[2].u = 0
+        moe.exec(d, got.table())
+    torch.cuda.synchronize()
+    for name in ("meta", "part", "out") + (("fq", "fs") if enc == "fp8blk" else ("fu", "fu8")):
+        rows = int(want.np("meta")[3 * cfg.E_all]) * abi.MPF_BM
+        a, b = want.np(name), got.np(name)
+        if name in ("fq", "fs", "fu", "fu8"):
+            a, b = a[:rows], b[:rows]
+        assert a.tobytes() == b.tobytes(), name
+    assert np.isfinite(ol.bf2f(got.np("out"))).all()
 
 
 def test_rows_per_expert_beyond_one_tile(moe, oracle):
