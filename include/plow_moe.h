@@ -154,7 +154,11 @@ enum {
     PLOW_MOE_ARM_W8A8_P16  = 3, /* DOWN only: as 2 with a bf16 part                                */
     PLOW_MOE_ARM_W8A8_XQ   = 6, /* GLU only, enc 1: t1 holds the bf16 rows, quantized 1x128 where they
                                    are loaded; equals op 184 + arm 2 bit for bit, writes arm 2's fq / fs
-                                   (runtime/amd/moe_pf_w8a8.h:118-121); t6 and i4 unused              */
+                                   (runtime/amd/moe_pf_w8a8.h:118-121); t6 unused. i4 is unused by the
+                                   reference; here a non-zero i4 states the rows of t1, which lets a batch
+                                   of many rows per expert run as quantizer + tiled arm 2 over the
+                                   context's staging (see plow_moe_reserve_staging: rows * (H + H / 32)
+                                   bytes); 0, or rows that do not fit, keep the streaming form         */
     PLOW_MOE_ARM_W4A16     = 8
 };
 

@@ -382,8 +382,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.N = I; g.K = H; g.E = E; g.pitch = Tn; g.T = Tn;
         /* SiLU, or the clamped SwiGLU when a limit is given (plow runtime/amd/op_gemm_common.h:1973-1981) */
         g.f1 = in->fj[1].f; g.act = g.f1 > 0.0f ? PLOW_MOE_ACT_SWIGLU_CLAMP : PLOW_MOE_ACT_SILU;
-        /* without a stated slot count: eight slots per token */
-        return launch_w8a8(c, h, slots_of(in, h, 8u * Tn), g, true, st);
+        return launch_w8a8(c, h, slots_of(in, h, 0u), g, true, st);
     }
     case PLOW_DOP_MOE_QUANT_FP8_BLOCK128: {
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2) && ten(in, T, 3) && ten(in, T, 4) && ten(in, T, 5),
@@ -429,9 +428,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.pitch = i[4]; g.act = i[5];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
-            /* without a stated slot count: the row pitch of the activation scales as the token count,
-             * eight slots per token */
-            return launch_w8a8(c, h, slots_of(in, h, 8u * i[4]), g, true, st);
+            return launch_w8a8(c, h, slots_of(in, h, 0u), g, true, st);
         }
         if (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ) {
             NEED(c, ten(in, T, 3) && ten(in, T, 7), "op 85 W8A8 (bf16 rows): t3 stab, t7 fs must be bound");
@@ -445,6 +442,24 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.meta = (const int32_t*)ten(in, T, 4); g.row_token = (const uint32_t*)ten(in, T, 5);
             g.N = I; g.K = H; g.E = E; g.act = i[5];
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
+            /* Many rows per expert, the caller states the rows of t1 in i4 (an extension of this library: the
+             * reference leaves i4 unused on this arm) and the context's staging holds them: the rows are
+             * quantized once, ahead of the GEMM, into the staging block, and the tiled form of arm 2 runs over
+             * them - the arm's definition (quantizer op followed by arm 2, bit for bit), where the streaming
+             * form would quantize every gathered row again in each of the expert's channel tiles. */
+            const uint32_t Tn = i[4], slots = slots_of(in, h, 0u);
+            const size_t qbytes = ws_up((size_t)Tn * H), sbytes = ws_up((size_t)Tn * (H / 128u) * 4u);
+            if (Tn && c->ws_base && qbytes + sbytes <= c->stage_bytes) {
+                GroupW8A8 t = g;
+                t.a = c->stage; t.a_scale = (const float*)((uint8_t*)c->stage + qbytes); t.a_bf16 = 0; t.pitch = Tn; t.T = Tn;
+                if (want_tiled(h, slots, t)) {
+                    const int qrc = launch_quant_block128(c->stage, ten(in, T, 1), (float*)((uint8_t*)c->stage + qbytes), Tn, H, Tn, st);
+                    if (qrc) return qrc;
+                    t.slots_bound = slots;
+                    t.w_nt = tiled_w_nt(slots, t.E, true);
+                    return launch_group_glu_w8a8_tiled(t, st);
+                }
+            }
             /* the streaming form serves this arm at every row count */
             return launch_group_glu_w8a8(g, st);
         }

@@ -286,6 +286,43 @@ __device__ __forceinline__ v2i ds_read8(uint32_t addr) {
     T5A_GROUP_N(7, N) T5A_SCALE_N(6, N)                                                                      \
     T5A_GROUP_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0) T5A_SCALE_N(7, N)                                        \
     T5A_SCALE_N((N) > 8 ? 8 : 0, (N) > 8 ? (N) : 0)
+/* ---- the same block with bf16 weights (W16): a weight row is 128 bytes of bf16 per 64-k block, in the token
+ *      rows' geometry and swizzle, read as the operand it is; no scales anywhere, the accumulators run straight
+ *      through K ---- */
+#define T5W_BLOCK_HEAD()                                                                                     \
+    const uint32_t ab = a_base + st * (uint32_t)sizeof(L.a[0]), wb = w_base + st * (256u * 128u) + cw * (32u * 128u);  \
+    const uint32_t b0 = ab + opb0, b1 = ab + opb1;
+#define T5W_GROUP_N(RG, N)                                                                                   \
+    if ((RG) < (N)) {                                                                                        \
+        asm volatile("s_waitcnt lgkmcnt(%2)"                                                                 \
+                     : "+v"(bx[(RG) % 3][0]), "+v"(bx[(RG) % 3][1])                                          \
+                     : "n"((RG) + 1 < (N) ? 2 : 0));                                                         \
+        if ((RG) + 2 < (N)) {                                                                                \
+            bx[((RG) + 2) % 3][0] = ds_read16<((RG) + 2) * 2048u>(b0);                                       \
+            bx[((RG) + 2) % 3][1] = ds_read16<((RG) + 2) * 2048u>(b1);                                       \
+        }                                                                                                    \
+        const v8bf B0 = __builtin_bit_cast(v8bf, bx[(RG) % 3][0]), B1 = __builtin_bit_cast(v8bf, bx[(RG) % 3][1]); \
+        acc[RG][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[0][0], B0, acc[RG][0], 0, 0, 0);            \
+        acc[RG][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[1][0], B0, acc[RG][1], 0, 0, 0);            \
+        acc[RG][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[0][1], B1, acc[RG][0], 0, 0, 0);            \
+        acc[RG][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[1][1], B1, acc[RG][1], 0, 0, 0);            \
+    }
+#define T5W_BLOCK_N(N)                                                                                       \
+    T5W_BLOCK_HEAD()                                                                                         \
+    v4i ar[2][2];                                                                                            \
+    ar[0][0] = ds_read16<0>(wb + opb0), ar[0][1] = ds_read16<0>(wb + opb1);                                  \
+    ar[1][0] = ds_read16<2048>(wb + opb0), ar[1][1] = ds_read16<2048>(wb + opb1);                            \
+    v4i bx[3][2];                                                                                            \
+    bx[0][0] = ds_read16<0>(b0), bx[0][1] = ds_read16<0>(b1);                                                \
+    if ((N) > 1) bx[1][0] = ds_read16<2048u>(b0), bx[1][1] = ds_read16<2048u>(b1);                           \
+    asm volatile("s_waitcnt lgkmcnt(%4)"                                                                     \
+                 : "+v"(ar[0][0]), "+v"(ar[0][1]), "+v"(ar[1][0]), "+v"(ar[1][1])                            \
+                 : "n"((N) > 1 ? 4 : 2));                                                                    \
+    v8bf aop[2][2];                                                                                          \
+    _Pragma("unroll") for (int x = 0; x < 2; x++)                                                            \
+        _Pragma("unroll") for (int k2 = 0; k2 < 2; k2++) aop[x][k2] = __builtin_bit_cast(v8bf, ar[x][k2]);   \
+    T5W_GROUP_N(0, N) T5W_GROUP_N(1, N) T5W_GROUP_N(2, N) T5W_GROUP_N(3, N)                                  \
+    T5W_GROUP_N(4, N) T5W_GROUP_N(5, N) T5W_GROUP_N(6, N) T5W_GROUP_N(7, N)
 /* ---- the block of the fp4 x fp4 arm: 256 k as two matrix instructions of 128 k, both operands e2m1 with
  *      their E8M0 bytes applied by the instruction itself (a lane's 32 k are one scale block, its byte goes
  *      in as a register: with constant scale arguments the compiler would pick the unscaled instruction).
@@ -367,13 +404,17 @@ __device__ __forceinline__ v8bf t5a_decode(v2i r) {
 /* NG: 16-row groups a tile may hold, 8 or 9 (see t5_nine_groups below). */
 /* A16: `a` holds bf16 rows [..][K] (no activation scales) and a block is 64 k: the bf16-activation arms
  * (block-fp8 weights: ops 85 / 86 arm 0; per-channel fp8 weights: ops 65 / 66). */
-/* AM: what the activation rows are. 0: e4m3 with scales (the W8A8 pairs); 1 (A16): bf16; 2 (A4): mxfp4 rows
+/* AM: what the operands are. 0: e4m3 rows with scales (the W8A8 pairs); 1 (A16): bf16 rows, fp8 weights; 3 (A16 and
+ * W16): bf16 rows and bf16 weights, no scales at all (ops 85 / 86 arm 0 at enc 0 over wtab[E][3], ops 75 / 76 over the
+ * fused table with PC as the layout switch); 2 (A4): mxfp4 rows
  * [..][K / 2] with E8M0 rows [..][K / 32] against mxfp4 weights, a block is 256 k, scales applied by the
  * matrix instruction (ops 85 / 86 with enc 2, arm 0). */
 template <bool GLU, bool PC, uint32_t NCW, int NG = 8, int AM = 0>
 __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     static_assert(NG == 8 || NG == 9, "a tile is eight or nine 16-row groups");
-    constexpr bool A16 = AM == 1, A4 = AM == 2;
+    constexpr bool A16 = AM == 1 || AM == 3, A4 = AM == 2, W16 = AM == 3;
+    constexpr bool W8 = A16 && !W16; /* fp8 weight rows under bf16 rows: 64 bytes per block */
+    static_assert(!W16 || NG == 8, "the bf16-weight form has 128-row tiles");
     static_assert(!A4 || (NG == 8 && !PC), "the fp4 arm has 128-row tiles and no per-channel mode");
     typedef typename std::conditional<A4, T5LdsA4, T5Lds>::type Lds;
     Lds& L = *(Lds*)lds_raw;
@@ -429,7 +470,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     const uint32_t K = g.K, KB = K / (A16 ? 64u : A4 ? 256u : 128u); /* blocks of the K loop */
     const uint32_t KS = K / 128u;                                    /* weight block scales along K */
     const uint32_t KA = A16 ? 2u * K : A4 ? K / 2u : K;              /* bytes of a token row */
-    const uint32_t KW = A4 ? K / 2u : K;                             /* bytes of a weight row */
+    const uint32_t KW = A4 ? K / 2u : W16 ? 2u * K : K;              /* bytes of a weight row */
     const uint32_t K32 = K / 32u;                                    /* A4: E8M0 bytes of a row */
     (void)KS, (void)K32;
     const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]);
@@ -507,7 +548,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         t.wp1 = (GLU && !PC) ? wtab_c[(size_t)t.e * 3u + 1u] : t.wp0;
         if (t.wp1 == 0ull) t.wp0 = 0ull; /* gate without up: not resident */
         t.sp0 = t.sp1 = 0ull;
-        if (!PC) {
+        if (!PC && !W16) {
             const auto* const stab_c = (const __attribute__((address_space(4))) uint64_t*)g.stab;
             t.sp0 = stab_c[(size_t)t.e * 3u + (GLU ? 0u : 2u)];
             t.sp1 = GLU ? stab_c[(size_t)t.e * 3u + 1u] : t.sp0;
@@ -591,7 +632,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 }
             }
             P.w0 = P.w1 = 0.0f;
-            if (!PC && !A4) {
+            if (!PC && !A4 && !W16) {
                 const float* S0 = (const float*)(uintptr_t)t.sp0;
                 const float* S1 = (const float*)(uintptr_t)t.sp1;
                 const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
@@ -605,20 +646,20 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             S.W0 = (const uint8_t*)(uintptr_t)t.wp0;
             S.nt = (w_nt && t.single) ? 1u : 0u;
             S.nine = (cw < 2u && rows > 128u) ? 1u : 0u;
-            S.W1 = !GLU ? S.W0 : PC ? S.W0 + (size_t)g.N * K /* up rows follow the N gate rows */
+            S.W1 = !GLU ? S.W0 : PC ? S.W0 + (size_t)g.N * KW /* up rows follow the N gate rows */
                                : (const uint8_t*)(uintptr_t)t.wp1;
 #pragma unroll
             for (uint32_t i = 0; i < 5u; i++) {
                 const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * (cw & 1u) + lr;
-                /* a pad row, or (fp4 arm: the staged rows end at g.T) a token past the rows that exist, reads row 0 */
-                const uint32_t src = (GLU && (P.tok[i] == PLOW_EXPERT_UNUSED || (A4 && g.T != 0u && P.tok[i] >= g.T))) ? 0u : P.tok[i];
+                /* a pad row, or (where the launch states the rows of `a` in g.T: staged rows end there) a token past the rows that exist, reads row 0 */
+                const uint32_t src = (GLU && (P.tok[i] == PLOW_EXPERT_UNUSED || (g.T != 0u && P.tok[i] >= g.T))) ? 0u : P.tok[i];
                 S.aoff[i] = src * KA + ((p ^ lds_swz8(row)) << 4);
             }
 #pragma unroll
             for (uint32_t i = 0; i < 8u; i++) { /* LDS weight rows R = 64 * cw + 8 * i + lr: consumer R / 32, group (R / 16) & 1 */
-                if (A16 && i >= 4u) { S.woff[i] = 0u; continue; }
-                /* A16: a load covers 16 rows x 64 B, lane -> (row l >> 2, 16-byte slot l & 3) */
-                const uint32_t R = A16 ? 64u * cw + 16u * i + (lane >> 2) : 64u * cw + 8u * i + lr;
+                if (W8 && i >= 4u) { S.woff[i] = 0u; continue; }
+                /* fp8 weights under bf16 rows: a load covers 16 rows x 64 B, lane -> (row l >> 2, 16-byte slot l & 3) */
+                const uint32_t R = W8 ? 64u * cw + 16u * i + (lane >> 2) : 64u * cw + 8u * i + lr;
                 uint32_t ch;
                 if (GLU) {
                     ch = nt * 128u + 16u * (R >> 5) + (R & 15u);
@@ -626,13 +667,13 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     ch = nt * 256u + R;
                     if (ch >= g.N) ch = 0; /* past the last channel: any valid row, never stored */
                 }
-                S.woff[i] = A16 ? ch * K + (((lane & 3u) ^ ((R >> 2) & 3u)) << 4) : ch * KW + ((p ^ lds_swz8(R)) << 4);
+                S.woff[i] = W8 ? ch * K + (((lane & 3u) ^ ((R >> 2) & 3u)) << 4) : ch * KW + ((p ^ lds_swz8(R)) << 4);
             }
             /* activation scale of row 64 * cw + lane (loader 3 repeats loader 0's 64 values); a pad row
              * reads tilep[0], which is always 0 */
             {
                 const uint32_t row = (cw < 3u ? cw : 0u) * 64u + lane;
-                const bool ok = P.stok != PLOW_EXPERT_UNUSED;
+                const bool ok = P.stok != PLOW_EXPERT_UNUSED && !(GLU && g.T != 0u && P.stok >= g.T); /* a token past the stated rows: zero scale */
                 if (GLU) {
                     S.ssrc = ok ? g.a_scale + P.stok : (const float*)(g.meta + 2u * g.E);
                     S.sstep = ok ? g.pitch : 0u;
@@ -680,8 +721,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                                                  (lds_void*)&L.as[st][(cw < 3u ? cw : 0u) * 64u], 4, 0, 0);
             }
             const uint8_t* const ak = A0 + (size_t)kb * 128u;
-            const uint8_t* const wk0 = S.W0 + (size_t)kb * (A16 ? 64u : 128u);
-            const uint8_t* const wk1 = S.W1 + (size_t)kb * (A16 ? 64u : 128u);
+            const uint8_t* const wk0 = S.W0 + (size_t)kb * (W8 ? 64u : 128u);
+            const uint8_t* const wk1 = S.W1 + (size_t)kb * (W8 ? 64u : 128u);
 #pragma unroll
             for (uint32_t i = 0; i < 4u; i++)
                 __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[i]),
@@ -689,7 +730,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             if (S.nine) /* the ninth group's rows */
                 __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[4]),
                                                  (lds_void*)&L.a[st][(128u + 8u * cw) * 128u], 16, 0, 0);
-            if (A16) {
+            if (W8) {
 #pragma unroll
                 for (uint32_t i = 0; i < 4u; i++) /* 16 weight rows of 64 bytes each */
                     __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 1u)) ? wk1 : wk0) + S.woff[i]),
@@ -732,7 +773,9 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                  * tile or the next) are outstanding. After the barrier the consumers are done with the
                  * block before kb, whose slot takes the block two ahead. */
                 if (kb + 1u < KB || more) { /* the loads that may stay outstanding are those of the block after kb */
-                    if (A16) { /* 4 token-row and 4 weight-row loads, no scales */
+                    if (W16) { /* 4 token-row and 8 weight-row loads, no scales */
+                        LOADER_BARRIER(12);
+                    } else if (A16) { /* 4 token-row and 4 weight-row loads, no scales */
                         if (kb + 1u < KB ? cur.nine : nxt.nine) LOADER_BARRIER(9); else LOADER_BARRIER(8);
                     } else if (A4) { /* 3 scale, 4 token-row, 8 weight-row loads */
                         LOADER_BARRIER(15);
@@ -793,6 +836,18 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     case 3u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(3)) } break;
                     case 2u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(2)) } break;
                     case 1u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(1)) } break;
+                    default: { T5_RUN_BLOCKS() } break;
+                }
+            } else if constexpr (W16) {
+                switch (ngrp_w) {
+                    case 8u: { T5_RUN_BLOCKS(T5W_BLOCK_N(8)) } break;
+                    case 7u: { T5_RUN_BLOCKS(T5W_BLOCK_N(7)) } break;
+                    case 6u: { T5_RUN_BLOCKS(T5W_BLOCK_N(6)) } break;
+                    case 5u: { T5_RUN_BLOCKS(T5W_BLOCK_N(5)) } break;
+                    case 4u: { T5_RUN_BLOCKS(T5W_BLOCK_N(4)) } break;
+                    case 3u: { T5_RUN_BLOCKS(T5W_BLOCK_N(3)) } break;
+                    case 2u: { T5_RUN_BLOCKS(T5W_BLOCK_N(2)) } break;
+                    case 1u: { T5_RUN_BLOCKS(T5W_BLOCK_N(1)) } break;
                     default: { T5_RUN_BLOCKS() } break;
                 }
             } else if constexpr (A16) {
@@ -881,10 +936,12 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     for (int rg = 0; rg < NG; rg++) {
                         const uint32_t row = 16u * (uint32_t)rg + r16;
                         bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
+                        /* bf16 weights (the reference's bf16 grouped ops write live rows only): pad rows stay untouched */
                         if (row >= rows) {
-                            if (erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
+                            if (!W16 && erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
                             continue;
                         }
+                        if (W16 && L.epi_idx[par][row] == PLOW_EXPERT_UNUSED) continue;
                         uint2 pk = make_uint2(0u, 0u);
                         if (L.epi_idx[par][row] != PLOW_EXPERT_UNUSED) {
                             float o[4];
@@ -988,7 +1045,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                         /* per-channel arm (plow runtime/amd/op_moe.h:6655-6700): g = acc * (as * wsc[n]); GLU
                          * stores bf16(act(g) * u) and zeroes the expert's pad rows, DOWN stores gate * acc, then
                          * * (as * wsc[h]) */
-                        const float* es = (const float*)(uintptr_t)g.stab[(size_t)t.e * 2u + (GLU ? 0u : 1u)];
+                        /* bf16 weights carry no scales: the same epilogues with every scale 1 */
+                        const float* es = W16 ? nullptr : (const float*)(uintptr_t)g.stab[(size_t)t.e * 2u + (GLU ? 0u : 1u)];
                         const uint32_t cnt_e = (uint32_t)g.meta[g.E + t.e], erow0 = r0 - (uint32_t)g.meta[t.e];
                         const uint32_t padded = ((cnt_e + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM;
                         if (wave_on && !GLU) {
@@ -1005,7 +1063,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
 #pragma unroll
                                     for (int i = 0; i < 4; i++) {
                                         y[x][i] = gate * acc[rg][x][i];
-                                        y[x][i] *= as * es[col + i];
+                                        if (!W16) y[x][i] *= as * es[col + i];
                                     }
                                 }
                                 down_store_f32(rg, y[0], y[1]);
@@ -1019,7 +1077,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                                 const bool mapped = A16 && g.row_partidx != nullptr;
                                 bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
                                 if (row >= rows) {
-                                    if (!mapped && erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
+                                    if (!W16 && !mapped && erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
                                     continue;
                                 }
                                 const uint32_t tok = L.epi_idx[par][row];
@@ -1028,15 +1086,16 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                                     if (tok == PLOW_EXPERT_UNUSED || orow_i == PLOW_EXPERT_UNUSED) continue;
                                     orow = (bf16_t*)g.out + (size_t)orow_i * g.N + ch0 + 4u * q;
                                 } else if (tok == PLOW_EXPERT_UNUSED) {
-                                    *(uint2*)orow = make_uint2(0u, 0u);
+                                    if (!W16) *(uint2*)orow = make_uint2(0u, 0u);
                                     continue;
                                 }
                                 const float as = A16 ? 1.0f : g.a_scale[tok];
                                 float o[4];
 #pragma unroll
                                 for (int i = 0; i < 4; i++)
-                                    o[i] = t5_glu(acc[rg][0][i] * (as * es[ch0 + 4u * q + i]),
-                                                   acc[rg][1][i] * (as * es[g.N + ch0 + 4u * q + i]), g.act, g.f0, g.f1);
+                                    o[i] = W16 ? t5_glu(acc[rg][0][i], acc[rg][1][i], g.act, g.f0, g.f1)
+                                               : t5_glu(acc[rg][0][i] * (as * es[ch0 + 4u * q + i]),
+                                                        acc[rg][1][i] * (as * es[g.N + ch0 + 4u * q + i]), g.act, g.f0, g.f1);
                                 uint2 pk;
                                 pk.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
                                 pk.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
@@ -1100,11 +1159,11 @@ __global__ __launch_bounds__((NCW + 4u) * 64u) void k_group_w8a8_tiled(GroupW8A8
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     t5_body<GLU, PC, NCW, NG>(g, lds_raw);
 }
-/* the same tiles with bf16 activations */
-template <bool GLU, bool PC>
+/* the same tiles with bf16 activations; W16: bf16 weights too (PC then only names the fused table layout) */
+template <bool GLU, bool PC, bool W16 = false>
 __global__ __launch_bounds__(12u * 64u) void k_group_a16_tiled(GroupW8A8 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    t5_body<GLU, PC, 8u, 8, 1>(g, lds_raw);
+    t5_body<GLU, PC, 8u, 8, W16 ? 3 : 1>(g, lds_raw);
 }
 
 
@@ -1132,6 +1191,8 @@ int plow_moe_w8a8_tiled_setup() {
     const bool ok = t5_set_attrs<8u, 8>() && t5_set_attrs<8u, 9>() && t5_set_attrs<4u, 8>() &&
                     a16((const void*)k_group_a16_tiled<true, false>) && a16((const void*)k_group_a16_tiled<false, false>) &&
                     a16((const void*)k_group_a16_tiled<true, true>) && a16((const void*)k_group_a16_tiled<false, true>) &&
+                    a16((const void*)k_group_a16_tiled<true, false, true>) && a16((const void*)k_group_a16_tiled<false, false, true>) &&
+                    a16((const void*)k_group_a16_tiled<true, true, true>) && a16((const void*)k_group_a16_tiled<false, true, true>) &&
                     hipFuncSetAttribute((const void*)k_group_a4w4_tiled<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                         (int)sizeof(T5LdsA4)) == hipSuccess &&
                     hipFuncSetAttribute((const void*)k_group_a4w4_tiled<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1194,6 +1255,16 @@ int launch_group_a16_tiled(const GroupW8A8& g, bool glu, hipStream_t st) {
     if (!group_w8a8_tiled_serves(g)) return PLOW_MOE_EINVAL;
     const uint32_t n_cu = plow_moe_n_cu();
     if (!n_cu) return PLOW_MOE_EDEVICE;
+    if (g.w_bf16) { /* bf16 weights: per_channel names the fused table layout ewt[E][2], nothing else */
+        if (glu) {
+            if (g.per_channel) k_group_a16_tiled<true, true, true><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
+            else k_group_a16_tiled<true, false, true><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
+        } else {
+            if (g.per_channel) k_group_a16_tiled<false, true, true><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
+            else k_group_a16_tiled<false, false, true><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
+        }
+        return 0;
+    }
     if (glu) {
         if (g.per_channel) k_group_a16_tiled<true, true><<<n_cu, 768, sizeof(T5Lds), st>>>(g);
         else k_group_a16_tiled<true, false><<<n_cu, 768, sizeof(T5Lds), st>>>(g);

@@ -88,6 +88,9 @@ struct GroupW8A8 {
      * [..][K / 32]; the GLU writes its output the same way into out / out_e8m0; stab holds E8M0 rows */
     const uint8_t* a_e8m0;
     uint8_t* out_e8m0;
+    /* bf16-activation tiled form (launch_group_a16_tiled): the weights are bf16 too, no scale tables; per_channel then
+     * only says that the tables are the fused pair ewt[E][2] = {gate_up [2N][K], down} instead of wtab[E][3] */
+    uint32_t w_bf16;
     /* tiled forms: when non-zero, the weight rows of an expert with a single row tile (read once) are loaded
      * non-temporal. Right while the launch is bound by the weight stream; from about 64 rows per expert on
      * average it is bound by what a CU's load path carries and the bit costs time */
@@ -120,8 +123,9 @@ int launch_group_down_w8a8_tiled(const GroupW8A8& g, hipStream_t st);
 /* whether the tiled form serves this shape (callers take the streaming form otherwise) */
 bool group_w8a8_tiled_serves(const GroupW8A8& g);
 /* the tiled form with bf16 activations (`a` bf16 [..][K], no activation scales): block-fp8 weights
- * (wtab / stab [E][3]; GLU writes bf16 rows, out_bf16 set) or per-channel fp8 weights (per_channel set,
- * tables [E][2]); GLU gathers rows by row_token and, per-channel mode only, may scatter them by
+ * (wtab / stab [E][3]; GLU writes bf16 rows, out_bf16 set), per-channel fp8 weights (per_channel set,
+ * tables [E][2]) or bf16 weights (w_bf16 set, either layout); GLU gathers rows by row_token and, in the
+ * fused-table layout only, may scatter them by
  * row_partidx; DOWN reads aligned rows, or slot rows when a_slots is set */
 int launch_group_a16_tiled(const GroupW8A8& g, bool glu, hipStream_t st);
 /* the tiled form with mxfp4 on both operands (K a multiple of 256, at least 512) */

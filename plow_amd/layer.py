@@ -221,7 +221,7 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
             if cfg.arm == "w8a8q":
                 p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
                                         t=[fq, x, wtab, stab, meta, row_token, None, fs],
-                                        i=[I, H, Ea, enc, 0, cfg.act, 0, abi.ARM_W8A8_XQ], f=cfg.act_f, slots=T * ka))
+                                        i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8_XQ], f=cfg.act_f, slots=T * ka))
             else:
                 xq = p._t("xq", "u8", (T, H), "scratch")
                 xs = p._t("xs", "f32", (H // 128, T), "scratch")

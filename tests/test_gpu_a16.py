@@ -332,13 +332,15 @@ def test_flat_mxfp4_refusals(moe):
     assert moe.check(abi.inst(abi.OP_MOE_DOWN_MX_PF, t=[0, 1, 2, 3, 4], i=[256, 128, 4]), t) == abi.E_INVAL
 
 
-@pytest.mark.parametrize("act", [0, 1])
-def test_bf16_grouped_fused_table_ops(moe, oracle, act):
+@pytest.mark.parametrize("act,T,stated", [(0, 40, False), (1, 40, False), (1, 400, True), (0, 150, True)])
+def test_bf16_grouped_fused_table_ops(moe, oracle, act, T, stated):
     """Reference ops 75 / 76 (bf16, fused table ewt[E][2]) on gathered rows with a non-resident expert and
-    an expert of more than 16 rows."""
-    print(f"[case] ops 75/76 act={act}", flush=True)
-    r = cases.rng_of(90 + act)
-    E, I, H, k, T = 5, 256, 384, 2, 40
+    an expert of more than 16 rows; with the routed rows stated and 60 to 400 rows per expert they run the
+    tiled kernel's bf16-weight form (partial, full and several 128-row tiles), which like the streaming form
+    writes live rows only."""
+    print(f"[case] ops 75/76 act={act} T={T} stated={stated}", flush=True)
+    r = cases.rng_of(90 + act + T)
+    E, I, H, k = 5, 256, 384, 2
     gu = [cases.randn_bf16(r, (2 * I, H), 0.05) for _ in range(E)]
     dn = [cases.randn_bf16(r, (H, I), 0.05) for _ in range(E)]
     x = cases.randn_bf16(r, (T, H), 1.0)
@@ -351,8 +353,8 @@ def test_bf16_grouped_fused_table_ops(moe, oracle, act):
     rows = len(al[2])
     ewt_h = np.array([[g.ctypes.data, d.ctypes.data] for g, d in zip(gu, dn)], dtype=np.uint64)
     ewt_h[3] = 0
-    glu = abi.inst(abi.OP_MOE_GROUP_GLU_GEMMA_PF, t=[0, 1, 2, 3, 4], i=[I, H, E, 0, 0, act])
-    down = abi.inst(abi.OP_MOE_GROUP_DOWN_GEMMA_PF, t=[0, 1, 2, 3, 4, 5], i=[H, I, E])
+    glu = abi.inst(abi.OP_MOE_GROUP_GLU_GEMMA_PF, t=[0, 1, 2, 3, 4], i=[I, H, E, 0, 0, act], slots=T * k if stated else 0)
+    down = abi.inst(abi.OP_MOE_GROUP_DOWN_GEMMA_PF, t=[0, 1, 2, 3, 4, 5], i=[H, I, E], slots=T * k if stated else 0)
     fu_h = np.full((rows, I), 0x1234, np.uint16)
     part_h = np.full((T * k, H), 9.0, np.float32)
     ol.run(oracle.plow_oracle_exec, glu, ol.table_of([fu_h, x, ewt_h, al[0], al[2]]), 4)

@@ -79,7 +79,7 @@ def test_few_tokens_as_matrix_vector_products(moe, oracle, T, k, H, I, arm):
         check_layer(plan, dev, host)
 
 
-@pytest.mark.parametrize("T", [1, 19, 100, 333])
+@pytest.mark.parametrize("T", [1, 19, 100, 333, 700])
 def test_glu_quantizes_bf16_rows_itself(moe, oracle, T):
     """Op 85 arm 6: bf16 rows in, quantized 1x128 where the kernel loads them, no quantizer op and no
     xq / xs tensors (plow runtime/amd/moe_pf_w8a8.h:118-121). The fq bytes and fs scales must also be the
@@ -91,6 +91,15 @@ def test_glu_quantizes_bf16_rows_itself(moe, oracle, T):
     plan, dev, host = both(moe, oracle, layer.MoeConfig("mini-xq", arm="w8a8q", **kw), seed=T)
     assert "xq" not in dev.t and "quant_x" not in plan.names
     check_layer(plan, dev, host)
+    # from 16 rows per expert on average the op runs as quantizer + tiled arm 2 over the context's staging (its i4
+    # states the rows): the bytes must be those of the two-op chain, which runs the same two kernels
+    if T * 5 >= 16 * 33:
+        ref = both(moe, oracle, layer.MoeConfig("mini-x2", arm="w8a8", **kw), seed=T)[1]
+        rows = int(dev.np("meta")[3 * plan.cfg.E_all]) * abi.MPF_BM
+        live = dev.np("row_partidx")[:rows] != abi.EXPERT_UNUSED
+        assert np.array_equal(dev.np("fq")[:rows][live], ref.np("fq")[:rows][live])
+        assert np.array_equal(dev.np("fs")[:rows][live].view(np.uint32), ref.np("fs")[:rows][live].view(np.uint32))
+        assert np.array_equal(dev.np("out"), ref.np("out"))
 
 
 @pytest.mark.parametrize("T,limit", [(1, 0.0), (19, 0.0), (100, 0.02), (333, 0.0), (700, 0.02)])  # from 16 rows per expert: tiled form
