@@ -231,6 +231,8 @@ static bool want_tiled(const Hint& h, uint32_t slots, const GroupW8A8& g) {
  * device, in meta: a one-workgroup launch adds it up into a word of the workspace, and both forms are
  * launched behind it; every workgroup of the form the word does not name returns at once (a few microseconds
  * per op, where the wrong form costs up to twenty times the op). */
+static uint32_t* next_form_word(PlowMoeCtx* c) { return c->ws.form_words + (c->form_seq++ % WS_FORM_WORDS); }
+
 static int launch_w8a8(PlowMoeCtx* c, const Hint& h, uint32_t slots, GroupW8A8& g, bool glu, hipStream_t st) {
     g.slots_bound = slots;
     g.w_nt = tiled_w_nt(slots, g.E, glu);
@@ -239,7 +241,7 @@ static int launch_w8a8(PlowMoeCtx* c, const Hint& h, uint32_t slots, GroupW8A8& 
         if (want_tiled(h, slots, g)) return glu ? launch_group_glu_w8a8_tiled(g, st) : launch_group_down_w8a8_tiled(g, st);
         return glu ? launch_group_glu_w8a8(g, st) : launch_group_down_w8a8(g, st);
     }
-    uint32_t* const word = c->ws.form_words + (c->form_seq++ % WS_FORM_WORDS);
+    uint32_t* const word = next_form_word(c);
     int rc = launch_pick_form(word, g.meta, g.E, st);
     if (rc) return rc;
     g.form_word = word;
@@ -480,6 +482,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.f0 = in->fj[0].f; g.f1 = in->fj[1].f;
             g.wcols = 3; g.wsel0 = 0; g.wsel1 = 1;
             g.slots_hint = slots_of(in, h, 0u);
+            if (!g.slots_hint && h.form != 0) g.form_ws = next_form_word(c); /* unknown rows: the form is chosen on the device */
             return launch_group_glu_a16(g, st);
         }
         if (enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_A4W4) {
@@ -570,6 +573,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.N = H; g.K = I; g.E = E; g.enc = enc;
             g.wcols = 3; g.wsel0 = 2; g.wsel1 = 2;
             g.slots_hint = slots_of(in, h, 0u);
+            if (!g.slots_hint && h.form != 0) g.form_ws = next_form_word(c); /* unknown rows: the form is chosen on the device */
             return launch_group_down_a16(g, st);
         }
         if (enc == PLOW_MOE_ENC_MXFP4 && (arm == PLOW_MOE_ARM_A4W4 || arm == PLOW_MOE_ARM_A4W4_P16)) {
@@ -685,6 +689,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = (const int32_t*)ten(in, T, 3);
         g.N = N; g.K = K; g.E = E; g.enc = PLOW_MOE_ENC_BF16; g.act = glu ? i[5] : 0u;
         g.slots_hint = slots_of(in, h, 0u);
+        if (!g.slots_hint && h.form != 0) g.form_ws = next_form_word(c); /* unknown rows: the form is chosen on the device */
         if (glu) {
             g.a_idx = (const uint32_t*)ten(in, T, 4);
             g.wsel0 = g.wsel1 = 0; g.wrow1 = N;

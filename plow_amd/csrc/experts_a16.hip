@@ -258,7 +258,7 @@ __global__ __launch_bounds__(AK_THREADS, GLU ? 2 : 4) void k_group_a16_stream(Gr
     const uint32_t tiles = g.N / AK_BN;
     const uint32_t e = g.E - 1u - blockIdx.x / tiles, ct = blockIdx.x % tiles; /* heavy (folded shared) expert first */
     const uint32_t cnt = g.meta ? (uint32_t)g.meta[g.E + e] : g.dense_rows;
-    if (cnt == 0u) return;
+    if (cnt == 0u || !form_is_mine(g)) return;
     if (g.wtab && g.wtab[(size_t)e * g.wcols + g.wsel0] == 0ull) return; /* expert not resident: skipped */
     if (g.stab && ENC != AENC_BF16 && g.stab[(size_t)e * g.wcols + g.wsel0] == 0ull) return;
     const uint32_t r0 = g.meta ? (uint32_t)g.meta[e] : 0u;
@@ -428,13 +428,21 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
          * row reads the pass's first row and is never stored */
         const uint32_t pc = lane % NP;
         const uint8_t* xsrc[NXI];
+        /* A load whose rows all lie past the expert's last row brings four bytes per lane of the pass's first row
+         * instead of sixteen of its own rows (one cache line instead of eight; the count of loads per step stays what
+         * the waits below assume): the LDS rows it would fill feed only the columns of pad rows in the matrix products
+         * (a column of the result depends on its own row alone), and those are never stored. With three rows in a pass
+         * of sixteen that is most of the row bytes a step asks of the L2. */
+        /* (bf16 weights: a step's rows are 2 KB against 32 KB of weight rows, nothing to win: always loaded) */
+        const uint32_t live = ENC == AENC_BF16 ? 0xFFFFFFFFu : cnt - rb;
+        const uint8_t* xdummy;
         {
             const uint32_t first = g.a_idx ? g.a_idx[r0 + rb] : r0 + rb;
 #pragma unroll
             for (uint32_t i = 0; i < NXI; i++) {
                 const uint32_t xrow = XRPL * (wv + AK_WAVES * i) + lane / NP;
                 xsrc[i] = nullptr;
-                if (wv + AK_WAVES * i < XL) {
+                if (wv + AK_WAVES * i < XL && XRPL * (wv + AK_WAVES * i) < live) {
                     const uint32_t off = rb + xrow;
                     uint32_t ai = off < cnt ? (g.a_idx ? g.a_idx[r0 + off] : r0 + off) : PLOW_EXPERT_UNUSED;
                     if (ai == PLOW_EXPERT_UNUSED) ai = first == PLOW_EXPERT_UNUSED ? 0u : first;
@@ -442,6 +450,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                     xsrc[i] = (const uint8_t*)g.a + (size_t)ai * K * 2u + (gp << 4);
                 }
             }
+            xdummy = (const uint8_t*)g.a + (size_t)(first == PLOW_EXPERT_UNUSED ? 0u : first) * K * 2u;
         }
         /* the B-operand rows of this lane: row c of each 16-row group */
         bool valid[RG];
@@ -496,9 +505,13 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
             }
 #pragma unroll
             for (uint32_t i = 0; i < NXI; i++)
-                if (wv + AK_WAVES * i < XL)
-                    __builtin_amdgcn_global_load_lds((const void*)(xsrc[i] + (size_t)ld_S * XROW),
-                                                     (dm_lds_void*)&L.x[ld_st][XRPL * (wv + AK_WAVES * i) * XROW], 16, 0, 0);
+                if (wv + AK_WAVES * i < XL) {
+                    if (XRPL * (wv + AK_WAVES * i) < live)
+                        __builtin_amdgcn_global_load_lds((const void*)(xsrc[i] + (size_t)ld_S * XROW),
+                                                         (dm_lds_void*)&L.x[ld_st][XRPL * (wv + AK_WAVES * i) * XROW], 16, 0, 0);
+                    else /* rows past the expert's last: a stand-in that keeps the load count */
+                        __builtin_amdgcn_global_load_lds((const void*)xdummy, (dm_lds_void*)&L.x[ld_st][XRPL * (wv + AK_WAVES * i) * XROW], 4, 0, 0);
+                }
             ld_st = ld_st + 1u == DM_STAGES ? 0u : ld_st + 1u;
             if (++ld_S == KS) ld_S = 0u, ld_t++;
         };
@@ -693,7 +706,7 @@ template <int ENC, bool GLU>
 __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
     DmWork w;
-    if (!a16_dma_work<ENC>(g, blockIdx.x, w)) return;
+    if (!form_is_mine(g) || !a16_dma_work<ENC>(g, blockIdx.x, w)) return;
     if (w.cnt <= 16u) a16_dma_body<ENC, GLU, 1>(g, dm_raw, w);
     else if (ENC == AENC_MXFP4 || w.cnt <= 32u) a16_dma_body<ENC, GLU, 2>(g, dm_raw, w);
     else a16_dma_body<ENC, GLU, ENC == AENC_MXFP4 ? 2 : 4>(g, dm_raw, w);
@@ -718,10 +731,12 @@ static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
  * its rows through a_idx (and may scatter through o_idx in per-channel mode: the slot-major ops), DOWN
  * reads aligned rows or, slot-major, the rows a_idx = o_idx names. Returns false when the call is not
  * of that kind (the streaming forms then serve it). */
+/* behind_choice: the batch's row count is unknown to the host; the launch goes out behind the device-side choice
+ * in g.form_ws and runs only if that names the tiled form */
 template <bool GLU>
-static bool a16_tiled_try(const GroupA16& g, hipStream_t st, int* rc) {
+static bool a16_tiled_try(const GroupA16& g, hipStream_t st, int* rc, bool behind_choice = false) {
     if (!plow_moe_tuning().a16_tiled || !g.meta || g.bias || g.wmul > 1u || g.dense_rows) return false;
-    if (g.slots_hint < 16u * g.E) return false;
+    if (behind_choice ? (g.slots_hint != 0u || !g.form_ws || !plow_moe_tuning().form_on_device) : g.slots_hint < 16u * g.E) return false;
     const bool w16 = g.enc == AENC_BF16;
     if (!w16 && !g.stab) return false;
     /* the table layout: fused pairs {gate_up, down} (per-channel fp8; bf16 through ops 75 / 76) or {gate, up, down} */
@@ -747,18 +762,31 @@ static bool a16_tiled_try(const GroupA16& g, hipStream_t st, int* rc) {
         w.a_slots = g.a_idx ? g.slots_hint : 0u;
     }
     if (!group_w8a8_tiled_serves(w)) return false;
+    if (behind_choice) {
+        if (!GLU && g.a_idx) return false; /* slot-major rows need the slot count, which such a caller states */
+        *rc = launch_pick_form(g.form_ws, g.meta, g.E, st);
+        if (*rc) return true;
+        w.form_word = g.form_ws, w.form_want = 1u;
+    }
     *rc = launch_group_a16_tiled(w, GLU, st);
     return true;
 }
 
 template <bool GLU>
-static int launch_a16(const GroupA16& g, hipStream_t st) {
+static int launch_a16(const GroupA16& g_in, hipStream_t st) {
+    GroupA16 g = g_in;
     if (g.N == 0 || g.K == 0 || g.E == 0 || g.N % AK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
     if ((uint64_t)g.E * (g.N / AK_BN) > 0x7FFFFFFFull) return PLOW_MOE_EINVAL;
     if (group_a16_gemv_serves(g)) return launch_group_a16_gemv(g, GLU, st); /* a handful of rows in all */
     {
         int rc = 0;
         if (a16_tiled_try<GLU>(g, st, &rc)) return rc;
+        /* no row count from the host: the tiled form goes out behind a choice made on the device from meta, and
+         * so does the streaming form below; the one the choice does not name returns at once */
+        if (a16_tiled_try<GLU>(g, st, &rc, true)) {
+            if (rc) return rc;
+            g.form_word = g.form_ws, g.form_want = 0u;
+        }
     }
     const dim3 grid(g.E * (g.N / AK_BN));
     /* second form: needs whole steps of K (one 128-byte line per weight row) and the block scales of a

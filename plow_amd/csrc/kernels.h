@@ -106,7 +106,8 @@ struct GroupW8A8 {
 };
 #if defined(__HIPCC__)
 /* whether this launch is the form the device-side choice names (always, when the launch carries no choice) */
-__device__ __forceinline__ bool form_is_mine(const GroupW8A8& g) {
+template <typename G>
+__device__ __forceinline__ bool form_is_mine(const G& g) {
     uint32_t form = g.form_want;
     if (g.form_word) form = *(const __attribute__((address_space(4))) uint32_t*)g.form_word; /* written by an earlier kernel: a scalar load */
     return form == g.form_want;
@@ -162,6 +163,12 @@ struct GroupA16 {
     /* matrix-vector form, DOWN with block-fp8 weights only: when set, `a` holds e4m3 rows [rows][K] and this their
      * f32 scales [rows][K / 128] (the intermediate of the fp8 x fp8 arm) */
     const float* a_f8scale;
+    /* Form chosen on the device (see GroupW8A8::form_word). form_ws: a word of workspace the launcher may use for the
+     * choice when slots_hint is 0 and the op could run tiled (NULL: unknown row counts take the streaming form);
+     * form_word / form_want: set by the launcher on the launches that stand behind the choice. */
+    uint32_t* form_ws;
+    const uint32_t* form_word;
+    uint32_t form_want;
 };
 /* the matrix-vector form of the same ops for batches that route a handful of rows in all (slots_hint says so) */
 bool group_a16_gemv_serves(const GroupA16& g);

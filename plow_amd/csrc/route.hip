@@ -441,14 +441,21 @@ int launch_router_score(float* out, const void* x, const void* w, uint32_t M, ui
             k_router_score_tile<4><<<g, 256, 0, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
         }
     } else if (!tune.score_tile8 && K % RSR_KC == 0u && (uint64_t)N * K * 2u < (1ull << 31) && (uint64_t)M * K * 2u < (1ull << 31) &&
-               (M < 16u || (uint64_t)M * N <= 2048u)) {
+               (M < 16u || (uint64_t)M * N <= 2048u || (!tune.score_row_narrow && (uint64_t)((N + 63) / 64) * ((M + 1u) / 2u) <= n_cu))) {
         /* measured against the 8 x 8 tile kernel below: ahead with one or two tokens per workgroup (6 of
          * 38 us at 1 x 384 x 7168) and with four on small score matrices (16 x 64 x 2048: 17 against
          * 25 us); with four tokens on a large one the shared LDS tile is the limit and the two are level */
         /* tokens per workgroup: as many as keep the weight rows' re-reads (once per workgroup row) low */
         const uint32_t lds = RSR_LDS;
         const uint32_t nx = (N + 63) / 64;
-        if (M >= 16u) k_router_score_row<4><<<dim3(nx, (M + 3u) / 4u), (4u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        /* a batch whose (token, 64 experts) chains fit the chip one or two to a workgroup keeps that shape beyond 16
+         * tokens: every output is one chain of K dependent multiply-adds whatever the tile, and the 8 x 8 tile kernel
+         * below runs 64 of them per wave where this one runs 64 per wave with the weight tile to itself */
+        if (!tune.score_row_narrow && M >= 16u && (uint64_t)nx * M <= n_cu)
+            k_router_score_row<1><<<dim3(nx, M), (1u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        else if (!tune.score_row_narrow && M >= 16u && (uint64_t)nx * ((M + 1u) / 2u) <= n_cu)
+            k_router_score_row<2><<<dim3(nx, (M + 1u) / 2u), (2u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        else if (M >= 16u) k_router_score_row<4><<<dim3(nx, (M + 3u) / 4u), (4u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
         else if (M >= 4u) k_router_score_row<2><<<dim3(nx, (M + 1u) / 2u), (2u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
         else k_router_score_row<1><<<dim3(nx, M), (1u + RSR_STAGERS) * 64u, lds, st>>>(out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
     } else {

@@ -16,6 +16,8 @@
  *                                              the vector-unit kernels at prefill sizes
  *   PLOW_MOE_A16_TILED        0                keep the bf16-activation arms on the streaming kernels at every row count
  *   PLOW_MOE_A16_GEMV         0                keep the bf16-activation arms off the matrix-vector form at a few tokens
+ *   PLOW_MOE_SCORE_ROW        narrow           router score: the one-token-per-wave kernel only below 16 tokens (default: while
+ *                                              its workgroups fit the chip)
  *   PLOW_MOE_FORM_ON_DEVICE   0                a grouped fp8 x fp8 op without a row count runs the streaming form
  *                                              (default: both forms are launched behind a choice made on the device)
  */
@@ -38,6 +40,7 @@ struct PlowMoeTuning {
     bool a16_tiled;
     bool a16_gemv;
     bool form_on_device;
+    bool score_row_narrow;
 };
 const PlowMoeTuning& plow_moe_tuning();
 

@@ -124,6 +124,31 @@ def test_per_channel_w8a8_tiled_many_rows(moe, oracle, T, E, k):
     check_chain(plan, dev, host)
 
 
+@pytest.mark.parametrize("enc,T,E,k", [("fp8blk", 333, 8, 4), ("fp8blk", 20, 8, 4), ("bf16", 300, 4, 2), ("bf16", 14, 4, 2)])
+def test_bf16_activation_ops_issued_alone_pick_their_form_on_the_device(moe, enc, T, E, k):
+    """Ops 85 / 86 on the bf16-activation arms issued one at a time with no row count stated: the tiled and the
+    streaming form both go out behind a choice made on the device from meta; the bytes must be those of the run
+    that states the count, at tiled and at streaming row counts."""
+    print(f"[case] a16 form on device enc={enc} T={T}", flush=True)
+    cfg = layer.MoeConfig("a16-alone", H=384, E=E, I=256, k=k, T=T, scoring="softmax", norm_topk=True, enc=enc, arm="a16",
+                          n_shared=1, shared_mode="fold")
+    plan = layer.plan_layer(cfg)
+    assert T * cfg.k_all > 36                                     # beyond the matrix-vector form, which only a stated count selects
+    want = synth.bind(plan, "cuda", seed=T)
+    moe.exec_many(plan.insts, want.table())
+    torch.cuda.synchronize()
+    got = synth.bind(plan, "cuda", seed=T)
+    for d in plan.insts:
+        d.fj[2].u = 0
+        moe.exec(d, got.table())
+    torch.cuda.synchronize()
+    rows = int(want.np("meta")[3 * cfg.E_all]) * abi.MPF_BM
+    live = want.np("row_partidx")[:rows] != abi.EXPERT_UNUSED
+    assert np.array_equal(want.np("fu")[:rows][live], got.np("fu")[:rows][live])
+    for name in ("part", "out"):
+        assert want.np(name).tobytes() == got.np(name).tobytes(), name
+
+
 def test_mxfp4_decode_ops_match_plow_cpu_golden(moe):
     """Ops 48 / 49 at enc 2 against vectors written by plow's flat mxfp4 kernels (ops 150 / 151),
     including a sentinel slot (GLU writes nothing, DOWN writes zeros)."""
