@@ -736,12 +736,16 @@ static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
 template <bool GLU>
 static bool a16_tiled_try(const GroupA16& g, hipStream_t st, int* rc, bool behind_choice = false) {
     if (!plow_moe_tuning().a16_tiled || !g.meta || g.bias || g.wmul > 1u || g.dense_rows) return false;
-    if (behind_choice ? (g.slots_hint != 0u || !g.form_ws || !plow_moe_tuning().form_on_device) : g.slots_hint < 16u * g.E) return false;
-    const bool w16 = g.enc == AENC_BF16;
+    /* mxfp4 DOWN: from 8 rows per expert on average (its streaming form re-streams an expert's weights per 32 rows
+     * and decodes every weight once per pass: measured below) */
+    const uint32_t per_e = (!GLU && g.enc == AENC_MXFP4) ? 8u : 16u;
+    if (behind_choice ? (g.slots_hint != 0u || !g.form_ws || !plow_moe_tuning().form_on_device) : g.slots_hint < per_e * g.E) return false;
+    const bool w16 = g.enc == AENC_BF16, w4 = g.enc == AENC_MXFP4;
     if (!w16 && !g.stab) return false;
     /* the table layout: fused pairs {gate_up, down} (per-channel fp8; bf16 through ops 75 / 76) or {gate, up, down} */
     const bool pc = g.enc == AENC_FP8PC || (w16 && g.wcols == 2u);
-    if (!pc && !w16 && g.enc != AENC_FP8BLK) return false;
+    if (!pc && !w16 && !w4 && g.enc != AENC_FP8BLK) return false;
+    if (w4 && (!plow_moe_tuning().a16_tiled_mx || (!GLU && g.a_idx))) return false; /* aligned rows only */
     if (g.wrow0) return false;
     if (pc) {
         if (g.wcols != 2u || (GLU ? (g.wsel0 != 0u || g.wsel1 != 0u || g.wrow1 != g.N) : g.wsel0 != 1u)) return false;
@@ -753,6 +757,7 @@ static bool a16_tiled_try(const GroupA16& g, hipStream_t st, int* rc, bool behin
     w.N = g.N, w.K = g.K, w.E = g.E, w.act = g.act, w.f0 = g.f0, w.f1 = g.f1;
     w.per_channel = pc ? 1u : 0u;
     w.w_bf16 = w16 ? 1u : 0u;
+    w.w_mxfp4 = w4 ? 1u : 0u;
     if (GLU) {
         if (!g.a_idx || (g.o_idx && !pc)) return false;
         w.row_token = g.a_idx, w.row_partidx = g.o_idx, w.out_bf16 = 1u;

@@ -85,6 +85,18 @@ struct T5LdsA4 {
 };
 static_assert(sizeof(T5LdsA4) <= 160u * 1024u, "the tile's LDS plan must fit one CU");
 
+/* the plan of the mxfp4-weight form under bf16 rows: a block is 128 k, a token row 256 bytes of bf16 (16-byte pieces
+ * swizzled by lds_swz16), a weight row 64 bytes of e2m1 with its four E8M0 bytes beside it; 128-row tiles */
+struct T5LdsW4 {
+    uint8_t a[T5_STAGES][128u * 256u];
+    uint8_t w[T5_STAGES][256u * 64u];
+    uint8_t ws[T5_STAGES][256u][4];
+    uint32_t epi_idx[2][T5_AS];
+    float epi_gate[2][T5_AS];
+    uint16_t prefix[1056];
+};
+static_assert(sizeof(T5LdsW4) <= 160u * 1024u, "the tile's LDS plan must fit one CU");
+
 typedef __attribute__((address_space(3))) void lds_void;
 
 /* The ring is written by direct global -> LDS loads that the compiler would otherwise fence
@@ -323,6 +335,45 @@ __device__ __forceinline__ v2i ds_read8(uint32_t addr) {
         _Pragma("unroll") for (int k2 = 0; k2 < 2; k2++) aop[x][k2] = __builtin_bit_cast(v8bf, ar[x][k2]);   \
     T5W_GROUP_N(0, N) T5W_GROUP_N(1, N) T5W_GROUP_N(2, N) T5W_GROUP_N(3, N)                                  \
     T5W_GROUP_N(4, N) T5W_GROUP_N(5, N) T5W_GROUP_N(6, N) T5W_GROUP_N(7, N)
+/* ---- the block with mxfp4 weights under bf16 rows (W4): 128 k. A lane's weight piece is 16 bytes of its row = the 32 k
+ *      of ONE E8M0 block (k 32q .. 32q + 31), decoded to bf16 with the scale folded in (exact, as the streaming
+ *      kernels do); matrix instruction j multiplies the lane's dword j (k 32q + 8j ..) with the token piece 4q + j,
+ *      so the four instructions of an operand pair cover the block's 128 k, each k once. Token pieces of group
+ *      RG + 1 are read while group RG multiplies (two buffers of four pieces). No scales outside the decode: the
+ *      accumulators run straight through K. ---- */
+#define T5X_BLOCK_HEAD()                                                                                     \
+    const uint32_t ab = a_base + st * (uint32_t)sizeof(L.a[0]) + r16 * 256u;                                 \
+    const uint32_t wb = w_base + st * (256u * 64u) + cw * (32u * 64u) + r16 * 64u + ((q ^ ((r16 >> 2) & 3u)) << 4); \
+    const uint32_t wsl = wsb_base + st * 1024u + (cw * 32u + r16) * 4u + q;
+#define T5X_READ_GROUP(BUF, RG)                                                                              \
+    bx[BUF][0] = ds_read16<(RG) * 4096u>(ab + xo0), bx[BUF][1] = ds_read16<(RG) * 4096u>(ab + xo1);          \
+    bx[BUF][2] = ds_read16<(RG) * 4096u>(ab + xo2), bx[BUF][3] = ds_read16<(RG) * 4096u>(ab + xo3);
+#define T5X_GROUP_N(RG, N)                                                                                   \
+    if ((RG) < (N)) {                                                                                        \
+        if ((RG) + 1 < (N)) { T5X_READ_GROUP(((RG) + 1) & 1, (RG) + 1) }                                      \
+        asm volatile("s_waitcnt lgkmcnt(%4)"                                                                 \
+                     : "+v"(bx[(RG) & 1][0]), "+v"(bx[(RG) & 1][1]), "+v"(bx[(RG) & 1][2]), "+v"(bx[(RG) & 1][3]) \
+                     : "n"((RG) + 1 < (N) ? 4 : 0));                                                         \
+        _Pragma("unroll") for (int j = 0; j < 4; j++) {                                                      \
+            const v8bf B = __builtin_bit_cast(v8bf, bx[(RG) & 1][j]);                                        \
+            acc[RG][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[0][j], B, acc[RG][0], 0, 0, 0);         \
+            acc[RG][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop[1][j], B, acc[RG][1], 0, 0, 0);         \
+        }                                                                                                    \
+    }
+#define T5X_BLOCK_N(N)                                                                                       \
+    T5X_BLOCK_HEAD()                                                                                         \
+    v4i ax[2];                                                                                               \
+    int sb[2];                                                                                               \
+    ax[0] = ds_read16<0>(wb), ax[1] = ds_read16<1024>(wb);                                                   \
+    sb[0] = ds_read1<0>(wsl), sb[1] = ds_read1<64>(wsl);                                                     \
+    v4i bx[2][4];                                                                                            \
+    T5X_READ_GROUP(0, 0)                                                                                     \
+    asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(ax[0]), "+v"(ax[1]), "+v"(sb[0]), "+v"(sb[1]));               \
+    v8bf aop[2][4];                                                                                          \
+    _Pragma("unroll") for (int x = 0; x < 2; x++)                                                            \
+        _Pragma("unroll") for (int j = 0; j < 4; j++) aop[x][j] = t5x_decode((uint32_t)ax[x][j], (uint32_t)sb[x]); \
+    T5X_GROUP_N(0, N) T5X_GROUP_N(1, N) T5X_GROUP_N(2, N) T5X_GROUP_N(3, N)                                  \
+    T5X_GROUP_N(4, N) T5X_GROUP_N(5, N) T5X_GROUP_N(6, N) T5X_GROUP_N(7, N)
 /* ---- the block of the fp4 x fp4 arm: 256 k as two matrix instructions of 128 k, both operands e2m1 with
  *      their E8M0 bytes applied by the instruction itself (a lane's 32 k are one scale block, its byte goes
  *      in as a register: with constant scale arguments the compiler would pick the unscaled instruction).
@@ -382,6 +433,15 @@ __device__ __forceinline__ v8bf t5a_decode(v2i r) {
     const v2bf p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((uint32_t)r[1], 1.0f, true);
     return (v8bf){p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
+/* eight e2m1 values of a dword (low nibble = even k) -> eight bf16, scaled by their block's E8M0 byte (exact) */
+__device__ __forceinline__ v8bf t5x_decode(uint32_t wd, uint32_t e8m0) {
+    const float sc = __uint_as_float(e8m0 << 23); /* 2^(s - 127) */
+    const v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 0);
+    const v2bf p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 1);
+    const v2bf p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 2);
+    const v2bf p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, sc, 3);
+    return (v8bf){p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
 /* the K loop of a tile for a consumer wave with N live groups (BODY empty: it only keeps the barriers) */
 #define T5_RUN_BLOCKS(BODY)                                                                                  \
     for (uint32_t kb = 0; kb < KB; kb++) {                                                                   \
@@ -412,11 +472,14 @@ __device__ __forceinline__ v8bf t5a_decode(v2i r) {
 template <bool GLU, bool PC, uint32_t NCW, int NG = 8, int AM = 0>
 __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     static_assert(NG == 8 || NG == 9, "a tile is eight or nine 16-row groups");
-    constexpr bool A16 = AM == 1 || AM == 3, A4 = AM == 2, W16 = AM == 3;
-    constexpr bool W8 = A16 && !W16; /* fp8 weight rows under bf16 rows: 64 bytes per block */
-    static_assert(!W16 || NG == 8, "the bf16-weight form has 128-row tiles");
+    constexpr bool A16 = AM == 1 || AM == 3 || AM == 4, A4 = AM == 2, W16 = AM == 3, W4 = AM == 4;
+    constexpr bool W8 = A16 && !W16 && !W4; /* fp8 weight rows under bf16 rows: 64 bytes per block */
+    constexpr bool W64 = W8 || W4;           /* weight rows of 64 bytes per block (16 rows per direct load) */
+    constexpr bool NOPAD = W16 || W4;        /* forms whose GLU writes live rows only, as the streaming kernels of those encodings do */
+    static_assert(!(W16 || W4) || NG == 8, "the bf16- and mxfp4-weight forms under bf16 rows have 128-row tiles");
+    static_assert(!W4 || !PC, "mxfp4 weights come through wtab / stab [E][3]");
     static_assert(!A4 || (NG == 8 && !PC), "the fp4 arm has 128-row tiles and no per-channel mode");
-    typedef typename std::conditional<A4, T5LdsA4, T5Lds>::type Lds;
+    typedef typename std::conditional<A4, T5LdsA4, typename std::conditional<W4, T5LdsW4, T5Lds>::type>::type Lds;
     Lds& L = *(Lds*)lds_raw;
     constexpr uint32_t BN = GLU ? 128u : 256u; /* output channels per tile */
     constexpr uint32_t NTHR = (NCW + 4u) * 64u, SUBS = 8u / NCW;
@@ -467,16 +530,18 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         }
     }
     const uint32_t total = (uint32_t)L.prefix[g.E - 1u] * NT;
-    const uint32_t K = g.K, KB = K / (A16 ? 64u : A4 ? 256u : 128u); /* blocks of the K loop */
+    const uint32_t K = g.K, KB = K / (W4 ? 128u : A16 ? 64u : A4 ? 256u : 128u); /* blocks of the K loop */
     const uint32_t KS = K / 128u;                                    /* weight block scales along K */
     const uint32_t KA = A16 ? 2u * K : A4 ? K / 2u : K;              /* bytes of a token row */
-    const uint32_t KW = A4 ? K / 2u : W16 ? 2u * K : K;              /* bytes of a weight row */
-    const uint32_t K32 = K / 32u;                                    /* A4: E8M0 bytes of a row */
+    const uint32_t KW = (A4 || W4) ? K / 2u : W16 ? 2u * K : K;      /* bytes of a weight row */
+    const uint32_t K32 = K / 32u;                                    /* A4, W4: E8M0 bytes of a row */
     (void)KS, (void)K32;
     const uint32_t a_base = lds_off(&L.a[0][0]), w_base = lds_off(&L.w[0][0]);
     uint32_t s_base = 0, c_base = 0, ts_base = 0, wsb_base = 0;
     if constexpr (A4) {
         ts_base = lds_off(&L.ts[0][0][0]), wsb_base = lds_off(&L.ws[0][0][0]);
+    } else if constexpr (W4) {
+        wsb_base = lds_off(&L.ws[0][0][0]);
     } else {
         s_base = lds_off(&L.as[0][0]), c_base = lds_off(&L.wsc[0][0][0]);
     }
@@ -489,7 +554,10 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
     const uint32_t opb0 = r16 * 128u + ((q ^ sw) << 4), opb1 = r16 * 128u + (((4u + q) ^ sw) << 4);
     const uint32_t swa = ((r16 >> 2) & 3u) * 2u;
     const uint32_t opa0 = r16 * 64u + ((q ^ swa) << 3), opa1 = r16 * 64u + (((4u + q) ^ swa) << 3);
-    (void)op_lo, (void)op_hi, (void)opb0, (void)opb1, (void)opa0, (void)opa1;
+    /* W4: this lane's token pieces 4q .. 4q + 3 of a 256-byte row */
+    const uint32_t sx = lds_swz16(r16);
+    const uint32_t xo0 = ((4u * q) ^ sx) << 4, xo1 = ((4u * q + 1u) ^ sx) << 4, xo2 = ((4u * q + 2u) ^ sx) << 4, xo3 = ((4u * q + 3u) ^ sx) << 4;
+    (void)op_lo, (void)op_hi, (void)opb0, (void)opb1, (void)opa0, (void)opa1, (void)xo0, (void)xo1, (void)xo2, (void)xo3;
 
     /* Workgroup w runs on XCD w % 8 (round-robin dispatch), and each XCD has its own L2. The logical
      * index below makes the 32 workgroups of one XCD take 32 consecutive tiles of every sweep, and the
@@ -576,7 +644,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
         struct Src {
             /* per-lane 32-bit byte offsets from uniform bases: the loads take (scalar base + k offset,
              * vector offset) */
-            uint32_t aoff[5], woff[8], sstep;
+            uint32_t aoff[8], woff[8], sstep;
             uint32_t nine; /* this loader has a ninth-group load in this tile (loaders 0 and 1, tiles of more than 128 rows) */
             /* A4: this lane's dword of the E8M0 rows: token row 32 * cw + l / 2 and weight rows 64 * cw + 32 * j + l / 2 */
             const uint8_t *tsp, *wsp[2];
@@ -590,17 +658,19 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
          * flight while the loader keeps feeding the tile before: fetch() only issues loads, finish()
          * uses them a few blocks later. Rows below the live count always hold a token. */
         struct Pre {
-            uint32_t tok[5], stok, eidx;
+            uint32_t tok[8], stok, eidx;
             uint32_t tsrow; /* A4: the row of `a` whose scale dword this lane loads */
             float w0, w1, egate;
         };
         auto fetch = [&](const Tile& t, Pre& P) {
             const uint32_t r0 = t.r0, rows = t.rows, nt = t.nt;
 #pragma unroll
-            for (uint32_t i = 0; i < 5u; i++) { /* token rows 32 * cw + 8 * i + lr, and for loaders 0 and 1 rows
-                                                 * 128 + 8 * cw + lr of the ninth group; a pad row reads the first row */
-                if (i == 4u && cw >= 2u) { P.tok[i] = 0u; continue; }
-                const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * cw + lr;
+            for (uint32_t i = 0; i < 8u; i++) { /* token rows 32 * cw + 8 * i + lr, and for loaders 0 and 1 rows
+                                                 * 128 + 8 * cw + lr of the ninth group; a pad row reads the first row.
+                                                 * W4 (256-byte rows, four to a load): rows 32 * cw + 4 * i + lane / 16 */
+                if (!W4 && i >= 5u) { P.tok[i] = 0u; continue; }
+                if (!W4 && i == 4u && cw >= 2u) { P.tok[i] = 0u; continue; }
+                const uint32_t row = W4 ? 32u * cw + 4u * i + (lane >> 4) : i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * cw + lr;
                 const uint32_t ar = r0 + (row < rows ? row : 0u);
                 if (GLU) {
                     P.tok[i] = g.row_token[ar];
@@ -632,7 +702,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 }
             }
             P.w0 = P.w1 = 0.0f;
-            if (!PC && !A4 && !W16) {
+            if (!PC && !A4 && !W16 && !W4) {
                 const float* S0 = (const float*)(uintptr_t)t.sp0;
                 const float* S1 = (const float*)(uintptr_t)t.sp1;
                 const uint32_t nb0 = GLU ? nt : 2u * nt, nb1 = GLU ? nt : (2u * nt + 1u < nblk ? 2u * nt + 1u : 2u * nt);
@@ -649,7 +719,14 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             S.W1 = !GLU ? S.W0 : PC ? S.W0 + (size_t)g.N * KW /* up rows follow the N gate rows */
                                : (const uint8_t*)(uintptr_t)t.wp1;
 #pragma unroll
-            for (uint32_t i = 0; i < 5u; i++) {
+            for (uint32_t i = 0; i < 8u; i++) {
+                if (!W4 && i >= 5u) { S.aoff[i] = 0u; continue; }
+                if (W4) { /* 256-byte rows: lane -> (row lane / 16 of the load's four, piece lane % 16) */
+                    const uint32_t row4 = 32u * cw + 4u * i + (lane >> 4);
+                    const uint32_t src4 = (GLU && (P.tok[i] == PLOW_EXPERT_UNUSED || (g.T != 0u && P.tok[i] >= g.T))) ? 0u : P.tok[i];
+                    S.aoff[i] = src4 * KA + (((lane & 15u) ^ lds_swz16(row4)) << 4);
+                    continue;
+                }
                 const uint32_t row = i < 4u ? 32u * cw + 8u * i + lr : 128u + 8u * (cw & 1u) + lr;
                 /* a pad row, or (where the launch states the rows of `a` in g.T: staged rows end there) a token past the rows that exist, reads row 0 */
                 const uint32_t src = (GLU && (P.tok[i] == PLOW_EXPERT_UNUSED || (g.T != 0u && P.tok[i] >= g.T))) ? 0u : P.tok[i];
@@ -657,9 +734,9 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
             }
 #pragma unroll
             for (uint32_t i = 0; i < 8u; i++) { /* LDS weight rows R = 64 * cw + 8 * i + lr: consumer R / 32, group (R / 16) & 1 */
-                if (W8 && i >= 4u) { S.woff[i] = 0u; continue; }
-                /* fp8 weights under bf16 rows: a load covers 16 rows x 64 B, lane -> (row l >> 2, 16-byte slot l & 3) */
-                const uint32_t R = W8 ? 64u * cw + 16u * i + (lane >> 2) : 64u * cw + 8u * i + lr;
+                if (W64 && i >= 4u) { S.woff[i] = 0u; continue; }
+                /* 64-byte weight rows (fp8 or mxfp4 under bf16 rows): a load covers 16 rows x 64 B, lane -> (row l >> 2, 16-byte slot l & 3) */
+                const uint32_t R = W64 ? 64u * cw + 16u * i + (lane >> 2) : 64u * cw + 8u * i + lr;
                 uint32_t ch;
                 if (GLU) {
                     ch = nt * 128u + 16u * (R >> 5) + (R & 15u);
@@ -667,7 +744,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     ch = nt * 256u + R;
                     if (ch >= g.N) ch = 0; /* past the last channel: any valid row, never stored */
                 }
-                S.woff[i] = W8 ? ch * K + (((lane & 3u) ^ ((R >> 2) & 3u)) << 4) : ch * KW + ((p ^ lds_swz8(R)) << 4);
+                S.woff[i] = W64 ? ch * KW + (((lane & 3u) ^ ((R >> 2) & 3u)) << 4) : ch * KW + ((p ^ lds_swz8(R)) << 4);
             }
             /* activation scale of row 64 * cw + lane (loader 3 repeats loader 0's 64 values); a pad row
              * reads tilep[0], which is always 0 */
@@ -686,7 +763,14 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     S.sstep = ok ? 1u : 0u;
                 }
             }
-            if constexpr (A4) {
+            if constexpr (W4) { /* the four E8M0 bytes of weight row 64 * cw + lane per block, a dword per lane */
+                const uint32_t R = 64u * cw + lane;
+                uint32_t ch = GLU ? nt * 128u + 16u * (R >> 5) + (R & 15u) : nt * 256u + R;
+                if (ch >= g.N) ch = 0;
+                S.wsp[0] = ((GLU && (R & 16u)) ? (const uint8_t*)(uintptr_t)t.sp1 : (const uint8_t*)(uintptr_t)t.sp0) + (size_t)ch * K32;
+                S.wsp[1] = S.wsp[0];
+                S.tsp = nullptr;
+            } else if constexpr (A4) {
                 S.tsp = g.a_e8m0 + (size_t)P.tsrow * K32 + (lane & 1u) * 4u;
                 const uint8_t* const SW0 = (const uint8_t*)(uintptr_t)t.sp0;
                 const uint8_t* const SW1 = (const uint8_t*)(uintptr_t)t.sp1;
@@ -697,7 +781,7 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     if (ch >= g.N) ch = 0;
                     S.wsp[j] = ((GLU && (R & 16u)) ? SW1 : SW0) + (size_t)ch * K32 + (lane & 1u) * 4u;
                 }
-            } else {
+            } else if constexpr (!W4) {
                 const uint32_t i = tid - NCW * 64u;
                 if (i < KS) {
                     L.wsc[par][0][i] = P.w0;
@@ -716,21 +800,30 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 __builtin_amdgcn_global_load_lds((const void*)(S.tsp + (size_t)kb * 8u), (lds_void*)&L.ts[st][32u * cw][0], 4, 0, 0);
                 __builtin_amdgcn_global_load_lds((const void*)(S.wsp[0] + (size_t)kb * 8u), (lds_void*)&L.ws[st][64u * cw][0], 4, 0, 0);
                 __builtin_amdgcn_global_load_lds((const void*)(S.wsp[1] + (size_t)kb * 8u), (lds_void*)&L.ws[st][64u * cw + 32u][0], 4, 0, 0);
+            } else if constexpr (W4) {
+                __builtin_amdgcn_global_load_lds((const void*)(S.wsp[0] + (size_t)kb * 4u), (lds_void*)&L.ws[st][64u * cw][0], 4, 0, 0);
             } else if constexpr (!A16) {
                 __builtin_amdgcn_global_load_lds((const void*)(S.ssrc + (size_t)kb * S.sstep),
                                                  (lds_void*)&L.as[st][(cw < 3u ? cw : 0u) * 64u], 4, 0, 0);
             }
-            const uint8_t* const ak = A0 + (size_t)kb * 128u;
-            const uint8_t* const wk0 = S.W0 + (size_t)kb * (W8 ? 64u : 128u);
-            const uint8_t* const wk1 = S.W1 + (size_t)kb * (W8 ? 64u : 128u);
+            const uint8_t* const ak = A0 + (size_t)kb * (W4 ? 256u : 128u);
+            const uint8_t* const wk0 = S.W0 + (size_t)kb * (W64 ? 64u : 128u);
+            const uint8_t* const wk1 = S.W1 + (size_t)kb * (W64 ? 64u : 128u);
+            if constexpr (W4) {
 #pragma unroll
-            for (uint32_t i = 0; i < 4u; i++)
-                __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[i]),
-                                                 (lds_void*)&L.a[st][(32u * cw + 8u * i) * 128u], 16, 0, 0);
-            if (S.nine) /* the ninth group's rows */
-                __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[4]),
-                                                 (lds_void*)&L.a[st][(128u + 8u * cw) * 128u], 16, 0, 0);
-            if (W8) {
+                for (uint32_t i = 0; i < 8u; i++) /* four token rows of 256 bytes each */
+                    __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[i]),
+                                                     (lds_void*)&L.a[st][(32u * cw + 4u * i) * 256u], 16, 0, 0);
+            } else {
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; i++)
+                    __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[i]),
+                                                     (lds_void*)&L.a[st][(32u * cw + 8u * i) * 128u], 16, 0, 0);
+                if (S.nine) /* the ninth group's rows */
+                    __builtin_amdgcn_global_load_lds((const void*)(ak + S.aoff[4]),
+                                                     (lds_void*)&L.a[st][(128u + 8u * cw) * 128u], 16, 0, 0);
+            }
+            if (W64) {
 #pragma unroll
                 for (uint32_t i = 0; i < 4u; i++) /* 16 weight rows of 64 bytes each */
                     __builtin_amdgcn_global_load_lds((const void*)(((GLU && (i & 1u)) ? wk1 : wk0) + S.woff[i]),
@@ -775,6 +868,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                 if (kb + 1u < KB || more) { /* the loads that may stay outstanding are those of the block after kb */
                     if (W16) { /* 4 token-row and 8 weight-row loads, no scales */
                         LOADER_BARRIER(12);
+                    } else if (W4) { /* 1 scale, 8 token-row, 4 weight-row loads */
+                        LOADER_BARRIER(13);
                     } else if (A16) { /* 4 token-row and 4 weight-row loads, no scales */
                         if (kb + 1u < KB ? cur.nine : nxt.nine) LOADER_BARRIER(9); else LOADER_BARRIER(8);
                     } else if (A4) { /* 3 scale, 4 token-row, 8 weight-row loads */
@@ -836,6 +931,18 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                     case 3u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(3)) } break;
                     case 2u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(2)) } break;
                     case 1u: { T5_RUN_BLOCKS(T5Q_BLOCK_N(1)) } break;
+                    default: { T5_RUN_BLOCKS() } break;
+                }
+            } else if constexpr (W4) {
+                switch (ngrp_w) {
+                    case 8u: { T5_RUN_BLOCKS(T5X_BLOCK_N(8)) } break;
+                    case 7u: { T5_RUN_BLOCKS(T5X_BLOCK_N(7)) } break;
+                    case 6u: { T5_RUN_BLOCKS(T5X_BLOCK_N(6)) } break;
+                    case 5u: { T5_RUN_BLOCKS(T5X_BLOCK_N(5)) } break;
+                    case 4u: { T5_RUN_BLOCKS(T5X_BLOCK_N(4)) } break;
+                    case 3u: { T5_RUN_BLOCKS(T5X_BLOCK_N(3)) } break;
+                    case 2u: { T5_RUN_BLOCKS(T5X_BLOCK_N(2)) } break;
+                    case 1u: { T5_RUN_BLOCKS(T5X_BLOCK_N(1)) } break;
                     default: { T5_RUN_BLOCKS() } break;
                 }
             } else if constexpr (W16) {
@@ -938,10 +1045,10 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                         bf16_t* orow = (bf16_t*)g.out + (size_t)(r0 + row) * g.N + ch0 + 4u * q;
                         /* bf16 weights (the reference's bf16 grouped ops write live rows only): pad rows stay untouched */
                         if (row >= rows) {
-                            if (!W16 && erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
+                            if (!NOPAD && erow0 + row >= cnt_e && erow0 + row < padded) *(uint2*)orow = make_uint2(0u, 0u); /* beyond the expert's rows: a row below its count is the next tile's */
                             continue;
                         }
-                        if (W16 && L.epi_idx[par][row] == PLOW_EXPERT_UNUSED) continue;
+                        if (NOPAD && L.epi_idx[par][row] == PLOW_EXPERT_UNUSED) continue;
                         uint2 pk = make_uint2(0u, 0u);
                         if (L.epi_idx[par][row] != PLOW_EXPERT_UNUSED) {
                             float o[4];
@@ -1007,7 +1114,8 @@ __device__ __forceinline__ void t5_body(const GroupW8A8& g, uint8_t* lds_raw) {
                      * the consumer's own weight slice of the ring stage it has just left: nobody else reads it,
                      * and the loaders refill it only after the next barrier. Every lane of the wave must call
                      * this. */
-                    const uint32_t stg = w_base + stl * (256u * 128u) + cw * (32u * 128u);
+                    /* (W4: its weight stage is 16 KB, so the 4 KB per consumer come from the token-row stage it has left as well) */
+                    const uint32_t stg = W4 ? a_base + stl * (uint32_t)sizeof(L.a[0]) + cw * (32u * 128u) : w_base + stl * (256u * 128u) + cw * (32u * 128u);
                     auto down_store_f32 = [&](int rg, v4f y0, v4f y1) {
                         const uint32_t buf = stg + (uint32_t)(rg & 1) * 2048u, wsw = r16 & 7u;
                         const uint32_t wr0 = buf + r16 * 128u + ((q ^ wsw) << 4), wr1 = buf + r16 * 128u + (((4u + q) ^ wsw) << 4);
@@ -1167,6 +1275,13 @@ __global__ __launch_bounds__(12u * 64u) void k_group_a16_tiled(GroupW8A8 g) {
 }
 
 
+/* mxfp4 weights under bf16 activations (ops 85 / 86 arm 8) */
+template <bool GLU>
+__global__ __launch_bounds__(12u * 64u) void k_group_a16w4_tiled(GroupW8A8 g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    t5_body<GLU, false, 8u, 8, 4>(g, lds_raw);
+}
+
 /* dynamic-LDS limits, once per device (plow_moe_device_setup) */
 template <bool GLU, bool PC, uint32_t NCW, int NG>
 static bool t5_set_attr() {
@@ -1193,6 +1308,10 @@ int plow_moe_w8a8_tiled_setup() {
                     a16((const void*)k_group_a16_tiled<true, true>) && a16((const void*)k_group_a16_tiled<false, true>) &&
                     a16((const void*)k_group_a16_tiled<true, false, true>) && a16((const void*)k_group_a16_tiled<false, false, true>) &&
                     a16((const void*)k_group_a16_tiled<true, true, true>) && a16((const void*)k_group_a16_tiled<false, true, true>) &&
+                    hipFuncSetAttribute((const void*)k_group_a16w4_tiled<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)sizeof(T5LdsW4)) == hipSuccess &&
+                    hipFuncSetAttribute((const void*)k_group_a16w4_tiled<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)sizeof(T5LdsW4)) == hipSuccess &&
                     hipFuncSetAttribute((const void*)k_group_a4w4_tiled<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                         (int)sizeof(T5LdsA4)) == hipSuccess &&
                     hipFuncSetAttribute((const void*)k_group_a4w4_tiled<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1255,6 +1374,12 @@ int launch_group_a16_tiled(const GroupW8A8& g, bool glu, hipStream_t st) {
     if (!group_w8a8_tiled_serves(g)) return PLOW_MOE_EINVAL;
     const uint32_t n_cu = plow_moe_n_cu();
     if (!n_cu) return PLOW_MOE_EDEVICE;
+    if (g.w_mxfp4) { /* mxfp4 weights with E8M0 rows through stab [E][3] */
+        if (g.per_channel) return PLOW_MOE_EINVAL;
+        if (glu) k_group_a16w4_tiled<true><<<n_cu, 768, sizeof(T5LdsW4), st>>>(g);
+        else k_group_a16w4_tiled<false><<<n_cu, 768, sizeof(T5LdsW4), st>>>(g);
+        return 0;
+    }
     if (g.w_bf16) { /* bf16 weights: per_channel names the fused table layout ewt[E][2], nothing else */
         if (glu) {
             if (g.per_channel) k_group_a16_tiled<true, true, true><<<n_cu, 768, sizeof(T5Lds), st>>>(g);

@@ -91,6 +91,8 @@ struct GroupW8A8 {
     /* bf16-activation tiled form (launch_group_a16_tiled): the weights are bf16 too, no scale tables; per_channel then
      * only says that the tables are the fused pair ewt[E][2] = {gate_up [2N][K], down} instead of wtab[E][3] */
     uint32_t w_bf16;
+    /* the same form with mxfp4 weights (wtab / stab [E][3], stab = E8M0 rows [N][K / 32]): a block is 128 k */
+    uint32_t w_mxfp4;
     /* tiled forms: when non-zero, the weight rows of an expert with a single row tile (read once) are loaded
      * non-temporal. Right while the launch is bound by the weight stream; from about 64 rows per expert on
      * average it is bound by what a CU's load path carries and the bit costs time */

@@ -15,6 +15,7 @@
  *   PLOW_MOE_SCORE_KERNEL     tile8 | valu     router score: keep the 8 x 8 tile kernel for few outputs / keep
  *                                              the vector-unit kernels at prefill sizes
  *   PLOW_MOE_A16_TILED        0                keep the bf16-activation arms on the streaming kernels at every row count
+ *   PLOW_MOE_A16_TILED_MX     0                keep mxfp4 weights under bf16 activations on the streaming kernels at every row count
  *   PLOW_MOE_A16_GEMV         0                keep the bf16-activation arms off the matrix-vector form at a few tokens
  *   PLOW_MOE_SCORE_ROW        narrow           router score: the one-token-per-wave kernel only below 16 tokens (default: while
  *                                              its workgroups fit the chip)
@@ -41,6 +42,7 @@ struct PlowMoeTuning {
     bool a16_gemv;
     bool form_on_device;
     bool score_row_narrow;
+    bool a16_tiled_mx;
 };
 const PlowMoeTuning& plow_moe_tuning();
 
