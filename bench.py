@@ -74,6 +74,8 @@ def make_cfg(layer, a, name, tokens):
         # from 128 tokens on, the decode ops (65 / 66 semantics, bf16 activations) below
         cfg.bias = True
         cfg.arm = "w8a8" if cfg.T >= 128 else "a16"
+        # the decode arm's ops 65 / 66 sort the slots themselves: plow's chain for them has no op 84
+        cfg.emit_align = False
     if a.arm == "w8a8det":      # the deterministic fused down -> combine on the block-fp8 W8A8 arm
         cfg.arm, cfg.det_combine = "w8a8", True
     elif a.arm:
@@ -130,8 +132,11 @@ def run_cell(a, name, tokens, steps, warmup, share=None, cpu_mode="full"):
             per_op[nm].append(evs[n].elapsed_time(evs[n + 1]) * 1e3)
     op_us = {n: statistics.mean(v) for n, v in per_op.items()}
 
-    meta = dev.np("meta")
-    cnt = meta[cfg.E_all:2 * cfg.E_all]
+    if "align" in plan.names:
+        cnt = dev.np("meta")[cfg.E_all:2 * cfg.E_all]
+    else:                                            # no op 84 in the chain: rows per expert from the routing table
+        eid = dev.np("table")["eid"]
+        cnt = np.bincount(eid[eid < cfg.E_all], minlength=cfg.E_all)
     hit = int((cnt > 0).sum())                       # experts whose weights must stream (incl. shared)
     rows = int(cnt.sum())
     eb = expert_bytes(cfg)

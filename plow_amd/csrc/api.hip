@@ -192,6 +192,11 @@ extern "C" int plow_moe_set_min_rows(PlowMoeCtx* ctx, int variant, int min_rows)
 struct Hint {
     int form;
     uint32_t slots;
+    /* The sort of a routing table that a slot-major op (48 / 49 / 65 / 66, 150 / 151) of THIS run left in the
+     * workspace: the next op of the run over the same table takes it instead of sorting again (a decode layer's
+     * DOWN after its GLU). Forgotten with the run, and within it whenever an op that writes routing tables runs. */
+    const void* sorted_table;
+    uint32_t sorted_nslot, sorted_E, sorted_kx;
 };
 
 /* Routed slots of the batch as far as this op can know them: the descriptor's own statement (fj[2].u,
@@ -252,8 +257,16 @@ static int launch_w8a8(PlowMoeCtx* c, const Hint& h, uint32_t slots, GroupW8A8& 
     return glu ? launch_group_glu_w8a8_tiled(g, st) : launch_group_down_w8a8_tiled(g, st);
 }
 
-static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStream_t st, bool launch, const Hint& h) {
+/* the workspace's sort serves this op: same table, slot count and expert count; the GLU also needs the same slots
+ * per input row (its row_token = slot / kx), the DOWN reads no row_token */
+static bool sort_reusable(const Hint& h, const void* table, uint32_t nslot, uint32_t E, uint32_t kx, bool glu) {
+    return h.sorted_table != nullptr && h.sorted_table == table && h.sorted_nslot == nslot && h.sorted_E == E && (!glu || h.sorted_kx == kx);
+}
+
+static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStream_t st, bool launch, Hint& h) {
     const uint32_t* i = in->i;
+    if (launch && (in->op == PLOW_DOP_MOE_ROUTER_TOPK || in->op == PLOW_DOP_MOE_ROUTER_TOPK_PF || in->op == PLOW_DOP_GEMM_F32))
+        h.sorted_table = nullptr; /* routing tables may change under the sort the workspace holds */
     switch (in->op) {
     case PLOW_DOP_GEMM_F32: {
         NEED(c, ten(in, T, 0) && ten(in, T, 1) && ten(in, T, 2), "op 180: t0 logits, t1 x, t2 W must be bound");
@@ -648,9 +661,13 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, act <= 1u, "op %u: activation %u is not served", (unsigned)in->op, act);
         if (!launch) return 0;
         /* align with k = slots per input row: row_token = slot / kx, row_partidx = slot */
-        int rc = launch_align(c->ws.meta, ten(in, T, 2), c->ws.row_token, c->ws.row_partidx, c->ws.row_gate,
+        int rc = 0;
+        if (!sort_reusable(h, ten(in, T, 2), nslot, E, kx, glu)) {
+            rc = launch_align(c->ws.meta, ten(in, T, 2), c->ws.row_token, c->ws.row_partidx, c->ws.row_gate,
                               (nslot + kx - 1u) / kx, E, kx, c->ws.chunk_hist, c->ws.max_chunks, st);
-        if (rc) return rc;
+            if (rc) return rc;
+            h.sorted_table = ten(in, T, 2), h.sorted_nslot = nslot, h.sorted_E = E, h.sorted_kx = kx;
+        }
         GroupA16 g = {};
         g.out = ten(in, T, 0); g.a = ten(in, T, 1);
         g.wtab = (const uint64_t*)ten(in, T, 3);
@@ -667,8 +684,14 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         }
         g.a_idx = c->ws.row_partidx; g.gate = c->ws.row_gate;
         g.wsel0 = g.wsel1 = pc ? 1u : 2u;
-        rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), g.wtab, g.stab, g.wcols, g.wsel0, nslot, E, N, st);
-        if (rc) return rc;
+        /* the rows of slots no expert serves are zeroed: by the matrix-vector form itself at a few rows (one launch
+         * less on a path that is all latency), by a launch of its own otherwise */
+        if (group_a16_gemv_serves(g)) {
+            g.zs_table = ten(in, T, 2), g.zs_nslot = nslot;
+        } else {
+            rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), g.wtab, g.stab, g.wcols, g.wsel0, nslot, E, N, st);
+            if (rc) return rc;
+        }
         return launch_group_down_a16(g, st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF:
@@ -745,9 +768,12 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             return launch_group_down_a16(g, st);
         }
         /* slot-major: sort the slots by expert into the context workspace (row_token = slot / k) */
-        rc = launch_align(c->ws.meta, ten(in, T, 2), c->ws.row_token, c->ws.row_partidx, c->ws.row_gate,
-                          nslot / kx, E, kx, c->ws.chunk_hist, c->ws.max_chunks, st);
-        if (rc) return rc;
+        if (!sort_reusable(h, ten(in, T, 2), nslot, E, kx, glu)) {
+            rc = launch_align(c->ws.meta, ten(in, T, 2), c->ws.row_token, c->ws.row_partidx, c->ws.row_gate,
+                              nslot / kx, E, kx, c->ws.chunk_hist, c->ws.max_chunks, st);
+            if (rc) return rc;
+            h.sorted_table = ten(in, T, 2), h.sorted_nslot = nslot, h.sorted_E = E, h.sorted_kx = kx;
+        }
         g.meta = c->ws.meta; g.slots_hint = nslot; g.o_idx = c->ws.row_partidx;
         if (glu) { g.a_idx = c->ws.row_token; return launch_group_glu_a16(g, st); }
         g.a_idx = c->ws.row_partidx; g.gate = c->ws.row_gate;
@@ -792,7 +818,7 @@ static int finish(PlowMoeCtx* c, int rc, const PlowDevInst* in) {
 
 /* the align op of a run states its routed slots (T * k) for the ops that follow it in the same run */
 static Hint hint_of_run(const PlowDevInst* insts, uint32_t n_inst, int form) {
-    Hint h = {form, 0u};
+    Hint h = {form, 0u, nullptr, 0u, 0u, 0u};
     for (uint32_t n = 0; n < n_inst; n++)
         if (insts[n].op == PLOW_DOP_MOE_ALIGN_PF) {
             const uint64_t slots = (uint64_t)insts[n].i[0] * insts[n].i[2];
@@ -803,7 +829,7 @@ static Hint hint_of_run(const PlowDevInst* insts, uint32_t n_inst, int form) {
 
 static int exec_run(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, void* const* tensors, void* stream,
                     int form) {
-    const Hint h = hint_of_run(insts, n_inst, form);
+    Hint h = hint_of_run(insts, n_inst, form);
     for (uint32_t n = 0; n < n_inst; n++) { /* refuse the whole run before launching any of it */
         const int rc = run_op(ctx, &insts[n], tensors, nullptr, false, h);
         if (rc) return rc;
@@ -818,13 +844,15 @@ static int exec_run(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, 
 extern "C" int plow_moe_check(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors) {
     if (!ctx || !inst || !tensors) return PLOW_MOE_EINVAL;
     ctx->err[0] = 0;
-    return run_op(ctx, inst, tensors, nullptr, false, Hint{-1, 0u});
+    Hint h = {-1, 0u, nullptr, 0u, 0u, 0u};
+    return run_op(ctx, inst, tensors, nullptr, false, h);
 }
 
 extern "C" int plow_moe_exec(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors, void* stream) {
     if (!ctx || !inst || !tensors) return PLOW_MOE_EINVAL;
     ctx->err[0] = 0;
-    return finish(ctx, run_op(ctx, inst, tensors, (hipStream_t)stream, true, Hint{-1, 0u}), inst);
+    Hint h = {-1, 0u, nullptr, 0u, 0u, 0u};
+    return finish(ctx, run_op(ctx, inst, tensors, (hipStream_t)stream, true, h), inst);
 }
 
 extern "C" int plow_moe_exec_many(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst,
@@ -862,7 +890,8 @@ extern "C" int plow_moe_exec_noalloc(const PlowDevInst* inst, void* const* tenso
     c.device = dev;
     c.min_rows[0] = c.min_rows[1] = -1;
     c.ws = ws_carve(base, PLOW_MOE_NOALLOC_MAX_EXPERTS, PLOW_MOE_NOALLOC_MAX_SLOTS); /* borrowed: ws_base stays NULL */
-    const int rc = finish(&c, run_op(&c, inst, tensors, (hipStream_t)stream, true, Hint{-1, 0u}), inst);
+    Hint h = {-1, 0u, nullptr, 0u, 0u, 0u};
+    const int rc = finish(&c, run_op(&c, inst, tensors, (hipStream_t)stream, true, h), inst);
     if (rc) say(c.err);
     return rc;
 }

@@ -125,6 +125,18 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
     const uint32_t srow_bytes = ENC == GV_MXFP4 ? K / 32u : (ENC == GV_FP8BLK ? (K / 128u) * 4u : 0u);
     const uint32_t wmul = g.wmul ? g.wmul : 1u;
 
+    /* slot-major DOWN: rows of slots that no expert serves are zeroed here, a slot per wave, while wave 0 of each
+     * workgroup lists the live rows */
+    if (!GLU && g.zs_table && !(g.out_bf16)) {
+        const PlowMoeRoute* const tab = (const PlowMoeRoute*)g.zs_table;
+        for (uint32_t sl = wave_id; sl < g.zs_nslot; sl += n_waves) {
+            const uint32_t e = tab[sl].eid;
+            const bool served = e < E && g.wtab[(size_t)e * g.wcols + g.wsel0] != 0ull &&
+                                (!g.stab || g.stab[(size_t)e * g.wcols + g.wsel0] != 0ull);
+            if (served) continue;
+            for (uint32_t h = lane; h < N; h += WAVE) ((float*)g.out)[(size_t)sl * N + h] = 0.0f;
+        }
+    }
     /* live rows in windows of GV_WINDOW, by their ordinal among the live rows */
     for (uint32_t base = 0;; base += GV_WINDOW) {
         __syncthreads();

@@ -171,6 +171,11 @@ struct GroupA16 {
     uint32_t* form_ws;
     const uint32_t* form_word;
     uint32_t form_want;
+    /* matrix-vector form, slot-major DOWN: when set, the routing table [zs_nslot] whose slots no expert serves
+     * (sentinel id, or an expert without resident weights) get their f32 output rows zeroed by this launch, as the
+     * reference's decode DOWN bodies do (plow runtime/cpu/dev/golden/moe.c:76-80) */
+    const void* zs_table;
+    uint32_t zs_nslot;
 };
 /* the matrix-vector form of the same ops for batches that route a handful of rows in all (slots_hint says so) */
 bool group_a16_gemv_serves(const GroupA16& g);

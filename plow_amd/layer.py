@@ -44,6 +44,8 @@ class MoeConfig:
     residual: bool = False
     part_bf16: bool = False         # block-fp8 W8A8 only: bf16 partials (arm 3) instead of f32
     router_raw: bool = False        # the score op carries its top-k (op 180 with the router mark): one launch at decode
+    emit_align: bool = True         # False: no op 84 in a chain whose expert ops are table driven (ops 65 / 66 sort the slots
+                                    # themselves; plow's decode chain for them is 56 -> 65 -> 66 -> 43)
     det_combine: bool = False       # block-fp8 W8A8 only: the deterministic fused down -> combine (op 83 zeroes a
                                     # [T][H] f64 fixed-point accumulator, op 86 adds into it, op 87 reads it as
                                     # one stream; plow runtime/amd/op_moe.h:2110-2165); no part tensor
@@ -168,8 +170,10 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
         p._emit("topk", abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[table, logit, part if det else None, bias],
                                  i=[H if det else 0, E, k, cfg.flags, T, cfg.tail, cfg.n_group, cfg.topk_group],
                                  f=[cfg.route_scale, 0.0]))
-    p._emit("align", abi.inst(abi.OP_MOE_ALIGN_PF, t=[meta, table, row_token, row_partidx, row_gate],
-                              i=[T, Ea, ka]))
+    slot_major = cfg.enc == "fp8pc" and cfg.arm != "w8a8"
+    if cfg.emit_align or not slot_major:
+        p._emit("align", abi.inst(abi.OP_MOE_ALIGN_PF, t=[meta, table, row_token, row_partidx, row_gate],
+                                  i=[T, Ea, ka]))
 
     if cfg.enc == "fp8pc":
         ewt = p._t("ewt", "u64", (Ea, 2), "table")
