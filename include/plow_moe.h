@@ -44,7 +44,7 @@ typedef struct {
                       * these ops carry no row count, and the kernel form that serves them best depends on
                       * it. Without it the count is taken from the align op (84) of the same
                       * plow_moe_exec_many / segment run, then from what the op's own operands imply,
-                      * then (fp8 x fp8 arms) from the routing meta on the device. Nothing is remembered
+                      * then (ops over a routing meta) from that meta on the device. Nothing is remembered
                       * between calls. The count only selects between kernel forms, which agree within
                       * the layer tolerance but not bit for bit: the tiled GLU takes SiLU from the
                       * hardware exp2 / reciprocal where the streaming form uses expf and an IEEE

@@ -103,10 +103,10 @@ def test_per_channel_fp8_layer(moe, oracle, T, arm):
                                            ("fp8pc", "a16", 300, 4, 2), ("fp8pc", "a16", 1030, 3, 1), ("fp8pc", "a16", 777, 8, 4),
                                            ("mxfp4", "a16", 300, 4, 2)])
 def test_bf16_activation_arms_many_rows(moe, oracle, enc, arm, T, E, k):
-    """Experts with 40..1030 rows on the bf16-activation arms: the fp8-weight arms (block and per-channel
-    scales) on the tiled kernels (from 16 rows per expert on average: partial, full and several 128-row
-    tiles, six 64-k blocks), bf16 and mxfp4 weights on passes of four (two) 16-row groups over the weights;
-    ragged last passes, pad rows, a folded shared expert of T rows."""
+    """Experts with 40..1030 rows on the bf16-activation arms, all on the tiled kernels (from 16 rows per
+    expert on average): fp8 weights (block and per-channel scales) and bf16 weights in 64-k blocks, mxfp4
+    weights in 128-k blocks; partial, full and several 128-row tiles, pad rows, a folded shared expert of
+    T rows."""
     print(f"[case] a16 many rows enc={enc} T={T} E={E} k={k}", flush=True)
     shared = dict(n_shared=1, shared_mode="fold") if enc != "fp8pc" else {}
     cfg = layer.MoeConfig("a16-rows", H=384, E=E, I=256, k=k, T=T, scoring="softmax", norm_topk=True, enc=enc, arm=arm, **shared)
