@@ -287,27 +287,54 @@ __global__ __launch_bounds__(AK_THREADS, GLU ? 2 : 4) void k_group_a16_stream(Gr
  * pass and 4 KB of weight rows per wave and step — three steps otherwise (mxfp4's step carries 8 KB of
  * activation rows and the E8M0 bytes; several row groups per pass multiply the activation ring) */
 template <int ENC, int RG> struct DmDepth { static constexpr uint32_t v = (ENC != AENC_MXFP4 && RG == 1) ? 4u : 3u; };
+#ifndef DM_MX_DOWN_STAGES1
+#define DM_MX_DOWN_STAGES1 6u
+#endif
+#ifndef DM_MX_DOWN_STAGES2
+#define DM_MX_DOWN_STAGES2 4u
+#endif
+/* Ring slots in use; loads are in flight for one step fewer. The GLU's two weight streams keep twice the bytes in
+ * flight per step and measured no faster at a fourth slot (the DOWN gained 3 %), so it stays at three. The mxfp4
+ * DOWN's step is 16 KB of weight rows per workgroup (one CU): two steps in flight are 32 KB, which does not keep the
+ * CU's share of the memory busy across the per-step barrier; its rings take what the LDS has. */
+template <int ENC, bool TWO, int RG> struct DmStages { /* TWO: two weight streams per wave (GLU; the wide DOWN) */
+    static constexpr uint32_t v = TWO ? 3u : (ENC == AENC_MXFP4 ? (RG == 1 ? DM_MX_DOWN_STAGES1 : DM_MX_DOWN_STAGES2) : DmDepth<ENC, RG>::v);
+};
 template <int ENC> struct DmGeom;
 template <> struct DmGeom<AENC_MXFP4> { static constexpr uint32_t KSTEP = 256u; };
 template <> struct DmGeom<AENC_FP8PC> { static constexpr uint32_t KSTEP = 128u; };
 template <> struct DmGeom<AENC_FP8BLK> { static constexpr uint32_t KSTEP = 128u; };
 template <> struct DmGeom<AENC_BF16> { static constexpr uint32_t KSTEP = 64u; };
-template <bool MX> struct DmWSlot;
-template <> struct DmWSlot<true> {
-    uint8_t w[2][16u * 128u]; /* [stream][row][128 B] */
-    uint8_t sc[2][256];       /* mxfp4: [stream][row][8 B]; lanes 32..63 write copies behind */
+/* mxfp4 scales, two ways. Chunked (MXC, rows of whole 16-byte pieces: K % 512 == 0): a wave brings the E8M0 bytes
+ * of FOUR steps, 32 bytes per weight row, with one 16-byte-per-lane direct load for both streams (lane = stream,
+ * row, half) into one of two buffers of its own; a row's scale line is then touched once per four steps and not once
+ * per step and stream, which matters because a step's weight rows push those lines out of the CU's 32 KB vector
+ * cache in between (Kimi-K2 shape, 128 tokens: GLU 1029 -> us). Per step otherwise: 8 bytes per row and stream
+ * into the ring slot. */
+template <bool SC, int NS> struct DmWSlot;
+template <int NS> struct DmWSlot<true, NS> {
+    uint8_t w[NS][16u * 128u]; /* [stream][row][128 B] */
+    uint8_t sc[NS][256];       /* [stream][row][8 B]; lanes 32..63 write copies behind */
 };
-template <> struct DmWSlot<false> {
-    uint8_t w[2][16u * 128u];
+template <int NS> struct DmWSlot<false, NS> {
+    uint8_t w[NS][16u * 128u];
 };
+/* A chunk's buffer is written again NB chunks later, when the load cursor, AH steps ahead of the multiplies, starts
+ * that chunk; the shortest chunk is two steps (K = 512, or the tail of K = 512 (2 j + 1)), so the multiplies have
+ * left it if AH <= 2 (NB - 1). */
+template <int NB, int NS> struct DmScaleChunks { uint8_t sch[AK_WAVES][NB][NS * 512]; }; /* [wave][buffer][stream][row][32 B] */
+template <int NS> struct DmScaleChunks<0, NS> {};
+template <uint32_t AH> struct DmChunkBufs { static constexpr int v = AH <= 2u ? 2 : (AH <= 4u ? 3 : 4); };
+template <bool ON> struct DmBlockScales;
+template <> struct DmBlockScales<true> { float bsc[4][2][128]; }; /* the weight block scales of the workgroup's tiles, all of K (K <= 16384) */
+template <> struct DmBlockScales<false> {};
 /* RG = 16-row groups of activation rows per pass over the weights: 1, 2 or 4 (mxfp4: 1 or 2), picked per
  * workgroup from its expert's row count: with more groups the weights are streamed less often and every
  * weight operand read from LDS feeds that many matrix instructions */
-template <int ENC, int RG>
-struct DmLds {
-    uint8_t x[DmDepth<ENC, RG>::v][RG * 16u * DmGeom<ENC>::KSTEP * 2u];
-    DmWSlot<ENC == AENC_MXFP4> ring[AK_WAVES][DmDepth<ENC, RG>::v];
-    float bsc[4][2][128]; /* block-fp8: the weight block scales of the workgroup's tiles, all of K (K <= 16384) */
+template <int ENC, bool TWO, int RG, bool MXC = false>
+struct DmLds : DmScaleChunks<MXC ? DmChunkBufs<DmStages<ENC, TWO, RG>::v - 1u>::v : 0, TWO ? 2 : 1>, DmBlockScales<ENC == AENC_FP8BLK> { /* bases: empty ones take no room */
+    uint8_t x[DmStages<ENC, TWO, RG>::v][RG * 16u * DmGeom<ENC>::KSTEP * 2u];
+    DmWSlot<ENC == AENC_MXFP4 && !MXC, TWO ? 2 : 1> ring[AK_WAVES][DmStages<ENC, TWO, RG>::v];
 };
 typedef __attribute__((address_space(3))) void dm_lds_void;
 __device__ __forceinline__ uint32_t dm_lds_off(const void* p) {
@@ -332,14 +359,26 @@ __device__ __forceinline__ float dm_read4(uint32_t addr) {
  * workgroup barrier */
 #define DM_WAIT_BARRIER(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(n) : "memory")
 
+/* the wait + barrier for `after` (at most A) steps of PER loads each still allowed in flight */
+template <int A, int PER>
+__device__ __forceinline__ void dm_wait_steps(uint32_t after) {
+    static_assert(A * PER <= 63, "the load counter holds six bits");
+    if constexpr (A == 0) {
+        DM_WAIT_BARRIER(0);
+    } else {
+        if (after == (uint32_t)A) DM_WAIT_BARRIER(A * PER);
+        else dm_wait_steps<A - 1, PER>(after);
+    }
+}
+
 /* What workgroup index `bid` of a logical grid of E * N / 128 works on: expert e (cnt rows), TPW channel tiles
  * from tile ct. False when it has nothing to do. */
 struct DmWork {
     uint32_t e, ct, TPW, cnt;
 };
-template <int ENC>
+template <int ENC, bool WIDE = false>
 __device__ __forceinline__ bool a16_dma_work(const GroupA16& g, uint32_t bid, DmWork& w) {
-    const uint32_t tiles = g.N / AK_BN;
+    const uint32_t tiles = g.N / (WIDE ? 2u * AK_BN : AK_BN);
     /* With plenty of tiles to go round and a short K loop, a workgroup takes TPW consecutive channel tiles
      * of its expert and keeps the load rings running across them, which hides the ramp of the loop. meta[3E], the
      * number of 64-row tiles, is at least the number of experts with rows. The grid has one workgroup per
@@ -359,22 +398,31 @@ __device__ __forceinline__ bool a16_dma_work(const GroupA16& g, uint32_t bid, Dm
 
 /* The body takes its LDS as a pointer, so that a kernel with a fixed launch shape (any 1-D grid, static LDS) can
  * walk the logical grid itself. */
-template <int ENC, bool GLU, int RG>
+/* WIDE (DOWN only): a wave owns 32 channels, two 16-row weight operands that share the activation operand, and the
+ * workgroup a tile of 256: the GLU's shape with the second stream 16 channels further down the same matrix. A step
+ * is then 32 KB of weight rows per workgroup instead of 16: half the barriers, waits and activation-row reads per
+ * weight byte. */
+template <int ENC, bool GLU, int RG, bool MXC = false, bool WIDE = false>
 __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw, const DmWork& work) {
-    DmLds<ENC, RG>& L = *(DmLds<ENC, RG>*)dm_raw;
-    /* ring slots in use; steps of loads in flight. The GLU's two weight streams already keep twice the bytes in
-     * flight per step and measured no faster at the fourth slot (the DOWN gained 3 %), so it stays at three */
-    constexpr uint32_t DM_STAGES = GLU ? 3u : DmDepth<ENC, RG>::v, AH = DM_STAGES - 1u;
-    typedef DmWSlot<ENC == AENC_MXFP4> Slot;
+    static_assert(!MXC || ENC == AENC_MXFP4, "chunked scales are the mxfp4 arm's");
+    static_assert(!(GLU && WIDE), "the wide form is the DOWN's");
+    constexpr bool TWO = GLU || WIDE;                   /* two weight streams per wave */
+    constexpr uint32_t BN = WIDE ? 2u * AK_BN : AK_BN;   /* channels per workgroup tile */
+    DmLds<ENC, TWO, RG, MXC>& L = *(DmLds<ENC, TWO, RG, MXC>*)dm_raw;
+    constexpr uint32_t DM_STAGES = DmStages<ENC, TWO, RG>::v, AH = DM_STAGES - 1u; /* ring slots; steps of loads in flight */
+    typedef DmWSlot<ENC == AENC_MXFP4 && !MXC, TWO ? 2 : 1> Slot;
     constexpr uint32_t KSTEP = DmGeom<ENC>::KSTEP, XROW = KSTEP * 2u; /* activation bytes per row and step */
     constexpr uint32_t NP = XROW / 16u;                              /* 16-byte pieces per activation row */
     constexpr uint32_t XL = RG * 16u * XROW / 1024u;                 /* 1 KB activation loads per step */
     constexpr uint32_t XRPL = 64u / NP;                              /* rows per activation load */
     constexpr uint32_t NXI = (XL + AK_WAVES - 1u) / AK_WAVES;        /* activation loads per wave and step (wave w: w, w + 8, ..) */
     static_assert(XL < AK_WAVES || XL % AK_WAVES == 0u, "activation loads must split evenly over the waves");
-    constexpr int NS = GLU ? 2 : 1;
-    /* direct loads per wave and step: weights 2 per stream, mxfp4 scales 1 per stream, rows NXI (waves below XL) */
-    constexpr int NLW = NS * (ENC == AENC_MXFP4 ? 3 : 2);
+    constexpr int NS = TWO ? 2 : 1;
+    /* direct loads per wave and step: weights 2 per stream, mxfp4 scales 1 per stream, rows NXI (waves below XL).
+     * Chunked mxfp4 scales are one more load every fourth step and not counted: a wait that allows n loads to be
+     * outstanding asks for everything older than the newest n, so an uncounted load makes it stricter by one and
+     * never looser. */
+    constexpr int NLW = NS * ((ENC == AENC_MXFP4 && !MXC) ? 3 : 2);
     const uint32_t e = work.e, ct = work.ct, TPW = work.TPW, cnt = work.cnt;
     const uint64_t* wt = g.wtab ? g.wtab + (size_t)e * g.wcols : nullptr;
     const uint64_t* stt = g.stab ? g.stab + (size_t)e * g.wcols : nullptr;
@@ -385,7 +433,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, k-chunk q */
     const uint32_t K = g.K, KS = K / KSTEP, N = g.N, GS = TPW * KS; /* steps of a pass over all its tiles */
-    const uint32_t chw = ct * AK_BN + wv * 16u;   /* this wave's first channel */
+    const uint32_t chw = ct * BN + wv * (WIDE ? 32u : 16u); /* this wave's first channel */
     const uint32_t wrow = ENC == AENC_BF16 ? K * 2u : (ENC == AENC_MXFP4 ? K / 2u : K); /* bytes per weight row */
     const uint32_t wmul = g.wmul ? g.wmul : 1u;
 
@@ -396,30 +444,41 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
     const float* pcs[2] = {nullptr, nullptr}; /* per-channel fp8: this lane's four output scales per stream */
 #pragma unroll
     for (int sidx = 0; sidx < NS; sidx++) {
-        const uint32_t sel = sidx ? g.wsel1 : g.wsel0;
-        const uint8_t* wbase = wt ? (const uint8_t*)(uintptr_t)wt[sel] : (const uint8_t*)g.wdirect[sidx];
+        /* the wide DOWN's second stream is the same matrix, 16 channels on */
+        const uint32_t sel = (sidx && !WIDE) ? g.wsel1 : g.wsel0;
+        const uint8_t* wbase = wt ? (const uint8_t*)(uintptr_t)wt[sel] : (const uint8_t*)g.wdirect[WIDE ? 0 : sidx];
         const uint8_t* sbase = stt ? (const uint8_t*)(uintptr_t)stt[sel] : nullptr;
-        const uint32_t wr0 = sidx ? g.wrow1 : g.wrow0;
+        const uint32_t wr0 = (sidx && !WIDE) ? g.wrow1 : g.wrow0;
+        const uint32_t chs = chw + ((sidx && WIDE) ? 16u : 0u); /* the stream's first channel */
 #pragma unroll
         for (uint32_t j = 0; j < 2u; j++) {
             const uint32_t R = 8u * j + lr;
-            wsrc[sidx][j] = wbase + (size_t)((chw + R) * wmul + wr0) * wrow + ((p ^ lds_swz8(R)) << 4);
+            wsrc[sidx][j] = wbase + (size_t)((chs + R) * wmul + wr0) * wrow + ((p ^ lds_swz8(R)) << 4);
         }
         /* mxfp4 scales: lane -> (row (lane & 31) >> 1, dword lane & 1) of the step's 8 bytes per row */
-        if (ENC == AENC_MXFP4)
-            ssrc[sidx] = sbase + (size_t)((chw + ((lane & 31u) >> 1)) * wmul + wr0) * (K / 32u) + (lane & 1u) * 4u;
-        if (ENC == AENC_FP8PC) pcs[sidx] = (const float*)sbase + wr0 + chw + 4u * q;
-        if (ENC == AENC_FP8BLK) { /* the channel blocks' scale rows go to LDS once */
+        if (ENC == AENC_MXFP4 && !MXC)
+            ssrc[sidx] = sbase + (size_t)((chs + ((lane & 31u) >> 1)) * wmul + wr0) * (K / 32u) + (lane & 1u) * 4u;
+        /* chunked: lanes 0..31 bring the first stream's bytes, lanes 32..63 the second's (one stream: they stay out);
+         * lane -> (row (lane & 31) >> 1, 16-byte half lane & 1) of the chunk's 32 bytes per row */
+        if (MXC && (sidx == 0 ? (lane < 32u || !TWO) : lane >= 32u))
+            ssrc[0] = sbase + (size_t)((chs + ((lane & 31u) >> 1)) * wmul + wr0) * (K / 32u) + (lane & 1u) * 16u;
+        if (ENC == AENC_FP8PC) pcs[sidx] = (const float*)sbase + wr0 + chs + 4u * q;
+        if (ENC == AENC_FP8BLK) { /* the channel blocks' scale rows go to LDS once (wide: the tile's two blocks) */
             for (uint32_t t = 0; t < TPW; t++) {
-                const float* bs = (const float*)sbase + (size_t)(((ct + t) * AK_BN + wr0) / 128u) * (K / 128u);
-                for (uint32_t i = threadIdx.x; i < K / 128u; i += AK_THREADS) L.bsc[t][sidx][i] = bs[i];
+                const float* bs = (const float*)sbase + (size_t)(((ct + t) * BN + (WIDE ? 128u * sidx : 0u) + wr0) / 128u) * (K / 128u);
+                if constexpr (ENC == AENC_FP8BLK)
+                    for (uint32_t i = threadIdx.x; i < K / 128u; i += AK_THREADS) L.bsc[t][sidx][i] = bs[i];
             }
         }
     }
     const uint32_t swz = lds_swz8(c), swx = lds_swz16(c);
     const uint32_t x_base = dm_lds_off(&L.x[0][0]);
     const uint32_t w_base = dm_lds_off(&L.ring[wv][0]);
-    const uint32_t b_base = dm_lds_off(&L.bsc[0][0][0]);
+    uint32_t b_base = 0u, sch_base = 0u;
+    if constexpr (ENC == AENC_FP8BLK) b_base = dm_lds_off(&L.bsc[0][0][0]);
+    constexpr uint32_t CKB = (uint32_t)DmChunkBufs<AH>::v, CKSZ = NS * 512u; /* scale chunk buffers and their size */
+    static_assert(AH <= 2u * (CKB - 1u), "a scale buffer must be free when its next chunk is loaded");
+    if constexpr (MXC) sch_base = dm_lds_off(&L.sch[wv][0][0]) + c * 32u;
     /* LDS position of logical piece P of activation row c */
     auto xpos = [&](uint32_t P) -> uint32_t { return NP >= 16u ? ((P & ~15u) | ((P ^ swx) & 15u)) : (P ^ swz); };
 
@@ -473,8 +532,8 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
             for (uint32_t t = 0; t < 4u; t++) {
                 pc0[t] = pc1[t] = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
                 if (t < TPW) {
-                    pc0[t] = *(const float4*)(pcs[0] + t * AK_BN);
-                    if (GLU) pc1[t] = *(const float4*)(pcs[1] + t * AK_BN);
+                    pc0[t] = *(const float4*)(pcs[0] + t * BN);
+                    if (TWO) pc1[t] = *(const float4*)(pcs[1] + t * BN);
                 }
             }
         }
@@ -489,31 +548,57 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
         }
 
         /* the load cursor walks (tile, step) in order; ring slots follow the running step count */
-        uint32_t ld_t = 0, ld_S = 0, ld_st = 0;
+        /* the cursor's addresses run along: one line on per step, from a tile's last step to the next tile's first */
+        uint32_t ld_S = 0, ld_st = 0, ld_ck = 0;
+        const uint8_t* wp[2][2] = {{wsrc[0][0], wsrc[0][1]}, {wsrc[1][0], wsrc[1][1]}};
+        const uint8_t* sp[2] = {ssrc[0], ssrc[1]};
+        const uint8_t* xp[NXI];
+#pragma unroll
+        for (uint32_t i = 0; i < NXI; i++) xp[i] = xsrc[i];
+        const size_t w_next = (size_t)BN * wmul * wrow - (size_t)KS * 128u, s_next = (size_t)BN * wmul * (K / 32u) - (size_t)KS * 8u;
         auto issue = [&]() {
             Slot* slot = &L.ring[wv][ld_st];
-            const size_t wofs = (size_t)ld_t * AK_BN * wmul * wrow + (size_t)ld_S * 128u;
+            if constexpr (MXC) {
+                if ((ld_S & 3u) == 0u) { /* the E8M0 bytes of steps ld_S .. ld_S + 3, ahead of the step's own loads */
+                    /* a half whose two steps lie past the row's end reads the first half again */
+                    const uint32_t back = (ld_S + 2u * (lane & 1u) < KS) ? 0u : 16u;
+                    if (TWO || lane < 32u)
+                        __builtin_amdgcn_global_load_lds((const void*)(sp[0] - back), (dm_lds_void*)&L.sch[wv][ld_ck][0], 16, 0, 0);
+                    ld_ck = ld_ck + 1u == CKB ? 0u : ld_ck + 1u;
+                }
+            }
 #pragma unroll
             for (int sidx = 0; sidx < NS; sidx++) {
 #pragma unroll
-                for (uint32_t j = 0; j < 2u; j++)
-                    __builtin_amdgcn_global_load_lds((const void*)(wsrc[sidx][j] + wofs),
-                                                     (dm_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, LOAD_NT);
-                if constexpr (ENC == AENC_MXFP4)
-                    __builtin_amdgcn_global_load_lds((const void*)(ssrc[sidx] + (size_t)ld_t * AK_BN * wmul * (K / 32u) + (size_t)ld_S * 8u),
-                                                     (dm_lds_void*)&slot->sc[sidx][0], 4, 0, 0); /* 8 bytes of a line per step: cached */
+                for (uint32_t j = 0; j < 2u; j++) {
+                    __builtin_amdgcn_global_load_lds((const void*)wp[sidx][j], (dm_lds_void*)&slot->w[sidx][8u * j * 128u], 16, 0, LOAD_NT);
+                    wp[sidx][j] += 128u;
+                }
+                if constexpr (ENC == AENC_MXFP4 && !MXC)
+                    __builtin_amdgcn_global_load_lds((const void*)sp[sidx], (dm_lds_void*)&slot->sc[sidx][0], 4, 0, 0); /* 8 bytes of a line per step: cached */
+                if constexpr (ENC == AENC_MXFP4) sp[sidx] += 8u;
             }
 #pragma unroll
             for (uint32_t i = 0; i < NXI; i++)
                 if (wv + AK_WAVES * i < XL) {
-                    if (XRPL * (wv + AK_WAVES * i) < live)
-                        __builtin_amdgcn_global_load_lds((const void*)(xsrc[i] + (size_t)ld_S * XROW),
-                                                         (dm_lds_void*)&L.x[ld_st][XRPL * (wv + AK_WAVES * i) * XROW], 16, 0, 0);
-                    else /* rows past the expert's last: a stand-in that keeps the load count */
+                    if (XRPL * (wv + AK_WAVES * i) < live) {
+                        __builtin_amdgcn_global_load_lds((const void*)xp[i], (dm_lds_void*)&L.x[ld_st][XRPL * (wv + AK_WAVES * i) * XROW], 16, 0, 0);
+                        xp[i] += XROW;
+                    } else { /* rows past the expert's last: a stand-in that keeps the load count */
                         __builtin_amdgcn_global_load_lds((const void*)xdummy, (dm_lds_void*)&L.x[ld_st][XRPL * (wv + AK_WAVES * i) * XROW], 4, 0, 0);
+                    }
                 }
             ld_st = ld_st + 1u == DM_STAGES ? 0u : ld_st + 1u;
-            if (++ld_S == KS) ld_S = 0u, ld_t++;
+            if (++ld_S == KS) { /* on to the next tile of the expert: its weight rows, the same activation rows again */
+                ld_S = 0u;
+#pragma unroll
+                for (int sidx = 0; sidx < NS; sidx++) {
+                    wp[sidx][0] += w_next, wp[sidx][1] += w_next;
+                    if constexpr (ENC == AENC_MXFP4) sp[sidx] += s_next;
+                }
+#pragma unroll
+                for (uint32_t i = 0; i < NXI; i++) xp[i] = xsrc[i];
+            }
         };
         v4f acc0[RG], acc1[RG];
 #pragma unroll
@@ -521,42 +606,58 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
         /* the row maps above are loaded (the count of outstanding loads starts at zero), and every wave
          * has left the pass before (its ring slots are free; the block scales are written) */
         DM_WAIT_BARRIER(0);
-        issue();
-        if (GS > 1u) issue();
-        if (AH > 2u && GS > 2u) issue();
-        uint32_t st = 0;
+#pragma unroll
+        for (uint32_t i = 0; i < AH; i++)
+            if (i < GS) issue();
+        uint32_t st = 0, ck = CKB - 1u; /* ck: the scale buffer of the chunk being used */
         for (uint32_t G = 0, t = 0, S = 0; G < GS; G++) {
+            if (MXC && (S & 3u) == 0u) ck = ck + 1u == CKB ? 0u : ck + 1u;
             /* loads return in order: step G has landed once at most the steps after it that were issued (AH - 1
              * of them, fewer at the end) are outstanding; after the barrier every wave's share of the rows is
              * there and nobody reads step G - 1 any more */
             const uint32_t after = GS - 1u - G < AH - 1u ? GS - 1u - G : AH - 1u; /* steps in flight behind step G */
             const bool loads_x = XL >= AK_WAVES || wv < XL;
-            if (after == 0u) DM_WAIT_BARRIER(0);
-            else if (after == 1u) { if (loads_x) DM_WAIT_BARRIER(NLW + (int)NXI); else DM_WAIT_BARRIER(NLW); }
-            else { if (loads_x) DM_WAIT_BARRIER(2 * (NLW + (int)NXI)); else DM_WAIT_BARRIER(2 * NLW); }
-            if (G + AH < GS) issue();
+            if (loads_x) dm_wait_steps<(int)AH - 1, NLW + (int)NXI>(after);
+            else dm_wait_steps<(int)AH - 1, NLW>(after);
+            /* mxfp4 (twice the multiplies and conversions per weight byte): the step's operand reads go out first and
+             * cross the LDS while the loads below are being issued */
+            if (ENC != AENC_MXFP4 && G + AH < GS) issue();
             const uint32_t wb = w_base + st * (uint32_t)sizeof(Slot), xb0 = x_base + st * (RG * 16u * XROW) + c * XROW;
             /* the weight operands of the step are read once and multiply every row group of the pass */
             if constexpr (ENC == AENC_MXFP4) {
-                uint2 e0 = dm_read8(wb + 4096u + c * 8u), e1 = e0;
-                if (GLU) e1 = dm_read8(wb + 4096u + 256u + c * 8u);
+                uint2 e0, e1;
+                if constexpr (MXC) {
+                    const uint32_t sa8 = sch_base + ck * CKSZ + (S & 3u) * 8u;
+                    e0 = dm_read8(sa8), e1 = e0;
+                    if (TWO) e1 = dm_read8(sa8 + 512u);
+                } else {
+                    e0 = dm_read8(wb + NS * 2048u + c * 8u), e1 = e0;
+                    if (TWO) e1 = dm_read8(wb + NS * 2048u + 256u + c * 8u);
+                }
                 v4i wa[2], wbv[2];
 #pragma unroll
                 for (uint32_t u = 0; u < 2u; u++) {
                     const uint32_t wo = c * 128u + (((4u * u + q) ^ swz) << 4);
                     wa[u] = dm_read16(wb + wo);
                     wbv[u] = wa[u];
-                    if (GLU) wbv[u] = dm_read16(wb + 2048u + wo);
+                    if (TWO) wbv[u] = dm_read16(wb + 2048u + wo);
                 }
+                v4i xa[2][4];
+#pragma unroll
+                for (uint32_t u = 0; u < 2u; u++)
+#pragma unroll
+                    for (uint32_t j = 0; j < 4u; j++) xa[u][j] = dm_read16(xb0 + (xpos(16u * u + 4u * q + j) << 4));
+                if (G + AH < GS) issue();
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e0), "+v"(e1), "+v"(wa[0]), "+v"(wa[1]), "+v"(wbv[0]), "+v"(wbv[1]));
 #pragma unroll
                 for (int rg = 0; rg < RG; rg++) {
-                    const uint32_t xb = xb0 + (uint32_t)rg * (16u * XROW);
-                    v4i xa[2][4];
+                    if (rg) {
+                        const uint32_t xb = xb0 + (uint32_t)rg * (16u * XROW);
 #pragma unroll
-                    for (uint32_t u = 0; u < 2u; u++)
+                        for (uint32_t u = 0; u < 2u; u++)
 #pragma unroll
-                        for (uint32_t j = 0; j < 4u; j++) xa[u][j] = dm_read16(xb + (xpos(16u * u + 4u * q + j) << 4));
+                            for (uint32_t j = 0; j < 4u; j++) xa[u][j] = dm_read16(xb + (xpos(16u * u + 4u * q + j) << 4));
+                    }
                     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[0][0]), "+v"(xa[0][1]), "+v"(xa[0][2]), "+v"(xa[0][3]));
                     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa[1][0]), "+v"(xa[1][1]), "+v"(xa[1][2]), "+v"(xa[1][3]));
 #pragma unroll
@@ -569,7 +670,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                         for (int j = 0; j < 4; j++) {
                             const v8bf B = __builtin_bit_cast(v8bf, xa[u][j]);
                             acc0[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(da, j, s0), B, acc0[rg], 0, 0, 0);
-                            if (GLU) acc1[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(db, j, s1), B, acc1[rg], 0, 0, 0);
+                            if (TWO) acc1[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<AENC_MXFP4>(db, j, s1), B, acc1[rg], 0, 0, 0);
                         }
                     }
                 }
@@ -581,7 +682,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                     const uint32_t wo = c * 128u + (((4u * j + q) ^ swz) << 4);
                     wa[j] = dm_read16(wb + wo);
                     wbv[j] = wa[j];
-                    if (GLU) wbv[j] = dm_read16(wb + 2048u + wo);
+                    if (TWO) wbv[j] = dm_read16(wb + 2048u + wo);
                 }
                 v4i xr[2][2];
 #pragma unroll
@@ -600,7 +701,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                     for (int j = 0; j < 2; j++) {
                         const v8bf B = __builtin_bit_cast(v8bf, xa[j]);
                         acc0[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wa[j]), B, acc0[rg], 0, 0, 0);
-                        if (GLU) acc1[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wbv[j]), B, acc1[rg], 0, 0, 0);
+                        if (TWO) acc1[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wbv[j]), B, acc1[rg], 0, 0, 0);
                     }
                 }
             } else {
@@ -613,10 +714,11 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                     const uint32_t wo = c * 128u + (((4u * h + q) ^ swz) << 4);
                     da.r[h] = dm_read16(wb + wo);
                     db.r[h] = da.r[h];
-                    if (GLU) db.r[h] = dm_read16(wb + 2048u + wo);
+                    if (TWO) db.r[h] = dm_read16(wb + 2048u + wo);
                 }
                 if (ENC == AENC_FP8BLK) {
-                    sa = dm_read4(b_base + t * 1024u + S * 4u);
+                    /* wide: both streams lie in one 128-channel block, the tile's first (waves 0..3) or second */
+                    sa = dm_read4(b_base + t * 1024u + (WIDE ? (wv >> 2) * 512u : 0u) + S * 4u);
                     sb = sa;
                     if (GLU) sb = dm_read4(b_base + t * 1024u + 512u + S * 4u);
                 }
@@ -640,17 +742,19 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                     for (int j = 0; j < 4; j++) {
                         const v8bf B = __builtin_bit_cast(v8bf, xa[j]);
                         t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(da, j), B, t0, 0, 0, 0);
-                        if (GLU) t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(db, j), B, t1, 0, 0, 0);
+                        if (TWO) t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_operand<ENC>(db, j), B, t1, 0, 0, 0);
                     }
                     if (ENC == AENC_FP8BLK) {
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
                             acc0[rg][i] = fmaf(t0[i], sa, acc0[rg][i]);
-                            if (GLU) acc1[rg][i] = fmaf(t1[i], sb, acc1[rg][i]);
+                            /* (wide: the block's one scale; a copy of sa made before the wait above would hold
+                             * what the register held before the read landed) */
+                            if (TWO) acc1[rg][i] = fmaf(t1[i], WIDE ? sa : sb, acc1[rg][i]);
                         }
                     } else {
                         acc0[rg] = t0;
-                        if (GLU) acc1[rg] = t1;
+                        if (TWO) acc1[rg] = t1;
                     }
                 }
             }
@@ -659,7 +763,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
             /* ---- a tile is done: lane holds channels chw + 128 t + 4q + i of row rb + c ---- */
             const uint32_t tdone = t;
             S = 0u, t++;
-            const uint32_t col = chw + tdone * AK_BN + 4u * q;
+            const uint32_t col = chw + tdone * BN + 4u * q;
             float4 s0 = pc0[0], s1 = pc1[0];
             if (ENC == AENC_FP8PC) {
 #pragma unroll
@@ -673,7 +777,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                 if (!valid[rg] || oi[rg] == PLOW_EXPERT_UNUSED) continue;
                 if (ENC == AENC_FP8PC) {
                     a0[0] *= s0.x, a0[1] *= s0.y, a0[2] *= s0.z, a0[3] *= s0.w;
-                    if (GLU) a1[0] *= s1.x, a1[1] *= s1.y, a1[2] *= s1.z, a1[3] *= s1.w;
+                    if (TWO) a1[0] *= s1.x, a1[1] *= s1.y, a1[2] *= s1.z, a1[3] *= s1.w;
                 }
                 if (GLU) {
                     uint2 o;
@@ -682,18 +786,41 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                     *(uint2*)((bf16_t*)g.out + (size_t)oi[rg] * N + col) = o;
                 } else {
                     const float gt = gate[rg];
-                    const float y0 = gt * a0[0], y1 = gt * a0[1], y2 = gt * a0[2], y3 = gt * a0[3];
-                    if (g.out_bf16) {
-                        uint2 o;
-                        o.x = (uint32_t)f2bf(g.gate ? y0 : a0[0]) | ((uint32_t)f2bf(g.gate ? y1 : a0[1]) << 16);
-                        o.y = (uint32_t)f2bf(g.gate ? y2 : a0[2]) | ((uint32_t)f2bf(g.gate ? y3 : a0[3]) << 16);
-                        *(uint2*)((bf16_t*)g.out + (size_t)oi[rg] * N + col) = o;
-                    } else {
-                        *(float4*)((float*)g.out + (size_t)oi[rg] * N + col) = make_float4(y0, y1, y2, y3);
-                    }
+                    auto put = [&](const v4f& a, uint32_t cl) {
+                        const float y0 = gt * a[0], y1 = gt * a[1], y2 = gt * a[2], y3 = gt * a[3];
+                        if (g.out_bf16) {
+                            uint2 o;
+                            o.x = (uint32_t)f2bf(g.gate ? y0 : a[0]) | ((uint32_t)f2bf(g.gate ? y1 : a[1]) << 16);
+                            o.y = (uint32_t)f2bf(g.gate ? y2 : a[2]) | ((uint32_t)f2bf(g.gate ? y3 : a[3]) << 16);
+                            *(uint2*)((bf16_t*)g.out + (size_t)oi[rg] * N + cl) = o;
+                        } else {
+                            *(float4*)((float*)g.out + (size_t)oi[rg] * N + cl) = make_float4(y0, y1, y2, y3);
+                        }
+                    };
+                    put(a0, col);
+                    if (WIDE) put(a1, col + 16u); /* the second stream's channels */
                 }
             }
         }
+    }
+}
+
+template <int ENC, bool GLU, bool WIDE>
+__device__ __forceinline__ void a16_dma_pick(const GroupA16& g, uint8_t* dm_raw) {
+    DmWork w;
+    if (!a16_dma_work<ENC, WIDE>(g, blockIdx.x, w)) return;
+    if constexpr (ENC == AENC_MXFP4) {
+        if (g.K % 512u == 0u) { /* whole 16-byte pieces of E8M0 bytes per row: scales four steps at a time */
+            if (w.cnt <= 16u) a16_dma_body<ENC, GLU, 1, true, WIDE>(g, dm_raw, w);
+            else a16_dma_body<ENC, GLU, 2, true, WIDE>(g, dm_raw, w);
+        } else {
+            if (w.cnt <= 16u) a16_dma_body<ENC, GLU, 1, false, WIDE>(g, dm_raw, w);
+            else a16_dma_body<ENC, GLU, 2, false, WIDE>(g, dm_raw, w);
+        }
+    } else {
+        if (w.cnt <= 16u) a16_dma_body<ENC, GLU, 1, false, WIDE>(g, dm_raw, w);
+        else if (w.cnt <= 32u) a16_dma_body<ENC, GLU, 2, false, WIDE>(g, dm_raw, w);
+        else a16_dma_body<ENC, GLU, 4, false, WIDE>(g, dm_raw, w);
     }
 }
 
@@ -705,22 +832,31 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
 template <int ENC, bool GLU>
 __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
-    DmWork w;
-    if (!form_is_mine(g) || !a16_dma_work<ENC>(g, blockIdx.x, w)) return;
-    if (w.cnt <= 16u) a16_dma_body<ENC, GLU, 1>(g, dm_raw, w);
-    else if (ENC == AENC_MXFP4 || w.cnt <= 32u) a16_dma_body<ENC, GLU, 2>(g, dm_raw, w);
-    else a16_dma_body<ENC, GLU, ENC == AENC_MXFP4 ? 2 : 4>(g, dm_raw, w);
+    if (!form_is_mine(g)) return;
+    if constexpr (!GLU) {
+        if (g.down_wide) { /* tiles of 256 channels (the launcher's grid counts them so) */
+            a16_dma_pick<ENC, GLU, true>(g, dm_raw);
+            return;
+        }
+    }
+    a16_dma_pick<ENC, GLU, false>(g, dm_raw);
 }
 
-template <int ENC> struct DmLdsMax {
-    static constexpr size_t a = sizeof(DmLds<ENC, 1>), b = sizeof(DmLds<ENC, 2>),
-                            c = sizeof(DmLds<ENC, ENC == AENC_MXFP4 ? 2 : 4>);
-    static constexpr size_t v = a > b ? (a > c ? a : c) : (b > c ? b : c);
+template <int ENC, bool TWO> struct DmLdsMax2 { /* over the row-group counts and scale forms of one stream count */
+    static constexpr bool MX = ENC == AENC_MXFP4;
+    static constexpr size_t a = sizeof(DmLds<ENC, TWO, 1, false>), b = sizeof(DmLds<ENC, TWO, 2, false>),
+                            c = MX ? sizeof(DmLds<ENC, TWO, 2, MX>) : sizeof(DmLds<ENC, TWO, 4, false>),
+                            d = sizeof(DmLds<ENC, TWO, 1, MX>);
+    static constexpr size_t ab = a > b ? a : b, cd = c > d ? c : d, v = ab > cd ? ab : cd;
+};
+template <int ENC, bool GLU> struct DmLdsMax { /* the DOWN kernel holds the one-stream and the wide bodies */
+    static constexpr size_t two = DmLdsMax2<ENC, true>::v, one = DmLdsMax2<ENC, false>::v;
+    static constexpr size_t v = GLU ? two : (two > one ? two : one);
 };
 template <int ENC, bool GLU>
 static int launch_a16_dma(const GroupA16& g, dim3 grid, hipStream_t st) {
-    static_assert(DmLdsMax<ENC>::v <= 160u * 1024u, "the rings must fit the CU's LDS");
-    k_group_a16_dma<ENC, GLU><<<grid, AK_THREADS, DmLdsMax<ENC>::v, st>>>(g);
+    static_assert(DmLdsMax<ENC, GLU>::v <= 160u * 1024u, "the rings must fit the CU's LDS");
+    k_group_a16_dma<ENC, GLU><<<grid, AK_THREADS, DmLdsMax<ENC, GLU>::v, st>>>(g);
     return 0;
 }
 
@@ -793,7 +929,7 @@ static int launch_a16(const GroupA16& g_in, hipStream_t st) {
             g.form_word = g.form_ws, g.form_want = 0u;
         }
     }
-    const dim3 grid(g.E * (g.N / AK_BN));
+    dim3 grid(g.E * (g.N / AK_BN));
     /* second form: needs whole steps of K (one 128-byte line per weight row) and the block scales of a
      * tile to fit its LDS table */
     bool dma = !plow_moe_tuning().a16_regs && !g.bias && g.K <= 16384u &&
@@ -808,6 +944,14 @@ static int launch_a16(const GroupA16& g_in, hipStream_t st) {
         const uint64_t wgs = (uint64_t)(g.slots_hint < g.E ? g.slots_hint : g.E) * (g.N / AK_BN);
         const uint32_t steps = g.K / (g.enc == AENC_MXFP4 ? 256u : (g.enc == AENC_BF16 ? 64u : 128u));
         if (steps <= 16u && wgs > (uint64_t)n_cu && wgs < 3ull * (uint64_t)n_cu) dma = false;
+    }
+    g.down_wide = 0u;
+    if (!GLU && dma && g.N % (2u * AK_BN) == 0u && g.meta && plow_moe_tuning().a16_down_wide) {
+        /* tiles of 256 channels while they still give every CU two workgroups and more */
+        const uint32_t n_cu = plow_moe_n_cu();
+        if (!n_cu) return PLOW_MOE_EDEVICE;
+        const uint64_t hit = g.slots_hint && g.slots_hint < g.E ? g.slots_hint : g.E;
+        if (hit * (g.N / (2u * AK_BN)) >= 2ull * n_cu) g.down_wide = 1u, grid = dim3(g.E * (g.N / (2u * AK_BN)));
     }
     switch (g.enc) {
     case AENC_BF16:
@@ -835,7 +979,7 @@ static int launch_a16(const GroupA16& g_in, hipStream_t st) {
 template <int ENC, bool GLU>
 static bool a16_set_attr() {
     return hipFuncSetAttribute((const void*)k_group_a16_dma<ENC, GLU>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)DmLdsMax<ENC>::v) == hipSuccess;
+                               (int)DmLdsMax<ENC, GLU>::v) == hipSuccess;
 }
 template <int ENC>
 static bool a16_set_attrs() {

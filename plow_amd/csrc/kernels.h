@@ -176,6 +176,8 @@ struct GroupA16 {
      * reference's decode DOWN bodies do (plow runtime/cpu/dev/golden/moe.c:76-80) */
     const void* zs_table;
     uint32_t zs_nslot;
+    /* streaming DOWN: set by the launcher when the workgroups take tiles of 256 channels (32 per wave) */
+    uint32_t down_wide;
 };
 /* the matrix-vector form of the same ops for batches that route a handful of rows in all (slots_hint says so) */
 bool group_a16_gemv_serves(const GroupA16& g);

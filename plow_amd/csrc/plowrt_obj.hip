@@ -79,7 +79,7 @@ __device__ __forceinline__ bool a16_ok(unsigned N, unsigned K, unsigned E) {
 }
 
 extern "C" __global__ __launch_bounds__(512) void plow_moe_fp8_glu_pf_gfx950(PLOWRT_GLU_ARGS) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[sizeof(DmLds<AENC_FP8BLK, 4>)];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[sizeof(DmLds<AENC_FP8BLK, true, 4>)];
     (void)x_scale; (void)out_scale; (void)x_pitch; (void)reserved;
     if (!a16_ok(inter, hidden, experts)) return;
     GroupA16 g = {};
@@ -96,7 +96,7 @@ extern "C" __global__ __launch_bounds__(512) void plow_moe_fp8_glu_pf_gfx950(PLO
 }
 
 extern "C" __global__ __launch_bounds__(512) void plow_moe_fp8_down_pf_gfx950(PLOWRT_DOWN_ARGS) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[sizeof(DmLds<AENC_FP8BLK, 4>)];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[sizeof(DmLds<AENC_FP8BLK, false, 4>)];
     (void)fu_scale; (void)reserved;
     if (!a16_ok(hidden, inter, experts)) return;
     GroupA16 g = {};

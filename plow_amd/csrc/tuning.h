@@ -43,6 +43,7 @@ struct PlowMoeTuning {
     bool form_on_device;
     bool score_row_narrow;
     bool a16_tiled_mx;
+    bool a16_down_wide;
 };
 const PlowMoeTuning& plow_moe_tuning();
 

@@ -113,6 +113,21 @@ def test_bf16_activation_arms_many_rows(moe, oracle, enc, arm, T, E, k):
     check_chain(*both(moe, oracle, cfg, seed=T))
 
 
+@pytest.mark.parametrize("enc,H,I,E,T", [("mxfp4", 2048, 512, 64, 64), ("mxfp4", 2048, 1536, 64, 64), ("mxfp4", 2048, 768, 64, 64),
+                                         ("mxfp4", 4096, 512, 128, 96), ("fp8blk", 2048, 512, 64, 16), ("fp8pc", 2048, 512, 64, 16),
+                                         ("bf16", 2048, 512, 64, 16)])
+def test_streaming_form_wide_down_tiles_and_scale_chunks(moe, oracle, enc, H, I, E, T):
+    """A few rows per expert on many experts: the weight-streaming form with the DOWN on tiles of 256 channels (two
+    16-channel operands per wave), every encoding. mxfp4 brings its E8M0 bytes four 256-k steps at a time: rows of
+    two steps (K = 512: every chunk is a tail), of six (one whole chunk and a tail), of three (K = 768, not whole
+    16-byte pieces: the per-step loads), and two tiles per workgroup with the chunks running across the tile boundary
+    (128 experts x 16 tiles)."""
+    print(f"[case] a16 streaming wide enc={enc} H={H} I={I} E={E} T={T}", flush=True)
+    shared = dict(n_shared=1, shared_mode="fold") if enc != "fp8pc" else {}
+    cfg = layer.MoeConfig("a16-wide", H=H, E=E, I=I, k=4, T=T, scoring="softmax", norm_topk=True, enc=enc, arm="a16", **shared)
+    check_chain(*both(moe, oracle, cfg, seed=H + I))
+
+
 @pytest.mark.parametrize("T,E,k", [(300, 4, 2), (1030, 3, 1), (640, 8, 4)])
 def test_per_channel_w8a8_tiled_many_rows(moe, oracle, T, E, k):
     """Ops 81 / 82 with 60..1030 rows per expert run the tiled (prefill) form: partial, full and
