@@ -178,6 +178,8 @@ struct GroupA16 {
     uint32_t zs_nslot;
     /* streaming DOWN: set by the launcher when the workgroups take tiles of 256 channels (32 per wave) */
     uint32_t down_wide;
+    /* streaming forms: set by the launcher when experts of a handful of rows run with per-wave copies of their rows */
+    uint32_t priv_rows;
 };
 /* the matrix-vector form of the same ops for batches that route a handful of rows in all (slots_hint says so) */
 bool group_a16_gemv_serves(const GroupA16& g);

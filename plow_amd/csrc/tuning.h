@@ -44,6 +44,7 @@ struct PlowMoeTuning {
     bool score_row_narrow;
     bool a16_tiled_mx;
     bool a16_down_wide;
+    bool a16_private_rows;
 };
 const PlowMoeTuning& plow_moe_tuning();
 

@@ -432,10 +432,10 @@ def test_matrix_vector_form_at_one_and_two_tokens(moe, oracle, enc, H, I, T, k):
     check_chain(*both(moe, oracle, cfg, seed=H + T))
 
 
-@pytest.mark.parametrize("enc,H,I,T,k", [("mxfp4", 768, 256, 24, 8), ("mxfp4", 3584, 512, 26, 8), ("fp8blk", 640, 384, 4, 8),
+@pytest.mark.parametrize("enc,H,I,T,k", [("mxfp4", 768, 256, 14, 8), ("mxfp4", 3584, 512, 13, 8), ("fp8blk", 640, 384, 4, 8),
                                          ("fp8pc", 1536, 640, 2, 8)])
 def test_matrix_vector_form_at_a_few_tokens(moe, oracle, enc, H, I, T, k):
-    """The largest batches the matrix-vector form is chosen for, per encoding (mxfp4 up to 240 routed rows,
+    """The largest batches the matrix-vector form is chosen for, per encoding (mxfp4 up to 128 routed rows,
     block fp8 36, per-channel fp8 18): 16 experts, so every expert holds several rows and streams its weights
     once per row."""
     print(f"[case] gemv few tokens enc={enc} H={H} I={I} T={T} k={k}", flush=True)
