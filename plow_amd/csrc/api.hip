@@ -684,14 +684,9 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         }
         g.a_idx = c->ws.row_partidx; g.gate = c->ws.row_gate;
         g.wsel0 = g.wsel1 = pc ? 1u : 2u;
-        /* the rows of slots no expert serves are zeroed: by the matrix-vector form itself at a few rows (one launch
-         * less on a path that is all latency), by a launch of its own otherwise */
-        if (group_a16_gemv_serves(g)) {
-            g.zs_table = ten(in, T, 2), g.zs_nslot = nslot;
-        } else {
-            rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), g.wtab, g.stab, g.wcols, g.wsel0, nslot, E, N, st);
-            if (rc) return rc;
-        }
+        /* the rows of slots no expert serves are zeroed by the launch itself (the matrix-vector and streaming forms) or
+         * by one of its own ahead of it (the others) */
+        g.zs_table = ten(in, T, 2), g.zs_nslot = nslot;
         return launch_group_down_a16(g, st);
     }
     case PLOW_DOP_MOE_GROUP_GLU_GEMMA_PF:
@@ -777,8 +772,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.meta = c->ws.meta; g.slots_hint = nslot; g.o_idx = c->ws.row_partidx;
         if (glu) { g.a_idx = c->ws.row_token; return launch_group_glu_a16(g, st); }
         g.a_idx = c->ws.row_partidx; g.gate = c->ws.row_gate;
-        rc = launch_zero_skipped((float*)ten(in, T, 0), ten(in, T, 2), wtab, stab, 3u, 0u, nslot, E, N, st);
-        if (rc) return rc;
+        g.zs_table = ten(in, T, 2), g.zs_nslot = nslot;
         return launch_group_down_a16(g, st);
     }
     case PLOW_DOP_GEMM_GLU:

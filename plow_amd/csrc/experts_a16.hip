@@ -899,6 +899,19 @@ __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
     if (!form_is_mine(g)) return;
     if constexpr (!GLU) {
+        /* slot-major DOWN: the f32 rows of slots that no expert serves are zeroed here, a slot per wave (the reference's
+         * decode DOWN bodies do it, plow runtime/cpu/dev/golden/moe.c:76-80): one launch less */
+        if (g.zs_table && !g.out_bf16) {
+            const PlowMoeRoute* const tab = (const PlowMoeRoute*)g.zs_table;
+            const uint32_t lane = threadIdx.x & 63u, n_waves = gridDim.x * AK_WAVES;
+            for (uint32_t sl = blockIdx.x * AK_WAVES + (threadIdx.x >> 6); sl < g.zs_nslot; sl += n_waves) {
+                const uint32_t e = tab[sl].eid;
+                const bool served = e < g.E && g.wtab[(size_t)e * g.wcols + g.wsel0] != 0ull &&
+                                    (!g.stab || g.stab[(size_t)e * g.wcols + g.wsel0] != 0ull);
+                if (served) continue;
+                for (uint32_t h = lane; h < g.N; h += WAVE) ((float*)g.out)[(size_t)sl * g.N + h] = 0.0f;
+            }
+        }
         if (g.down_wide) { /* tiles of 256 channels (the launcher's grid counts them so) */
             a16_dma_pick<ENC, GLU, true>(g, dm_raw);
             return;
@@ -975,6 +988,10 @@ static bool a16_tiled_try(const GroupA16& g, hipStream_t st, int* rc, bool behin
         if (*rc) return true;
         w.form_word = g.form_ws, w.form_want = 1u;
     }
+    if (!GLU && g.zs_table) { /* (the streaming forms zero unserved slots themselves) */
+        *rc = launch_zero_skipped((float*)g.out, g.zs_table, g.wtab, g.stab, g.wcols, g.wsel0, g.zs_nslot, g.E, g.N, st);
+        if (*rc) return true;
+    }
     *rc = launch_group_a16_tiled(w, GLU, st);
     return true;
 }
@@ -993,6 +1010,7 @@ static int launch_a16(const GroupA16& g_in, hipStream_t st) {
         if (a16_tiled_try<GLU>(g, st, &rc, true)) {
             if (rc) return rc;
             g.form_word = g.form_ws, g.form_want = 0u;
+            g.zs_table = nullptr; /* zeroed by a launch of its own ahead of the tiled form */
         }
     }
     dim3 grid(g.E * (g.N / AK_BN));
@@ -1022,6 +1040,11 @@ static int launch_a16(const GroupA16& g_in, hipStream_t st) {
         if (!n_cu) return PLOW_MOE_EDEVICE;
         const uint64_t hit = g.slots_hint && g.slots_hint < g.E ? g.slots_hint : g.E;
         if (hit * (g.N / (2u * AK_BN)) >= 2ull * n_cu) g.down_wide = 1u, grid = dim3(g.E * (g.N / (2u * AK_BN)));
+    }
+    if (!dma && !GLU && g.zs_table) { /* the register form leaves the unserved slots to a launch of their own */
+        const int zrc = launch_zero_skipped((float*)g.out, g.zs_table, g.wtab, g.stab, g.wcols, g.wsel0, g.zs_nslot, g.E, g.N, st);
+        if (zrc) return zrc;
+        g.zs_table = nullptr;
     }
     switch (g.enc) {
     case AENC_BF16:
