@@ -17,6 +17,11 @@
  *   PLOW_MOE_A16_TILED        0                keep the bf16-activation arms on the streaming kernels at every row count
  *   PLOW_MOE_A16_TILED_MX     0                keep mxfp4 weights under bf16 activations on the streaming kernels at every row count
  *   PLOW_MOE_A16_GEMV         0                keep the bf16-activation arms off the matrix-vector form at a few tokens
+ *   PLOW_MOE_A16_DOWN_WIDE    0                streaming bf16-activation DOWN on tiles of 128 channels (default: 256 while
+ *                                              they give every CU two workgroups)
+ *   PLOW_MOE_A16_PRIVATE_ROWS 0                streaming bf16-activation kernels: experts of a handful of rows share the
+ *                                              workgroup's row ring like the others (default: per-wave copies on fp8 and
+ *                                              bf16 weights)
  *   PLOW_MOE_SCORE_ROW        narrow           router score: the one-token-per-wave kernel only below 16 tokens (default: while
  *                                              its workgroups fit the chip)
  *   PLOW_MOE_FORM_ON_DEVICE   0                a grouped fp8 x fp8 op without a row count runs the streaming form
