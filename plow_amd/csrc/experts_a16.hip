@@ -271,18 +271,22 @@ __global__ __launch_bounds__(AK_THREADS, GLU ? 2 : 4) void k_group_a16_stream(Gr
  * instruction. That instruction rate, not memory, bounds it. Here a step is one whole 128-byte line per
  * weight row (256 k of mxfp4, 128 k of fp8, 64 k of bf16), and
  *   weights   per wave and stream 16 rows x 128 B = two direct loads (8 consecutive lanes per line) into a
- *             wave-private ring; mxfp4: the step's E8M0 bytes (8 per row) by one 4-byte direct load per
- *             stream; block-fp8: the tile's block scales sit in LDS for all of K;
+ *             wave-private ring; mxfp4: the E8M0 bytes of four steps (32 per row) by one 16-byte direct load
+ *             per wave (8 per row and step by a 4-byte load per stream where rows are not whole 16-byte
+ *             pieces); block-fp8: the tile's block scales sit in LDS for all of K;
  *   rows      the 16 activation rows of the pass are the same for all eight waves: 16 rows x 2 bytes per k
  *             of the step, in a ring shared by the workgroup and loaded 1 KB per wave (the first 8, 4 or 2
- *             waves);
+ *             waves); experts of a handful of rows: a copy per wave instead (PRIV below);
  *   sync      rings of three steps, loads two steps ahead; per step each wave waits for its own loads
- *             (s_waitcnt vmcnt) and all meet at one barrier, after which the step before is free;
+ *             (s_waitcnt vmcnt) and all meet at one barrier, after which the step before is free (none
+ *             with per-wave rows);
+ *   DOWN      tiles of 128 channels, 16 per wave, or of 256 with two weight operands per wave (WIDE below);
  *   swizzle   direct loads write LDS contiguously, so bank conflicts are avoided on the global side:
  *             LDS piece p of weight row r holds global piece p ^ lds_swz8(r), and likewise for
  *             activation rows of 128 B; piece p of a longer activation row r holds global piece
  *             (p & ~15) | ((p ^ lds_swz16(r)) & 15).
- * Same arithmetic and the same order of additions as the first form. */
+ * Same arithmetic as the first form, and the same order of additions except with per-wave rows, where a wave
+ * starts its walk over K at a column of its own. */
 /* ring depth: four steps (loads three ahead) where the rings leave room in the CU's 160 KB — one row group per
  * pass and 4 KB of weight rows per wave and step — three steps otherwise (mxfp4's step carries 8 KB of
  * activation rows and the E8M0 bytes; several row groups per pass multiply the activation ring) */
@@ -889,11 +893,13 @@ __device__ __forceinline__ void a16_dma_pick(const GroupA16& g, uint8_t* dm_raw)
     }
 }
 
-/* One kernel, three instances of the body: a workgroup takes the one that covers its expert's rows in the fewest
- * passes over the weights (16, 32 or 64 rows per pass; mxfp4 16 or 32, its rings fill the LDS at 32). Routing is
- * skewed: at 4 rows per expert on average the hot experts hold 30 to 60, and a second pass re-reads the weights
- * from memory (Qwen3 shape, 64 tokens: GLU 325 us with 16-row passes for all, 289 us with 32-row passes for
- * all, which in turn costs the few-row experts 3 % in row loads and multiplies they do not need). */
+/* One kernel, several instances of the body, picked per workgroup from its expert's row count (a16_dma_pick): the
+ * private-row form for a handful of rows (fp8 and bf16 weights, two-stream shapes), else the one that covers the
+ * rows in the fewest passes over the weights (16, 32 or 64 rows per pass; mxfp4 16 or 32, its rings fill the LDS at
+ * 32). Routing is skewed: at 4 rows per expert on average the hot experts hold 30 to 60, and a second pass re-reads
+ * the weights from memory (Qwen3 shape, 64 tokens: GLU 325 us with 16-row passes for all, 289 us with 32-row passes
+ * for all, which in turn costs the few-row experts 3 % in row loads and multiplies they do not need). The DOWN holds
+ * the bodies for tiles of 128 and of 256 channels; the launcher's grid says which (g.down_wide). */
 template <int ENC, bool GLU>
 __global__ __launch_bounds__(AK_THREADS) void k_group_a16_dma(GroupA16 g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t dm_raw[];
