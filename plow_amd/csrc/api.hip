@@ -792,6 +792,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         g.wdirect[0] = ten(in, T, 2); g.wdirect[1] = glu ? ten(in, T, 5) : ten(in, T, 2);
         g.N = N; g.K = K; g.E = 1; g.enc = 0; g.act = glu ? i[5] : 0u;
         g.wcols = 1; g.out_bf16 = 1; g.dense_rows = M;
+        if (c->ws_base && c->stage) g.split_ws = c->stage, g.split_ws_bytes = c->stage_bytes; /* few rows: K split over workgroups */
         return glu ? launch_group_glu_a16(g, st) : launch_group_down_a16(g, st);
     }
     default:

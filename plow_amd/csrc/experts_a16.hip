@@ -454,13 +454,20 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
     const uint64_t* stt = g.stab ? g.stab + (size_t)e * g.wcols : nullptr;
     if (wt && wt[g.wsel0] == 0ull) return; /* expert not resident: skipped */
     if (stt && ENC != AENC_BF16 && stt[g.wsel0] == 0ull) return;
-    const uint32_t r0 = g.meta ? (uint32_t)g.meta[e] : 0u;
+    /* K split (dense bf16 ops): slice e % ksplit of tensor e / ksplit; rows 0 .. of the activations, rows
+     * e * dense_rows .. of the output */
+    const uint32_t ksp = ENC == AENC_BF16 ? g.ksplit : 0u;
+    const uint32_t r0 = g.meta ? (uint32_t)g.meta[e] : (ksp ? e * g.dense_rows : 0u);
+    const uint32_t xr0 = ksp ? 0u : r0; /* the expert's first activation row */
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t c = lane & 15u, q = lane >> 4; /* operand layout: row / channel c, k-chunk q */
     const uint32_t K = g.K, KS = K / KSTEP, N = g.N, GS = TPW * KS; /* steps of a pass over all its tiles */
+    const uint32_t KP = ksp ? g.kpitch : K;                        /* elements per row in memory */
+    const size_t kofs = ksp ? (size_t)(e % ksp) * K * 2u : 0u;     /* the slice's first byte in a row */
+    const uint8_t* const abase = (const uint8_t*)g.a + kofs;
     const uint32_t chw = ct * BN + wv * (WIDE ? 32u : 16u); /* this wave's first channel */
-    const uint32_t wrow = ENC == AENC_BF16 ? K * 2u : (ENC == AENC_MXFP4 ? K / 2u : K); /* bytes per weight row */
+    const uint32_t wrow = ENC == AENC_BF16 ? KP * 2u : (ENC == AENC_MXFP4 ? K / 2u : K); /* bytes per weight row */
     const uint32_t wmul = g.wmul ? g.wmul : 1u;
 
     /* weight loads: load j covers rows 8j .. 8j + 7 of a stream (lane = row lr of the group, piece p) */
@@ -472,7 +479,8 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
     for (int sidx = 0; sidx < NS; sidx++) {
         /* the wide DOWN's second stream is the same matrix, 16 channels on */
         const uint32_t sel = (sidx && !WIDE) ? g.wsel1 : g.wsel0;
-        const uint8_t* wbase = wt ? (const uint8_t*)(uintptr_t)wt[sel] : (const uint8_t*)g.wdirect[WIDE ? 0 : sidx];
+        const uint8_t* wbase = wt ? (const uint8_t*)(uintptr_t)wt[sel]
+                                  : (const uint8_t*)g.wdirect[ksp ? e / ksp : (WIDE ? 0 : sidx)] + kofs;
         const uint8_t* sbase = stt ? (const uint8_t*)(uintptr_t)stt[sel] : nullptr;
         const uint32_t wr0 = (sidx && !WIDE) ? g.wrow1 : g.wrow0;
         const uint32_t chs = chw + ((sidx && WIDE) ? 16u : 0u); /* the stream's first channel */
@@ -527,7 +535,7 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
         const uint8_t* xdummy;
         bool xlane[NXI]; /* private rings: this lane's row exists */
         {
-            const uint32_t first = g.a_idx ? g.a_idx[r0 + rb] : r0 + rb;
+            const uint32_t first = g.a_idx ? g.a_idx[xr0 + rb] : xr0 + rb;
 #pragma unroll
             for (uint32_t i = 0; i < NXI; i++) {
                 const uint32_t xrow0 = PRIV ? XRPL * i : XRPL * (wv + AK_WAVES * i); /* the load's first row */
@@ -536,13 +544,13 @@ __device__ __forceinline__ void a16_dma_body(const GroupA16& g, uint8_t* dm_raw,
                 xlane[i] = !PRIV || xrow < live;
                 if ((PRIV || wv + AK_WAVES * i < XL) && xrow0 < live) {
                     const uint32_t off = rb + xrow;
-                    uint32_t ai = off < cnt ? (g.a_idx ? g.a_idx[r0 + off] : r0 + off) : PLOW_EXPERT_UNUSED;
+                    uint32_t ai = off < cnt ? (g.a_idx ? g.a_idx[xr0 + off] : xr0 + off) : PLOW_EXPERT_UNUSED;
                     if (ai == PLOW_EXPERT_UNUSED) ai = first == PLOW_EXPERT_UNUSED ? 0u : first;
                     const uint32_t gp = NP >= 16u ? ((pc & ~15u) | ((pc ^ lds_swz16(xrow)) & 15u)) : (pc ^ lds_swz8(xrow));
-                    xsrc[i] = (const uint8_t*)g.a + (size_t)ai * K * 2u + (gp << 4);
+                    xsrc[i] = abase + (size_t)ai * KP * 2u + (gp << 4);
                 }
             }
-            xdummy = (const uint8_t*)g.a + (size_t)(first == PLOW_EXPERT_UNUSED ? 0u : first) * K * 2u;
+            xdummy = abase + (size_t)(first == PLOW_EXPERT_UNUSED ? 0u : first) * KP * 2u;
         }
         /* the B-operand rows of this lane: row c of each 16-row group */
         bool valid[RG];
@@ -1002,11 +1010,141 @@ static bool a16_tiled_try(const GroupA16& g, hipStream_t st, int* rc, bool behin
     return true;
 }
 
+/* K split of a dense op, second launch: output row m = the sum over the slices, in slice order, of the partial rows
+ * the first launch wrote (part: [mats * S][M][N] f32, matrix-major), through the activation for the GLU (gate =
+ * matrix 0, up = matrix 1); a thread takes four channels. */
+__global__ __launch_bounds__(64) void k_ksplit_finish(bf16_t* __restrict__ out, const float* __restrict__ part, uint32_t M,
+                                                       uint32_t N, uint32_t S, uint32_t glu, uint32_t act, float f0, float f1) {
+    const size_t n4 = (size_t)M * (N / 4u), plane = (size_t)M * N;
+    /* eight slices' loads go out together; the adds keep the slice order */
+    auto sum = [&](const float* p) -> float4 {
+        float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (uint32_t s0 = 0; s0 < S; s0 += 8u) {
+            float4 t[8];
+#pragma unroll
+            for (uint32_t j = 0; j < 8u; j++) t[j] = s0 + j < S ? *(const float4*)(p + (size_t)(s0 + j) * plane) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+            for (uint32_t j = 0; j < 8u; j++) {
+                if (s0 + j == 0u) a = t[0]; /* (0 + x would turn a -0 sum into +0) */
+                else if (s0 + j < S) a.x += t[j].x, a.y += t[j].y, a.z += t[j].z, a.w += t[j].w;
+            }
+        }
+        return a;
+    };
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
+        const float* p = part + i * 4u;
+        float4 a = sum(p);
+        if (glu) {
+            const float4 b = sum(p + S * plane);
+            a.x = moe_glu(a.x, b.x, act, f0, f1), a.y = moe_glu(a.y, b.y, act, f0, f1);
+            a.z = moe_glu(a.z, b.z, act, f0, f1), a.w = moe_glu(a.w, b.w, act, f0, f1);
+        }
+        uint2 o;
+        o.x = (uint32_t)f2bf(a.x) | ((uint32_t)f2bf(a.y) << 16);
+        o.y = (uint32_t)f2bf(a.z) | ((uint32_t)f2bf(a.w) << 16);
+        *(uint2*)(out + i * 4u) = o;
+    }
+}
+
+template <bool GLU>
+static int launch_a16(const GroupA16& g_in, hipStream_t st);
+
+/* A dense op (one expert, bf16 weights) of a few rows has N / 128 channel tiles per matrix, a few dozen workgroups
+ * on a chip of 256 CUs, each walking the whole K: the op then takes as long as one CU needs for its tile's rows
+ * (shared expert of the small bf16 layer, 16 tokens: GLU 22 workgroups). Here K is split S ways: the streaming
+ * DOWN kernel runs mats * S "experts" (slice s of matrix m) that write f32 partial rows into the caller's scratch,
+ * and a second launch adds the slices up in slice order and applies the epilogue. Returns false when the op is not
+ * of that kind or the scratch does not hold the partial rows. */
+template <bool GLU>
+static bool a16_dense_split_try(const GroupA16& g, hipStream_t st, int* rc) {
+    const PlowMoeTuning& tune = plow_moe_tuning();
+    if (!tune.a16_dense_split || tune.a16_regs || g.meta || g.wtab || !g.dense_rows || g.dense_rows >= 128u || g.E != 1u ||
+        g.enc != AENC_BF16 || g.bias || !g.split_ws || !g.out_bf16 || g.ksplit || g.a_idx || g.o_idx || g.gate || g.wmul > 1u ||
+        g.wrow0 || (GLU && g.wrow1))
+        return false;
+    const uint32_t n_cu = plow_moe_n_cu();
+    if (!n_cu) return false;
+    const uint32_t mats = GLU ? 2u : 1u, tiles = g.N / AK_BN, steps = g.K / 64u;
+    if (g.K % 64u || g.K > 16384u || mats * tiles >= n_cu) return false;
+    /* the fewest slices that give every CU a workgroup, each of four steps (256 k) at least; failing that the most */
+    uint32_t S = 0u;
+    for (uint32_t d = 2u; d * 4u <= steps; d++) {
+        if (steps % d || (g.K / d) % 128u) continue; /* (the streaming form takes whole 128-k pairs of steps) */
+        if ((uint64_t)mats * d * g.dense_rows * g.N * 4u > g.split_ws_bytes) break;
+        S = d;
+        if (mats * d * tiles >= n_cu) break;
+    }
+    if (S < 2u) return false;
+    GroupA16 p = g;
+    p.out = g.split_ws, p.out_bf16 = 0u, p.act = 0u;
+    p.E = mats * S, p.ksplit = S, p.kpitch = g.K, p.K = g.K / S;
+    p.split_ws = nullptr;
+    *rc = launch_a16<false>(p, st);
+    if (*rc) return true;
+    const size_t n4 = (size_t)g.dense_rows * (g.N / 4u);
+    const uint32_t blocks = (uint32_t)((n4 + 63u) / 64u); /* a wave per workgroup: the op is a handful of rows */
+    k_ksplit_finish<<<blocks, 64, 0, st>>>((bf16_t*)g.out, (const float*)g.split_ws, g.dense_rows, g.N, S, GLU ? 1u : 0u, g.act, g.f0, g.f1);
+    return true;
+}
+
+/* A dense op of many rows as a one-expert batch of the tiled kernel: this launch writes what that kernel reads from
+ * memory into the caller's scratch: the expert's pointer row {w0, w1, w0}, its meta {first row 0, M rows} and the
+ * identity row maps with gate 1. */
+#define DENSE_TAB_BYTES 256u
+__global__ __launch_bounds__(256) void k_dense_tables(uint8_t* base, const void* w0, const void* w1, uint32_t M, uint32_t map_bytes) {
+    const uint32_t r = blockIdx.x * 256u + threadIdx.x;
+    if (r == 0u) {
+        uint64_t* const wtab = (uint64_t*)base;
+        wtab[0] = (uint64_t)(uintptr_t)w0, wtab[1] = (uint64_t)(uintptr_t)w1, wtab[2] = (uint64_t)(uintptr_t)w0;
+        int32_t* const meta = (int32_t*)(base + 64u);
+        meta[0] = 0, meta[1] = (int32_t)M;
+    }
+    if (r < M) {
+        ((uint32_t*)(base + DENSE_TAB_BYTES))[r] = r;
+        ((uint32_t*)(base + DENSE_TAB_BYTES + map_bytes))[r] = r;
+        ((float*)(base + DENSE_TAB_BYTES + 2u * (size_t)map_bytes))[r] = 1.0f;
+    }
+}
+
+/* Dense ops beyond the rows the K split takes: the tiled MFMA kernel over bf16 weights, which reads an expert's
+ * weights once per 128 rows where the streaming form re-streams them per 64 and has N / 128 workgroups in all. */
+template <bool GLU>
+static bool a16_dense_tiled_try(const GroupA16& g, hipStream_t st, int* rc) {
+    const PlowMoeTuning& tune = plow_moe_tuning();
+    if (!tune.a16_tiled || !tune.a16_dense_split || g.meta || g.wtab || g.dense_rows < 128u || g.E != 1u || g.enc != AENC_BF16 ||
+        g.bias || !g.split_ws || !g.out_bf16 || g.ksplit || g.a_idx || g.o_idx || g.gate || g.wmul > 1u || g.wrow0 || g.wrow1)
+        return false;
+    const uint32_t M = g.dense_rows;
+    const size_t map_bytes = ((size_t)M * 4u + 255u) & ~(size_t)255u;
+    if (map_bytes > 0x7FFFFFFFull || DENSE_TAB_BYTES + 3u * map_bytes > g.split_ws_bytes) return false;
+    uint8_t* const base = (uint8_t*)g.split_ws;
+    GroupA16 t = g;
+    t.split_ws = nullptr, t.dense_rows = 0u, t.slots_hint = M;
+    t.wtab = (const uint64_t*)base, t.meta = (const int32_t*)(base + 64u), t.wcols = 3u;
+    if (GLU) t.wsel0 = 0u, t.wsel1 = 1u, t.a_idx = (const uint32_t*)(base + DENSE_TAB_BYTES);
+    else t.wsel0 = t.wsel1 = 2u, t.o_idx = (const uint32_t*)(base + DENSE_TAB_BYTES + map_bytes),
+         t.gate = (const float*)(base + DENSE_TAB_BYTES + 2u * map_bytes);
+    /* would the tiled form take it? (asked before anything is launched) */
+    {
+        GroupW8A8 w = {};
+        w.N = g.N, w.K = g.K, w.E = 1u, w.w_bf16 = 1u, w.meta = t.meta;
+        if (!group_w8a8_tiled_serves(w)) return false;
+    }
+    k_dense_tables<<<(M + 255u) / 256u, 256, 0, st>>>(base, g.wdirect[0], g.wdirect[1], M, (uint32_t)map_bytes);
+    if (!a16_tiled_try<GLU>(t, st, rc, false)) *rc = PLOW_MOE_EINVAL; /* (the checks above are the tiled form's own) */
+    return true;
+}
+
 template <bool GLU>
 static int launch_a16(const GroupA16& g_in, hipStream_t st) {
     GroupA16 g = g_in;
     if (g.N == 0 || g.K == 0 || g.E == 0 || g.N % AK_BN || g.K % 128u) return PLOW_MOE_EINVAL;
     if ((uint64_t)g.E * (g.N / AK_BN) > 0x7FFFFFFFull) return PLOW_MOE_EINVAL;
+    {
+        int rc = 0;
+        if (a16_dense_split_try<GLU>(g, st, &rc)) return rc;
+        if (a16_dense_tiled_try<GLU>(g, st, &rc)) return rc;
+    }
     if (group_a16_gemv_serves(g)) return launch_group_a16_gemv(g, GLU, st); /* a handful of rows in all */
     {
         int rc = 0;
@@ -1040,6 +1178,7 @@ static int launch_a16(const GroupA16& g_in, hipStream_t st) {
      * small bf16 layer, 16 tokens: 110 -> 103 us), behind on mxfp4, whose step carries twice the row bytes per weight
      * byte (Kimi-K2 shape, 64 tokens: GLU 654 -> 681 us) */
     g.priv_rows = (plow_moe_tuning().a16_private_rows && g.enc != AENC_MXFP4) ? 1u : 0u;
+    if (g.ksplit && !dma) return PLOW_MOE_EINVAL; /* (a16_dense_split_try asks for nothing the second form refuses) */
     if (!GLU && dma && g.N % (2u * AK_BN) == 0u && g.meta && plow_moe_tuning().a16_down_wide) {
         /* tiles of 256 channels while they still give every CU two workgroups and more */
         const uint32_t n_cu = plow_moe_n_cu();

@@ -180,6 +180,14 @@ struct GroupA16 {
     uint32_t down_wide;
     /* streaming forms: set by the launcher when experts of a handful of rows run with per-wave copies of their rows */
     uint32_t priv_rows;
+    /* Dense ops of a few rows (one expert, no meta, bf16 weights): scratch the launcher may use to split K over
+     * several workgroups per channel tile (NULL: never split). split_ws holds f32 partial rows. */
+    void* split_ws;
+    size_t split_ws_bytes;
+    /* set by the launcher on a K-split launch: "expert" v of the launch is K slice v % ksplit (K columns starting at
+     * (v % ksplit) * K of rows whose pitch is kpitch) of weight tensor wdirect[v / ksplit]; it reads activation rows
+     * 0 .. dense_rows - 1 and writes output rows v * dense_rows .. */
+    uint32_t ksplit, kpitch;
 };
 /* the matrix-vector form of the same ops for batches that route a handful of rows in all (slots_hint says so) */
 bool group_a16_gemv_serves(const GroupA16& g);

@@ -22,6 +22,9 @@
  *   PLOW_MOE_A16_PRIVATE_ROWS 0                streaming bf16-activation kernels: experts of a handful of rows share the
  *                                              workgroup's row ring like the others (default: per-wave copies on fp8 and
  *                                              bf16 weights)
+ *   PLOW_MOE_A16_DENSE_SPLIT  0                dense bf16 ops of a few rows walk the whole K in one workgroup per channel
+ *                                              tile (default: K split over several workgroups while the tiles are
+ *                                              fewer than the CUs)
  *   PLOW_MOE_SCORE_ROW        narrow           router score: the one-token-per-wave kernel only below 16 tokens (default: while
  *                                              its workgroups fit the chip)
  *   PLOW_MOE_FORM_ON_DEVICE   0                a grouped fp8 x fp8 op without a row count runs the streaming form
@@ -50,6 +53,7 @@ struct PlowMoeTuning {
     bool a16_tiled_mx;
     bool a16_down_wide;
     bool a16_private_rows;
+    bool a16_dense_split;
 };
 const PlowMoeTuning& plow_moe_tuning();
 

@@ -295,6 +295,33 @@ def test_dense_ops_against_oracle(moe, oracle):
     close(ol.bf2f(yg[1:]), ol.bf2f(y_h[1:]), "dense y")
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 2816, 2048), (1, 1408, 2816), (64, 512, 5632), (7, 128, 1024), (100, 1408, 2048),
+                                   (128, 512, 1024), (600, 1408, 2048), (1500, 256, 512)])
+def test_dense_ops_split_k_or_run_tiled(moe, oracle, M, N, K):
+    """Below 128 rows and with fewer channel tiles than CUs the dense ops run as K slices plus a second launch that
+    adds the slices up (GLU: before the activation): shapes of the small bf16 layer's shared expert, a K whose step
+    count has an odd factor, a single tile, two row passes. From 128 rows they run on the tiled kernel as a
+    one-expert batch whose tables a set-up launch writes."""
+    r = cases.rng_of(M + N + K)
+    x = cases.randn_bf16(r, (M + 3, K), 1.0)
+    wg, wu, wd = cases.randn_bf16(r, (N, K), 0.03), cases.randn_bf16(r, (N, K), 0.03), cases.randn_bf16(r, (K, N), 0.03)
+    glu = abi.inst(abi.OP_GEMM_GLU, t=[0, 1, 2, None, None, 5], i=[M + 3, N, K, 0, 0, 1])
+    gemm = abi.inst(abi.OP_GEMM, t=[0, 1, 2], i=[M, K, N, 0, 3, 1])   # a_row0 = 3, c_row0 = 1
+    fu_h, y_h = np.zeros((M + 3, N), np.uint16), np.zeros((M + 1, K), np.uint16)
+    ol.run(oracle.plow_oracle_exec, glu, ol.table_of([fu_h, x, wg, None, None, wu]), 4)
+    ol.run(oracle.plow_oracle_exec, gemm, ol.table_of([y_h, fu_h, wd]), 4)
+    fu_d = torch.zeros((M + 3, N), dtype=torch.int16, device="cuda")
+    y_d = torch.zeros((M + 1, K), dtype=torch.int16, device="cuda")
+    for _ in range(2):  # the scratch is reused: a second run over it gives the same rows
+        moe.exec(glu, dev_table([fu_d, to_dev(x), to_dev(wg), None, None, to_dev(wu)]))
+        moe.exec(gemm, dev_table([y_d, to_dev(fu_h), to_dev(wd)]))
+    torch.cuda.synchronize()
+    close(ol.bf2f(fu_d.cpu().numpy().view(np.uint16)), ol.bf2f(fu_h), "dense fu")
+    yg = y_d.cpu().numpy().view(np.uint16)
+    assert np.all(yg[0] == 0)
+    close(ol.bf2f(yg[1:]), ol.bf2f(y_h[1:]), "dense y")
+
+
 # the last three: activations that transform the up branch too (2 situ, 3 swiglu_oai), immediates in fj[0..1]
 @pytest.mark.parametrize("layout,with_bias,act,fimm", [(1, False, 1, ()), (0, True, 0, ()), (0, False, 1, ()), (1, True, 1, ()),
                                                         (0, True, 3, (1.702, 7.0)), (1, True, 2, (2.0, 1.5)), (1, False, 2, (3.0, 0.0))])
