@@ -176,7 +176,13 @@ enum {
     PLOW_ROUTE_SIGMOID   = 1u, /* else softmax */
     PLOW_ROUTE_NORM_TOPK = 2u,
     PLOW_ROUTE_BIAS      = 4u, /* t3 is bound */
-    PLOW_ROUTE_F32_LOGIT = 8u
+    PLOW_ROUTE_F32_LOGIT = 8u,
+    /* selection by a [vocab][k] lookup table instead of by score. Refused: the reference's dispatch of ops 56 / 83
+     * binds no table either (runtime/amd/interp.hip:6485-6488 passes null for it) */
+    PLOW_ROUTE_HASH      = 16u,
+    /* score = sqrt(softplus(logit)) = sqrtf(log1pf(expf(-|l|)) + max(l, 0)), a third transform beside sigmoid
+     * and softmax (runtime/amd/op_moe.h:485-494); takes precedence over bit 0 as there */
+    PLOW_ROUTE_SQRT_SOFTPLUS = 32u
 };
 
 /* ---- error codes -------------------------------------------------------------------------------- */

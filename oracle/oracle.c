@@ -125,7 +125,12 @@ static void route_one(PlowMoeRoute* tab, const void* logit, const float* bias, u
     for (uint32_t j = PLOW_ROUTE_MAX_TOPK; j < k; j++) { tab[j].eid = PLOW_EXPERT_UNUSED; tab[j].gate = 0.0f; }
     if (k > PLOW_ROUTE_MAX_TOPK) k = PLOW_ROUTE_MAX_TOPK;
 #define LOGIT(e) ((f32l ? ((const float*)logit)[e] : orc_bf2f(((const orc_bf16*)logit)[e])) * ls)
-    if (sigmoid) {
+    if (flags & PLOW_ROUTE_SQRT_SOFTPLUS) { /* runtime/amd/op_moe.h:485-494: log1p(exp(-|l|)) + max(l, 0) cannot overflow */
+        for (uint32_t e = 0; e < n_exp; e++) {
+            const float l = LOGIT(e);
+            score[e] = sqrtf(log1pf(expf(-fabsf(l))) + fmaxf(l, 0.0f));
+        }
+    } else if (sigmoid) {
         for (uint32_t e = 0; e < n_exp; e++) score[e] = 1.0f / (1.0f + expf(-LOGIT(e)));
     } else {
         float m = -1e30f, s = 0.0f;

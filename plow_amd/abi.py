@@ -46,7 +46,7 @@ ARM_A16, ARM_W8A8, ARM_W8A8_P16, ARM_W8A8_XQ, ARM_W4A16 = 0, 2, 3, 6, 8
 ARM_A4W4, ARM_A4W4_P16 = 0, 1     # enc 2: fp4 on both operands (the reference's default for mxfp4); DOWN with a bf16 part
 ROUTER_RAW_MARK = 0x52545241       # op 180 i7: the score carries its top-k (one launch)
 ACT_GELU_TANH, ACT_SILU = 0, 1
-ROUTE_SIGMOID, ROUTE_NORM_TOPK, ROUTE_BIAS, ROUTE_F32_LOGIT = 1, 2, 4, 8
+ROUTE_SIGMOID, ROUTE_NORM_TOPK, ROUTE_BIAS, ROUTE_F32_LOGIT, ROUTE_HASH, ROUTE_SQRT_SOFTPLUS = 1, 2, 4, 8, 16, 32
 
 E_OK, E_INVAL, E_UNSUPPORTED, E_DEVICE, E_NOMEM, ROLLBACK = 0, -22, -95, -5, -12, 1
 

@@ -263,6 +263,7 @@ static bool sort_reusable(const Hint& h, const void* table, uint32_t nslot, uint
     return h.sorted_table != nullptr && h.sorted_table == table && h.sorted_nslot == nslot && h.sorted_E == E && (!glu || h.sorted_kx == kx);
 }
 
+#define ROUTE_FLAGS_SERVED (PLOW_ROUTE_SIGMOID | PLOW_ROUTE_NORM_TOPK | PLOW_ROUTE_BIAS | PLOW_ROUTE_F32_LOGIT | PLOW_ROUTE_SQRT_SOFTPLUS)
 static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStream_t st, bool launch, Hint& h) {
     const uint32_t* i = in->i;
     if (launch && (in->op == PLOW_DOP_MOE_ROUTER_TOPK || in->op == PLOW_DOP_MOE_ROUTER_TOPK_PF || in->op == PLOW_DOP_GEMM_F32))
@@ -278,6 +279,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             NEED(c, ten(in, T, 3) && ten(in, T, 5), "op 180 (router): t3 table and t5 counters must be bound");
             NEED(c, E <= 1024u && k >= 1u, "op 180 (router): n_exp %u above 1024 or k = 0", E);
             NEED(c, (flags & PLOW_ROUTE_F32_LOGIT) != 0u, "op 180 (router): the top-k reads the f32 logits, flag bit 3 must be set");
+            NEED(c, (flags & ~ROUTE_FLAGS_SERVED) == 0u, "op 180 (router): flags 0x%x ask for hash selection (bit 4, no table operand on this op) or an unknown transform", flags);
             NEED(c, ((flags & PLOW_ROUTE_BIAS) != 0u) == (ten(in, T, 4) != nullptr), "op 180 (router): bias flag (bit 2) and the t4 binding disagree");
             if (ng > 1u && tg > 0u && tg < ng)
                 NEED(c, ng <= PLOW_ROUTE_MAX_GROUPS && E % ng == 0u && E / ng >= 2u && (uint64_t)tg * (E / ng) >= (k < 16u ? k : 16u),
@@ -304,6 +306,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, ten(in, T, 0) && ten(in, T, 1), "router top-k: t0 table and t1 logits must be bound");
         NEED(c, E >= 1u && E <= 1024u, "router top-k: n_exp %u outside 1..1024", E);
         NEED(c, k >= 1u, "router top-k: k = 0");
+        NEED(c, (flags & ~ROUTE_FLAGS_SERVED) == 0u, "router top-k: flags 0x%x ask for hash selection (bit 4, no table operand on this op) or an unknown transform", flags);
         /* the bias operand is read by the GPU reference only under flag bit 2 and by the CPU reference
          * whenever it is bound: a packet where the two disagree is ambiguous and refused */
         NEED(c, ((flags & PLOW_ROUTE_BIAS) != 0u) == (ten(in, T, 3) != nullptr),

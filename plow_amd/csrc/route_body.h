@@ -7,6 +7,7 @@
 
 #include "common.h"
 #include "pm_expf.h"
+#include "pm_log1pf.h"
 
 /* Few outputs (decode): TOK tokens x 64 experts per workgroup, one consumer wave per token. Every output
  * is a chain of K dependent multiply-adds (9.3 cycles, 3.9 ns, a step on this chip whatever the operands:
@@ -206,7 +207,16 @@ __device__ __forceinline__ void router_topk_token(const RouterArgs& a, uint32_t 
             sc[j] = (f32l ? ((const float*)a.logit)[(size_t)tok * E + e]
                           : bf2f(((const bf16_t*)a.logit)[(size_t)tok * E + e])) * ls;
     }
-    if (sigmoid) {
+    if (a.flags & PLOW_ROUTE_SQRT_SOFTPLUS) { /* sqrt(softplus(l)), softplus as log1p(exp(-|l|)) + max(l, 0) */
+#pragma unroll
+        for (uint32_t j = 0; j < RT_EPL; j++) {
+            const float ex = pm_expf_lanes(-fabsf(sc[j]), tab); /* in [0, 1], or NaN from a NaN logit */
+            const float sp = (ex == ex ? pm_log1pf_unit(ex) : ex) + fmaxf(sc[j], 0.0f);
+            /* the correctly rounded root: the binary64 root of a binary32 number, rounded once more, is the
+             * binary32 root (a root never lies within 2^-49 of a rounding boundary of binary32) */
+            sc[j] = (float)__builtin_sqrt((double)sp);
+        }
+    } else if (sigmoid) {
 #pragma unroll
         for (uint32_t j = 0; j < RT_EPL; j++) sc[j] = 1.0f / (1.0f + pm_expf_lanes(-sc[j], tab));
     } else {

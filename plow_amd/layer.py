@@ -25,7 +25,7 @@ class MoeConfig:
     I: int
     k: int
     T: int
-    scoring: str = "sigmoid"        # or "softmax"
+    scoring: str = "sigmoid"        # or "softmax", "sqrtsoftplus"
     norm_topk: bool = True
     bias: bool = False
     n_group: int = 1
@@ -75,6 +75,8 @@ class MoeConfig:
         f = abi.ROUTE_F32_LOGIT
         if self.scoring == "sigmoid":
             f |= abi.ROUTE_SIGMOID
+        if self.scoring == "sqrtsoftplus":
+            f |= abi.ROUTE_SQRT_SOFTPLUS
         if self.norm_topk:
             f |= abi.ROUTE_NORM_TOPK
         if self.bias:

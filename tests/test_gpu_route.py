@@ -73,6 +73,8 @@ def test_route_and_align_match_plow_cpu_golden(moe, case):
     (64, 6, 16, 8, 0, 0, 0),
     (1000, 16, 5, 1 | 8, 20, 7, 0),
     (96, 20, 3, 8, 0, 0, 1),                     # k above 16: sentinel slots
+    (256, 6, 700, 32 | 2 | 4 | 8, 0, 0, 1),      # sqrt-softplus scores (DeepSeek-V4 routing), bias + renorm
+    (384, 8, 33, 32 | 1 | 8, 8, 3, 0),           # the same with bit 0 also set (sqrt-softplus wins) and groups
 ])
 def test_route_and_align_match_oracle(moe, oracle, E, k, T, flags, ng, tg, tail):
     print(f"[case] route-oracle E={E} k={k} T={T} flags={flags} groups={ng}/{tg}", flush=True)
@@ -121,7 +123,8 @@ def test_align_of_long_tables(moe, oracle, T, E, k):
     assert np.all(dev[1][rows:] == 7)
 
 
-@pytest.mark.parametrize("flags", [1 | 8, 1 | 2 | 8, 2 | 8, 8], ids=["sigmoid", "sigmoid-renorm", "softmax-renorm", "softmax"])
+@pytest.mark.parametrize("flags", [1 | 8, 1 | 2 | 8, 2 | 8, 8, 32 | 8, 32 | 2 | 8],
+                         ids=["sigmoid", "sigmoid-renorm", "softmax-renorm", "softmax", "sqrtsoftplus", "sqrtsoftplus-renorm"])
 def test_route_on_logits_at_the_ends_of_the_exponential(moe, oracle, flags):
     """Logits that drive the score transform's exponential through its special inputs: overflow and underflow
     thresholds (88.72, -103.97) and their neighbours, the |x| >= 88 test, infinities (sigmoid only: a softmax
@@ -134,7 +137,7 @@ def test_route_on_logits_at_the_ends_of_the_exponential(moe, oracle, flags):
     for v in list(edge[:13]):
         edge = np.append(edge, [np.nextafter(v, np.float32(0)), np.nextafter(v, np.float32(1e9))])
     edge = np.concatenate([edge, -edge]).astype(np.float32)
-    sigmoid = bool(flags & 1)
+    sigmoid = bool(flags & (1 | 32))                     # the per-expert transforms (sqrt-softplus: the same ends)
     if sigmoid:
         edge = np.concatenate([edge, np.array([np.inf, -np.inf], np.float32)])
     logit = (r.standard_normal((T, E)) * 2.0).astype(np.float32)
@@ -257,6 +260,11 @@ def test_refusals(moe):
     assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1, None, 3], i=[0, 64, 4, 1, 2]), t) == abi.E_INVAL
     assert "bias" in moe.last_error()
     assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 1, 2, 0, 8, 1]), t) == 0
+    # hash selection (flag bit 4) has no table operand on this op; bits above 5 name nothing
+    assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 1 | 16, 2]), t) == abi.E_INVAL
+    assert "hash" in moe.last_error()
+    assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 64, 2]), t) == abi.E_INVAL
+    assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 32 | 8, 2]), t) == 0
     assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 60, 8, 1, 2, 0, 8, 4]), t) == abi.E_INVAL
     assert moe.check(abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[0, 1], i=[0, 64, 8, 1, 2, 0, 32, 2]), t) == abi.E_INVAL
     assert moe.check(abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5], i=[256, 256, 4, 2, 0, 1, 0, 5]), t) == abi.E_UNSUPPORTED

@@ -123,6 +123,37 @@ def test_flat_selection_is_descending_argsort(oracle):
             assert np.allclose(tab["gate"][t], score[t, order], rtol=1e-6)
 
 
+def test_sqrt_softplus_scores_and_selection(oracle):
+    """Flag bit 5: score = sqrt(softplus(logit)), checked against float64 (the gate of an un-normalized, unscaled
+    table is the score itself), selection = descending argsort of score + bias, bit 0 ignored beside it, and the
+    closed-form ends: softplus(l) -> l for large l, -> exp(l) for very negative l, softplus(0) = ln 2."""
+    r = cases.rng_of(41)
+    E, k, T = 96, 8, 30
+    lg = (r.standard_normal((T, E)) * 4).astype(np.float32)
+    bias = (r.standard_normal(E) * 0.2).astype(np.float32)
+    ref = np.sqrt(np.logaddexp(0.0, lg.astype(np.float64)))
+    tab = route(oracle, lg, bias, E, k, 8 | 4 | 32, route_scale=1.0)
+    sel = ref.astype(np.float32) + bias
+    for t in range(T):
+        order = sorted(range(E), key=lambda e: (-sel[t, e], e))[:k]
+        assert list(tab["eid"][t]) == order
+        assert np.allclose(tab["gate"][t], ref[t, order], rtol=3e-7, atol=0)
+    both = route(oracle, lg, bias, E, k, 8 | 4 | 32 | 1, route_scale=1.0)
+    assert np.array_equal(both.view(np.uint8), tab.view(np.uint8))
+    sig = route(oracle, lg, bias, E, k, 8 | 4 | 1, route_scale=1.0)
+    assert not np.array_equal(sig["gate"], tab["gate"])
+    ends = np.array([[0.0, 30.0, 100.0, -30.0, -100.0, 3e38, -3e38, np.inf, -np.inf, 1.0]], np.float32)
+    e = route(oracle, ends, None, 10, 10, 8 | 32, route_scale=1.0)
+    got = dict(zip(e["eid"][0].tolist(), e["gate"][0].tolist()))
+    assert got[0] == np.float32(np.sqrt(np.log(2.0)))
+    assert got[1] == np.float32(np.sqrt(30.0)) and got[2] == np.float32(10.0)
+    assert np.isclose(got[3], np.exp(-15.0), rtol=1e-6) and got[4] == 0.0   # exp(-100) is below the f32 range
+    assert got[5] == np.float32(np.sqrt(np.float64(np.float32(3e38)))) and got[6] == 0.0
+    assert got[7] == np.inf and got[8] == 0.0
+    norm = route(oracle, lg, bias, E, k, 8 | 4 | 32 | 2, route_scale=2.0)
+    assert np.allclose(norm["gate"].sum(1), 2.0, rtol=1e-5)
+
+
 def test_logit_scale_and_shared_tail(oracle):
     lg = (cases.rng_of(5).standard_normal((6, 32))).astype(np.float32)
     a = route(oracle, lg * np.float32(0.5), None, 32, 4, 8 | 1)
