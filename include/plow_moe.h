@@ -152,6 +152,15 @@ enum {
     PLOW_MOE_ARM_A4W4_P16  = 1, /* DOWN only, enc 2: as 0 with a bf16 part                         */
     PLOW_MOE_ARM_W8A8      = 2, /* enc 1: e4m3 activations with 1x128 scales; DOWN writes f32 part */
     PLOW_MOE_ARM_W8A8_P16  = 3, /* DOWN only: as 2 with a bf16 part                                */
+    /* enc 1, two-term e4m3 activations x ~= s * (hi + lo / 16) per 1x128 group, about the precision of bf16
+     * (runtime/amd/moe_pf_w8a8.h:81-92, :115-117; interp.hip:6509-6518, :6560-6571). 85 arm 4: t1 = bf16 x rows,
+     * t0 = fq rows [hi I | lo I] (2 I bytes), t7 = fs f32 [rows][I / 128]. 86 arm 4 (f32 part) / 5 (bf16 part): t1 =
+     * those fq rows, t5 = fs. Served on the bf16-activation kernels over the context's staging, which holds the
+     * aligned intermediate rows as bf16 (rows * I * 2 bytes; the routed row count must be known: an align op in the
+     * same run or fj[2]): the GLU multiplies the bf16 rows themselves where the reference multiplies their two
+     * terms, and writes the two-term rows; the DOWN multiplies bf16(s * (hi + lo / 16)) */
+    PLOW_MOE_ARM_W8A8_SPLIT     = 4,
+    PLOW_MOE_ARM_W8A8_SPLIT_P16 = 5, /* DOWN only */
     PLOW_MOE_ARM_W8A8_XQ   = 6, /* GLU only, enc 1: t1 holds the bf16 rows, quantized 1x128 where they
                                    are loaded; equals op 184 + arm 2 bit for bit, writes arm 2's fq / fs
                                    (runtime/amd/moe_pf_w8a8.h:118-121); t6 unused. i4 is unused by the

@@ -390,6 +390,24 @@ static float dot_fp8blk_a8(const float* wf, const float* srow, const float* a, c
     return acc;
 }
 
+/* The same with two-term activations a ~= as * (hi + lo / 16) (plow runtime/amd/moe_pf_w8a8.h:375-384): the block's
+ * lo products join its hi products at 2^-4 before the scales multiply. */
+static float dot_fp8blk_a8_split(const float* wf, const float* srow, const float* ahi, const float* alo, const float* as,
+                                 uint32_t K) {
+    float acc = 0.0f;
+    for (uint32_t k0 = 0, kb = 0; k0 < K; k0 += 128u, kb++) {
+        const float t = block_dot(wf + k0, ahi + k0, 128u) + 0.0625f * block_dot(wf + k0, alo + k0, 128u);
+        acc = fmaf(t, as[kb] * srow[kb], acc);
+    }
+    return acc;
+}
+
+/* One value into its two e4m3 terms (moe_pf_w8a8.h:84-92): hi = e4m3(t), lo = e4m3((t - hi) * 16) */
+static void split_e4m3(float t, uint8_t* hi, uint8_t* lo) {
+    *hi = orc_f32_to_e4m3(t);
+    *lo = orc_f32_to_e4m3((t - e4m3_lut[*hi]) * 16.0f);
+}
+
 /* mxfp4 weights, bf16 activations (mxfp4_common.h plow_mxfp4_row_dot): sequential f32 per 32-block,
  * the E8M0 scale multiplied once per block. */
 static float dot_mxfp4(const float* wf, const uint8_t* s, const float* a, uint32_t K) {
@@ -517,8 +535,13 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
     const uint32_t arm = in->i[7], pitch = in->i[4];
     /* arm 6: t1 holds the bf16 rows; each 1x128 group is quantized with op 184's arithmetic and the
      * rest is arm 2 (plow runtime/amd/moe_pf_w8a8.h:118-121, :255-283) */
-    const int xq_inline = enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ;
+    /* arm 4: as arm 6 with two e4m3 terms per value, on the way in and on the way out: t0 = fq rows [hi I | lo I]
+     * (plow runtime/amd/moe_pf_w8a8.h:115-117, :251-283, :434-452) */
+    const int split = enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_SPLIT;
+    const int xq_inline = (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_XQ) || split;
     const int w8a8 = (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8) || xq_inline;
+    float* rowlo = NULL; /* arm 4: [cached row][H] the lo terms of the rows split here */
+    uint32_t rowlo_cap = 0;
     /* enc 2, arm 0 (the reference's default for mxfp4): fp4 on both operands. t1 = bf16 rows, quantized per
      * 32 with mx_act_quant32; t0 = fu as mxfp4 [R][I/2]; t6 = row_partidx (pad rows are skipped);
      * t7 = the E8M0 rows [R][I/32] it writes (plow runtime/amd/interp.hip:6496-6499, op_moe.h:4183-4632) */
@@ -548,6 +571,7 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
         if (rc.expert != e) {
             cache_fit(&rc, cnt);
             if (xq_inline && rowxs_cap < cnt) { free(rowxs); rowxs = malloc((size_t)cnt * KB * 4u); rowxs_cap = cnt; }
+            if (split && rowlo_cap < cnt) { free(rowlo); rowlo = malloc((size_t)cnt * H * 4u); rowlo_cap = cnt; }
             if (a4w4 && rowsa_cap < cnt) { free(rowsa); rowsa = malloc((size_t)cnt * (H / 32u)); rowsa_cap = cnt; }
             for (uint32_t q = 0; q < cnt; q++) {
                 const uint32_t tok = row_token[r0 + q];
@@ -560,9 +584,15 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
                         for (uint32_t j = 0; j < 128u; j++) amax = fmaxf(amax, fabsf(orc_bf2f(src[kb * 128u + j])));
                         const float sc = amax * (1.0f / 448.0f), inv = 1.0f / sc;
                         rowxs[(size_t)q * KB + kb] = sc;
-                        for (uint32_t j = 0; j < 128u; j++)
-                            rc.a[(size_t)q * H + kb * 128u + j] =
-                                e4m3_lut[orc_f32_to_e4m3(orc_bf2f(src[kb * 128u + j]) * inv)];
+                        for (uint32_t j = 0; j < 128u; j++) {
+                            const float t = orc_bf2f(src[kb * 128u + j]) * inv;
+                            if (split) {
+                                uint8_t bh, bl;
+                                split_e4m3(t, &bh, &bl);
+                                rc.a[(size_t)q * H + kb * 128u + j] = e4m3_lut[bh];
+                                rowlo[(size_t)q * H + kb * 128u + j] = e4m3_lut[bl];
+                            } else rc.a[(size_t)q * H + kb * 128u + j] = e4m3_lut[orc_f32_to_e4m3(t)];
+                        }
                     }
                 } else if (a4w4) { /* the row as raw e2m1 values plus its E8M0 bytes */
                     const orc_bf16* src = (const orc_bf16*)TEN(in, T, 1) + (size_t)tok * H;
@@ -629,8 +659,11 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
                     const float* a = rc.a + (size_t)q * H;
                     const float* as = xq_inline ? rowxs + (size_t)q * KB : xs + tok;
                     const uint32_t as_step = xq_inline ? 1u : pitch;
-                    const float g = dot_fp8blk_a8(wg, (const float*)Sg + (size_t)g0 * KB, a, as, as_step, H);
-                    const float u = dot_fp8blk_a8(wu, (const float*)Su + (size_t)g0 * KB, a, as, as_step, H);
+                    const float* al = split ? rowlo + (size_t)q * H : NULL;
+                    const float g = split ? dot_fp8blk_a8_split(wg, (const float*)Sg + (size_t)g0 * KB, a, al, as, H)
+                                          : dot_fp8blk_a8(wg, (const float*)Sg + (size_t)g0 * KB, a, as, as_step, H);
+                    const float u = split ? dot_fp8blk_a8_split(wu, (const float*)Su + (size_t)g0 * KB, a, al, as, H)
+                                          : dot_fp8blk_a8(wu, (const float*)Su + (size_t)g0 * KB, a, as, as_step, H);
                     v[(size_t)q * 128u + (n - n0)] = glu_pair(g, u, act, in->fj[0].f, in->fj[1].f);
                 }
             }
@@ -640,12 +673,14 @@ static void op_group_glu(const PlowDevInst* in, uint32_t slice, uint32_t nblk, v
                 for (uint32_t j = 0; j < n1 - n0; j++) amax = fmaxf(amax, fabsf(v[(size_t)q * 128u + j]));
                 const float s = amax * (1.0f / 448.0f), inv = 1.0f / s;
                 fs[(size_t)(r0 + q) * G + g0] = s;
-                for (uint32_t j = 0; j < n1 - n0; j++)
-                    fq[(size_t)(r0 + q) * I + n0 + j] = orc_f32_to_e4m3(v[(size_t)q * 128u + j] * inv);
+                for (uint32_t j = 0; j < n1 - n0; j++) {
+                    if (split) split_e4m3(v[(size_t)q * 128u + j] * inv, &fq[(size_t)(r0 + q) * 2u * I + n0 + j], &fq[(size_t)(r0 + q) * 2u * I + I + n0 + j]);
+                    else fq[(size_t)(r0 + q) * I + n0 + j] = orc_f32_to_e4m3(v[(size_t)q * 128u + j] * inv);
+                }
             }
         }
     }
-    free(wg); free(wu); free(v); free(rowxs); free(rowsa);
+    free(wg); free(wu); free(v); free(rowxs); free(rowsa); free(rowlo);
     cache_free(&rc);
 }
 
@@ -676,12 +711,15 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
     const uint32_t* row_partidx = TEN(in, T, 6);
     const float* row_gate = TEN(in, T, 7);
     const uint32_t H = in->i[0], I = in->i[1], E = in->i[2], enc = in->i[3], arm = in->i[7];
-    const int w8a8 = enc == PLOW_MOE_ENC_FP8BLK &&
-                     (arm == PLOW_MOE_ARM_W8A8 || arm == PLOW_MOE_ARM_W8A8_P16);
+    /* arms 4 / 5: t1 = fq rows [hi I | lo I], both terms through the block sums (plow runtime/amd/interp.hip:6560-6571) */
+    const int split = enc == PLOW_MOE_ENC_FP8BLK && (arm == PLOW_MOE_ARM_W8A8_SPLIT || arm == PLOW_MOE_ARM_W8A8_SPLIT_P16);
+    float* rowlo = NULL;
+    uint32_t rowlo_cap = 0;
+    const int w8a8 = (enc == PLOW_MOE_ENC_FP8BLK && (arm == PLOW_MOE_ARM_W8A8 || arm == PLOW_MOE_ARM_W8A8_P16)) || split;
     /* enc 2, arm 0 / 1: fp4 on both operands; t1 = fu as mxfp4 [R][I/2], t5 = its E8M0 rows [R][I/32];
      * arm 1 = bf16 part (plow runtime/amd/interp.hip:6581-6589: i7 = part16 on the generic body) */
     const int a4w4 = enc == PLOW_MOE_ENC_MXFP4 && (arm == PLOW_MOE_ARM_A16 || arm == 1u);
-    const int part16 = (w8a8 && arm == PLOW_MOE_ARM_W8A8_P16) || (a4w4 && arm == 1u);
+    const int part16 = (w8a8 && (arm == PLOW_MOE_ARM_W8A8_P16 || arm == PLOW_MOE_ARM_W8A8_SPLIT_P16)) || (a4w4 && arm == 1u);
     /* i5: t0 is the f64 [T][H] accumulator of the deterministic fused combine; log2(k) + 1, or 256 + k */
     const uint32_t det_k = !in->i[5] ? 0u : in->i[5] > 256u ? in->i[5] - 256u : 1u << (in->i[5] - 1u);
     const float* fs = TEN(in, T, 5);
@@ -699,10 +737,14 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
         const void* Sd = stab ? (const void*)(uintptr_t)stab[(size_t)e * 3u + 2u] : NULL;
         if (rc.expert != e) {
             cache_fit(&rc, cnt);
+            if (split && rowlo_cap < cnt) { free(rowlo); rowlo = malloc((size_t)cnt * I * 4u); rowlo_cap = cnt; }
             for (uint32_t q = 0; q < cnt; q++) {
                 rc.live[q] = row_partidx[r0 + q] != PLOW_EXPERT_UNUSED;
                 if (!rc.live[q]) continue;
-                if (w8a8) decode_e4m3_row(rc.a + (size_t)q * I, (const uint8_t*)TEN(in, T, 1) + (size_t)(r0 + q) * I, I);
+                if (split) {
+                    decode_e4m3_row(rc.a + (size_t)q * I, (const uint8_t*)TEN(in, T, 1) + (size_t)(r0 + q) * 2u * I, I);
+                    decode_e4m3_row(rowlo + (size_t)q * I, (const uint8_t*)TEN(in, T, 1) + (size_t)(r0 + q) * 2u * I + I, I);
+                } else if (w8a8) decode_e4m3_row(rc.a + (size_t)q * I, (const uint8_t*)TEN(in, T, 1) + (size_t)(r0 + q) * I, I);
                 else if (a4w4) decode_mxfp4_row(rc.a + (size_t)q * I, (const uint8_t*)TEN(in, T, 1) + (size_t)(r0 + q) * (I / 2u), I);
                 else decode_bf16_row(rc.a + (size_t)q * I, (const orc_bf16*)TEN(in, T, 1) + (size_t)(r0 + q) * I, I);
             }
@@ -717,7 +759,9 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
                 if (!rc.live[q]) continue;
                 const uint32_t r = r0 + q, pidx = row_partidx[r];
                 const float* a = rc.a + (size_t)q * I;
-                const float acc = w8a8 ? dot_fp8blk_a8(wd, (const float*)Sd + (size_t)g0 * KB, a,
+                const float acc = split ? dot_fp8blk_a8_split(wd, (const float*)Sd + (size_t)g0 * KB, a, rowlo + (size_t)q * I,
+                                                              fs + (size_t)r * KB, I)
+                                  : w8a8 ? dot_fp8blk_a8(wd, (const float*)Sd + (size_t)g0 * KB, a,
                                                        fs + (size_t)r * KB, 1u, I)
                                   : a4w4 ? dot_a4w4(wd, rs.sb, a, (const uint8_t*)TEN(in, T, 5) + (size_t)r * (I / 32u), I)
                                          : enc_dot(enc, wd, rs, a, I);
@@ -728,7 +772,7 @@ static void op_group_down(const PlowDevInst* in, uint32_t slice, uint32_t nblk, 
             }
         }
     }
-    free(wd);
+    free(wd); free(rowlo);
     cache_free(&rc);
 }
 
@@ -1509,4 +1553,8 @@ float plow_oracle_e4m3_to_f32(uint8_t b) { return orc_e4m3_to_f32(b); }
 float plow_oracle_e2m1(uint8_t nib) { return orc_e2m1(nib); }
 float plow_oracle_e8m0(uint8_t s) { return orc_e8m0(s); }
 void plow_oracle_f2bf_n(uint16_t* dst, const float* src, size_t n) { for (size_t i = 0; i < n; i++) dst[i] = orc_f2bf(src[i]); }
+void plow_oracle_split_e4m3_n(uint8_t* hi, uint8_t* lo, const float* src, size_t n) {
+    if (!e4m3_lut_ready) { for (uint32_t b = 0; b < 256u; b++) e4m3_lut[b] = orc_e4m3_to_f32((uint8_t)b); e4m3_lut_ready = 1; }
+    for (size_t i = 0; i < n; i++) split_e4m3(src[i], &hi[i], &lo[i]);
+}
 void plow_oracle_e4m3_encode_n(uint8_t* dst, const float* src, size_t n) { for (size_t i = 0; i < n; i++) dst[i] = orc_f32_to_e4m3(src[i]); }

@@ -27,6 +27,8 @@ float    plow_oracle_e2m1(uint8_t nib);
 float    plow_oracle_e8m0(uint8_t s);
 void     plow_oracle_f2bf_n(uint16_t* dst, const float* src, size_t n);
 void     plow_oracle_e4m3_encode_n(uint8_t* dst, const float* src, size_t n);
+/* the two e4m3 terms of ops 85 / 86 arms 4 / 5: hi = e4m3(v), lo = e4m3((v - hi) * 16) */
+void     plow_oracle_split_e4m3_n(uint8_t* hi, uint8_t* lo, const float* src, size_t n);
 /* the activation quantizer of the fp4 x fp4 arm (ops 85 / 86, enc 2, arm 0): n_blocks 32-blocks of f32 ->
  * 16 bytes and one E8M0 byte each; its two primitives */
 void     plow_oracle_mx_act_quant(uint8_t* out, uint8_t* scales, const float* v, size_t n_blocks);

@@ -42,7 +42,7 @@ OP_MOE_QUANT_FP8_BLOCK128 = 189
 OP_MOE_DOWN_FP8_BLOCK128 = 190
 
 ENC_BF16, ENC_FP8BLK, ENC_MXFP4 = 0, 1, 2
-ARM_A16, ARM_W8A8, ARM_W8A8_P16, ARM_W8A8_XQ, ARM_W4A16 = 0, 2, 3, 6, 8
+ARM_A16, ARM_W8A8, ARM_W8A8_P16, ARM_W8A8_SPLIT, ARM_W8A8_SPLIT_P16, ARM_W8A8_XQ, ARM_W4A16 = 0, 2, 3, 4, 5, 6, 8
 ARM_A4W4, ARM_A4W4_P16 = 0, 1     # enc 2: fp4 on both operands (the reference's default for mxfp4); DOWN with a bf16 part
 ROUTER_RAW_MARK = 0x52545241       # op 180 i7: the score carries its top-k (one launch)
 ACT_GELU_TANH, ACT_SILU = 0, 1

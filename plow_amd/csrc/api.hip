@@ -202,6 +202,13 @@ struct Hint {
 /* Routed slots of the batch as far as this op can know them: the descriptor's own statement (fj[2].u,
  * an extension of this library: no MoE op of the reference uses the third immediate), else the align op
  * of the same run, else what the op's own operands imply (`own`, 0 = nothing). */
+/* aligned rows of a batch of `slots` routed rows over E experts at most (every expert's last tile of 64 may be
+ * partial); 0 when the slot count is unknown or the bound does not fit 32 bits */
+static uint32_t split_rows_bound(uint32_t slots, uint32_t E) {
+    const uint64_t b = (uint64_t)slots + (uint64_t)E * (PLOW_MPF_BM - 1u);
+    return slots && b <= 0xFFFFFFFFull ? (uint32_t)(((b + PLOW_MPF_BM - 1u) / PLOW_MPF_BM) * PLOW_MPF_BM) : 0u;
+}
+
 static uint32_t slots_of(const PlowDevInst* in, const Hint& h, uint32_t own) {
     if (in->fj[2].u) return in->fj[2].u;
     if (h.slots) return h.slots;
@@ -481,8 +488,19 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             /* the streaming form serves this arm at every row count */
             return launch_group_glu_w8a8(g, st);
         }
+        /* two-term arm: the bf16-activation GLU into the staging, then the split of its rows */
+        const bool split = enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_W8A8_SPLIT;
+        const uint32_t split_rows = split ? split_rows_bound(slots_of(in, h, 0u), E) : 0u;
+        if (split) {
+            NEED(c, ten(in, T, 7), "op 85 two-term arm: t7 fs must be bound");
+            NEED(c, c->ws_base && c->stage, "op 85 two-term arm: needs a context (its staging block)");
+            NEED(c, split_rows != 0u, "op 85 two-term arm: the routed row count must be known (an align op in the same run, or fj[2])");
+            NEED(c, (uint64_t)split_rows * I * 2u <= c->stage_bytes,
+                 "op 85 two-term arm: %u aligned rows of width %u need %llu bytes of staging, the context holds %zu: call plow_moe_reserve_staging first",
+                 split_rows, I, (unsigned long long)split_rows * I * 2u, c->stage_bytes);
+        }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
-                         (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
+                         (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) || split ||
                          (enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_W4A16);
         if (a16) {
             NEED(c, enc == PLOW_MOE_ENC_BF16 || ten(in, T, 3), "op 85: t3 stab must be bound for encoding %u", enc);
@@ -490,7 +508,7 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             NEED(c, i[5] <= 2u || i[5] == PLOW_MOE_ACT_SWIGLU_CLAMP, "op 85: activation %u is not served", i[5]);
             if (!launch) return 0;
             GroupA16 g = {};
-            g.out = ten(in, T, 0); g.a = ten(in, T, 1);
+            g.out = split ? c->stage : ten(in, T, 0); g.a = ten(in, T, 1);
             g.wtab = (const uint64_t*)ten(in, T, 2);
             g.stab = enc == PLOW_MOE_ENC_BF16 ? nullptr : (const uint64_t*)ten(in, T, 3);
             g.meta = (const int32_t*)ten(in, T, 4); g.a_idx = (const uint32_t*)ten(in, T, 5);
@@ -499,6 +517,11 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.wcols = 3; g.wsel0 = 0; g.wsel1 = 1;
             g.slots_hint = slots_of(in, h, 0u);
             if (!g.slots_hint && h.form != 0) g.form_ws = next_form_word(c); /* unknown rows: the form is chosen on the device */
+            if (split) {
+                const int grc = launch_group_glu_a16(g, st);
+                if (grc) return grc;
+                return launch_split_block128(ten(in, T, 0), (float*)ten(in, T, 7), c->stage, g.meta, g.a_idx, I, E, split_rows, st);
+            }
             return launch_group_glu_a16(g, st);
         }
         if (enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_A4W4) {
@@ -573,15 +596,32 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             }
             return launch_w8a8(c, h, slots_of(in, h, 0u), g, false, st);
         }
+        /* two-term arms: the rows back to bf16 in the staging, then the bf16-activation DOWN */
+        const bool split = enc == PLOW_MOE_ENC_FP8BLK && (arm == PLOW_MOE_ARM_W8A8_SPLIT || arm == PLOW_MOE_ARM_W8A8_SPLIT_P16);
+        const uint32_t split_rows = split ? split_rows_bound(slots_of(in, h, 0u), E) : 0u;
+        if (split) {
+            NEED(c, ten(in, T, 5), "op 86 two-term arm: t5 fs must be bound");
+            NEED(c, c->ws_base && c->stage, "op 86 two-term arm: needs a context (its staging block)");
+            NEED(c, split_rows != 0u, "op 86 two-term arm: the routed row count must be known (an align op in the same run, or fj[2])");
+            NEED(c, (uint64_t)split_rows * I * 2u <= c->stage_bytes,
+                 "op 86 two-term arm: %u aligned rows of width %u need %llu bytes of staging, the context holds %zu: call plow_moe_reserve_staging first",
+                 split_rows, I, (unsigned long long)split_rows * I * 2u, c->stage_bytes);
+        }
         const bool a16 = (enc == PLOW_MOE_ENC_BF16 && arm == PLOW_MOE_ARM_A16) ||
-                         (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) ||
+                         (enc == PLOW_MOE_ENC_FP8BLK && arm == PLOW_MOE_ARM_A16) || split ||
                          (enc == PLOW_MOE_ENC_MXFP4 && arm == PLOW_MOE_ARM_W4A16);
         if (a16) {
             NEED(c, enc == PLOW_MOE_ENC_BF16 || ten(in, T, 3), "op 86: t3 stab must be bound for encoding %u", enc);
             NEED(c, I % 128u == 0u && H % 128u == 0u, "op 86: I %u and H %u must be multiples of 128", I, H);
             if (!launch) return 0;
+            if (split) {
+                const int jrc = launch_join_block128(c->stage, ten(in, T, 1), (const float*)ten(in, T, 5), (const int32_t*)ten(in, T, 4),
+                                                     (const uint32_t*)ten(in, T, 6), I, E, split_rows, st);
+                if (jrc) return jrc;
+            }
             GroupA16 g = {};
-            g.out = ten(in, T, 0); g.a = ten(in, T, 1);
+            g.out = ten(in, T, 0); g.a = split ? c->stage : ten(in, T, 1);
+            g.out_bf16 = arm == PLOW_MOE_ARM_W8A8_SPLIT_P16 ? 1u : 0u;
             g.wtab = (const uint64_t*)ten(in, T, 2);
             g.stab = enc == PLOW_MOE_ENC_BF16 ? nullptr : (const uint64_t*)ten(in, T, 3);
             g.meta = (const int32_t*)ten(in, T, 4);

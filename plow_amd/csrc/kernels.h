@@ -40,6 +40,12 @@ int launch_combine_det(void* out, const void* residual, const void* shared, cons
                        hipStream_t st);
 int launch_zero_f64(double* p, size_t n, hipStream_t st);
 
+/* aligned bf16 rows -> two-term e4m3 rows [hi K | lo K] + scales [row][K / 128], and back (rows_bound: an upper bound
+ * of the aligned rows, for the grid; the kernels read the count from meta) */
+int launch_split_block128(void* fq, float* fs, const void* fu, const int32_t* meta, const uint32_t* row_token, uint32_t K,
+                          uint32_t E, uint32_t rows_bound, hipStream_t st);
+int launch_join_block128(void* out, const void* fq, const float* fs, const int32_t* meta, const uint32_t* row_partidx,
+                         uint32_t K, uint32_t E, uint32_t rows_bound, hipStream_t st);
 int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uint32_t K, uint32_t pitch,
                           hipStream_t st);
 int launch_quant_block128_scatter(void* hq, const void* fu, float* scale, const void* meta, const void* row_partidx,

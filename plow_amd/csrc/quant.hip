@@ -48,6 +48,103 @@ int launch_quant_block128(void* xq, const void* x, float* scale, uint32_t M, uin
     return 0;
 }
 
+__device__ __forceinline__ float e4m3_to_f32(uint32_t byte) { return __builtin_amdgcn_cvt_f32_fp8((int)byte, 0); }
+
+/* Two-term e4m3 rows of the fp8 x fp8 arms 4 / 5 of ops 85 / 86 (plow runtime/amd/moe_pf_w8a8.h:81-92, :420-452):
+ * per 1x128 group s = max(amax, 1e-10) / 448, t = v / s, hi = e4m3(t), lo = e4m3((t - hi) * 16); a row is
+ * [hi K | lo K] bytes and its scales [K / 128] f32, row-major. The rows are the tilep[E] * 64 aligned rows of
+ * `meta`; a pad row (row_token sentinel) leaves as the split of zeros, as the reference writes it. 16 lanes per
+ * (row, group), eight values each. */
+__global__ __launch_bounds__(256) void k_split_block128(uint8_t* __restrict__ fq, float* __restrict__ fs,
+                                                        const bf16_t* __restrict__ fu, const int32_t* __restrict__ meta,
+                                                        const uint32_t* __restrict__ row_token, uint32_t K, uint32_t E) {
+    const uint32_t groups = K / 128u, sub = threadIdx.x & 15u;
+    const size_t ngroup = (size_t)((uint32_t)meta[3u * E] * PLOW_MPF_BM) * groups;
+    for (size_t grp = ((size_t)blockIdx.x * 256u + threadIdx.x) / 16u; grp < ngroup; grp += (size_t)gridDim.x * 16u) {
+        const uint32_t row = (uint32_t)(grp / groups), g = (uint32_t)(grp % groups);
+        const bool live = row_token[row] != PLOW_EXPERT_UNUSED;
+        uint4 raw = make_uint4(0u, 0u, 0u, 0u);
+        if (live) raw = *(const uint4*)(fu + (size_t)row * K + g * 128u + sub * 8u);
+        const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+        float f[8];
+        float amax = 1e-10f; /* the amax is floored, not the scale */
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            f[2 * j] = __uint_as_float(v[j] << 16);
+            f[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+            amax = fmaxf(amax, fmaxf(fabsf(f[2 * j]), fabsf(f[2 * j + 1])));
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 16));
+        const float s = amax * (1.0f / 448.0f);
+        const float inv = 1.0f / s;
+        if (sub == 0) fs[(size_t)row * groups + g] = s;
+        float t[8], d[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[j] = f[j] * inv;
+        uint2 hi, lo;
+        hi.x = cvt4_e4m3(t[0], t[1], t[2], t[3]);
+        hi.y = cvt4_e4m3(t[4], t[5], t[6], t[7]);
+#pragma unroll
+        for (int j = 0; j < 8; j++) d[j] = e4m3_to_f32(((j < 4 ? hi.x : hi.y) >> (8 * (j & 3))) & 0xFFu);
+        lo.x = cvt4_e4m3((t[0] - d[0]) * 16.0f, (t[1] - d[1]) * 16.0f, (t[2] - d[2]) * 16.0f, (t[3] - d[3]) * 16.0f);
+        lo.y = cvt4_e4m3((t[4] - d[4]) * 16.0f, (t[5] - d[5]) * 16.0f, (t[6] - d[6]) * 16.0f, (t[7] - d[7]) * 16.0f);
+        uint8_t* const at = fq + (size_t)row * 2u * K + g * 128u + sub * 8u;
+        *(uint2*)at = hi;
+        *(uint2*)(at + K) = lo;
+    }
+}
+
+int launch_split_block128(void* fq, float* fs, const void* fu, const int32_t* meta, const uint32_t* row_token, uint32_t K,
+                          uint32_t E, uint32_t rows_bound, hipStream_t st) {
+    if (K % 128u || !rows_bound || !fq || !fs || !fu || !meta || !row_token) return PLOW_MOE_EINVAL;
+    const size_t ngroup = (size_t)rows_bound * (K / 128u);
+    uint32_t blocks = (uint32_t)((ngroup + 15u) / 16u);
+    if (blocks > 8192u) blocks = 8192u;
+    k_split_block128<<<blocks, 256, 0, st>>>((uint8_t*)fq, fs, (const bf16_t*)fu, meta, row_token, K, E);
+    return 0;
+}
+
+/* The way back: the aligned rows [hi K | lo K] with their 1x128 scales as bf16 rows s * (hi + lo / 16), which is what
+ * the two terms stand for; rows whose slot is the sentinel are skipped. */
+__global__ __launch_bounds__(256) void k_join_block128(bf16_t* __restrict__ out, const uint8_t* __restrict__ fq,
+                                                       const float* __restrict__ fs, const int32_t* __restrict__ meta,
+                                                       const uint32_t* __restrict__ row_partidx, uint32_t K, uint32_t E) {
+    const uint32_t groups = K / 128u, sub = threadIdx.x & 15u;
+    const size_t ngroup = (size_t)((uint32_t)meta[3u * E] * PLOW_MPF_BM) * groups;
+    for (size_t grp = ((size_t)blockIdx.x * 256u + threadIdx.x) / 16u; grp < ngroup; grp += (size_t)gridDim.x * 16u) {
+        const uint32_t row = (uint32_t)(grp / groups), g = (uint32_t)(grp % groups);
+        if (row_partidx[row] == PLOW_EXPERT_UNUSED) continue;
+        const uint8_t* const at = fq + (size_t)row * 2u * K + g * 128u + sub * 8u;
+        const uint2 hi = *(const uint2*)at, lo = *(const uint2*)(at + K);
+        const float s = fs[(size_t)row * groups + g];
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float v[2];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int e = 2 * j + h;
+                const float a = e4m3_to_f32(((e < 4 ? hi.x : hi.y) >> (8 * (e & 3))) & 0xFFu);
+                const float b = e4m3_to_f32(((e < 4 ? lo.x : lo.y) >> (8 * (e & 3))) & 0xFFu);
+                v[h] = s * fmaf(b, 0.0625f, a);
+            }
+            o[j] = (uint32_t)f2bf(v[0]) | ((uint32_t)f2bf(v[1]) << 16);
+        }
+        *(uint4*)(out + (size_t)row * K + g * 128u + sub * 8u) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+int launch_join_block128(void* out, const void* fq, const float* fs, const int32_t* meta, const uint32_t* row_partidx,
+                         uint32_t K, uint32_t E, uint32_t rows_bound, hipStream_t st) {
+    if (K % 128u || !rows_bound || !out || !fq || !fs || !meta || !row_partidx) return PLOW_MOE_EINVAL;
+    const size_t ngroup = (size_t)rows_bound * (K / 128u);
+    uint32_t blocks = (uint32_t)((ngroup + 15u) / 16u);
+    if (blocks > 8192u) blocks = 8192u;
+    k_join_block128<<<blocks, 256, 0, st>>>((bf16_t*)out, (const uint8_t*)fq, fs, meta, row_partidx, K, E);
+    return 0;
+}
+
 /* bf16 rows -> mxfp4 rows with one E8M0 byte per 32 values: the activation quantizer of the fp4 x fp4 arm
  * of ops 85 / 86 (plow runtime/amd/op_moe.h:4132-4179, amd_common.h:1031-1111). Four lanes per 32-block,
  * eight values each; value 2i sits in the low nibble of byte i. */

@@ -150,7 +150,7 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
     row_token = p._t("row_token", "u32", (R,), "scratch")
     row_partidx = p._t("row_partidx", "u32", (R,), "scratch")
     row_gate = p._t("row_gate", "f32", (R,), "scratch")
-    p16 = cfg.part_bf16 and ((cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q")) or
+    p16 = cfg.part_bf16 and ((cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q", "w8a8split")) or
                              (cfg.enc == "mxfp4" and cfg.arm == "a4w4"))
     det = cfg.det_combine and cfg.enc == "fp8blk" and cfg.arm in ("w8a8", "w8a8q")
     assert not (det and p16)
@@ -221,10 +221,16 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
                                      t=[out, hq, hs, wtab, stab, meta, row_partidx, row_gate],
                                      i=[I, H, Ea, ka, T], slots=T * ka))
             return p
-        if enc == abi.ENC_FP8BLK and cfg.arm in ("w8a8", "w8a8q"):
-            fq = p._t("fq", "u8", (R, I), "scratch")
+        if enc == abi.ENC_FP8BLK and cfg.arm in ("w8a8", "w8a8q", "w8a8split"):
+            two = cfg.arm == "w8a8split"   # two e4m3 terms per value: rows [hi I | lo I]
+            fq = p._t("fq", "u8", (R, 2 * I if two else I), "scratch")
             fs = p._t("fs", "f32", (R, I // 128), "scratch")
-            if cfg.arm == "w8a8q":
+            if two:
+                assert not det, "the deterministic combine is the plain arm's"
+                p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
+                                        t=[fq, x, wtab, stab, meta, row_token, None, fs],
+                                        i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8_SPLIT], f=cfg.act_f, slots=T * ka))
+            elif cfg.arm == "w8a8q":
                 p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_PF,
                                         t=[fq, x, wtab, stab, meta, row_token, None, fs],
                                         i=[I, H, Ea, enc, T, cfg.act, 0, abi.ARM_W8A8_XQ], f=cfg.act_f, slots=T * ka))
@@ -238,7 +244,8 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
             p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_PF,
                                      t=[part, fq, wtab, stab, meta, fs, row_partidx, row_gate],
                                      i=[H, I, Ea, enc, 0, (256 + ka) if det else 0, 0,
-                                        abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8], slots=T * ka))
+                                        (abi.ARM_W8A8_SPLIT_P16 if p16 else abi.ARM_W8A8_SPLIT) if two
+                                        else (abi.ARM_W8A8_P16 if p16 else abi.ARM_W8A8)], slots=T * ka))
         elif enc == abi.ENC_MXFP4 and cfg.arm == "a4w4":
             # fp4 on both operands: the GLU quantizes its bf16 rows per 32 and writes the intermediate as
             # mxfp4 with E8M0 rows; i4 = T (the rows of x) is what this library's quantizer pass needs

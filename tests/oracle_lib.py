@@ -38,6 +38,7 @@ def load_oracle():
     lib.plow_oracle_e8m0.restype = C.c_float
     lib.plow_oracle_f2bf_n.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
     lib.plow_oracle_e4m3_encode_n.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.plow_oracle_split_e4m3_n.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
     lib.plow_oracle_mx_act_quant.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
     lib.plow_oracle_mx_act_e8m0.argtypes = [C.c_float]
     lib.plow_oracle_mx_act_e8m0.restype = C.c_uint8

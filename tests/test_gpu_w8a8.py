@@ -102,6 +102,58 @@ def test_glu_quantizes_bf16_rows_itself(moe, oracle, T):
         assert np.array_equal(dev.np("out"), ref.np("out"))
 
 
+@pytest.mark.parametrize("T,p16", [(1, False), (19, True), (100, False), (333, True), (700, False)])
+def test_two_term_arms(moe, oracle, T, p16):
+    """Ops 85 / 86 arms 4 / 5: the intermediate as two e4m3 terms per value, rows [hi I | lo I] with 1x128 scales
+    (plow runtime/amd/moe_pf_w8a8.h:81-92, :115-117). The library multiplies the bf16 rows themselves where the
+    reference multiplies their two terms (which stand for them to 2^-8), so the stored rows are compared as
+    values, s * (hi + lo / 16), at the precision the two terms carry; few rows per expert (streaming kernels,
+    matrix-vector form at one token) and many (tiled kernels)."""
+    print(f"[case] w8a8 two-term T={T} p16={p16}", flush=True)
+    cfg = layer.MoeConfig("mini-split", H=512, E=32, I=256, k=4, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          n_group=4, topk_group=2, route_scale=2.5, enc="fp8blk", arm="w8a8split", part_bf16=p16,
+                          n_shared=1, shared_mode="fold")
+    plan, dev, host = both(moe, oracle, cfg, seed=T)
+    rows = assert_routing_equal(plan, dev, host)
+    I = cfg.I
+    live = host.np("row_partidx")[:rows] != abi.EXPERT_UNUSED
+    e4 = lambda b: torch.from_numpy(np.ascontiguousarray(b)).view(torch.float8_e4m3fn).float().numpy()
+    def rows_of(t):
+        fq, fs = t.np("fq")[:rows][live], t.np("fs")[:rows][live]
+        return np.repeat(fs, 128, axis=1) * (e4(fq[:, :I]) + e4(fq[:, I:]) / 16.0), fs
+    vd, fsd = rows_of(dev)
+    vh, fsh = rows_of(host)
+    assert np.allclose(fsd, fsh, rtol=1e-2)
+    amax = np.repeat(np.abs(vh).reshape(vh.shape[0], -1, 128).max(2), 128, axis=1)
+    err = (np.abs(vd - vh) / np.maximum(amax, 1e-20)).max()
+    print(f"[parity] two-term rows: max |dev - ref| / group amax = {err:.3e}", flush=True)
+    assert err < 2.0 ** -5
+    relL2 = np.sqrt(((vd - vh) ** 2).sum() / (vh ** 2).sum())
+    print(f"[parity] two-term rows: relL2 = {relL2:.3e}", flush=True)
+    assert relL2 < 5e-3
+    if p16:
+        assert_output_close(dev.np("part").reshape(-1), host.np("part").reshape(-1), "part (bf16)")
+    else:
+        pd, ph = dev.np("part"), host.np("part")
+        assert np.all(np.isfinite(pd))
+        assert np.abs(pd - ph).max() / np.abs(ph).max() < 2e-2
+    assert_output_close(dev.np("out"), host.np("out"))
+
+
+def test_two_term_arm_refusals(moe):
+    """The arms keep their aligned intermediate rows in the context's staging: a batch it does not hold, or a row
+    count the op cannot know, is refused before anything is launched."""
+    t = torch.zeros(64, device="cuda")
+    from gpu_harness import dev_table
+    tab = dev_table([t] * 8)
+    big = abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5, None, 7], i=[2048, 7168, 257, 1, 4096, 1, 0, abi.ARM_W8A8_SPLIT], slots=4096 * 9)
+    assert moe.check(big, tab) == abi.E_INVAL and "staging" in moe.last_error()
+    unknown = abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[512, 256, 33, 1, 0, 0, 0, abi.ARM_W8A8_SPLIT_P16])
+    assert moe.check(unknown, tab) == abi.E_INVAL and "row count" in moe.last_error()
+    ok = abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[512, 256, 33, 1, 0, 0, 0, abi.ARM_W8A8_SPLIT], slots=400)
+    assert moe.check(ok, tab) == 0
+
+
 @pytest.mark.parametrize("T,limit", [(1, 0.0), (19, 0.0), (100, 0.02), (333, 0.0), (700, 0.02)])  # from 16 rows per expert: tiled form
 def test_atomic_chain_ops_188_189_190(moe, oracle, T, limit):
     """The block-fp8 chain with a bf16 intermediate (op 188), a slot-major quantized copy of it (op 189)

@@ -401,6 +401,76 @@ def test_fp8blk_layer_against_f64_over_the_same_bytes(oracle, arm):
         assert np.allclose(part[s], y, rtol=2e-5, atol=2e-5 * np.abs(y).max())
 
 
+def test_fp8blk_two_term_arms_against_f64_over_bf16_activations(oracle):
+    """Arms 4 (GLU) and 4 / 5 (DOWN): two e4m3 terms per value, s * (hi + lo / 16). Pinned by what the two terms are
+    for: (1) the stored rows [hi | lo] decode to the f64 GLU of the bf16 inputs to about bf16 precision (2^-7 of the
+    group's amax; a dropped lo term or a wrong 1/16 leaves the single term's 2^-4), (2) over a sweep of the whole
+    e4m3 range hi is the nearest e4m3 value and hi + lo / 16 lies within 2^-8 of the value (2^-14 absolute at the
+    bottom), (3) the DOWN equals an f64 product over the decoded rows, and lands several times closer to the all-f64
+    layer than the single-term arm 2 does, (4) arm 5 is arm 4 rounded to bf16."""
+    r = cases.rng_of(31)
+    E, T, H, I, k = 4, 9, 256, 256, 2
+    W, S, wtab, stab = build_fp8(oracle, r, E, T, H, I, False, False)
+    tab = np.zeros(T * k, dtype=ol.ROUTE_DT)
+    for t in range(T):
+        tab["eid"][t * k:(t + 1) * k] = r.choice(E, k, replace=False)
+    tab["gate"] = (r.random(T * k) + 0.1).astype(np.float32)
+    al = cases.align_arrays(tab, T, E, k)
+    run(oracle, cases.align_inst(T, E, k), al)
+    R = al[2].shape[0]
+    x = cases.randn_bf16(r, (T, H), 1.0)
+    e4 = lambda b: torch.from_numpy(np.ascontiguousarray(b)).view(torch.float8_e4m3fn).double().numpy()
+    fq, fs = np.zeros((R, 2 * I), np.uint8), np.zeros((R, I // 128), np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5, None, 7], i=[I, H, E, 1, T, 1, 0, 4]),
+        [fq, x, wtab, stab, al[0], al[2], None, fs], 2)
+    part = np.zeros((T * k, H), np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[H, I, E, 1, 0, 0, 0, 4]),
+        [part, fq, wtab, stab, al[0], fs, al[3], al[4]], 2)
+    p16 = np.zeros((T * k, H), np.uint16)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[H, I, E, 1, 0, 0, 0, 5]),
+        [p16, fq, wtab, stab, al[0], fs, al[3], al[4]], 2)
+    # the single-term chain on the same inputs
+    xq, xs = np.zeros((T, H), np.uint8), np.zeros((H // 128, T), np.float32)
+    run(oracle, abi.inst(abi.OP_QUANT_FP8_BLOCK128, t=[0, 1, 2], i=[T, H, T]), [xq, x, xs])
+    fq1, fs1 = np.zeros((R, I), np.uint8), np.zeros((R, I // 128), np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_GLU_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[I, H, E, 1, T, 1, 0, 2]),
+        [fq1, xq, wtab, stab, al[0], al[2], xs, fs1], 2)
+    part1 = np.zeros((T * k, H), np.float32)
+    run(oracle, abi.inst(abi.OP_MOE_GROUP_DOWN_PF, t=[0, 1, 2, 3, 4, 5, 6, 7], i=[H, I, E, 1, 0, 0, 0, 2]),
+        [part1, fq1, wtab, stab, al[0], fs1, al[3], al[4]], 2)
+    # (2)
+    sweep = np.concatenate([np.linspace(-448, 448, 200001), np.geomspace(2.0 ** -12, 448, 50000), [0.0, 448.0, -448.0]]).astype(np.float32)
+    bh, bl = np.zeros(sweep.size, np.uint8), np.zeros(sweep.size, np.uint8)
+    oracle.plow_oracle_split_e4m3_n(bh.ctypes.data, bl.ctypes.data, sweep.ctypes.data, sweep.size)
+    assert np.array_equal(bh, torch.from_numpy(sweep).to(torch.float8_e4m3fn).view(torch.uint8).numpy())
+    two = e4(bh) + e4(bl) / 16.0
+    assert np.all(np.abs(two - sweep) <= np.maximum(np.abs(sweep.astype(np.float64)) * 2.0 ** -8, 2.0 ** -14))
+    assert np.mean(np.abs(e4(bh) - sweep) > np.abs(sweep) * 2.0 ** -6) > 0.3   # which one term alone does not reach
+    silu = lambda g: g / (1.0 + np.exp(-g))
+    xa = ol.bf2f(x).astype(np.float64)
+    sc = np.repeat(fs.astype(np.float64), 128, axis=1)
+    hi, lo = e4(fq[:, :I]), e4(fq[:, I:])
+    fa = sc * (hi + lo / 16.0)
+    err2 = err1 = ref2 = 0.0
+    for row in range(int(al[0][-1]) * 64):
+        s = al[3][row]
+        if s == abi.EXPERT_UNUSED:
+            continue
+        e, t = tab["eid"][s], s // k
+        v = silu(dequant(W["g"][e][1], S["g"][e]) @ xa[t]) * (dequant(W["u"][e][1], S["u"][e]) @ xa[t])
+        amax = np.abs(v).reshape(-1, 128).max(1).repeat(128)
+        assert np.all(np.abs(fa[row] - v) <= amax * 2.0 ** -7 + 1e-9)                   # (1)
+        assert np.abs(sc[row] * hi[row] - v).max() > np.abs(fa[row] - v).max() * 4      # lo carries real bits
+        y = tab["gate"][s] * (dequant(W["d"][e][1], S["d"][e]) @ fa[row])
+        assert np.all(np.abs(part[s] - y) <= 1e-5 * np.abs(y).max() + 1e-6)             # (3)
+        yref = tab["gate"][s] * (dequant(W["d"][e][1], S["d"][e]) @ v)
+        err2 += ((part[s] - yref) ** 2).sum(); err1 += ((part1[s] - yref) ** 2).sum(); ref2 += (yref ** 2).sum()
+        assert np.array_equal(p16[s], ol.f2bf(part[s]))                                 # (4)
+    rel2, rel1 = np.sqrt(err2 / ref2), np.sqrt(err1 / ref2)
+    print(f"two-term relL2 {rel2:.2e}, single-term {rel1:.2e}")
+    assert rel2 < 4e-3 and rel2 * 8 < rel1
+
+
 def test_fp8blk_inline_quant_arm_equals_quantizer_plus_plain_arm(oracle):
     """Op 85 arm 6 takes the bf16 rows and quantizes each 1x128 group itself: by definition the quantizer
     op followed by arm 2, bit for bit (plow runtime/amd/moe_pf_w8a8.h:118-121)."""
