@@ -76,6 +76,10 @@ def make_cfg(layer, a, name, tokens):
         cfg.arm = "w8a8" if cfg.T >= 128 else "a16"
         # the decode arm's ops 65 / 66 sort the slots themselves: plow's chain for them has no op 84
         cfg.emit_align = False
+    if name == "c4" and not a.arm and cfg.T * cfg.k_all <= 128:
+        # a few tokens: plow's decode experts (ops 48 / 49, table driven, slot-major rows; no op 84 in their chain),
+        # the same arithmetic as arm 8 of the grouped ops the larger batches run
+        cfg.arm, cfg.emit_align = "a16dec", False
     if a.arm == "w8a8det":      # the deterministic fused down -> combine on the block-fp8 W8A8 arm
         cfg.arm, cfg.det_combine = "w8a8", True
     elif a.arm:

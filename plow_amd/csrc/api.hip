@@ -703,6 +703,20 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
         NEED(c, E <= c->ws.max_e && nslot <= c->ws.max_slots, "op %u: %u slots / %u experts exceed the workspace (%u slots, %u experts)", (unsigned)in->op, nslot, E, c->ws.max_slots, c->ws.max_e);
         NEED(c, act <= 1u, "op %u: activation %u is not served", (unsigned)in->op, act);
         if (!launch) return 0;
+        if (plow_moe_tuning().gemv_direct) {
+            /* a handful of slots on the matrix-vector form: the table itself lists the rows, nothing is sorted */
+            GroupA16 d = {};
+            d.out = ten(in, T, 0); d.a = ten(in, T, 1);
+            d.wtab = (const uint64_t*)ten(in, T, 3);
+            d.stab = enc == PLOW_MOE_ENC_BF16 ? nullptr : (const uint64_t*)ten(in, T, 4);
+            d.N = N; d.K = K; d.E = E; d.enc = enc; d.act = act;
+            d.wcols = pc ? 2u : 3u;
+            d.slots_hint = nslot;
+            d.tab_direct = ten(in, T, 2), d.tab_nslot = nslot, d.tab_kx = glu ? kx : 1u;
+            if (glu) d.wsel0 = 0, d.wsel1 = pc ? 0u : 1u, d.wrow1 = pc ? N : 0u;
+            else d.wsel0 = d.wsel1 = pc ? 1u : 2u, d.zs_table = ten(in, T, 2), d.zs_nslot = nslot;
+            if (group_a16_gemv_serves(d)) return launch_group_a16_gemv(d, glu, st);
+        }
         /* align with k = slots per input row: row_token = slot / kx, row_partidx = slot */
         int rc = 0;
         if (!sort_reusable(h, ten(in, T, 2), nslot, E, kx, glu)) {

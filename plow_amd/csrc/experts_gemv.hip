@@ -140,7 +140,25 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
     /* live rows in windows of GV_WINDOW, by their ordinal among the live rows */
     for (uint32_t base = 0;; base += GV_WINDOW) {
         __syncthreads();
-        if (wv == 0) { /* one wave lists the window: experts 64 at a time, rows appended in expert order */
+        if (wv == 0 && g.tab_direct) { /* the table's live slots in slot order (all of them fit one window) */
+            const PlowMoeRoute* const tab = (const PlowMoeRoute*)g.tab_direct;
+            uint32_t eid[GV_WINDOW / WAVE];
+#pragma unroll
+            for (uint32_t j = 0; j < GV_WINDOW / WAVE; j++) {
+                const uint32_t sl = j * WAVE + lane;
+                eid[j] = sl < g.tab_nslot ? tab[sl].eid : PLOW_EXPERT_UNUSED;
+            }
+            uint32_t seen = 0;
+#pragma unroll
+            for (uint32_t j = 0; j < GV_WINDOW / WAVE; j++) {
+                const bool live = eid[j] < E;
+                const unsigned long long m = __ballot(live);
+                const uint32_t ord = seen + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+                if (live && base == 0u) l_row[ord] = j * WAVE + lane, l_exp[ord] = eid[j];
+                seen += (uint32_t)__popcll(m);
+            }
+            if (lane == 0) l_n = base == 0u ? seen : 0u;
+        } else if (wv == 0) { /* one wave lists the window: experts 64 at a time, rows appended in expert order */
             /* every count and offset is asked for before the first is used: one trip to memory, not one per chunk */
             uint32_t cnt_r[GV_ECHUNKS], off_r[GV_ECHUNKS];
 #pragma unroll
@@ -209,10 +227,10 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
                                        stt ? (const uint8_t*)(uintptr_t)stt[GLU ? g.wsel1 : g.wsel0] : nullptr};
             const uint32_t wr[2] = {g.wrow0, GLU ? g.wrow1 : g.wrow0};
             const bool resident = wbase[0] && wbase[1] && (ENC == GV_BF16 || (sbase[0] && sbase[1]));
-            const uint32_t orow = g.o_idx ? g.o_idx[row] : row;
+            const uint32_t orow = g.tab_direct ? row : (g.o_idx ? g.o_idx[row] : row);
             if (resident && orow != PLOW_EXPERT_UNUSED && c_lo < c_hi) {
                 /* the row of activations: the lane's slice of every piece */
-                const uint32_t arow = g.a_idx ? g.a_idx[row] : row;
+                const uint32_t arow = g.tab_direct ? row / g.tab_kx : (g.a_idx ? g.a_idx[row] : row);
                 const uint8_t* xsrc = (const uint8_t*)g.a + (size_t)arow * K * (XF8 ? 1u : 2u);
                 v4i x[ITER][XQ];
                 float xs[ITER];
@@ -234,7 +252,7 @@ __global__ __launch_bounds__(GV_WAVES* WAVE) void k_group_a16_gemv(GroupA16 g) {
                             x[it][j] = p < pieces ? *(const v4i*)(xsrc + ((size_t)p * XQ + j) * 16u) : (v4i){0, 0, 0, 0};
                     }
                 }
-                const float gate = (!GLU && g.gate) ? g.gate[row] : 1.0f;
+                const float gate = GLU ? 1.0f : (g.tab_direct ? ((const PlowMoeRoute*)g.tab_direct)[row].gate : (g.gate ? g.gate[row] : 1.0f));
                 /* per-channel scales: lane l applies the scale of channel c0 + l when the 64 results of a group are
                  * stored; those of the wave's first group (usually its only one) are asked for here, with the
                  * activations, and not one by one inside the loop */
@@ -351,9 +369,10 @@ static uint32_t gv_max_slots(uint32_t enc) {
 }
 
 bool group_a16_gemv_serves(const GroupA16& g) {
-    if (!plow_moe_tuning().a16_gemv || !g.meta || !g.wtab || g.bias || g.slots_hint == 0u || g.enc > GV_FP8PC ||
+    if (!plow_moe_tuning().a16_gemv || (!g.meta && !g.tab_direct) || !g.wtab || g.bias || g.slots_hint == 0u || g.enc > GV_FP8PC ||
         g.slots_hint > gv_max_slots(g.enc))
         return false;
+    if (g.tab_direct && (g.tab_nslot > GV_WINDOW || !g.tab_kx || g.a_f8scale)) return false;
     if (g.enc != GV_BF16 && !g.stab) return false;
     if (g.a_f8scale && (g.enc != GV_FP8BLK || g.a_idx)) return false; /* quantized activations: block-fp8 DOWN on aligned rows */
     const uint32_t row_bytes = g.enc == GV_BF16 ? g.K * 2u : (g.enc == GV_MXFP4 ? g.K / 2u : g.K);

@@ -186,6 +186,11 @@ struct GroupA16 {
     uint32_t down_wide;
     /* streaming forms: set by the launcher when experts of a handful of rows run with per-wave copies of their rows */
     uint32_t priv_rows;
+    /* matrix-vector form of the slot-major ops: when set, the routing table [tab_nslot] itself lists the rows (row =
+     * slot, in slot order; its expert and gate from the table; its input row slot / tab_kx, its output row the slot)
+     * and meta, a_idx, o_idx and gate are not read: no sort ahead of the op */
+    const void* tab_direct;
+    uint32_t tab_nslot, tab_kx;
     /* Dense ops of a few rows (one expert, no meta, bf16 weights): scratch the launcher may use to split K over
      * several workgroups per channel tile (NULL: never split). split_ws holds f32 partial rows. */
     void* split_ws;

@@ -22,6 +22,8 @@
  *   PLOW_MOE_A16_PRIVATE_ROWS 0                streaming bf16-activation kernels: experts of a handful of rows share the
  *                                              workgroup's row ring like the others (default: per-wave copies on fp8 and
  *                                              bf16 weights)
+ *   PLOW_MOE_GEMV_DIRECT      0                slot-major ops of a handful of slots sort their slots like the others (default: the
+ *                                              matrix-vector form lists its rows from the routing table itself)
  *   PLOW_MOE_A16_DENSE_SPLIT  0                dense bf16 ops of a few rows walk the whole K in one workgroup per channel
  *                                              tile (default: K split over several workgroups while the tiles are
  *                                              fewer than the CUs)
@@ -54,6 +56,7 @@ struct PlowMoeTuning {
     bool a16_down_wide;
     bool a16_private_rows;
     bool a16_dense_split;
+    bool gemv_direct;
 };
 const PlowMoeTuning& plow_moe_tuning();
 

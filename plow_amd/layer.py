@@ -172,7 +172,7 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
         p._emit("topk", abi.inst(abi.OP_MOE_ROUTER_TOPK_PF, t=[table, logit, part if det else None, bias],
                                  i=[H if det else 0, E, k, cfg.flags, T, cfg.tail, cfg.n_group, cfg.topk_group],
                                  f=[cfg.route_scale, 0.0]))
-    slot_major = cfg.enc == "fp8pc" and cfg.arm != "w8a8"
+    slot_major = (cfg.enc == "fp8pc" and cfg.arm != "w8a8") or cfg.arm == "a16dec"
     if cfg.emit_align or not slot_major:
         p._emit("align", abi.inst(abi.OP_MOE_ALIGN_PF, t=[meta, table, row_token, row_partidx, row_gate],
                                   i=[T, Ea, ka]))
@@ -205,7 +205,14 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
         enc = {"bf16": abi.ENC_BF16, "fp8blk": abi.ENC_FP8BLK, "mxfp4": abi.ENC_MXFP4}[cfg.enc]
         wtab = p._t("wtab", "u64", (Ea, 3), "table")
         stab = p._t("stab", "u64", (Ea, 3), "table") if enc != abi.ENC_BF16 else None
-        if enc == abi.ENC_FP8BLK and cfg.arm == "w8a8atomic":
+        if cfg.arm == "a16dec":
+            # plow's decode experts (ops 48 / 49): bf16 activations, table driven, slot-major rows, no op 84
+            fu = p._t("fu", "bf16", (T * ka, I), "scratch")
+            p._emit("glu", abi.inst(abi.OP_MOE_GROUP_GLU_FP8_BLK, t=[fu, x, table, wtab, stab],
+                                    i=[T * ka, I, H, Ea, ka, cfg.act, enc]))
+            p._emit("down", abi.inst(abi.OP_MOE_GROUP_DOWN_FP8_BLK, t=[part, fu, table, wtab, stab],
+                                     i=[T * ka, H, I, Ea, 0, 0, enc]))
+        elif enc == abi.ENC_FP8BLK and cfg.arm == "w8a8atomic":
             assert cfg.shared_mode != "dense" and not cfg.residual, "the atomic chain has no combine op"
             xq = p._t("xq", "u8", (T, H), "scratch")
             xs = p._t("xs", "f32", (H // 128, T), "scratch")
@@ -221,7 +228,9 @@ def plan_layer(cfg: MoeConfig, with_router_score: bool = True) -> LayerPlan:
                                      t=[out, hq, hs, wtab, stab, meta, row_partidx, row_gate],
                                      i=[I, H, Ea, ka, T], slots=T * ka))
             return p
-        if enc == abi.ENC_FP8BLK and cfg.arm in ("w8a8", "w8a8q", "w8a8split"):
+        if cfg.arm == "a16dec":
+            pass
+        elif enc == abi.ENC_FP8BLK and cfg.arm in ("w8a8", "w8a8q", "w8a8split"):
             two = cfg.arm == "w8a8split"   # two e4m3 terms per value: rows [hi I | lo I]
             fq = p._t("fq", "u8", (R, 2 * I if two else I), "scratch")
             fs = p._t("fs", "f32", (R, I // 128), "scratch")

@@ -113,6 +113,20 @@ def test_bf16_activation_arms_many_rows(moe, oracle, enc, arm, T, E, k):
     check_chain(*both(moe, oracle, cfg, seed=T))
 
 
+@pytest.mark.parametrize("enc", ["bf16", "fp8blk", "mxfp4"])
+@pytest.mark.parametrize("T", [1, 3, 12, 40])
+def test_decode_expert_ops_48_49_in_a_layer(moe, oracle, enc, T):
+    """The table-driven decode experts (ops 48 / 49, slot-major rows) as the layer's expert ops, every weight encoding:
+    a handful of slots (the matrix-vector form lists its rows from the routing table itself, nothing is sorted),
+    and more (the slots are sorted into the context's workspace first)."""
+    print(f"[case] ops 48 / 49 layer enc={enc} T={T}", flush=True)
+    cfg = layer.MoeConfig("a16-dec", H=512, E=16, I=256, k=4, T=T, scoring="sigmoid", norm_topk=True, bias=True,
+                          enc=enc, arm="a16dec", n_shared=1, shared_mode="fold")
+    plan, dev, host = both(moe, oracle, cfg, seed=T)
+    assert [i.op for i in plan.insts][3:5] == [abi.OP_MOE_GROUP_GLU_FP8_BLK, abi.OP_MOE_GROUP_DOWN_FP8_BLK]
+    check_chain(plan, dev, host)
+
+
 @pytest.mark.parametrize("enc,H,I,E,T", [("mxfp4", 2048, 512, 64, 64), ("mxfp4", 2048, 1536, 64, 64), ("mxfp4", 2048, 768, 64, 64),
                                          ("mxfp4", 4096, 512, 128, 96), ("fp8blk", 2048, 512, 64, 16), ("fp8pc", 2048, 512, 64, 16),
                                          ("bf16", 2048, 512, 64, 16)])
