@@ -819,6 +819,13 @@ static int run_op(PlowMoeCtx* c, const PlowDevInst* in, void* const* T, hipStrea
             g.o_idx = (const uint32_t*)ten(in, T, 6); g.gate = (const float*)ten(in, T, 7);
             return launch_group_down_a16(g, st);
         }
+        if (plow_moe_tuning().gemv_direct) { /* a handful of slots: the table itself lists the rows, nothing is sorted */
+            GroupA16 d = g;
+            d.slots_hint = nslot;
+            d.tab_direct = ten(in, T, 2), d.tab_nslot = nslot, d.tab_kx = glu ? kx : 1u;
+            if (!glu) d.zs_table = ten(in, T, 2), d.zs_nslot = nslot;
+            if (group_a16_gemv_serves(d)) return launch_group_a16_gemv(d, glu, st);
+        }
         /* slot-major: sort the slots by expert into the context workspace (row_token = slot / k) */
         if (!sort_reusable(h, ten(in, T, 2), nslot, E, kx, glu)) {
             rc = launch_align(c->ws.meta, ten(in, T, 2), c->ws.row_token, c->ws.row_partidx, c->ws.row_gate,
