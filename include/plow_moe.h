@@ -225,7 +225,12 @@ void plow_moe_destroy(PlowMoeCtx* ctx);
  * width `hidden`: it allocates (call it at set-up, never under stream capture), keeps every earlier block
  * until plow_moe_destroy (graphs captured before stay valid) and returns PLOW_MOE_ENOMEM after seven
  * growths or when the device is out of memory. No counterpart in the reference, which quantizes every
- * gathered row inside its GEMM kernel (runtime/amd/op_moe.h:3948-4720). */
+ * gathered row inside its GEMM kernel (runtime/amd/op_moe.h:3948-4720).
+ * The same block is the scratch of three other ops, each of which writes what it keeps there and reads it back
+ * before it returns its last launch (ops of one context therefore belong on one stream at a time): op 85 arm 6 at
+ * many rows (rows * (H + H / 32) bytes), the two-term arms 4 / 5 of ops 85 / 86 (aligned rows * I * 2 bytes: refused
+ * when they do not fit) and the dense ops 20 / 8 (K-slice partial sums of a few rows, or the one-expert tables of
+ * many: kept on their plain form when they do not fit). */
 #define PLOW_MOE_STAGE_DEFAULT_BYTES (32u << 20)
 int plow_moe_reserve_staging(PlowMoeCtx* ctx, size_t token_rows, size_t hidden);
 

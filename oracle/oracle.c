@@ -12,7 +12,7 @@
  *   op 83/56 router top-k      runtime/cpu/dev/golden/moe_route.c:27-86 (flat arm);
  *                              group-limited arm runtime/common/moe_route_key.h:61-80 +
  *                              runtime/amd/op_moe.h:377-420; shared tail slot op_moe.h:2417-2434;
- *                              logit scale op_moe.h:444-446
+ *                              logit scale op_moe.h:444-446; sqrt-softplus scores op_moe.h:485-494
  *   op 84 align                runtime/cpu/dev/golden/moe_route.c:91-127
  *   op 87/43 combine           runtime/cpu/dev/golden/moe_route.c:130-147; t_row0 / part16
  *                              runtime/amd/interp.hip:6605-6635
@@ -28,6 +28,9 @@
  *   op 48/49 (all enc)         runtime/cpu/dev/golden/moe.c:21-174 with runtime/cpu/dev/
  *                              mxfp4_common.h:30-40 as the row dot; op_moe.h:1234-1399
  *   op 85 enc 1 arm 6          runtime/amd/moe_pf_w8a8.h:118-121, :255-283 (quantizer + arm 2)
+ *   op 85 enc 1 arm 4, and
+ *   op 86 enc 1 arm 4/5        runtime/amd/moe_pf_w8a8.h:81-92 (the split), :251-283 (on the way in), :375-384
+ *                              (both terms through a block's sum), :434-452 (on the way out)
  *   op 188/189/190             runtime/amd/op_moe_fp8_block128.h:7-88, op_gemm_common.h:1845-2010,
  *                              :2582-2621 (SCATTER), interp.hip:5282-5310; op 190 adds in aligned-row
  *                              order where the device adds atomically in no fixed order
@@ -38,7 +41,10 @@
  *
  * Parity pins are listed per function in tests/test_oracle_*.py. Unpinned at bit level (tolerance
  * level only): the f32 summation order INSIDE one 128-K block of the fp8 x fp8 arms, which the
- * reference leaves to its MFMA; this file sums a block with eight interleaved f32 partials.
+ * reference leaves to its MFMA; this file sums a block with eight interleaved f32 partials. The
+ * sqrt-softplus scores use the C library's expf / log1pf / sqrtf where the reference, device code only, uses
+ * its device library's: parity with those bits is unpinned (the expression itself is pinned against f64 and
+ * its closed-form ends).
  */
 #define _GNU_SOURCE /* sched_getaffinity, pthread_setaffinity_np */
 #include "oracle.h"
