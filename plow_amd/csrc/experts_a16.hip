@@ -1099,10 +1099,10 @@ __global__ __launch_bounds__(256) void k_dense_tables(uint8_t* base, const void*
         int32_t* const meta = (int32_t*)(base + 64u);
         meta[0] = 0, meta[1] = (int32_t)M;
     }
-    if (r < M) {
-        ((uint32_t*)(base + DENSE_TAB_BYTES))[r] = r;
-        ((uint32_t*)(base + DENSE_TAB_BYTES + map_bytes))[r] = r;
-        ((float*)(base + DENSE_TAB_BYTES + 2u * (size_t)map_bytes))[r] = 1.0f;
+    if (r < map_bytes / 4u) { /* the maps run on to a multiple of 256 rows: entries past the last row are pad rows */
+        ((uint32_t*)(base + DENSE_TAB_BYTES))[r] = r < M ? r : PLOW_EXPERT_UNUSED;
+        ((uint32_t*)(base + DENSE_TAB_BYTES + map_bytes))[r] = r < M ? r : PLOW_EXPERT_UNUSED;
+        ((float*)(base + DENSE_TAB_BYTES + 2u * (size_t)map_bytes))[r] = r < M ? 1.0f : 0.0f;
     }
 }
 
@@ -1115,7 +1115,7 @@ static bool a16_dense_tiled_try(const GroupA16& g, hipStream_t st, int* rc) {
         g.bias || !g.split_ws || !g.out_bf16 || g.ksplit || g.a_idx || g.o_idx || g.gate || g.wmul > 1u || g.wrow0 || g.wrow1)
         return false;
     const uint32_t M = g.dense_rows;
-    const size_t map_bytes = ((size_t)M * 4u + 255u) & ~(size_t)255u;
+    const size_t map_bytes = (((size_t)M + 255u) & ~(size_t)255u) * 4u;
     if (map_bytes > 0x7FFFFFFFull || DENSE_TAB_BYTES + 3u * map_bytes > g.split_ws_bytes) return false;
     uint8_t* const base = (uint8_t*)g.split_ws;
     GroupA16 t = g;
@@ -1130,7 +1130,7 @@ static bool a16_dense_tiled_try(const GroupA16& g, hipStream_t st, int* rc) {
         w.N = g.N, w.K = g.K, w.E = 1u, w.w_bf16 = 1u, w.meta = t.meta;
         if (!group_w8a8_tiled_serves(w)) return false;
     }
-    k_dense_tables<<<(M + 255u) / 256u, 256, 0, st>>>(base, g.wdirect[0], g.wdirect[1], M, (uint32_t)map_bytes);
+    k_dense_tables<<<(uint32_t)(map_bytes / 1024u), 256, 0, st>>>(base, g.wdirect[0], g.wdirect[1], M, (uint32_t)map_bytes);
     if (!a16_tiled_try<GLU>(t, st, rc, false)) *rc = PLOW_MOE_EINVAL; /* (the checks above are the tiled form's own) */
     return true;
 }
