@@ -54,6 +54,19 @@ def test_c4_kimi_k2_mxfp4_decode(moe, oracle, B):
     assert_output_close(dev.np("out"), host.np("out"), f"c4 B={B} out")
 
 
+@pytest.mark.parametrize("B", [1, 4, 14])
+def test_c4_kimi_k2_mxfp4_decode_on_the_decode_expert_ops(moe, oracle, B):
+    """The chain the benchmark runs at a few tokens: plow's table-driven decode experts (ops 48 / 49, slot-major
+    rows) in place of the grouped ops, no op 84 among the ops timed (the plan here keeps it, for the row maps the
+    routing check reads); up to 128 routed rows the matrix-vector form lists its rows from the routing table."""
+    import dataclasses
+    cfg = dataclasses.replace(layer.config("c4", B), arm="a16dec")
+    plan, dev, host = both(moe, oracle, cfg, seed=0)
+    assert [i.op for i in plan.insts if i.op in (48, 49)] == [48, 49]
+    assert_routing_equal(plan, dev, host)
+    assert_output_close(dev.np("out"), host.np("out"), f"c4 B={B} out (ops 48 / 49)")
+
+
 def print_popularity(cnt, T, k, s=1.2):
     """The realised expert popularity (share of the tokens that chose the expert, experts sorted by it) next to
     what Zipf(s) gives: k experts drawn without replacement with weights rank^-s (10000 seeded draws by the
