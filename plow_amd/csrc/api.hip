@@ -77,6 +77,10 @@ struct PlowMoeCtx {
     uint32_t n_stage;
     void* stage;
     size_t stage_bytes;
+    /* a second stream (default priority) and the two events that fork it off the caller's stream and join it back:
+     * the dense shared-expert ops of a run go there while the routed experts run (exec_run) */
+    hipStream_t side;
+    hipEvent_t ev_fork, ev_join;
 };
 
 /* bytes of staging the fp4 x fp4 GLU needs for `rows` token rows of width H */
@@ -149,6 +153,16 @@ extern "C" int plow_moe_create(PlowMoeCtx** out, int device) {
         plow_moe_destroy(c);
         return PLOW_MOE_ENOMEM;
     }
+    (void)hipGetDevice(&prev);
+    (void)hipSetDevice(device);
+    const bool side_ok = hipStreamCreateWithFlags(&c->side, hipStreamNonBlocking) == hipSuccess &&
+                         hipEventCreateWithFlags(&c->ev_fork, hipEventDisableTiming) == hipSuccess &&
+                         hipEventCreateWithFlags(&c->ev_join, hipEventDisableTiming) == hipSuccess;
+    (void)hipSetDevice(prev);
+    if (!side_ok) {
+        plow_moe_destroy(c);
+        return PLOW_MOE_EDEVICE;
+    }
     *out = c;
     return 0;
 }
@@ -166,6 +180,9 @@ extern "C" int plow_moe_reserve_staging(PlowMoeCtx* ctx, size_t token_rows, size
 
 extern "C" void plow_moe_destroy(PlowMoeCtx* ctx) {
     if (!ctx) return;
+    if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
+    if (ctx->ev_join) (void)hipEventDestroy(ctx->ev_join);
+    if (ctx->side) (void)hipStreamDestroy(ctx->side);
     (void)hipFree(ctx->ws_base);
     for (uint32_t n = 0; n < ctx->n_stage; n++) (void)hipFree(ctx->stage_blocks[n]);
     delete ctx;
@@ -886,6 +903,73 @@ static Hint hint_of_run(const PlowDevInst* insts, uint32_t n_inst, int form) {
     return h;
 }
 
+/* Operand slots an op writes (bit j: t[j]); every slot for an op this table does not know */
+static uint32_t out_slots(const PlowDevInst* in) {
+    switch (in->op) {
+    case PLOW_DOP_GEMM_F32: return in->i[7] == PLOW_ROUTER_RAW_MARK ? (1u | 8u | 32u) : 1u;
+    case PLOW_DOP_MOE_ROUTER_TOPK:
+    case PLOW_DOP_MOE_ROUTER_TOPK_PF: return 1u | 4u;
+    case PLOW_DOP_MOE_ALIGN_PF: return 1u | 4u | 8u | 16u;
+    case PLOW_DOP_MOE_GROUP_GLU_PF: return 1u | 128u;
+    case PLOW_DOP_MOE_GROUP_DOWN_PF:
+    case PLOW_DOP_MOE_COMBINE_PF:
+    case PLOW_DOP_GEMM_GLU:
+    case PLOW_DOP_GEMM: return 1u;
+    default: return 0xFFu;
+    }
+}
+/* the op keeps something in the context's staging while it runs */
+static bool uses_staging(const PlowDevInst* in) {
+    if (in->op == PLOW_DOP_GEMM_GLU || in->op == PLOW_DOP_GEMM) return true;
+    if (in->op == PLOW_DOP_MOE_GROUP_GLU_PF)
+        return (in->i[3] == PLOW_MOE_ENC_FP8BLK && (in->i[7] == PLOW_MOE_ARM_W8A8_XQ || in->i[7] == PLOW_MOE_ARM_W8A8_SPLIT)) ||
+               (in->i[3] == PLOW_MOE_ENC_MXFP4 && in->i[7] == PLOW_MOE_ARM_A4W4);
+    if (in->op == PLOW_DOP_MOE_GROUP_DOWN_PF)
+        return in->i[3] == PLOW_MOE_ENC_FP8BLK && (in->i[7] == PLOW_MOE_ARM_W8A8_SPLIT || in->i[7] == PLOW_MOE_ARM_W8A8_SPLIT_P16);
+    return false;
+}
+/* `x` (an op of the run) may run beside dense op `d`: x neither touches what d writes nor writes what d reads */
+static bool beside(const PlowDevInst* x, const PlowDevInst* d) {
+    if (uses_staging(x)) return false;
+    const uint32_t xo = out_slots(x);
+    for (int j = 0; j < 8; j++) {
+        if (x->t[j] == PLOW_TENSOR_NONE) continue;
+        if (x->t[j] == d->t[0]) return false;
+        if ((xo >> j) & 1u)
+            for (int q = 1; q < 8; q++)
+                if (d->t[q] != PLOW_TENSOR_NONE && x->t[j] == d->t[q]) return false;
+    }
+    return true;
+}
+
+/* A run's dense shared-expert ops (20 / 8: a few dozen workgroups each at a few tokens) go to the context's second
+ * stream, forked off the caller's stream ahead of the ops before them that touch none of their operands (the routed
+ * experts, whose last round leaves CUs idle) and joined again before the op that follows them: the run's result is
+ * that of its ops in order. [a, b): the block of dense ops; h: the first op that runs beside it. */
+static bool dense_overlap_plan(const PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, uint32_t* a, uint32_t* b, uint32_t* h) {
+    if (!ctx->side || !plow_moe_tuning().dense_overlap) return false;
+    uint32_t lo = n_inst;
+    for (uint32_t n = 0; n < n_inst; n++)
+        if (insts[n].op == PLOW_DOP_GEMM_GLU || insts[n].op == PLOW_DOP_GEMM) { lo = n; break; }
+    if (lo == n_inst || lo == 0u) return false;
+    uint32_t hi = lo;
+    while (hi < n_inst && (insts[hi].op == PLOW_DOP_GEMM_GLU || insts[hi].op == PLOW_DOP_GEMM)) hi++;
+    for (uint32_t n = hi; n < n_inst; n++) /* one block only */
+        if (insts[n].op == PLOW_DOP_GEMM_GLU || insts[n].op == PLOW_DOP_GEMM) return false;
+    for (uint32_t n = lo; n < hi; n++) /* a few rows each: larger ones fill the chip by themselves */
+        if (insts[n].i[0] >= 128u) return false;
+    uint32_t first = lo;
+    while (first > 0u) {
+        bool ok = true;
+        for (uint32_t d = lo; d < hi && ok; d++) ok = beside(&insts[first - 1u], &insts[d]);
+        if (!ok) break;
+        first--;
+    }
+    if (first == lo) return false;
+    *a = lo, *b = hi, *h = first;
+    return true;
+}
+
 static int exec_run(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, void* const* tensors, void* stream,
                     int form) {
     Hint h = hint_of_run(insts, n_inst, form);
@@ -893,11 +977,28 @@ static int exec_run(PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, 
         const int rc = run_op(ctx, &insts[n], tensors, nullptr, false, h);
         if (rc) return rc;
     }
-    for (uint32_t n = 0; n < n_inst; n++) {
-        const int rc = finish(ctx, run_op(ctx, &insts[n], tensors, (hipStream_t)stream, true, h), &insts[n]);
-        if (rc) return rc;
+    const hipStream_t st = (hipStream_t)stream;
+    uint32_t da = 0, db = 0, dh = 0;
+    if (!dense_overlap_plan(ctx, insts, n_inst, &da, &db, &dh)) {
+        for (uint32_t n = 0; n < n_inst; n++) {
+            const int rc = finish(ctx, run_op(ctx, &insts[n], tensors, st, true, h), &insts[n]);
+            if (rc) return rc;
+        }
+        return 0;
     }
-    return 0;
+    int rc = 0;
+    for (uint32_t n = 0; n < dh && !rc; n++) rc = finish(ctx, run_op(ctx, &insts[n], tensors, st, true, h), &insts[n]);
+    if (rc) return rc;
+    if (hipEventRecord(ctx->ev_fork, st) != hipSuccess || hipStreamWaitEvent(ctx->side, ctx->ev_fork, 0) != hipSuccess)
+        return fail(ctx, PLOW_MOE_EDEVICE, "the run's second stream could not be forked");
+    for (uint32_t n = da; n < db && !rc; n++) rc = finish(ctx, run_op(ctx, &insts[n], tensors, ctx->side, true, h), &insts[n]);
+    for (uint32_t n = dh; n < da && !rc; n++) rc = finish(ctx, run_op(ctx, &insts[n], tensors, st, true, h), &insts[n]);
+    /* joined whatever happened in between: a capture of the caller's stream must not end with the fork open */
+    if (hipEventRecord(ctx->ev_join, ctx->side) != hipSuccess || hipStreamWaitEvent(st, ctx->ev_join, 0) != hipSuccess)
+        return fail(ctx, PLOW_MOE_EDEVICE, "the run's second stream could not be joined");
+    if (rc) return rc;
+    for (uint32_t n = db; n < n_inst && !rc; n++) rc = finish(ctx, run_op(ctx, &insts[n], tensors, st, true, h), &insts[n]);
+    return rc;
 }
 
 extern "C" int plow_moe_check(PlowMoeCtx* ctx, const PlowDevInst* inst, void* const* tensors) {

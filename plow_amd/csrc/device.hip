@@ -36,6 +36,7 @@ const PlowMoeTuning& plow_moe_tuning() {
         t.a16_private_rows = !is("PLOW_MOE_A16_PRIVATE_ROWS", "0");
         t.a16_dense_split = !is("PLOW_MOE_A16_DENSE_SPLIT", "0");
         t.gemv_direct = !is("PLOW_MOE_GEMV_DIRECT", "0");
+        t.dense_overlap = !is("PLOW_MOE_DENSE_OVERLAP", "0");
         t.form_on_device = !is("PLOW_MOE_FORM_ON_DEVICE", "0");
         t.score_row_narrow = is("PLOW_MOE_SCORE_ROW", "narrow");
     });

@@ -24,6 +24,8 @@
  *                                              bf16 weights)
  *   PLOW_MOE_GEMV_DIRECT      0                slot-major ops of a handful of slots sort their slots like the others (default: the
  *                                              matrix-vector form lists its rows from the routing table itself)
+ *   PLOW_MOE_DENSE_OVERLAP    0                a run's dense shared-expert ops of a few rows stay on the caller's stream, in
+ *                                              their place (default: on the context's second stream beside the routed experts)
  *   PLOW_MOE_A16_DENSE_SPLIT  0                dense bf16 ops of a few rows walk the whole K in one workgroup per channel
  *                                              tile (default: K split over several workgroups while the tiles are
  *                                              fewer than the CUs)
@@ -57,6 +59,7 @@ struct PlowMoeTuning {
     bool a16_private_rows;
     bool a16_dense_split;
     bool gemv_direct;
+    bool dense_overlap;
 };
 const PlowMoeTuning& plow_moe_tuning();
 

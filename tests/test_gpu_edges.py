@@ -153,15 +153,19 @@ def test_per_row_quant_refusals_and_poison(moe):
     assert np.all((q & 0x7F) == 0x7F)
 
 
-@pytest.mark.parametrize("arm,enc,T", [("w8a8", "fp8blk", 24), ("a16", "mxfp4", 5), ("w8a8", "fp8blk", 600), ("a4w4", "mxfp4", 300)])
+@pytest.mark.parametrize("arm,enc,T", [("w8a8", "fp8blk", 24), ("a16", "mxfp4", 5), ("w8a8", "fp8blk", 600), ("a4w4", "mxfp4", 300),
+                                       ("a16", "bf16", 9), ("a16", "bf16", 200)])
 def test_layer_chain_replays_from_a_hip_graph(moe, arm, enc, T):
     """The op chain of a layer allocates nothing and clears nothing through the runtime, so a caller may
     capture it: captured once, replayed four times with new activations and other work in between, every
-    replay must equal the eager result bit for bit."""
+    replay must equal the eager result bit for bit. The bf16 cases carry two dense shared experts (ops 20 / 8):
+    at a few tokens those run on the context's second stream, forked off and joined back inside the captured run,
+    as K slices with their partial sums in the staging; at 200 tokens on the tiled kernel in their place."""
     from plow_amd import layer, synth
     print(f"[case] graph replay arm={arm} enc={enc} T={T}", flush=True)
+    shared = dict(n_shared=2, shared_mode="dense") if enc == "bf16" else dict(n_shared=1, shared_mode="fold")
     cfg = layer.MoeConfig("graph", H=512, E=16, I=512 if arm == "a4w4" else 256, k=4, T=T, scoring="sigmoid", norm_topk=True,
-                          bias=True, enc=enc, arm=arm, n_shared=1, shared_mode="fold")
+                          bias=True, enc=enc, arm=arm, **shared)
     plan = layer.plan_layer(cfg)
     dev = synth.bind(plan, "cuda", seed=11)
     insts, table = abi.inst_array(plan.insts), dev.table()
