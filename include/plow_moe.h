@@ -212,9 +212,10 @@ typedef struct PlowMoeCtx PlowMoeCtx;
 uint32_t plow_moe_abi(void);
 
 /* Create / destroy an operator context on HIP device `device`. The context owns a fixed workspace
- * (routing scratch of the slot-major ops) and PLOW_MOE_STAGE_DEFAULT_BYTES of staging for the fp4 x fp4
- * arm; no op allocates, frees or waits for the device (the ownership contract of
- * runtime/cpu/dev/cpu_dev.h:5-7). Replaces the per-engine load step of moe_lt.rs:697-814. */
+ * (routing scratch of the slot-major ops), PLOW_MOE_STAGE_DEFAULT_BYTES of staging for the fp4 x fp4
+ * arm, and a second stream with two events (a run's dense shared-expert ops are launched there beside the
+ * routed experts, forked off and joined back to the caller's stream inside the run); no op allocates, frees
+ * or waits for the device (the ownership contract of runtime/cpu/dev/cpu_dev.h:5-7). Replaces the per-engine load step of moe_lt.rs:697-814. */
 int  plow_moe_create(PlowMoeCtx** out, int device);
 void plow_moe_destroy(PlowMoeCtx* ctx);
 
