@@ -944,7 +944,7 @@ static bool beside(const PlowDevInst* x, const PlowDevInst* d) {
 
 /* A run's dense shared-expert ops (20 / 8: a few dozen workgroups each at a few tokens) go to the context's second
  * stream, forked off the caller's stream ahead of the ops before them that touch none of their operands (the routed
- * experts, whose last round leaves CUs idle) and joined again before the op that follows them: the run's result is
+ * experts, whose final pass of workgroups leaves CUs idle) and joined again before the op that follows them: the run's result is
  * that of its ops in order. [a, b): the block of dense ops; h: the first op that runs beside it. */
 static bool dense_overlap_plan(const PlowMoeCtx* ctx, const PlowDevInst* insts, uint32_t n_inst, uint32_t* a, uint32_t* b, uint32_t* h) {
     if (!ctx->side || !plow_moe_tuning().dense_overlap) return false;
