@@ -84,6 +84,8 @@ def make_cfg(layer, a, name, tokens):
         cfg.arm, cfg.det_combine = "w8a8", True
     elif a.arm:
         cfg.arm = a.arm
+    if a.part_bf16:             # plow's bf16-partial arms (op 86 i7 = 3 / 1 / 5, op 87 i7 = 1): half the bytes of the part round trip
+        cfg.part_bf16 = True
     # --raw-router: below 16 tokens the decode router as one op, the score carrying its top-k, as plow emits it
     # (crates/devgen/src/mla.rs:3294-3312); the same bytes, and measured level with the two ops per layer
     if cfg.T < 16 and not cfg.det_combine and a.raw_router:
@@ -254,6 +256,7 @@ def main():
     ap.add_argument("--arm", default="", help="override the configuration's arm (a16 | w8a8 | w8a8q | w8a8atomic | w8a8det | a4w4)")
     ap.add_argument("--zipf", type=float, default=-1.0, help="override the expert popularity exponent")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--part-bf16", action="store_true", help="bf16 partial rows between DOWN and combine (the reference's part16 arms) instead of f32")
     ap.add_argument("--raw-router", action="store_true", help="below 16 tokens: the score op carries its top-k (one launch)")
     ap.add_argument("--calib", action="store_true",
                     help="also run a plain 1 GiB device copy three times (a kernel of known traffic, "
