@@ -194,3 +194,36 @@ def test_layer_chain_replays_from_a_hip_graph(moe, arm, enc, T):
         assert torch.equal(dev.t["table"], want_table), f"replay {n}: routing differs"
         assert torch.equal(dev.t["out"], want_out), f"replay {n}: output differs"
         assert bool(torch.isfinite(scratch))
+
+
+def test_dense_ops_on_the_second_stream_keep_the_order_of_the_run(moe):
+    """A run's dense ops of a few rows are launched on the context's second stream beside the ops before them that
+    share no operand with them. Two runs of [RMSNorm, dense GLU, dense GEMM]: one where the GLU reads the row the
+    norm writes (it must wait for it) and one where the norm works on tensors of its own (the dense ops may run
+    beside it); both must give the bytes of the same ops issued one at a time."""
+    M, N, K = 24, 256, 512
+    r = cases.rng_of(77)
+    x, other = to_dev(cases.randn_bf16(r, (M, K), 1.0)), to_dev(cases.randn_bf16(r, (M, K), 1.0))
+    wg, wu, wd = (to_dev(cases.randn_bf16(r, s, 0.05)) for s in ((N, K), (N, K), (K, N)))
+    st = torch.cuda.current_stream().cuda_stream
+    for norm_in, norm_out in ((0, 1), (8, 9)):   # handles: 0 x, 1 xn, 2 wg, 3 wu, 4 fu, 5 wd, 6 y, 8 other, 9 other_n
+        ops = [abi.inst(abi.OP_RMSNORM, t=[norm_out, norm_in, None], i=[M, K], f=[1e-6]),
+               abi.inst(abi.OP_GEMM_GLU, t=[4, 1, 2, None, None, 3], i=[M, N, K, 0, 0, 1]),
+               abi.inst(abi.OP_GEMM, t=[6, 4, 5], i=[M, K, N, 0, 0, 0])]
+        res = []
+        for many in (False, True):
+            xn = torch.zeros((M, K), dtype=torch.int16, device="cuda") if norm_out == 1 else x.clone()
+            fu = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+            y = torch.zeros((M, K), dtype=torch.int16, device="cuda")
+            on = torch.zeros((M, K), dtype=torch.int16, device="cuda")
+            tab = dev_table([x, xn, wg, wu, fu, wd, y, None, other, on])
+            if many:
+                moe.exec_many(abi.inst_array(ops), tab, st)
+            else:
+                for op in ops:
+                    moe.exec(op, tab, st)
+            torch.cuda.synchronize()
+            res.append((fu.clone(), y.clone(), on.clone(), xn.clone()))
+        for a, b in zip(*res):
+            assert torch.equal(a, b)
+        assert bool((res[1][1] != 0).any())
