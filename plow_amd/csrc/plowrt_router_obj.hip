@@ -60,6 +60,7 @@ extern "C" __global__ __launch_bounds__(512) void plow_router_decode(RouterDecod
                               a.n_group, a.topk_group, a.route_scale, 0.0f};
         if (a.n_exp <= 128u) router_topk_token<2>(t, row, (float*)lds);
         else if (a.n_exp <= 256u) router_topk_token<4>(t, row, (float*)lds);
+        else if (a.n_exp <= 384u) router_topk_token<6>(t, row, (float*)lds);
         else router_topk_token<8>(t, row, (float*)lds);
         if (a.signal_add) { /* the table is written: tell whoever waits on the counter */
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");

@@ -484,6 +484,7 @@ int launch_router_topk(void* table, const void* logit, const float* bias, uint32
     const dim3 g((T + RT_WAVES - 1) / RT_WAVES), b(RT_WAVES * WAVE);
     if (n_exp <= 128u) k_router_topk<2><<<g, b, 0, st>>>(a);
     else if (n_exp <= 256u) k_router_topk<4><<<g, b, 0, st>>>(a);
+    else if (n_exp <= 384u) k_router_topk<6><<<g, b, 0, st>>>(a); /* (384 experts: six per lane, no idle candidates in the rounds) */
     else if (n_exp <= 512u) k_router_topk<8><<<g, b, 0, st>>>(a);
     else k_router_topk<16><<<g, b, 0, st>>>(a);
     return 0;

@@ -354,6 +354,7 @@ __device__ __forceinline__ void router_topk_token(const RouterArgs& a, uint32_t 
 __device__ __forceinline__ void router_topk_token_any(const RouterArgs& a, uint32_t tok, float* score) {
     if (a.n_exp <= 128u) router_topk_token<2>(a, tok, score);
     else if (a.n_exp <= 256u) router_topk_token<4>(a, tok, score);
+    else if (a.n_exp <= 384u) router_topk_token<6>(a, tok, score);
     else if (a.n_exp <= 512u) router_topk_token<8>(a, tok, score);
     else router_topk_token<16>(a, tok, score);
 }
