@@ -482,10 +482,15 @@ int launch_router_topk(void* table, const void* logit, const float* bias, uint32
     RouterArgs a = {(PlowMoeRoute*)table, logit, bias, n_exp, k, flags, T, tail, n_group, topk_group,
                     route_scale, logit_scale};
     const dim3 g((T + RT_WAVES - 1) / RT_WAVES), b(RT_WAVES * WAVE);
-    if (n_exp <= 128u) k_router_topk<2><<<g, b, 0, st>>>(a);
+    /* the smallest instance that holds the experts: a lane's idle candidates cost every selection round */
+    if (n_exp <= 64u) k_router_topk<1><<<g, b, 0, st>>>(a);
+    else if (n_exp <= 128u) k_router_topk<2><<<g, b, 0, st>>>(a);
+    else if (n_exp <= 192u) k_router_topk<3><<<g, b, 0, st>>>(a);
     else if (n_exp <= 256u) k_router_topk<4><<<g, b, 0, st>>>(a);
-    else if (n_exp <= 384u) k_router_topk<6><<<g, b, 0, st>>>(a); /* (384 experts: six per lane, no idle candidates in the rounds) */
+    else if (n_exp <= 320u) k_router_topk<5><<<g, b, 0, st>>>(a);
+    else if (n_exp <= 384u) k_router_topk<6><<<g, b, 0, st>>>(a);
     else if (n_exp <= 512u) k_router_topk<8><<<g, b, 0, st>>>(a);
+    else if (n_exp <= 768u) k_router_topk<12><<<g, b, 0, st>>>(a);
     else k_router_topk<16><<<g, b, 0, st>>>(a);
     return 0;
 }

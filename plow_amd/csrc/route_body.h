@@ -352,7 +352,8 @@ __device__ __forceinline__ void router_topk_token(const RouterArgs& a, uint32_t 
 
 /* the same with the form picked inside the kernel (the fused decode routers) */
 __device__ __forceinline__ void router_topk_token_any(const RouterArgs& a, uint32_t tok, float* score) {
-    if (a.n_exp <= 128u) router_topk_token<2>(a, tok, score);
+    if (a.n_exp <= 64u) router_topk_token<1>(a, tok, score);
+    else if (a.n_exp <= 128u) router_topk_token<2>(a, tok, score);
     else if (a.n_exp <= 256u) router_topk_token<4>(a, tok, score);
     else if (a.n_exp <= 384u) router_topk_token<6>(a, tok, score);
     else if (a.n_exp <= 512u) router_topk_token<8>(a, tok, score);
