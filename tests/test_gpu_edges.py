@@ -154,13 +154,15 @@ def test_per_row_quant_refusals_and_poison(moe):
 
 
 @pytest.mark.parametrize("arm,enc,T", [("w8a8", "fp8blk", 24), ("a16", "mxfp4", 5), ("w8a8", "fp8blk", 600), ("a4w4", "mxfp4", 300),
-                                       ("a16", "bf16", 9), ("a16", "bf16", 200)])
+                                       ("a16", "bf16", 9), ("a16", "bf16", 200), ("a16dec", "mxfp4", 3), ("a16dec", "fp8blk", 40)])
 def test_layer_chain_replays_from_a_hip_graph(moe, arm, enc, T):
     """The op chain of a layer allocates nothing and clears nothing through the runtime, so a caller may
     capture it: captured once, replayed four times with new activations and other work in between, every
     replay must equal the eager result bit for bit. The bf16 cases carry two dense shared experts (ops 20 / 8):
     at a few tokens those run on the context's second stream, forked off and joined back inside the captured run,
-    as K slices with their partial sums in the staging; at 200 tokens on the tiled kernel in their place."""
+    as K slices with their partial sums in the staging; at 200 tokens on the tiled kernel in their place. The a16dec
+    cases run the table-driven decode experts (ops 48 / 49): at 3 tokens the matrix-vector form reads its rows from
+    the routing table the captured top-k writes, at 40 the slots are sorted into the context's workspace."""
     from plow_amd import layer, synth
     print(f"[case] graph replay arm={arm} enc={enc} T={T}", flush=True)
     shared = dict(n_shared=2, shared_mode="dense") if enc == "bf16" else dict(n_shared=1, shared_mode="fold")
